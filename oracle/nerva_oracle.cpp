@@ -1,0 +1,873 @@
+// CPU oracle for the batch-1 decode path.
+//
+// TEST INFRASTRUCTURE ONLY. This file is a scalar restatement of the arithmetic
+// in the reference's CPU model crate and of the staging (where values are
+// rounded to 16 bits) used by its device decode session. It is compiled by
+// oracle/Makefile into oracle/libnerva_oracle.so and is linked/loaded only by
+// the tests, by the smoke check and by the CPU-baseline leg of the benchmark.
+// Nothing in the shipped library may call into it.
+//
+// Every function cites the reference file:line it restates (paths relative to
+// the reference checkout). Loop order and f32 accumulation order follow the
+// Rust code (sequential left-to-right sums, no FMA contraction: build with
+// -ffp-contract=off).
+//
+// Pinning status (what fixes each function independent of this file):
+//   codecs                     - reference known-answer tables (tests/golden/kat.json)
+//   fnv1a                      - reference hashes (block output hash, token hashes)
+//   gemv / fp8 gemv            - reference KAT [0, 1072, 4.90625]; f64 brute force
+//   rms_norm / per-head norm   - closed forms (unit gamma -> RMS 1), numpy f64
+//   rope                       - reference closed-form KAT (angles 1.0 and 0.01)
+//   blockwise attention        - equals dense softmax (numpy f64), reference GQA cases
+//   argmax                     - brute force, reference final-head KAT (token 1)
+//   moe route / experts        - reference closed-form KATs
+//   block forward              - reference output bits [16126, 17299] + FNV hash
+//   greedy loop                - reference token stream [1,2,3,0]
+//   synthetic generator        - not a reference function (defined by this build)
+// No function of this oracle is "parity unpinned".
+
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <vector>
+
+#define NVO_API extern "C" __attribute__((visibility("default")))
+
+// ---------------------------------------------------------------------------
+// Codecs  (crates/nerva-model/src/precision/bits.rs)
+// ---------------------------------------------------------------------------
+
+static inline float bits_to_f32(uint32_t bits) {
+  float value;
+  memcpy(&value, &bits, 4);
+  return value;
+}
+static inline uint32_t f32_to_bits(float value) {
+  uint32_t bits;
+  memcpy(&bits, &value, 4);
+  return bits;
+}
+
+// bits.rs:4-6
+NVO_API float nvo_bf16_to_f32(uint16_t bits) { return bits_to_f32((uint32_t)bits << 16); }
+
+// bits.rs:8-18 (RNE via bits + 0x7fff + lsb; NaN keeps the top half and sets bit 0)
+NVO_API uint16_t nvo_f32_to_bf16(float value) {
+  uint32_t bits = f32_to_bits(value);
+  uint32_t exponent = bits & 0x7f800000u;
+  uint32_t mantissa = bits & 0x007fffffu;
+  if (exponent == 0x7f800000u && mantissa != 0) {
+    return (uint16_t)((bits >> 16) | 1u);
+  }
+  uint32_t lsb = (bits >> 16) & 1u;
+  return (uint16_t)((bits + 0x7fffu + lsb) >> 16);
+}
+
+// bits.rs:20-45
+NVO_API float nvo_f16_to_f32(uint16_t bits) {
+  uint32_t sign = ((uint32_t)(bits & 0x8000u)) << 16;
+  uint32_t exp = (bits >> 10) & 0x1fu;
+  uint32_t frac = bits & 0x03ffu;
+  if (exp == 0) {
+    if (frac == 0) return bits_to_f32(sign);
+    uint32_t mantissa = frac;
+    int exponent = -14;
+    while ((mantissa & 0x0400u) == 0) {
+      mantissa <<= 1;
+      exponent -= 1;
+    }
+    mantissa &= 0x03ffu;
+    uint32_t f32_exp = (uint32_t)(exponent + 127);
+    return bits_to_f32(sign | (f32_exp << 23) | (mantissa << 13));
+  }
+  if (exp == 0x1f) return bits_to_f32(sign | 0x7f800000u | (frac << 13));
+  return bits_to_f32(sign | ((exp + 112u) << 23) | (frac << 13));
+}
+
+// bits.rs:47-85
+NVO_API uint16_t nvo_f32_to_f16(float value) {
+  uint32_t bits = f32_to_bits(value);
+  uint16_t sign = (uint16_t)((bits >> 16) & 0x8000u);
+  int exp = (int)((bits >> 23) & 0xffu);
+  uint32_t mant = bits & 0x007fffffu;
+  if (exp == 255) return (uint16_t)(sign | 0x7c00u | (mant != 0 ? 0x0200u : 0u));
+  int half_exp = exp - 127 + 15;
+  if (half_exp >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (half_exp <= 0) {
+    if (half_exp < -10) return sign;
+    uint32_t mantissa = mant | 0x00800000u;
+    uint32_t shift = (uint32_t)(14 - half_exp);
+    uint16_t half = (uint16_t)(mantissa >> shift);
+    uint32_t round_bit = 1u << (shift - 1);
+    uint32_t round_mask = round_bit - 1;
+    uint32_t remainder = mantissa & (round_bit | round_mask);
+    if (remainder > round_bit || (remainder == round_bit && (half & 1) != 0)) half += 1;
+    return (uint16_t)(sign | half);
+  }
+  uint16_t half = (uint16_t)(((uint16_t)half_exp << 10) | (uint16_t)(mant >> 13));
+  uint32_t remainder = mant & 0x1fffu;
+  if (remainder > 0x1000u || (remainder == 0x1000u && (half & 1) != 0)) half += 1;
+  return (uint16_t)(sign | half);
+}
+
+// bits.rs:87-104  (e4m3fn: no infinities, 0x7f/0xff are NaN, subnormal step 2^-9)
+NVO_API float nvo_fp8_e4m3fn_to_f32(uint8_t bits) {
+  float sign = (bits & 0x80) ? -1.0f : 1.0f;
+  int exp = (bits >> 3) & 0x0f;
+  int frac = bits & 0x07;
+  if (exp == 0) {
+    if (frac == 0) return sign * 0.0f;
+    return sign * (float)frac * (1.0f / 8.0f) * ldexpf(1.0f, -6);
+  }
+  if (exp == 0x0f && frac == 0x07) return NAN;
+  return sign * (1.0f + (float)frac * (1.0f / 8.0f)) * ldexpf(1.0f, exp - 7);
+}
+
+// crates/nerva-cuda/src/deepseek_quant/fp8.rs:18-72 (RNE, saturate to +-448, NaN -> 0x7f)
+NVO_API uint8_t nvo_f32_to_fp8_e4m3fn(float value) {
+  uint32_t bits = f32_to_bits(value);
+  uint8_t sign = (uint8_t)((bits >> 24) & 0x80u);
+  uint32_t abs_bits = bits & 0x7fffffffu;
+  if (abs_bits > 0x7f800000u) return 0x7f;
+  float abs_value = bits_to_f32(abs_bits);
+  if (abs_value > 448.0f) return (uint8_t)(sign | 0x7e);
+  if (abs_value < 0.015625f) {
+    uint32_t quantum = (uint32_t)nearbyintf(abs_value * 512.0f);  // default mode = ties-to-even
+    return (uint8_t)(sign | (uint8_t)quantum);
+  }
+  int exp32 = (int)(abs_bits >> 23) - 127;
+  uint32_t mant = abs_bits & 0x007fffffu;
+  uint32_t q = mant >> 20;
+  uint32_t r = mant & 0x000fffffu;
+  if (r > 0x80000u || (r == 0x80000u && (q & 1u) == 1u)) {
+    q += 1;
+    if (q == 8) {
+      q = 0;
+      exp32 += 1;
+    }
+  }
+  return (uint8_t)(sign | (uint8_t)((((uint32_t)(exp32 + 7)) << 3) | q));
+}
+
+// bits.rs:106-108
+NVO_API float nvo_e8m0_to_f32(uint8_t bits) { return bits_to_f32((uint32_t)bits << 23); }
+
+static inline float decode16(uint32_t dtype, uint16_t bits) {
+  return dtype == 0 ? nvo_f16_to_f32(bits) : nvo_bf16_to_f32(bits);
+}
+static inline uint16_t encode16(uint32_t dtype, float value) {
+  return dtype == 0 ? nvo_f32_to_f16(value) : nvo_f32_to_bf16(value);
+}
+static inline float round16(uint32_t dtype, float value) {
+  return decode16(dtype, encode16(dtype, value));
+}
+
+NVO_API void nvo_encode16(uint32_t dtype, const float *in, uint16_t *out, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) out[i] = encode16(dtype, in[i]);
+}
+NVO_API void nvo_decode16(uint32_t dtype, const uint16_t *in, float *out, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) out[i] = decode16(dtype, in[i]);
+}
+NVO_API void nvo_encode_fp8(const float *in, uint8_t *out, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) out[i] = nvo_f32_to_fp8_e4m3fn(in[i]);
+}
+NVO_API void nvo_decode_fp8(const uint8_t *in, float *out, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) out[i] = nvo_fp8_e4m3fn_to_f32(in[i]);
+}
+
+// ---------------------------------------------------------------------------
+// FNV-1a-64 over little-endian bytes (common/hash.rs:3-32, precision/bits.rs:362-371)
+// ---------------------------------------------------------------------------
+NVO_API uint64_t nvo_fnv1a(const uint8_t *bytes, uint64_t n) {
+  uint64_t hash = 0xcbf29ce484222325ull;
+  for (uint64_t i = 0; i < n; ++i) {
+    hash ^= (uint64_t)bytes[i];
+    hash *= 0x00000100000001b3ull;
+  }
+  return hash;
+}
+
+// ---------------------------------------------------------------------------
+// Block math  (precision/block/ops.rs, common/math.rs, common/rope.rs)
+// ---------------------------------------------------------------------------
+
+// ops.rs:75-91: y[r] = sum_c dec(W[r,c]) * x[c], f32, sequential.
+NVO_API void nvo_gemv_encoded(uint32_t dtype, const uint16_t *w, uint64_t rows, uint64_t cols,
+                              const float *x, float *y) {
+  for (uint64_t r = 0; r < rows; ++r) {
+    const uint16_t *row = w + r * cols;
+    float sum = 0.0f;
+    for (uint64_t c = 0; c < cols; ++c) sum += decode16(dtype, row[c]) * x[c];
+    y[r] = sum;
+  }
+}
+
+// Same loop, rows split across OpenMP threads. Used only to time the CPU baseline.
+NVO_API void nvo_gemv_encoded_mt(uint32_t dtype, const uint16_t *w, uint64_t rows, uint64_t cols,
+                                 const float *x, float *y) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < (int64_t)rows; ++r) {
+    const uint16_t *row = w + (uint64_t)r * cols;
+    float sum = 0.0f;
+    for (uint64_t c = 0; c < cols; ++c) sum += decode16(dtype, row[c]) * x[c];
+    y[r] = sum;
+  }
+}
+
+// Device-session staging of the same contract: the GEMV input is a 16-bit
+// vector (native/cuda/hf_decode_sequence/projection.cu:63-79 takes encoded
+// input; kernels.cu:147,430,610 round the producers' outputs).
+NVO_API void nvo_gemv_encoded_x16(uint32_t dtype, const uint16_t *w, uint64_t rows, uint64_t cols,
+                                  const uint16_t *x, float *y) {
+  std::vector<float> xf(cols);
+  for (uint64_t c = 0; c < cols; ++c) xf[c] = decode16(dtype, x[c]);
+  nvo_gemv_encoded(dtype, w, rows, cols, xf.data(), y);
+}
+
+// crates/nerva-cuda/src/tests/deepseek_quant.rs:689-713.
+// out[token*rows + row] = sum_c (fp8(W[row,c]) * S[row/br, c/bc]) * bf16(x[token,c])
+NVO_API void nvo_fp8_f32_scale_gemm_tokens(const uint8_t *w, const float *scales,
+                                           const uint16_t *x, uint32_t input_dtype, uint64_t rows,
+                                           uint64_t cols, uint64_t tokens, uint64_t block_rows,
+                                           uint64_t block_cols, float *out) {
+  uint64_t scale_cols = (cols + block_cols - 1) / block_cols;
+  float table[256];
+  for (int i = 0; i < 256; ++i) table[i] = nvo_fp8_e4m3fn_to_f32((uint8_t)i);
+  std::vector<float> xf(cols);
+  for (uint64_t t = 0; t < tokens; ++t) {
+    for (uint64_t c = 0; c < cols; ++c) xf[c] = decode16(input_dtype, x[t * cols + c]);
+    for (uint64_t r = 0; r < rows; ++r) {
+      float sum = 0.0f;
+      const float *srow = scales + (r / block_rows) * scale_cols;
+      for (uint64_t c = 0; c < cols; ++c) {
+        float weight = table[w[r * cols + c]] * srow[c / block_cols];
+        sum += weight * xf[c];
+      }
+      out[t * rows + r] = sum;
+    }
+  }
+}
+
+// Same contract with an f32 input vector (the MoE down projection consumes the
+// f32 SwiGLU activation: native/cuda/hf_decode_sequence/deepseek/kernels_sparse_moe.inc.cu:323-397).
+static void fp8_gemv_f32x(const uint8_t *w, const float *scales, const float *x, uint64_t rows,
+                          uint64_t cols, uint64_t block_rows, uint64_t block_cols, float *out,
+                          const float *table) {
+  uint64_t scale_cols = (cols + block_cols - 1) / block_cols;
+  for (uint64_t r = 0; r < rows; ++r) {
+    float sum = 0.0f;
+    const float *srow = scales + (r / block_rows) * scale_cols;
+    for (uint64_t c = 0; c < cols; ++c) {
+      float weight = table[w[r * cols + c]] * srow[c / block_cols];
+      sum += weight * x[c];
+    }
+    out[r] = sum;
+  }
+}
+
+// ops.rs:31-50
+NVO_API void nvo_rms_norm_encoded(uint32_t dtype, const float *x, const uint16_t *gamma, uint64_t n,
+                                  float eps, float *out) {
+  float sum = 0.0f;
+  for (uint64_t i = 0; i < n; ++i) sum += x[i] * x[i];
+  float mean_square = sum / (float)n;
+  float scale = 1.0f / sqrtf(mean_square + eps);
+  for (uint64_t i = 0; i < n; ++i) out[i] = x[i] * scale * decode16(dtype, gamma[i]);
+}
+
+// ops.rs:52-73 (gamma[head_dim] shared by all heads; same eps as the layer norm)
+NVO_API void nvo_per_head_rms_norm(uint32_t dtype, const uint16_t *gamma, uint64_t head_dim,
+                                   float *values, uint64_t n, float eps) {
+  for (uint64_t start = 0; start + head_dim <= n; start += head_dim) {
+    float *head = values + start;
+    float sum = 0.0f;
+    for (uint64_t i = 0; i < head_dim; ++i) sum += head[i] * head[i];
+    float scale = 1.0f / sqrtf(sum / (float)head_dim + eps);
+    for (uint64_t i = 0; i < head_dim; ++i) head[i] *= scale * decode16(dtype, gamma[i]);
+  }
+}
+
+// common/rope.rs:54-79 (half-split pairs (i, i+d/2); angle computed in f32)
+NVO_API void nvo_rope(uint64_t head_dim, uint64_t heads, uint64_t position, float theta,
+                      float *values) {
+  uint64_t half = head_dim / 2;
+  for (uint64_t h = 0; h < heads; ++h) {
+    float *v = values + h * head_dim;
+    for (uint64_t i = 0; i < half; ++i) {
+      float exponent = (float)(2 * i) / (float)head_dim;
+      float angle = (float)position / powf(theta, exponent);
+      float s = sinf(angle), c = cosf(angle);
+      float left = v[i], right = v[i + half];
+      v[i] = left * c - right * s;
+      v[i + half] = right * c + left * s;
+    }
+  }
+}
+
+// common/math.rs:76-82
+static inline float silu(float v) { return v / (1.0f + expf(-v)); }
+static inline float sigmoidf(float v) { return 1.0f / (1.0f + expf(-v)); }
+NVO_API float nvo_silu(float v) { return silu(v); }
+
+// common/math.rs:47-52
+static inline float dotf(const float *a, const float *b, uint64_t n) {
+  float sum = 0.0f;
+  for (uint64_t i = 0; i < n; ++i) sum += a[i] * b[i];
+  return sum;
+}
+
+// attention/exact/run.rs:13-127. KV is given as `nblocks` blocks; block b holds
+// counts[b] tokens, keys/values laid out [token][kv_heads*head_dim] f32.
+NVO_API int nvo_attention_blockwise(uint32_t heads, uint32_t kv_heads, uint32_t head_dim,
+                                    const float *query, const float *const *keys,
+                                    const float *const *values, const uint64_t *counts,
+                                    uint64_t nblocks, float *output) {
+  uint64_t hd = head_dim, kvh = (uint64_t)kv_heads * hd, group = heads / kv_heads;
+  std::vector<float> local(heads * hd, 0.0f), gm(heads, -INFINITY), gl(heads, 0.0f);
+  for (uint64_t i = 0; i < heads * hd; ++i) output[i] = 0.0f;
+  float scale = 1.0f / sqrtf((float)head_dim);
+  uint64_t total = 0;
+  for (uint64_t b = 0; b < nblocks; ++b) {
+    if (counts[b] == 0) continue;
+    total += counts[b];
+    for (uint64_t h = 0; h < heads; ++h) {
+      uint64_t kv = h / group;  // common/shape.rs kv_head_for_attention_head
+      float *lo = local.data() + h * hd;
+      for (uint64_t i = 0; i < hd; ++i) lo[i] = 0.0f;
+      float lm = -INFINITY, ll = 0.0f;
+      for (uint64_t t = 0; t < counts[b]; ++t) {
+        const float *k = keys[b] + t * kvh + kv * hd;
+        const float *v = values[b] + t * kvh + kv * hd;
+        float score = dotf(query + h * hd, k, hd) * scale;
+        float next_m = fmaxf(lm, score);
+        float old_scale = ll == 0.0f ? 0.0f : expf(lm - next_m);
+        float new_scale = expf(score - next_m);
+        for (uint64_t i = 0; i < hd; ++i) lo[i] = lo[i] * old_scale + v[i] * new_scale;
+        ll = ll * old_scale + new_scale;
+        lm = next_m;
+      }
+      float next_m = fmaxf(gm[h], lm);
+      float global_scale = gl[h] == 0.0f ? 0.0f : expf(gm[h] - next_m);
+      float local_scale = expf(lm - next_m);
+      float *go = output + h * hd;
+      for (uint64_t i = 0; i < hd; ++i) go[i] = go[i] * global_scale + lo[i] * local_scale;
+      gl[h] = gl[h] * global_scale + ll * local_scale;
+      gm[h] = next_m;
+    }
+  }
+  if (total == 0) return -1;
+  for (uint64_t h = 0; h < heads; ++h) {
+    if (gl[h] == 0.0f || !isfinite(gl[h])) return -1;
+    for (uint64_t i = 0; i < hd; ++i) output[h * hd + i] /= gl[h];
+  }
+  return 0;
+}
+
+// Paged 16-bit KV variant of the same recurrence: the device session reads every
+// key/value back from the cache as 16-bit (kernels.cu:387-390, 404-423), with
+// element index (((layer*n_blocks + table[t/B])*B + t%B)*kv_hidden + kv_off)
+// (types.cuh:328-337). `kv_tokens` keys are visible (0..kv_tokens-1).
+NVO_API int nvo_attention_paged16(uint32_t dtype, uint32_t heads, uint32_t kv_heads,
+                                  uint32_t head_dim, uint32_t block_tokens, const float *query,
+                                  const uint16_t *kcache, const uint16_t *vcache,
+                                  const uint32_t *table, uint64_t layer, uint64_t n_blocks,
+                                  uint64_t kv_tokens, float *output) {
+  uint64_t hd = head_dim, kvh = (uint64_t)kv_heads * hd, group = heads / kv_heads;
+  if (kv_tokens == 0) return -1;
+  float scale = 1.0f / sqrtf((float)head_dim);
+  std::vector<float> kf(hd), vf(hd);
+  for (uint64_t h = 0; h < heads; ++h) {
+    uint64_t kv = h / group;
+    float *o = output + h * hd;
+    for (uint64_t i = 0; i < hd; ++i) o[i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    for (uint64_t t = 0; t < kv_tokens; ++t) {
+      uint64_t base =
+          (((layer * n_blocks + table[t / block_tokens]) * block_tokens + t % block_tokens) * kvh) +
+          kv * hd;
+      for (uint64_t i = 0; i < hd; ++i) {
+        kf[i] = decode16(dtype, kcache[base + i]);
+        vf[i] = decode16(dtype, vcache[base + i]);
+      }
+      float score = dotf(query + h * hd, kf.data(), hd) * scale;
+      float next_m = fmaxf(m, score);
+      float old_scale = l == 0.0f ? 0.0f : expf(m - next_m);
+      float new_scale = expf(score - next_m);
+      for (uint64_t i = 0; i < hd; ++i) o[i] = o[i] * old_scale + vf[i] * new_scale;
+      l = l * old_scale + new_scale;
+      m = next_m;
+    }
+    if (l == 0.0f || !isfinite(l)) return -1;
+    for (uint64_t i = 0; i < hd; ++i) o[i] /= l;
+  }
+  return 0;
+}
+
+// common/token.rs:33-58: first maximum (strict >). Returns -1 on empty input or
+// any non-finite logit (CPU contract). `skip_nonfinite` selects the device
+// sampler's rule instead (sampler.cu:89-119, 35-40: non-finite candidates are
+// skipped; value desc, index asc).
+NVO_API int nvo_greedy_argmax(const float *logits, uint64_t n, int skip_nonfinite, uint32_t *out) {
+  if (n == 0) return -1;
+  if (!skip_nonfinite) {
+    if (!isfinite(logits[0])) return -1;
+    uint64_t best = 0;
+    float best_value = logits[0];
+    for (uint64_t i = 1; i < n; ++i) {
+      if (!isfinite(logits[i])) return -1;
+      if (logits[i] > best_value) {
+        best = i;
+        best_value = logits[i];
+      }
+    }
+    *out = (uint32_t)best;
+    return 0;
+  }
+  int found = 0;
+  uint64_t best = 0;
+  float best_value = 0.0f;
+  for (uint64_t i = 0; i < n; ++i) {
+    if (!isfinite(logits[i])) continue;
+    if (!found || logits[i] > best_value) {
+      found = 1;
+      best = i;
+      best_value = logits[i];
+    }
+  }
+  *out = (uint32_t)best;
+  return found ? 0 : -1;
+}
+
+// ---------------------------------------------------------------------------
+// MoE  (precision/block/moe.rs:1107-1155,1254-1326; reference/moe.rs:76-166)
+// ---------------------------------------------------------------------------
+
+// Softmax route: p = softmax(logits) (max-subtracted), top-k by (p desc via
+// total order, index asc), optional renormalisation of the selected weights.
+NVO_API int nvo_moe_route_softmax(const float *logits, uint32_t num_experts, uint32_t top_k,
+                                  uint32_t normalize, uint32_t *ids, float *weights) {
+  if (top_k == 0 || top_k > num_experts) return -1;
+  float maxv = -INFINITY;
+  for (uint32_t i = 0; i < num_experts; ++i) {
+    if (!isfinite(logits[i])) return -1;
+    maxv = fmaxf(maxv, logits[i]);
+  }
+  std::vector<float> probs(num_experts);
+  for (uint32_t i = 0; i < num_experts; ++i) probs[i] = expf(logits[i] - maxv);
+  float sum = 0.0f;
+  for (uint32_t i = 0; i < num_experts; ++i) sum += probs[i];
+  if (sum > 0.0f && isfinite(sum))
+    for (uint32_t i = 0; i < num_experts; ++i) probs[i] /= sum;
+  std::vector<uint32_t> order(num_experts);
+  for (uint32_t i = 0; i < num_experts; ++i) order[i] = i;
+  // probabilities are finite and >= 0, so total_cmp order == numeric order
+  std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+    if (probs[a] != probs[b]) return probs[a] > probs[b];
+    return a < b;
+  });
+  float selected_sum = 0.0f;
+  for (uint32_t k = 0; k < top_k; ++k) {
+    ids[k] = order[k];
+    weights[k] = probs[order[k]];
+    selected_sum += weights[k];
+  }
+  if (normalize && selected_sum > 0.0f && isfinite(selected_sum))
+    for (uint32_t k = 0; k < top_k; ++k) weights[k] /= selected_sum;
+  return 0;
+}
+
+// reference/moe.rs:121-139
+static inline float swiglu(float gate, float up, int clamp, float limit) {
+  if (clamp) {
+    float g = fminf(gate, limit);
+    float u = fminf(fmaxf(up, -limit), limit);
+    return silu(g) * u;
+  }
+  return silu(gate) * up;
+}
+
+// reference/moe.rs:76-119 (+ shared expert :141-166 when shared_* are non-null).
+// w_gate/w_up [E][I][H], w_down [E][H][I], f32.
+NVO_API int nvo_moe_forward_f32(uint32_t hidden, uint32_t inter, uint32_t num_experts,
+                                uint32_t top_k, uint32_t clamp, float limit, const float *input,
+                                const uint32_t *expert_ids, const float *expert_weights,
+                                const float *w_gate, const float *w_up, const float *w_down,
+                                uint32_t shared_inter, const float *shared_gate,
+                                const float *shared_up, const float *shared_down, float *output) {
+  for (uint32_t i = 0; i < hidden; ++i) output[i] = 0.0f;
+  std::vector<float> act(std::max(inter, shared_inter));
+  uint64_t stride = (uint64_t)inter * hidden;
+  for (uint32_t k = 0; k < top_k; ++k) {
+    uint32_t e = expert_ids[k];
+    if (e >= num_experts) return -1;
+    for (uint32_t r = 0; r < inter; ++r) {
+      float g = dotf(w_gate + e * stride + (uint64_t)r * hidden, input, hidden);
+      float u = dotf(w_up + e * stride + (uint64_t)r * hidden, input, hidden);
+      act[r] = swiglu(g, u, (int)clamp, limit);
+    }
+    for (uint32_t h = 0; h < hidden; ++h)
+      output[h] += expert_weights[k] * dotf(w_down + e * stride + (uint64_t)h * inter, act.data(), inter);
+  }
+  if (shared_gate != nullptr) {
+    for (uint32_t r = 0; r < shared_inter; ++r) {
+      float g = dotf(shared_gate + (uint64_t)r * hidden, input, hidden);
+      float u = dotf(shared_up + (uint64_t)r * hidden, input, hidden);
+      act[r] = swiglu(g, u, (int)clamp, limit);
+    }
+    for (uint32_t h = 0; h < hidden; ++h)
+      output[h] += dotf(shared_down + (uint64_t)h * shared_inter, act.data(), shared_inter);
+  }
+  return 0;
+}
+
+// FP8 block-scaled experts: the same expert loop as nvo_moe_forward_f32 with
+// every dot product replaced by the block-scaled FP8 contract
+// (deepseek_quant.rs:689-713). Expert e's tensors start at e*rows*cols bytes
+// and e*ceil(rows/br)*ceil(cols/bc) scales. The input is a 16-bit vector; the
+// SwiGLU activation stays f32 into the down projection. The shared expert
+// (index `shared_index` into the same tensors, or < 0 for none) has weight 1.
+NVO_API int nvo_moe_fp8_forward(uint32_t hidden, uint32_t inter, uint32_t num_experts,
+                                uint32_t top_k, uint32_t block, uint32_t input_dtype,
+                                const uint16_t *input, const uint32_t *expert_ids,
+                                const float *expert_weights, const uint8_t *w_gate,
+                                const float *s_gate, const uint8_t *w_up, const float *s_up,
+                                const uint8_t *w_down, const float *s_down, int32_t shared_index,
+                                int threads, float *output) {
+  float table[256];
+  for (int i = 0; i < 256; ++i) table[i] = nvo_fp8_e4m3fn_to_f32((uint8_t)i);
+  uint64_t gu_scales = (uint64_t)((inter + block - 1) / block) * ((hidden + block - 1) / block);
+  uint64_t dn_scales = (uint64_t)((hidden + block - 1) / block) * ((inter + block - 1) / block);
+  uint64_t stride = (uint64_t)inter * hidden;
+  std::vector<float> x(hidden);
+  for (uint32_t i = 0; i < hidden; ++i) x[i] = decode16(input_dtype, input[i]);
+  for (uint32_t i = 0; i < hidden; ++i) output[i] = 0.0f;
+  uint32_t total = top_k + (shared_index >= 0 ? 1u : 0u);
+  std::vector<float> g(inter), u(inter), act(inter), down(hidden);
+  (void)threads;
+  for (uint32_t k = 0; k < total; ++k) {
+    uint32_t e = k < top_k ? expert_ids[k] : (uint32_t)shared_index;
+    float weight = k < top_k ? expert_weights[k] : 1.0f;
+    if (e >= num_experts) return -1;
+    fp8_gemv_f32x(w_gate + e * stride, s_gate + e * gu_scales, x.data(), inter, hidden, block,
+                  block, g.data(), table);
+    fp8_gemv_f32x(w_up + e * stride, s_up + e * gu_scales, x.data(), inter, hidden, block, block,
+                  u.data(), table);
+    for (uint32_t r = 0; r < inter; ++r) act[r] = silu(g[r]) * u[r];
+    fp8_gemv_f32x(w_down + e * stride, s_down + e * dn_scales, act.data(), hidden, inter, block,
+                  block, down.data(), table);
+    for (uint32_t h = 0; h < hidden; ++h) output[h] += weight * down[h];
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Dense model: block forward, prefill, greedy loop.
+// ---------------------------------------------------------------------------
+
+typedef struct NvoLayer {
+  const uint16_t *rms_attn, *rms_mlp;
+  const uint16_t *w_q, *w_k, *w_v, *w_o;
+  const uint16_t *q_norm, *k_norm;           // optional [head_dim]
+  const uint16_t *q_bias, *k_bias, *v_bias, *o_bias;  // optional
+  const uint16_t *w_gate, *w_up, *w_down;
+} NvoLayer;
+
+typedef struct NvoModel {
+  uint32_t dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab, layers;
+  float rms_eps, rope_theta;  // rope_theta <= 0 disables RoPE
+  const uint16_t *embeddings;
+  const NvoLayer *layer;
+  const uint16_t *final_norm;
+  const uint16_t *lm_head;
+} NvoModel;
+
+// staging 0: the Rust CPU reference (f32 inside a block, f32 KV, hidden encoded
+//            to 16 bits at every block boundary: kv_finish.rs:74, kv.rs:140-141).
+// staging 1: the device session (Appendix of the design notes): GEMV inputs and
+//            KV are 16-bit, GEMV outputs/norms/softmax f32; the residual stream
+//            stays f32 across layers for decode tokens (kernels.cu:661-663) and
+//            is encoded per layer for prompt tokens (prefill_kernels.cu:494-508).
+struct NvoContext {
+  NvoModel m;
+  int staging;
+  uint64_t max_ctx;
+  uint64_t len;                       // tokens in KV
+  std::vector<std::vector<float>> kf, vf;        // staging 0: [layer][t*kvh]
+  std::vector<std::vector<uint16_t>> k16, v16;   // staging 1
+  std::vector<float> logits;
+  int threads;
+};
+
+static void gemv_auto(const NvoContext *c, const uint16_t *w, uint64_t rows, uint64_t cols,
+                      const float *x, float *y) {
+  if (c->threads > 1)
+    nvo_gemv_encoded_mt(c->m.dtype, w, rows, cols, x, y);
+  else
+    nvo_gemv_encoded(c->m.dtype, w, rows, cols, x, y);
+}
+
+static void add_bias(uint32_t dtype, const uint16_t *bias, float *v, uint64_t n) {
+  if (bias == nullptr) return;
+  for (uint64_t i = 0; i < n; ++i) v[i] += decode16(dtype, bias[i]);  // ops.rs:93-99
+}
+
+static void round_vec(uint32_t dtype, float *v, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) v[i] = round16(dtype, v[i]);
+}
+
+// One transformer block for a token rotated at `rope_pos` and stored at KV slot
+// `pos` (== number of tokens already in this layer's KV). x: f32[hidden] in, f32[hidden] out.
+// Order: kv.rs:96-205 (norm, q/k/v projections, bias, per-head norm, RoPE,
+// append, attention over 0..pos) then kv_finish.rs:10-75.
+static int block_forward(NvoContext *c, uint32_t l, uint64_t rope_pos, uint64_t pos, int prompt_token,
+                         float *x) {
+  const NvoModel &m = c->m;
+  const NvoLayer &w = m.layer[l];
+  uint64_t H = m.hidden, A = (uint64_t)m.heads * m.head_dim, KV = (uint64_t)m.kv_heads * m.head_dim;
+  uint64_t I = m.intermediate;
+  std::vector<float> n(H), q(A), k(KV), v(KV), attn(A), r(H), mn(H), g(I), u(I), ff(I), d(H);
+  nvo_rms_norm_encoded(m.dtype, x, w.rms_attn, H, m.rms_eps, n.data());
+  if (c->staging == 1) round_vec(m.dtype, n.data(), H);
+  gemv_auto(c, w.w_q, A, H, n.data(), q.data());
+  gemv_auto(c, w.w_k, KV, H, n.data(), k.data());
+  gemv_auto(c, w.w_v, KV, H, n.data(), v.data());
+  add_bias(m.dtype, w.q_bias, q.data(), A);
+  add_bias(m.dtype, w.k_bias, k.data(), KV);
+  add_bias(m.dtype, w.v_bias, v.data(), KV);
+  if (w.q_norm) nvo_per_head_rms_norm(m.dtype, w.q_norm, m.head_dim, q.data(), A, m.rms_eps);
+  if (w.k_norm) nvo_per_head_rms_norm(m.dtype, w.k_norm, m.head_dim, k.data(), KV, m.rms_eps);
+  if (m.rope_theta > 0.0f) {
+    nvo_rope(m.head_dim, m.heads, rope_pos, m.rope_theta, q.data());
+    nvo_rope(m.head_dim, m.kv_heads, rope_pos, m.rope_theta, k.data());
+  }
+  if (pos >= c->max_ctx) return -1;
+  int rc;
+  if (c->staging == 0) {
+    memcpy(c->kf[l].data() + pos * KV, k.data(), KV * 4);
+    memcpy(c->vf[l].data() + pos * KV, v.data(), KV * 4);
+    const float *kp = c->kf[l].data(), *vp = c->vf[l].data();
+    uint64_t count = pos + 1;
+    rc = nvo_attention_blockwise(m.heads, m.kv_heads, m.head_dim, q.data(), &kp, &vp, &count, 1,
+                                 attn.data());
+  } else {
+    for (uint64_t i = 0; i < KV; ++i) {
+      c->k16[l][pos * KV + i] = encode16(m.dtype, k[i]);
+      c->v16[l][pos * KV + i] = encode16(m.dtype, v[i]);
+    }
+    // contiguous cache == identity block table with one block spanning max_ctx
+    uint32_t table0 = 0;
+    rc = nvo_attention_paged16(m.dtype, m.heads, m.kv_heads, m.head_dim, (uint32_t)c->max_ctx,
+                               q.data(), c->k16[l].data(), c->v16[l].data(), &table0, 0, 1,
+                               pos + 1, attn.data());
+    round_vec(m.dtype, attn.data(), A);
+  }
+  if (rc != 0) return rc;
+  gemv_auto(c, w.w_o, H, A, attn.data(), r.data());
+  add_bias(m.dtype, w.o_bias, r.data(), H);
+  for (uint64_t i = 0; i < H; ++i) r[i] += x[i];
+  nvo_rms_norm_encoded(m.dtype, r.data(), w.rms_mlp, H, m.rms_eps, mn.data());
+  if (c->staging == 1) round_vec(m.dtype, mn.data(), H);
+  gemv_auto(c, w.w_gate, I, H, mn.data(), g.data());
+  gemv_auto(c, w.w_up, I, H, mn.data(), u.data());
+  for (uint64_t i = 0; i < I; ++i) ff[i] = silu(g[i]) * u[i];
+  if (c->staging == 1) round_vec(m.dtype, ff.data(), I);
+  gemv_auto(c, w.w_down, H, I, ff.data(), d.data());
+  for (uint64_t i = 0; i < H; ++i) x[i] = r[i] + d[i];
+  if (c->staging == 0 || prompt_token) round_vec(m.dtype, x, H);
+  return 0;
+}
+
+NVO_API NvoContext *nvo_ctx_create(const NvoModel *model, uint64_t max_ctx, int staging,
+                                   int threads) {
+  NvoContext *c = new NvoContext();
+  c->m = *model;
+  c->staging = staging;
+  c->max_ctx = max_ctx;
+  c->len = 0;
+  c->threads = threads;
+  uint64_t KV = (uint64_t)model->kv_heads * model->head_dim;
+  if (staging == 0) {
+    c->kf.assign(model->layers, std::vector<float>(max_ctx * KV));
+    c->vf.assign(model->layers, std::vector<float>(max_ctx * KV));
+  } else {
+    c->k16.assign(model->layers, std::vector<uint16_t>(max_ctx * KV));
+    c->v16.assign(model->layers, std::vector<uint16_t>(max_ctx * KV));
+  }
+  c->logits.resize(model->vocab);
+  return c;
+}
+
+NVO_API void nvo_ctx_destroy(NvoContext *c) { delete c; }
+NVO_API void nvo_ctx_reset(NvoContext *c) { c->len = 0; }
+NVO_API uint64_t nvo_ctx_len(const NvoContext *c) { return c->len; }
+NVO_API const float *nvo_ctx_logits(const NvoContext *c) { return c->logits.data(); }
+
+// Install externally produced 16-bit KV for one layer (staging 1), tokens
+// [0, tokens) laid out [token][kv_hidden]. Lets the CPU baseline time decode
+// steps on a long context without running a CPU prefill.
+NVO_API int nvo_ctx_load_kv16(NvoContext *c, uint32_t layer, const uint16_t *k, const uint16_t *v,
+                              uint64_t tokens) {
+  if (c->staging != 1 || layer >= c->m.layers || tokens > c->max_ctx) return -1;
+  uint64_t KV = (uint64_t)c->m.kv_heads * c->m.head_dim;
+  memcpy(c->k16[layer].data(), k, tokens * KV * 2);
+  memcpy(c->v16[layer].data(), v, tokens * KV * 2);
+  return 0;
+}
+NVO_API void nvo_ctx_set_len(NvoContext *c, uint64_t len) { c->len = len; }
+
+// Read back this context's KV row (staging 1) for tests.
+NVO_API int nvo_ctx_read_kv16(const NvoContext *c, uint32_t layer, uint64_t token, uint16_t *k,
+                              uint16_t *v) {
+  if (c->staging != 1 || layer >= c->m.layers || token >= c->len) return -1;
+  uint64_t KV = (uint64_t)c->m.kv_heads * c->m.head_dim;
+  memcpy(k, c->k16[layer].data() + token * KV, KV * 2);
+  memcpy(v, c->v16[layer].data() + token * KV, KV * 2);
+  return 0;
+}
+
+// Forward one token at position c->len through every layer; optionally produce
+// logits (final norm + lm_head; causal_lm/decode.rs:82-101). `hidden_out`
+// (optional) receives the f32 hidden state after the last layer.
+NVO_API int nvo_ctx_forward_token(NvoContext *c, uint32_t token, int prompt_token, int want_logits,
+                                  float *hidden_out) {
+  const NvoModel &m = c->m;
+  if (token >= m.vocab) return -1;
+  uint64_t H = m.hidden;
+  std::vector<float> x(H);
+  for (uint64_t i = 0; i < H; ++i) x[i] = decode16(m.dtype, m.embeddings[(uint64_t)token * H + i]);
+  uint64_t pos = c->len;
+  for (uint32_t l = 0; l < m.layers; ++l) {
+    int rc = block_forward(c, l, pos, pos, prompt_token, x.data());
+    if (rc != 0) return rc;
+  }
+  c->len = pos + 1;
+  if (hidden_out) memcpy(hidden_out, x.data(), H * 4);
+  if (want_logits) {
+    std::vector<float> n(H);
+    nvo_rms_norm_encoded(m.dtype, x.data(), m.final_norm, H, m.rms_eps, n.data());
+    if (c->staging == 1) round_vec(m.dtype, n.data(), H);
+    gemv_auto(c, m.lm_head, m.vocab, H, n.data(), c->logits.data());
+  }
+  return 0;
+}
+
+// causal_lm/context.rs:41-120: prefill all prompt tokens, sample token 0, then
+// embed(token) -> layers -> final norm -> lm_head -> argmax per step; stop after
+// emitting `eos_token` when has_eos. Returns the number of tokens written.
+// margins (optional, [steps]) receives top1-top2 logit margin per emitted token.
+NVO_API int nvo_greedy_decode(NvoContext *c, const uint32_t *prompt, uint32_t prompt_count,
+                              uint32_t steps, uint32_t has_eos, uint32_t eos_token,
+                              uint32_t *out_tokens, float *margins) {
+  if (prompt_count == 0 || steps == 0) return -1;
+  c->len = 0;
+  for (uint32_t i = 0; i < prompt_count; ++i) {
+    int rc = nvo_ctx_forward_token(c, prompt[i], 1, i + 1 == prompt_count, nullptr);
+    if (rc != 0) return -1;
+  }
+  uint32_t produced = 0;
+  for (;;) {
+    uint32_t token = 0;
+    int rc = nvo_greedy_argmax(c->logits.data(), c->m.vocab, c->staging == 1, &token);
+    if (rc != 0) return -1;
+    if (margins) {
+      float best = c->logits[token], second = -INFINITY;
+      for (uint32_t i = 0; i < c->m.vocab; ++i)
+        if (i != token && isfinite(c->logits[i])) second = fmaxf(second, c->logits[i]);
+      margins[produced] = best - second;
+    }
+    out_tokens[produced++] = token;
+    if ((has_eos && token == eos_token) || produced == steps) break;
+    rc = nvo_ctx_forward_token(c, token, 0, 1, nullptr);
+    if (rc != 0) return -1;
+  }
+  return (int)produced;
+}
+
+// Single block forward as the one-shot block probe exposes it
+// (crates/nerva-cuda/src/tests/block.rs:58-108): 16-bit input and output, fresh KV.
+NVO_API int nvo_block_forward(const NvoModel *model, const uint16_t *input, uint64_t position,
+                              int staging, uint16_t *output) {
+  NvoModel one = *model;
+  one.layers = 1;
+  NvoContext *c = nvo_ctx_create(&one, 1, staging, 1);
+  uint64_t H = one.hidden;
+  std::vector<float> x(H);
+  for (uint64_t i = 0; i < H; ++i) x[i] = decode16(one.dtype, input[i]);
+  // tokens before `position` are not visible in the probe: it attends to itself only.
+  int rc = block_forward(c, 0, position, 0, 1, x.data());
+  for (uint64_t i = 0; i < H; ++i) output[i] = encode16(one.dtype, x[i]);
+  nvo_ctx_destroy(c);
+  return rc;
+}
+
+// ---------------------------------------------------------------------------
+// Synthetic tensors. Not a reference function: a counter-based generator that
+// host and device evaluate bit-identically (integer hash, one exact int->float
+// conversion, one f32 multiply, one f32 add, then RNE to 16 bits).
+//   u   = 12 sixteen-bit fields of three splitmix64 outputs, summed (Irwin-Hall n=12)
+//   val = mean + float(2*sum - 786420) * (std / 131072)        [std of the sum = 65536]
+// ---------------------------------------------------------------------------
+static inline uint64_t splitmix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+static inline uint64_t tensor_key(uint64_t seed, uint64_t tensor_id) {
+  return splitmix64(seed ^ (tensor_id * 0xD6E8FEB86659FD93ull));
+}
+static inline float synth_value(uint64_t key, uint64_t index, float mean, float scale) {
+  uint32_t sum = 0;
+  for (int j = 0; j < 3; ++j) {
+    uint64_t h = splitmix64(key + (3 * index + (uint64_t)j) * 0x9E3779B97F4A7C15ull);
+    sum += (uint32_t)(h & 0xffff) + (uint32_t)((h >> 16) & 0xffff) +
+           (uint32_t)((h >> 32) & 0xffff) + (uint32_t)(h >> 48);
+  }
+  int32_t centered = (int32_t)(2 * sum) - 786420;
+  float scaled = (float)centered * scale;
+  return mean + scaled;
+}
+NVO_API float nvo_synth_scale(float std) { return std / 131072.0f; }
+NVO_API void nvo_synth_f32(uint64_t seed, uint64_t tensor_id, uint64_t offset, uint64_t n,
+                           float mean, float std, float *out) {
+  uint64_t key = tensor_key(seed, tensor_id);
+  float scale = nvo_synth_scale(std);
+  for (uint64_t i = 0; i < n; ++i) out[i] = synth_value(key, offset + i, mean, scale);
+}
+NVO_API void nvo_synth_16(uint32_t dtype, uint64_t seed, uint64_t tensor_id, uint64_t offset,
+                          uint64_t n, float mean, float std, uint16_t *out) {
+  uint64_t key = tensor_key(seed, tensor_id);
+  float scale = nvo_synth_scale(std);
+  for (uint64_t i = 0; i < n; ++i) out[i] = encode16(dtype, synth_value(key, offset + i, mean, scale));
+}
+NVO_API void nvo_synth_tokens(uint64_t seed, uint64_t tensor_id, uint64_t n, uint32_t vocab,
+                              uint32_t *out) {
+  uint64_t key = tensor_key(seed, tensor_id);
+  for (uint64_t i = 0; i < n; ++i)
+    out[i] = (uint32_t)(splitmix64(key + i * 0x9E3779B97F4A7C15ull) % vocab);
+}
+// FP8 tensor [rows x cols] quantised per block: S = amax/448 (f32 divide),
+// q = e4m3_rne(w / S); S = 1 for an all-zero block.
+NVO_API void nvo_synth_fp8_block(uint64_t seed, uint64_t tensor_id, uint64_t rows, uint64_t cols,
+                                 uint64_t block, float std, uint8_t *w, float *scales) {
+  uint64_t key = tensor_key(seed, tensor_id);
+  float scale = nvo_synth_scale(std);
+  uint64_t sc = (cols + block - 1) / block, sr = (rows + block - 1) / block;
+  for (uint64_t br = 0; br < sr; ++br)
+    for (uint64_t bc = 0; bc < sc; ++bc) {
+      float amax = 0.0f;
+      uint64_t r1 = std::min(rows, (br + 1) * block), c1 = std::min(cols, (bc + 1) * block);
+      for (uint64_t r = br * block; r < r1; ++r)
+        for (uint64_t c = bc * block; c < c1; ++c)
+          amax = fmaxf(amax, fabsf(synth_value(key, r * cols + c, 0.0f, scale)));
+      float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+      scales[br * sc + bc] = s;
+      for (uint64_t r = br * block; r < r1; ++r)
+        for (uint64_t c = bc * block; c < c1; ++c)
+          w[r * cols + c] = nvo_f32_to_fp8_e4m3fn(synth_value(key, r * cols + c, 0.0f, scale) / s);
+    }
+}

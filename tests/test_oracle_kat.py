@@ -1,0 +1,451 @@
+"""The CPU oracle against every known-answer vector the reference's tests hold
+for this path (tests/golden/kat.json), plus checks the mathematics fixes."""
+import math
+
+import numpy as np
+import pytest
+
+import oracle as O
+from conftest import hx
+
+
+def test_f16_bf16_codecs(kat):
+    for value, bits in kat["f16_encode"]["cases"]:
+        assert O.lib.nvo_f32_to_f16(value) == hx(bits)
+    for bits, value in kat["f16_decode"]["cases"]:
+        assert O.lib.nvo_f16_to_f32(hx(bits)) == value
+    for value, bits in kat["bf16_encode"]["cases"]:
+        assert O.lib.nvo_f32_to_bf16(value) == hx(bits)
+    for bits, value in kat["bf16_decode"]["cases"]:
+        assert O.lib.nvo_bf16_to_f32(hx(bits)) == value
+
+
+def test_f16_codec_against_numpy_exhaustive():
+    bits = np.arange(65536, dtype=np.uint16)
+    ours = O.decode16(O.F16, bits)
+    ref = bits.view(np.float16).astype(np.float32)
+    finite = np.isfinite(ref)
+    assert np.array_equal(ours[finite].view(np.uint32), ref[finite].view(np.uint32))
+    assert np.all(np.isnan(ours[np.isnan(ref)]))
+    # encode: every finite f16 value round-trips, and random f32 agree with numpy RNE
+    assert np.array_equal(O.encode16(O.F16, ref[finite]), bits[finite])
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(200000) * np.exp(rng.uniform(-12, 12, 200000))).astype(np.float32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(O.encode16(O.F16, x), x.astype(np.float16).view(np.uint16))
+
+
+def test_bf16_codec_rne_against_integer_model():
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(200000) * np.exp(rng.uniform(-30, 30, 200000))).astype(np.float32)
+    got = O.encode16(O.BF16, x)
+    # independent model: nearest bf16 by exhaustive neighbour comparison in f64
+    lo = (x.view(np.uint32) >> 16).astype(np.uint32)
+    cand = np.stack([lo, lo + 1]).astype(np.uint32)
+    vals = (cand << 16).view(np.float32).astype(np.float64)
+    err = np.abs(vals - x.astype(np.float64))
+    pick_hi = (err[1] < err[0]) | ((err[1] == err[0]) & (cand[0] & 1 == 1))
+    want = np.where(pick_hi, cand[1], cand[0]).astype(np.uint16)
+    assert np.array_equal(got, want)
+    # decode is the exact widening
+    b = np.arange(65536, dtype=np.uint16)
+    assert np.array_equal(O.decode16(O.BF16, b).view(np.uint32), b.astype(np.uint32) << 16)
+
+
+def test_fp8_decode_table(kat):
+    k = kat["fp8_decode"]
+    for bits, value in k["cases"]:
+        assert O.lib.nvo_fp8_e4m3fn_to_f32(hx(bits)) == value
+    for bits in k["nan"]:
+        assert math.isnan(O.lib.nvo_fp8_e4m3fn_to_f32(hx(bits)))
+    z = O.lib.nvo_fp8_e4m3fn_to_f32(hx(k["negative_zero"]))
+    assert z == 0.0 and math.copysign(1.0, z) == -1.0
+
+
+def test_fp8_decode_closed_form_all_codes():
+    for code in range(256):
+        s = -1.0 if code & 0x80 else 1.0
+        e, m = (code >> 3) & 15, code & 7
+        got = O.lib.nvo_fp8_e4m3fn_to_f32(code)
+        if e == 15 and m == 7:
+            assert math.isnan(got)
+        elif e == 0:
+            assert got == s * m * 2.0 ** -9
+        else:
+            assert got == s * (1 + m / 8) * 2.0 ** (e - 7)
+
+
+def test_fp8_encode(kat):
+    k = kat["fp8_encode"]
+    dec = lambda c: O.lib.nvo_fp8_e4m3fn_to_f32(c)
+    enc = lambda v: O.lib.nvo_f32_to_fp8_e4m3fn(v)
+    lo, hi = (hx(v) for v in k["round_trip_codes"])
+    for code in range(lo, hi + 1):
+        assert enc(dec(code)) == code
+    for a, b in k["tie_ranges"]:
+        for low in range(hx(a), hx(b) + 1):
+            mid = (dec(low) + dec(low + 1)) / 2.0
+            assert enc(mid) == (low if low & 1 == 0 else low + 1)
+    for value, bits in k["special"]:
+        v = float(value) if isinstance(value, str) else value
+        assert enc(v) == hx(bits), (value, bits)
+
+
+def test_fp8_encode_nearest_brute_force():
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal(50000) * np.exp(rng.uniform(-8, 6, 50000))).astype(np.float32)
+    x = x[np.abs(x) <= 448]
+    codes = np.array([c for c in range(256) if (c & 0x7f) != 0x7f], np.uint8)
+    table = O.decode_fp8(codes).astype(np.float64)
+    got = O.decode_fp8(O.encode_fp8(x)).astype(np.float64)
+    best = np.min(np.abs(table[None, :] - x[:, None].astype(np.float64)), axis=1)
+    assert np.array_equal(np.abs(got - x), best)
+
+
+def test_e8m0(kat):
+    for bits, f32bits in kat["e8m0"]["cases"]:
+        assert np.float32(O.lib.nvo_e8m0_to_f32(hx(bits))).view(np.uint32) == hx(f32bits)
+    assert math.isinf(O.lib.nvo_e8m0_to_f32(hx(kat["e8m0"]["inf"])))
+
+
+def test_fp8_block_dequant(kat):
+    k = kat["fp8_block_dequant"]
+    w = np.array([hx(v) for v in k["weights"]], np.uint8).reshape(k["rows"], k["cols"])
+    s = np.array([O.lib.nvo_e8m0_to_f32(hx(v)) for v in k["e8m0_scales"]], np.float32).reshape(2, 2)
+    deq = O.decode_fp8(w) * np.repeat(np.repeat(s, k["block_rows"], 0), k["block_cols"], 1)[:k["rows"], :k["cols"]]
+    assert deq.ravel().tolist() == k["expected"]
+
+
+def test_fp8_f32_scale_matvec(kat):
+    k = kat["fp8_f32_scale_matvec"]
+    w = np.array([hx(v) for v in k["weights"]], np.uint8)
+    x16 = O.encode16(O.BF16, np.array(k["input"], np.float32))
+    y = O.fp8_gemm_tokens(w, k["scales"], x16, k["rows"], k["cols"], 1, k["block_rows"], k["block_cols"])
+    assert y[0].tolist() == k["expected"]
+
+
+def test_fp8_gemm_tokens_ragged_vs_f64(kat):
+    k = kat["fp8_gemm_tokens_ragged"]
+    rows, cols, tokens = k["rows"], k["cols"], k["tokens"]
+    pat = [hx(v) for v in k["weight_pattern"]]
+    w = np.array([pat[i % len(pat)] for i in range(rows * cols)], np.uint8)
+    x = np.array([((i % 17) - 8) / 32 for i in range(tokens * cols)], np.float32)
+    x16 = O.encode16(O.BF16, x)
+    s = np.array(k["scales"], np.float32)
+    y = O.fp8_gemm_tokens(w, s, x16, rows, cols, tokens, k["block_rows"], k["block_cols"])
+    wf = O.decode_fp8(w).reshape(rows, cols).astype(np.float64)
+    sf = np.repeat(np.repeat(s.reshape(2, 2), 128, 0), 128, 1)[:rows, :cols]
+    ref = O.decode16(O.BF16, x16).reshape(tokens, cols).astype(np.float64) @ (wf * sf).T
+    assert np.max(np.abs(y - ref)) < k["abs_tol"]
+
+
+def test_fnv1a_known_hashes(kat):
+    # token hash published with the real-checkpoint parity artifact
+    k = kat["token_parity_real_checkpoint"]
+    assert O.fnv1a(np.array(k["tokens"], np.uint32)) == int(k["hash"])
+    # 16-bit output hash of the f16 block probe
+    b = kat["block_f16"]
+    assert O.fnv1a(np.array(b["output_bits"], np.uint16)) == int(b["output_hash"])
+    assert O.fnv1a(np.zeros(0, np.uint8)) == 0xcbf29ce484222325
+
+
+def test_gemv_vs_f64_and_transposition():
+    rng = np.random.default_rng(3)
+    rows, cols = 37, 53
+    w = O.encode16(O.BF16, rng.normal(0, 0.02, (rows, cols)))
+    x = rng.standard_normal(cols).astype(np.float32)
+    y = O.gemv(O.BF16, w, x)
+    ref = O.decode16(O.BF16, w).astype(np.float64) @ x.astype(np.float64)
+    assert np.allclose(y, ref, rtol=0, atol=1e-6)
+    # a transposed operand or dropped column would fail this one
+    e = np.zeros(cols, np.float32)
+    e[7] = 1.0
+    assert np.array_equal(O.gemv(O.BF16, w, e), O.decode16(O.BF16, w[:, 7]))
+    assert np.array_equal(O.gemv(O.BF16, w, x, threads=4), y)
+    assert np.array_equal(O.gemv_x16(O.BF16, w, O.encode16(O.BF16, x)),
+                          O.gemv(O.BF16, w, O.decode16(O.BF16, O.encode16(O.BF16, x))))
+
+
+def test_rms_norm_closed_forms():
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal(256).astype(np.float32) * 3
+    ones = O.encode16(O.BF16, np.ones(256))
+    y = O.rms_norm(O.BF16, x, ones, 0.0)
+    assert abs(np.sqrt(np.mean(y.astype(np.float64) ** 2)) - 1.0) < 1e-6
+    g = O.encode16(O.BF16, rng.normal(1, 0.02, 256))
+    y = O.rms_norm(O.BF16, x, g, 1e-6)
+    xd = x.astype(np.float64)
+    ref = xd / np.sqrt(np.mean(xd ** 2) + 1e-6) * O.decode16(O.BF16, g)
+    assert np.allclose(y, ref, rtol=1e-6, atol=1e-7)
+    # per-head: each head normalised on its own with a shared gamma
+    v = rng.standard_normal(4 * 32).astype(np.float32)
+    gh = O.encode16(O.BF16, rng.normal(1, 0.02, 32))
+    out = O.per_head_rms_norm(O.BF16, gh, 32, v, 1e-6)
+    for h in range(4):
+        seg = v[h * 32:(h + 1) * 32].astype(np.float64)
+        ref = seg / np.sqrt(np.mean(seg ** 2) + 1e-6) * O.decode16(O.BF16, gh)
+        assert np.allclose(out[h * 32:(h + 1) * 32], ref, rtol=1e-6, atol=1e-7)
+
+
+def test_rope_kat_and_invariants(kat):
+    k = kat["rope"]
+    q = O.rope(k["head_dim"], 1, k["position"], k["theta"], k["query"])
+    kk = O.rope(k["head_dim"], 1, k["position"], k["theta"], k["key"])
+    a0, a1 = (np.float32(a) for a in k["angles"])
+    s0, c0, s1, c1 = np.sin(a0), np.cos(a0), np.sin(a1), np.cos(a1)
+    eq = [1 * c0 - 3 * s0, 2 * c1 - 4 * s1, 3 * c0 + 1 * s0, 4 * c1 + 2 * s1]
+    ek = [0.5 * c0 + 0.25 * s0, -c1 - 0.75 * s1, -0.25 * c0 + 0.5 * s0, 0.75 * c1 - 1.0 * s1]
+    assert np.max(np.abs(q - eq)) < k["tol"] and np.max(np.abs(kk - ek)) < k["tol"]
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal(3 * 128).astype(np.float32)
+    assert np.array_equal(O.rope(128, 3, 0, 1e6, v), v)  # position 0 is the identity
+    r = O.rope(128, 3, 4096, 1e6, v).reshape(3, 2, 64)
+    vv = v.reshape(3, 2, 64)
+    assert np.allclose(r[:, 0] ** 2 + r[:, 1] ** 2, vv[:, 0] ** 2 + vv[:, 1] ** 2, rtol=1e-5)
+    # the angle is computed in f32 (position / powf(theta, 2i/d)): an f64 angle would differ
+    # by up to ~2.5e-4 rad at this position. Model powf as the correctly rounded power.
+    i = np.arange(64, dtype=np.float32)
+    expo = ((2 * i) / np.float32(128)).astype(np.float32)
+    ang = np.float32(4096) / np.power(1e6, expo.astype(np.float64)).astype(np.float32)
+    assert ang.dtype == np.float32
+    ref0 = vv[0, 0] * np.cos(ang) - vv[0, 1] * np.sin(ang)
+    assert np.allclose(r[0, 0], ref0, atol=2e-5)
+
+
+def _dense_attention(heads, kv_heads, hd, q, keys, values):
+    q = np.asarray(q, np.float64).reshape(heads, hd)
+    k = np.asarray(keys, np.float64).reshape(-1, kv_heads, hd)
+    v = np.asarray(values, np.float64).reshape(-1, kv_heads, hd)
+    out = np.zeros((heads, hd))
+    for h in range(heads):
+        kv = h // (heads // kv_heads)
+        s = k[:, kv] @ q[h] / math.sqrt(hd)
+        p = np.exp(s - s.max())
+        out[h] = (p / p.sum()) @ v[:, kv]
+    return out.ravel()
+
+
+@pytest.mark.parametrize("name", ["attention_two_blocks", "attention_gqa"])
+def test_attention_equals_dense_softmax(kat, name):
+    k = kat[name]
+    kvh = k["kv_heads"] * k["head_dim"]
+    keys = np.array(k["keys"], np.float32).reshape(-1, kvh)
+    vals = np.array(k["values"], np.float32).reshape(-1, kvh)
+    blocks, t = [], 0
+    for n in k["block_tokens"]:
+        blocks.append((keys[t:t + n], vals[t:t + n]))
+        t += n
+    out = O.attention_blockwise(k["heads"], k["kv_heads"], k["head_dim"], k["query"], blocks)
+    ref = _dense_attention(k["heads"], k["kv_heads"], k["head_dim"], k["query"], keys, vals)
+    assert np.max(np.abs(out - ref)) < k["tol"]
+
+
+def test_attention_rejects_empty():
+    with pytest.raises(ValueError):
+        O.attention_blockwise(1, 1, 2, [1.0, 0.0], [])
+
+
+def test_paged_attention_permutation_invariance_and_dense():
+    rng = np.random.default_rng(6)
+    heads, kvh_n, hd, bt, tokens, layers = 8, 2, 16, 4, 37, 2
+    n_blocks = 12
+    kvh = kvh_n * hd
+    q = rng.standard_normal(heads * hd).astype(np.float32)
+    k = O.encode16(O.BF16, rng.standard_normal((tokens, kvh)))
+    v = O.encode16(O.BF16, rng.standard_normal((tokens, kvh)))
+    outs = []
+    for seed in (0, 1):
+        table = np.random.default_rng(seed).permutation(n_blocks).astype(np.uint32)
+        kc = np.zeros((layers, n_blocks, bt, kvh), np.uint16)
+        vc = np.zeros_like(kc)
+        for t in range(tokens):
+            kc[1, table[t // bt], t % bt] = k[t]
+            vc[1, table[t // bt], t % bt] = v[t]
+        outs.append(O.attention_paged16(O.BF16, heads, kvh_n, hd, bt, q, kc, vc, table, 1, n_blocks, tokens))
+    assert np.array_equal(outs[0], outs[1])
+    ref = _dense_attention(heads, kvh_n, hd, q, O.decode16(O.BF16, k), O.decode16(O.BF16, v))
+    assert np.max(np.abs(outs[0] - ref)) < 2e-6
+
+
+def test_argmax(kat):
+    rng = np.random.default_rng(7)
+    l = rng.standard_normal(1000).astype(np.float32)
+    assert O.greedy_argmax(l) == int(np.argmax(l))
+    l[[10, 500]] = l.max() + 1  # tie -> lowest index
+    assert O.greedy_argmax(l) == 10
+    l[3] = np.nan
+    with pytest.raises(ValueError):
+        O.greedy_argmax(l)
+    assert O.greedy_argmax(l, skip_nonfinite=True) == 10
+    l[10] = np.inf
+    assert O.greedy_argmax(l, skip_nonfinite=True) == 500
+    with pytest.raises(ValueError):
+        O.greedy_argmax(np.zeros(0, np.float32))
+
+
+def test_final_head_kat(kat):
+    k = kat["final_head"]
+    h = O.decode16(O.F16, np.array([hx(v) for v in k["hidden_bits"]], np.uint16))
+    g = np.array([hx(v) for v in k["final_norm"]], np.uint16)
+    w = np.array([hx(v) for v in k["lm_head"]], np.uint16).reshape(k["vocab"], k["hidden"])
+    logits = O.gemv(O.F16, w, O.rms_norm(O.F16, h, g, k["rms_eps"]))
+    assert O.greedy_argmax(logits) == k["token"]
+
+
+def _tiny_block_model(k, dtype):
+    one = lambda name: np.array([hx(v) for v in k[name]], np.uint16)
+    layer = dict(rms_attn=one("rms"), rms_mlp=one("rms"), w_q=one("identity"), w_k=one("identity"),
+                 w_v=one("identity"), w_o=one("identity"), w_gate=one("gate"), w_up=one("identity"),
+                 w_down=one("identity"))
+    return O.Model(dtype, k["hidden"], k["heads"], k["kv_heads"], k["head_dim"], k["intermediate"], 1,
+                   k["rms_eps"], None, np.zeros(k["hidden"], np.uint16), [layer], one("rms"),
+                   np.zeros(k["hidden"], np.uint16))
+
+
+def test_block_forward_f16_kat(kat):
+    k = kat["block_f16"]
+    model = _tiny_block_model(k, O.F16)
+    x = np.array([hx(v) for v in k["input"]], np.uint16)
+    out = O.block_forward(model, x, k["position"], staging=0)
+    assert out.tolist() == k["output_bits"]
+    assert O.fnv1a(out) == int(k["output_hash"])
+    # the device-session staging rounds three more intermediates; on this vector
+    # it lands on the same bits
+    assert O.block_forward(model, x, k["position"], staging=1).tolist() == k["output_bits"]
+
+
+def test_block_f32_closed_form_and_smoke_hash(kat):
+    k = kat["block_f32"]
+    f = np.float32
+    x = np.array(k["input"], f)
+    eps = f(k["rms_eps"])
+    s1 = f(1) / np.sqrt((x[0] * x[0] + x[1] * x[1]) / f(2) + eps)
+    attn = x * s1
+    r = x + attn
+    s2 = f(1) / np.sqrt((r[0] * r[0] + r[1] * r[1]) / f(2) + eps)
+    mn = r * s2
+    silu = np.array([O.lib.nvo_silu(float(f(k["gate_diag"]) * m)) for m in mn], f)
+    out = (r + silu * mn).astype(f)
+    assert O.fnv1a(out) == int(k["smoke_output_hash"])
+
+
+def _seq_model(k, qk_norm):
+    one = lambda name: np.array([hx(v) for v in k[name]], np.uint16)
+    layer = dict(rms_attn=one("rms"), rms_mlp=one("rms"), w_q=one("matrix"), w_k=one("matrix"),
+                 w_v=one("matrix"), w_o=one("matrix"), w_gate=one("matrix"), w_up=one("matrix"),
+                 w_down=one("matrix"))
+    if qk_norm:
+        layer.update(q_norm=one("rms"), k_norm=one("rms"))
+    return O.Model(O.F16, k["hidden"], k["heads"], k["kv_heads"], k["head_dim"], k["intermediate"],
+                   k["vocab"], k["rms_eps"], k["rope_theta"], one("embeddings"), [layer], one("rms"),
+                   one("lm_head"))
+
+
+@pytest.mark.parametrize("staging", [0, 1])
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_greedy_stream_kat(kat, staging, qk_norm):
+    k = kat["decode_sequence"]
+    ctx = O.Context(_seq_model(k, qk_norm), 8, staging=staging)
+    tokens, _ = ctx.greedy_decode(k["prompt"], k["steps"])
+    assert tokens.tolist() == k["tokens"]
+    tokens, _ = ctx.greedy_decode(k["prompt"], k["steps"], eos=k["eos_token"])
+    assert tokens.tolist() == k["tokens_with_eos"]
+
+
+def test_moe_routed_clamp_kat(kat):
+    k = kat["moe_routed_clamp"]
+    x = np.array(k["input"], np.float32)
+    out = O.moe_forward_f32(k["hidden"], k["intermediate"], x, k["expert_ids"], k["expert_weights"],
+                            k["w_gate"], k["w_up"], k["w_down"], limit=k["swiglu_limit"])
+    H, I = k["hidden"], k["intermediate"]
+    wg = np.array(k["w_gate"]).reshape(-1, I, H)
+    wu = np.array(k["w_up"]).reshape(-1, I, H)
+    wd = np.array(k["w_down"]).reshape(-1, H, I)
+    lim = k["swiglu_limit"]
+    ref = np.zeros(H)
+    for e, wt in zip(k["expert_ids"], k["expert_weights"]):
+        g = np.minimum(wg[e] @ x.astype(np.float64), lim)
+        u = np.clip(wu[e] @ x.astype(np.float64), -lim, lim)
+        ref += wt * (wd[e] @ (g / (1 + np.exp(-g)) * u))
+    assert np.max(np.abs(out - ref)) < k["tol"]
+
+
+def test_moe_full_shared_kat(kat):
+    k = kat["moe_full_shared"]
+    x = np.array(k["input"], np.float64)
+    H, I, SI = k["hidden"], k["intermediate"], k["shared_intermediate"]
+    weights = [0.6, 0.9]  # any weights: the combine is linear in them
+    out = O.moe_forward_f32(H, I, x, k["expert_ids"], weights, k["w_gate"], k["w_up"], k["w_down"],
+                            shared=(SI, k["shared_w_gate"], k["shared_w_up"], k["shared_w_down"]))
+    wg = np.array(k["w_gate"]).reshape(-1, I, H)
+    wu = np.array(k["w_up"]).reshape(-1, I, H)
+    wd = np.array(k["w_down"]).reshape(-1, H, I)
+    silu = lambda g: g / (1 + np.exp(-g))
+    ref = np.zeros(H)
+    for e, wt in zip(k["expert_ids"], weights):
+        ref += wt * (wd[e] @ (silu(wg[e] @ x) * (wu[e] @ x)))
+    sg = np.array(k["shared_w_gate"]).reshape(SI, H)
+    su = np.array(k["shared_w_up"]).reshape(SI, H)
+    sd = np.array(k["shared_w_down"]).reshape(H, SI)
+    ref += sd @ (silu(sg @ x) * (su @ x))
+    assert np.max(np.abs(out - ref)) < k["tol"]
+
+
+def test_moe_route_softmax_rules():
+    rng = np.random.default_rng(8)
+    logits = rng.standard_normal(256).astype(np.float32)
+    ids, w = O.moe_route_softmax(logits, 8, True)
+    p = np.exp(logits.astype(np.float64) - logits.max())
+    p /= p.sum()
+    order = sorted(range(256), key=lambda i: (-p[i], i))[:8]
+    assert ids.tolist() == order
+    assert abs(w.sum() - 1) < 1e-6 and np.allclose(w, p[order] / p[order].sum(), rtol=1e-5)
+    ids2, w2 = O.moe_route_softmax(logits, 8, False)
+    assert ids2.tolist() == order and np.allclose(w2, p[order], rtol=1e-5)
+    tie = np.zeros(6, np.float32)
+    ids3, _ = O.moe_route_softmax(tie, 3, True)
+    assert ids3.tolist() == [0, 1, 2]  # equal probabilities -> index ascending
+
+
+def test_moe_fp8_identity_like_reduces_to_weighted_sum():
+    # With gate rows = 0 the activation is silu(0)*u = 0: output must be exactly 0.
+    H, I, E, B = 256, 128, 3, 128
+    zero = np.zeros((E, I, H), np.uint8)
+    one_s = np.ones((E, I // B, H // B), np.float32)
+    rng = np.random.default_rng(9)
+    wu = O.encode_fp8(rng.normal(0, 1, (E, I, H)))
+    wd = O.encode_fp8(rng.normal(0, 1, (E, H, I)))
+    sd = np.ones((E, H // B, I // B), np.float32)
+    x16 = O.encode16(O.BF16, rng.standard_normal(H))
+    out = O.moe_fp8_forward(H, I, E, B, x16, [2, 0], [0.5, 0.5], zero, one_s, wu, one_s, wd, sd)
+    assert np.all(out == 0)
+    # general case against f64
+    wg = O.encode_fp8(rng.normal(0, 1, (E, I, H)))
+    sg = rng.uniform(0.01, 0.05, (E, I // B, H // B)).astype(np.float32)
+    sdn = rng.uniform(0.01, 0.05, (E, H // B, I // B)).astype(np.float32)
+    out = O.moe_fp8_forward(H, I, E, B, x16, [2, 0], [0.7, 0.3], wg, sg, wu, sg, wd, sdn, shared_index=1)
+    x = O.decode16(O.BF16, x16).astype(np.float64)
+    silu = lambda g: g / (1 + np.exp(-g))
+    ref = np.zeros(H)
+    for e, wt in ((2, 0.7), (0, 0.3), (1, 1.0)):
+        G = O.decode_fp8(wg[e]).astype(np.float64) * np.kron(sg[e], np.ones((B, B)))
+        U = O.decode_fp8(wu[e]).astype(np.float64) * np.kron(sg[e], np.ones((B, B)))
+        D = O.decode_fp8(wd[e]).astype(np.float64) * np.kron(sdn[e], np.ones((B, B)))
+        ref += wt * (D @ (silu(G @ x) * (U @ x)))
+    assert np.linalg.norm(out - ref) / np.linalg.norm(ref) < 1e-5
+
+
+def test_synth_generator_statistics_and_determinism():
+    a = O.synth_f32(0x4E45525641, 3, 200000, 0.0, 0.02)
+    assert abs(a.mean()) < 2e-4 and abs(a.std() - 0.02) < 2e-4
+    assert np.array_equal(a[1000:2000], O.synth_f32(0x4E45525641, 3, 1000, 0.0, 0.02, offset=1000))
+    assert not np.array_equal(a[:1000], O.synth_f32(0x4E45525641, 4, 1000, 0.0, 0.02))
+    g = O.decode16(O.BF16, O.synth_16(O.BF16, 1, 2, 4096, 1.0, 0.02))
+    assert abs(g.mean() - 1) < 2e-3
+    t = O.synth_tokens(1, 9, 10000, 151936)
+    assert t.max() < 151936 and len(set(t.tolist())) > 9000
+    w, s = O.synth_fp8_block(5, 6, 130, 260, 128, 0.02)
+    assert s.shape == (2, 3) and np.all(s > 0)
+    deq = O.decode_fp8(w) * np.kron(s, np.ones((128, 128), np.float32))[:130, :260]
+    src = O.synth_f32(5, 6, 130 * 260, 0.0, 0.02).reshape(130, 260)
+    assert np.max(np.abs(deq - src)) <= np.max(s) * 448 * 2 ** -4 + 1e-9  # half-ulp of e4m3 at amax
