@@ -1,0 +1,549 @@
+/* nerva_hip_api.h - flat C ABI of libnerva_hip (MI355X / gfx950 decode backend).
+ *
+ * This is the boundary a `nerva-hip` host crate binds, the way `nerva-cuda`
+ * binds native/cuda/nerva_cuda_api.h in the reference. Every struct marked
+ * "mirrors" has the same field order, widths and enum values as the cited
+ * NervaCuda... struct (the `cuda_error` slot carries a hipError_t and is named
+ * `hip_error`), so the Rust #[repr(C)] mirrors only need their prefix changed.
+ * include/nerva_hip_layout_check.hpp static_asserts the sizes and key offsets.
+ *
+ * Conventions (reference: nerva_cuda_api.h:2141-2310,
+ * session_api_lifecycle.inc.cu:5-55,1117-1144, native_stubs.rs:5-33):
+ *   - every call returns 0 on success and -1 on failure;
+ *   - a null `out` returns -1; otherwise `out` is zeroed and status = -1 first;
+ *   - no device present: status = -1, hip_error = 100 (hipErrorNoDevice);
+ *   - nothing throws, aborts or logs across this boundary;
+ *   - a session is driven by one host thread at a time; callers serialise.
+ *
+ * Citations are reference paths (relative to the reference checkout).
+ */
+#ifndef NERVA_HIP_API_H_
+#define NERVA_HIP_API_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NERVA_HIP_DTYPE_F16 0u  /* types.cuh:9 */
+#define NERVA_HIP_DTYPE_BF16 1u /* types.cuh:10 */
+#define NERVA_HIP_MLP_DENSE 0u  /* types.cuh:12 */
+#define NERVA_HIP_ATTENTION_FULL 0u /* types.cuh:14 */
+#define NERVA_HIP_SLOT_REQUEST_ID 1u  /* types.cuh:34 */
+#define NERVA_HIP_SLOT_SEQUENCE_ID 1u /* types.cuh:35 */
+#define NERVA_HIP_SLOT_DEVICE_COMPLETE 1u /* types.cuh:36 */
+#define NERVA_HIP_KV_BLOCK_TOKENS 16u /* types.cuh:64 */
+#define NERVA_HIP_ERROR_NO_DEVICE 100 /* native_stubs.rs:5-16 */
+#define NERVA_HIP_ERROR_NOT_SUPPORTED 801 /* hipErrorNotSupported */
+#define NERVA_HIP_ERROR_INVALID_VALUE 1 /* hipErrorInvalidValue */
+
+/* mirrors NervaCudaDeviceSmokeResult (nerva_cuda_api.h:9-27) */
+typedef struct NervaHipDeviceSmokeResult {
+  int32_t status, hip_error;
+  uint32_t value;
+  int32_t device_count, device_ordinal, driver_version, runtime_version,
+      compute_capability_major, compute_capability_minor, posix_fd_handle_supported,
+      vmm_posix_fd_export_verified, gpu_direct_rdma_supported,
+      gpu_direct_rdma_with_cuda_vmm_supported;
+  uint64_t total_global_mem, free_global_mem;
+  char gpu_name[128], pci_bus_id[32];
+} NervaHipDeviceSmokeResult;
+
+/* mirrors NervaCudaSyntheticTokenSlot (nerva_cuda_api.h:29-37); 40 bytes.
+ * The sampler writes {1, 1, pos, token, pos+1, 1, 0} (sampler.cu:394-407). */
+typedef struct NervaHipSyntheticTokenSlot {
+  uint32_t request_id, sequence_id;
+  uint64_t token_index;
+  uint32_t token;
+  uint64_t version;
+  uint32_t completion, host_copied;
+} NervaHipSyntheticTokenSlot;
+
+/* mirrors NervaCudaHfDecodeChainLayer (nerva_cuda_api.h:255-332). Host
+ * pointers to row-major [out, in] 16-bit matrices, read only during create.
+ * This backend runs dense full-attention layers: a non-zero mlp_kind,
+ * attention_kind, linear_* or deepseek_* field, or a non-null w_q_gate /
+ * router / expert / w_linear_* pointer, fails create with
+ * hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED. */
+typedef struct NervaHipHfDecodeChainLayer {
+  const uint16_t *rms_attn_weight, *rms_mlp_weight, *w_q, *w_q_gate, *w_k, *q_norm_weight,
+      *k_norm_weight, *w_v, *w_o, *q_bias, *k_bias, *v_bias, *o_bias, *w_gate, *w_up, *w_down,
+      *w_router, *w_expert_gate_up, *w_expert_down, *w_shared_expert_gate, *w_shared_expert_up,
+      *w_shared_expert_down, *w_shared_expert_router;
+  uint32_t linear_key_heads, linear_value_heads, linear_key_head_dim, linear_value_head_dim,
+      linear_conv_kernel;
+  const uint16_t *w_linear_conv, *w_linear_qkv, *w_linear_z, *w_linear_b, *w_linear_a,
+      *w_linear_dt_bias;
+  const float *w_linear_a_log;
+  const uint16_t *w_linear_norm, *w_linear_out;
+  uint32_t mlp_kind, moe_intermediate, shared_expert_intermediate, num_experts,
+      experts_per_token, norm_topk_prob, attention_kind, deepseek_mode, deepseek_flags,
+      deepseek_storage, deepseek_hc_mult, deepseek_hc_sinkhorn_iters, deepseek_q_lora_rank,
+      deepseek_kv_lora_rank, deepseek_o_lora_rank, deepseek_o_groups, deepseek_qk_nope_head_dim,
+      deepseek_qk_rope_head_dim, deepseek_v_head_dim, deepseek_compress_ratio,
+      deepseek_index_topk, deepseek_index_n_heads, deepseek_index_head_dim,
+      deepseek_router_num_groups, deepseek_router_topk_groups;
+  float deepseek_routed_scaling_factor, deepseek_hc_eps, deepseek_hc_post_alpha;
+  uint32_t deepseek_rope_scaling_type, deepseek_rope_original_max_position;
+  float deepseek_rope_scaling_factor, deepseek_rope_extrapolation_factor,
+      deepseek_rope_attn_factor, deepseek_rope_beta_fast, deepseek_rope_beta_slow,
+      deepseek_rope_mscale, deepseek_rope_mscale_all_dim, deepseek_compress_rope_theta,
+      deepseek_swiglu_limit;
+} NervaHipHfDecodeChainLayer;
+
+/* mirrors NervaCudaHfDecodeSequenceWeightBlock (nerva_cuda_api.h:380-391) */
+typedef struct NervaHipHfDecodeSequenceWeightBlock {
+  const uint16_t *host_source;
+  const char *source_file;
+  uint64_t source_file_len, file_offset_begin, block_id, block_version, offset_bytes, bytes;
+  uint32_t strategy, reserved;
+} NervaHipHfDecodeSequenceWeightBlock;
+
+/* mirrors NervaCudaHfDecodeSamplerConfig (nerva_cuda_api.h:393-399).
+ * Greedy <=> !(temperature > 0) || top_k == 1 (sampler.cu:89). Only greedy is
+ * implemented: any other configuration fails start with NOT_SUPPORTED. */
+typedef struct NervaHipHfDecodeSamplerConfig {
+  float temperature, top_p;
+  uint32_t top_k, reserved;
+  uint64_t seed;
+} NervaHipHfDecodeSamplerConfig;
+
+/* mirrors NervaCudaHfDecodeSequenceRequest (nerva_cuda_api.h:401-434) */
+typedef struct NervaHipHfDecodeSequenceRequest {
+  uint32_t dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab_size, layer_count,
+      steps, seed_token;
+  const uint32_t *prompt_tokens;
+  uint32_t prompt_token_count, has_eos_token, eos_token;
+  float rms_eps, rope_theta;
+  const uint16_t *embeddings;
+  const NervaHipHfDecodeChainLayer *layers;
+  const uint16_t *final_norm_weight, *lm_head;
+  uint32_t planned_weight_blocks, planned_gpu_resident_blocks, planned_gpu_staged_blocks;
+  uint64_t planned_weight_bytes, planned_gpu_resident_weight_bytes,
+      planned_gpu_staged_weight_bytes;
+  const NervaHipHfDecodeSequenceWeightBlock *planned_weight_descriptors;
+  uint32_t planned_weight_descriptor_count;
+  uint64_t planned_weight_descriptor_hash;
+  uint32_t *output_tokens;
+  uint32_t output_token_capacity;
+  NervaHipHfDecodeSamplerConfig sampler;
+} NervaHipHfDecodeSequenceRequest;
+
+/* mirrors NervaCudaHfDecodeSequenceResult (nerva_cuda_api.h:436-513) */
+typedef struct NervaHipHfDecodeSequenceResult {
+  int32_t status, hip_error, device_count;
+  uint32_t dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab_size, layer_count,
+      steps, seed_token, observed_tokens, last_token;
+  uint64_t observed_token_hash, resident_weight_bytes;
+  uint32_t planned_weight_blocks, planned_gpu_resident_blocks, planned_gpu_staged_blocks;
+  uint64_t planned_weight_bytes, planned_gpu_resident_weight_bytes,
+      planned_gpu_staged_weight_bytes, descriptor_gpu_resident_h2d_bytes,
+      descriptor_gpu_staged_h2d_bytes;
+  uint32_t planned_weight_descriptor_count;
+  uint64_t planned_weight_descriptor_hash, resident_kv_bytes, deepseek_mhc_residual_bytes,
+      deepseek_mhc_post_mix_bytes, deepseek_mhc_comb_mix_bytes, kv_tokens, device_arena_bytes,
+      pinned_host_bytes, h2d_bytes, d2h_bytes, graph_replays, graph_nodes, graph_launches,
+      graph_captures, graph_cache_hits, kernel_launches, experimental_rt_selector_launches;
+  uint32_t experimental_rt_sparse_attention_active, experimental_rt_dense_attention_chunks,
+      experimental_rt_attention_chunks, experimental_rt_reserved;
+  uint64_t device_elapsed_ns, projection_ns, qkv_projection_ns, attention_output_projection_ns,
+      gate_up_projection_ns, down_projection_ns, lm_head_projection_ns, attention_ns, mlp_ns,
+      norm_ns, sampling_ns, sync_calls, host_causality_edges, hot_path_allocations,
+      deepseek_compressor_state_writes, deepseek_compressed_kv_writes,
+      deepseek_indexer_state_writes, deepseek_indexer_kv_writes,
+      deepseek_compressed_kv_attention_reads, deepseek_compressed_kv_attention_slots_scanned,
+      deepseek_sparse_topk_selections, deepseek_sparse_topk_slots_selected,
+      deepseek_sparse_topk_candidates_scored, deepseek_sparse_topk_selection_hash,
+      deepseek_v3_grouped_router_selections, deepseek_v4_bias_router_selections,
+      deepseek_v4_hash_router_selections, deepseek_raw_attention_tokens_scanned,
+      deepseek_sparse_attention_output_hash;
+} NervaHipHfDecodeSequenceResult;
+
+typedef struct NervaHipHfDecodeSequenceSession NervaHipHfDecodeSequenceSession;
+
+/* mirrors NervaCudaHfDecodeSequenceSessionCreateRequest (nerva_cuda_api.h:606-638) */
+typedef struct NervaHipHfDecodeSequenceSessionCreateRequest {
+  uint32_t dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab_size, layer_count,
+      max_context_tokens;
+  float rms_eps, rope_theta;
+  const uint16_t *embeddings;
+  const NervaHipHfDecodeChainLayer *layers;
+  const uint16_t *final_norm_weight, *lm_head;
+  uint32_t planned_weight_blocks, planned_gpu_resident_blocks, planned_gpu_staged_blocks;
+  uint64_t planned_weight_bytes, planned_gpu_resident_weight_bytes,
+      planned_gpu_staged_weight_bytes;
+  const NervaHipHfDecodeSequenceWeightBlock *planned_weight_descriptors;
+  uint32_t planned_weight_descriptor_count;
+  uint64_t planned_weight_descriptor_hash;
+  uint32_t detailed_profile, experimental_rt_decode, experimental_rt_mode,
+      experimental_rt_page_tokens, experimental_rt_pages, experimental_rt_local_window_tokens,
+      experimental_rt_sink_tokens;
+} NervaHipHfDecodeSequenceSessionCreateRequest;
+
+/* mirrors NervaCudaHfDecodeSequenceSessionCreateResult (nerva_cuda_api.h:640-687) */
+typedef struct NervaHipHfDecodeSequenceSessionCreateResult {
+  int32_t status, hip_error, failure_stage, device_count;
+  uint32_t dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab_size, layer_count,
+      max_context_tokens, prefill_chunk_tokens, head_threads;
+  uint64_t resident_weight_bytes;
+  uint32_t planned_weight_blocks, planned_gpu_resident_blocks, planned_gpu_staged_blocks;
+  uint64_t planned_weight_bytes, planned_gpu_resident_weight_bytes,
+      planned_gpu_staged_weight_bytes, descriptor_gpu_resident_h2d_bytes,
+      descriptor_gpu_staged_h2d_bytes;
+  uint32_t planned_weight_descriptor_count;
+  uint64_t planned_weight_descriptor_hash;
+  uint32_t experimental_rt_decode_requested, experimental_rt_decode_enabled,
+      experimental_rt_mode, experimental_rt_page_tokens, experimental_rt_pages,
+      experimental_rt_local_window_tokens, experimental_rt_sink_tokens,
+      deepseek_v4_attention_aux_streams, deepseek_v4_attention_events;
+  uint64_t deepseek_v4_swa_kv_bytes, deepseek_mhc_residual_bytes, deepseek_mhc_post_mix_bytes,
+      deepseek_mhc_comb_mix_bytes, resident_kv_bytes, device_arena_bytes, pinned_host_bytes,
+      h2d_bytes, sync_calls, hot_path_allocations, device_memory_bandwidth_bps;
+} NervaHipHfDecodeSequenceSessionCreateResult;
+
+/* mirrors NervaCudaHfDecodeSequenceSessionRunRequest (nerva_cuda_api.h:694-705) */
+typedef struct NervaHipHfDecodeSequenceSessionRunRequest {
+  NervaHipHfDecodeSequenceSession *session;
+  uint32_t steps, seed_token;
+  const uint32_t *prompt_tokens;
+  uint32_t prompt_token_count, has_eos_token, eos_token;
+  uint32_t *output_tokens;
+  uint32_t output_token_capacity;
+  NervaHipHfDecodeSamplerConfig sampler;
+} NervaHipHfDecodeSequenceSessionRunRequest;
+
+/* mirrors NervaCudaHfDecodeSequenceSessionStartRequest (nerva_cuda_api.h:707-714) */
+typedef struct NervaHipHfDecodeSequenceSessionStartRequest {
+  NervaHipHfDecodeSequenceSession *session;
+  const uint32_t *prompt_tokens;
+  uint32_t prompt_token_count, has_eos_token, eos_token;
+  NervaHipHfDecodeSamplerConfig sampler;
+} NervaHipHfDecodeSequenceSessionStartRequest;
+
+/* mirrors NervaCudaHfDecodeSequenceSessionAdvanceRequest (nerva_cuda_api.h:716-721) */
+typedef struct NervaHipHfDecodeSequenceSessionAdvanceRequest {
+  NervaHipHfDecodeSequenceSession *session;
+  uint32_t steps;
+  uint32_t *output_tokens;
+  uint32_t output_token_capacity;
+} NervaHipHfDecodeSequenceSessionAdvanceRequest;
+
+/* mirrors NervaCudaDeepSeekQuantDequantResult (nerva_cuda_api.h:1338-1354) */
+typedef struct NervaHipDeepSeekQuantDequantResult {
+  int32_t status, hip_error, device_count;
+  uint32_t rows, cols, block_rows, block_cols;
+  uint64_t output_hash, device_arena_bytes, pinned_host_bytes, h2d_bytes, d2h_bytes,
+      kernel_launches, sync_calls, hot_path_allocations;
+} NervaHipDeepSeekQuantDequantResult;
+
+/* mirrors NervaCudaDeepSeekQuantFp8F32ScaleEncodedMatvecRequest
+ * (nerva_cuda_api.h:1367-1377). All pointers are HOST pointers. */
+typedef struct NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest {
+  uint32_t rows, cols, block_rows, block_cols, input_dtype;
+  const uint8_t *weights;
+  const float *scales;
+  const uint16_t *input;
+  float *output;
+} NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest;
+
+/* mirrors NervaCudaDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest
+ * (nerva_cuda_api.h:1379-1390). input [tokens x cols], output [tokens x rows]. */
+typedef struct NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest {
+  uint32_t rows, cols, tokens, block_rows, block_cols, input_dtype;
+  const uint8_t *weights;
+  const float *scales;
+  const uint16_t *input;
+  float *output;
+} NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest;
+
+/* mirrors NervaCudaProjectionBenchRequest (nerva_cuda_api.h:1075-1082) */
+typedef struct NervaHipProjectionBenchRequest {
+  uint32_t dtype, rows, cols, iterations, warmup_iterations, block_tokens;
+} NervaHipProjectionBenchRequest;
+
+/* mirrors NervaCudaProjectionBenchResult (nerva_cuda_api.h:1084-1144). The
+ * cublaslt_* slots stay zero (no vendor GEMV on this backend); custom_* is the
+ * hand-written kernel. */
+typedef struct NervaHipProjectionBenchResult {
+  int32_t status, hip_error, device_count, device_ordinal, compute_capability_major,
+      compute_capability_minor;
+  uint32_t dtype, rows, cols, block_tokens, iterations, warmup_iterations;
+  uint64_t matrix_bytes, input_bytes, output_bytes, cublaslt_total_ns, cublaslt_avg_ns,
+      cublaslt_default_total_ns, cublaslt_default_avg_ns;
+  uint32_t cublaslt_heuristic_count, cublaslt_best_heuristic_index;
+  uint64_t cublaslt_best_heuristic_total_ns, cublaslt_best_heuristic_avg_ns, custom_total_ns,
+      custom_avg_ns, cublaslt_graph_total_ns, cublaslt_graph_avg_ns,
+      cublaslt_default_graph_total_ns, cublaslt_default_graph_avg_ns,
+      cublaslt_best_heuristic_graph_total_ns, cublaslt_best_heuristic_graph_avg_ns,
+      custom_graph_total_ns, custom_graph_avg_ns, cublaslt_graph_nodes, custom_graph_nodes,
+      graph_replays, graph_captures;
+  uint32_t selected_graph_strategy;
+  uint64_t cublaslt_effective_bandwidth_bps, custom_effective_bandwidth_bps;
+  uint32_t selected_strategy, mismatch_count;
+  float max_abs_diff;
+  uint64_t kernel_launches, sync_calls, device_allocations, device_frees, device_arena_bytes,
+      hot_path_allocations, block_cublaslt_total_ns, block_cublaslt_avg_ns,
+      block_cublaslt_per_token_ns, block_cublaslt_graph_total_ns, block_cublaslt_graph_avg_ns,
+      block_cublaslt_graph_per_token_ns, block_cublaslt_graph_nodes,
+      block_cublaslt_speedup_x1000, block_cublaslt_graph_speedup_x1000,
+      block_cublaslt_effective_bandwidth_bps;
+} NervaHipProjectionBenchResult;
+
+/* mirrors NervaCudaDeepSeekMoeForwardRequest (nerva_cuda_api.h:2023-2037); host f32 pointers */
+typedef struct NervaHipDeepSeekMoeForwardRequest {
+  uint32_t hidden_size, intermediate_size, num_experts, top_k, clamp_swiglu;
+  float swiglu_limit;
+  const float *input;
+  const uint32_t *expert_ids;
+  const float *expert_weights, *w_gate, *w_up, *w_down;
+  float *output;
+} NervaHipDeepSeekMoeForwardRequest;
+
+/* mirrors NervaCudaDeepSeekMoeForwardResult (nerva_cuda_api.h:2039-2058) */
+typedef struct NervaHipDeepSeekMoeForwardResult {
+  int32_t status, hip_error, device_count, moe_error;
+  uint32_t hidden_size, intermediate_size, num_experts, top_k, clamp_swiglu;
+  float swiglu_limit;
+  uint64_t output_hash, device_arena_bytes, pinned_host_bytes, h2d_bytes, d2h_bytes,
+      kernel_launches, sync_calls, hot_path_allocations;
+} NervaHipDeepSeekMoeForwardResult;
+
+/* ------------------------------------------------------------------------
+ * Entry points that replace a reference entry point one for one.
+ * ---------------------------------------------------------------------- */
+
+/* replaces nerva_cuda_device_smoke (nerva_cuda_api.h:2141) */
+int nerva_hip_device_smoke(NervaHipDeviceSmokeResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_u16 (nerva_cuda_api.h:2157-2159):
+ * create + start + advance(steps) + destroy in one call. */
+int nerva_hip_hf_decode_sequence_u16(const NervaHipHfDecodeSequenceRequest *request,
+                                     NervaHipHfDecodeSequenceResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_create (nerva_cuda_api.h:2163-2166) */
+int nerva_hip_hf_decode_sequence_session_create(
+    const NervaHipHfDecodeSequenceSessionCreateRequest *request,
+    NervaHipHfDecodeSequenceSessionCreateResult *out, NervaHipHfDecodeSequenceSession **session);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_run (nerva_cuda_api.h:2167-2169) */
+int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessionRunRequest *request,
+                                             NervaHipHfDecodeSequenceResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_start (nerva_cuda_api.h:2170-2172):
+ * prefills the whole prompt and samples token 0 into slots[prompt_count-1]. */
+int nerva_hip_hf_decode_sequence_session_start(
+    const NervaHipHfDecodeSequenceSessionStartRequest *request, NervaHipHfDecodeSequenceResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_advance (nerva_cuda_api.h:2173-2175):
+ * the first advance(steps) returns `steps` tokens with steps-1 graph replays. */
+int nerva_hip_hf_decode_sequence_session_advance(
+    const NervaHipHfDecodeSequenceSessionAdvanceRequest *request,
+    NervaHipHfDecodeSequenceResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_destroy (nerva_cuda_api.h:2216-2218) */
+int nerva_hip_hf_decode_sequence_session_destroy(NervaHipHfDecodeSequenceSession *session,
+                                                 NervaHipHfDecodeSequenceSessionCreateResult *out);
+
+/* replaces nerva_cuda_deepseek_quant_fp8_f32_scale_encoded_matvec (nerva_cuda_api.h:2245-2247) */
+int nerva_hip_deepseek_quant_fp8_f32_scale_encoded_matvec(
+    const NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest *request,
+    NervaHipDeepSeekQuantDequantResult *out);
+
+/* replaces nerva_cuda_deepseek_quant_fp8_f32_scale_encoded_gemm_tokens (nerva_cuda_api.h:2248-2250) */
+int nerva_hip_deepseek_quant_fp8_f32_scale_encoded_gemm_tokens(
+    const NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest *request,
+    NervaHipDeepSeekQuantDequantResult *out);
+
+/* replaces nerva_cuda_projection_bench (nerva_cuda_api.h:2227-2228). Unlike the
+ * reference's loop, which re-reads one matrix, this one cycles through enough
+ * distinct copies of the matrix to exceed 1 GiB so that the 256 MB last-level
+ * cache cannot serve repeats (set NERVA_HIP_BENCH_RESIDENT=1 to re-read one copy). */
+int nerva_hip_projection_bench(const NervaHipProjectionBenchRequest *request,
+                               NervaHipProjectionBenchResult *out);
+
+/* replaces nerva_cuda_deepseek_moe_forward (nerva_cuda_api.h:2302-2304): f32
+ * routed experts with optional SwiGLU clamp, host pointers. */
+int nerva_hip_deepseek_moe_forward(const NervaHipDeepSeekMoeForwardRequest *request,
+                                   NervaHipDeepSeekMoeForwardResult *out);
+
+/* ------------------------------------------------------------------------
+ * Device-pointer operator entry points. The reference exposes these kernels
+ * only inside its session (native/cuda/hf_decode_sequence/session_decode_prefill.inc.cu:74-372);
+ * they are exported here so each one can be checked and timed on its own.
+ * All pointers are DEVICE pointers obtained from nerva_hip_malloc; `stream`
+ * is a hipStream_t or NULL for the library's own stream. Launch only: call
+ * nerva_hip_stream_synchronize before reading results. Return 0 / -1 and
+ * leave the hipError_t in *hip_error when it is non-null.
+ * ---------------------------------------------------------------------- */
+
+typedef struct NervaHipGemvRequest {
+  uint32_t dtype;            /* NERVA_HIP_DTYPE_* of weights and 16-bit vectors */
+  uint32_t rows, cols;       /* W is row-major [rows x cols] (for swiglu: [2*rows x cols], gate rows first) */
+  uint32_t prologue;         /* 0: input16 is the 16-bit x;  1: x = round16(rmsnorm(input_f32, gamma, eps)) */
+  uint32_t epilogue;         /* 0: f32 out; 1: f32 out = y + residual; 2: out16 = round16(silu(gate)*up);
+                                3: out16 = round16(y) */
+  uint32_t round_output;     /* epilogue 1: round the sum to 16 bits (prompt-token staging) */
+  float rms_eps;
+  const uint16_t *weights;
+  const uint16_t *input16;   /* [cols] */
+  const float *input_f32;    /* [cols] */
+  const uint16_t *gamma;     /* [cols] */
+  const uint16_t *bias;      /* optional [rows] */
+  const float *residual;     /* [rows] */
+  float *output_f32;         /* [rows] */
+  uint16_t *output16;        /* [rows] */
+} NervaHipGemvRequest;
+
+/* y = W.x weight-streaming GEMV (mat_vec_encoded_row_major, precision/block/ops.rs:75-91;
+ * device staging projection.cu:63-79) with the fused prologues/epilogues of the
+ * decode step (device_ops.cuh:317-332, kernels.cu:577-612,651-668). */
+int nerva_hip_gemv(const NervaHipGemvRequest *request, void *stream, int32_t *hip_error);
+
+typedef struct NervaHipFp8GemvRequest {
+  uint32_t rows, cols, block_rows, block_cols;
+  uint32_t input_dtype;      /* dtype of input16 */
+  const uint8_t *weights;    /* e4m3fn [rows x cols] */
+  const float *scales;       /* [ceil(rows/block_rows) x ceil(cols/block_cols)] */
+  const uint16_t *input16;   /* [cols], or NULL */
+  const float *input_f32;    /* [cols], used when input16 is NULL */
+  float *output;             /* [rows] */
+} NervaHipFp8GemvRequest;
+
+/* y[r] = sum_c (e4m3(W[r,c]) * S[r/br, c/bc]) * x[c], dequantised in f32 registers
+ * (reference contract: crates/nerva-cuda/src/tests/deepseek_quant.rs:689-713). */
+int nerva_hip_fp8_gemv(const NervaHipFp8GemvRequest *request, void *stream, int32_t *hip_error);
+
+typedef struct NervaHipPagedAttentionRequest {
+  uint32_t dtype, heads, kv_heads, head_dim;
+  uint32_t layer, block_count;  /* KV cache holds [layers][block_count] blocks of 16 tokens */
+  uint32_t position;            /* index of the token being decoded; keys 0..position are attended */
+  uint32_t append;              /* 1: qkv_f32 carries k,v of this token -> norm/RoPE/round/append first */
+  float rms_eps, rope_theta;    /* rope_theta <= 0 disables RoPE */
+  const float *qkv_f32;         /* [heads*hd | kv_heads*hd | kv_heads*hd] raw projections */
+  const uint16_t *q_norm, *k_norm;        /* optional [head_dim] */
+  const uint16_t *q_bias, *k_bias, *v_bias; /* optional */
+  uint16_t *k_cache, *v_cache;  /* [layer][block][kv_head][16][head_dim], 16-bit */
+  const uint32_t *block_table;  /* [block_count] logical -> physical */
+  void *workspace;              /* nerva_hip_paged_attention_workspace_bytes() bytes, zero-initialised once */
+  float *output_f32;            /* optional [heads*hd] */
+  uint16_t *output16;           /* [heads*hd] rounded */
+} NervaHipPagedAttentionRequest;
+
+/* Fused per-head RMSNorm + RoPE + KV append + paged GQA split-KV decode attention
+ * (kernels.cu:287-555, attention_kernels.cu:263-760; exact_blockwise_attention_into,
+ * attention/exact/run.rs:13-127). */
+int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *request, void *stream,
+                               int32_t *hip_error);
+uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim);
+/* Element offset of (layer, physical block, kv_head, token-in-block, 0) in the cache arrays. */
+uint64_t nerva_hip_kv_cache_offset(uint32_t block_count, uint32_t kv_heads, uint32_t head_dim,
+                                   uint32_t layer, uint32_t physical_block, uint32_t kv_head,
+                                   uint32_t token_in_block);
+
+typedef struct NervaHipArgmaxRequest {
+  uint32_t count;
+  const float *logits;
+  uint32_t *token;           /* device u32 */
+  void *workspace;           /* nerva_hip_argmax_workspace_bytes() bytes, zero-initialised once */
+} NervaHipArgmaxRequest;
+
+/* First maximum among finite logits, ties to the lowest index (sampler.cu:35-40,89-119;
+ * greedy_argmax, common/token.rs:33-58). */
+int nerva_hip_argmax(const NervaHipArgmaxRequest *request, void *stream, int32_t *hip_error);
+uint64_t nerva_hip_argmax_workspace_bytes(void);
+
+typedef struct NervaHipMoeFp8Request {
+  uint32_t hidden, intermediate, num_experts, top_k, block, input_dtype;
+  int32_t shared_index;         /* expert index of the always-on shared expert, or -1 */
+  const uint16_t *input16;      /* [hidden] */
+  const uint32_t *expert_ids;   /* device [top_k] */
+  const float *expert_weights;  /* device [top_k] */
+  const uint8_t *w_gate, *w_up; /* [E][intermediate][hidden] e4m3fn */
+  const float *s_gate, *s_up;   /* [E][ceil(I/block)][ceil(H/block)] */
+  const uint8_t *w_down;        /* [E][hidden][intermediate] */
+  const float *s_down;          /* [E][ceil(H/block)][ceil(I/block)] */
+  float *activation;            /* scratch f32 [(top_k+1) * intermediate] */
+  float *output;                /* f32 [hidden] */
+} NervaHipMoeFp8Request;
+
+/* out = sum_k w_k * Wd_e(swiglu(Wg_e x, Wu_e x)) + shared(x) with FP8 block-scaled
+ * expert weights (reference/moe.rs:76-166, precision/block/moe.rs:744-859;
+ * kernels_sparse_moe.inc.cu:323-397,787-946). */
+int nerva_hip_moe_fp8_experts(const NervaHipMoeFp8Request *request, void *stream, int32_t *hip_error);
+
+typedef struct NervaHipMoeRouteRequest {
+  uint32_t num_experts, top_k, normalize;
+  const float *logits;       /* device [num_experts] */
+  uint32_t *expert_ids;      /* device [top_k] */
+  float *expert_weights;     /* device [top_k] */
+} NervaHipMoeRouteRequest;
+
+/* softmax -> top-k by (probability desc, index asc) -> optional renormalisation
+ * (select_moe_route_for_logits Softmax arm, precision/block/moe.rs:1107-1155,1303-1326). */
+int nerva_hip_moe_route_softmax(const NervaHipMoeRouteRequest *request, void *stream,
+                                int32_t *hip_error);
+
+/* ------------------------------------------------------------------------
+ * Device memory / stream plumbing for hosts that have no HIP binding of their own.
+ * ---------------------------------------------------------------------- */
+int nerva_hip_malloc(void **device_ptr, uint64_t bytes);
+int nerva_hip_free(void *device_ptr);
+int nerva_hip_memcpy_h2d(void *device_dst, const void *host_src, uint64_t bytes);
+int nerva_hip_memcpy_d2h(void *host_dst, const void *device_src, uint64_t bytes);
+int nerva_hip_memset(void *device_dst, int value, uint64_t bytes);
+int nerva_hip_stream_synchronize(void *stream);
+/* Counts hipMalloc/hipHostMalloc calls made by the library since load (hot-path allocation audit). */
+uint64_t nerva_hip_allocation_count(void);
+
+/* Synthetic tensors generated on the device by the counter-based generator the
+ * tests' CPU oracle also implements (values are bit-identical on both sides):
+ * value = mean + float(2*sum12(u16) - 786420) * (std/131072), rounded to `dtype`. */
+int nerva_hip_synth_fill_16(void *device_dst, uint32_t dtype, uint64_t seed, uint64_t tensor_id,
+                            uint64_t count, float mean, float std);
+int nerva_hip_synth_fill_f32(void *device_dst, uint64_t seed, uint64_t tensor_id, uint64_t count,
+                             float mean, float std);
+int nerva_hip_synth_fill_fp8_block(void *device_weights, void *device_scales, uint64_t seed,
+                                   uint64_t tensor_id, uint64_t rows, uint64_t cols, uint64_t block,
+                                   float std);
+
+/* ------------------------------------------------------------------------
+ * Benchmark helpers (no reference counterpart).
+ * ---------------------------------------------------------------------- */
+
+/* Same request as session_create but every weight pointer is ignored: weights
+ * are generated on the device (N(0, weight_std), norms 1 + N(0, weight_std)) from
+ * `seed`, so a 16 GB model never crosses PCIe. Tensor ids: 1 embeddings,
+ * 2 final_norm, 3 lm_head, 16*(layer+1)+k for the k-th pointer of the layer in
+ * struct order (rms_attn=0, rms_mlp=1, w_q=2, w_k=4, q_norm=5, k_norm=6, w_v=7,
+ * w_o=8, w_gate=13, w_up=14, w_down=15). */
+int nerva_hip_bench_session_create_synthetic(
+    const NervaHipHfDecodeSequenceSessionCreateRequest *request, uint64_t seed, float weight_std,
+    uint32_t with_qk_norm, NervaHipHfDecodeSequenceSessionCreateResult *out,
+    NervaHipHfDecodeSequenceSession **session);
+
+typedef struct NervaHipStepProfile {
+  int32_t status, hip_error;
+  uint32_t position, launches;
+  /* average device ns per launch over `repeats` un-graphed steps, hipEvent pairs around each launch */
+  uint64_t embed_ns, qkv_ns, attention_ns, o_ns, gate_up_ns, down_ns, lm_head_ns, total_ns;
+  uint64_t qkv_bytes, attention_bytes, o_bytes, gate_up_bytes, down_bytes, lm_head_bytes;
+} NervaHipStepProfile;
+
+/* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT
+ * advancing it or publishing tokens, bracketing each launch with hipEvents on
+ * the session stream (the reference's detailed_profile pass:
+ * session_profile.inc.cu:35-56, session_decode_prefill.inc.cu:374-809). */
+int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uint32_t repeats,
+                                   NervaHipStepProfile *out);
+
+/* Reads back the f32 logits of the last sampled position (vocab_size floats) and
+ * one KV row (kv_heads*head_dim 16-bit values each for K and V) for parity tests. */
+int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *session, float *host_logits);
+int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *session, uint32_t layer, uint32_t token,
+                              uint16_t *host_k, uint16_t *host_v);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NERVA_HIP_API_H_ */

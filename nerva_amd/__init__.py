@@ -1,0 +1,15 @@
+"""nerva_amd: MI355X (gfx950) batch-1 decode backend behind the nerva C ABI.
+
+The product is nerva_amd/libnerva_hip.so (HIP kernels + C ABI, see
+include/nerva_hip_api.h). This package only loads it and offers thin numpy
+plumbing for tests and benchmarks; all arithmetic runs in the HIP library and
+importing a compute helper without the built library raises.
+"""
+from . import abi
+from .runtime import (DeviceBuffer, Device, device_available, gemv, fp8_gemv, paged_attention,
+                      argmax, moe_fp8_experts, moe_route_softmax, PagedKvCache)
+from .session import DecodeSession, ModelWeights, Qwen3_8B
+
+__all__ = ["abi", "DeviceBuffer", "Device", "device_available", "gemv", "fp8_gemv",
+           "paged_attention", "argmax", "moe_fp8_experts", "moe_route_softmax", "PagedKvCache",
+           "DecodeSession", "ModelWeights", "Qwen3_8B"]

@@ -1,0 +1,511 @@
+// Fused decode attention for one new token:
+//   bias -> per-head RMSNorm (q_norm/k_norm) -> half-split RoPE -> K/V rounded to
+//   16 bits and appended to the paged cache -> split-KV online-softmax attention
+//   over keys 0..pos -> merge of the splits -> 16-bit attention output.
+// Reference: hf_layer_qkv_prepare_kernel / chunk kernels / reduce kernel
+// (kernels.cu:287-555, attention_kernels.cu:263-760), per_head_rms_norm
+// (precision/block/ops.rs:52-73), apply_rotary_to_heads (common/rope.rs:54-79),
+// exact_blockwise_attention_into (attention/exact/run.rs:13-127).
+//
+// gfx950 mapping of the fast path (head_dim 128, G = heads/kv_heads in {1,2,4,8}):
+//   grid (kv_heads, splits); a wave owns whole 16-token KV blocks. One block tile
+//   of one kv head is 4 KiB contiguous, fetched by four 1 KiB load instructions
+//   in exactly the register layout the math wants: load i, lane l holds the 8
+//   dims (l%16)*8.. of token 4i + l/16. So a 16-lane DPP row reduces one q.k, the
+//   probabilities land in the lanes that hold the matching V slice, and K/V never
+//   need a shuffle through LDS; the next tile's 8 loads are in flight while the
+//   current one is consumed. All G query heads of the kv head share each K/V
+//   register (1 unpack, G FMAs). LDS only carries q and the cross-wave merge.
+//   The last workgroup to finish a kv head merges its split partials (arrival
+//   counter; nobody waits), so a layer needs no separate reduce launch.
+#include "attn_decode.cuh"
+
+namespace nv {
+
+namespace {
+
+constexpr int kHD = 128;
+
+// Sum over the 16 lanes of a DPP row; every lane of the row gets the total.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
+template <uint32_t DT>
+__device__ __forceinline__ void unpack8(const uint4 &v, float (&f)[8]) {
+  unpack2<DT>(v.x, f[0], f[1]);
+  unpack2<DT>(v.y, f[2], f[3]);
+  unpack2<DT>(v.z, f[4], f[5]);
+  unpack2<DT>(v.w, f[6], f[7]);
+}
+
+// One wave prepares one 128-wide head: lane l owns the RoPE pair (l, l+64).
+// out[] receives f32; when out16 != null the value is rounded first and the 16-bit
+// copy is stored too (K/V that go to the cache).
+template <uint32_t DT>
+__device__ __forceinline__ void prep_head128(const float *src, const uint16_t *bias,
+                                             const uint16_t *gamma, const float *rope_freq,
+                                             uint32_t pos, float eps, int lane, float *out,
+                                             uint16_t *out16) {
+  float x0 = src[lane], x1 = src[lane + 64];
+  if (bias != nullptr) {
+    x0 += dec16<DT>(bias[lane]);
+    x1 += dec16<DT>(bias[lane + 64]);
+  }
+  if (gamma != nullptr) {
+    const float ss = wave_sum(x0 * x0 + x1 * x1);
+    const float scale = 1.0f / sqrtf(ss / 128.0f + eps);
+    x0 *= scale * dec16<DT>(gamma[lane]);
+    x1 *= scale * dec16<DT>(gamma[lane + 64]);
+  }
+  if (rope_freq != nullptr) {
+    const float angle = static_cast<float>(pos) / rope_freq[lane];
+    float s, c;
+    sincosf(angle, &s, &c);
+    const float r0 = x0 * c - x1 * s;
+    const float r1 = x1 * c + x0 * s;
+    x0 = r0;
+    x1 = r1;
+  }
+  if (out16 != nullptr) {
+    out16[lane] = enc16<DT>(x0);
+    out16[lane + 64] = enc16<DT>(x1);
+    x0 = round16<DT>(x0);
+    x1 = round16<DT>(x1);
+  }
+  if (out != nullptr) {
+    out[lane] = x0;
+    out[lane + 64] = x1;
+  }
+}
+
+template <uint32_t DT, int G>
+__global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
+  __shared__ __align__(16) float q_s[G][kHD];
+  __shared__ __align__(16) uint16_t knew[kHD];
+  __shared__ __align__(16) uint16_t vnew[kHD];
+  __shared__ float wm[kWavesPerBlock][G];
+  __shared__ float wl[kWavesPerBlock][G];
+  __shared__ __align__(16) float wacc[kWavesPerBlock][G][kHD];
+  __shared__ uint32_t is_last;
+
+  const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
+  if (p.cursor != nullptr && pos >= p.max_steps) return;
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t kvh = blockIdx.x, split = blockIdx.y, S = gridDim.y;
+  const uint32_t n_keys = pos + 1;
+  const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
+  const uint32_t bps = (nblk + S - 1) / S;
+  const uint32_t b0 = split * bps;
+  const uint32_t b1 = min(nblk, b0 + bps);
+  const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
+  const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
+  const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
+
+  // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
+  for (int g = wave; g < G; g += kWavesPerBlock) {
+    const uint32_t h = kvh * G + g;
+    prep_head128<DT>(p.qkv + h * kHD, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq,
+                     pos, p.eps, lane, q_s[g], nullptr);
+  }
+  if (owns_new) {
+    if (wave == (G % kWavesPerBlock)) {
+      prep_head128<DT>(p.qkv + A + kvh * kHD, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm,
+                       p.rope_freq, pos, p.eps, lane, nullptr, knew);
+    } else if (wave == ((G + 1) % kWavesPerBlock)) {
+      prep_head128<DT>(p.qkv + A + KV + kvh * kHD, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr,
+                       nullptr, pos, p.eps, lane, nullptr, vnew);
+    }
+  }
+  __syncthreads();
+  if (owns_new && wave == 0 && lane < 32) {
+    // publish the rounded row to the cache: 16 lanes x 16 B for K, 16 for V
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[new_block], kvh);
+    const int piece = lane & 15;
+    uint16_t *dst = (lane < 16 ? p.k_cache : p.v_cache) + tile + new_row * kHD + piece * 8;
+    const uint16_t *src = (lane < 16 ? knew : vnew) + piece * 8;
+    *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
+  }
+
+  // ---- per-lane query slice: dims part*8..part*8+7 of every head of the group
+  const int part = lane & 15, trow = lane >> 4;
+  float qr[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float4 a = *reinterpret_cast<const float4 *>(&q_s[g][part * 8]);
+    const float4 b = *reinterpret_cast<const float4 *>(&q_s[g][part * 8 + 4]);
+    qr[g][0] = a.x; qr[g][1] = a.y; qr[g][2] = a.z; qr[g][3] = a.w;
+    qr[g][4] = b.x; qr[g][5] = b.y; qr[g][6] = b.z; qr[g][7] = b.w;
+  }
+  const float scale = 1.0f / sqrtf(static_cast<float>(kHD));
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[g][d] = 0.0f;
+  }
+
+  uint4 kreg[4], vreg[4];
+  uint32_t b = b0 + wave;
+  if (b < b1) {
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kreg[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
+      vreg[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
+    }
+  }
+  for (; b < b1; b += kWavesPerBlock) {
+    // issue the next tile's loads before touching the current one
+    uint4 knext[4], vnext[4];
+    const uint32_t bn = b + kWavesPerBlock;
+    if (bn < b1) {
+      const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[bn], kvh);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        knext[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
+        vnext[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
+      }
+    }
+    if (owns_new && b == new_block) {
+      // the row written above may not be visible to this CU's loads yet: splice it from LDS
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (static_cast<uint32_t>(i * 4 + trow) == new_row) {
+          kreg[i] = *reinterpret_cast<const uint4 *>(knew + part * 8);
+          vreg[i] = *reinterpret_cast<const uint4 *>(vnew + part * 8);
+        }
+      }
+    }
+    float s[G][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float kf[8];
+      unpack8<DT>(kreg[i], kf);
+      const bool valid = b * kKvBlockTokens + i * 4 + trow < n_keys;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(qr[g][e], kf[e], d);
+        d = row16_sum(d) * scale;
+        s[g][i] = valid ? d : -INFINITY;
+      }
+    }
+    float pr[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mb = fmaxf(fmaxf(s[g][0], s[g][1]), fmaxf(s[g][2], s[g][3]));
+      mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
+      mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+      const float m_new = fmaxf(m[g], mb);   // finite: every processed tile has a valid token
+      const float alpha = expf(m[g] - m_new);
+      float psum = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pr[g][i] = expf(s[g][i] - m_new);
+        psum += pr[g][i];
+      }
+      l[g] = l[g] * alpha + psum;
+      m[g] = m_new;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) acc[g][d] *= alpha;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float vf[8];
+      unpack8<DT>(vreg[i], vf);
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(pr[g][i], vf[d], acc[g][d]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kreg[i] = knext[i];
+      vreg[i] = vnext[i];
+    }
+  }
+
+  // ---- merge the four token rows of the wave, then the four waves
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    l[g] += __shfl_xor(l[g], 16, kWave);
+    l[g] += __shfl_xor(l[g], 32, kWave);
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      acc[g][d] += __shfl_xor(acc[g][d], 16, kWave);
+      acc[g][d] += __shfl_xor(acc[g][d], 32, kWave);
+    }
+    if (lane < 16) {
+      *reinterpret_cast<float4 *>(&wacc[wave][g][part * 8]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+      *reinterpret_cast<float4 *>(&wacc[wave][g][part * 8 + 4]) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+    }
+    if (lane == 0) {
+      wm[wave][g] = m[g];
+      wl[wave][g] = l[g];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < G * kHD; e += kBlock) {
+    const int g = e / kHD, d = e % kHD;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) M = fmaxf(M, wm[w][g]);
+    float L = 0.0f, o = 0.0f;
+    if (M > -INFINITY) {
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        const float f = expf(wm[w][g] - M);  // exp(-inf) = 0 for idle waves
+        L += wl[w][g] * f;
+        o += wacc[w][g][d] * f;
+      }
+    }
+    const uint32_t h = kvh * G + g;
+    p.part_acc[(static_cast<uint64_t>(h) * S + split) * kHD + d] = o;
+    if (d == 0) {
+      p.part_m[h * S + split] = M;
+      p.part_l[h * S + split] = L;
+    }
+  }
+
+  // ---- last workgroup of this kv head merges the splits
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    const uint32_t ticket =
+        __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = ticket == S - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  for (int e = threadIdx.x; e < G * kHD; e += kBlock) {
+    const int g = e / kHD, d = e % kHD;
+    const uint32_t h = kvh * G + g;
+    float M = -INFINITY;
+    for (uint32_t s2 = 0; s2 < S; ++s2) M = fmaxf(M, p.part_m[h * S + s2]);
+    float L = 0.0f, o = 0.0f;
+    for (uint32_t s2 = 0; s2 < S; ++s2) {
+      const float pm = p.part_m[h * S + s2];
+      if (pm > -INFINITY) {
+        const float f = expf(pm - M);
+        L += p.part_l[h * S + s2] * f;
+        o += p.part_acc[(static_cast<uint64_t>(h) * S + s2) * kHD + d] * f;
+      }
+    }
+    if (L > 0.0f && isfinite(L)) o /= L;
+    if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
+    p.out16[h * kHD + d] = enc16<DT>(o);
+  }
+  if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Any head_dim (even when RoPE is on) / any group size: one workgroup per query
+// head, waves stride over tokens, lanes over dims. Used for shapes the fast path
+// does not cover (the tiny known-answer models).
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock) void attn_generic_kernel(AttnParams p) {
+  extern __shared__ __align__(16) float sm[];
+  __shared__ float red[kWavesPerBlock];
+  __shared__ float wm[kWavesPerBlock], wl[kWavesPerBlock];
+  const uint32_t hd = p.head_dim, half = hd / 2;
+  float *q = sm;                 // [hd]
+  float *kn = sm + hd;           // [hd] rounded new key
+  float *vn = sm + 2 * hd;       // [hd] rounded new value
+  float *wacc = sm + 3 * hd;     // [waves][hd]
+
+  const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
+  if (p.cursor != nullptr && pos >= p.max_steps) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t h = blockIdx.x, group = p.heads / p.kv_heads, kvh = h / group;
+  const uint32_t A = p.heads * hd, KV = p.kv_heads * hd;
+  const uint32_t n_keys = pos + 1;
+
+  // q: bias -> per-head norm -> RoPE
+  float ss = 0.0f;
+  for (uint32_t d = threadIdx.x; d < hd; d += kBlock) {
+    float v = p.qkv[h * hd + d];
+    if (p.q_bias) v += dec16<DT>(p.q_bias[h * hd + d]);
+    q[d] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  if (p.q_norm) {
+    const float sc = 1.0f / sqrtf(ss / static_cast<float>(hd) + p.eps);
+    for (uint32_t d = threadIdx.x; d < hd; d += kBlock) q[d] *= sc * dec16<DT>(p.q_norm[d]);
+  }
+  __syncthreads();
+  if (p.rope_freq) {
+    for (uint32_t i = threadIdx.x; i < half; i += kBlock) {
+      const float angle = static_cast<float>(pos) / p.rope_freq[i];
+      float s, c;
+      sincosf(angle, &s, &c);
+      const float a = q[i], b = q[i + half];
+      q[i] = a * c - b * s;
+      q[i + half] = b * c + a * s;
+    }
+  }
+  if (p.append) {
+    float ks = 0.0f;
+    for (uint32_t d = threadIdx.x; d < hd; d += kBlock) {
+      float kv = p.qkv[A + kvh * hd + d];
+      if (p.k_bias) kv += dec16<DT>(p.k_bias[kvh * hd + d]);
+      kn[d] = kv;
+      ks += kv * kv;
+      float vv = p.qkv[A + KV + kvh * hd + d];
+      if (p.v_bias) vv += dec16<DT>(p.v_bias[kvh * hd + d]);
+      vn[d] = vv;
+    }
+    ks = block_sum(ks, red);
+    if (p.k_norm) {
+      const float sc = 1.0f / sqrtf(ks / static_cast<float>(hd) + p.eps);
+      for (uint32_t d = threadIdx.x; d < hd; d += kBlock) kn[d] *= sc * dec16<DT>(p.k_norm[d]);
+    }
+    __syncthreads();
+    if (p.rope_freq) {
+      for (uint32_t i = threadIdx.x; i < half; i += kBlock) {
+        const float angle = static_cast<float>(pos) / p.rope_freq[i];
+        float s, c;
+        sincosf(angle, &s, &c);
+        const float a = kn[i], b = kn[i + half];
+        kn[i] = a * c - b * s;
+        kn[i + half] = b * c + a * s;
+      }
+    }
+    __syncthreads();
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, hd, p.layer,
+                                         p.table[pos / kKvBlockTokens], kvh) +
+                          static_cast<uint64_t>(pos % kKvBlockTokens) * hd;
+    for (uint32_t d = threadIdx.x; d < hd; d += kBlock) {
+      const uint16_t k16 = enc16<DT>(kn[d]), v16 = enc16<DT>(vn[d]);
+      if (h % group == 0) {
+        p.k_cache[tile + d] = k16;
+        p.v_cache[tile + d] = v16;
+      }
+      kn[d] = dec16<DT>(k16);
+      vn[d] = dec16<DT>(v16);
+    }
+  }
+  __syncthreads();
+
+  constexpr int kMaxPerLane = 8;  // head_dim <= 512
+  float acc[kMaxPerLane];
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) acc[j] = 0.0f;
+  float m = -INFINITY, l = 0.0f;
+  const float scale = 1.0f / sqrtf(static_cast<float>(hd));
+  for (uint32_t t = wave; t < n_keys; t += kWavesPerBlock) {
+    const bool fresh = p.append && t == pos;
+    const uint64_t row = kv_tile_offset(p.block_count, p.kv_heads, hd, p.layer,
+                                        p.table[t / kKvBlockTokens], kvh) +
+                         static_cast<uint64_t>(t % kKvBlockTokens) * hd;
+    float partial = 0.0f;
+    for (uint32_t d = lane; d < hd; d += kWave)
+      partial = fmaf(q[d], fresh ? kn[d] : dec16<DT>(p.k_cache[row + d]), partial);
+    const float score = wave_sum(partial) * scale;
+    const float m_new = fmaxf(m, score);
+    const float alpha = l == 0.0f ? 0.0f : expf(m - m_new);
+    const float pnew = expf(score - m_new);
+#pragma unroll
+    for (int j = 0; j < kMaxPerLane; ++j) {
+      const uint32_t d = lane + j * kWave;
+      if (d < hd) acc[j] = acc[j] * alpha + (fresh ? vn[d] : dec16<DT>(p.v_cache[row + d])) * pnew;
+    }
+    l = l * alpha + pnew;
+    m = m_new;
+  }
+#pragma unroll
+  for (int j = 0; j < kMaxPerLane; ++j) {
+    const uint32_t d = lane + j * kWave;
+    if (d < hd) wacc[wave * hd + d] = acc[j];
+  }
+  if (lane == 0) {
+    wm[wave] = m;
+    wl[wave] = l;
+  }
+  __syncthreads();
+  float M = -INFINITY;
+  for (int w = 0; w < kWavesPerBlock; ++w) M = fmaxf(M, wm[w]);
+  for (uint32_t d = threadIdx.x; d < hd; d += kBlock) {
+    float L = 0.0f, o = 0.0f;
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      if (wm[w] > -INFINITY) {
+        const float f = expf(wm[w] - M);
+        L += wl[w] * f;
+        o += wacc[w * hd + d] * f;
+      }
+    }
+    if (L > 0.0f && isfinite(L)) o /= L;
+    if (p.out_f32) p.out_f32[h * hd + d] = o;
+    p.out16[h * hd + d] = enc16<DT>(o);
+  }
+}
+
+template <uint32_t DT>
+hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
+  const uint32_t group = p.heads / p.kv_heads;
+  const bool fast = p.head_dim == kHD && (group == 1 || group == 2 || group == 4 || group == 8) &&
+                    p.part_acc != nullptr && p.splits >= 1;
+  if (fast) {
+    const dim3 grid(p.kv_heads, p.splits);
+    switch (group) {
+      case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1>), grid, dim3(kBlock), 0, stream, p); break;
+      case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2>), grid, dim3(kBlock), 0, stream, p); break;
+      case 4: hipLaunchKernelGGL((attn_fast_kernel<DT, 4>), grid, dim3(kBlock), 0, stream, p); break;
+      default: hipLaunchKernelGGL((attn_fast_kernel<DT, 8>), grid, dim3(kBlock), 0, stream, p); break;
+    }
+  } else {
+    if (p.head_dim > 512) return hipErrorInvalidValue;
+    const size_t lds = static_cast<size_t>(3 + kWavesPerBlock) * p.head_dim * sizeof(float);
+    hipLaunchKernelGGL((attn_generic_kernel<DT>), dim3(p.heads), dim3(kBlock), lds, stream, p);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+uint64_t attn_workspace_bytes(uint32_t heads, uint32_t head_dim) {
+  const uint64_t acc = static_cast<uint64_t>(heads) * kAttnMaxSplits * head_dim * sizeof(float);
+  const uint64_t ml = static_cast<uint64_t>(heads) * kAttnMaxSplits * sizeof(float) * 2;
+  return acc + ml + 1024 * sizeof(uint32_t);
+}
+
+void attn_bind_workspace(AttnParams &p, void *workspace) {
+  char *base = static_cast<char *>(workspace);
+  const uint64_t acc = static_cast<uint64_t>(p.heads) * kAttnMaxSplits * p.head_dim * sizeof(float);
+  const uint64_t ml = static_cast<uint64_t>(p.heads) * kAttnMaxSplits * sizeof(float);
+  p.part_acc = reinterpret_cast<float *>(base);
+  p.part_m = reinterpret_cast<float *>(base + acc);
+  p.part_l = reinterpret_cast<float *>(base + acc + ml);
+  p.counters = reinterpret_cast<uint32_t *>(base + acc + 2 * ml);
+}
+
+hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t stream) {
+  if (p.qkv == nullptr || p.k_cache == nullptr || p.v_cache == nullptr || p.table == nullptr ||
+      p.out16 == nullptr)
+    return hipErrorInvalidValue;
+  if (p.heads == 0 || p.kv_heads == 0 || p.head_dim == 0 || p.heads % p.kv_heads != 0 ||
+      p.block_count == 0 || p.kv_heads > 1024)
+    return hipErrorInvalidValue;
+  if (p.rope_freq != nullptr && p.head_dim % 2 != 0) return hipErrorInvalidValue;
+  if (p.splits > kAttnMaxSplits) return hipErrorInvalidValue;
+  if (p.cursor == nullptr &&
+      static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+    return hipErrorInvalidValue;
+  if (dtype == kBF16) return launch_dt<kBF16>(p, stream);
+  if (dtype == kF16) return launch_dt<kF16>(p, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace nv

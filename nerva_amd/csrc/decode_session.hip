@@ -1,0 +1,1123 @@
+// Decode session: one static device arena, weights resident, paged KV cache,
+// the whole decode step captured once as a hipGraph and replayed per token.
+// Replaces the reference's session object and lifecycle entry points
+// (native/cuda/hf_decode_sequence/session_api_lifecycle.inc.cu:1-1311,
+// session_decode_prefill.inc.cu:74-372, session_graph_result.inc.cu:87-209).
+//
+// One decode step is 2 + 5*layers launches, with no host round trip:
+//   embed               x = f32(emb[token]); token = prompt[pos] or slots[pos-1].token
+//   per layer
+//     qkv   GEMV  [rmsnorm(x, g_attn) prologue]                  -> qkv f32
+//     attn  q/k norm + RoPE + KV append + split-KV attention      -> attn 16-bit
+//     o     GEMV  [+ o_bias + x epilogue]                         -> r f32
+//     gate_up GEMV [rmsnorm(r, g_mlp) prologue, silu(g)*u epilogue] -> ff 16-bit
+//     down  GEMV  [+ r epilogue]                                  -> x f32
+//   lm_head GEMV [rmsnorm(x, g_final) prologue, argmax epilogue]  -> slot[pos], cursor = pos+1
+// Every kernel reads the position from device memory, so one captured graph
+// serves every position and every prompt length.
+#include <math.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "argmax.cuh"
+#include "attn_decode.cuh"
+#include "gemv_stream.cuh"
+#include "runtime_state.hpp"
+#include "synth_fill.cuh"
+
+using namespace nv;
+
+namespace {
+
+using Slot = NervaHipSyntheticTokenSlot;
+
+struct LayerDev {
+  const uint16_t *rms_attn, *rms_mlp, *wqkv, *q_norm, *k_norm, *q_bias, *k_bias, *v_bias, *wo, *o_bias,
+      *wgu, *wdown;
+};
+
+enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
+enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLKinds };
+
+struct StepProfiler {
+  hipStream_t stream;
+  std::vector<hipEvent_t> events;  // pairs
+  std::vector<int> kinds;
+  size_t used = 0;
+  hipError_t before(int kind) {
+    if (used + 2 > events.size()) {
+      for (int i = 0; i < 2; ++i) {
+        hipEvent_t e;
+        hipError_t err = hipEventCreate(&e);
+        if (err != hipSuccess) return err;
+        events.push_back(e);
+      }
+    }
+    kinds.push_back(kind);
+    return hipEventRecord(events[used], stream);
+  }
+  hipError_t after() {
+    hipError_t err = hipEventRecord(events[used + 1], stream);
+    used += 2;
+    return err;
+  }
+  ~StepProfiler() {
+    for (hipEvent_t e : events) (void)hipEventDestroy(e);
+  }
+};
+
+}  // namespace
+
+struct NervaHipHfDecodeSequenceSession {
+  uint32_t dtype = 0, hidden = 0, heads = 0, kv_heads = 0, head_dim = 0, intermediate = 0, vocab = 0,
+           layers = 0, max_ctx = 0;
+  float eps = 0.0f, theta = 0.0f;
+  hipStream_t stream = nullptr;
+  char *arena = nullptr;
+  uint64_t arena_bytes = 0;
+  char *pinned = nullptr;
+  uint64_t pinned_bytes = 0;
+  std::vector<LayerDev> layer;
+  const uint16_t *emb = nullptr, *final_norm = nullptr, *lm_head = nullptr;
+  uint16_t *kc = nullptr, *vc = nullptr;
+  uint32_t block_count = 0;
+  uint32_t *table = nullptr, *prompt = nullptr, *state = nullptr;  // state[0] cursor, state[1] prompt count
+  Slot *slots = nullptr;
+  float *x = nullptr, *r = nullptr, *qkv = nullptr, *logits = nullptr, *rope_freq = nullptr;
+  uint16_t *attn16 = nullptr, *ff16 = nullptr;
+  void *attn_ws = nullptr, *sample_ws = nullptr;
+  uint32_t attn_splits = 1;
+  Slot *host_slots = nullptr;
+  uint32_t *host_prompt = nullptr;
+  uint32_t *host_state = nullptr;
+  hipGraph_t graph[2] = {nullptr, nullptr};
+  hipGraphExec_t exec[2] = {nullptr, nullptr};
+  uint64_t graph_nodes[2] = {0, 0};
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  // echo of the caller's weight plan
+  uint32_t planned_weight_blocks = 0, planned_gpu_resident_blocks = 0, planned_gpu_staged_blocks = 0,
+           planned_weight_descriptor_count = 0;
+  uint64_t planned_weight_bytes = 0, planned_gpu_resident_weight_bytes = 0,
+           planned_gpu_staged_weight_bytes = 0, planned_weight_descriptor_hash = 0;
+  uint64_t resident_weight_bytes = 0, kv_bytes = 0;
+  // active sequence
+  bool started = false, finished = false;
+  uint32_t prompt_count = 0, observed = 0, cursor = 0, seed_token = 0, has_eos = 0, eos = 0;
+};
+
+using Session = NervaHipHfDecodeSequenceSession;
+
+namespace {
+
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, const uint32_t *prompt,
+                                                       const Slot *slots, const uint32_t *state,
+                                                       uint32_t max_steps, uint32_t hidden,
+                                                       uint32_t vocab, float *x) {
+  const uint32_t pos = state[0];
+  if (pos >= max_steps) return;
+  uint32_t token = pos < state[1] ? prompt[pos] : slots[pos - 1].token;
+  if (token >= vocab) token = 0;  // prompts are validated on the host; sampled ids are < vocab
+  const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < hidden; i += gridDim.x * kBlock)
+    x[i] = dec16<DT>(row[i]);
+}
+
+__global__ void advance_cursor_kernel(uint32_t *state, uint32_t max_steps) {
+  if (threadIdx.x == 0 && blockIdx.x == 0 && state[0] < max_steps) state[0] = state[0] + 1u;
+}
+
+struct Carver {
+  uint64_t offset = 0;
+  uint64_t take(uint64_t bytes) {
+    const uint64_t at = offset;
+    offset += (bytes + 255u) & ~uint64_t{255};
+    return at;
+  }
+};
+
+bool layer_supported(const NervaHipHfDecodeChainLayer &l) {
+  if (l.w_q_gate || l.w_router || l.w_expert_gate_up || l.w_expert_down || l.w_shared_expert_gate ||
+      l.w_shared_expert_up || l.w_shared_expert_down || l.w_shared_expert_router || l.w_linear_conv ||
+      l.w_linear_qkv || l.w_linear_z || l.w_linear_b || l.w_linear_a || l.w_linear_dt_bias ||
+      l.w_linear_a_log || l.w_linear_norm || l.w_linear_out)
+    return false;
+  if (l.linear_key_heads || l.linear_value_heads || l.linear_key_head_dim || l.linear_value_head_dim ||
+      l.linear_conv_kernel)
+    return false;
+  if (l.mlp_kind != NERVA_HIP_MLP_DENSE || l.attention_kind != NERVA_HIP_ATTENTION_FULL) return false;
+  if (l.moe_intermediate || l.shared_expert_intermediate || l.num_experts || l.experts_per_token)
+    return false;
+  if (l.deepseek_mode || l.deepseek_flags || l.deepseek_hc_mult || l.deepseek_q_lora_rank ||
+      l.deepseek_kv_lora_rank || l.deepseek_o_lora_rank || l.deepseek_compress_ratio ||
+      l.deepseek_index_topk)
+    return false;
+  return true;
+}
+
+bool layer_has_weights(const NervaHipHfDecodeChainLayer &l) {
+  return l.rms_attn_weight && l.rms_mlp_weight && l.w_q && l.w_k && l.w_v && l.w_o && l.w_gate &&
+         l.w_up && l.w_down;
+}
+
+void destroy_session(Session *s) {
+  if (s == nullptr) return;
+  if (s->stream) (void)hipStreamSynchronize(s->stream);
+  for (int i = 0; i < 2; ++i) {
+    if (s->exec[i]) (void)hipGraphExecDestroy(s->exec[i]);
+    if (s->graph[i]) (void)hipGraphDestroy(s->graph[i]);
+  }
+  if (s->ev0) (void)hipEventDestroy(s->ev0);
+  if (s->ev1) (void)hipEventDestroy(s->ev1);
+  if (s->arena) (void)hipFree(s->arena);
+  if (s->pinned) (void)hipHostFree(s->pinned);
+  if (s->stream) (void)hipStreamDestroy(s->stream);
+  delete s;
+}
+
+hipError_t run_launch(StepProfiler *prof, int kind, hipError_t (*fn)(void *), void *ctx) {
+  hipError_t err = hipSuccess;
+  if (prof) err = prof->before(kind);
+  if (err == hipSuccess) err = fn(ctx);
+  if (prof && err == hipSuccess) err = prof->after();
+  return err;
+}
+
+// Enqueue one step on the session stream (eagerly or under stream capture).
+hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
+  hipStream_t st = s->stream;
+  const uint32_t A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim;
+  hipError_t err = hipSuccess;
+#define NV_STEP(kind, expr)                         \
+  do {                                              \
+    if (prof && err == hipSuccess) err = prof->before(kind); \
+    if (err == hipSuccess) err = (expr);            \
+    if (prof && err == hipSuccess) err = prof->after();      \
+    if (err != hipSuccess) return err;              \
+  } while (0)
+
+  {
+    const uint32_t blocks = std::min<uint32_t>((s->hidden + kBlock - 1) / kBlock, 64u);
+    if (prof) err = prof->before(kLEmbed);
+    if (err != hipSuccess) return err;
+    if (s->dtype == kBF16)
+      hipLaunchKernelGGL(embed_kernel<kBF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
+                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x);
+    else
+      hipLaunchKernelGGL(embed_kernel<kF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
+                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x);
+    err = hipGetLastError();
+    if (prof && err == hipSuccess) err = prof->after();
+    if (err != hipSuccess) return err;
+  }
+  for (uint32_t l = 0; l < s->layers; ++l) {
+    const LayerDev &w = s->layer[l];
+    {
+      GemvParams p{};
+      p.w = w.wqkv;
+      p.xf = s->x;
+      p.gamma = w.rms_attn;
+      p.out_f32 = s->qkv;
+      p.rows = A + 2 * KV;
+      p.cols = s->hidden;
+      p.eps = s->eps;
+      p.cursor = s->state;
+      p.max_steps = s->max_ctx;
+      NV_STEP(kLQkv, launch_gemv(s->dtype, kProRmsNorm, kEpiF32, p, st));
+    }
+    {
+      AttnParams p{};
+      p.heads = s->heads;
+      p.kv_heads = s->kv_heads;
+      p.head_dim = s->head_dim;
+      attn_bind_workspace(p, s->attn_ws);
+      p.qkv = s->qkv;
+      p.q_norm = w.q_norm;
+      p.k_norm = w.k_norm;
+      p.q_bias = w.q_bias;
+      p.k_bias = w.k_bias;
+      p.v_bias = w.v_bias;
+      p.k_cache = s->kc;
+      p.v_cache = s->vc;
+      p.table = s->table;
+      p.rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
+      p.out_f32 = nullptr;
+      p.out16 = s->attn16;
+      p.layer = l;
+      p.block_count = s->block_count;
+      p.splits = s->attn_splits;
+      p.eps = s->eps;
+      p.cursor = s->state;
+      p.max_steps = s->max_ctx;
+      p.append = 1;
+      NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
+    }
+    {
+      GemvParams p{};
+      p.w = w.wo;
+      p.x16 = s->attn16;
+      p.bias = w.o_bias;
+      p.residual = s->x;
+      p.out_f32 = s->r;
+      p.rows = s->hidden;
+      p.cols = A;
+      p.cursor = s->state;
+      p.max_steps = s->max_ctx;
+      NV_STEP(kLO, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
+    }
+    {
+      GemvParams p{};
+      p.w = w.wgu;
+      p.xf = s->r;
+      p.gamma = w.rms_mlp;
+      p.out16 = s->ff16;
+      p.rows = s->intermediate;
+      p.cols = s->hidden;
+      p.eps = s->eps;
+      p.cursor = s->state;
+      p.max_steps = s->max_ctx;
+      NV_STEP(kLGateUp, launch_gemv(s->dtype, kProRmsNorm, kEpiSwiglu, p, st));
+    }
+    {
+      GemvParams p{};
+      p.w = w.wdown;
+      p.x16 = s->ff16;
+      p.residual = s->r;
+      p.out_f32 = s->x;
+      p.rows = s->hidden;
+      p.cols = s->intermediate;
+      // prompt tokens carry a 16-bit hidden state between layers (prefill_kernels.cu:494-508)
+      p.round_out = mode == kDecodeStep ? 0u : 1u;
+      p.cursor = s->state;
+      p.max_steps = s->max_ctx;
+      NV_STEP(kLDown, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
+    }
+  }
+  if (mode == kPromptStep) {
+    if (prof) err = prof->before(kLAdvance);
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(advance_cursor_kernel, dim3(1), dim3(64), 0, st, s->state, s->max_ctx);
+    err = hipGetLastError();
+    if (prof && err == hipSuccess) err = prof->after();
+    return err;
+  }
+  GemvParams p{};
+  p.w = s->lm_head;
+  p.xf = s->x;
+  p.gamma = s->final_norm;
+  p.out_f32 = s->logits;
+  p.rows = s->vocab;
+  p.cols = s->hidden;
+  p.eps = s->eps;
+  p.cursor = s->state;
+  p.max_steps = s->max_ctx;
+  sample_bind_workspace(p.sample, s->sample_ws);
+  p.sample.slots = s->slots;
+  p.sample.cursor_rw = s->state;
+  NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st));
+#undef NV_STEP
+  return hipSuccess;
+}
+
+// graph index 0: decode step, 1: prompt step
+hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
+  if (s->exec[which] != nullptr) {
+    if (out) {
+      out->graph_nodes = s->graph_nodes[which];
+      out->graph_cache_hits += 1;
+    }
+    return hipSuccess;
+  }
+  hipGraph_t graph = nullptr;
+  hipError_t err = hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal);
+  if (err != hipSuccess) return err;
+  hipError_t step_err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
+  err = hipStreamEndCapture(s->stream, &graph);
+  if (step_err != hipSuccess) err = step_err;
+  size_t nodes = 0;
+  if (err == hipSuccess) err = hipGraphGetNodes(graph, nullptr, &nodes);
+  hipGraphExec_t exec = nullptr;
+  if (err == hipSuccess) err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (err != hipSuccess) {
+    if (graph) (void)hipGraphDestroy(graph);
+    return err;
+  }
+  s->graph[which] = graph;
+  s->exec[which] = exec;
+  s->graph_nodes[which] = nodes;
+  if (out) {
+    out->graph_nodes = nodes;
+    out->graph_captures += 1;
+  }
+  return hipSuccess;
+}
+
+void fill_header(const Session *s, NervaHipHfDecodeSequenceResult *out, uint32_t steps,
+                 uint32_t seed_token) {
+  out->device_count = 1;
+  out->dtype = s->dtype;
+  out->hidden = s->hidden;
+  out->heads = s->heads;
+  out->kv_heads = s->kv_heads;
+  out->head_dim = s->head_dim;
+  out->intermediate = s->intermediate;
+  out->vocab_size = s->vocab;
+  out->layer_count = s->layers;
+  out->steps = steps;
+  out->seed_token = seed_token;
+  out->resident_weight_bytes = s->resident_weight_bytes;
+  out->planned_weight_blocks = s->planned_weight_blocks;
+  out->planned_gpu_resident_blocks = s->planned_gpu_resident_blocks;
+  out->planned_gpu_staged_blocks = s->planned_gpu_staged_blocks;
+  out->planned_weight_bytes = s->planned_weight_bytes;
+  out->planned_gpu_resident_weight_bytes = s->planned_gpu_resident_weight_bytes;
+  out->planned_gpu_staged_weight_bytes = s->planned_gpu_staged_weight_bytes;
+  out->descriptor_gpu_resident_h2d_bytes = s->planned_gpu_resident_weight_bytes;
+  out->descriptor_gpu_staged_h2d_bytes = s->planned_gpu_staged_weight_bytes;
+  out->planned_weight_descriptor_count = s->planned_weight_descriptor_count;
+  out->planned_weight_descriptor_hash = s->planned_weight_descriptor_hash;
+}
+
+bool sampler_valid(const NervaHipHfDecodeSamplerConfig &c) {
+  return isfinite(c.temperature) && c.temperature >= 0.0f && isfinite(c.top_p) && c.top_p > 0.0f &&
+         c.top_p <= 1.0f;
+}
+bool sampler_greedy(const NervaHipHfDecodeSamplerConfig &c) {
+  return !(c.temperature > 0.0f) || c.top_k == 1;  // sampler.cu:89
+}
+
+uint32_t observed_count(uint32_t steps, uint32_t has_eos, uint32_t eos, const Slot *slots) {
+  uint32_t count = steps;
+  for (uint32_t i = 0; i < steps; ++i) {
+    if (slots[i].completion != NERVA_HIP_SLOT_DEVICE_COMPLETE) {
+      count = i;
+      break;
+    }
+    if (has_eos != 0 && slots[i].token == eos) {
+      count = i + 1;
+      break;
+    }
+  }
+  return count;
+}
+
+bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
+  for (uint32_t i = 0; i < count; ++i) {
+    if (slots[i].request_id != NERVA_HIP_SLOT_REQUEST_ID || slots[i].sequence_id != NERVA_HIP_SLOT_SEQUENCE_ID ||
+        slots[i].completion != NERVA_HIP_SLOT_DEVICE_COMPLETE || slots[i].token_index != first_index + i)
+      return false;
+  }
+  return true;
+}
+
+hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t prompt_count,
+                          NervaHipHfDecodeSequenceResult *out) {
+  hipError_t err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  memcpy(s->host_prompt, prompt_tokens, static_cast<uint64_t>(prompt_count) * sizeof(uint32_t));
+  s->host_state[0] = 0;
+  s->host_state[1] = prompt_count;
+  if (err == hipSuccess)
+    err = hipMemcpyAsync(s->state, s->host_state, 2 * sizeof(uint32_t), hipMemcpyHostToDevice, s->stream);
+  if (err == hipSuccess)
+    err = hipMemcpyAsync(s->prompt, s->host_prompt, static_cast<uint64_t>(prompt_count) * sizeof(uint32_t),
+                         hipMemcpyHostToDevice, s->stream);
+  out->h2d_bytes = static_cast<uint64_t>(prompt_count) * sizeof(uint32_t);
+  return err;
+}
+
+int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool synthetic, uint64_t seed,
+                float weight_std, uint32_t with_qk_norm, NervaHipHfDecodeSequenceSessionCreateResult *out,
+                Session **session_out) {
+  if (!begin_result(out)) return -1;
+  if (session_out == nullptr) return -1;
+  *session_out = nullptr;
+  out->failure_stage = 1;
+  if (rq == nullptr || rq->dtype > 1 || rq->hidden == 0 || rq->heads == 0 || rq->kv_heads == 0 ||
+      rq->head_dim == 0 || rq->intermediate == 0 || rq->vocab_size == 0 || rq->layer_count == 0 ||
+      rq->max_context_tokens == 0 || rq->heads % rq->kv_heads != 0 || !(rq->rms_eps >= 0.0f) ||
+      !isfinite(rq->rms_eps) || !isfinite(rq->rope_theta))
+    return -1;
+  if (rq->rope_theta > 0.0f && rq->head_dim % 2 != 0) return -1;
+  if (!synthetic) {
+    if (rq->embeddings == nullptr || rq->layers == nullptr || rq->final_norm_weight == nullptr ||
+        rq->lm_head == nullptr)
+      return -1;
+    for (uint32_t l = 0; l < rq->layer_count; ++l)
+      if (!layer_has_weights(rq->layers[l])) return -1;
+  }
+  if (rq->planned_weight_descriptor_count != 0 && rq->planned_weight_descriptors == nullptr) return -1;
+  // explicit, never silent: features outside the dense full-attention path are refused
+  bool supported = rq->experimental_rt_decode == 0 && rq->head_dim <= 512 &&
+                   static_cast<uint64_t>(rq->intermediate) * 2 <= 60 * 1024 &&
+                   static_cast<uint64_t>(rq->hidden) * 2 <= 60 * 1024 &&
+                   static_cast<uint64_t>(rq->heads) * rq->head_dim * 2 <= 60 * 1024;
+  if (!synthetic && rq->layers != nullptr)
+    for (uint32_t l = 0; l < rq->layer_count && supported; ++l) supported = layer_supported(rq->layers[l]);
+  if (!supported) {
+    out->hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED;
+    return -1;
+  }
+  if (!device_ready(&out->hip_error)) return -1;
+  out->device_count = 1;
+  out->dtype = rq->dtype;
+  out->hidden = rq->hidden;
+  out->heads = rq->heads;
+  out->kv_heads = rq->kv_heads;
+  out->head_dim = rq->head_dim;
+  out->intermediate = rq->intermediate;
+  out->vocab_size = rq->vocab_size;
+  out->layer_count = rq->layer_count;
+  out->max_context_tokens = rq->max_context_tokens;
+  out->prefill_chunk_tokens = 1;
+  out->head_threads = kBlock;
+  out->experimental_rt_decode_requested = rq->experimental_rt_decode;
+
+  const uint64_t allocs_before = allocation_count();
+  const uint64_t H = rq->hidden, A = static_cast<uint64_t>(rq->heads) * rq->head_dim,
+                 KV = static_cast<uint64_t>(rq->kv_heads) * rq->head_dim, I = rq->intermediate,
+                 V = rq->vocab_size, L = rq->layer_count, HD = rq->head_dim;
+  const uint32_t block_count = (rq->max_context_tokens + kKvBlockTokens - 1) / kKvBlockTokens;
+
+  Session *s = new (std::nothrow) Session();
+  if (s == nullptr) return -1;
+  s->dtype = rq->dtype;
+  s->hidden = rq->hidden;
+  s->heads = rq->heads;
+  s->kv_heads = rq->kv_heads;
+  s->head_dim = rq->head_dim;
+  s->intermediate = rq->intermediate;
+  s->vocab = rq->vocab_size;
+  s->layers = rq->layer_count;
+  s->max_ctx = rq->max_context_tokens;
+  s->eps = rq->rms_eps;
+  s->theta = rq->rope_theta;
+  s->block_count = block_count;
+  s->planned_weight_blocks = rq->planned_weight_blocks;
+  s->planned_gpu_resident_blocks = rq->planned_gpu_resident_blocks;
+  s->planned_gpu_staged_blocks = rq->planned_gpu_staged_blocks;
+  s->planned_weight_bytes = rq->planned_weight_bytes;
+  s->planned_gpu_resident_weight_bytes = rq->planned_gpu_resident_weight_bytes;
+  s->planned_gpu_staged_weight_bytes = rq->planned_gpu_staged_weight_bytes;
+  s->planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
+  s->planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
+  // enough splits to put >= 2 workgroups on every CU, never more than KV blocks
+  {
+    uint32_t splits = (512 + rq->kv_heads - 1) / rq->kv_heads;
+    splits = std::min(splits, kAttnMaxSplits);
+    splits = std::min(splits, std::max(1u, block_count));
+    s->attn_splits = std::max(1u, splits);
+  }
+
+  // ---- arena layout ------------------------------------------------------
+  struct LayerOff {
+    uint64_t rms_attn, rms_mlp, wqkv, q_norm, k_norm, q_bias, k_bias, v_bias, wo, o_bias, wgu, wdown;
+  };
+  const uint64_t kNone = ~uint64_t{0};
+  Carver c;
+  uint64_t weight_elems = 0;
+  const uint64_t off_emb = c.take(V * H * 2);
+  weight_elems += V * H;
+  std::vector<LayerOff> lo(L);
+  for (uint32_t l = 0; l < L; ++l) {
+    const NervaHipHfDecodeChainLayer *src = synthetic ? nullptr : &rq->layers[l];
+    lo[l].rms_attn = c.take(H * 2);
+    lo[l].rms_mlp = c.take(H * 2);
+    lo[l].wqkv = c.take((A + 2 * KV) * H * 2);
+    const bool qn = synthetic ? with_qk_norm != 0 : src->q_norm_weight != nullptr;
+    const bool kn = synthetic ? with_qk_norm != 0 : src->k_norm_weight != nullptr;
+    lo[l].q_norm = qn ? c.take(HD * 2) : kNone;
+    lo[l].k_norm = kn ? c.take(HD * 2) : kNone;
+    lo[l].q_bias = (!synthetic && src->q_bias) ? c.take(A * 2) : kNone;
+    lo[l].k_bias = (!synthetic && src->k_bias) ? c.take(KV * 2) : kNone;
+    lo[l].v_bias = (!synthetic && src->v_bias) ? c.take(KV * 2) : kNone;
+    lo[l].wo = c.take(H * A * 2);
+    lo[l].o_bias = (!synthetic && src->o_bias) ? c.take(H * 2) : kNone;
+    lo[l].wgu = c.take(2 * I * H * 2);
+    lo[l].wdown = c.take(H * I * 2);
+    weight_elems += 2 * H + (A + 2 * KV) * H + H * A + 3 * I * H;
+    if (qn) weight_elems += HD;
+    if (kn) weight_elems += HD;
+    if (lo[l].q_bias != kNone) weight_elems += A;
+    if (lo[l].k_bias != kNone) weight_elems += KV;
+    if (lo[l].v_bias != kNone) weight_elems += KV;
+    if (lo[l].o_bias != kNone) weight_elems += H;
+  }
+  const uint64_t off_final = c.take(H * 2);
+  const uint64_t off_lm = c.take(V * H * 2);
+  weight_elems += H + V * H;
+  s->resident_weight_bytes = weight_elems * 2;
+  const uint64_t kv_half = L * block_count * KV * kKvBlockTokens * 2;
+  const uint64_t off_kc = c.take(kv_half);
+  const uint64_t off_vc = c.take(kv_half);
+  s->kv_bytes = 2 * kv_half;
+  const uint64_t off_table = c.take(static_cast<uint64_t>(block_count) * 4);
+  const uint64_t off_prompt = c.take(static_cast<uint64_t>(rq->max_context_tokens) * 4);
+  const uint64_t off_slots = c.take(static_cast<uint64_t>(rq->max_context_tokens) * sizeof(Slot));
+  const uint64_t off_state = c.take(64);
+  const uint64_t off_x = c.take(H * 4);
+  const uint64_t off_r = c.take(H * 4);
+  const uint64_t off_qkv = c.take((A + 2 * KV) * 4);
+  const uint64_t off_logits = c.take(V * 4);
+  const uint64_t off_attn16 = c.take(A * 2);
+  const uint64_t off_ff16 = c.take(I * 2);
+  const uint64_t off_rope = c.take(HD * 4);
+  const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
+  const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
+  s->arena_bytes = c.offset;
+
+  if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
+    // session_api_oneshot.inc.cu: a weight plan that disagrees with the arena is rejected
+    destroy_session(s);
+    return -1;
+  }
+
+  hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
+  out->failure_stage = 2;
+  if (err == hipSuccess) err = counted_malloc(reinterpret_cast<void **>(&s->arena), s->arena_bytes);
+  out->failure_stage = 3;
+  s->pinned_bytes = static_cast<uint64_t>(rq->max_context_tokens) * (sizeof(Slot) + 4) + 256;
+  if (err == hipSuccess) err = counted_host_malloc(reinterpret_cast<void **>(&s->pinned), s->pinned_bytes);
+  if (err == hipSuccess) err = hipEventCreate(&s->ev0);
+  if (err == hipSuccess) err = hipEventCreate(&s->ev1);
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    destroy_session(s);
+    return -1;
+  }
+  s->host_slots = reinterpret_cast<Slot *>(s->pinned);
+  s->host_prompt = reinterpret_cast<uint32_t *>(s->pinned + static_cast<uint64_t>(rq->max_context_tokens) * sizeof(Slot));
+  s->host_state = s->host_prompt + rq->max_context_tokens;
+
+  auto dev16 = [&](uint64_t off) { return off == kNone ? nullptr : reinterpret_cast<uint16_t *>(s->arena + off); };
+  s->emb = dev16(off_emb);
+  s->final_norm = dev16(off_final);
+  s->lm_head = dev16(off_lm);
+  s->kc = dev16(off_kc);
+  s->vc = dev16(off_vc);
+  s->table = reinterpret_cast<uint32_t *>(s->arena + off_table);
+  s->prompt = reinterpret_cast<uint32_t *>(s->arena + off_prompt);
+  s->slots = reinterpret_cast<Slot *>(s->arena + off_slots);
+  s->state = reinterpret_cast<uint32_t *>(s->arena + off_state);
+  s->x = reinterpret_cast<float *>(s->arena + off_x);
+  s->r = reinterpret_cast<float *>(s->arena + off_r);
+  s->qkv = reinterpret_cast<float *>(s->arena + off_qkv);
+  s->logits = reinterpret_cast<float *>(s->arena + off_logits);
+  s->attn16 = dev16(off_attn16);
+  s->ff16 = dev16(off_ff16);
+  s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
+  s->attn_ws = s->arena + off_attn_ws;
+  s->sample_ws = s->arena + off_sample_ws;
+  s->layer.resize(L);
+  for (uint32_t l = 0; l < L; ++l) {
+    s->layer[l] = LayerDev{dev16(lo[l].rms_attn), dev16(lo[l].rms_mlp), dev16(lo[l].wqkv),
+                           dev16(lo[l].q_norm),   dev16(lo[l].k_norm),  dev16(lo[l].q_bias),
+                           dev16(lo[l].k_bias),   dev16(lo[l].v_bias),  dev16(lo[l].wo),
+                           dev16(lo[l].o_bias),   dev16(lo[l].wgu),     dev16(lo[l].wdown)};
+  }
+
+  // ---- weights -------------------------------------------------------------
+  out->failure_stage = 4;
+  uint64_t h2d = 0;
+  auto upload = [&](uint64_t off, const uint16_t *src, uint64_t elems) {
+    if (err != hipSuccess || off == kNone) return;
+    err = hipMemcpy(s->arena + off, src, elems * 2, hipMemcpyHostToDevice);
+    h2d += elems * 2;
+  };
+  auto fill = [&](uint64_t off, uint64_t tensor_id, uint64_t elems, float mean) {
+    if (err != hipSuccess || off == kNone) return;
+    err = launch_synth_16(s->arena + off, s->dtype, seed, tensor_id, elems, mean, weight_std, s->stream);
+  };
+  if (synthetic) {
+    fill(off_emb, 1, V * H, 0.0f);
+    fill(off_final, 2, H, 1.0f);
+    fill(off_lm, 3, V * H, 0.0f);
+    for (uint32_t l = 0; l < L; ++l) {
+      const uint64_t base = 16ull * (l + 1);
+      fill(lo[l].rms_attn, base + 0, H, 1.0f);
+      fill(lo[l].rms_mlp, base + 1, H, 1.0f);
+      fill(lo[l].wqkv, base + 2, A * H, 0.0f);
+      fill(lo[l].wqkv + A * H * 2, base + 4, KV * H, 0.0f);
+      fill(lo[l].q_norm, base + 5, HD, 1.0f);
+      fill(lo[l].k_norm, base + 6, HD, 1.0f);
+      fill(lo[l].wqkv + (A + KV) * H * 2, base + 7, KV * H, 0.0f);
+      fill(lo[l].wo, base + 8, H * A, 0.0f);
+      fill(lo[l].wgu, base + 13, I * H, 0.0f);
+      fill(lo[l].wgu + I * H * 2, base + 14, I * H, 0.0f);
+      fill(lo[l].wdown, base + 15, H * I, 0.0f);
+    }
+  } else {
+    upload(off_emb, rq->embeddings, V * H);
+    upload(off_final, rq->final_norm_weight, H);
+    upload(off_lm, rq->lm_head, V * H);
+    for (uint32_t l = 0; l < L; ++l) {
+      const NervaHipHfDecodeChainLayer &src = rq->layers[l];
+      upload(lo[l].rms_attn, src.rms_attn_weight, H);
+      upload(lo[l].rms_mlp, src.rms_mlp_weight, H);
+      // [q; k; v] rows back to back = one (A + 2KV) x H matrix (kernels.cu:741-769)
+      upload(lo[l].wqkv, src.w_q, A * H);
+      upload(lo[l].wqkv + A * H * 2, src.w_k, KV * H);
+      upload(lo[l].wqkv + (A + KV) * H * 2, src.w_v, KV * H);
+      upload(lo[l].q_norm, src.q_norm_weight, HD);
+      upload(lo[l].k_norm, src.k_norm_weight, HD);
+      upload(lo[l].q_bias, src.q_bias, A);
+      upload(lo[l].k_bias, src.k_bias, KV);
+      upload(lo[l].v_bias, src.v_bias, KV);
+      upload(lo[l].wo, src.w_o, H * A);
+      upload(lo[l].o_bias, src.o_bias, H);
+      // [gate; up] rows back to back (kernels.cu:771-802)
+      upload(lo[l].wgu, src.w_gate, I * H);
+      upload(lo[l].wgu + I * H * 2, src.w_up, I * H);
+      upload(lo[l].wdown, src.w_down, H * I);
+    }
+  }
+  // ---- state ---------------------------------------------------------------
+  out->failure_stage = 5;
+  if (err == hipSuccess) {
+    std::vector<uint32_t> table(block_count);
+    for (uint32_t i = 0; i < block_count; ++i) table[i] = i;  // identity (kernels.cu:733-739)
+    err = hipMemcpy(s->table, table.data(), table.size() * 4, hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess && s->theta > 0.0f) {
+    // powf(theta, 2i/d) evaluated once on the host in f32 (common/rope.rs:69-70); the
+    // kernels divide the f32 position by it.
+    std::vector<float> freq(HD / 2);
+    for (uint32_t i = 0; i < HD / 2; ++i)
+      freq[i] = powf(s->theta, static_cast<float>(2 * i) / static_cast<float>(HD));
+    err = hipMemcpy(s->rope_freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_workspace_bytes(rq->heads, rq->head_dim), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    destroy_session(s);
+    return -1;
+  }
+  out->failure_stage = 0;
+  out->resident_weight_bytes = s->resident_weight_bytes;
+  out->planned_weight_blocks = s->planned_weight_blocks;
+  out->planned_gpu_resident_blocks = s->planned_gpu_resident_blocks;
+  out->planned_gpu_staged_blocks = s->planned_gpu_staged_blocks;
+  out->planned_weight_bytes = s->planned_weight_bytes;
+  out->planned_gpu_resident_weight_bytes = s->planned_gpu_resident_weight_bytes;
+  out->planned_gpu_staged_weight_bytes = s->planned_gpu_staged_weight_bytes;
+  out->descriptor_gpu_resident_h2d_bytes = s->planned_gpu_resident_weight_bytes;
+  out->descriptor_gpu_staged_h2d_bytes = s->planned_gpu_staged_weight_bytes;
+  out->planned_weight_descriptor_count = s->planned_weight_descriptor_count;
+  out->planned_weight_descriptor_hash = s->planned_weight_descriptor_hash;
+  out->resident_kv_bytes = s->kv_bytes;
+  out->device_arena_bytes = s->arena_bytes;
+  out->pinned_host_bytes = s->pinned_bytes;
+  out->h2d_bytes = h2d;
+  out->sync_calls = 1;
+  out->hot_path_allocations = 0;
+  (void)allocs_before;
+  {
+    // device-reported memory clock x bus width, like session_api_lifecycle.inc.cu:84-106
+    int clock_khz = 0, bus_bits = 0;
+    if (hipDeviceGetAttribute(&clock_khz, hipDeviceAttributeMemoryClockRate, 0) == hipSuccess &&
+        hipDeviceGetAttribute(&bus_bits, hipDeviceAttributeMemoryBusWidth, 0) == hipSuccess)
+      out->device_memory_bandwidth_bps = static_cast<uint64_t>(clock_khz) * 1000ull * 2ull * (static_cast<uint64_t>(bus_bits) / 8ull);
+  }
+  out->status = 0;
+  *session_out = s;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nerva_hip_hf_decode_sequence_session_create(const NervaHipHfDecodeSequenceSessionCreateRequest *request,
+                                                NervaHipHfDecodeSequenceSessionCreateResult *out,
+                                                NervaHipHfDecodeSequenceSession **session) {
+  return create_impl(request, false, 0, 0.0f, 0, out, session);
+}
+
+int nerva_hip_bench_session_create_synthetic(const NervaHipHfDecodeSequenceSessionCreateRequest *request,
+                                             uint64_t seed, float weight_std, uint32_t with_qk_norm,
+                                             NervaHipHfDecodeSequenceSessionCreateResult *out,
+                                             NervaHipHfDecodeSequenceSession **session) {
+  return create_impl(request, true, seed, weight_std, with_qk_norm, out, session);
+}
+
+int nerva_hip_hf_decode_sequence_session_destroy(NervaHipHfDecodeSequenceSession *session,
+                                                 NervaHipHfDecodeSequenceSessionCreateResult *out) {
+  if (out != nullptr) {
+    memset(out, 0, sizeof(*out));
+    out->status = -1;
+  }
+  if (session == nullptr) return -1;
+  if (out != nullptr) {
+    out->device_count = 1;
+    out->dtype = session->dtype;
+    out->hidden = session->hidden;
+    out->heads = session->heads;
+    out->kv_heads = session->kv_heads;
+    out->head_dim = session->head_dim;
+    out->intermediate = session->intermediate;
+    out->vocab_size = session->vocab;
+    out->layer_count = session->layers;
+    out->max_context_tokens = session->max_ctx;
+    out->resident_weight_bytes = session->resident_weight_bytes;
+    out->resident_kv_bytes = session->kv_bytes;
+    out->device_arena_bytes = session->arena_bytes;
+    out->pinned_host_bytes = session->pinned_bytes;
+    out->sync_calls = 1;
+    out->status = 0;
+  }
+  destroy_session(session);
+  return 0;
+}
+
+int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSessionStartRequest *request,
+                                               NervaHipHfDecodeSequenceResult *out) {
+  if (!begin_result(out)) return -1;
+  if (request == nullptr || request->session == nullptr || request->prompt_tokens == nullptr ||
+      request->prompt_token_count == 0 || !sampler_valid(request->sampler))
+    return -1;
+  Session *s = request->session;
+  if (request->prompt_token_count > s->max_ctx) return -1;
+  for (uint32_t i = 0; i < request->prompt_token_count; ++i)
+    if (request->prompt_tokens[i] >= s->vocab) return -1;
+  if (!sampler_greedy(request->sampler)) {
+    out->device_count = 1;
+    out->hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED;
+    return -1;
+  }
+  const uint32_t P = request->prompt_token_count;
+  fill_header(s, out, 0, request->prompt_tokens[P - 1]);
+  s->started = false;
+  hipError_t err = reset_sequence(s, request->prompt_tokens, P, out);
+  // prefill: P-1 prompt steps (graph replay) + one prompt step with the LM head and sampler
+  if (err == hipSuccess && P > 1) err = ensure_graph(s, 1, out);
+  if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
+  for (uint32_t i = 0; err == hipSuccess && i + 1 < P; ++i) {
+    err = hipGraphLaunch(s->exec[1], s->stream);
+    if (err == hipSuccess) {
+      out->graph_replays += 1;
+      out->graph_launches += 1;
+      out->kernel_launches += s->graph_nodes[1];
+    }
+  }
+  if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
+  if (err == hipSuccess) out->kernel_launches += 2 + 5ull * s->layers;
+  if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  s->prompt_count = P;
+  s->has_eos = request->has_eos_token;
+  s->eos = request->eos_token;
+  s->seed_token = request->prompt_tokens[P - 1];
+  s->observed = 0;
+  s->cursor = P;
+  s->started = true;
+  s->finished = false;
+  out->resident_kv_bytes = s->kv_bytes;
+  out->kv_tokens = P;
+  out->device_arena_bytes = s->arena_bytes;
+  out->pinned_host_bytes = static_cast<uint64_t>(s->max_ctx) * sizeof(Slot);
+  out->status = 0;
+  return 0;
+}
+
+int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceSessionAdvanceRequest *request,
+                                                 NervaHipHfDecodeSequenceResult *out) {
+  if (!begin_result(out)) return -1;
+  if (request == nullptr || request->session == nullptr || request->output_tokens == nullptr ||
+      request->steps == 0 || request->output_token_capacity < request->steps)
+    return -1;
+  Session *s = request->session;
+  if (!s->started || s->finished || s->prompt_count == 0) return -1;
+  const uint32_t P = s->prompt_count;
+  const uint32_t slot_start = P - 1u + s->observed;
+  const uint64_t target64 = static_cast<uint64_t>(P) + s->observed + request->steps - 1u;
+  if (target64 > s->max_ctx || target64 < s->cursor) return -1;
+  const uint32_t target = static_cast<uint32_t>(target64);
+  const uint32_t run_count = target - s->cursor;
+  const uint32_t seed = s->observed == 0 ? s->seed_token : s->host_slots[slot_start - 1u].token;
+  fill_header(s, out, request->steps, seed);
+
+  hipError_t err = hipSuccess;
+  if (run_count != 0) err = ensure_graph(s, 0, out);
+  const uint64_t allocs_before = allocation_count();
+  if (err == hipSuccess && run_count != 0) err = hipEventRecord(s->ev0, s->stream);
+  for (uint32_t step = 0; err == hipSuccess && step < run_count; ++step) {
+    err = hipGraphLaunch(s->exec[0], s->stream);
+    if (err == hipSuccess) {
+      out->graph_replays += 1;
+      out->graph_launches += 1;
+      out->kernel_launches += s->graph_nodes[0];
+    }
+    // With a stop token the host looks at each token so that it can stop launching
+    // (session_api_lifecycle.inc.cu:1206-1234); without one the loop never syncs.
+    if (err == hipSuccess && s->has_eos != 0) {
+      const uint32_t pos = s->cursor + step;
+      err = hipMemcpyAsync(&s->host_slots[pos], &s->slots[pos], sizeof(Slot), hipMemcpyDeviceToHost, s->stream);
+      if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+      out->sync_calls += 1;
+      out->d2h_bytes += sizeof(Slot);
+      if (err == hipSuccess && s->host_slots[pos].completion == NERVA_HIP_SLOT_DEVICE_COMPLETE &&
+          s->host_slots[pos].token == s->eos)
+        break;
+    }
+  }
+  if (err == hipSuccess && run_count != 0) err = hipEventRecord(s->ev1, s->stream);
+  const uint64_t slots_bytes = static_cast<uint64_t>(request->steps) * sizeof(Slot);
+  if (err == hipSuccess) {
+    err = hipMemcpyAsync(s->host_slots + slot_start, s->slots + slot_start, slots_bytes,
+                         hipMemcpyDeviceToHost, s->stream);
+    out->d2h_bytes = slots_bytes;
+  }
+  if (err == hipSuccess) {
+    err = hipStreamSynchronize(s->stream);
+    out->sync_calls += 1;
+  }
+  out->hot_path_allocations = allocation_count() - allocs_before;
+  if (err == hipSuccess && run_count != 0) {
+    float ms = 0.0f;
+    err = hipEventElapsedTime(&ms, s->ev0, s->ev1);
+    if (err == hipSuccess && ms > 0.0f) {
+      out->device_elapsed_ns = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+      if (out->device_elapsed_ns == 0) out->device_elapsed_ns = 1;
+    }
+  }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  const Slot *observed = s->host_slots + slot_start;
+  out->observed_tokens = observed_count(request->steps, s->has_eos, s->eos, observed);
+  for (uint32_t i = 0; i < out->observed_tokens; ++i) request->output_tokens[i] = observed[i].token;
+  out->last_token = out->observed_tokens == 0 ? 0 : request->output_tokens[out->observed_tokens - 1];
+  out->observed_token_hash = fnv1a_bytes(request->output_tokens, static_cast<size_t>(out->observed_tokens) * 4);
+  out->resident_kv_bytes = s->kv_bytes;
+  out->kv_tokens = slot_start + out->observed_tokens;
+  out->device_arena_bytes = s->arena_bytes;
+  out->pinned_host_bytes = static_cast<uint64_t>(s->max_ctx) * sizeof(Slot);
+  out->host_causality_edges = 0;
+  out->status = out->observed_tokens > 0 && slots_consistent(observed, out->observed_tokens, slot_start) ? 0 : -1;
+  if (out->status == 0) {
+    s->observed += out->observed_tokens;
+    s->cursor = out->observed_tokens < request->steps ? s->max_ctx : target;
+    s->finished = out->observed_tokens < request->steps || out->kv_tokens >= s->max_ctx;
+  }
+  return out->status == 0 ? 0 : -1;
+}
+
+int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessionRunRequest *request,
+                                             NervaHipHfDecodeSequenceResult *out) {
+  if (!begin_result(out)) return -1;
+  if (request == nullptr || request->session == nullptr || request->prompt_tokens == nullptr ||
+      request->output_tokens == nullptr || request->steps == 0 || request->prompt_token_count == 0 ||
+      request->output_token_capacity < request->steps ||
+      request->prompt_tokens[request->prompt_token_count - 1u] != request->seed_token ||
+      !sampler_valid(request->sampler) ||
+      request->prompt_token_count > UINT32_MAX - request->steps + 1u)
+    return -1;
+  Session *s = request->session;
+  const uint32_t P = request->prompt_token_count;
+  const uint32_t context_steps = P + request->steps - 1u;
+  if (context_steps > s->max_ctx) return -1;
+  for (uint32_t i = 0; i < P; ++i)
+    if (request->prompt_tokens[i] >= s->vocab) return -1;
+  if (!sampler_greedy(request->sampler)) {
+    out->device_count = 1;
+    out->hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED;
+    return -1;
+  }
+  fill_header(s, out, request->steps, request->seed_token);
+  s->started = false;
+  hipError_t err = reset_sequence(s, request->prompt_tokens, P, out);
+  // the decode-step graph walks every position, prompt included (session_api_lifecycle.inc.cu:748-990)
+  if (err == hipSuccess) err = ensure_graph(s, 0, out);
+  const uint64_t allocs_before = allocation_count();
+  if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
+  for (uint32_t step = 0; err == hipSuccess && step < context_steps; ++step) {
+    err = hipGraphLaunch(s->exec[0], s->stream);
+    if (err == hipSuccess) {
+      out->graph_replays += 1;
+      out->graph_launches += 1;
+      out->kernel_launches += s->graph_nodes[0];
+    }
+  }
+  if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
+  const uint64_t slots_bytes = static_cast<uint64_t>(context_steps) * sizeof(Slot);
+  if (err == hipSuccess) {
+    err = hipMemcpyAsync(s->host_slots, s->slots, slots_bytes, hipMemcpyDeviceToHost, s->stream);
+    out->d2h_bytes = slots_bytes;
+  }
+  if (err == hipSuccess) {
+    err = hipStreamSynchronize(s->stream);
+    out->sync_calls += 1;
+  }
+  out->hot_path_allocations = allocation_count() - allocs_before;
+  if (err == hipSuccess) {
+    float ms = 0.0f;
+    err = hipEventElapsedTime(&ms, s->ev0, s->ev1);
+    if (err == hipSuccess && ms > 0.0f) out->device_elapsed_ns = std::max<uint64_t>(1, static_cast<uint64_t>(static_cast<double>(ms) * 1e6));
+  }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  const uint32_t output_start = P - 1u;
+  const Slot *observed = s->host_slots + output_start;
+  out->observed_tokens = observed_count(request->steps, request->has_eos_token, request->eos_token, observed);
+  for (uint32_t i = 0; i < out->observed_tokens; ++i) request->output_tokens[i] = observed[i].token;
+  out->last_token = out->observed_tokens == 0 ? 0 : request->output_tokens[out->observed_tokens - 1];
+  out->observed_token_hash = fnv1a_bytes(request->output_tokens, static_cast<size_t>(out->observed_tokens) * 4);
+  out->resident_kv_bytes = s->kv_bytes;
+  out->kv_tokens = output_start + out->observed_tokens;
+  out->device_arena_bytes = s->arena_bytes;
+  out->pinned_host_bytes = static_cast<uint64_t>(s->max_ctx) * sizeof(Slot);
+  out->host_causality_edges = 0;
+  out->status = out->observed_tokens > 0 && slots_consistent(observed, out->observed_tokens, output_start) ? 0 : -1;
+  return out->status == 0 ? 0 : -1;
+}
+
+int nerva_hip_hf_decode_sequence_u16(const NervaHipHfDecodeSequenceRequest *rq, NervaHipHfDecodeSequenceResult *out) {
+  if (!begin_result(out)) return -1;
+  if (rq == nullptr || rq->prompt_tokens == nullptr || rq->prompt_token_count == 0 || rq->steps == 0 ||
+      rq->output_tokens == nullptr || rq->output_token_capacity < rq->steps ||
+      rq->prompt_token_count > UINT32_MAX - rq->steps + 1u)
+    return -1;
+  NervaHipHfDecodeSequenceSessionCreateRequest cr{};
+  cr.dtype = rq->dtype;
+  cr.hidden = rq->hidden;
+  cr.heads = rq->heads;
+  cr.kv_heads = rq->kv_heads;
+  cr.head_dim = rq->head_dim;
+  cr.intermediate = rq->intermediate;
+  cr.vocab_size = rq->vocab_size;
+  cr.layer_count = rq->layer_count;
+  cr.max_context_tokens = rq->prompt_token_count + rq->steps - 1u;
+  cr.rms_eps = rq->rms_eps;
+  cr.rope_theta = rq->rope_theta;
+  cr.embeddings = rq->embeddings;
+  cr.layers = rq->layers;
+  cr.final_norm_weight = rq->final_norm_weight;
+  cr.lm_head = rq->lm_head;
+  cr.planned_weight_blocks = rq->planned_weight_blocks;
+  cr.planned_gpu_resident_blocks = rq->planned_gpu_resident_blocks;
+  cr.planned_gpu_staged_blocks = rq->planned_gpu_staged_blocks;
+  cr.planned_weight_bytes = rq->planned_weight_bytes;
+  cr.planned_gpu_resident_weight_bytes = rq->planned_gpu_resident_weight_bytes;
+  cr.planned_gpu_staged_weight_bytes = rq->planned_gpu_staged_weight_bytes;
+  cr.planned_weight_descriptors = rq->planned_weight_descriptors;
+  cr.planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
+  cr.planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
+  NervaHipHfDecodeSequenceSessionCreateResult cres;
+  Session *s = nullptr;
+  if (create_impl(&cr, false, 0, 0.0f, 0, &cres, &s) != 0) {
+    out->hip_error = cres.hip_error;
+    out->device_count = cres.device_count;
+    return -1;
+  }
+  NervaHipHfDecodeSequenceSessionRunRequest run{};
+  run.session = s;
+  run.steps = rq->steps;
+  run.seed_token = rq->seed_token;
+  run.prompt_tokens = rq->prompt_tokens;
+  run.prompt_token_count = rq->prompt_token_count;
+  run.has_eos_token = rq->has_eos_token;
+  run.eos_token = rq->eos_token;
+  run.output_tokens = rq->output_tokens;
+  run.output_token_capacity = rq->output_token_capacity;
+  run.sampler = rq->sampler;
+  const int rc = nerva_hip_hf_decode_sequence_session_run(&run, out);
+  if (rc == 0) out->h2d_bytes += cres.h2d_bytes;
+  destroy_session(s);
+  return rc;
+}
+
+int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t repeats, NervaHipStepProfile *out) {
+  if (!begin_result(out)) return -1;
+  if (s == nullptr || repeats == 0 || !s->started) return -1;
+  hipError_t err = hipStreamSynchronize(s->stream);
+  uint32_t pos = 0;
+  if (err == hipSuccess) err = hipMemcpy(&pos, s->state, 4, hipMemcpyDeviceToHost);
+  if (err == hipSuccess && pos >= s->max_ctx) err = hipErrorInvalidValue;
+  Slot saved;
+  if (err == hipSuccess) err = hipMemcpy(&saved, s->slots + pos, sizeof(Slot), hipMemcpyDeviceToHost);
+  StepProfiler prof;
+  prof.stream = s->stream;
+  uint64_t sums[kLKinds] = {0};
+  uint64_t counts[kLKinds] = {0};
+  uint64_t total = 0;
+  for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {  // first pass is a warm-up
+    prof.used = 0;
+    prof.kinds.clear();
+    err = enqueue_step(s, kDecodeStep, &prof);
+    if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+    // undo the step: cursor and the published slot
+    if (err == hipSuccess) err = hipMemcpy(s->state, &pos, 4, hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(s->slots + pos, &saved, sizeof(Slot), hipMemcpyHostToDevice);
+    if (err != hipSuccess || rep == 0) continue;
+    for (size_t i = 0; i < prof.kinds.size(); ++i) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, prof.events[2 * i], prof.events[2 * i + 1]) == hipSuccess) {
+        sums[prof.kinds[i]] += static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+        counts[prof.kinds[i]] += 1;
+      }
+    }
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, prof.events[0], prof.events[prof.used - 1]) == hipSuccess)
+      total += static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+    out->launches = static_cast<uint32_t>(prof.kinds.size());
+  }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
+  out->position = pos;
+  out->embed_ns = avg(kLEmbed);
+  out->qkv_ns = avg(kLQkv);
+  out->attention_ns = avg(kLAttn);
+  out->o_ns = avg(kLO);
+  out->gate_up_ns = avg(kLGateUp);
+  out->down_ns = avg(kLDown);
+  out->lm_head_ns = avg(kLHead);
+  out->total_ns = total / repeats;
+  const uint64_t H = s->hidden, A = static_cast<uint64_t>(s->heads) * s->head_dim,
+                 KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim, I = s->intermediate, V = s->vocab;
+  // algorithmic bytes per launch: weights + input vector + output vector (+ norm weights / residual)
+  out->qkv_bytes = (A + 2 * KV) * H * 2 + H * 4 + H * 2 + (A + 2 * KV) * 4;
+  out->attention_bytes = 2 * (static_cast<uint64_t>(pos) + 1) * KV * 2 + (A + 2 * KV) * 4 + 2 * KV * 2 + A * 2;
+  out->o_bytes = H * A * 2 + A * 2 + H * 4 + H * 4;
+  out->gate_up_bytes = 2 * I * H * 2 + H * 4 + H * 2 + I * 2;
+  out->down_bytes = H * I * 2 + I * 2 + H * 4 + H * 4;
+  out->lm_head_bytes = V * H * 2 + H * 4 + H * 2 + V * 4;
+  out->status = 0;
+  return 0;
+}
+
+int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *s, float *host_logits) {
+  if (s == nullptr || host_logits == nullptr) return -1;
+  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
+  return hipMemcpy(host_logits, s->logits, static_cast<uint64_t>(s->vocab) * 4, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+
+int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t token,
+                              uint16_t *host_k, uint16_t *host_v) {
+  if (s == nullptr || host_k == nullptr || host_v == nullptr || layer >= s->layers || token >= s->max_ctx)
+    return -1;
+  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
+  const uint32_t block = token / kKvBlockTokens, row = token % kKvBlockTokens;  // identity table
+  for (uint32_t h = 0; h < s->kv_heads; ++h) {
+    const uint64_t off = kv_tile_offset(s->block_count, s->kv_heads, s->head_dim, layer, block, h) +
+                         static_cast<uint64_t>(row) * s->head_dim;
+    if (hipMemcpy(host_k + h * s->head_dim, s->kc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    if (hipMemcpy(host_v + h * s->head_dim, s->vc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,359 @@
+// FP8-e4m3fn weight-streaming GEMV with f32 block scales, and the MoE expert
+// kernels built on it. Weights are dequantised in f32 registers
+// (value = e4m3(W[r,c]) * S[r/br][c/bc], no 16-bit rounding in between), which
+// is the contract of the reference's own check
+// (crates/nerva-cuda/src/tests/deepseek_quant.rs:689-713); the reference CUDA
+// kernel's extra bf16 rounding (deepseek/projection.inc.cu:19-23) is not reproduced.
+//
+// Mapping: one wave owns NR rows; a load instruction covers 64 lanes x 16 B =
+// 1024 columns; a lane's 16 weights share one block scale when block_cols is a
+// multiple of 16, so the scale multiplies a 16-term partial sum once.
+// x is kept in LDS as f32 (bf16/f16 inputs widen exactly).
+#include "fp8_gemv.cuh"
+
+#include <algorithm>
+
+#include "fp8_codec.cuh"
+
+namespace nv {
+
+namespace {
+
+__device__ __forceinline__ float dot16_fp8(const uint4 &w, const float *x) {
+  float f[4];
+  float acc = 0.0f;
+  const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    fp8x4_to_f32(words[i], f);
+    const float4 xv = *reinterpret_cast<const float4 *>(x + 4 * i);
+    acc = fmaf(f[0], xv.x, acc);
+    acc = fmaf(f[1], xv.y, acc);
+    acc = fmaf(f[2], xv.z, acc);
+    acc = fmaf(f[3], xv.w, acc);
+  }
+  return acc;
+}
+
+// Stage x (16-bit or f32) into LDS as f32.
+template <uint32_t DT>
+__device__ __forceinline__ void stage_x(float *xs, const uint16_t *x16, const float *xf, uint32_t cols) {
+  if (x16 != nullptr) {
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) xs[c] = dec16<DT>(x16[c]);
+  } else {
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) xs[c] = xf[c];
+  }
+}
+
+// UU consecutive 1024-column chunks of NR rows, all loads issued before the first use.
+template <int NR, int UU>
+__device__ __forceinline__ void fp8_chunks(const uint8_t *const (&wrow)[NR], const float *const (&srow)[NR],
+                                           const float *xs, uint32_t chunk, uint32_t block_cols,
+                                           int lane, float (&acc)[NR]) {
+  uint4 wv[NR][UU];
+  const uint32_t c0 = chunk * 1024u + lane * 16;
+#pragma unroll
+  for (int u = 0; u < UU; ++u)
+#pragma unroll
+    for (int k = 0; k < NR; ++k) wv[k][u] = load_stream(wrow[k] + c0 + u * 1024u);
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+    const uint32_t c = c0 + u * 1024u;
+    const uint32_t sidx = c / block_cols;
+#pragma unroll
+    for (int k = 0; k < NR; ++k) acc[k] = fmaf(srow[k][sidx], dot16_fp8(wv[k][u], xs + c), acc[k]);
+  }
+}
+
+// NR rows x all columns for one wave; FAST: cols % 1024 == 0, block_cols % 16 == 0,
+// 16-byte aligned rows.
+template <int NR, bool FAST>
+__device__ __forceinline__ void fp8_rows(const uint8_t *const (&wrow)[NR], const float *const (&srow)[NR],
+                                         const float *xs, uint32_t cols, uint32_t block_cols, int lane,
+                                         float (&acc)[NR]) {
+  if constexpr (FAST) {
+    const uint32_t nchunks = cols / 1024u;
+    uint32_t chunk = 0;
+    for (; chunk + 4 <= nchunks; chunk += 4) fp8_chunks<NR, 4>(wrow, srow, xs, chunk, block_cols, lane, acc);
+    if (chunk + 2 <= nchunks) {
+      fp8_chunks<NR, 2>(wrow, srow, xs, chunk, block_cols, lane, acc);
+      chunk += 2;
+    }
+    if (chunk < nchunks) fp8_chunks<NR, 1>(wrow, srow, xs, chunk, block_cols, lane, acc);
+  } else {
+    for (uint32_t c = lane; c < cols; c += kWave) {
+#pragma unroll
+      for (int k = 0; k < NR; ++k) {
+        const float w = fp8_e4m3fn_to_f32_sw(wrow[k][c]) * srow[k][c / block_cols];
+        acc[k] = fmaf(w, xs[c], acc[k]);
+      }
+    }
+  }
+}
+
+template <uint32_t DT, int NR, bool FAST>
+__global__ __launch_bounds__(kBlock) void fp8_gemv_kernel(Fp8GemvParams p) {
+  extern __shared__ __align__(16) float xsf[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  for (uint32_t token = 0; token < p.tokens; ++token) {
+    if (token != 0) __syncthreads();
+    stage_x<DT>(xsf, p.x16 ? p.x16 + static_cast<uint64_t>(token) * p.cols : nullptr,
+                p.xf ? p.xf + static_cast<uint64_t>(token) * p.cols : nullptr, p.cols);
+    __syncthreads();
+    const uint32_t scale_cols = (p.cols + p.block_cols - 1) / p.block_cols;
+    const uint32_t units = (p.rows + NR - 1) / NR;
+    for (uint32_t unit = blockIdx.x * kWavesPerBlock + wave; unit < units;
+         unit += gridDim.x * kWavesPerBlock) {
+      const uint8_t *wrow[NR];
+      const float *srow[NR];
+      float acc[NR];
+#pragma unroll
+      for (int k = 0; k < NR; ++k) {
+        const uint32_t r = min(unit * NR + k, p.rows - 1);
+        wrow[k] = p.w + static_cast<uint64_t>(r) * p.cols;
+        srow[k] = p.scales + static_cast<uint64_t>(r / p.block_rows) * scale_cols;
+        acc[k] = 0.0f;
+      }
+      fp8_rows<NR, FAST>(wrow, srow, xsf, p.cols, p.block_cols, lane, acc);
+#pragma unroll
+      for (int k = 0; k < NR; ++k) {
+        const float y = wave_sum(acc[k]);
+        const uint32_t r = unit * NR + k;
+        if (lane == 0 && r < p.rows) p.out[static_cast<uint64_t>(token) * p.rows + r] = y;
+      }
+    }
+  }
+}
+
+// MoE gate/up: unit = (slot k, row i); the wave computes gate.x and up.x of expert
+// e_k and stores act[k][i] = silu(g) * u as f32.
+template <uint32_t DT, bool FAST>
+__global__ __launch_bounds__(kBlock) void moe_gate_up_kernel(MoeFp8Params p) {
+  extern __shared__ __align__(16) float xsf[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  stage_x<DT>(xsf, p.x16, nullptr, p.hidden);
+  __syncthreads();
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const uint32_t units = slots * p.inter;
+  const uint32_t sc = (p.hidden + p.block - 1) / p.block;
+  const uint64_t scale_stride = static_cast<uint64_t>((p.inter + p.block - 1) / p.block) * sc;
+  const uint64_t w_stride = static_cast<uint64_t>(p.inter) * p.hidden;
+  for (uint32_t unit = blockIdx.x * kWavesPerBlock + wave; unit < units;
+       unit += gridDim.x * kWavesPerBlock) {
+    const uint32_t k = unit / p.inter, i = unit % p.inter;
+    uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);
+    if (e >= p.num_experts) e = 0;  // ids are validated on the host when they are host-visible
+    const uint8_t *wrow[2] = {p.w_gate + e * w_stride + static_cast<uint64_t>(i) * p.hidden,
+                              p.w_up + e * w_stride + static_cast<uint64_t>(i) * p.hidden};
+    const float *srow[2] = {p.s_gate + e * scale_stride + static_cast<uint64_t>(i / p.block) * sc,
+                            p.s_up + e * scale_stride + static_cast<uint64_t>(i / p.block) * sc};
+    float acc[2] = {0.0f, 0.0f};
+    fp8_rows<2, FAST>(wrow, srow, xsf, p.hidden, p.block, lane, acc);
+    const float g = wave_sum(acc[0]);
+    const float u = wave_sum(acc[1]);
+    if (lane == 0) p.act[static_cast<uint64_t>(k) * p.inter + i] = silu(g) * u;
+  }
+}
+
+// MoE down + combine: the wave owns NR output rows h and walks the selected
+// experts in slot order, so out[h] = sum_k w_k * (Wd_k[h,:] . act[k]) is summed in
+// a fixed order (no atomics). act[k] is staged through LDS one expert at a time.
+template <int NR, bool FAST>
+__global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
+  extern __shared__ __align__(16) float acts[];  // 2 x inter floats (double buffer)
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const uint32_t sc = (p.inter + p.block - 1) / p.block;
+  const uint64_t scale_stride = static_cast<uint64_t>((p.hidden + p.block - 1) / p.block) * sc;
+  const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * p.inter;
+  const uint32_t unit = blockIdx.x * kWavesPerBlock + wave;  // grid covers all rows exactly
+  float total[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) total[r] = 0.0f;
+  for (uint32_t k = 0; k < slots; ++k) {
+    float *buf = acts + (k & 1u) * p.inter;
+    for (uint32_t c = threadIdx.x; c < p.inter; c += kBlock)
+      buf[c] = p.act[static_cast<uint64_t>(k) * p.inter + c];
+    __syncthreads();  // double buffer: the previous expert's readers are at most one step behind
+    uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);
+    if (e >= p.num_experts) e = 0;
+    const float weight = k < p.top_k ? p.expert_weights[k] : 1.0f;
+    const uint8_t *wrow[NR];
+    const float *srow[NR];
+    float acc[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      const uint32_t h = min(unit * NR + r, p.hidden - 1);
+      wrow[r] = p.w_down + e * w_stride + static_cast<uint64_t>(h) * p.inter;
+      srow[r] = p.s_down + e * scale_stride + static_cast<uint64_t>(h / p.block) * sc;
+      acc[r] = 0.0f;
+    }
+    fp8_rows<NR, FAST>(wrow, srow, buf, p.inter, p.block, lane, acc);
+#pragma unroll
+    for (int r = 0; r < NR; ++r) total[r] = fmaf(weight, wave_sum(acc[r]), total[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const uint32_t h = unit * NR + r;
+    if (lane == 0 && h < p.hidden) p.out[h] = total[r];
+  }
+}
+
+// softmax over E logits, top-k by (probability desc, index asc), optional
+// renormalisation (precision/block/moe.rs:1107-1155,1254-1268,1303-1326).
+// One workgroup; E <= 1024. Selection is k rounds of a block-wide argmax.
+__global__ __launch_bounds__(kBlock) void moe_route_kernel(MoeRouteParams p) {
+  __shared__ float probs[1024];
+  __shared__ float red[kWavesPerBlock];
+  __shared__ uint32_t red_i[kWavesPerBlock];
+  __shared__ uint32_t red_h[kWavesPerBlock];
+  __shared__ float sel_w[64];
+  float m = -INFINITY;
+  for (uint32_t i = threadIdx.x; i < p.num_experts; i += kBlock) m = fmaxf(m, p.logits[i]);
+  m = wave_max(m);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < p.num_experts; i += kBlock) probs[i] = expf(p.logits[i] - m);
+  __syncthreads();
+  // The reference sums probabilities sequentially; do the same on one thread so
+  // that ties and ordering see identical values (E is tiny).
+  if (threadIdx.x == 0) {
+    float sum = 0.0f;
+    for (uint32_t i = 0; i < p.num_experts; ++i) sum += probs[i];
+    red[0] = sum;
+  }
+  __syncthreads();
+  const float sum = red[0];
+  __syncthreads();
+  if (sum > 0.0f && isfinite(sum))
+    for (uint32_t i = threadIdx.x; i < p.num_experts; i += kBlock) probs[i] = probs[i] / sum;
+  __syncthreads();
+  for (uint32_t k = 0; k < p.top_k; ++k) {
+    Best b{0.0f, 0u, 0u};
+    for (uint32_t i = threadIdx.x; i < p.num_experts; i += kBlock) {
+      Best c{probs[i], i, probs[i] >= 0.0f ? 1u : 0u};  // taken entries are marked -1
+      if (better(c, b)) b = c;
+    }
+    b = wave_best(b);
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      red[threadIdx.x / kWave] = b.value;
+      red_i[threadIdx.x / kWave] = b.index;
+      red_h[threadIdx.x / kWave] = b.has;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      Best t{red[0], red_i[0], red_h[0]};
+      for (int w = 1; w < kWavesPerBlock; ++w) {
+        Best o{red[w], red_i[w], red_h[w]};
+        if (better(o, t)) t = o;
+      }
+      p.expert_ids[k] = t.index;
+      sel_w[k] = t.value;
+      probs[t.index] = -1.0f;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    float selected = 0.0f;
+    for (uint32_t k = 0; k < p.top_k; ++k) selected += sel_w[k];
+    const bool norm = p.normalize && selected > 0.0f && isfinite(selected);
+    for (uint32_t k = 0; k < p.top_k; ++k) p.expert_weights[k] = norm ? sel_w[k] / selected : sel_w[k];
+  }
+}
+
+bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+}  // namespace
+
+hipError_t launch_fp8_gemv(const Fp8GemvParams &p, hipStream_t stream) {
+  if (p.w == nullptr || p.scales == nullptr || p.out == nullptr || (p.x16 == nullptr && p.xf == nullptr))
+    return hipErrorInvalidValue;
+  if (p.rows == 0 || p.cols == 0 || p.block_rows == 0 || p.block_cols == 0 || p.tokens == 0)
+    return hipErrorInvalidValue;
+  if (p.input_dtype > kBF16) return hipErrorInvalidValue;
+  const size_t lds = static_cast<size_t>(p.cols) * sizeof(float);
+  if (lds > 60 * 1024) return hipErrorInvalidValue;
+  const bool fast = p.cols % 1024u == 0 && p.block_cols % 16u == 0 && aligned16(p.w);
+  if (fast) {
+    // short rows: more rows per wave to keep the same number of bytes in flight
+    if (p.cols <= 2048u) {
+      const uint32_t units = (p.rows + 3) / 4;
+      const uint32_t blocks = std::min<uint32_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
+      if (p.input_dtype == kBF16)
+        hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 4, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+      else
+        hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 4, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    } else {
+      const uint32_t units = (p.rows + 1) / 2;
+      const uint32_t blocks = std::min<uint32_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
+      if (p.input_dtype == kBF16)
+        hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 2, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+      else
+        hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 2, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    }
+  } else {
+    const uint32_t blocks = std::min<uint32_t>((p.rows + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
+    if (p.input_dtype == kBF16)
+      hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 1, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    else
+      hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 1, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
+  if (p.x16 == nullptr || p.expert_ids == nullptr || p.expert_weights == nullptr ||
+      p.w_gate == nullptr || p.w_up == nullptr || p.w_down == nullptr || p.s_gate == nullptr ||
+      p.s_up == nullptr || p.s_down == nullptr || p.act == nullptr || p.out == nullptr)
+    return hipErrorInvalidValue;
+  if (p.hidden == 0 || p.inter == 0 || p.num_experts == 0 || p.top_k == 0 || p.block == 0 ||
+      p.top_k > p.num_experts || p.input_dtype > kBF16)
+    return hipErrorInvalidValue;
+  if (p.shared_index >= static_cast<int32_t>(p.num_experts)) return hipErrorInvalidValue;
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  if (static_cast<size_t>(p.hidden) * 4 > 60 * 1024 || static_cast<size_t>(p.inter) * 8 > 60 * 1024)
+    return hipErrorInvalidValue;
+  const bool fast_gu = p.hidden % 1024u == 0 && p.block % 16u == 0 && aligned16(p.w_gate) && aligned16(p.w_up);
+  const bool fast_dn = p.inter % 1024u == 0 && p.block % 16u == 0 && aligned16(p.w_down);
+  {
+    const uint64_t units = static_cast<uint64_t>(slots) * p.inter;
+    const uint32_t blocks =
+        static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 32u));
+    const size_t lds = static_cast<size_t>(p.hidden) * sizeof(float);
+    if (p.input_dtype == kBF16) {
+      if (fast_gu) hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+      else hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    } else {
+      if (fast_gu) hipLaunchKernelGGL((moe_gate_up_kernel<kF16, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+      else hipLaunchKernelGGL((moe_gate_up_kernel<kF16, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    }
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  {
+    constexpr int NR = 2;
+    const uint32_t units = (p.hidden + NR - 1) / NR;
+    const uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
+    const size_t lds = static_cast<size_t>(p.inter) * 2 * sizeof(float);
+    if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((moe_down_kernel<NR, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_route(const MoeRouteParams &p, hipStream_t stream) {
+  if (p.logits == nullptr || p.expert_ids == nullptr || p.expert_weights == nullptr)
+    return hipErrorInvalidValue;
+  if (p.num_experts == 0 || p.num_experts > 1024 || p.top_k == 0 || p.top_k > p.num_experts ||
+      p.top_k > 64)
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(kBlock), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace nv

@@ -1,0 +1,119 @@
+// Shared device helpers: 16-bit / fp8 codecs, wave64 reductions, error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nv {
+
+constexpr uint32_t kF16 = 0;
+constexpr uint32_t kBF16 = 1;
+constexpr int kWave = 64;          // CDNA wavefront
+constexpr int kBlock = 256;        // 4 waves per workgroup everywhere in this library
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+// ---- 16-bit codecs -------------------------------------------------------
+// bf16: widen = shift; narrow = round-to-nearest-even on the dropped 16 bits
+// (reference: precision/bits.rs:4-18, device_ops.cuh:9-31).
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+  return __uint_as_float(static_cast<uint32_t>(b) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float v) {
+  uint32_t bits = __float_as_uint(v);
+  if ((bits & 0x7f800000u) == 0x7f800000u && (bits & 0x007fffffu) != 0) {
+    return static_cast<uint16_t>((bits >> 16) | 1u);
+  }
+  return static_cast<uint16_t>((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float f16_to_f32(uint16_t b) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, b));
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float v) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));  // v_cvt_f16_f32: RNE
+}
+
+template <uint32_t DT>
+__device__ __forceinline__ float dec16(uint16_t b) {
+  if constexpr (DT == kBF16) return bf16_to_f32(b);
+  else return f16_to_f32(b);
+}
+template <uint32_t DT>
+__device__ __forceinline__ uint16_t enc16(float v) {
+  if constexpr (DT == kBF16) return f32_to_bf16(v);
+  else return f32_to_f16(v);
+}
+template <uint32_t DT>
+__device__ __forceinline__ float round16(float v) {
+  return dec16<DT>(enc16<DT>(v));
+}
+// One dword = two packed 16-bit values (little endian: low half first).
+template <uint32_t DT>
+__device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+  if constexpr (DT == kBF16) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  } else {
+    lo = f16_to_f32(static_cast<uint16_t>(w & 0xffffu));
+    hi = f16_to_f32(static_cast<uint16_t>(w >> 16));
+  }
+}
+
+// ---- wave64 / block reductions -------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+// Sum over a 256-thread block; every thread gets the result. `scratch` is
+// kWavesPerBlock floats of LDS. Fixed combination order -> deterministic.
+__device__ __forceinline__ float block_sum(float v, float *scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+
+// (value desc, index asc) among finite candidates; `has` false = no candidate yet
+// (reference: sampler.cu:35-40).
+struct Best {
+  float value;
+  uint32_t index;
+  uint32_t has;
+};
+__device__ __forceinline__ bool better(const Best &a, const Best &b) {
+  if (!a.has) return false;
+  if (!b.has) return true;
+  return a.value > b.value || (a.value == b.value && a.index < b.index);
+}
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    Best other;
+    other.value = __shfl_xor(b.value, o, kWave);
+    other.index = __shfl_xor(b.index, o, kWave);
+    other.has = __shfl_xor(b.has, o, kWave);
+    if (better(other, b)) b = other;
+  }
+  return b;
+}
+
+// 16-byte streaming load that does not pollute the caches with single-use weights.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream(const void *p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+}  // namespace nv

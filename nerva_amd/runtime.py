@@ -1,0 +1,241 @@
+"""numpy <-> device plumbing over the C ABI (no torch: the library owns its HIP runtime)."""
+import ctypes as C
+
+import numpy as np
+
+from . import abi
+
+F16, BF16 = 0, 1
+
+
+def device_available():
+    """True when libnerva_hip.so loads and reports a usable GPU."""
+    lib = abi.load()
+    res = abi.NervaHipDeviceSmokeResult()
+    return lib.nerva_hip_device_smoke(C.byref(res)) == 0
+
+
+class Device:
+    @staticmethod
+    def smoke():
+        res = abi.NervaHipDeviceSmokeResult()
+        rc = abi.load().nerva_hip_device_smoke(C.byref(res))
+        return rc, res
+
+    @staticmethod
+    def synchronize():
+        if abi.load().nerva_hip_stream_synchronize(None) != 0:
+            raise RuntimeError("stream synchronize failed")
+
+    @staticmethod
+    def allocation_count():
+        return int(abi.load().nerva_hip_allocation_count())
+
+
+class DeviceBuffer:
+    """A device allocation made through nerva_hip_malloc."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        ptr = C.c_void_p()
+        if abi.load().nerva_hip_malloc(C.byref(ptr), self.nbytes) != 0 or not ptr.value:
+            raise MemoryError("nerva_hip_malloc(%d) failed" % self.nbytes)
+        self.ptr = ptr.value
+
+    @classmethod
+    def from_numpy(cls, array):
+        array = np.ascontiguousarray(array)
+        buf = cls(max(array.nbytes, 16))
+        buf.dtype, buf.shape = array.dtype, array.shape
+        if array.nbytes:
+            buf.upload(array)
+        return buf
+
+    @classmethod
+    def zeros(cls, nbytes):
+        buf = cls(nbytes)
+        if abi.load().nerva_hip_memset(buf.ptr, 0, buf.nbytes) != 0:
+            raise RuntimeError("memset failed")
+        return buf
+
+    def upload(self, array, offset=0):
+        array = np.ascontiguousarray(array)
+        assert offset + array.nbytes <= self.nbytes
+        if abi.load().nerva_hip_memcpy_h2d(self.ptr + offset, array.ctypes.data, array.nbytes) != 0:
+            raise RuntimeError("h2d copy failed")
+
+    def numpy(self, dtype, count=None, offset=0):
+        dtype = np.dtype(dtype)
+        count = (self.nbytes - offset) // dtype.itemsize if count is None else count
+        out = np.empty(count, dtype)
+        if abi.load().nerva_hip_memcpy_d2h(out.ctypes.data, self.ptr + offset, out.nbytes) != 0:
+            raise RuntimeError("d2h copy failed")
+        return out
+
+    def at(self, byte_offset):
+        return self.ptr + byte_offset
+
+    def free(self):
+        if getattr(self, "ptr", None):
+            abi.load().nerva_hip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _check(rc, err, what):
+    if rc != 0:
+        raise RuntimeError("%s failed (hip_error=%d)" % (what, err.value))
+
+
+def _ptr(buf):
+    if buf is None:
+        return None
+    return buf.ptr if isinstance(buf, DeviceBuffer) else int(buf)
+
+
+def gemv(dtype, weights, rows, cols, *, input16=None, input_f32=None, gamma=None, eps=0.0, bias=None,
+         residual=None, out_f32=None, out16=None, epilogue=0, round_output=False, sync=True):
+    """Launch nerva_hip_gemv on device buffers. prologue is implied by which input is given."""
+    req = abi.NervaHipGemvRequest()
+    req.dtype, req.rows, req.cols = dtype, rows, cols
+    req.prologue = 0 if input16 is not None else 1
+    req.epilogue = epilogue
+    req.round_output = int(round_output)
+    req.rms_eps = eps
+    req.weights, req.input16, req.input_f32 = _ptr(weights), _ptr(input16), _ptr(input_f32)
+    req.gamma, req.bias, req.residual = _ptr(gamma), _ptr(bias), _ptr(residual)
+    req.output_f32, req.output16 = _ptr(out_f32), _ptr(out16)
+    err = C.c_int32(0)
+    _check(abi.load().nerva_hip_gemv(C.byref(req), None, C.byref(err)), err, "nerva_hip_gemv")
+    if sync:
+        Device.synchronize()
+
+
+def fp8_gemv(weights, scales, rows, cols, block_rows, block_cols, out, *, input16=None, input_f32=None,
+             input_dtype=BF16, sync=True):
+    req = abi.NervaHipFp8GemvRequest()
+    req.rows, req.cols, req.block_rows, req.block_cols = rows, cols, block_rows, block_cols
+    req.input_dtype = input_dtype
+    req.weights, req.scales = _ptr(weights), _ptr(scales)
+    req.input16, req.input_f32, req.output = _ptr(input16), _ptr(input_f32), _ptr(out)
+    err = C.c_int32(0)
+    _check(abi.load().nerva_hip_fp8_gemv(C.byref(req), None, C.byref(err)), err, "nerva_hip_fp8_gemv")
+    if sync:
+        Device.synchronize()
+
+
+class PagedKvCache:
+    """K/V arrays in the library's layout [layer][block][kv_head][16][head_dim] + a block table."""
+
+    def __init__(self, layers, block_count, kv_heads, head_dim, table=None):
+        self.layers, self.block_count, self.kv_heads, self.head_dim = layers, block_count, kv_heads, head_dim
+        self.elems = layers * block_count * kv_heads * 16 * head_dim
+        self.k = DeviceBuffer.zeros(self.elems * 2)
+        self.v = DeviceBuffer.zeros(self.elems * 2)
+        table = np.arange(block_count, dtype=np.uint32) if table is None else np.asarray(table, np.uint32)
+        self.table_host = table
+        self.table = DeviceBuffer.from_numpy(table)
+
+    def offset(self, layer, token, kv_head):
+        lib = abi.load()
+        return int(lib.nerva_hip_kv_cache_offset(self.block_count, self.kv_heads, self.head_dim, layer,
+                                                 int(self.table_host[token // 16]), kv_head, token % 16))
+
+    def host_layout(self, layer, k_rows, v_rows):
+        """Scatter [tokens, kv_heads*head_dim] 16-bit rows into host images of the cache arrays."""
+        kimg = np.zeros(self.elems, np.uint16)
+        vimg = np.zeros(self.elems, np.uint16)
+        tokens = k_rows.shape[0]
+        hd = self.head_dim
+        for t in range(tokens):
+            for h in range(self.kv_heads):
+                o = self.offset(layer, t, h)
+                kimg[o:o + hd] = k_rows[t, h * hd:(h + 1) * hd]
+                vimg[o:o + hd] = v_rows[t, h * hd:(h + 1) * hd]
+        return kimg, vimg
+
+    def fill(self, layer, k_rows, v_rows):
+        kimg, vimg = self.host_layout(layer, k_rows, v_rows)
+        self.k.upload(kimg)
+        self.v.upload(vimg)
+
+    def read_row(self, layer, token):
+        hd = self.head_dim
+        k = np.empty(self.kv_heads * hd, np.uint16)
+        v = np.empty(self.kv_heads * hd, np.uint16)
+        for h in range(self.kv_heads):
+            o = self.offset(layer, token, h)
+            k[h * hd:(h + 1) * hd] = self.k.numpy(np.uint16, hd, o * 2)
+            v[h * hd:(h + 1) * hd] = self.v.numpy(np.uint16, hd, o * 2)
+        return k, v
+
+
+def paged_attention(dtype, heads, kv_heads, head_dim, cache, layer, position, qkv_f32, workspace, out16,
+                    *, out_f32=None, append=True, eps=1e-6, rope_theta=0.0, q_norm=None, k_norm=None,
+                    q_bias=None, k_bias=None, v_bias=None, sync=True):
+    req = abi.NervaHipPagedAttentionRequest()
+    req.dtype, req.heads, req.kv_heads, req.head_dim = dtype, heads, kv_heads, head_dim
+    req.layer, req.block_count, req.position, req.append = layer, cache.block_count, position, int(append)
+    req.rms_eps, req.rope_theta = eps, rope_theta
+    req.qkv_f32 = _ptr(qkv_f32)
+    req.q_norm, req.k_norm = _ptr(q_norm), _ptr(k_norm)
+    req.q_bias, req.k_bias, req.v_bias = _ptr(q_bias), _ptr(k_bias), _ptr(v_bias)
+    req.k_cache, req.v_cache, req.block_table = cache.k.ptr, cache.v.ptr, cache.table.ptr
+    req.workspace, req.output_f32, req.output16 = _ptr(workspace), _ptr(out_f32), _ptr(out16)
+    err = C.c_int32(0)
+    _check(abi.load().nerva_hip_paged_gqa_decode(C.byref(req), None, C.byref(err)), err,
+           "nerva_hip_paged_gqa_decode")
+    if sync:
+        Device.synchronize()
+
+
+def attention_workspace(heads, head_dim):
+    return DeviceBuffer.zeros(abi.load().nerva_hip_paged_attention_workspace_bytes(heads, head_dim))
+
+
+def argmax(logits_buf, count, workspace=None):
+    lib = abi.load()
+    ws = workspace or DeviceBuffer.zeros(lib.nerva_hip_argmax_workspace_bytes())
+    tok = DeviceBuffer.zeros(16)
+    req = abi.NervaHipArgmaxRequest()
+    req.count, req.logits, req.token, req.workspace = count, _ptr(logits_buf), tok.ptr, ws.ptr
+    err = C.c_int32(0)
+    _check(lib.nerva_hip_argmax(C.byref(req), None, C.byref(err)), err, "nerva_hip_argmax")
+    Device.synchronize()
+    return int(tok.numpy(np.uint32, 1)[0])
+
+
+def moe_route_softmax(logits, top_k, normalize=True):
+    logits = np.ascontiguousarray(logits, np.float32)
+    dl = DeviceBuffer.from_numpy(logits)
+    ids = DeviceBuffer.zeros(max(16, top_k * 4))
+    wts = DeviceBuffer.zeros(max(16, top_k * 4))
+    req = abi.NervaHipMoeRouteRequest()
+    req.num_experts, req.top_k, req.normalize = logits.size, top_k, int(normalize)
+    req.logits, req.expert_ids, req.expert_weights = dl.ptr, ids.ptr, wts.ptr
+    err = C.c_int32(0)
+    _check(abi.load().nerva_hip_moe_route_softmax(C.byref(req), None, C.byref(err)), err,
+           "nerva_hip_moe_route_softmax")
+    Device.synchronize()
+    return ids.numpy(np.uint32, top_k), wts.numpy(np.float32, top_k), ids, wts
+
+
+def moe_fp8_experts(hidden, inter, num_experts, top_k, block, x16, ids, weights, w_gate, s_gate, w_up,
+                    s_up, w_down, s_down, act, out, *, shared_index=-1, input_dtype=BF16, sync=True):
+    req = abi.NervaHipMoeFp8Request()
+    req.hidden, req.intermediate, req.num_experts, req.top_k = hidden, inter, num_experts, top_k
+    req.block, req.input_dtype, req.shared_index = block, input_dtype, shared_index
+    req.input16, req.expert_ids, req.expert_weights = _ptr(x16), _ptr(ids), _ptr(weights)
+    req.w_gate, req.w_up, req.w_down = _ptr(w_gate), _ptr(w_up), _ptr(w_down)
+    req.s_gate, req.s_up, req.s_down = _ptr(s_gate), _ptr(s_up), _ptr(s_down)
+    req.activation, req.output = _ptr(act), _ptr(out)
+    err = C.c_int32(0)
+    _check(abi.load().nerva_hip_moe_fp8_experts(C.byref(req), None, C.byref(err)), err,
+           "nerva_hip_moe_fp8_experts")
+    if sync:
+        Device.synchronize()

@@ -1,0 +1,183 @@
+"""Decode-session wrapper over the C ABI (create / start / advance / run / destroy).
+
+Mirrors the request/summary objects of the reference's host crate
+(crates/nerva-cuda/src/decode/hf_sequence/session/request.rs,
+crates/nerva-cuda/src/decode/hf_sequence/request.rs): the caller owns host
+weights, the library owns the opaque session.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import abi
+
+Qwen3_8B = dict(dtype=1, hidden=4096, heads=32, kv_heads=8, head_dim=128, intermediate=12288,
+                vocab=151936, layers=36, rms_eps=1e-6, rope_theta=1e6)
+
+_LAYER_FIELDS = {
+    "rms_attn": "rms_attn_weight", "rms_mlp": "rms_mlp_weight", "w_q": "w_q", "w_k": "w_k",
+    "w_v": "w_v", "w_o": "w_o", "q_norm": "q_norm_weight", "k_norm": "k_norm_weight",
+    "q_bias": "q_bias", "k_bias": "k_bias", "v_bias": "v_bias", "o_bias": "o_bias",
+    "w_gate": "w_gate", "w_up": "w_up", "w_down": "w_down",
+}
+
+
+def _u16(a):
+    return None if a is None else np.ascontiguousarray(a, np.uint16)
+
+
+class ModelWeights:
+    """Host weights (16-bit numpy arrays, row-major [out, in]) of a dense decoder."""
+
+    def __init__(self, dtype, hidden, heads, kv_heads, head_dim, intermediate, vocab, rms_eps,
+                 rope_theta, embeddings, layers, final_norm, lm_head):
+        self.dtype, self.hidden, self.heads, self.kv_heads = dtype, hidden, heads, kv_heads
+        self.head_dim, self.intermediate, self.vocab = head_dim, intermediate, vocab
+        self.rms_eps, self.rope_theta = rms_eps, rope_theta
+        self.embeddings, self.final_norm, self.lm_head = _u16(embeddings), _u16(final_norm), _u16(lm_head)
+        self.layers = [{k: _u16(v) for k, v in layer.items()} for layer in layers]
+        self.c_layers = (abi.NervaHipHfDecodeChainLayer * len(self.layers))()
+        for cl, layer in zip(self.c_layers, self.layers):
+            for key, field in _LAYER_FIELDS.items():
+                arr = layer.get(key)
+                setattr(cl, field, arr.ctypes.data if arr is not None else None)
+
+    def fill_dims(self, req):
+        req.dtype, req.hidden, req.heads, req.kv_heads = self.dtype, self.hidden, self.heads, self.kv_heads
+        req.head_dim, req.intermediate, req.vocab_size = self.head_dim, self.intermediate, self.vocab
+        req.layer_count = len(self.layers)
+        req.rms_eps, req.rope_theta = self.rms_eps, self.rope_theta or 0.0
+        req.embeddings = self.embeddings.ctypes.data
+        req.layers = self.c_layers
+        req.final_norm_weight = self.final_norm.ctypes.data
+        req.lm_head = self.lm_head.ctypes.data
+
+
+def greedy_sampler():
+    cfg = abi.NervaHipHfDecodeSamplerConfig()
+    cfg.temperature, cfg.top_p, cfg.top_k, cfg.seed = 0.0, 1.0, 0, 0
+    return cfg
+
+
+class DecodeSession:
+    def __init__(self, handle, create_result, vocab, kv_hidden):
+        self.handle, self.create_result, self.vocab, self.kv_hidden = handle, create_result, vocab, kv_hidden
+        self.lib = abi.load()
+
+    @classmethod
+    def create(cls, weights, max_context, **extra):
+        lib = abi.load()
+        req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
+        weights.fill_dims(req)
+        req.max_context_tokens = max_context
+        for k, v in extra.items():
+            setattr(req, k, v)
+        res = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+        handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+        rc = lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(res), C.byref(handle))
+        if rc != 0:
+            raise RuntimeError("session_create failed: status=%d hip_error=%d stage=%d"
+                               % (res.status, res.hip_error, res.failure_stage))
+        return cls(handle, res, weights.vocab, weights.kv_heads * weights.head_dim)
+
+    @classmethod
+    def create_synthetic(cls, cfg, max_context, seed=0x4E45525641, weight_std=0.02, qk_norm=True):
+        lib = abi.load()
+        req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
+        req.dtype, req.hidden, req.heads, req.kv_heads = cfg["dtype"], cfg["hidden"], cfg["heads"], cfg["kv_heads"]
+        req.head_dim, req.intermediate, req.vocab_size = cfg["head_dim"], cfg["intermediate"], cfg["vocab"]
+        req.layer_count, req.max_context_tokens = cfg["layers"], max_context
+        req.rms_eps, req.rope_theta = cfg["rms_eps"], cfg["rope_theta"] or 0.0
+        res = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+        handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+        rc = lib.nerva_hip_bench_session_create_synthetic(C.byref(req), seed, weight_std, int(qk_norm),
+                                                          C.byref(res), C.byref(handle))
+        if rc != 0:
+            raise RuntimeError("synthetic session_create failed: status=%d hip_error=%d stage=%d"
+                               % (res.status, res.hip_error, res.failure_stage))
+        return cls(handle, res, cfg["vocab"], cfg["kv_heads"] * cfg["head_dim"])
+
+    def start(self, prompt, eos=None, sampler=None):
+        prompt = np.ascontiguousarray(prompt, np.uint32)
+        req = abi.NervaHipHfDecodeSequenceSessionStartRequest()
+        req.session = self.handle
+        req.prompt_tokens, req.prompt_token_count = prompt.ctypes.data, prompt.size
+        req.has_eos_token, req.eos_token = int(eos is not None), int(eos or 0)
+        req.sampler = sampler or greedy_sampler()
+        res = abi.NervaHipHfDecodeSequenceResult()
+        rc = self.lib.nerva_hip_hf_decode_sequence_session_start(C.byref(req), C.byref(res))
+        return rc, res
+
+    def advance(self, steps, capacity=None):
+        out = np.zeros(capacity if capacity is not None else steps, np.uint32)
+        req = abi.NervaHipHfDecodeSequenceSessionAdvanceRequest()
+        req.session, req.steps = self.handle, steps
+        req.output_tokens, req.output_token_capacity = out.ctypes.data, out.size
+        res = abi.NervaHipHfDecodeSequenceResult()
+        rc = self.lib.nerva_hip_hf_decode_sequence_session_advance(C.byref(req), C.byref(res))
+        return rc, res, out[:res.observed_tokens]
+
+    def run(self, prompt, steps, eos=None, sampler=None, seed_token=None):
+        prompt = np.ascontiguousarray(prompt, np.uint32)
+        out = np.zeros(steps, np.uint32)
+        req = abi.NervaHipHfDecodeSequenceSessionRunRequest()
+        req.session, req.steps = self.handle, steps
+        req.seed_token = int(prompt[-1]) if seed_token is None else seed_token
+        req.prompt_tokens, req.prompt_token_count = prompt.ctypes.data, prompt.size
+        req.has_eos_token, req.eos_token = int(eos is not None), int(eos or 0)
+        req.output_tokens, req.output_token_capacity = out.ctypes.data, out.size
+        req.sampler = sampler or greedy_sampler()
+        res = abi.NervaHipHfDecodeSequenceResult()
+        rc = self.lib.nerva_hip_hf_decode_sequence_session_run(C.byref(req), C.byref(res))
+        return rc, res, out[:res.observed_tokens]
+
+    def profile_step(self, repeats=3):
+        res = abi.NervaHipStepProfile()
+        rc = self.lib.nerva_hip_session_profile_step(self.handle, repeats, C.byref(res))
+        return rc, res
+
+    def logits(self):
+        out = np.empty(self.vocab, np.float32)
+        if self.lib.nerva_hip_session_read_logits(self.handle, out.ctypes.data) != 0:
+            raise RuntimeError("read_logits failed")
+        return out
+
+    def kv_row(self, layer, token):
+        k = np.empty(self.kv_hidden, np.uint16)
+        v = np.empty(self.kv_hidden, np.uint16)
+        if self.lib.nerva_hip_session_read_kv(self.handle, layer, token, k.ctypes.data, v.ctypes.data) != 0:
+            raise RuntimeError("read_kv failed")
+        return k, v
+
+    def destroy(self):
+        if self.handle:
+            res = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+            rc = self.lib.nerva_hip_hf_decode_sequence_session_destroy(self.handle, C.byref(res))
+            self.handle = None
+            return rc, res
+        return -1, None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def decode_sequence_oneshot(weights, prompt, steps, eos=None, plan=None):
+    """nerva_hip_hf_decode_sequence_u16: create + run + destroy in one call."""
+    lib = abi.load()
+    prompt = np.ascontiguousarray(prompt, np.uint32)
+    out = np.zeros(steps, np.uint32)
+    req = abi.NervaHipHfDecodeSequenceRequest()
+    weights.fill_dims(req)
+    req.steps, req.seed_token = steps, int(prompt[-1])
+    req.prompt_tokens, req.prompt_token_count = prompt.ctypes.data, prompt.size
+    req.has_eos_token, req.eos_token = int(eos is not None), int(eos or 0)
+    req.output_tokens, req.output_token_capacity = out.ctypes.data, out.size
+    req.sampler = greedy_sampler()
+    for k, v in (plan or {}).items():
+        setattr(req, k, v)
+    res = abi.NervaHipHfDecodeSequenceResult()
+    rc = lib.nerva_hip_hf_decode_sequence_u16(C.byref(req), C.byref(res))
+    return rc, res, out[:res.observed_tokens]

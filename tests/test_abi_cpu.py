@@ -1,0 +1,184 @@
+"""CPU-only checks of the C ABI boundary: the shared library loads, exports every symbol the
+header declares, mirrors the reference struct layouts, and fails closed without a device.
+No compute is attempted here."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from nerva_amd import abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# sizeof/offsetof of the NervaCuda... originals (x86-64 SysV), see include/nerva_hip_layout_check.hpp
+REFERENCE_SIZES = {
+    "NervaHipDeviceSmokeResult": 232, "NervaHipSyntheticTokenSlot": 40, "NervaHipHfDecodeChainLayer": 440,
+    "NervaHipHfDecodeSequenceWeightBlock": 72, "NervaHipHfDecodeSamplerConfig": 24,
+    "NervaHipHfDecodeSequenceRequest": 208, "NervaHipHfDecodeSequenceResult": 528,
+    "NervaHipHfDecodeSequenceSessionCreateRequest": 176, "NervaHipHfDecodeSequenceSessionCreateResult": 272,
+    "NervaHipHfDecodeSequenceSessionRunRequest": 80, "NervaHipHfDecodeSequenceSessionStartRequest": 56,
+    "NervaHipHfDecodeSequenceSessionAdvanceRequest": 32, "NervaHipDeepSeekQuantDequantResult": 96,
+    "NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest": 56,
+    "NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest": 56, "NervaHipProjectionBenchRequest": 24,
+    "NervaHipProjectionBenchResult": 408, "NervaHipDeepSeekMoeForwardRequest": 80,
+    "NervaHipDeepSeekMoeForwardResult": 104,
+}
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(abi.LIBRARY):
+        from nerva_amd import build
+        build.build()
+    return abi.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = abi.declared_symbols()
+    assert len(names) >= 30
+    for name in names:
+        assert hasattr(lib, name), name
+    for required in ("nerva_hip_device_smoke", "nerva_hip_hf_decode_sequence_u16",
+                     "nerva_hip_hf_decode_sequence_session_create", "nerva_hip_hf_decode_sequence_session_start",
+                     "nerva_hip_hf_decode_sequence_session_advance", "nerva_hip_hf_decode_sequence_session_run",
+                     "nerva_hip_hf_decode_sequence_session_destroy",
+                     "nerva_hip_deepseek_quant_fp8_f32_scale_encoded_matvec", "nerva_hip_projection_bench",
+                     "nerva_hip_deepseek_moe_forward", "nerva_hip_gemv", "nerva_hip_fp8_gemv",
+                     "nerva_hip_paged_gqa_decode", "nerva_hip_argmax", "nerva_hip_moe_fp8_experts"):
+        assert required in names
+
+
+def test_struct_layouts_mirror_reference():
+    for name, size in REFERENCE_SIZES.items():
+        assert C.sizeof(abi.STRUCTS[name]) == size, name
+    assert abi.NervaHipSyntheticTokenSlot.version.offset == 24
+    assert abi.NervaHipHfDecodeChainLayer.mlp_kind.offset == 280
+    assert abi.NervaHipHfDecodeSequenceResult.observed_token_hash.offset == 64
+    assert abi.NervaHipHfDecodeSequenceResult.hot_path_allocations.offset == 400
+    assert abi.NervaHipHfDecodeSequenceSessionCreateRequest.detailed_profile.offset == 144
+    assert abi.NervaHipHfDecodeSequenceSessionStartRequest.sampler.offset == 32
+
+
+def test_layout_check_header_compiles(tmp_path):
+    src = tmp_path / "layout.cpp"
+    src.write_text('#include "nerva_hip_layout_check.hpp"\nint main() { return 0; }\n')
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(src)], check=True)
+    subprocess.run(["gcc", "-std=c99", "-fsyntax-only", "-x", "c", os.path.join(ROOT, "include", "nerva_hip_api.h")],
+                   check=True)
+
+
+def _has_gpu(lib):
+    res = abi.NervaHipDeviceSmokeResult()
+    return lib.nerva_hip_device_smoke(C.byref(res)) == 0
+
+
+def test_null_out_and_null_request_fail_closed(lib):
+    """out == NULL -> -1; otherwise the result is zeroed and status = -1
+    (session_api_lifecycle.inc.cu:5-55, 1117-1144)."""
+    assert lib.nerva_hip_device_smoke(None) == -1
+    assert lib.nerva_hip_hf_decode_sequence_session_start(None, None) == -1
+    res = abi.NervaHipHfDecodeSequenceResult()
+    C.memset(C.byref(res), 0xAB, C.sizeof(res))
+    assert lib.nerva_hip_hf_decode_sequence_session_start(None, C.byref(res)) == -1
+    assert res.status == -1 and res.hip_error == 0 and res.hidden == 0 and res.hot_path_allocations == 0
+    C.memset(C.byref(res), 0xAB, C.sizeof(res))
+    assert lib.nerva_hip_hf_decode_sequence_session_advance(None, C.byref(res)) == -1 and res.status == -1
+    assert lib.nerva_hip_hf_decode_sequence_session_run(None, C.byref(res)) == -1 and res.status == -1
+    assert lib.nerva_hip_hf_decode_sequence_u16(None, C.byref(res)) == -1 and res.status == -1
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    assert lib.nerva_hip_hf_decode_sequence_session_create(None, C.byref(cres), C.byref(handle)) == -1
+    assert cres.status == -1 and not handle
+    assert lib.nerva_hip_hf_decode_sequence_session_destroy(None, C.byref(cres)) == -1 and cres.status == -1
+    q = abi.NervaHipDeepSeekQuantDequantResult()
+    assert lib.nerva_hip_deepseek_quant_fp8_f32_scale_encoded_matvec(None, C.byref(q)) == -1 and q.status == -1
+    p = abi.NervaHipProjectionBenchResult()
+    assert lib.nerva_hip_projection_bench(None, C.byref(p)) == -1 and p.status == -1
+    m = abi.NervaHipDeepSeekMoeForwardResult()
+    assert lib.nerva_hip_deepseek_moe_forward(None, C.byref(m)) == -1 and m.status == -1
+
+
+def test_zero_dim_and_missing_weights_are_rejected_before_the_device(lib):
+    req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    req.dtype, req.hidden, req.heads, req.kv_heads, req.head_dim = 1, 0, 1, 1, 2
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.status == -1 and cres.hip_error == 0 and cres.failure_stage == 1
+    req.hidden, req.intermediate, req.vocab_size, req.layer_count, req.max_context_tokens = 2, 2, 4, 1, 4
+    req.rms_eps = 1e-5
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.hip_error == 0                      # null weight pointers: invalid argument, not a device error
+    req.heads, req.kv_heads = 3, 2                  # heads not divisible by kv_heads
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    req.dtype = 2
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+
+
+def _tiny_request():
+    z = np.zeros(8, np.uint16)
+    layer = (abi.NervaHipHfDecodeChainLayer * 1)()
+    for f in ("rms_attn_weight", "rms_mlp_weight", "w_q", "w_k", "w_v", "w_o", "w_gate", "w_up", "w_down"):
+        setattr(layer[0], f, z.ctypes.data)
+    req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
+    req.dtype, req.hidden, req.heads, req.kv_heads, req.head_dim = 0, 2, 1, 1, 2
+    req.intermediate, req.vocab_size, req.layer_count, req.max_context_tokens = 2, 4, 1, 4
+    req.rms_eps = 1e-5
+    req.embeddings = req.final_norm_weight = req.lm_head = z.ctypes.data
+    req.layers = layer
+    return req, layer, z
+
+
+def test_unsupported_features_are_refused_explicitly(lib):
+    """MoE / linear-attention / DeepSeek / RT fields: status -1 with NOT_SUPPORTED, never silently ignored."""
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    for field, value in (("mlp_kind", 1), ("attention_kind", 2), ("deepseek_mode", 1), ("num_experts", 8),
+                         ("linear_key_heads", 2)):
+        req, layer, z = _tiny_request()
+        setattr(layer[0], field, value)
+        assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+        assert cres.hip_error == abi.NERVA_HIP_ERROR_NOT_SUPPORTED, field
+    req, layer, z = _tiny_request()
+    layer[0].w_router = z.ctypes.data
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.hip_error == abi.NERVA_HIP_ERROR_NOT_SUPPORTED
+    req, layer, z = _tiny_request()
+    req.experimental_rt_decode = 1
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.hip_error == abi.NERVA_HIP_ERROR_NOT_SUPPORTED
+
+
+def test_no_device_reports_error_100(lib):
+    """Without a GPU every call that needs one reports status -1, hip_error 100
+    (the reference's stub build: crates/nerva-cuda/src/native_stubs.rs:5-33)."""
+    if _has_gpu(lib):
+        pytest.skip("a GPU is present")
+    smoke = abi.NervaHipDeviceSmokeResult()
+    assert lib.nerva_hip_device_smoke(C.byref(smoke)) == -1
+    assert smoke.status == -1 and smoke.hip_error == abi.NERVA_HIP_ERROR_NO_DEVICE
+    req, layer, z = _tiny_request()
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.status == -1 and cres.hip_error == abi.NERVA_HIP_ERROR_NO_DEVICE and not handle
+    breq = abi.NervaHipProjectionBenchRequest()
+    breq.dtype, breq.rows, breq.cols, breq.iterations = 1, 64, 64, 1
+    bres = abi.NervaHipProjectionBenchResult()
+    assert lib.nerva_hip_projection_bench(C.byref(breq), C.byref(bres)) == -1
+    assert bres.hip_error == abi.NERVA_HIP_ERROR_NO_DEVICE
+    ptr = C.c_void_p()
+    assert lib.nerva_hip_malloc(C.byref(ptr), 64) == -1 and not ptr.value
+
+
+def test_python_package_has_no_cpu_fallback():
+    """The shipped package must not import the oracle or carry a CPU compute path."""
+    pkg = os.path.join(ROOT, "nerva_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cuh", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f
+                assert "libnerva_oracle" not in text and "nvo_" not in text, f

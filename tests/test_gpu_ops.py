@@ -1,0 +1,473 @@
+"""GPU parity tests of the operator entry points, through the C ABI, against the CPU oracle.
+
+Tolerances (stated by the task): relative L2 <= 1e-3 for BF16/FP8 GEMV and attention with
+FP32 accumulation; integer/byte results (codecs, generator, argmax, routing ids) bit-exact.
+"""
+import numpy as np
+import pytest
+
+import nerva_amd as N
+import oracle as O
+from nerva_amd import abi
+from nerva_amd.runtime import attention_workspace
+
+pytestmark = pytest.mark.gpu
+
+BF16, F16 = 1, 0
+SEED = 0x4E45525641
+REL_L2 = 1e-3
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def dev(a):
+    return N.DeviceBuffer.from_numpy(a)
+
+
+def test_device_smoke():
+    rc, res = N.Device.smoke()
+    assert rc == 0 and res.status == 0 and res.device_count >= 1
+    assert res.value == 0x4E455256
+    print("GPU:", res.gpu_name.decode(), "mem", res.total_global_mem >> 30, "GiB", flush=True)
+
+
+def test_synthetic_generator_matches_oracle_bit_for_bit():
+    lib = abi.load()
+    n = 100003
+    for dtype in (BF16, F16):
+        buf = N.DeviceBuffer(n * 2)
+        assert lib.nerva_hip_synth_fill_16(buf.ptr, dtype, SEED, 7, n, 1.0, 0.02) == 0
+        assert np.array_equal(buf.numpy(np.uint16), O.synth_16(dtype, SEED, 7, n, 1.0, 0.02))
+    buf = N.DeviceBuffer(n * 4)
+    assert lib.nerva_hip_synth_fill_f32(buf.ptr, SEED, 8, n, 0.0, 1.0) == 0
+    assert np.array_equal(buf.numpy(np.float32).view(np.uint32), O.synth_f32(SEED, 8, n, 0.0, 1.0).view(np.uint32))
+    rows, cols, block = 130, 260, 128
+    w = N.DeviceBuffer(rows * cols)
+    s = N.DeviceBuffer(2 * 3 * 4)
+    assert lib.nerva_hip_synth_fill_fp8_block(w.ptr, s.ptr, SEED, 9, rows, cols, block, 0.02) == 0
+    ow, os_ = O.synth_fp8_block(SEED, 9, rows, cols, block, 0.02)
+    assert np.array_equal(s.numpy(np.float32).view(np.uint32), os_.ravel().view(np.uint32))
+    assert np.array_equal(w.numpy(np.uint8), ow.ravel())
+
+
+# ---------------------------------------------------------------------------
+# BF16/F16 GEMV family
+# ---------------------------------------------------------------------------
+
+def _gemv_case(dtype, rows, cols, seed, std=0.02):
+    rng = np.random.default_rng(seed)
+    w = O.encode16(dtype, rng.normal(0, std, (rows, cols)))
+    x = O.encode16(dtype, rng.normal(0, 1, cols))
+    return w, x
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (6144, 4096), (1030, 12288), (37, 520), (5, 2), (3, 4104), (2, 7)])
+def test_gemv_plain_matches_oracle(dtype, rows, cols):
+    """Config 1 (q_proj 4096x4096 bf16, x bf16, bf16 out) plus ragged / unaligned shapes."""
+    w, x = _gemv_case(dtype, rows, cols, rows * 31 + cols)
+    ref = O.gemv_x16(dtype, w, x)
+    dw, dx = dev(w), dev(x)
+    y32 = N.DeviceBuffer(rows * 4)
+    N.gemv(dtype, dw, rows, cols, input16=dx, out_f32=y32, epilogue=0)
+    got = y32.numpy(np.float32)
+    assert rel_l2(got, ref) <= REL_L2
+    assert np.max(np.abs(got - ref)) <= 1e-3 * max(1.0, np.max(np.abs(ref)))
+    y16 = N.DeviceBuffer(max(16, rows * 2))
+    N.gemv(dtype, dw, rows, cols, input16=dx, out16=y16, epilogue=3)
+    got16 = O.decode16(dtype, y16.numpy(np.uint16, rows))
+    assert rel_l2(got16, O.decode16(dtype, O.encode16(dtype, ref))) <= 4e-3  # one 16-bit rounding of y
+    # rounding the device's own f32 result reproduces its 16-bit output exactly
+    assert np.array_equal(y16.numpy(np.uint16, rows), O.encode16(dtype, got))
+
+
+def test_gemv_linearity_and_unit_vectors_full_size():
+    """Size-independent properties at the full q_proj size: W.e_j = column j; W.(a+b) = W.a + W.b."""
+    rows = cols = 4096
+    w = O.synth_16(BF16, SEED, 100, rows * cols, 0.0, 0.02).reshape(rows, cols)
+    dw = dev(w)
+    y = N.DeviceBuffer(rows * 4)
+    e = np.zeros(cols, np.float32)
+    e[1234] = 1.0
+    N.gemv(BF16, dw, rows, cols, input16=dev(O.encode16(BF16, e)), out_f32=y)
+    assert np.array_equal(y.numpy(np.float32), O.decode16(BF16, w[:, 1234]))
+    a = O.encode16(BF16, np.random.default_rng(1).integers(-8, 8, cols).astype(np.float32))
+    b = O.encode16(BF16, np.random.default_rng(2).integers(-8, 8, cols).astype(np.float32))
+    ab = O.encode16(BF16, O.decode16(BF16, a) + O.decode16(BF16, b))  # small integers: exact in bf16
+    outs = []
+    for v in (a, b, ab):
+        N.gemv(BF16, dw, rows, cols, input16=dev(v), out_f32=y)
+        outs.append(y.numpy(np.float32).astype(np.float64))
+    assert rel_l2(outs[2], outs[0] + outs[1]) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("cols,rows", [(4096, 6144), (520, 64), (6, 3)])
+def test_gemv_rmsnorm_prologue(dtype, cols, rows):
+    """qkv projection: x = round16(rmsnorm(h, gamma)) fused in front of the GEMV."""
+    rng = np.random.default_rng(cols)
+    h = rng.normal(0, 1, cols).astype(np.float32)
+    gamma = O.encode16(dtype, rng.normal(1, 0.02, cols))
+    w = O.encode16(dtype, rng.normal(0, 0.02, (rows, cols)))
+    n16 = O.encode16(dtype, O.rms_norm(dtype, h, gamma, 1e-6))
+    ref = O.gemv_x16(dtype, w, n16)
+    y = N.DeviceBuffer(rows * 4)
+    N.gemv(dtype, dev(w), rows, cols, input_f32=dev(h), gamma=dev(gamma), eps=1e-6, out_f32=y)
+    assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
+
+
+@pytest.mark.parametrize("full", [False, True])
+def test_mlp_block_matches_oracle(full):
+    """Config 2: RMSNorm -> fused gate+up GEMV -> SiLU(gate)*up -> down GEMV -> residual add."""
+    hidden, inter = (4096, 12288) if full else (512, 1536)
+    dtype = BF16
+    if full:
+        wgu = O.synth_16(dtype, SEED, 200, 2 * inter * hidden, 0.0, 0.02).reshape(2 * inter, hidden)
+        wd = O.synth_16(dtype, SEED, 201, hidden * inter, 0.0, 0.02).reshape(hidden, inter)
+    else:
+        rng = np.random.default_rng(5)
+        wgu = O.encode16(dtype, rng.normal(0, 0.02, (2 * inter, hidden)))
+        wd = O.encode16(dtype, rng.normal(0, 0.02, (hidden, inter)))
+    h = O.decode16(dtype, O.synth_16(dtype, SEED, 202, hidden, 0.0, 1.0))
+    gamma = O.synth_16(dtype, SEED, 203, hidden, 1.0, 0.02)
+    # oracle, device-session staging
+    m16 = O.encode16(dtype, O.rms_norm(dtype, h, gamma, 1e-6))
+    gu = O.gemv(dtype, wgu, O.decode16(dtype, m16), threads=8)
+    g, u = gu[:inter], gu[inter:]
+    ff = (g / (1.0 + np.exp(-g.astype(np.float64)))).astype(np.float32) * u
+    ff16 = O.encode16(dtype, ff)
+    ref = h + O.gemv(dtype, wd, O.decode16(dtype, ff16), threads=8)
+    # device
+    dff = N.DeviceBuffer(inter * 2)
+    dout = N.DeviceBuffer(hidden * 4)
+    dh = dev(h)
+    N.gemv(dtype, dev(wgu), inter, hidden, input_f32=dh, gamma=dev(gamma), eps=1e-6, out16=dff, epilogue=2)
+    N.gemv(dtype, dev(wd), hidden, inter, input16=dff, residual=dh, out_f32=dout, epilogue=1)
+    got_ff = O.decode16(dtype, dff.numpy(np.uint16))
+    assert rel_l2(got_ff, O.decode16(dtype, ff16)) <= 3e-3  # 16-bit rounding of an f32 result
+    assert rel_l2(dout.numpy(np.float32), ref) <= REL_L2
+    # prompt-token staging: the sum is rounded to 16 bits
+    N.gemv(dtype, dev(wd), hidden, inter, input16=dff, residual=dh, out_f32=dout, epilogue=1, round_output=True)
+    got = dout.numpy(np.float32)
+    assert np.array_equal(got, O.decode16(dtype, O.encode16(dtype, got)))
+
+
+def test_gemv_bias_and_invalid_arguments():
+    rows, cols = 64, 512
+    w, x = _gemv_case(BF16, rows, cols, 3)
+    bias = O.encode16(BF16, np.random.default_rng(4).normal(0, 1, rows))
+    y = N.DeviceBuffer(rows * 4)
+    N.gemv(BF16, dev(w), rows, cols, input16=dev(x), bias=dev(bias), out_f32=y)
+    assert rel_l2(y.numpy(np.float32), O.gemv_x16(BF16, w, x) + O.decode16(BF16, bias)) <= REL_L2
+    lib = abi.load()
+    req = abi.NervaHipGemvRequest()
+    import ctypes as C
+    err = C.c_int32(0)
+    assert lib.nerva_hip_gemv(None, None, C.byref(err)) == -1
+    assert lib.nerva_hip_gemv(C.byref(req), None, C.byref(err)) == -1 and err.value != 0  # all-null request
+    req.dtype, req.rows, req.cols, req.epilogue = 7, 4, 4, 0
+    assert lib.nerva_hip_gemv(C.byref(req), None, C.byref(err)) == -1
+
+
+# ---------------------------------------------------------------------------
+# FP8 block-scaled GEMV
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("cols", [1024, 3])
+def test_fp8_decode_all_256_codes(cols):
+    """Every e4m3fn code through the device decode (hardware path at cols=1024, bit path at cols=3)."""
+    w = np.zeros((256, cols), np.uint8)
+    w[:, 0] = np.arange(256)
+    x = np.zeros(cols, np.float32)
+    x[0] = 1.0
+    y = N.DeviceBuffer(256 * 4)
+    scales = np.ones((2, -(-cols // 128)), np.float32)
+    N.fp8_gemv(dev(w), dev(scales), 256, cols, 128, 128, y, input16=dev(O.encode16(BF16, x)))
+    got = y.numpy(np.float32)
+    want = O.decode_fp8(np.arange(256, dtype=np.uint8))
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan], want[~nan])
+
+
+def test_fp8_matvec_kat_host_pointer_abi(kat):
+    import ctypes as C
+    k = kat["fp8_f32_scale_matvec"]
+    w = np.array([int(v, 16) for v in k["weights"]], np.uint8)
+    s = np.array(k["scales"], np.float32)
+    x16 = O.encode16(BF16, np.array(k["input"], np.float32))
+    out = np.zeros(k["rows"], np.float32)
+    req = abi.NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest()
+    req.rows, req.cols, req.block_rows, req.block_cols, req.input_dtype = k["rows"], k["cols"], k["block_rows"], k["block_cols"], BF16
+    req.weights, req.scales, req.input, req.output = w.ctypes.data, s.ctypes.data, x16.ctypes.data, out.ctypes.data
+    res = abi.NervaHipDeepSeekQuantDequantResult()
+    assert abi.load().nerva_hip_deepseek_quant_fp8_f32_scale_encoded_matvec(C.byref(req), C.byref(res)) == 0
+    assert out.tolist() == k["expected"]
+    assert (res.rows, res.cols, res.block_rows, res.block_cols) == (3, 4, 2, 2)
+    assert res.kernel_launches == 1 and res.sync_calls == 1 and res.hot_path_allocations == 0
+    assert res.output_hash == O.fnv1a(out) != 0
+
+
+def test_fp8_gemm_tokens_ragged_kat(kat):
+    import ctypes as C
+    k = kat["fp8_gemm_tokens_ragged"]
+    rows, cols, tokens = k["rows"], k["cols"], k["tokens"]
+    pat = [int(v, 16) for v in k["weight_pattern"]]
+    w = np.array([pat[i % len(pat)] for i in range(rows * cols)], np.uint8)
+    x16 = O.encode16(BF16, np.array([((i % 17) - 8) / 32 for i in range(tokens * cols)], np.float32))
+    s = np.array(k["scales"], np.float32)
+    out = np.zeros(tokens * rows, np.float32)
+    req = abi.NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest()
+    req.rows, req.cols, req.tokens, req.block_rows, req.block_cols, req.input_dtype = rows, cols, tokens, 128, 128, BF16
+    req.weights, req.scales, req.input, req.output = w.ctypes.data, s.ctypes.data, x16.ctypes.data, out.ctypes.data
+    res = abi.NervaHipDeepSeekQuantDequantResult()
+    assert abi.load().nerva_hip_deepseek_quant_fp8_f32_scale_encoded_gemm_tokens(C.byref(req), C.byref(res)) == 0
+    ref = O.fp8_gemm_tokens(w, s, x16, rows, cols, tokens, 128, 128)
+    assert np.max(np.abs(out.reshape(tokens, rows) - ref)) < k["abs_tol"]
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 7168), (7168, 2048), (300, 1024), (130, 260)])
+def test_fp8_gemv_matches_oracle(rows, cols):
+    w, s = O.synth_fp8_block(SEED, rows + cols, rows, cols, 128, 0.02)
+    x16 = O.synth_16(BF16, SEED, 11, cols, 0.0, 1.0)
+    ref = O.fp8_gemm_tokens(w, s, x16, rows, cols, 1, 128, 128)[0]
+    y = N.DeviceBuffer(rows * 4)
+    N.fp8_gemv(dev(w), dev(s), rows, cols, 128, 128, y, input16=dev(x16))
+    assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
+    xf = O.decode16(BF16, x16)
+    N.fp8_gemv(dev(w), dev(s), rows, cols, 128, 128, y, input_f32=dev(xf))
+    assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
+
+
+# ---------------------------------------------------------------------------
+# Paged GQA decode attention
+# ---------------------------------------------------------------------------
+
+def _attention_case(dtype, heads, kv_heads, hd, tokens, theta, qk_norm, seed, layers=2, layer=1, bias=False):
+    rng = np.random.default_rng(seed)
+    kvh = kv_heads * hd
+    n_blocks = tokens // 16 + 2
+    table = rng.permutation(n_blocks).astype(np.uint32)
+    k_rows = O.encode16(dtype, rng.normal(0, 1, (tokens, kvh)))
+    v_rows = O.encode16(dtype, rng.normal(0, 1, (tokens, kvh)))
+    qkv = rng.normal(0, 1, heads * hd + 2 * kvh).astype(np.float32)
+    qn = O.encode16(dtype, rng.normal(1, 0.02, hd)) if qk_norm else None
+    kn = O.encode16(dtype, rng.normal(1, 0.02, hd)) if qk_norm else None
+    biases = [O.encode16(dtype, rng.normal(0, 0.1, n)) for n in (heads * hd, kvh, kvh)] if bias else [None] * 3
+    return dict(dtype=dtype, heads=heads, kv_heads=kv_heads, hd=hd, tokens=tokens, theta=theta, table=table,
+                n_blocks=n_blocks, k_rows=k_rows, v_rows=v_rows, qkv=qkv, qn=qn, kn=kn, biases=biases,
+                layers=layers, layer=layer)
+
+
+def _attention_oracle(c, eps=1e-6):
+    """Reference staging: bias -> per-head norm -> RoPE -> K/V rounded -> attention over pos+1 keys."""
+    dtype, heads, kv_heads, hd = c["dtype"], c["heads"], c["kv_heads"], c["hd"]
+    A, KV = heads * hd, kv_heads * hd
+    pos = c["tokens"]
+    q, k, v = c["qkv"][:A].copy(), c["qkv"][A:A + KV].copy(), c["qkv"][A + KV:].copy()
+    for vec, b in zip((q, k, v), c["biases"]):
+        if b is not None:
+            vec += O.decode16(dtype, b)
+    if c["qn"] is not None:
+        q = O.per_head_rms_norm(dtype, c["qn"], hd, q, eps)
+        k = O.per_head_rms_norm(dtype, c["kn"], hd, k, eps)
+    if c["theta"]:
+        q = O.rope(hd, heads, pos, c["theta"], q)
+        k = O.rope(hd, kv_heads, pos, c["theta"], k)
+    k16, v16 = O.encode16(dtype, k), O.encode16(dtype, v)
+    # oracle cache layout [layer][block][16][kv_hidden]
+    kc = np.zeros((c["layers"], c["n_blocks"], 16, KV), np.uint16)
+    vc = np.zeros_like(kc)
+    rows_k = np.vstack([c["k_rows"], k16[None]])
+    rows_v = np.vstack([c["v_rows"], v16[None]])
+    for t in range(pos + 1):
+        kc[c["layer"], c["table"][t // 16], t % 16] = rows_k[t]
+        vc[c["layer"], c["table"][t // 16], t % 16] = rows_v[t]
+    out = O.attention_paged16(dtype, heads, kv_heads, hd, 16, q, kc, vc, c["table"], c["layer"],
+                              c["n_blocks"], pos + 1)
+    return out, k16, v16
+
+
+def _attention_device(c, eps=1e-6):
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], c["kv_heads"], c["hd"], c["table"])
+    cache.fill(c["layer"], c["k_rows"], c["v_rows"])
+    ws = attention_workspace(c["heads"], c["hd"])
+    A = c["heads"] * c["hd"]
+    out16 = N.DeviceBuffer(max(16, A * 2))
+    out32 = N.DeviceBuffer(A * 4)
+    opt = lambda a: dev(a) if a is not None else None
+    qb, kb, vb = (opt(b) for b in c["biases"])
+    N.paged_attention(c["dtype"], c["heads"], c["kv_heads"], c["hd"], cache, c["layer"], c["tokens"],
+                      dev(c["qkv"]), ws, out16, out_f32=out32, append=True, eps=eps,
+                      rope_theta=c["theta"] or 0.0, q_norm=opt(c["qn"]), k_norm=opt(c["kn"]),
+                      q_bias=qb, k_bias=kb, v_bias=vb)
+    k_new, v_new = cache.read_row(c["layer"], c["tokens"])
+    return out32.numpy(np.float32), out16.numpy(np.uint16, A), k_new, v_new, cache, ws
+
+
+@pytest.mark.parametrize("tokens", [0, 1, 15, 16, 17, 100, 1000, 4096])
+def test_paged_attention_config3_shapes(tokens):
+    """Config 3: 32 q / 8 kv heads x 128, bf16 16-token blocks, permuted table, QK-norm, RoPE 1e6."""
+    c = _attention_case(BF16, 32, 8, 128, tokens, 1e6, True, 1000 + tokens)
+    ref, k16, v16 = _attention_oracle(c)
+    got32, got16, k_new, v_new, _, _ = _attention_device(c)
+    # the appended K row passes through powf/sincos: allow 1 unit in the last place of the 16-bit value
+    assert np.max(np.abs(k_new.astype(np.int32) - k16.astype(np.int32))) <= 1
+    assert np.mean(k_new != k16) < 0.02
+    assert np.array_equal(v_new, v16)
+    assert rel_l2(got32, ref) <= REL_L2
+    assert np.array_equal(got16, O.encode16(BF16, got32))
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd,dtype,theta,qk_norm,bias", [
+    (8, 8, 128, BF16, 1e4, False, False),     # MHA, no norm
+    (16, 8, 128, F16, 1e6, True, True),       # group 2, f16, biases
+    (64, 8, 128, BF16, 0, True, False),       # group 8, no RoPE
+    (4, 2, 64, BF16, 1e4, True, True),        # generic path: head_dim 64
+    (6, 2, 32, F16, 1e4, False, False),       # generic path: group 3
+    (1, 1, 2, F16, 0, False, False),          # tiny known-answer geometry
+])
+def test_paged_attention_other_geometries(heads, kv_heads, hd, dtype, theta, qk_norm, bias):
+    for tokens in (0, 5, 70):
+        c = _attention_case(dtype, heads, kv_heads, hd, tokens, theta, qk_norm, heads * 7 + tokens, bias=bias)
+        ref, k16, v16 = _attention_oracle(c)
+        got32, got16, k_new, v_new, _, _ = _attention_device(c)
+        assert np.max(np.abs(k_new.astype(np.int32) - k16.astype(np.int32))) <= 1
+        assert np.array_equal(v_new, v16)
+        assert rel_l2(got32, ref) <= REL_L2
+
+
+def test_paged_attention_permutation_invariance_and_repeatability():
+    """Same logical KV under two block tables gives the same bits; so does calling twice."""
+    base = _attention_case(BF16, 32, 8, 128, 777, 1e6, True, 42)
+    outs = []
+    for seed in (1, 2):
+        c = dict(base)
+        c["table"] = np.random.default_rng(seed).permutation(base["n_blocks"]).astype(np.uint32)
+        got32, _, _, _, _, _ = _attention_device(c)
+        outs.append(got32)
+        got_again, _, _, _, _, _ = _attention_device(c)
+        assert np.array_equal(got32, got_again)
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_paged_attention_no_append_reads_cache_only():
+    c = _attention_case(BF16, 32, 8, 128, 200, 1e6, True, 9)
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
+    cache.fill(c["layer"], c["k_rows"], c["v_rows"])
+    ws = attention_workspace(32, 128)
+    out16, out32 = N.DeviceBuffer(4096 * 2), N.DeviceBuffer(4096 * 4)
+    N.paged_attention(BF16, 32, 8, 128, cache, c["layer"], 199, dev(c["qkv"]), ws, out16, out_f32=out32,
+                      append=False, rope_theta=1e6, q_norm=dev(c["qn"]), k_norm=dev(c["kn"]))
+    q = O.rope(128, 32, 199, 1e6, O.per_head_rms_norm(BF16, c["qn"], 128, c["qkv"][:4096], 1e-6))
+    kc = np.zeros((c["layers"], c["n_blocks"], 16, 1024), np.uint16)
+    vc = np.zeros_like(kc)
+    for t in range(200):
+        kc[c["layer"], c["table"][t // 16], t % 16] = c["k_rows"][t]
+        vc[c["layer"], c["table"][t // 16], t % 16] = c["v_rows"][t]
+    ref = O.attention_paged16(BF16, 32, 8, 128, 16, q, kc, vc, c["table"], c["layer"], c["n_blocks"], 200)
+    assert rel_l2(out32.numpy(np.float32), ref) <= REL_L2
+
+
+# ---------------------------------------------------------------------------
+# argmax, MoE
+# ---------------------------------------------------------------------------
+
+def test_argmax_matches_oracle_rules():
+    rng = np.random.default_rng(0)
+    for n in (1, 4, 1000, 151936):
+        l = rng.normal(0, 1, n).astype(np.float32)
+        assert N.argmax(dev(l), n) == O.greedy_argmax(l, skip_nonfinite=True)
+    l = rng.normal(0, 1, 151936).astype(np.float32)
+    l[[777, 150000, 90000]] = l.max() + 1.0   # exact three-way tie -> lowest index
+    assert N.argmax(dev(l), l.size) == 777
+    l[100] = np.nan
+    l[777] = np.inf                             # non-finite candidates are skipped
+    assert N.argmax(dev(l), l.size) == 90000 == O.greedy_argmax(l, skip_nonfinite=True)
+    ws = N.DeviceBuffer.zeros(abi.load().nerva_hip_argmax_workspace_bytes())
+    for _ in range(3):                          # the workspace re-arms itself
+        assert N.argmax(dev(l), l.size, ws) == 90000
+
+
+def test_moe_route_matches_oracle():
+    rng = np.random.default_rng(3)
+    for e, k, norm in ((256, 8, True), (256, 8, False), (64, 6, True), (5, 5, True)):
+        logits = rng.normal(0, 1, e).astype(np.float32)
+        ids, wts, _, _ = N.moe_route_softmax(logits, k, norm)
+        rid, rw = O.moe_route_softmax(logits, k, norm)
+        assert ids.tolist() == rid.tolist()
+        assert np.allclose(wts, rw, rtol=2e-6, atol=0)
+    ids, _, _, _ = N.moe_route_softmax(np.zeros(6, np.float32), 3, True)
+    assert ids.tolist() == [0, 1, 2]
+
+
+@pytest.mark.parametrize("hidden,inter,experts,top_k", [(1024, 1024, 6, 2), (7168, 2048, 12, 8)])
+def test_moe_fp8_experts_match_oracle(hidden, inter, experts, top_k):
+    """Config 4 geometry (hidden 7168, intermediate 2048, top-8 + 1 shared) on a 12-expert bank."""
+    B = 128
+    wg = np.empty((experts, inter, hidden), np.uint8)
+    wu = np.empty_like(wg)
+    wd = np.empty((experts, hidden, inter), np.uint8)
+    sg = np.empty((experts, inter // B, hidden // B), np.float32)
+    su = np.empty_like(sg)
+    sd = np.empty((experts, hidden // B, inter // B), np.float32)
+    for e in range(experts):
+        wg[e], sg[e] = O.synth_fp8_block(SEED, 300 + e, inter, hidden, B, 0.02)
+        wu[e], su[e] = O.synth_fp8_block(SEED, 400 + e, inter, hidden, B, 0.02)
+        wd[e], sd[e] = O.synth_fp8_block(SEED, 500 + e, hidden, inter, B, 0.02)
+    x16 = O.synth_16(BF16, SEED, 12, hidden, 0.0, 1.0)
+    logits = O.synth_f32(SEED, 13, experts - 1, 0.0, 1.0)      # the last expert is the shared one
+    ids, wts, dids, dwts = N.moe_route_softmax(logits, top_k, True)
+    rid, rw = O.moe_route_softmax(logits, top_k, True)
+    assert ids.tolist() == rid.tolist()
+    ref = O.moe_fp8_forward(hidden, inter, experts, B, x16, rid, rw, wg, sg, wu, su, wd, sd,
+                            shared_index=experts - 1)
+    act = N.DeviceBuffer((top_k + 1) * inter * 4)
+    out = N.DeviceBuffer(hidden * 4)
+    N.moe_fp8_experts(hidden, inter, experts, top_k, B, dev(x16), dids, dwts, dev(wg), dev(sg), dev(wu),
+                      dev(su), dev(wd), dev(sd), act, out, shared_index=experts - 1)
+    assert rel_l2(out.numpy(np.float32), ref) <= REL_L2
+    # no shared expert
+    ref2 = O.moe_fp8_forward(hidden, inter, experts, B, x16, rid, rw, wg, sg, wu, su, wd, sd)
+    N.moe_fp8_experts(hidden, inter, experts, top_k, B, dev(x16), dids, dwts, dev(wg), dev(sg), dev(wu),
+                      dev(su), dev(wd), dev(sd), act, out, shared_index=-1)
+    assert rel_l2(out.numpy(np.float32), ref2) <= REL_L2
+
+
+def test_moe_forward_f32_kat_host_pointer_abi(kat):
+    import ctypes as C
+    k = kat["moe_routed_clamp"]
+    f = lambda v: np.array(v, np.float32)
+    x, wg, wu, wd = f(k["input"]), f(k["w_gate"]), f(k["w_up"]), f(k["w_down"])
+    ids, wts = np.array(k["expert_ids"], np.uint32), f(k["expert_weights"])
+    out = np.zeros(k["hidden"], np.float32)
+    req = abi.NervaHipDeepSeekMoeForwardRequest()
+    req.hidden_size, req.intermediate_size, req.num_experts, req.top_k = k["hidden"], k["intermediate"], 2, 2
+    req.clamp_swiglu, req.swiglu_limit = 1, k["swiglu_limit"]
+    req.input, req.expert_ids, req.expert_weights = x.ctypes.data, ids.ctypes.data, wts.ctypes.data
+    req.w_gate, req.w_up, req.w_down, req.output = wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, out.ctypes.data
+    res = abi.NervaHipDeepSeekMoeForwardResult()
+    assert abi.load().nerva_hip_deepseek_moe_forward(C.byref(req), C.byref(res)) == 0
+    ref = O.moe_forward_f32(k["hidden"], k["intermediate"], x, ids, wts, wg, wu, wd, limit=k["swiglu_limit"])
+    assert np.max(np.abs(out - ref)) < k["tol"]
+    assert res.hot_path_allocations == 0 and res.sync_calls == 1
+    ids[0] = 9  # out-of-range expert id is refused before touching the device
+    assert abi.load().nerva_hip_deepseek_moe_forward(C.byref(req), C.byref(res)) == -1 and res.moe_error != 0
+
+
+def test_projection_bench_runs_and_checks_itself():
+    import ctypes as C
+    req = abi.NervaHipProjectionBenchRequest()
+    req.dtype, req.rows, req.cols, req.iterations, req.warmup_iterations, req.block_tokens = BF16, 4096, 4096, 40, 5, 1
+    res = abi.NervaHipProjectionBenchResult()
+    assert abi.load().nerva_hip_projection_bench(C.byref(req), C.byref(res)) == 0
+    assert res.mismatch_count == 0 and res.max_abs_diff < 1e-2
+    assert res.hot_path_allocations == 0 and res.graph_captures == 1
+    assert res.matrix_bytes == 4096 * 4096 * 2 and res.custom_avg_ns > 0 and res.custom_graph_avg_ns > 0
+    print("q_proj GEMV eager %d ns, graph %d ns, %.0f GB/s" % (
+        res.custom_avg_ns, res.custom_graph_avg_ns,
+        (res.matrix_bytes + res.input_bytes + res.output_bytes) / res.custom_graph_avg_ns), flush=True)

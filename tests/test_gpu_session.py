@@ -1,0 +1,273 @@
+"""GPU parity tests of the decode session (create / start / advance / run / destroy) through the
+C ABI: the reference's end-to-end known-answer streams, and random small models against the CPU
+oracle (logits, KV rows, greedy token streams)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import nerva_amd as N
+import oracle as O
+from conftest import hx
+from nerva_amd import abi
+from nerva_amd.session import decode_sequence_oneshot
+
+pytestmark = pytest.mark.gpu
+
+BF16, F16 = 1, 0
+REL_L2 = 1e-3
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def kat_models(kat, qk_norm):
+    k = kat["decode_sequence"]
+    one = lambda name: np.array([hx(v) for v in k[name]], np.uint16)
+    layer = dict(rms_attn=one("rms"), rms_mlp=one("rms"), w_q=one("matrix"), w_k=one("matrix"),
+                 w_v=one("matrix"), w_o=one("matrix"), w_gate=one("matrix"), w_up=one("matrix"),
+                 w_down=one("matrix"))
+    if qk_norm:
+        layer.update(q_norm=one("rms"), k_norm=one("rms"))
+    args = (F16, k["hidden"], k["heads"], k["kv_heads"], k["head_dim"], k["intermediate"], k["vocab"],
+            k["rms_eps"], k["rope_theta"], one("embeddings"), [layer], one("rms"), one("lm_head"))
+    return N.ModelWeights(*args), k
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_reference_greedy_stream_kat(kat, qk_norm):
+    """hidden 2 / vocab 4 model, prompt [0], 4 steps -> [1,2,3,0]; with eos 2 -> [1,2]
+    (crates/nerva-cuda/src/tests/decode_sequence.rs:123-223, decode_sequence_qk_norm.rs:11-91)."""
+    weights, k = kat_models(kat, qk_norm)
+    rc, res, tokens = decode_sequence_oneshot(weights, k["prompt"], k["steps"])
+    assert rc == 0 and res.status == 0
+    assert tokens.tolist() == k["tokens"]
+    assert res.observed_tokens == 4 and res.last_token == 0 and res.kv_tokens == 4
+    assert res.observed_token_hash == O.fnv1a(np.array(k["tokens"], np.uint32))
+    assert res.graph_replays == 4 and res.graph_launches == 4 and res.sync_calls == 1
+    assert res.host_causality_edges == 0 and res.hot_path_allocations == 0
+    assert res.resident_weight_bytes == (108 if qk_norm else 100)
+    assert res.kernel_launches == res.graph_replays * res.graph_nodes
+    rc, res, tokens = decode_sequence_oneshot(weights, k["prompt"], k["steps"], eos=k["eos_token"])
+    assert rc == 0 and tokens.tolist() == k["tokens_with_eos"]
+    assert res.kv_tokens == k["kv_tokens_with_eos"] and res.graph_replays == 4
+
+
+def test_weight_plan_echo_and_mismatch(kat):
+    weights, k = kat_models(kat, False)
+    plan = dict(planned_weight_blocks=12, planned_gpu_resident_blocks=6, planned_gpu_staged_blocks=6,
+                planned_weight_bytes=100, planned_gpu_resident_weight_bytes=52,
+                planned_gpu_staged_weight_bytes=48, planned_weight_descriptor_hash=1234)
+    rc, res, tokens = decode_sequence_oneshot(weights, k["prompt"], k["steps"], plan=plan)
+    assert rc == 0 and tokens.tolist() == k["tokens"]
+    assert res.planned_weight_blocks == 12 and res.planned_weight_bytes == res.resident_weight_bytes == 100
+    assert res.planned_gpu_resident_weight_bytes == 52 and res.planned_gpu_staged_weight_bytes == 48
+    assert res.descriptor_gpu_resident_h2d_bytes == 52 and res.descriptor_gpu_staged_h2d_bytes == 48
+    plan["planned_weight_bytes"] = 99  # a plan that disagrees with the arena is rejected
+    rc, res, _ = decode_sequence_oneshot(weights, k["prompt"], k["steps"], plan=plan)
+    assert rc == -1 and res.status == -1
+
+
+def test_session_lifecycle_kat(kat):
+    """create -> start -> advance in pieces; token accounting of the reference
+    (session_api_lifecycle.inc.cu:992-1311): the first advance(n) does n-1 replays."""
+    weights, k = kat_models(kat, True)
+    s = N.DecodeSession.create(weights, 16)
+    assert s.create_result.status == 0 and s.create_result.hot_path_allocations == 0
+    assert s.create_result.resident_weight_bytes == 108 and s.create_result.resident_kv_bytes > 0
+    rc, res, _ = s.advance(1)
+    assert rc == -1                                   # advance before start
+    rc, res = s.start([0])
+    assert rc == 0 and res.kv_tokens == 1 and res.seed_token == 0
+    rc, res, t1 = s.advance(2)
+    assert rc == 0 and t1.tolist() == [1, 2] and res.graph_replays == 1 and res.seed_token == 0
+    assert res.hot_path_allocations == 0 and res.host_causality_edges == 0 and res.sync_calls == 1
+    rc, res, t2 = s.advance(6)
+    assert rc == 0 and t2.tolist() == [3, 0, 1, 2, 3, 0] and res.graph_replays == 6
+    assert res.seed_token == 2 and res.kv_tokens == 8 and res.graph_cache_hits == 1
+    rc, res, _ = s.advance(20)                        # past max_context_tokens
+    assert rc == -1
+    # restart on the same session with a 3-token prompt and a stop token
+    rc, res = s.start([2, 1, 0], eos=3)
+    assert rc == 0 and res.kv_tokens == 3
+    rc, res, t3 = s.advance(5)
+    assert rc == 0 and t3.tolist() == [1, 2, 3] and res.observed_tokens == 3
+    rc, res, _ = s.advance(1)                         # finished after the stop token
+    assert rc == -1
+    # run(): the step graph walks the prompt too
+    rc, res, t4 = s.run([0], 4)
+    assert rc == 0 and t4.tolist() == [1, 2, 3, 0] and res.graph_replays == 4
+    rc, dres = s.destroy()
+    assert rc == 0 and dres.status == 0
+
+
+def test_argument_validation_on_device(kat):
+    weights, k = kat_models(kat, False)
+    s = N.DecodeSession.create(weights, 8)
+    rc, res = s.start([7])                            # token >= vocab
+    assert rc == -1 and res.status == -1
+    rc, res = s.start([])
+    assert rc == -1
+    rc, res = s.start(list(range(4)) * 3)             # prompt longer than the context
+    assert rc == -1
+    sampler = abi.NervaHipHfDecodeSamplerConfig()
+    sampler.temperature, sampler.top_p, sampler.top_k = 0.7, 0.9, 40
+    rc, res = s.start([0], sampler=sampler)           # non-greedy sampling: explicit refusal
+    assert rc == -1 and res.hip_error == abi.NERVA_HIP_ERROR_NOT_SUPPORTED
+    sampler.top_p = 0.0
+    rc, res = s.start([0], sampler=sampler)           # invalid sampler config
+    assert rc == -1 and res.hip_error == 0
+    rc, res = s.start([0])
+    assert rc == 0
+    rc, res, _ = s.advance(3, capacity=2)             # capacity < steps
+    assert rc == -1
+    rc, res, _ = s.run([0, 1], 3, seed_token=0)       # seed token must be the last prompt token
+    assert rc == -1
+    s.destroy()
+
+
+def random_model(dtype, hidden, heads, kv_heads, hd, inter, vocab, layers, seed, theta=1e6, qk_norm=True,
+                 bias=False, std=0.05):
+    rng = np.random.default_rng(seed)
+    e = lambda shape, mean=0.0, s=std: O.encode16(dtype, rng.normal(mean, s, shape))
+    A, KV = heads * hd, kv_heads * hd
+    ls = []
+    for _ in range(layers):
+        l = dict(rms_attn=e(hidden, 1.0, 0.02), rms_mlp=e(hidden, 1.0, 0.02), w_q=e((A, hidden)),
+                 w_k=e((KV, hidden)), w_v=e((KV, hidden)), w_o=e((hidden, A)), w_gate=e((inter, hidden)),
+                 w_up=e((inter, hidden)), w_down=e((hidden, inter)))
+        if qk_norm:
+            l.update(q_norm=e(hd, 1.0, 0.02), k_norm=e(hd, 1.0, 0.02))
+        if bias:
+            l.update(q_bias=e(A, 0, 0.1), k_bias=e(KV, 0, 0.1), v_bias=e(KV, 0, 0.1), o_bias=e(hidden, 0, 0.1))
+        ls.append(l)
+    args = (dtype, hidden, heads, kv_heads, hd, inter, vocab, 1e-6, theta, e((vocab, hidden), 0, 1.0), ls,
+            e(hidden, 1.0, 0.02), e((vocab, hidden)))
+    return N.ModelWeights(*args), O.Model(*args)
+
+
+def assert_streams_agree(device_tokens, oracle_tokens, margins, logit_scale):
+    """Identical greedy streams wherever the oracle's top-2 margin exceeds the tolerance."""
+    n = min(len(device_tokens), len(oracle_tokens))
+    for i in range(n):
+        if device_tokens[i] != oracle_tokens[i]:
+            assert margins[i] <= 2e-3 * logit_scale, (i, device_tokens[i], oracle_tokens[i], margins[i])
+            return i
+    return n
+
+
+GEOMETRIES = [
+    # dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias
+    (BF16, 512, 4, 1, 128, 1024, 1000, 3, 1e6, True, False),   # fast attention path, group 4 (Qwen3-like)
+    (BF16, 1024, 8, 8, 128, 1536, 777, 2, 1e4, False, True),   # MHA, biases, no qk-norm
+    (F16, 256, 4, 2, 64, 520, 300, 2, 1e4, True, False),       # generic attention path, guarded GEMV
+    (BF16, 96, 6, 2, 16, 200, 50, 2, 0, False, False),         # group 3, no RoPE, cols % 8 == 0 only
+]
+
+
+@pytest.mark.parametrize("geom", GEOMETRIES)
+def test_session_matches_oracle_logits_kv_and_stream(geom):
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
+    weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, hidden, theta, qk_norm, bias)
+    prompt = np.random.default_rng(1).integers(0, vocab, 21).astype(np.uint32)
+    steps = 24
+    ctx = O.Context(omodel, 64, staging=1)
+    otokens, margins = ctx.greedy_decode(prompt, steps)
+    s = N.DecodeSession.create(weights, 64)
+    rc, res = s.start(prompt)
+    assert rc == 0
+    # logits after prefill: compare with an oracle context that stops right after the prompt
+    ctx2 = O.Context(omodel, 64, staging=1)
+    for i, t in enumerate(prompt):
+        ctx2.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
+    ref_logits = ctx2.logits()
+    got_logits = s.logits()
+    assert rel_l2(got_logits, ref_logits) <= REL_L2
+    for layer in range(layers):
+        for token in (0, 7, len(prompt) - 1):
+            gk, gv = s.kv_row(layer, token)
+            rk, rv = ctx2.read_kv16(layer, token)
+            assert rel_l2(O.decode16(dtype, gk), O.decode16(dtype, rk)) <= 2e-3
+            assert rel_l2(O.decode16(dtype, gv), O.decode16(dtype, rv)) <= 2e-3
+    rc, res, tokens = s.advance(steps)
+    assert rc == 0 and res.observed_tokens == steps and res.graph_replays == steps - 1
+    assert res.hot_path_allocations == 0 and res.host_causality_edges == 0 and res.sync_calls == 1
+    scale = float(np.max(np.abs(ref_logits)))
+    agreed = assert_streams_agree(tokens.tolist(), otokens.tolist(), margins, scale)
+    assert agreed >= 1
+    assert res.observed_token_hash == O.fnv1a(tokens)
+    # determinism: the same prompt again gives the same stream and hash
+    rc, _ = s.start(prompt)
+    rc, res2, tokens2 = s.advance(steps)
+    assert tokens2.tolist() == tokens.tolist() and res2.observed_token_hash == res.observed_token_hash
+    assert res2.graph_captures == 0 and res2.graph_cache_hits == 1
+    s.destroy()
+
+
+def test_run_walks_prompt_with_decode_staging():
+    """session_run feeds prompt tokens through the decode-step graph (f32 residual stream,
+    no per-layer rounding), unlike start(), which uses the prompt staging."""
+    weights, omodel = random_model(BF16, 512, 4, 1, 128, 1024, 500, 2, 77)
+    prompt = np.array([5, 17, 400, 3, 250], np.uint32)
+    ctx = O.Context(omodel, 32, staging=1)
+    for i, t in enumerate(prompt):
+        ctx.forward_token(int(t), prompt_token=False, want_logits=True)
+    ref = ctx.logits()
+    s = N.DecodeSession.create(weights, 32)
+    rc, res, tokens = s.run(prompt, 1)
+    assert rc == 0 and res.graph_replays == len(prompt)
+    assert rel_l2(s.logits(), ref) <= REL_L2
+    assert tokens[0] == O.greedy_argmax(ref, skip_nonfinite=True) or \
+        np.sort(ref)[-1] - np.sort(ref)[-2] < 2e-3 * np.max(np.abs(ref))
+    s.destroy()
+
+
+def test_eager_profile_pass_leaves_state_untouched():
+    weights, omodel = random_model(BF16, 512, 4, 1, 128, 1024, 500, 2, 5)
+    s = N.DecodeSession.create(weights, 48)
+    prompt = np.arange(9, dtype=np.uint32)
+    s.start(prompt)
+    rc, res, a = s.advance(4)
+    rc, prof = s.profile_step(2)
+    assert rc == 0 and prof.status == 0 and prof.launches == 2 + 5 * 2
+    assert prof.gate_up_ns > 0 and prof.lm_head_ns > 0 and prof.position == len(prompt) + 3
+    rc, res, b = s.advance(6)
+    s.start(prompt)
+    rc, res, full = s.advance(10)
+    assert np.concatenate([a, b]).tolist() == full.tolist()   # profiling did not disturb the sequence
+    s.destroy()
+
+
+def test_synthetic_session_matches_oracle_weights():
+    """Device-generated weights (benchmark path) equal the oracle's generator bit for bit, so the
+    CPU baseline can rebuild the same model on the host."""
+    cfg = dict(dtype=BF16, hidden=512, heads=4, kv_heads=1, head_dim=128, intermediate=1024, vocab=600,
+               layers=2, rms_eps=1e-6, rope_theta=1e6)
+    seed, std = 0x4E45525641, 0.02
+    s = N.DecodeSession.create_synthetic(cfg, 64, seed=seed, weight_std=std, qk_norm=True)
+    H, A, KV, I, V, HD = 512, 512, 128, 1024, 600, 128
+    g = lambda tid, n, mean=0.0: O.synth_16(BF16, seed, tid, n, mean, std)
+    layers = []
+    for l in range(2):
+        b = 16 * (l + 1)
+        layers.append(dict(rms_attn=g(b, H, 1.0), rms_mlp=g(b + 1, H, 1.0), w_q=g(b + 2, A * H).reshape(A, H),
+                           w_k=g(b + 4, KV * H).reshape(KV, H), q_norm=g(b + 5, HD, 1.0), k_norm=g(b + 6, HD, 1.0),
+                           w_v=g(b + 7, KV * H).reshape(KV, H), w_o=g(b + 8, H * A).reshape(H, A),
+                           w_gate=g(b + 13, I * H).reshape(I, H), w_up=g(b + 14, I * H).reshape(I, H),
+                           w_down=g(b + 15, H * I).reshape(H, I)))
+    omodel = O.Model(BF16, H, 4, 1, HD, I, V, 1e-6, 1e6, g(1, V * H).reshape(V, H), layers, g(2, H, 1.0),
+                     g(3, V * H).reshape(V, H))
+    prompt = O.synth_tokens(seed, 1000, 12, V)
+    ctx = O.Context(omodel, 64, staging=1)
+    otokens, margins = ctx.greedy_decode(prompt, 8)
+    rc, res = s.start(prompt)
+    assert rc == 0
+    rc, res, tokens = s.advance(8)
+    assert rc == 0
+    ctx2 = O.Context(omodel, 64, staging=1)
+    for i, t in enumerate(prompt):
+        ctx2.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
+    assert_streams_agree(tokens.tolist(), otokens.tolist(), margins, float(np.max(np.abs(ctx2.logits()))))
+    s.destroy()
