@@ -279,9 +279,11 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
   }
 
   // ---- last workgroup of this kv head merges the splits
+  // Every thread that stored a partial releases its own stores to device scope
+  // before the workgroup's arrival is counted.
+  __threadfence();
   __syncthreads();
   if (threadIdx.x == 0) {
-    __threadfence();
     const uint32_t ticket =
         __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     is_last = ticket == S - 1 ? 1u : 0u;
