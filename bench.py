@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Benchmark of the batch-1 decode hot path on one MI355X.
+
+Workload (BASELINE.json configs[4], the one the metric is quoted on): Qwen3-8B-architecture
+decoder, random-init bf16 weights generated on the device, batch 1, a prompt of 8192 random
+token ids prefilled into the paged KV cache, then greedy decode under hipGraph replay.
+A "step" is one decoded token (one graph replay = the whole per-token weight + KV stream).
+
+Prints ONE JSON line: whole-step tok/s, plus
+  roofline     - the dominant kernel (fused gate_up GEMV): algorithmic bytes / average launch
+                 duration measured with hipEvent pairs on the session stream, vs 8 TB/s HBM;
+  cpu_baseline - the CPU oracle (scalar port of the reference's CPU path) timed on this
+                 host on a bounded sample of the same decode step, extrapolated to tok/s.
+"""
+import argparse
+import concurrent.futures
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+SEED = 0x4E45525641
+WEIGHT_STD = 0.02
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def step_bytes(cfg, ctx_tokens):
+    """Algorithmic bytes one decode step must move: every weight once + the KV read + KV write."""
+    H, A = cfg["hidden"], cfg["heads"] * cfg["head_dim"]
+    KV, I, V, L, HD = cfg["kv_heads"] * cfg["head_dim"], cfg["intermediate"], cfg["vocab"], cfg["layers"], cfg["head_dim"]
+    per_layer = ((A + 2 * KV) * H + H * A + 3 * I * H) * 2
+    norms = (L * (2 * H + 2 * HD) + H) * 2
+    weights = L * per_layer + V * H * 2 + norms + H * 2
+    kv_read = L * 2 * KV * 2 * ctx_tokens
+    kv_write = L * 2 * KV * 2
+    return weights + kv_read + kv_write, weights
+
+
+def cpu_baseline(session, cfg, position, token, layers_sampled, threads_all):
+    """Time the oracle on `layers_sampled` layers + LM head of one decode step at `position`,
+    on 1 core and on all cores, with the device's own weights (regenerated bit-identically on
+    the host) and the KV cache downloaded from the device prefill."""
+    import oracle as O
+    H, A = cfg["hidden"], cfg["heads"] * cfg["head_dim"]
+    KV, I, V, HD, dt = cfg["kv_heads"] * cfg["head_dim"], cfg["intermediate"], cfg["vocab"], cfg["head_dim"], cfg["dtype"]
+
+    def gen(tid, n, mean=0.0):
+        chunk = 1 << 24
+        out = np.empty(n, np.uint16)
+
+        def work(start):
+            m = min(chunk, n - start)
+            out[start:start + m] = O.synth_16(dt, SEED, tid, m, mean, WEIGHT_STD, offset=start)
+        with concurrent.futures.ThreadPoolExecutor(max_workers=threads_all) as pool:
+            list(pool.map(work, range(0, n, chunk)))
+        return out
+
+    t0 = time.time()
+    layers = []
+    for l in range(layers_sampled):
+        b = 16 * (l + 1)
+        layers.append(dict(rms_attn=gen(b, H, 1.0), rms_mlp=gen(b + 1, H, 1.0), w_q=gen(b + 2, A * H).reshape(A, H),
+                           w_k=gen(b + 4, KV * H).reshape(KV, H), q_norm=gen(b + 5, HD, 1.0), k_norm=gen(b + 6, HD, 1.0),
+                           w_v=gen(b + 7, KV * H).reshape(KV, H), w_o=gen(b + 8, H * A).reshape(H, A),
+                           w_gate=gen(b + 13, I * H).reshape(I, H), w_up=gen(b + 14, I * H).reshape(I, H),
+                           w_down=gen(b + 15, H * I).reshape(H, I)))
+    emb = np.zeros((token + 1, H), np.uint16)
+    emb[token] = O.synth_16(dt, SEED, 1, H, 0.0, WEIGHT_STD, offset=token * H)
+    lm_head = gen(3, V * H).reshape(V, H)
+    final_norm = gen(2, H, 1.0)
+    model = O.Model(dt, H, cfg["heads"], cfg["kv_heads"], HD, I, V, cfg["rms_eps"], cfg["rope_theta"], emb, layers,
+                    final_norm, lm_head)
+    kv = [session.kv_range(l, 0, position) for l in range(layers_sampled)]
+    log("[cpu] host weights + KV ready in %.1f s" % (time.time() - t0))
+    result = {}
+    logits = None
+    for threads in (1, threads_all):
+        os.environ["OMP_NUM_THREADS"] = str(threads)
+        ctx = O.Context(model, position + 2, staging=1, threads=threads)
+        for l, (k, v) in enumerate(kv):
+            ctx.load_kv16(l, k, v)
+        ctx.set_len(position)
+        t0 = time.time()
+        hidden = ctx.forward_token(token, prompt_token=False, want_logits=False)
+        t_layers = time.time() - t0
+        t0 = time.time()
+        normed = O.decode16(dt, O.encode16(dt, O.rms_norm(dt, hidden, final_norm, cfg["rms_eps"])))
+        logits = O.gemv(dt, lm_head, normed, threads=threads)
+        t_head = time.time() - t0
+        per_token = t_layers * cfg["layers"] / layers_sampled + t_head
+        result[threads] = dict(tok_s=1.0 / per_token, layers_s=t_layers, head_s=t_head)
+        log("[cpu] %d thread(s): %d layers %.2f s, lm_head %.2f s -> %.4f tok/s (extrapolated)"
+            % (threads, layers_sampled, t_layers, t_head, 1.0 / per_token))
+        ctx.close()
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=8192, help="prompt tokens prefilled before decoding")
+    ap.add_argument("--layers", type=int, default=36, help="(debug) fewer layers = NOT the named workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-layers", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path is a single-device decode loop and no multi-GPU "
+              "figure exists for it (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import nerva_amd as N
+    rc, smoke = N.Device.smoke()
+    if rc != 0:
+        log("no usable GPU (hip_error=%d): the HIP path cannot run, and there is no CPU fallback" % smoke.hip_error)
+        sys.exit(1)
+    cfg = dict(N.Qwen3_8B)
+    cfg["layers"] = args.layers
+    max_ctx = args.prompt + args.warmup + args.steps + 16
+    t0 = time.time()
+    session = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=WEIGHT_STD, qk_norm=True)
+    log("[bench] %s: session created in %.1f s, arena %.2f GB (weights %.2f GB, KV %.2f GB)" % (
+        smoke.gpu_name.decode(), time.time() - t0, session.create_result.device_arena_bytes / 1e9,
+        session.create_result.resident_weight_bytes / 1e9, session.create_result.resident_kv_bytes / 1e9))
+    prompt = np.random.default_rng(SEED).integers(0, cfg["vocab"], args.prompt).astype(np.uint32)
+    t0 = time.time()
+    rc, res = session.start(prompt)
+    assert rc == 0, "start failed: hip_error=%d" % res.hip_error
+    rc, res, first = session.advance(1)      # token 0 was sampled by the prefill; this only syncs
+    assert rc == 0
+    log("[bench] prefill of %d tokens: %.1f s" % (args.prompt, time.time() - t0))
+    if args.warmup:
+        rc, res, _ = session.advance(args.warmup)
+        assert rc == 0
+    allocs = N.Device.allocation_count()
+    t0 = time.perf_counter()
+    rc, res, tokens = session.advance(args.steps)
+    elapsed = time.perf_counter() - t0
+    assert rc == 0 and res.observed_tokens == args.steps and res.graph_replays == args.steps
+    assert res.hot_path_allocations == 0 and N.Device.allocation_count() == allocs
+    tok_s = args.steps / elapsed
+    ctx_mid = args.prompt + 1 + args.warmup + args.steps // 2
+    bytes_step, bytes_weights = step_bytes(cfg, ctx_mid)
+    log("[bench] %d steps in %.3f s -> %.1f tok/s, %.3f ms/step, device %.3f ms/step, graph nodes %d" % (
+        args.steps, elapsed, tok_s, 1e3 * elapsed / args.steps, res.device_elapsed_ns / 1e6 / args.steps, res.graph_nodes))
+
+    # dominant kernel: fused gate_up GEMV, timed live with hipEvent pairs around each eager launch
+    rc, prof = session.profile_step(3)
+    assert rc == 0
+    per_kind = {k: (getattr(prof, k + "_ns"), getattr(prof, k + "_bytes")) for k in
+                ("qkv", "attention", "o", "gate_up", "down", "lm_head")}
+    for k, (ns, b) in per_kind.items():
+        log("[profile] %-9s %8.2f us  %7.1f GB/s  (%.1f%% of HBM peak)" % (k, ns / 1e3, b / max(ns, 1), 100 * b / max(ns, 1) / HBM_PEAK_GBS))
+    gu_ns, gu_bytes = per_kind["gate_up"]
+    roofline = dict(bound="hbm", kernel="gemv_kernel<bf16, rmsnorm prologue, swiglu epilogue> (gate_up 24576x4096)",
+                    achieved=round(gu_bytes / gu_ns, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(gu_bytes / gu_ns / HBM_PEAK_GBS, 4), traffic=None,
+                    bytes_per_launch=gu_bytes, avg_launch_us=round(gu_ns / 1e3, 2),
+                    whole_step_bytes=bytes_step, whole_step_frac=round(bytes_step * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+                    per_kernel_frac={k: round(b / max(ns, 1) / HBM_PEAK_GBS, 4) for k, (ns, b) in per_kind.items()})
+
+    cpu = None
+    if not args.no_cpu:
+        try:
+            threads_all = min(os.cpu_count() or 1, 16)
+            position = args.prompt + args.warmup + args.steps      # tokens now in the KV cache
+            layers_sampled = min(args.cpu_layers, cfg["layers"])
+            r = cpu_baseline(session, cfg, position, int(tokens[-1]), layers_sampled, threads_all)
+            cpu = dict(value=round(r[1]["tok_s"], 5), unit="tok/s", cores=1, kind="port",
+                       sample="1 decode token at ctx %d: %d of %d layers + lm_head timed on the oracle, extrapolated to %d layers"
+                              % (position, layers_sampled, cfg["layers"], cfg["layers"]),
+                       all_cores_value=round(r[threads_all]["tok_s"], 5), all_cores=threads_all)
+        except Exception as e:  # the CPU leg never hides the GPU result
+            log("[cpu] baseline failed: %r" % (e,))
+    session.destroy()
+
+    line = dict(metric="decode tok/s Qwen3-8B bs1", value=round(tok_s, 2), unit="tok/s", n_gpus=1,
+                steps=args.steps, warmup=args.warmup, ms_per_step=round(1e3 * elapsed / args.steps, 4),
+                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+                config=dict(workload="configs[4]: full Qwen3-8B-architecture decode step, %d layers, hidden 4096, "
+                                     "32q/8kv x128, MLP 12288, vocab 151936, random-init bf16 N(0,0.02), batch 1, "
+                                     "prompt %d prefilled, %d greedy tokens under hipGraph replay"
+                                     % (cfg["layers"], args.prompt, args.steps),
+                            prompt_tokens=args.prompt, context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
+                            hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
+                            gpu=smoke.gpu_name.decode()),
+                roofline=roofline, cpu_baseline=cpu)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

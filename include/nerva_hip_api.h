@@ -542,6 +542,11 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *session, float *host_logits);
 int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *session, uint32_t layer, uint32_t token,
                               uint16_t *host_k, uint16_t *host_v);
+/* Same for tokens [first_token, first_token + token_count): host_k / host_v receive
+ * [token_count][kv_heads*head_dim] rows (the layout a contiguous CPU cache uses). */
+int nerva_hip_session_read_kv_range(NervaHipHfDecodeSequenceSession *session, uint32_t layer,
+                                    uint32_t first_token, uint32_t token_count, uint16_t *host_k,
+                                    uint16_t *host_v);
 
 #ifdef __cplusplus
 }

@@ -28,35 +28,39 @@ __global__ __launch_bounds__(kBlock) void argmax_kernel(const float *logits, uin
     red_h[wave] = b.has;
   }
   __syncthreads();
-  Best block_best{red[0], red_i[0], red_h[0]};
-  for (int w = 1; w < kWavesPerBlock; ++w) {
-    Best o{red[w], red_i[w], red_h[w]};
-    if (better(o, block_best)) block_best = o;
+  if (threadIdx.x == 0) {
+    Best block_best{red[0], red_i[0], red_h[0]};
+    for (int w = 1; w < kWavesPerBlock; ++w) {
+      Best o{red[w], red_i[w], red_h[w]};
+      if (better(o, block_best)) block_best = o;
+    }
+    s.part_value[blockIdx.x] = block_best.value;
+    s.part_index[blockIdx.x] = block_best.index;
+    s.part_has[blockIdx.x] = block_best.has;
   }
-  __syncthreads();
-  sample_finish(s, block_best, red, red_i, red_h);
 }
 
 }  // namespace
 
-uint64_t sample_workspace_bytes() { return (3ull * kSampleMaxBlocks + 64) * sizeof(uint32_t); }
+uint64_t sample_workspace_bytes() { return 3ull * kSampleMaxBlocks * sizeof(uint32_t); }
 
 void sample_bind_workspace(SampleParams &s, void *workspace) {
   uint32_t *base = static_cast<uint32_t *>(workspace);
-  s.counter = base;  // first 64 words: counter + padding
-  s.part_value = reinterpret_cast<float *>(base + 64);
-  s.part_index = base + 64 + kSampleMaxBlocks;
-  s.part_has = base + 64 + 2 * kSampleMaxBlocks;
+  s.part_value = reinterpret_cast<float *>(base);
+  s.part_index = base + kSampleMaxBlocks;
+  s.part_has = base + 2 * kSampleMaxBlocks;
 }
 
 hipError_t launch_argmax(const float *logits, uint32_t count, const SampleParams &s,
                          hipStream_t stream) {
-  if (logits == nullptr || count == 0 || s.counter == nullptr) return hipErrorInvalidValue;
+  if (logits == nullptr || count == 0 || s.part_value == nullptr) return hipErrorInvalidValue;
   uint32_t blocks = (count + kBlock * 8 - 1) / (kBlock * 8);
   if (blocks > 512) blocks = 512;
   if (blocks == 0) blocks = 1;
   hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(kBlock), 0, stream, logits, count, s);
-  return hipGetLastError();
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return launch_sample_finish(s, blocks, nullptr, 0, stream);
 }
 
 }  // namespace nv

@@ -25,6 +25,7 @@ struct AttnParams {
   uint16_t *k_cache, *v_cache;
   const uint32_t *table;       // [block_count]
   const float *rope_freq;      // [hd/2]: powf(theta, 2i/hd), or null = no RoPE
+  const float *rope_cs;        // optional [hd]: cos | sin of pos / rope_freq[i], precomputed for this step
   float *part_acc;             // [heads][splits][hd]  un-normalised partial outputs
   float *part_m, *part_l;      // [heads][splits]
   uint32_t *counters;          // [kv_heads] arrival counters, zero between launches

@@ -8,7 +8,8 @@
 // exact_blockwise_attention_into (attention/exact/run.rs:13-127).
 //
 // gfx950 mapping of the fast path (head_dim 128, G = heads/kv_heads in {1,2,4,8}):
-//   grid (kv_heads, splits); a wave owns whole 16-token KV blocks. One block tile
+//   grid (kv_heads, splits), 8 waves per workgroup; a wave owns whole 16-token KV
+//   blocks of its workgroup's token range. One block tile
 //   of one kv head is 4 KiB contiguous, fetched by four 1 KiB load instructions
 //   in exactly the register layout the math wants: load i, lane l holds the 8
 //   dims (l%16)*8.. of token 4i + l/16. So a 16-lane DPP row reduces one q.k, the
@@ -25,6 +26,7 @@ namespace nv {
 namespace {
 
 constexpr int kHD = 128;
+constexpr int kAttnWaves = 8;   // waves per workgroup of the fast path (group 8 uses half)
 
 // Sum over the 16 lanes of a DPP row; every lane of the row gets the total.
 __device__ __forceinline__ float row16_sum(float v) {
@@ -46,11 +48,13 @@ __device__ __forceinline__ void unpack8(const uint4 &v, float (&f)[8]) {
 // One wave prepares one 128-wide head: lane l owns the RoPE pair (l, l+64).
 // out[] receives f32; when out16 != null the value is rounded first and the 16-bit
 // copy is stored too (K/V that go to the cache).
+// rope_cs (optional): cos at [i], sin at [64 + i] of this step's angles, computed once
+// per step; without it the angle pos / rope_freq[i] is evaluated here.
 template <uint32_t DT>
 __device__ __forceinline__ void prep_head128(const float *src, const uint16_t *bias,
                                              const uint16_t *gamma, const float *rope_freq,
-                                             uint32_t pos, float eps, int lane, float *out,
-                                             uint16_t *out16) {
+                                             const float *rope_cs, uint32_t pos, float eps, int lane,
+                                             float *out, uint16_t *out16) {
   float x0 = src[lane], x1 = src[lane + 64];
   if (bias != nullptr) {
     x0 += dec16<DT>(bias[lane]);
@@ -63,9 +67,13 @@ __device__ __forceinline__ void prep_head128(const float *src, const uint16_t *b
     x1 *= scale * dec16<DT>(gamma[lane + 64]);
   }
   if (rope_freq != nullptr) {
-    const float angle = static_cast<float>(pos) / rope_freq[lane];
     float s, c;
-    sincosf(angle, &s, &c);
+    if (rope_cs != nullptr) {
+      c = rope_cs[lane];
+      s = rope_cs[64 + lane];
+    } else {
+      sincosf(static_cast<float>(pos) / rope_freq[lane], &s, &c);
+    }
     const float r0 = x0 * c - x1 * s;
     const float r1 = x1 * c + x0 * s;
     x0 = r0;
@@ -83,14 +91,19 @@ __device__ __forceinline__ void prep_head128(const float *src, const uint16_t *b
   }
 }
 
-template <uint32_t DT, int G>
-__global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
+// W waves per workgroup. A workgroup owns one kv head and one contiguous range of
+// 16-token tiles; wave w takes tiles b0+w, b0+w+W, ... Many waves per workgroup
+// keep the number of split partials (and so the merge) small while the whole KV
+// range is in flight at once: the kernel lives only a few memory latencies.
+template <uint32_t DT, int G, int W>
+__global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
+  constexpr int kThreads = W * kWave;
   __shared__ __align__(16) float q_s[G][kHD];
   __shared__ __align__(16) uint16_t knew[kHD];
   __shared__ __align__(16) uint16_t vnew[kHD];
-  __shared__ float wm[kWavesPerBlock][G];
-  __shared__ float wl[kWavesPerBlock][G];
-  __shared__ __align__(16) float wacc[kWavesPerBlock][G][kHD];
+  __shared__ float wm[W][G];
+  __shared__ float wl[W][G];
+  __shared__ __align__(16) float wacc[W][G][kHD];
   __shared__ uint32_t is_last;
 
   const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
@@ -101,26 +114,42 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
   const uint32_t kvh = blockIdx.x, split = blockIdx.y, S = gridDim.y;
   const uint32_t n_keys = pos + 1;
   const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
-  const uint32_t bps = (nblk + S - 1) / S;
+  // at least W tiles per active split so that every wave of a workgroup has work
+  uint32_t bps = (nblk + S - 1) / S;
+  bps = ((bps + W - 1) / W) * W;
+  const uint32_t active = (nblk + bps - 1) / bps;
+  if (split >= active) return;  // idle splits neither store a partial nor take a ticket
   const uint32_t b0 = split * bps;
   const uint32_t b1 = min(nblk, b0 + bps);
   const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
   const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
 
+  // ---- first tile of every wave: issue its loads before anything else
+  uint4 kreg[4], vreg[4];
+  uint32_t b = b0 + wave;
+  if (b < b1) {
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kreg[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
+      vreg[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
+    }
+  }
+
   // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
-  for (int g = wave; g < G; g += kWavesPerBlock) {
+  for (int g = wave; g < G; g += W) {
     const uint32_t h = kvh * G + g;
     prep_head128<DT>(p.qkv + h * kHD, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq,
-                     pos, p.eps, lane, q_s[g], nullptr);
+                     p.rope_cs, pos, p.eps, lane, q_s[g], nullptr);
   }
   if (owns_new) {
-    if (wave == (G % kWavesPerBlock)) {
+    if (wave == (G % W)) {
       prep_head128<DT>(p.qkv + A + kvh * kHD, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm,
-                       p.rope_freq, pos, p.eps, lane, nullptr, knew);
-    } else if (wave == ((G + 1) % kWavesPerBlock)) {
+                       p.rope_freq, p.rope_cs, pos, p.eps, lane, nullptr, knew);
+    } else if (wave == ((G + 1) % W)) {
       prep_head128<DT>(p.qkv + A + KV + kvh * kHD, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr,
-                       nullptr, pos, p.eps, lane, nullptr, vnew);
+                       nullptr, nullptr, pos, p.eps, lane, nullptr, vnew);
     }
   }
   __syncthreads();
@@ -133,16 +162,7 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
     *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
   }
 
-  // ---- per-lane query slice: dims part*8..part*8+7 of every head of the group
   const int part = lane & 15, trow = lane >> 4;
-  float qr[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float4 a = *reinterpret_cast<const float4 *>(&q_s[g][part * 8]);
-    const float4 b = *reinterpret_cast<const float4 *>(&q_s[g][part * 8 + 4]);
-    qr[g][0] = a.x; qr[g][1] = a.y; qr[g][2] = a.z; qr[g][3] = a.w;
-    qr[g][4] = b.x; qr[g][5] = b.y; qr[g][6] = b.z; qr[g][7] = b.w;
-  }
   const float scale = 1.0f / sqrtf(static_cast<float>(kHD));
 
   float m[G], l[G], acc[G][8];
@@ -154,20 +174,10 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
     for (int d = 0; d < 8; ++d) acc[g][d] = 0.0f;
   }
 
-  uint4 kreg[4], vreg[4];
-  uint32_t b = b0 + wave;
-  if (b < b1) {
-    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      kreg[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
-      vreg[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
-    }
-  }
-  for (; b < b1; b += kWavesPerBlock) {
+  for (; b < b1; b += W) {
     // issue the next tile's loads before touching the current one
     uint4 knext[4], vnext[4];
-    const uint32_t bn = b + kWavesPerBlock;
+    const uint32_t bn = b + W;
     if (bn < b1) {
       const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[bn], kvh);
 #pragma unroll
@@ -186,6 +196,7 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
         }
       }
     }
+    // scores: s[g][i] for token 4i + trow, all G heads share each unpacked K register
     float s[G][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -194,14 +205,20 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
       const bool valid = b * kKvBlockTokens + i * 4 + trow < n_keys;
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float d = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qr[g][e], kf[e], d);
+        const float4 qa = *reinterpret_cast<const float4 *>(&q_s[g][part * 8]);
+        const float4 qb = *reinterpret_cast<const float4 *>(&q_s[g][part * 8 + 4]);
+        float d = qa.x * kf[0];
+        d = fmaf(qa.y, kf[1], d);
+        d = fmaf(qa.z, kf[2], d);
+        d = fmaf(qa.w, kf[3], d);
+        d = fmaf(qb.x, kf[4], d);
+        d = fmaf(qb.y, kf[5], d);
+        d = fmaf(qb.z, kf[6], d);
+        d = fmaf(qb.w, kf[7], d);
         d = row16_sum(d) * scale;
         s[g][i] = valid ? d : -INFINITY;
       }
     }
-    float pr[G][4];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float mb = fmaxf(fmaxf(s[g][0], s[g][1]), fmaxf(s[g][2], s[g][3]));
@@ -212,8 +229,8 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
       float psum = 0.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        pr[g][i] = expf(s[g][i] - m_new);
-        psum += pr[g][i];
+        s[g][i] = expf(s[g][i] - m_new);     // scores become probabilities in place
+        psum += s[g][i];
       }
       l[g] = l[g] * alpha + psum;
       m[g] = m_new;
@@ -227,7 +244,7 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
 #pragma unroll
       for (int g = 0; g < G; ++g)
 #pragma unroll
-        for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(pr[g][i], vf[d], acc[g][d]);
+        for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(s[g][i], vf[d], acc[g][d]);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -236,7 +253,7 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
     }
   }
 
-  // ---- merge the four token rows of the wave, then the four waves
+  // ---- merge the four token rows of the wave, then the W waves
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     l[g] += __shfl_xor(l[g], 16, kWave);
@@ -256,60 +273,100 @@ __global__ __launch_bounds__(kBlock) void attn_fast_kernel(AttnParams p) {
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < G * kHD; e += kBlock) {
-    const int g = e / kHD, d = e % kHD;
+  // ---- merge of the W waves: W*G scale factors once, then every thread owns (g, d) pairs
+  __shared__ float wf[W][G];    // exp(m_w - M_g), 0 for idle waves
+  __shared__ float bM[G], bL[G];
+  __shared__ __align__(16) float bacc[G][kHD];
+  if (threadIdx.x < W * G) {
+    const int w = threadIdx.x / G, g = threadIdx.x % G;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) M = fmaxf(M, wm[w][g]);
+    for (int w2 = 0; w2 < W; ++w2) M = fmaxf(M, wm[w2][g]);
+    wf[w][g] = wm[w][g] > -INFINITY ? expf(wm[w][g] - M) : 0.0f;
+    if (w == 0) bM[g] = M;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < G * kHD; e += kThreads) {
+    const int g = e / kHD, d = e % kHD;
     float L = 0.0f, o = 0.0f;
-    if (M > -INFINITY) {
 #pragma unroll
-      for (int w = 0; w < kWavesPerBlock; ++w) {
-        const float f = expf(wm[w][g] - M);  // exp(-inf) = 0 for idle waves
-        L += wl[w][g] * f;
-        o += wacc[w][g][d] * f;
-      }
+    for (int w = 0; w < W; ++w) {
+      L = fmaf(wl[w][g], wf[w][g], L);
+      o = fmaf(wacc[w][g][d], wf[w][g], o);
     }
     const uint32_t h = kvh * G + g;
-    p.part_acc[(static_cast<uint64_t>(h) * S + split) * kHD + d] = o;
-    if (d == 0) {
-      p.part_m[h * S + split] = M;
-      p.part_l[h * S + split] = L;
+    if (active == 1) {
+      // a single split holds every key: this is the final result, nothing to exchange
+      if (L > 0.0f && isfinite(L)) o /= L;
+      if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
+      p.out16[h * kHD + d] = enc16<DT>(o);
+    } else {
+      bacc[g][d] = o;
+      if (d == 0) bL[g] = L;
     }
   }
-
-  // ---- last workgroup of this kv head merges the splits
-  // Every thread that stored a partial releases its own stores to device scope
-  // before the workgroup's arrival is counted.
-  __threadfence();
+  if (active == 1) return;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t ticket =
-        __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = ticket == S - 1 ? 1u : 0u;
+  // The workgroup's partial leaves through ONE wave, which then releases it to device
+  // scope once and takes the arrival ticket: one fence per workgroup.
+  if (wave == 0) {
+    for (int e = lane; e < G * kHD; e += kWave) {
+      const int g = e / kHD, d = e % kHD;
+      const uint32_t h = kvh * G + g;
+      p.part_acc[(static_cast<uint64_t>(h) * S + split) * kHD + d] = bacc[g][d];
+      if (d == 0) {
+        p.part_m[h * S + split] = bM[g];
+        p.part_l[h * S + split] = bL[g];
+      }
+    }
+    __threadfence();
+    if (lane == 0) {
+      const uint32_t ticket =
+          __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = ticket == active - 1 ? 1u : 0u;
+    }
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
-  for (int e = threadIdx.x; e < G * kHD; e += kBlock) {
+  __threadfence();  // acquire: the other workgroups' partials
+  // ---- the last workgroup of this kv head merges the splits: factors once, then (g, d) pairs
+  __shared__ float sf[kAttnMaxSplits][G];   // exp(m_s - M_g) / L_g
+  __shared__ float sm_[kAttnMaxSplits][G], sl_[kAttnMaxSplits][G];
+  for (uint32_t e = threadIdx.x; e < active * G; e += kThreads) {
+    const uint32_t s2 = e / G, g = e % G;
+    const uint32_t h = kvh * G + g;
+    sm_[s2][g] = p.part_m[h * S + s2];
+    sl_[s2][g] = p.part_l[h * S + s2];
+  }
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < active * G; e += kThreads) {
+    const uint32_t s2 = e / G, g = e % G;
+    float M = -INFINITY;
+    for (uint32_t t = 0; t < active; ++t) M = fmaxf(M, sm_[t][g]);
+    float L = 0.0f;
+    for (uint32_t t = 0; t < active; ++t) L = fmaf(sl_[t][g], expf(sm_[t][g] - M), L);
+    const float f = expf(sm_[s2][g] - M);
+    sf[s2][g] = (L > 0.0f && isfinite(L)) ? f / L : f;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < G * kHD; e += kThreads) {
     const int g = e / kHD, d = e % kHD;
     const uint32_t h = kvh * G + g;
-    float M = -INFINITY;
-    for (uint32_t s2 = 0; s2 < S; ++s2) M = fmaxf(M, p.part_m[h * S + s2]);
-    float L = 0.0f, o = 0.0f;
-    for (uint32_t s2 = 0; s2 < S; ++s2) {
-      const float pm = p.part_m[h * S + s2];
-      if (pm > -INFINITY) {
-        const float f = expf(pm - M);
-        L += p.part_l[h * S + s2] * f;
-        o += p.part_acc[(static_cast<uint64_t>(h) * S + s2) * kHD + d] * f;
-      }
+    const float *src = p.part_acc + static_cast<uint64_t>(h) * S * kHD + d;
+    float o = 0.0f;
+    uint32_t s2 = 0;
+    for (; s2 + 4 <= active; s2 += 4) {
+      const float a0 = src[(s2 + 0) * kHD], a1 = src[(s2 + 1) * kHD], a2 = src[(s2 + 2) * kHD], a3 = src[(s2 + 3) * kHD];
+      o = fmaf(a0, sf[s2 + 0][g], o);
+      o = fmaf(a1, sf[s2 + 1][g], o);
+      o = fmaf(a2, sf[s2 + 2][g], o);
+      o = fmaf(a3, sf[s2 + 3][g], o);
     }
-    if (L > 0.0f && isfinite(L)) o /= L;
+    for (; s2 < active; ++s2) o = fmaf(src[s2 * kHD], sf[s2][g], o);
     if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
     p.out16[h * kHD + d] = enc16<DT>(o);
   }
-  if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Any head_dim (even when RoPE is on) / any group size: one workgroup per query
@@ -462,10 +519,10 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
   if (fast) {
     const dim3 grid(p.kv_heads, p.splits);
     switch (group) {
-      case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1>), grid, dim3(kBlock), 0, stream, p); break;
-      case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2>), grid, dim3(kBlock), 0, stream, p); break;
-      case 4: hipLaunchKernelGGL((attn_fast_kernel<DT, 4>), grid, dim3(kBlock), 0, stream, p); break;
-      default: hipLaunchKernelGGL((attn_fast_kernel<DT, 8>), grid, dim3(kBlock), 0, stream, p); break;
+      case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+      case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+      case 4: hipLaunchKernelGGL((attn_fast_kernel<DT, 4, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+      default: hipLaunchKernelGGL((attn_fast_kernel<DT, 8, kAttnWaves / 2>), grid, dim3(kAttnWaves / 2 * kWave), 0, stream, p); break;
     }
   } else {
     if (p.head_dim > 512) return hipErrorInvalidValue;

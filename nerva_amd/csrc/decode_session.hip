@@ -4,7 +4,7 @@
 // (native/cuda/hf_decode_sequence/session_api_lifecycle.inc.cu:1-1311,
 // session_decode_prefill.inc.cu:74-372, session_graph_result.inc.cu:87-209).
 //
-// One decode step is 2 + 5*layers launches, with no host round trip:
+// One decode step is 3 + 5*layers launches, with no host round trip:
 //   embed               x = f32(emb[token]); token = prompt[pos] or slots[pos-1].token
 //   per layer
 //     qkv   GEMV  [rmsnorm(x, g_attn) prologue]                  -> qkv f32
@@ -12,7 +12,8 @@
 //     o     GEMV  [+ o_bias + x epilogue]                         -> r f32
 //     gate_up GEMV [rmsnorm(r, g_mlp) prologue, silu(g)*u epilogue] -> ff 16-bit
 //     down  GEMV  [+ r epilogue]                                  -> x f32
-//   lm_head GEMV [rmsnorm(x, g_final) prologue, argmax epilogue]  -> slot[pos], cursor = pos+1
+//   lm_head GEMV [rmsnorm(x, g_final) prologue, per-workgroup argmax epilogue]
+//   sample finish (one workgroup)                                  -> slot[pos], cursor = pos+1
 // Every kernel reads the position from device memory, so one captured graph
 // serves every position and every prompt length.
 #include <math.h>
@@ -84,7 +85,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint32_t block_count = 0;
   uint32_t *table = nullptr, *prompt = nullptr, *state = nullptr;  // state[0] cursor, state[1] prompt count
   Slot *slots = nullptr;
-  float *x = nullptr, *r = nullptr, *qkv = nullptr, *logits = nullptr, *rope_freq = nullptr;
+  float *x = nullptr, *r = nullptr, *qkv = nullptr, *logits = nullptr, *rope_freq = nullptr, *rope_cs = nullptr;
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
   void *attn_ws = nullptr, *sample_ws = nullptr;
   uint32_t attn_splits = 1;
@@ -114,9 +115,19 @@ template <uint32_t DT>
 __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, const uint32_t *prompt,
                                                        const Slot *slots, const uint32_t *state,
                                                        uint32_t max_steps, uint32_t hidden,
-                                                       uint32_t vocab, float *x) {
+                                                       uint32_t vocab, float *x, const float *rope_freq,
+                                                       float *rope_cs, uint32_t half_dim) {
   const uint32_t pos = state[0];
   if (pos >= max_steps) return;
+  // this step's RoPE angles, once: cos at [i], sin at [half_dim + i] (f32 angle = pos / theta^(2i/d))
+  if (rope_freq != nullptr && blockIdx.x == 0) {
+    for (uint32_t i = threadIdx.x; i < half_dim; i += kBlock) {
+      float sn, cs;
+      sincosf(static_cast<float>(pos) / rope_freq[i], &sn, &cs);
+      rope_cs[i] = cs;
+      rope_cs[half_dim + i] = sn;
+    }
+  }
   uint32_t token = pos < state[1] ? prompt[pos] : slots[pos - 1].token;
   if (token >= vocab) token = 0;  // prompts are validated on the host; sampled ids are < vocab
   const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
@@ -199,14 +210,17 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
 
   {
     const uint32_t blocks = std::min<uint32_t>((s->hidden + kBlock - 1) / kBlock, 64u);
+    const float *rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
     if (prof) err = prof->before(kLEmbed);
     if (err != hipSuccess) return err;
     if (s->dtype == kBF16)
       hipLaunchKernelGGL(embed_kernel<kBF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
-                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x);
+                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
+                         s->head_dim / 2);
     else
       hipLaunchKernelGGL(embed_kernel<kF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
-                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x);
+                         s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
+                         s->head_dim / 2);
     err = hipGetLastError();
     if (prof && err == hipSuccess) err = prof->after();
     if (err != hipSuccess) return err;
@@ -242,6 +256,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
       p.v_cache = s->vc;
       p.table = s->table;
       p.rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
+      p.rope_cs = s->theta > 0.0f ? s->rope_cs : nullptr;
       p.out_f32 = nullptr;
       p.out16 = s->attn16;
       p.layer = l;
@@ -316,6 +331,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
   p.sample.slots = s->slots;
   p.sample.cursor_rw = s->state;
   NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st));
+  // one small workgroup reduces the per-workgroup candidates, writes slot[pos], bumps the cursor
+  NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows), s->state,
+                                          s->max_ctx, st));
 #undef NV_STEP
   return hipSuccess;
 }
@@ -562,6 +580,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_attn16 = c.take(A * 2);
   const uint64_t off_ff16 = c.take(I * 2);
   const uint64_t off_rope = c.take(HD * 4);
+  const uint64_t off_rope_cs = c.take(HD * 4);
   const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
   s->arena_bytes = c.offset;
@@ -606,6 +625,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->attn16 = dev16(off_attn16);
   s->ff16 = dev16(off_ff16);
   s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
+  s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
   s->sample_ws = s->arena + off_sample_ws;
   s->layer.resize(L);
@@ -805,7 +825,7 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
     }
   }
   if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
-  if (err == hipSuccess) out->kernel_launches += 2 + 5ull * s->layers;
+  if (err == hipSuccess) out->kernel_launches += 3 + 5ull * s->layers;
   if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
@@ -1116,6 +1136,33 @@ int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *s, uint32_t layer
                          static_cast<uint64_t>(row) * s->head_dim;
     if (hipMemcpy(host_k + h * s->head_dim, s->kc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
     if (hipMemcpy(host_v + h * s->head_dim, s->vc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  }
+  return 0;
+}
+
+int nerva_hip_session_read_kv_range(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t first_token,
+                                    uint32_t token_count, uint16_t *host_k, uint16_t *host_v) {
+  if (s == nullptr || host_k == nullptr || host_v == nullptr || layer >= s->layers ||
+      static_cast<uint64_t>(first_token) + token_count > s->max_ctx)
+    return -1;
+  if (token_count == 0) return 0;
+  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
+  const uint32_t hd = s->head_dim, kvh = s->kv_heads;
+  const uint64_t KV = static_cast<uint64_t>(kvh) * hd;
+  const uint32_t b0 = first_token / kKvBlockTokens, b1 = (first_token + token_count - 1) / kKvBlockTokens;
+  // one layer's blocks are contiguous (identity table): copy them whole, then reorder on the host
+  const uint64_t per_block = KV * kKvBlockTokens;
+  std::vector<uint16_t> kimg((b1 - b0 + 1) * per_block), vimg((b1 - b0 + 1) * per_block);
+  const uint64_t off = kv_tile_offset(s->block_count, kvh, hd, layer, b0, 0);
+  if (hipMemcpy(kimg.data(), s->kc + off, kimg.size() * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  if (hipMemcpy(vimg.data(), s->vc + off, vimg.size() * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  for (uint32_t t = 0; t < token_count; ++t) {
+    const uint32_t tok = first_token + t, blk = tok / kKvBlockTokens - b0, row = tok % kKvBlockTokens;
+    for (uint32_t h = 0; h < kvh; ++h) {
+      const uint64_t src = (static_cast<uint64_t>(blk) * kvh + h) * kKvBlockTokens * hd + static_cast<uint64_t>(row) * hd;
+      memcpy(host_k + t * KV + h * hd, kimg.data() + src, hd * 2);
+      memcpy(host_v + t * KV + h * hd, vimg.data() + src, hd * 2);
+    }
   }
   return 0;
 }

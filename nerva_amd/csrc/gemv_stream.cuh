@@ -8,9 +8,15 @@
 //   * one wave owns NR rows at a time and walks the full K extent with
 //     64 lanes x 16 B = 1 KiB per load instruction; U x NR loads are issued
 //     back to back before the first FMA (U*NR KiB in flight per wave);
+//   * the first U chunks of a wave's rows are requested BEFORE the prologue
+//     touches x: the weight stream does not depend on x, so the HBM latency of
+//     the first loads overlaps the norm / LDS staging instead of following it;
 //   * x lives in LDS as packed 16-bit values (<= 24 KiB at K = 12288), written
 //     once per block by the prologue, read with ds_read_b128;
-//   * partial sums are reduced with wave shuffles; lane 0 runs the epilogue.
+//   * partial sums are reduced with wave shuffles; lane 0 runs the epilogue;
+//   * the grid is capped at a few workgroups per CU and waves loop over units
+//     with the next unit's head already requested, so the per-workgroup prologue
+//     (x staging, RMSNorm) is paid a few hundred times per launch, not per 4 rows.
 //
 // Reference contracts: mat_vec_encoded_row_major (precision/block/ops.rs:75-91),
 // rms_norm_to_encoded (device_ops.cuh:317-332), mlp-norm/ff/finish kernels
@@ -25,11 +31,14 @@ namespace nv {
 enum : int { kProX16 = 0, kProRmsNorm = 1 };
 enum : int { kEpiF32 = 0, kEpiResidual = 1, kEpiSwiglu = 2, kEpiOut16 = 3, kEpiArgmax = 4 };
 
+// Device sampler state. The LM-head GEMV (or the stand-alone argmax kernel) stores
+// one candidate per workgroup; sample_finish_kernel (one workgroup) reduces them
+// and publishes the token. Single-address atomics serialise at ~0.1 us each on
+// this part, so thousands of workgroups must not take tickets on one counter.
 struct SampleParams {
-  float *part_value;       // [grid] per-block best
-  uint32_t *part_index;    // [grid]
-  uint32_t *part_has;      // [grid]
-  uint32_t *counter;       // arrival counter, zero between launches
+  float *part_value;       // [kSampleMaxBlocks] per-workgroup best
+  uint32_t *part_index;
+  uint32_t *part_has;
   NervaHipSyntheticTokenSlot *slots;  // optional: publish slot[pos] and bump the cursor
   uint32_t *cursor_rw;
   uint32_t *token_out;     // optional: plain token output (operator entry point)
@@ -81,82 +90,34 @@ __device__ __forceinline__ float dot8(const uint4 &w, const uint4 &x, float acc)
   return dot2w<DT, DOT2>(w.w, x.w, acc);
 }
 
-// Final stage of the device sampler: called by every block after it has stored
-// its per-block best; the last block to arrive reduces all partials, publishes
-// the token and re-arms the counter. No block waits on another.
-__device__ __forceinline__ void sample_finish(const SampleParams &s, Best block_best, float *red_v,
-                                              uint32_t *red_i, uint32_t *red_h) {
-  __shared__ uint32_t is_last;
-  const uint32_t nblocks = gridDim.x;
-  if (threadIdx.x == 0) {
-    s.part_value[blockIdx.x] = block_best.value;
-    s.part_index[blockIdx.x] = block_best.index;
-    s.part_has[blockIdx.x] = block_best.has;
-    __threadfence();
-    uint32_t ticket = __hip_atomic_fetch_add(s.counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = ticket == nblocks - 1 ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  Best b{0.0f, 0u, 0u};
-  for (uint32_t i = threadIdx.x; i < nblocks; i += kBlock) {
-    Best o;
-    o.value = __hip_atomic_load(s.part_value + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    o.index = __hip_atomic_load(s.part_index + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    o.has = __hip_atomic_load(s.part_has + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (better(o, b)) b = o;
-  }
-  b = wave_best(b);
-  const int wave = threadIdx.x / kWave;
-  if ((threadIdx.x & (kWave - 1)) == 0) {
-    red_v[wave] = b.value;
-    red_i[wave] = b.index;
-    red_h[wave] = b.has;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    Best t{red_v[0], red_i[0], red_h[0]};
-    for (int w = 1; w < kWavesPerBlock; ++w) {
-      Best o{red_v[w], red_i[w], red_h[w]};
-      if (better(o, t)) t = o;
-    }
-    const uint32_t token = t.has ? t.index : 0u;
-    if (s.token_out != nullptr) *s.token_out = token;
-    if (s.slots != nullptr) {
-      const uint32_t pos = *s.cursor_rw;
-      NervaHipSyntheticTokenSlot slot;
-      slot.request_id = NERVA_HIP_SLOT_REQUEST_ID;
-      slot.sequence_id = NERVA_HIP_SLOT_SEQUENCE_ID;
-      slot.token_index = pos;
-      slot.token = token;
-      slot.version = static_cast<uint64_t>(pos) + 1u;
-      slot.completion = NERVA_HIP_SLOT_DEVICE_COMPLETE;
-      slot.host_copied = 0;
-      s.slots[pos] = slot;
-      *s.cursor_rw = pos + 1u;
-    }
-    __hip_atomic_store(s.counter, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-
-// UU consecutive 512-column chunks of NR rows: all UU*NR loads are issued before
-// the first FMA so that the wave keeps UU*NR KiB in flight.
-template <uint32_t DT, int NR, int UU, bool DOT2>
-__device__ __forceinline__ void row_chunks(const uint16_t *const (&wrow)[NR], const uint16_t *xs,
-                                           uint32_t chunk, int lane, float (&acc)[NR]) {
-  uint4 wv[NR][UU];
+// Issue UU consecutive 512-column chunks of NR rows (loads only).
+template <int NR, int UU, int CAP>
+__device__ __forceinline__ void chunks_load(const uint16_t *const (&wrow)[NR], uint32_t chunk, int lane,
+                                            uint4 (&wv)[NR][CAP]) {
   const uint32_t c0 = chunk * (kWave * 8) + lane * 8;
 #pragma unroll
   for (int u = 0; u < UU; ++u)
 #pragma unroll
     for (int k = 0; k < NR; ++k) wv[k][u] = load_stream(wrow[k] + c0 + u * (kWave * 8));
+}
+// Consume them against x in LDS.
+template <uint32_t DT, int NR, int UU, int CAP, bool DOT2>
+__device__ __forceinline__ void chunks_fma(const uint4 (&wv)[NR][CAP], const uint16_t *xs, uint32_t chunk,
+                                           int lane, float (&acc)[NR]) {
+  const uint32_t c0 = chunk * (kWave * 8) + lane * 8;
 #pragma unroll
   for (int u = 0; u < UU; ++u) {
     const uint4 xv = *reinterpret_cast<const uint4 *>(xs + c0 + u * (kWave * 8));
 #pragma unroll
     for (int k = 0; k < NR; ++k) acc[k] = dot8<DT, DOT2>(wv[k][u], xv, acc[k]);
   }
+}
+template <uint32_t DT, int NR, int UU, bool DOT2>
+__device__ __forceinline__ void row_chunks(const uint16_t *const (&wrow)[NR], const uint16_t *xs,
+                                           uint32_t chunk, int lane, float (&acc)[NR]) {
+  uint4 wv[NR][UU];
+  chunks_load<NR, UU, UU>(wrow, chunk, lane, wv);
+  chunks_fma<DT, NR, UU, UU, DOT2>(wv, xs, chunk, lane, acc);
 }
 
 enum : int { kScalar = 0, kVecGuarded = 1, kVecFull = 2 };
@@ -176,6 +137,47 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint32_t cols = p.cols;
+  const uint32_t units = (EPI == kEpiSwiglu) ? p.rows : (p.rows + NR - 1) / NR;
+  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
+  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
+  const uint32_t nchunks = cols / (kWave * 8);
+
+  auto unit_rows = [&](uint32_t unit, uint32_t (&row)[NR], const uint16_t *(&wrow)[NR], bool (&live)[NR]) {
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      if constexpr (EPI == kEpiSwiglu) {
+        row[k] = unit + k * p.rows;  // k = 0 gate row, k = 1 up row
+        live[k] = true;
+      } else {
+        row[k] = unit * NR + k;
+        live[k] = row[k] < p.rows;
+      }
+      wrow[k] = p.w + static_cast<uint64_t>(live[k] ? row[k] : 0u) * cols;
+    }
+  };
+
+  // ---- request the head of this wave's first rows before x is touched -------
+  // head = the first min(U, nchunks) chunks (a power of two), the same for every unit.
+  const uint32_t head = nchunks >= static_cast<uint32_t>(U) ? U : (U > 4 && nchunks >= 4) ? 4u : (U > 2 && nchunks >= 2) ? 2u : 1u;
+  // (a macro, not a lambda: the buffers must stay in VGPRs, and an array that is handed to a
+  // closure by reference ends up in scratch memory)
+#define NV_GEMV_HEAD_LOAD(UNIT, DST)                                                              \
+  do {                                                                                            \
+    uint32_t row_[NR];                                                                            \
+    const uint16_t *wrow_[NR];                                                                    \
+    bool live_[NR];                                                                               \
+    unit_rows((UNIT), row_, wrow_, live_);                                                        \
+    if (head == static_cast<uint32_t>(U)) chunks_load<NR, U, U>(wrow_, 0, lane, DST);             \
+    else if (U > 4 && head == 4) chunks_load<NR, (U > 4 ? 4 : 1), U>(wrow_, 0, lane, DST);        \
+    else if (U > 2 && head == 2) chunks_load<NR, (U > 2 ? 2 : 1), U>(wrow_, 0, lane, DST);        \
+    else chunks_load<NR, 1, U>(wrow_, 0, lane, DST);                                              \
+  } while (0)
+  // Two head buffers that swap roles every unit (no register copies: a copy would wait for
+  // the very loads it is meant to overlap).
+  uint4 buf[2][NR][U];
+  if constexpr (MODE == kVecFull) {
+    if (wave_global < units) NV_GEMV_HEAD_LOAD(wave_global, buf[0]);
+  }
 
   // ---- prologue: x -> LDS as 16-bit ------------------------------------
   if constexpr (PRO == kProX16) {
@@ -189,49 +191,69 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
     // x = round16(v * rsqrt(mean(v^2) + eps) * gamma)
     float ss = 0.0f;
     if constexpr (MODE != kScalar) {
-      for (uint32_t c = threadIdx.x * 4; c < cols; c += kBlock * 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(p.xf + c);
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8) {
+        const float4 a = *reinterpret_cast<const float4 *>(p.xf + c);
+        const float4 b = *reinterpret_cast<const float4 *>(p.xf + c + 4);
+        ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
       }
     } else {
       for (uint32_t c = threadIdx.x; c < cols; c += kBlock) ss += p.xf[c] * p.xf[c];
     }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / static_cast<float>(cols) + p.eps);
-    for (uint32_t c = threadIdx.x; c < cols; c += kBlock)
-      xs[c] = enc16<DT>(p.xf[c] * scale * dec16<DT>(p.gamma[c]));
+    if constexpr (MODE != kScalar) {
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8) {
+        const float4 a = *reinterpret_cast<const float4 *>(p.xf + c);   // second touch: L1/L2 hit
+        const float4 b = *reinterpret_cast<const float4 *>(p.xf + c + 4);
+        const uint4 g = *reinterpret_cast<const uint4 *>(p.gamma + c);
+        float g0, g1, g2, g3, g4, g5, g6, g7;
+        unpack2<DT>(g.x, g0, g1);
+        unpack2<DT>(g.y, g2, g3);
+        unpack2<DT>(g.z, g4, g5);
+        unpack2<DT>(g.w, g6, g7);
+        uint4 o;
+        o.x = enc16<DT>(a.x * scale * g0) | (static_cast<uint32_t>(enc16<DT>(a.y * scale * g1)) << 16);
+        o.y = enc16<DT>(a.z * scale * g2) | (static_cast<uint32_t>(enc16<DT>(a.w * scale * g3)) << 16);
+        o.z = enc16<DT>(b.x * scale * g4) | (static_cast<uint32_t>(enc16<DT>(b.y * scale * g5)) << 16);
+        o.w = enc16<DT>(b.z * scale * g6) | (static_cast<uint32_t>(enc16<DT>(b.w * scale * g7)) << 16);
+        *reinterpret_cast<uint4 *>(xs + c) = o;
+      }
+    } else {
+      for (uint32_t c = threadIdx.x; c < cols; c += kBlock)
+        xs[c] = enc16<DT>(p.xf[c] * scale * dec16<DT>(p.gamma[c]));
+    }
   }
   __syncthreads();
 
   // ---- main loop: each wave owns NR rows per iteration -------------------
-  const uint32_t units = (EPI == kEpiSwiglu) ? p.rows : (p.rows + NR - 1) / NR;
-  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
-  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
   Best best{0.0f, 0u, 0u};
 
-  for (uint32_t unit = wave_global; unit < units; unit += wave_stride) {
+  // One unit of NR rows per phase. buf[ph] holds the unit's head (requested earlier); the
+  // head of the unit after it goes into buf[ph ^ 1] before buf[ph] is consumed, so the
+  // wave's load queue is never empty between rows.
+  for (uint32_t unit0 = wave_global; unit0 < units; unit0 += 2 * wave_stride) {
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+    const uint32_t unit = unit0 + ph * wave_stride;
+    if (unit >= units) break;
     uint32_t row[NR];
     const uint16_t *wrow[NR];
     bool live[NR];
-#pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      if constexpr (EPI == kEpiSwiglu) {
-        row[k] = unit + k * p.rows;  // k = 0 gate row, k = 1 up row
-        live[k] = true;
-      } else {
-        row[k] = unit * NR + k;
-        live[k] = row[k] < p.rows;
-      }
-      wrow[k] = p.w + static_cast<uint64_t>(live[k] ? row[k] : 0u) * cols;
-    }
+    unit_rows(unit, row, wrow, live);
     float acc[NR];
 #pragma unroll
     for (int k = 0; k < NR; ++k) acc[k] = 0.0f;
 
     if constexpr (MODE == kVecFull) {
       // cols % 512 == 0: every lane has a full 16-byte chunk in every step, no guards.
-      uint32_t chunk = 0;
-      const uint32_t nchunks = cols / (kWave * 8);
+      // The head of the NEXT unit is requested before this unit's head is consumed, so the
+      // wave never sits with an empty load queue between rows.
+      if (unit + wave_stride < units) NV_GEMV_HEAD_LOAD(unit + wave_stride, buf[ph ^ 1]);
+      if (head == static_cast<uint32_t>(U)) chunks_fma<DT, NR, U, U, DOT2>(buf[ph], xs, 0, lane, acc);
+      else if (U > 4 && head == 4) chunks_fma<DT, NR, (U > 4 ? 4 : 1), U, DOT2>(buf[ph], xs, 0, lane, acc);
+      else if (U > 2 && head == 2) chunks_fma<DT, NR, (U > 2 ? 2 : 1), U, DOT2>(buf[ph], xs, 0, lane, acc);
+      else chunks_fma<DT, NR, 1, U, DOT2>(buf[ph], xs, 0, lane, acc);
+      uint32_t chunk = head;
       for (; chunk + U <= nchunks; chunk += U) row_chunks<DT, NR, U, DOT2>(wrow, xs, chunk, lane, acc);
       if constexpr (U > 4) {
         if (chunk + 4 <= nchunks) {
@@ -310,35 +332,43 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
       }
     }
   }
+  }
+#undef NV_GEMV_HEAD_LOAD
 
   if constexpr (EPI == kEpiArgmax) {
+    // one candidate per workgroup; sample_finish_kernel reduces them
     if (lane == 0) {
       red[wave] = best.value;
       red_i[wave] = best.index;
       red_h[wave] = best.has;
     }
     __syncthreads();
-    Best block_best{red[0], red_i[0], red_h[0]};
-    for (int w = 1; w < kWavesPerBlock; ++w) {
-      Best o{red[w], red_i[w], red_h[w]};
-      if (better(o, block_best)) block_best = o;
+    if (threadIdx.x == 0) {
+      Best block_best{red[0], red_i[0], red_h[0]};
+      for (int w = 1; w < kWavesPerBlock; ++w) {
+        Best o{red[w], red_i[w], red_h[w]};
+        if (better(o, block_best)) block_best = o;
+      }
+      p.sample.part_value[blockIdx.x] = block_best.value;
+      p.sample.part_index[blockIdx.x] = block_best.index;
+      p.sample.part_has[blockIdx.x] = block_best.has;
     }
-    __syncthreads();
-    sample_finish(p.sample, block_best, red, red_i, red_h);
   }
 }
 
-// Host-side tuning knobs (set by the launcher; overridable for sweeps).
+// Host-side tuning knobs (overridable for sweeps).
 struct GemvTuning {
-  int rows_per_wave = 2;   // NR for non-swiglu epilogues (1 or 2)
-  int unroll = 8;          // U (4 or 8)
-  int dot2 = 0;
-  int max_blocks = 0;      // 0 = automatic
+  int max_blocks = 0;      // 0 = library default (a few workgroups per CU)
 };
 
 hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvParams &p,
                        hipStream_t stream, const GemvTuning *tuning = nullptr);
 uint32_t gemv_grid_blocks(int epilogue, uint32_t rows, int rows_per_wave, int max_blocks);
-constexpr uint32_t kSampleMaxBlocks = 4096;  // capacity of SampleParams::part_* arrays
+// Number of workgroups (= sampler candidates) an LM-head launch over `rows` rows uses.
+uint32_t gemv_sample_blocks(uint32_t rows);
+// Reduce `count` per-workgroup candidates and publish the token (one workgroup).
+hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,
+                                uint32_t max_steps, hipStream_t stream);
+constexpr uint32_t kSampleMaxBlocks = 65536;  // capacity of SampleParams::part_* arrays
 
 }  // namespace nv

@@ -149,6 +149,14 @@ class DecodeSession:
             raise RuntimeError("read_kv failed")
         return k, v
 
+    def kv_range(self, layer, first, count):
+        k = np.empty((count, self.kv_hidden), np.uint16)
+        v = np.empty((count, self.kv_hidden), np.uint16)
+        if self.lib.nerva_hip_session_read_kv_range(self.handle, layer, first, count, k.ctypes.data,
+                                                    v.ctypes.data) != 0:
+            raise RuntimeError("read_kv_range failed")
+        return k, v
+
     def destroy(self):
         if self.handle:
             res = abi.NervaHipHfDecodeSequenceSessionCreateResult()

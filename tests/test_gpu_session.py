@@ -268,7 +268,7 @@ def test_eager_profile_pass_leaves_state_untouched():
     s.start(prompt)
     rc, res, a = s.advance(4)
     rc, prof = s.profile_step(2)
-    assert rc == 0 and prof.status == 0 and prof.launches == 2 + 5 * 2
+    assert rc == 0 and prof.status == 0 and prof.launches == 3 + 5 * 2
     assert prof.gate_up_ns > 0 and prof.lm_head_ns > 0 and prof.position == len(prompt) + 3
     rc, res, b = s.advance(6)
     s.start(prompt)
