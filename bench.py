@@ -8,7 +8,7 @@ A "step" is one decoded token (one graph replay = the whole per-token weight + K
 
 Prints ONE JSON line: whole-step tok/s, plus
   roofline     - the dominant kernel (fused gate_up GEMV): algorithmic bytes / average launch
-                 duration measured with hipEvent pairs on the session stream, vs 8 TB/s HBM;
+                 duration measured with hipEvents on the session stream, vs 8 TB/s HBM;
   cpu_baseline - the CPU oracle (scalar port of the reference's CPU path) timed on this
                  host on a bounded sample of the same decode step, extrapolated to tok/s.
 """
@@ -25,6 +25,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one gate_up launch moves at the Qwen3-8B shape (24576x4096 bf16): FETCH_SIZE + WRITE_SIZE
+# per dispatch from two `rocprofv3 --pmc` runs, each scaled by what the counter reads for a plain
+# 256 MiB copy kernel (profiles/gate_up_gemv_hbm_traffic_pmc.txt). Not measurable in-process.
+GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201779003}
 SEED = 0x4E45525641
 WEIGHT_STD = 0.02
 
@@ -113,6 +117,8 @@ def main():
     ap.add_argument("--layers", type=int, default=36, help="(debug) fewer layers = NOT the named workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-layers", type=int, default=2)
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also launch one plain copy kernel of this size (memory-counter calibration runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is a single-device decode loop and no multi-GPU "
@@ -142,11 +148,16 @@ def main():
     if args.warmup:
         rc, res, _ = session.advance(args.warmup)
         assert rc == 0
+    if args.copy_probe_mib:
+        src, dst = (N.DeviceBuffer.zeros(args.copy_probe_mib << 20) for _ in range(2))
+        N.Device.copy(dst, src, args.copy_probe_mib << 20)
+        N.Device.synchronize()
     allocs = N.Device.allocation_count()
     t0 = time.perf_counter()
     rc, res, tokens = session.advance(args.steps)
     elapsed = time.perf_counter() - t0
-    assert rc == 0 and res.observed_tokens == args.steps and res.graph_replays == args.steps
+    eager = os.environ.get("NERVA_HIP_EAGER_STEPS") == "1"   # kernel-tracing mode, see decode_session.hip
+    assert rc == 0 and res.observed_tokens == args.steps and (eager or res.graph_replays == args.steps)
     assert res.hot_path_allocations == 0 and N.Device.allocation_count() == allocs
     tok_s = args.steps / elapsed
     ctx_mid = args.prompt + 1 + args.warmup + args.steps // 2
@@ -154,17 +165,24 @@ def main():
     log("[bench] %d steps in %.3f s -> %.1f tok/s, %.3f ms/step, device %.3f ms/step, graph nodes %d" % (
         args.steps, elapsed, tok_s, 1e3 * elapsed / args.steps, res.device_elapsed_ns / 1e6 / args.steps, res.graph_nodes))
 
-    # dominant kernel: fused gate_up GEMV, timed live with hipEvent pairs around each eager launch
+    # Per-kernel durations, timed live with hipEvents on the session stream. "stream" figures
+    # bracket all 36 launches of one kind (one per layer, distinct weights) with ONE event pair and
+    # divide by the count: the kernel's own duration, which is what a kernel trace reports. The
+    # per-launch event pairs of the eager pass add the event/dispatch gap of every launch.
     rc, prof = session.profile_step(3)
     assert rc == 0
-    per_kind = {k: (getattr(prof, k + "_ns"), getattr(prof, k + "_bytes")) for k in
-                ("qkv", "attention", "o", "gate_up", "down", "lm_head")}
-    for k, (ns, b) in per_kind.items():
-        log("[profile] %-9s %8.2f us  %7.1f GB/s  (%.1f%% of HBM peak)" % (k, ns / 1e3, b / max(ns, 1), 100 * b / max(ns, 1) / HBM_PEAK_GBS))
+    per_kind = {}
+    for k in ("qkv", "attention", "o", "gate_up", "down", "lm_head"):
+        paired = getattr(prof, k + "_ns")
+        ns = getattr(prof, k + "_stream_ns", 0) or paired
+        per_kind[k] = (ns, getattr(prof, k + "_bytes"))
+        log("[profile] %-9s %8.2f us (event pair per launch %8.2f us)  %7.1f GB/s  (%.1f%% of HBM peak)" % (
+            k, ns / 1e3, paired / 1e3, per_kind[k][1] / max(ns, 1), 100 * per_kind[k][1] / max(ns, 1) / HBM_PEAK_GBS))
     gu_ns, gu_bytes = per_kind["gate_up"]
     roofline = dict(bound="hbm", kernel="gemv_kernel<bf16, rmsnorm prologue, swiglu epilogue> (gate_up 24576x4096)",
                     achieved=round(gu_bytes / gu_ns, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(gu_bytes / gu_ns / HBM_PEAK_GBS, 4), traffic=None,
+                    frac=round(gu_bytes / gu_ns / HBM_PEAK_GBS, 4),
+                    traffic=GATE_UP_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"])),
                     bytes_per_launch=gu_bytes, avg_launch_us=round(gu_ns / 1e3, 2),
                     whole_step_bytes=bytes_step, whole_step_frac=round(bytes_step * tok_s / 1e9 / HBM_PEAK_GBS, 4),
                     per_kernel_frac={k: round(b / max(ns, 1) / HBM_PEAK_GBS, 4) for k, (ns, b) in per_kind.items()})

@@ -495,6 +495,9 @@ int nerva_hip_memset(void *device_dst, int value, uint64_t bytes);
 int nerva_hip_stream_synchronize(void *stream);
 /* Counts hipMalloc/hipHostMalloc calls made by the library since load (hot-path allocation audit). */
 uint64_t nerva_hip_allocation_count(void);
+/* Plain device-to-device copy kernel (16-byte aligned pointers and size): moves exactly `bytes`
+ * in and `bytes` out, the known-size transfer memory counters are calibrated against. */
+int nerva_hip_copy_d2d(void *device_dst, const void *device_src, uint64_t bytes, void *stream);
 
 /* Synthetic tensors generated on the device by the counter-based generator the
  * tests' CPU oracle also implements (values are bit-identical on both sides):
@@ -528,6 +531,9 @@ typedef struct NervaHipStepProfile {
   /* average device ns per launch over `repeats` un-graphed steps, hipEvent pairs around each launch */
   uint64_t embed_ns, qkv_ns, attention_ns, o_ns, gate_up_ns, down_ns, lm_head_ns, total_ns;
   uint64_t qkv_bytes, attention_bytes, o_bytes, gate_up_bytes, down_bytes, lm_head_bytes;
+  /* average device ns per launch when the `layers` launches of one kind run back to back
+   * between a single hipEvent pair (no per-launch event gap): the kernel's own duration */
+  uint64_t qkv_stream_ns, attention_stream_ns, o_stream_ns, gate_up_stream_ns, down_stream_ns;
 } NervaHipStepProfile;
 
 /* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT

@@ -17,6 +17,8 @@
 // Every kernel reads the position from device memory, so one captured graph
 // serves every position and every prompt length.
 #include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
 
 #include <algorithm>
 #include <vector>
@@ -135,6 +137,13 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
     x[i] = dec16<DT>(row[i]);
 }
 
+__global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    state[0] = cursor;
+    state[1] = prompt_count;
+  }
+}
+
 __global__ void advance_cursor_kernel(uint32_t *state, uint32_t max_steps) {
   if (threadIdx.x == 0 && blockIdx.x == 0 && state[0] < max_steps) state[0] = state[0] + 1u;
 }
@@ -187,28 +196,22 @@ void destroy_session(Session *s) {
   delete s;
 }
 
-hipError_t run_launch(StepProfiler *prof, int kind, hipError_t (*fn)(void *), void *ctx) {
-  hipError_t err = hipSuccess;
-  if (prof) err = prof->before(kind);
-  if (err == hipSuccess) err = fn(ctx);
-  if (prof && err == hipSuccess) err = prof->after();
-  return err;
-}
-
-// Enqueue one step on the session stream (eagerly or under stream capture).
-hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
+// Enqueue one step on the session stream (eagerly or under stream capture). With
+// `only` >= 0 just the per-layer launches of that kind are enqueued (profiling).
+hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only = -1) {
   hipStream_t st = s->stream;
   const uint32_t A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim;
   hipError_t err = hipSuccess;
 #define NV_STEP(kind, expr)                         \
   do {                                              \
+    if (only >= 0 && only != (kind)) break;         \
     if (prof && err == hipSuccess) err = prof->before(kind); \
     if (err == hipSuccess) err = (expr);            \
     if (prof && err == hipSuccess) err = prof->after();      \
     if (err != hipSuccess) return err;              \
   } while (0)
 
-  {
+  if (only < 0) {
     const uint32_t blocks = std::min<uint32_t>((s->hidden + kBlock - 1) / kBlock, 64u);
     const float *rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
     if (prof) err = prof->before(kLEmbed);
@@ -309,6 +312,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
       NV_STEP(kLDown, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
     }
   }
+  if (only >= 0) return hipSuccess;
   if (mode == kPromptStep) {
     if (prof) err = prof->before(kLAdvance);
     if (err != hipSuccess) return err;
@@ -338,8 +342,24 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof) {
   return hipSuccess;
 }
 
+// NERVA_HIP_EAGER_STEPS=1 launches every step kernel by kernel instead of replaying the
+// captured graph. It exists for kernel tracing only: replaying a hipGraph under
+// `rocprofv3 --kernel-trace` crashes inside the runtime on this stack. Results and
+// per-kernel durations are the same; the graph counters then report zero replays.
+bool eager_steps() {
+  static const bool eager = [] {
+    const char *v = getenv("NERVA_HIP_EAGER_STEPS");
+    return v != nullptr && v[0] == '1';
+  }();
+  return eager;
+}
+
+// Launch one step: graph replay, or the same kernels eagerly (tracing mode).
+hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out);
+
 // graph index 0: decode step, 1: prompt step
 hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
+  if (eager_steps()) return hipSuccess;
   if (s->exec[which] != nullptr) {
     if (out) {
       out->graph_nodes = s->graph_nodes[which];
@@ -369,6 +389,21 @@ hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *o
     out->graph_captures += 1;
   }
   return hipSuccess;
+}
+
+hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
+  if (eager_steps()) {
+    hipError_t err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
+    if (err == hipSuccess) out->kernel_launches += (which == 0 ? 3 : 2) + 5ull * s->layers;
+    return err;
+  }
+  hipError_t err = hipGraphLaunch(s->exec[which], s->stream);
+  if (err == hipSuccess) {
+    out->graph_replays += 1;
+    out->graph_launches += 1;
+    out->kernel_launches += s->graph_nodes[which];
+  }
+  return err;
 }
 
 void fill_header(const Session *s, NervaHipHfDecodeSequenceResult *out, uint32_t steps,
@@ -431,15 +466,18 @@ bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
 
 hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t prompt_count,
                           NervaHipHfDecodeSequenceResult *out) {
-  hipError_t err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
-  memcpy(s->host_prompt, prompt_tokens, static_cast<uint64_t>(prompt_count) * sizeof(uint32_t));
-  s->host_state[0] = 0;
-  s->host_state[1] = prompt_count;
+  // Not on the per-token path: the prompt is copied synchronously (the caller's buffer may be
+  // reused as soon as this returns) and the cursor is set by a one-thread kernel in stream order.
+  hipError_t err = hipStreamSynchronize(s->stream);
   if (err == hipSuccess)
-    err = hipMemcpyAsync(s->state, s->host_state, 2 * sizeof(uint32_t), hipMemcpyHostToDevice, s->stream);
+    err = hipMemcpy(s->prompt, prompt_tokens, static_cast<uint64_t>(prompt_count) * sizeof(uint32_t),
+                    hipMemcpyHostToDevice);
   if (err == hipSuccess)
-    err = hipMemcpyAsync(s->prompt, s->host_prompt, static_cast<uint64_t>(prompt_count) * sizeof(uint32_t),
-                         hipMemcpyHostToDevice, s->stream);
+    err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  if (err == hipSuccess) {
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count);
+    err = hipGetLastError();
+  }
   out->h2d_bytes = static_cast<uint64_t>(prompt_count) * sizeof(uint32_t);
   return err;
 }
@@ -519,9 +557,11 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->planned_gpu_staged_weight_bytes = rq->planned_gpu_staged_weight_bytes;
   s->planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
   s->planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
-  // enough splits to put >= 2 workgroups on every CU, never more than KV blocks
+  // Split-KV factor of the decode attention. Every active split costs a device-scope
+  // release + an arrival ticket + one more partial for the last workgroup to merge
+  // (~0.4 us each, measured), so the grid is kept to ~128 workgroups of 8 waves.
   {
-    uint32_t splits = (512 + rq->kv_heads - 1) / rq->kv_heads;
+    uint32_t splits = (128 + rq->kv_heads - 1) / rq->kv_heads;
     splits = std::min(splits, kAttnMaxSplits);
     splits = std::min(splits, std::max(1u, block_count));
     s->attn_splits = std::max(1u, splits);
@@ -817,12 +857,7 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
   if (err == hipSuccess && P > 1) err = ensure_graph(s, 1, out);
   if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
   for (uint32_t i = 0; err == hipSuccess && i + 1 < P; ++i) {
-    err = hipGraphLaunch(s->exec[1], s->stream);
-    if (err == hipSuccess) {
-      out->graph_replays += 1;
-      out->graph_launches += 1;
-      out->kernel_launches += s->graph_nodes[1];
-    }
+    err = launch_step(s, 1, out);
   }
   if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
   if (err == hipSuccess) out->kernel_launches += 3 + 5ull * s->layers;
@@ -869,12 +904,7 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
   const uint64_t allocs_before = allocation_count();
   if (err == hipSuccess && run_count != 0) err = hipEventRecord(s->ev0, s->stream);
   for (uint32_t step = 0; err == hipSuccess && step < run_count; ++step) {
-    err = hipGraphLaunch(s->exec[0], s->stream);
-    if (err == hipSuccess) {
-      out->graph_replays += 1;
-      out->graph_launches += 1;
-      out->kernel_launches += s->graph_nodes[0];
-    }
+    err = launch_step(s, 0, out);
     // With a stop token the host looks at each token so that it can stop launching
     // (session_api_lifecycle.inc.cu:1206-1234); without one the loop never syncs.
     if (err == hipSuccess && s->has_eos != 0) {
@@ -960,12 +990,7 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
   const uint64_t allocs_before = allocation_count();
   if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
   for (uint32_t step = 0; err == hipSuccess && step < context_steps; ++step) {
-    err = hipGraphLaunch(s->exec[0], s->stream);
-    if (err == hipSuccess) {
-      out->graph_replays += 1;
-      out->graph_launches += 1;
-      out->kernel_launches += s->graph_nodes[0];
-    }
+    err = launch_step(s, 0, out);
   }
   if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
   const uint64_t slots_bytes = static_cast<uint64_t>(context_steps) * sizeof(Slot);
@@ -1096,6 +1121,31 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
     out->hip_error = static_cast<int32_t>(err);
     return -1;
   }
+  // back-to-back pass: all `layers` launches of one kind between a single event pair, so the
+  // figure is the kernel's own duration without the per-launch event gaps
+  uint64_t stream_ns[kLKinds] = {0};
+  for (int kind = kLQkv; err == hipSuccess && kind <= kLDown; ++kind) {
+    uint64_t acc = 0;
+    for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
+      err = hipEventRecord(s->ev0, s->stream);
+      if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
+      if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
+      if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+      float ms = 0.0f;
+      if (err == hipSuccess) err = hipEventElapsedTime(&ms, s->ev0, s->ev1);
+      if (rep > 0) acc += static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+    }
+    stream_ns[kind] = acc / (static_cast<uint64_t>(repeats) * s->layers);
+  }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  out->qkv_stream_ns = stream_ns[kLQkv];
+  out->attention_stream_ns = stream_ns[kLAttn];
+  out->o_stream_ns = stream_ns[kLO];
+  out->gate_up_stream_ns = stream_ns[kLGateUp];
+  out->down_stream_ns = stream_ns[kLDown];
   auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
   out->position = pos;
   out->embed_ns = avg(kLEmbed);

@@ -149,6 +149,16 @@ struct DeviceBuffers {
 
 using namespace nv;
 
+namespace {
+// Plain 16-byte-per-lane copy: reads and writes exactly `vecs * 16` bytes. Used to calibrate
+// memory counters (what a counter reads for a transfer of known size).
+__global__ __launch_bounds__(kBlock) void plain_copy_kernel(uint4 *dst, const uint4 *src, uint64_t vecs) {
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < vecs;
+       i += static_cast<uint64_t>(gridDim.x) * kBlock)
+    dst[i] = src[i];
+}
+}  // namespace
+
 extern "C" {
 
 int nerva_hip_device_smoke(NervaHipDeviceSmokeResult *out) {
@@ -189,7 +199,7 @@ int nerva_hip_device_smoke(NervaHipDeviceSmokeResult *out) {
   out->compute_capability_minor = prop.minor;
   out->total_global_mem = total_bytes;
   out->free_global_mem = free_bytes;
-  strncpy(out->gpu_name, prop.name, sizeof(out->gpu_name) - 1);
+  strncpy(out->gpu_name, prop.name[0] != '\0' ? prop.name : prop.gcnArchName, sizeof(out->gpu_name) - 1);
   char bus[32] = {0};
   if (hipDeviceGetPCIBusId(bus, sizeof(bus), 0) == hipSuccess) strncpy(out->pci_bus_id, bus, sizeof(out->pci_bus_id) - 1);
   out->status = value == probe ? 0 : -1;
@@ -232,6 +242,18 @@ int nerva_hip_stream_synchronize(void *stream) {
   return hipStreamSynchronize(resolve_stream(stream)) == hipSuccess ? 0 : -1;
 }
 uint64_t nerva_hip_allocation_count(void) { return allocation_count(); }
+
+int nerva_hip_copy_d2d(void *device_dst, const void *device_src, uint64_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (device_dst == nullptr || device_src == nullptr || (bytes & 15u) != 0 ||
+      (reinterpret_cast<uintptr_t>(device_dst) & 15u) != 0 || (reinterpret_cast<uintptr_t>(device_src) & 15u) != 0)
+    return -1;
+  const uint64_t vecs = bytes / 16;
+  const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((vecs + kBlock - 1) / kBlock, 256u * 16u));
+  hipLaunchKernelGGL(plain_copy_kernel, dim3(blocks), dim3(kBlock), 0, resolve_stream(stream),
+                     static_cast<uint4 *>(device_dst), static_cast<const uint4 *>(device_src), vecs);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 int nerva_hip_synth_fill_16(void *device_dst, uint32_t dtype, uint64_t seed, uint64_t tensor_id,
                             uint64_t count, float mean, float std) {

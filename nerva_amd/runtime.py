@@ -31,6 +31,12 @@ class Device:
     def allocation_count():
         return int(abi.load().nerva_hip_allocation_count())
 
+    @staticmethod
+    def copy(dst, src, nbytes):
+        """Plain device copy kernel of a known size (memory-counter calibration)."""
+        if abi.load().nerva_hip_copy_d2d(dst.ptr, src.ptr, nbytes, None) != 0:
+            raise RuntimeError("copy_d2d failed")
+
 
 class DeviceBuffer:
     """A device allocation made through nerva_hip_malloc."""

@@ -471,3 +471,14 @@ def test_projection_bench_runs_and_checks_itself():
     print("q_proj GEMV eager %d ns, graph %d ns, %.0f GB/s" % (
         res.custom_avg_ns, res.custom_graph_avg_ns,
         (res.matrix_bytes + res.input_bytes + res.output_bytes) / res.custom_graph_avg_ns), flush=True)
+
+
+def test_plain_copy_kernel_is_exact_and_rejects_unaligned():
+    rng = np.random.default_rng(11)
+    for nbytes in (16, 4096 + 16, (3 << 20) + 48):
+        src = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        a, b = dev(src), N.DeviceBuffer.zeros(nbytes)
+        N.Device.copy(b, a, nbytes)
+        assert np.array_equal(b.numpy(np.uint8, nbytes), src)
+    assert abi.load().nerva_hip_copy_d2d(b.ptr, a.ptr, 24, None) == -1
+    assert abi.load().nerva_hip_copy_d2d(b.ptr + 4, a.ptr, 16, None) == -1
