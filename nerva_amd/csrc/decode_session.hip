@@ -336,7 +336,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   p.sample.cursor_rw = s->state;
   NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st));
   // one small workgroup reduces the per-workgroup candidates, writes slot[pos], bumps the cursor
-  NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows), s->state,
+  NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows, p.cols), s->state,
                                           s->max_ctx, st));
 #undef NV_STEP
   return hipSuccess;

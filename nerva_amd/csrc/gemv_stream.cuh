@@ -356,16 +356,247 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Production-shape kernel: cols % (512 * B) == 0, 16-byte aligned rows, cols <= 12288.
+// Same contract as gemv_kernel, leaner register budget (about 64 VGPRs instead of
+// ~150) so that 6-8 workgroups stay resident per CU and a whole 4096-row matrix is
+// on the machine at once. A wave walks a flat list of request batches - (its 1st
+// row, columns 0..512B), (1st row, next 512B columns), ..., (2nd row, ...) - with two
+// batches in flight in two register buffers that swap roles (fully unrolled, no
+// register copies). The activation vector and the first two weight batches are
+// requested before anything waits, the step guard is read after that, and the
+// residual element of a row is requested together with the row's first batch.
+// ---------------------------------------------------------------------------
+// Register budget as resident waves per SIMD (= workgroups per CU): 6 with a 16-bit input,
+// 5 with the RMSNorm prologue, which holds the f32 activations and the norm weights in
+// registers across the first weight requests (a budget of 6 makes it spill).
+constexpr int fast_waves_per_simd(int prologue) { return prologue == kProRmsNorm ? 5 : 6; }
+constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per lane
+
+template <uint32_t DT, int PRO, int EPI, int NR, int B>
+__global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
+  extern __shared__ __align__(16) uint16_t xs[];
+  __shared__ float red[kWavesPerBlock];
+  __shared__ uint32_t red_i[kWavesPerBlock];
+  __shared__ uint32_t red_h[kWavesPerBlock];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t cols = p.cols;
+  const uint32_t units = p.rows;  // NR == 1: rows; kEpiSwiglu (NR == 2): gate/up pairs
+  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
+  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
+  const uint32_t bpr = cols / (kWave * 8 * B);  // request batches per row
+  const uint32_t my_units = wave_global < units ? (units - wave_global + wave_stride - 1) / wave_stride : 0u;
+  const uint32_t total = my_units * bpr;
+
+  // ---- 1. activation loads (L2 hits), kept in registers until the weights are requested
+  constexpr int kXV = kFastMaxCols / (kBlock * 8);  // 6
+  uint4 xraw[PRO == kProX16 ? kXV : 1];
+  float4 xa[PRO == kProRmsNorm ? 2 : 1], xb[PRO == kProRmsNorm ? 2 : 1];
+  uint4 gw[PRO == kProRmsNorm ? 2 : 1];
+  const bool norm_in_regs = cols <= kBlock * 16;
+  if constexpr (PRO == kProX16) {
+#pragma unroll
+    for (int i = 0; i < kXV; ++i) {
+      const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+      xraw[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (c < cols) xraw[i] = *reinterpret_cast<const uint4 *>(p.x16 + c);
+    }
+  } else {
+    if (norm_in_regs) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        if (c < cols) {
+          xa[i] = *reinterpret_cast<const float4 *>(p.xf + c);
+          xb[i] = *reinterpret_cast<const float4 *>(p.xf + c + 4);
+          gw[i] = *reinterpret_cast<const uint4 *>(p.gamma + c);
+        }
+      }
+    }
+  }
+
+  // ---- 2. weight request state + the first two batches
+  uint32_t iu = wave_global, ib = 0;  // next batch to request: unit, batch within the row
+  const uint16_t *wp[NR];
+  uint4 buf0[NR][B], buf1[NR][B];
+  float res0 = 0.0f, res1 = 0.0f;     // residual element requested with a row's first batch
+#define NV_FAST_ISSUE(DST, RES)                                                                   \
+  do {                                                                                            \
+    if (ib == 0) {                                                                                \
+      _Pragma("unroll") for (int k = 0; k < NR; ++k)                                              \
+        wp[k] = p.w + static_cast<uint64_t>(iu + k * p.rows) * cols + lane * 8;                   \
+      if constexpr (EPI == kEpiResidual) {                                                        \
+        if (lane == 0) RES = p.residual[iu];                                                      \
+      }                                                                                           \
+    }                                                                                             \
+    _Pragma("unroll") for (int u = 0; u < B; ++u)                                                 \
+      _Pragma("unroll") for (int k = 0; k < NR; ++k) DST[k][u] = load_stream(wp[k] + u * (kWave * 8)); \
+    _Pragma("unroll") for (int k = 0; k < NR; ++k) wp[k] += B * (kWave * 8);                      \
+    if (++ib == bpr) {                                                                            \
+      ib = 0;                                                                                     \
+      iu += wave_stride;                                                                          \
+    }                                                                                             \
+  } while (0)
+  if (total > 0) NV_FAST_ISSUE(buf0, res0);
+  if (total > 1) NV_FAST_ISSUE(buf1, res1);
+
+  // ---- 3. step guard (after the requests: they do not depend on it and are always in bounds)
+  if (p.cursor != nullptr && *p.cursor >= p.max_steps) return;
+
+  // ---- 4. prologue: x -> LDS as 16-bit
+  if constexpr (PRO == kProX16) {
+#pragma unroll
+    for (int i = 0; i < kXV; ++i) {
+      const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+      if (c < cols) *reinterpret_cast<uint4 *>(xs + c) = xraw[i];
+    }
+  } else {
+    float ss = 0.0f;
+    if (norm_in_regs) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        if (c < cols)
+          ss += xa[i].x * xa[i].x + xa[i].y * xa[i].y + xa[i].z * xa[i].z + xa[i].w * xa[i].w +
+                xb[i].x * xb[i].x + xb[i].y * xb[i].y + xb[i].z * xb[i].z + xb[i].w * xb[i].w;
+      }
+    } else {
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8) {
+        const float4 a = *reinterpret_cast<const float4 *>(p.xf + c);
+        const float4 b = *reinterpret_cast<const float4 *>(p.xf + c + 4);
+        ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+      }
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / static_cast<float>(cols) + p.eps);
+    auto emit = [&](uint32_t c, const float4 &a, const float4 &b, const uint4 &g) {
+      float g0, g1, g2, g3, g4, g5, g6, g7;
+      unpack2<DT>(g.x, g0, g1);
+      unpack2<DT>(g.y, g2, g3);
+      unpack2<DT>(g.z, g4, g5);
+      unpack2<DT>(g.w, g6, g7);
+      uint4 o;
+      o.x = enc16<DT>(a.x * scale * g0) | (static_cast<uint32_t>(enc16<DT>(a.y * scale * g1)) << 16);
+      o.y = enc16<DT>(a.z * scale * g2) | (static_cast<uint32_t>(enc16<DT>(a.w * scale * g3)) << 16);
+      o.z = enc16<DT>(b.x * scale * g4) | (static_cast<uint32_t>(enc16<DT>(b.y * scale * g5)) << 16);
+      o.w = enc16<DT>(b.z * scale * g6) | (static_cast<uint32_t>(enc16<DT>(b.w * scale * g7)) << 16);
+      *reinterpret_cast<uint4 *>(xs + c) = o;
+    };
+    if (norm_in_regs) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        if (c < cols) emit(c, xa[i], xb[i], gw[i]);
+      }
+    } else {
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8)
+        emit(c, *reinterpret_cast<const float4 *>(p.xf + c), *reinterpret_cast<const float4 *>(p.xf + c + 4),
+             *reinterpret_cast<const uint4 *>(p.gamma + c));
+    }
+  }
+  __syncthreads();
+
+  // ---- 5. main loop
+  Best best{0.0f, 0u, 0u};
+  uint32_t cu = wave_global, cb = 0;  // batch being consumed: unit, batch within the row
+  float acc[NR];
+  float res_cur = 0.0f;
+#define NV_FAST_CONSUME(SRC, RES)                                                                 \
+  do {                                                                                            \
+    if (cb == 0) {                                                                                \
+      _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = 0.0f;                               \
+      res_cur = RES;                                                                              \
+    }                                                                                             \
+    const uint32_t c0 = cb * (B * kWave * 8) + lane * 8;                                          \
+    _Pragma("unroll") for (int u = 0; u < B; ++u) {                                               \
+      const uint4 xv = *reinterpret_cast<const uint4 *>(xs + c0 + u * (kWave * 8));               \
+      _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = dot8<DT, false>(SRC[k][u], xv, acc[k]); \
+    }                                                                                             \
+    if (++cb == bpr) {                                                                            \
+      cb = 0;                                                                                     \
+      _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = wave_sum(acc[k]);                   \
+      if (lane == 0) {                                                                            \
+        if constexpr (EPI == kEpiSwiglu) {                                                        \
+          float g = acc[0], u = acc[NR - 1];                                                      \
+          if (p.bias != nullptr) {                                                                \
+            g += dec16<DT>(p.bias[cu]);                                                           \
+            u += dec16<DT>(p.bias[cu + p.rows]);                                                  \
+          }                                                                                       \
+          p.out16[cu] = enc16<DT>(silu(g) * u);                                                   \
+        } else {                                                                                  \
+          float y = acc[0];                                                                       \
+          if (p.bias != nullptr) y += dec16<DT>(p.bias[cu]);                                      \
+          if constexpr (EPI == kEpiF32) {                                                         \
+            p.out_f32[cu] = y;                                                                    \
+          } else if constexpr (EPI == kEpiResidual) {                                             \
+            y += res_cur;                                                                         \
+            if (p.round_out) y = round16<DT>(y);                                                  \
+            p.out_f32[cu] = y;                                                                    \
+          } else if constexpr (EPI == kEpiOut16) {                                                \
+            p.out16[cu] = enc16<DT>(y);                                                           \
+          } else if constexpr (EPI == kEpiArgmax) {                                               \
+            p.out_f32[cu] = y;                                                                    \
+            Best cand{y, cu, isfinite(y) ? 1u : 0u};                                              \
+            if (better(cand, best)) best = cand;                                                  \
+          }                                                                                       \
+        }                                                                                         \
+      }                                                                                           \
+      cu += wave_stride;                                                                          \
+    }                                                                                             \
+  } while (0)
+
+  for (uint32_t t = 0; t < total; t += 2) {
+    NV_FAST_CONSUME(buf0, res0);
+    if (t + 2 < total) NV_FAST_ISSUE(buf0, res0);
+    if (t + 1 < total) {
+      NV_FAST_CONSUME(buf1, res1);
+      if (t + 3 < total) NV_FAST_ISSUE(buf1, res1);
+    }
+  }
+#undef NV_FAST_ISSUE
+#undef NV_FAST_CONSUME
+
+  if constexpr (EPI == kEpiArgmax) {
+    if (lane == 0) {
+      red[wave] = best.value;
+      red_i[wave] = best.index;
+      red_h[wave] = best.has;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      Best block_best{red[0], red_i[0], red_h[0]};
+      for (int w = 1; w < kWavesPerBlock; ++w) {
+        Best o{red[w], red_i[w], red_h[w]};
+        if (better(o, block_best)) block_best = o;
+      }
+      p.sample.part_value[blockIdx.x] = block_best.value;
+      p.sample.part_index[blockIdx.x] = block_best.index;
+      p.sample.part_has[blockIdx.x] = block_best.has;
+    }
+  }
+}
+
 // Host-side tuning knobs (overridable for sweeps).
 struct GemvTuning {
   int max_blocks = 0;      // 0 = library default (a few workgroups per CU)
+  bool force_generic = false;  // never take the lean production-shape kernel
 };
 
 hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvParams &p,
                        hipStream_t stream, const GemvTuning *tuning = nullptr);
-uint32_t gemv_grid_blocks(int epilogue, uint32_t rows, int rows_per_wave, int max_blocks);
-// Number of workgroups (= sampler candidates) an LM-head launch over `rows` rows uses.
-uint32_t gemv_sample_blocks(uint32_t rows);
+// Kernel variant and grid of a launch (shared by the launcher and by callers that size
+// per-workgroup outputs). `vec16` = every pointer is 16-byte aligned.
+struct GemvPlan {
+  int mode;         // kScalar / kVecGuarded / kVecFull / kFast
+  uint32_t blocks;
+};
+constexpr int kFast = 3;  // the lean production-shape kernel
+GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,
+                   const struct GemvTuning *tuning);
+// Number of workgroups (= sampler candidates) an LM-head launch over [rows x cols] uses.
+uint32_t gemv_sample_blocks(uint32_t rows, uint32_t cols);
 // Reduce `count` per-workgroup candidates and publish the token (one workgroup).
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,
                                 uint32_t max_steps, hipStream_t stream);

@@ -1,4 +1,6 @@
 // Host launcher for the weight-streaming GEMV kernels (gemv_stream.cuh).
+#include <algorithm>
+
 #include "gemv_stream.cuh"
 
 namespace nv {
@@ -10,9 +12,13 @@ namespace {
 // launch; one row per wave with the whole 4096-wide row (8 KiB) in flight and an
 // uncapped grid is the best or tied-best on every decode shape.
 constexpr int kDefaultNR = 1;
-constexpr int kDefaultU = 8;        // NR * U = 8 KiB per wave per request batch
+#ifndef NV_GEMV_U
+#define NV_GEMV_U 8
+#endif
+constexpr int kDefaultU = NV_GEMV_U;  // chunks of 1 KiB in flight per wave per request batch
 constexpr bool kDefaultDot2 = false;
-constexpr uint32_t kDefaultMaxBlocks = 256u * 6u;  // workgroups per launch: 6 per CU
+constexpr uint32_t kCus = 256;                     // gfx950: 8 XCDs x 32 CUs
+constexpr uint32_t kDefaultMaxBlocks = kCus * 6u;  // generic kernels: 6 workgroups per CU
 
 // One workgroup: reduce the per-workgroup candidates, publish the token.
 __global__ __launch_bounds__(1024) void sample_finish_kernel(SampleParams s, uint32_t count,
@@ -61,7 +67,10 @@ __global__ __launch_bounds__(1024) void sample_finish_kernel(SampleParams s, uin
 template <uint32_t DT, int PRO, int EPI, int MODE>
 hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream) {
   constexpr int NR = EPI == kEpiSwiglu ? 2 : kDefaultNR;  // swiglu: the gate row and the up row
-  if constexpr (MODE == kVecFull) {
+  if constexpr (MODE == kFast) {
+    hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR>), dim3(blocks), dim3(kBlock), lds,
+                       stream, p);
+  } else if constexpr (MODE == kVecFull) {
     hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, kDefaultU / NR, kVecFull, kDefaultDot2>),
                        dim3(blocks), dim3(kBlock), lds, stream, p);
   } else if constexpr (MODE == kVecGuarded) {
@@ -99,13 +108,39 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 }  // namespace
 
-uint32_t gemv_grid_blocks(int epilogue, uint32_t rows, int rows_per_wave, int max_blocks) {
-  const uint32_t units = epilogue == kEpiSwiglu ? rows : (rows + rows_per_wave - 1) / rows_per_wave;
-  uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
-  uint32_t cap = max_blocks > 0 ? static_cast<uint32_t>(max_blocks) : kDefaultMaxBlocks;
-  if (epilogue == kEpiArgmax && cap > kSampleMaxBlocks) cap = kSampleMaxBlocks;
-  if (blocks > cap) blocks = cap;
-  return blocks == 0 ? 1 : blocks;
+// kFast needs cols % 2048 == 0 (% 1024 for the gate/up pair) and cols <= kFastMaxCols.
+GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,
+                   const GemvTuning *tuning) {
+  GemvPlan plan;
+  const bool vec = vec16 && cols % 8 == 0;
+  plan.mode = !vec ? kScalar : (cols % (kWave * 8) == 0 ? kVecFull : kVecGuarded);
+  const uint32_t fast_cols = epilogue == kEpiSwiglu ? kWave * 8 * 2 : kWave * 8 * 4;
+  if (plan.mode == kVecFull && cols % fast_cols == 0 && cols <= static_cast<uint32_t>(kFastMaxCols) &&
+      !(tuning && tuning->force_generic))
+    plan.mode = kFast;
+  // one wave per unit (a row, or a gate/up pair)
+  const uint32_t want = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+  uint32_t blocks = want;
+  if (tuning && tuning->max_blocks > 0) {
+    blocks = std::min<uint32_t>(want, static_cast<uint32_t>(tuning->max_blocks));
+  } else if (plan.mode == kFast) {
+    // Workgroups that fit the machine at once: register budget, and the LDS copy of x.
+    const uint32_t by_lds = (160u * 1024u) / (cols * 2u + 1024u);
+    const uint32_t resident =
+        kCus * std::min<uint32_t>(static_cast<uint32_t>(fast_waves_per_simd(prologue)), std::max(by_lds, 1u));
+    if (want <= resident) {
+      blocks = want;                       // everything is on the machine at once, one unit per wave
+    } else if (want <= 2 * resident) {
+      blocks = (want + 1) / 2;             // exactly two units per wave, pipelined in one round
+    } else {
+      blocks = std::min(want, kCus * 8u);  // long launches: oversubscribe, the dispatcher evens the tail
+    }
+  } else {
+    blocks = std::min(want, kDefaultMaxBlocks);
+  }
+  if (epilogue == kEpiArgmax && blocks > kSampleMaxBlocks) blocks = kSampleMaxBlocks;
+  plan.blocks = blocks == 0 ? 1 : blocks;
+  return plan;
 }
 
 hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvParams &p,
@@ -122,24 +157,29 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
     return hipErrorInvalidValue;
   if (dtype != kF16 && dtype != kBF16) return hipErrorInvalidValue;
 
-  const bool vec = (p.cols % 8 == 0) && aligned16(p.w) &&
-                   (prologue == kProX16 ? aligned16(p.x16) : aligned16(p.xf));
+  const bool vec16 = aligned16(p.w) && (prologue == kProX16 ? aligned16(p.x16)
+                                                             : (aligned16(p.xf) && aligned16(p.gamma)));
   const size_t lds = static_cast<size_t>((p.cols + 7) / 8 * 8) * sizeof(uint16_t);
   if (lds > 60 * 1024) return hipErrorInvalidValue;  // K up to 30720 fits one workgroup's LDS
-  const uint32_t blocks = gemv_grid_blocks(epilogue, p.rows, kDefaultNR, tuning ? tuning->max_blocks : 0);
-
-  const int mode = !vec ? kScalar : (p.cols % (kWave * 8) == 0 ? kVecFull : kVecGuarded);
+  const GemvPlan plan = gemv_plan(prologue, epilogue, p.rows, p.cols, vec16, tuning);
+  const int mode = plan.mode;
+  const uint32_t blocks = plan.blocks;
   if (dtype == kBF16) {
+    if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, blocks, lds, stream);
     if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
     if (mode == kVecGuarded) return launch_pro<kBF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream);
     return launch_pro<kBF16, kScalar>(prologue, epilogue, p, blocks, lds, stream);
   }
+  if (mode == kFast) return launch_pro<kF16, kFast>(prologue, epilogue, p, blocks, lds, stream);
   if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
   if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream);
   return launch_pro<kF16, kScalar>(prologue, epilogue, p, blocks, lds, stream);
 }
 
-uint32_t gemv_sample_blocks(uint32_t rows) { return gemv_grid_blocks(kEpiArgmax, rows, kDefaultNR, 0); }
+uint32_t gemv_sample_blocks(uint32_t rows, uint32_t cols) {
+  // session buffers come from a 256-byte-granular arena, so the aligned plan is the one launched
+  return gemv_plan(kProRmsNorm, kEpiArgmax, rows, cols, true, nullptr).blocks;
+}
 
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,
                                 uint32_t max_steps, hipStream_t stream) {
