@@ -436,10 +436,13 @@ typedef struct NervaHipPagedAttentionRequest {
 int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *request, void *stream,
                                int32_t *hip_error);
 uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim);
-/* Element offset of (layer, physical block, kv_head, token-in-block, 0) in the cache arrays. */
+/* Element offset of (layer, physical block, kv_head, token-in-block, dim) in the K (is_value 0)
+ * or V (is_value 1) cache array. A (block, kv_head) tile of 16 tokens x head_dim elements is
+ * contiguous; inside it the order is the library's own (matrix-core operand order at head_dim
+ * 128, row-major otherwise), so hosts that fill or read a cache go through this function. */
 uint64_t nerva_hip_kv_cache_offset(uint32_t block_count, uint32_t kv_heads, uint32_t head_dim,
                                    uint32_t layer, uint32_t physical_block, uint32_t kv_head,
-                                   uint32_t token_in_block);
+                                   uint32_t token_in_block, uint32_t dim, uint32_t is_value);
 
 typedef struct NervaHipArgmaxRequest {
   uint32_t count;

@@ -8,14 +8,32 @@ namespace nv {
 constexpr uint32_t kKvBlockTokens = 16;   // tokens per paged KV block (types.cuh:64)
 constexpr uint32_t kAttnMaxSplits = 64;   // split-KV partials per kv head
 
-// KV cache layout (library-owned): [layer][physical block][kv_head][16 tokens][head_dim]
+// KV cache layout (library-owned): [layer][physical block][kv_head][tile of 16 tokens x head_dim]
 // 16-bit, K and V in separate arrays. One (block, kv_head) tile is contiguous
 // (4 KiB at head_dim 128), so a wave streams it with four 1 KiB load instructions.
+// Inside a tile, head_dim 128 is stored in matrix-core operand order (kv_k_elem, kv_v_elem);
+// every other head_dim is row-major [token][dim].
 __host__ __device__ __forceinline__ uint64_t kv_tile_offset(uint32_t block_count, uint32_t kv_heads,
                                                             uint32_t head_dim, uint32_t layer,
                                                             uint32_t physical_block, uint32_t kv_head) {
   return ((static_cast<uint64_t>(layer) * block_count + physical_block) * kv_heads + kv_head) *
          kKvBlockTokens * head_dim;
+}
+
+// Element offset of (token row, dim d) inside a K tile. head_dim 128: load j of lane
+// l = (d%32/8)*16 + row holds dims 32j + 8*(l/16) .. +7 of token l%16, the A operand of a
+// 16x16x32 matrix-core product over dims.
+__host__ __device__ __forceinline__ uint32_t kv_k_elem(uint32_t head_dim, uint32_t row, uint32_t d) {
+  if (head_dim != 128) return row * head_dim + d;
+  return (d / 32) * 512 + (((d % 32) / 8) * 16 + row) * 8 + d % 8;
+}
+// Same for a V tile. head_dim 128: load j of lane l = (row/4)*16 + d%16 holds tokens
+// 4*(l/16) .. +3 of dim 32j + l%16, then of dim 32j + 16 + l%16: the A operands of two
+// 16x16x16 products over tokens (V transposed).
+__host__ __device__ __forceinline__ uint32_t kv_v_elem(uint32_t head_dim, uint32_t row, uint32_t d) {
+  if (head_dim != 128) return row * head_dim + d;
+  const uint32_t slab = d / 16, n = d % 16;
+  return (slab / 2) * 512 + ((row / 4) * 16 + n) * 8 + (slab % 2) * 4 + row % 4;
 }
 
 struct AttnParams {

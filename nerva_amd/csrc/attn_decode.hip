@@ -9,15 +9,11 @@
 //
 // gfx950 mapping of the fast path (head_dim 128, G = heads/kv_heads in {1,2,4,8}):
 //   grid (kv_heads, splits), 8 waves per workgroup; a wave owns whole 16-token KV
-//   blocks of its workgroup's token range. One block tile
-//   of one kv head is 4 KiB contiguous, fetched by four 1 KiB load instructions
-//   in exactly the register layout the math wants: load i, lane l holds the 8
-//   dims (l%16)*8.. of token 4i + l/16. So a 16-lane DPP row reduces one q.k, the
-//   probabilities land in the lanes that hold the matching V slice, and K/V never
-//   need a shuffle through LDS; the next tile's 8 loads are in flight while the
-//   current one is consumed. All G query heads of the kv head share each K/V
-//   register (1 unpack, G FMAs). LDS only carries q and the cross-wave merge.
-//   The last workgroup to finish a kv head merges its split partials (arrival
+//   tiles of its workgroup's token range and runs q.K^T and P.V on the matrix cores
+//   (details at attn_fast_kernel). The cache keeps each tile in matrix-operand order,
+//   so a tile is eight coalesced 1 KiB loads straight into operand registers; two tiles
+//   are in flight per wave. LDS only carries q, the new K/V row and the cross-wave
+//   merge. The last workgroup to finish a kv head merges its split partials (arrival
 //   counter; nobody waits), so a layer needs no separate reduce launch.
 #include "attn_decode.cuh"
 
@@ -27,23 +23,6 @@ namespace {
 
 constexpr int kHD = 128;
 constexpr int kAttnWaves = 8;   // waves per workgroup of the fast path (group 8 uses half)
-
-// Sum over the 16 lanes of a DPP row; every lane of the row gets the total.
-__device__ __forceinline__ float row16_sum(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
-  return v;
-}
-
-template <uint32_t DT>
-__device__ __forceinline__ void unpack8(const uint4 &v, float (&f)[8]) {
-  unpack2<DT>(v.x, f[0], f[1]);
-  unpack2<DT>(v.y, f[2], f[3]);
-  unpack2<DT>(v.z, f[4], f[5]);
-  unpack2<DT>(v.w, f[6], f[7]);
-}
 
 // One wave prepares one 128-wide head: lane l owns the RoPE pair (l, l+64).
 // out[] receives f32; when out16 != null the value is rounded first and the 16-bit
@@ -91,10 +70,145 @@ __device__ __forceinline__ void prep_head128(const float *src, const uint16_t *b
   }
 }
 
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// D(16x16) += A(16x32) . B(32x16): lane l holds A[l%16][8*(l/16)..+7], B[8*(l/16)..+7][l%16] and
+// D[4*(l/16)..+3][l%16].
+template <uint32_t DT>
+__device__ __forceinline__ f32x4_t mfma_k32(const uint4 &a, const uint4 &b, f32x4_t c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+// D(16x16) += A(16x16) . B(16x16): four contraction elements per lane, 4*(l/16)..+3.
+template <uint32_t DT>
+__device__ __forceinline__ f32x4_t mfma_k16(const uint2 &a, const uint2 &b, f32x4_t c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
+                                                     __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                 __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+}
+
+// Lane i of a 16-lane row receives lane i + N (shl) / i - N (shr); lanes without a source get 0.
+template <int N>
+__device__ __forceinline__ float row_shl(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + N, 0xF, 0xF, true));
+}
+template <int N>
+__device__ __forceinline__ float row_shr(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x110 + N, 0xF, 0xF, true));
+}
+
+// v = hi + lo with hi, lo 16-bit: the pair carries 16 (bf16) / 22 (f16) mantissa bits, so a
+// matrix-core product against exact 16-bit K/V data loses nothing that matters to f32 math.
+template <uint32_t DT>
+__device__ __forceinline__ void split16(float v, uint16_t &hi, uint16_t &lo) {
+  hi = enc16<DT>(v);
+  lo = enc16<DT>(v - dec16<DT>(hi));
+}
+
+// Requests one (block, kv head) tile: four 1 KiB loads each for K and V.
+__device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t b, uint32_t kvh, int lane,
+                                               uint4 (&k)[4], uint4 (&v)[4]) {
+  const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    k[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
+    v[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
+  }
+}
+
+// One 16-token tile against the G query heads of the kv head (see attn_fast_kernel).
+template <uint32_t DT, int G>
+__device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], const uint4 (&qx)[4], uint32_t b,
+                                          uint32_t n_keys, int col, int grp, bool splice, uint32_t new_row,
+                                          const uint16_t *knew, const uint16_t *vnew, float &m, float &l,
+                                          f32x4_t (&acc)[8]) {
+  if (splice) {
+    // the row published by this workgroup may not be visible to its own loads yet: take it from LDS
+    if (static_cast<uint32_t>(col) == new_row) {  // K operand: lane = (token col, dims grp*8..)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kreg[j] = *reinterpret_cast<const uint4 *>(knew + j * 32 + grp * 8);
+    }
+    if (static_cast<uint32_t>(grp) == new_row / 4) {  // V operand: lane = (dim col of a slab, tokens grp*4..)
+      const uint32_t e = new_row % 4;
+      const uint32_t sh = (e & 1u) * 16u, keep = ~(0xffffu << sh);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t v0 = vnew[(2 * j) * 16 + col], v1 = vnew[(2 * j + 1) * 16 + col];
+        if (e < 2) {
+          vreg[j].x = (vreg[j].x & keep) | (v0 << sh);
+          vreg[j].z = (vreg[j].z & keep) | (v1 << sh);
+        } else {
+          vreg[j].y = (vreg[j].y & keep) | (v0 << sh);
+          vreg[j].w = (vreg[j].w & keep) | (v1 << sh);
+        }
+      }
+    }
+  }
+  // scores of tokens b*16 + grp*4 + r for column col
+  f32x4_t c{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) c = mfma_k32<DT>(kreg[j], qx[j], c);
+  float sc[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    // hi column + lo column of the same head (either order: one f32 add). Both shifts run
+    // with every lane active: a lane-crossing read from a lane that sits out returns 0.
+    const float from_up = row_shl<G>(c[r]), from_down = row_shr<G>(c[r]);
+    const float other = col < G ? from_up : from_down;
+    const bool valid = b * kKvBlockTokens + grp * 4 + r < n_keys;
+    sc[r] = valid ? c[r] + other : -INFINITY;
+  }
+  float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+  mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
+  mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+  const float m_new = fmaxf(m, mb);   // finite: every processed tile has a valid token
+  const float alpha = expf(m - m_new);
+  uint32_t px[2];
+  float psum = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 4; r += 2) {
+    const float p0 = expf(sc[r] - m_new), p1 = expf(sc[r + 1] - m_new);
+    psum += p0 + p1;
+    uint16_t h0, l0, h1, l1;
+    split16<DT>(p0, h0, l0);
+    split16<DT>(p1, h1, l1);
+    px[r / 2] = col < G ? (h0 | (static_cast<uint32_t>(h1) << 16)) : (l0 | (static_cast<uint32_t>(l1) << 16));
+  }
+  l = l * alpha + psum;
+  m = m_new;
+  const uint2 pb = make_uint2(px[0], px[1]);
+#pragma unroll
+  for (int s2 = 0; s2 < 8; ++s2) {
+    acc[s2] *= alpha;
+    const uint4 &vr = vreg[s2 / 2];
+    const uint2 va = (s2 & 1) ? make_uint2(vr.z, vr.w) : make_uint2(vr.x, vr.y);
+    acc[s2] = mfma_k16<DT>(va, pb, acc[s2]);
+  }
+}
+
 // W waves per workgroup. A workgroup owns one kv head and one contiguous range of
-// 16-token tiles; wave w takes tiles b0+w, b0+w+W, ... Many waves per workgroup
-// keep the number of split partials (and so the merge) small while the whole KV
-// range is in flight at once: the kernel lives only a few memory latencies.
+// 16-token tiles; wave w takes tiles b0+w, b0+w+W, ...  Both products of a tile run on
+// the matrix cores:
+//   S^T[token][col] = K[token][dim] . Qx[dim][col]   4 x mfma 16x16x32 (contraction: 128 dims)
+//   O^T[dim][col]  += V^T[dim][token] . Px[token][col]   8 x mfma 16x16x16 (one per 16 dims)
+// with 16 columns = G query heads x {hi, lo}: the f32 q (pre-scaled by 1/sqrt(d)) and the f32
+// probabilities are split into two 16-bit parts that occupy columns g and g + G, so products
+// against the 16-bit K/V stay f32-accurate. The S^T result layout (lane = column, 4 tokens of
+// its lane group) is exactly the B-operand layout of the second product, and the O^T
+// accumulators are indexed by the same column, so m, l and the rescale never cross lanes.
+// The cache stores tiles in operand order (kv_k_elem / kv_v_elem): every load is one coalesced
+// 1 KiB instruction and lands in the registers the matrix core reads.
 template <uint32_t DT, int G, int W>
 __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   constexpr int kThreads = W * kWave;
@@ -126,16 +240,9 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
 
   // ---- first tile of every wave: issue its loads before anything else
-  uint4 kreg[4], vreg[4];
+  uint4 kreg[4], vreg[4], kreg1[4], vreg1[4];  // two tiles in flight per wave, roles swap
   uint32_t b = b0 + wave;
-  if (b < b1) {
-    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      kreg[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
-      vreg[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
-    }
-  }
+  if (b < b1) attn_load_tile(p, b, kvh, lane, kreg, vreg);
 
   // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
   for (int g = wave; g < G; g += W) {
@@ -153,124 +260,71 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
     }
   }
   __syncthreads();
-  if (owns_new && wave == 0 && lane < 32) {
-    // publish the rounded row to the cache: 16 lanes x 16 B for K, 16 for V
+  if (owns_new && wave == 0) {
+    // publish the rounded row to the cache in operand order
     const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[new_block], kvh);
-    const int piece = lane & 15;
-    uint16_t *dst = (lane < 16 ? p.k_cache : p.v_cache) + tile + new_row * kHD + piece * 8;
-    const uint16_t *src = (lane < 16 ? knew : vnew) + piece * 8;
-    *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
+    if (lane < 16) {  // K: 16 pieces of 8 consecutive dims
+      *reinterpret_cast<uint4 *>(p.k_cache + tile + kv_k_elem(kHD, new_row, lane * 8)) =
+          *reinterpret_cast<const uint4 *>(knew + lane * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {  // V: one 16-bit element per dim
+      const uint32_t d = lane + i * kWave;
+      p.v_cache[tile + kv_v_elem(kHD, new_row, d)] = vnew[d];
+    }
   }
 
-  const int part = lane & 15, trow = lane >> 4;
+  const int col = lane & 15, grp = lane >> 4;
   const float scale = 1.0f / sqrtf(static_cast<float>(kHD));
 
-  float m[G], l[G], acc[G][8];
+  // B operand of the first product: column `col` of Qx for dims j*32 + grp*8 .. +7
+  uint4 qx[4];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = -INFINITY;
-    l[g] = 0.0f;
+  for (int j = 0; j < 4; ++j) {
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    if (col < 2 * G) {
+      const float *src = &q_s[col < G ? col : col - G][j * 32 + grp * 8];
 #pragma unroll
-    for (int d = 0; d < 8; ++d) acc[g][d] = 0.0f;
+      for (int e = 0; e < 4; ++e) {
+        uint16_t h0, l0, h1, l1;
+        split16<DT>(src[2 * e] * scale, h0, l0);
+        split16<DT>(src[2 * e + 1] * scale, h1, l1);
+        w[e] = col < G ? (h0 | (static_cast<uint32_t>(h1) << 16)) : (l0 | (static_cast<uint32_t>(l1) << 16));
+      }
+    }
+    qx[j] = make_uint4(w[0], w[1], w[2], w[3]);
   }
 
-  for (; b < b1; b += W) {
-    // issue the next tile's loads before touching the current one
-    uint4 knext[4], vnext[4];
-    const uint32_t bn = b + W;
-    if (bn < b1) {
-      const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[bn], kvh);
+  float m = -INFINITY, l = 0.0f;  // of column `col` (both copies of a head track the same values)
+  f32x4_t acc[8];                  // O^T[dims s*16 + grp*4 .. +3][col]
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        knext[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
-        vnext[i] = load_stream(p.v_cache + tile + i * 512 + lane * 8);
-      }
-    }
-    if (owns_new && b == new_block) {
-      // the row written above may not be visible to this CU's loads yet: splice it from LDS
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (static_cast<uint32_t>(i * 4 + trow) == new_row) {
-          kreg[i] = *reinterpret_cast<const uint4 *>(knew + part * 8);
-          vreg[i] = *reinterpret_cast<const uint4 *>(vnew + part * 8);
-        }
-      }
-    }
-    // scores: s[g][i] for token 4i + trow, all G heads share each unpacked K register
-    float s[G][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float kf[8];
-      unpack8<DT>(kreg[i], kf);
-      const bool valid = b * kKvBlockTokens + i * 4 + trow < n_keys;
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const float4 qa = *reinterpret_cast<const float4 *>(&q_s[g][part * 8]);
-        const float4 qb = *reinterpret_cast<const float4 *>(&q_s[g][part * 8 + 4]);
-        float d = qa.x * kf[0];
-        d = fmaf(qa.y, kf[1], d);
-        d = fmaf(qa.z, kf[2], d);
-        d = fmaf(qa.w, kf[3], d);
-        d = fmaf(qb.x, kf[4], d);
-        d = fmaf(qb.y, kf[5], d);
-        d = fmaf(qb.z, kf[6], d);
-        d = fmaf(qb.w, kf[7], d);
-        d = row16_sum(d) * scale;
-        s[g][i] = valid ? d : -INFINITY;
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float mb = fmaxf(fmaxf(s[g][0], s[g][1]), fmaxf(s[g][2], s[g][3]));
-      mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
-      mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
-      const float m_new = fmaxf(m[g], mb);   // finite: every processed tile has a valid token
-      const float alpha = expf(m[g] - m_new);
-      float psum = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        s[g][i] = expf(s[g][i] - m_new);     // scores become probabilities in place
-        psum += s[g][i];
-      }
-      l[g] = l[g] * alpha + psum;
-      m[g] = m_new;
-#pragma unroll
-      for (int d = 0; d < 8; ++d) acc[g][d] *= alpha;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float vf[8];
-      unpack8<DT>(vreg[i], vf);
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(s[g][i], vf[d], acc[g][d]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      kreg[i] = knext[i];
-      vreg[i] = vnext[i];
+  for (int s2 = 0; s2 < 8; ++s2) acc[s2] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  if (b + W < b1) attn_load_tile(p, b + W, kvh, lane, kreg1, vreg1);
+  for (; b < b1; b += 2 * W) {
+    attn_tile<DT, G>(kreg, vreg, qx, b, n_keys, col, grp, owns_new && b == new_block, new_row, knew, vnew, m, l, acc);
+    if (b + 2 * W < b1) attn_load_tile(p, b + 2 * W, kvh, lane, kreg, vreg);
+    if (b + W < b1) {
+      attn_tile<DT, G>(kreg1, vreg1, qx, b + W, n_keys, col, grp, owns_new && b + W == new_block, new_row, knew, vnew, m, l, acc);
+      if (b + 3 * W < b1) attn_load_tile(p, b + 3 * W, kvh, lane, kreg1, vreg1);
     }
   }
 
-  // ---- merge the four token rows of the wave, then the W waves
+  // ---- wave result: tokens of the four lane groups, then hi + lo columns; then the W waves
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    l[g] += __shfl_xor(l[g], 16, kWave);
-    l[g] += __shfl_xor(l[g], 32, kWave);
-#pragma unroll
-    for (int d = 0; d < 8; ++d) {
-      acc[g][d] += __shfl_xor(acc[g][d], 16, kWave);
-      acc[g][d] += __shfl_xor(acc[g][d], 32, kWave);
-    }
-    if (lane < 16) {
-      *reinterpret_cast<float4 *>(&wacc[wave][g][part * 8]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-      *reinterpret_cast<float4 *>(&wacc[wave][g][part * 8 + 4]) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
-    }
-    if (lane == 0) {
-      wm[wave][g] = m[g];
-      wl[wave][g] = l[g];
-    }
+  for (int s2 = 0; s2 < 8; ++s2) {
+    float4 o;
+    o.x = acc[s2][0] + row_shl<G>(acc[s2][0]);
+    o.y = acc[s2][1] + row_shl<G>(acc[s2][1]);
+    o.z = acc[s2][2] + row_shl<G>(acc[s2][2]);
+    o.w = acc[s2][3] + row_shl<G>(acc[s2][3]);
+    if (col < G) *reinterpret_cast<float4 *>(&wacc[wave][col][s2 * 16 + grp * 4]) = o;
+  }
+  if (lane < G) {
+    wm[wave][lane] = m;
+    wl[wave][lane] = l;
   }
   __syncthreads();
   // ---- merge of the W waves: W*G scale factors once, then every thread owns (g, d) pairs
@@ -444,13 +498,13 @@ __global__ __launch_bounds__(kBlock) void attn_generic_kernel(AttnParams p) {
     }
     __syncthreads();
     const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, hd, p.layer,
-                                         p.table[pos / kKvBlockTokens], kvh) +
-                          static_cast<uint64_t>(pos % kKvBlockTokens) * hd;
+                                         p.table[pos / kKvBlockTokens], kvh);
+    const uint32_t prow = pos % kKvBlockTokens;
     for (uint32_t d = threadIdx.x; d < hd; d += kBlock) {
       const uint16_t k16 = enc16<DT>(kn[d]), v16 = enc16<DT>(vn[d]);
       if (h % group == 0) {
-        p.k_cache[tile + d] = k16;
-        p.v_cache[tile + d] = v16;
+        p.k_cache[tile + kv_k_elem(hd, prow, d)] = k16;
+        p.v_cache[tile + kv_v_elem(hd, prow, d)] = v16;
       }
       kn[d] = dec16<DT>(k16);
       vn[d] = dec16<DT>(v16);
@@ -466,12 +520,12 @@ __global__ __launch_bounds__(kBlock) void attn_generic_kernel(AttnParams p) {
   const float scale = 1.0f / sqrtf(static_cast<float>(hd));
   for (uint32_t t = wave; t < n_keys; t += kWavesPerBlock) {
     const bool fresh = p.append && t == pos;
-    const uint64_t row = kv_tile_offset(p.block_count, p.kv_heads, hd, p.layer,
-                                        p.table[t / kKvBlockTokens], kvh) +
-                         static_cast<uint64_t>(t % kKvBlockTokens) * hd;
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, hd, p.layer,
+                                         p.table[t / kKvBlockTokens], kvh);
+    const uint32_t trow = t % kKvBlockTokens;
     float partial = 0.0f;
     for (uint32_t d = lane; d < hd; d += kWave)
-      partial = fmaf(q[d], fresh ? kn[d] : dec16<DT>(p.k_cache[row + d]), partial);
+      partial = fmaf(q[d], fresh ? kn[d] : dec16<DT>(p.k_cache[tile + kv_k_elem(hd, trow, d)]), partial);
     const float score = wave_sum(partial) * scale;
     const float m_new = fmaxf(m, score);
     const float alpha = l == 0.0f ? 0.0f : expf(m - m_new);
@@ -479,7 +533,7 @@ __global__ __launch_bounds__(kBlock) void attn_generic_kernel(AttnParams p) {
 #pragma unroll
     for (int j = 0; j < kMaxPerLane; ++j) {
       const uint32_t d = lane + j * kWave;
-      if (d < hd) acc[j] = acc[j] * alpha + (fresh ? vn[d] : dec16<DT>(p.v_cache[row + d])) * pnew;
+      if (d < hd) acc[j] = acc[j] * alpha + (fresh ? vn[d] : dec16<DT>(p.v_cache[tile + kv_v_elem(hd, trow, d)])) * pnew;
     }
     l = l * alpha + pnew;
     m = m_new;

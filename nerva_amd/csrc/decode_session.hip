@@ -1175,21 +1175,6 @@ int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *s, float *hos
   return hipMemcpy(host_logits, s->logits, static_cast<uint64_t>(s->vocab) * 4, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
 }
 
-int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t token,
-                              uint16_t *host_k, uint16_t *host_v) {
-  if (s == nullptr || host_k == nullptr || host_v == nullptr || layer >= s->layers || token >= s->max_ctx)
-    return -1;
-  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
-  const uint32_t block = token / kKvBlockTokens, row = token % kKvBlockTokens;  // identity table
-  for (uint32_t h = 0; h < s->kv_heads; ++h) {
-    const uint64_t off = kv_tile_offset(s->block_count, s->kv_heads, s->head_dim, layer, block, h) +
-                         static_cast<uint64_t>(row) * s->head_dim;
-    if (hipMemcpy(host_k + h * s->head_dim, s->kc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
-    if (hipMemcpy(host_v + h * s->head_dim, s->vc + off, s->head_dim * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  }
-  return 0;
-}
-
 int nerva_hip_session_read_kv_range(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t first_token,
                                     uint32_t token_count, uint16_t *host_k, uint16_t *host_v) {
   if (s == nullptr || host_k == nullptr || host_v == nullptr || layer >= s->layers ||
@@ -1206,15 +1191,30 @@ int nerva_hip_session_read_kv_range(NervaHipHfDecodeSequenceSession *s, uint32_t
   const uint64_t off = kv_tile_offset(s->block_count, kvh, hd, layer, b0, 0);
   if (hipMemcpy(kimg.data(), s->kc + off, kimg.size() * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
   if (hipMemcpy(vimg.data(), s->vc + off, vimg.size() * 2, hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  // in-tile element order of one row, computed once per row index
+  std::vector<uint32_t> kmap(kKvBlockTokens * hd), vmap(kKvBlockTokens * hd);
+  for (uint32_t row = 0; row < kKvBlockTokens; ++row)
+    for (uint32_t d = 0; d < hd; ++d) {
+      kmap[row * hd + d] = kv_k_elem(hd, row, d);
+      vmap[row * hd + d] = kv_v_elem(hd, row, d);
+    }
   for (uint32_t t = 0; t < token_count; ++t) {
     const uint32_t tok = first_token + t, blk = tok / kKvBlockTokens - b0, row = tok % kKvBlockTokens;
     for (uint32_t h = 0; h < kvh; ++h) {
-      const uint64_t src = (static_cast<uint64_t>(blk) * kvh + h) * kKvBlockTokens * hd + static_cast<uint64_t>(row) * hd;
-      memcpy(host_k + t * KV + h * hd, kimg.data() + src, hd * 2);
-      memcpy(host_v + t * KV + h * hd, vimg.data() + src, hd * 2);
+      const uint64_t tile = (static_cast<uint64_t>(blk) * kvh + h) * kKvBlockTokens * hd;
+      uint16_t *dk = host_k + t * KV + h * hd, *dv = host_v + t * KV + h * hd;
+      for (uint32_t d = 0; d < hd; ++d) {
+        dk[d] = kimg[tile + kmap[row * hd + d]];
+        dv[d] = vimg[tile + vmap[row * hd + d]];
+      }
     }
   }
   return 0;
+}
+
+int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t token,
+                              uint16_t *host_k, uint16_t *host_v) {
+  return nerva_hip_session_read_kv_range(s, layer, token, 1, host_k, host_v);
 }
 
 }  // extern "C"

@@ -322,9 +322,10 @@ uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head
 
 uint64_t nerva_hip_kv_cache_offset(uint32_t block_count, uint32_t kv_heads, uint32_t head_dim,
                                    uint32_t layer, uint32_t physical_block, uint32_t kv_head,
-                                   uint32_t token_in_block) {
+                                   uint32_t token_in_block, uint32_t dim, uint32_t is_value) {
+  if (token_in_block >= kKvBlockTokens || dim >= head_dim) return ~uint64_t{0};
   return kv_tile_offset(block_count, kv_heads, head_dim, layer, physical_block, kv_head) +
-         static_cast<uint64_t>(token_in_block) * head_dim;
+         (is_value ? kv_v_elem(head_dim, token_in_block, dim) : kv_k_elem(head_dim, token_in_block, dim));
 }
 
 int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *r, void *stream,

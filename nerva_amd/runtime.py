@@ -136,7 +136,7 @@ def fp8_gemv(weights, scales, rows, cols, block_rows, block_cols, out, *, input1
 
 
 class PagedKvCache:
-    """K/V arrays in the library's layout [layer][block][kv_head][16][head_dim] + a block table."""
+    """K/V arrays in the library's layout [layer][block][kv_head][16-token tile] + a block table."""
 
     def __init__(self, layers, block_count, kv_heads, head_dim, table=None):
         self.layers, self.block_count, self.kv_heads, self.head_dim = layers, block_count, kv_heads, head_dim
@@ -147,22 +147,39 @@ class PagedKvCache:
         self.table_host = table
         self.table = DeviceBuffer.from_numpy(table)
 
-    def offset(self, layer, token, kv_head):
+    def tile_offset(self, layer, token, kv_head):
+        """Element offset of the (block, kv_head) tile that holds `token`."""
         lib = abi.load()
         return int(lib.nerva_hip_kv_cache_offset(self.block_count, self.kv_heads, self.head_dim, layer,
-                                                 int(self.table_host[token // 16]), kv_head, token % 16))
+                                                 int(self.table_host[token // 16]), kv_head, 0, 0, 0))
+
+    def _tile_maps(self):
+        """In-tile element index of (row, dim) for K and V, as the library lays tiles out."""
+        if getattr(self, "_maps", None) is None:
+            lib = abi.load()
+            hd = self.head_dim
+            kmap = np.empty((16, hd), np.int64)
+            vmap = np.empty((16, hd), np.int64)
+            for row in range(16):
+                for d in range(hd):
+                    kmap[row, d] = lib.nerva_hip_kv_cache_offset(1, 1, hd, 0, 0, 0, row, d, 0)
+                    vmap[row, d] = lib.nerva_hip_kv_cache_offset(1, 1, hd, 0, 0, 0, row, d, 1)
+            assert sorted(kmap.ravel()) == list(range(16 * hd)) and sorted(vmap.ravel()) == list(range(16 * hd))
+            self._maps = (kmap, vmap)
+        return self._maps
 
     def host_layout(self, layer, k_rows, v_rows):
         """Scatter [tokens, kv_heads*head_dim] 16-bit rows into host images of the cache arrays."""
         kimg = np.zeros(self.elems, np.uint16)
         vimg = np.zeros(self.elems, np.uint16)
+        kmap, vmap = self._tile_maps()
         tokens = k_rows.shape[0]
         hd = self.head_dim
         for t in range(tokens):
             for h in range(self.kv_heads):
-                o = self.offset(layer, t, h)
-                kimg[o:o + hd] = k_rows[t, h * hd:(h + 1) * hd]
-                vimg[o:o + hd] = v_rows[t, h * hd:(h + 1) * hd]
+                o = self.tile_offset(layer, t, h)
+                kimg[o + kmap[t % 16]] = k_rows[t, h * hd:(h + 1) * hd]
+                vimg[o + vmap[t % 16]] = v_rows[t, h * hd:(h + 1) * hd]
         return kimg, vimg
 
     def fill(self, layer, k_rows, v_rows):
@@ -172,12 +189,15 @@ class PagedKvCache:
 
     def read_row(self, layer, token):
         hd = self.head_dim
+        kmap, vmap = self._tile_maps()
         k = np.empty(self.kv_heads * hd, np.uint16)
         v = np.empty(self.kv_heads * hd, np.uint16)
         for h in range(self.kv_heads):
-            o = self.offset(layer, token, h)
-            k[h * hd:(h + 1) * hd] = self.k.numpy(np.uint16, hd, o * 2)
-            v[h * hd:(h + 1) * hd] = self.v.numpy(np.uint16, hd, o * 2)
+            o = self.tile_offset(layer, token, h)
+            ktile = self.k.numpy(np.uint16, 16 * hd, o * 2)
+            vtile = self.v.numpy(np.uint16, 16 * hd, o * 2)
+            k[h * hd:(h + 1) * hd] = ktile[kmap[token % 16]]
+            v[h * hd:(h + 1) * hd] = vtile[vmap[token % 16]]
         return k, v
 
 

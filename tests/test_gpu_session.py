@@ -180,8 +180,13 @@ GEOMETRIES = [
 @pytest.mark.parametrize("geom", GEOMETRIES)
 def test_single_layer_short_prompt_is_tight(geom):
     """One layer and a 1- or 2-token prompt leave no room for 16-bit ties to compound: the whole
-    step (embed, norms, GEMVs, RoPE, attention, LM head) must agree with the oracle at 1e-3."""
+    step (embed, norms, GEMVs, RoPE, attention, LM head) must agree with the oracle at 1e-3 in
+    f16. In bf16 a single value that sits within 1e-6 of a rounding boundary (attention output,
+    SwiGLU output and norm outputs are rounded to 16 bit) may land on the other side, which moves
+    one activation by 2^-8 relative and the logits of this tiny model by up to ~3e-3: the bound
+    is one such flip, 6e-3."""
     dtype, hidden, heads, kv, hd, inter, vocab, _, theta, qk_norm, bias = geom
+    tol = REL_L2 if dtype == F16 else 6e-3
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, 1, hidden + 1, theta, qk_norm, bias)
     s = N.DecodeSession.create(weights, 32)
     for prompt in ([3], [vocab - 1, 11]):
@@ -190,7 +195,7 @@ def test_single_layer_short_prompt_is_tight(geom):
             ctx.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
         rc, res = s.start(prompt)
         assert rc == 0
-        assert rel_l2(s.logits(), ctx.logits()) <= REL_L2
+        assert rel_l2(s.logits(), ctx.logits()) <= tol
         gk, gv = s.kv_row(0, len(prompt) - 1)
         rk, rv = ctx.read_kv16(0, len(prompt) - 1)
         # summation order may move a value across a 16-bit tie: at most one unit, on few elements
