@@ -116,6 +116,17 @@ __device__ __forceinline__ void split16(float v, uint16_t &hi, uint16_t &lo) {
   lo = enc16<DT>(v - dec16<DT>(hi));
 }
 
+// Device-scope coherent accesses: written through / read around the XCD-local L2, so data
+// exchanged between workgroups inside one kernel needs no cache flush or invalidate.
+__device__ __forceinline__ void store_coherent(float *ptr, float v) {
+  __hip_atomic_store(ptr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float *ptr) {
+  return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Returns when every store this wave has issued has been performed.
+__device__ __forceinline__ void wait_stores_performed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Requests one (block, kv head) tile: four 1 KiB loads each for K and V.
 __device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t b, uint32_t kvh, int lane,
                                                uint4 (&k)[4], uint4 (&v)[4]) {
@@ -329,8 +340,7 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   __syncthreads();
   // ---- merge of the W waves: W*G scale factors once, then every thread owns (g, d) pairs
   __shared__ float wf[W][G];    // exp(m_w - M_g), 0 for idle waves
-  __shared__ float bM[G], bL[G];
-  __shared__ __align__(16) float bacc[G][kHD];
+  __shared__ float bM[G];
   if (threadIdx.x < W * G) {
     const int w = threadIdx.x / G, g = threadIdx.x % G;
     float M = -INFINITY;
@@ -355,68 +365,58 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
       if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
       p.out16[h * kHD + d] = enc16<DT>(o);
     } else {
-      bacc[g][d] = o;
-      if (d == 0) bL[g] = L;
+      // The partial leaves through device-coherent stores (written through, no cache flush).
+      store_coherent(p.part_acc + (static_cast<uint64_t>(h) * S + split) * kHD + d, o);
+      if (d == 0) {
+        store_coherent(p.part_m + h * S + split, bM[g]);
+        store_coherent(p.part_l + h * S + split, L);
+      }
     }
   }
   if (active == 1) return;
+  // Every wave waits until its own stores have been performed, the barrier collects the waves,
+  // and only then one lane takes the arrival ticket of this kv head.
+  wait_stores_performed();
   __syncthreads();
-  // The workgroup's partial leaves through ONE wave, which then releases it to device
-  // scope once and takes the arrival ticket: one fence per workgroup.
-  if (wave == 0) {
-    for (int e = lane; e < G * kHD; e += kWave) {
-      const int g = e / kHD, d = e % kHD;
-      const uint32_t h = kvh * G + g;
-      p.part_acc[(static_cast<uint64_t>(h) * S + split) * kHD + d] = bacc[g][d];
-      if (d == 0) {
-        p.part_m[h * S + split] = bM[g];
-        p.part_l[h * S + split] = bL[g];
-      }
-    }
-    __threadfence();
-    if (lane == 0) {
-      const uint32_t ticket =
-          __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      is_last = ticket == active - 1 ? 1u : 0u;
-    }
+  if (threadIdx.x == 0) {
+    const uint32_t ticket =
+        __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = ticket == active - 1 ? 1u : 0u;
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();  // acquire: the other workgroups' partials
-  // ---- the last workgroup of this kv head merges the splits: factors once, then (g, d) pairs
-  __shared__ float sf[kAttnMaxSplits][G];   // exp(m_s - M_g) / L_g
-  __shared__ float sm_[kAttnMaxSplits][G], sl_[kAttnMaxSplits][G];
-  for (uint32_t e = threadIdx.x; e < active * G; e += kThreads) {
-    const uint32_t s2 = e / G, g = e % G;
-    const uint32_t h = kvh * G + g;
-    sm_[s2][g] = p.part_m[h * S + s2];
-    sl_[s2][g] = p.part_l[h * S + s2];
-  }
-  __syncthreads();
-  for (uint32_t e = threadIdx.x; e < active * G; e += kThreads) {
-    const uint32_t s2 = e / G, g = e % G;
-    float M = -INFINITY;
-    for (uint32_t t = 0; t < active; ++t) M = fmaxf(M, sm_[t][g]);
-    float L = 0.0f;
-    for (uint32_t t = 0; t < active; ++t) L = fmaf(sl_[t][g], expf(sm_[t][g] - M), L);
-    const float f = expf(sm_[s2][g] - M);
-    sf[s2][g] = (L > 0.0f && isfinite(L)) ? f / L : f;
-  }
-  __syncthreads();
+  // ---- the last workgroup of this kv head merges the splits. Each thread owns (g, d) and reads
+  // the partials with device-coherent loads, sixteen splits per round trip, in split order.
   for (int e = threadIdx.x; e < G * kHD; e += kThreads) {
     const int g = e / kHD, d = e % kHD;
     const uint32_t h = kvh * G + g;
+    const float *pm = p.part_m + h * S, *pl = p.part_l + h * S;
     const float *src = p.part_acc + static_cast<uint64_t>(h) * S * kHD + d;
-    float o = 0.0f;
-    uint32_t s2 = 0;
-    for (; s2 + 4 <= active; s2 += 4) {
-      const float a0 = src[(s2 + 0) * kHD], a1 = src[(s2 + 1) * kHD], a2 = src[(s2 + 2) * kHD], a3 = src[(s2 + 3) * kHD];
-      o = fmaf(a0, sf[s2 + 0][g], o);
-      o = fmaf(a1, sf[s2 + 1][g], o);
-      o = fmaf(a2, sf[s2 + 2][g], o);
-      o = fmaf(a3, sf[s2 + 3][g], o);
+    float M = -INFINITY, L = 0.0f, o = 0.0f;
+    for (uint32_t s0 = 0; s0 < active; s0 += 16) {
+      float mm[16], ll[16], aa[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool on = s0 + i < active;
+        mm[i] = on ? load_coherent(pm + s0 + i) : -INFINITY;
+        ll[i] = on ? load_coherent(pl + s0 + i) : 0.0f;
+        aa[i] = on ? load_coherent(src + static_cast<uint64_t>(s0 + i) * kHD) : 0.0f;
+      }
+      float Mc = M;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) Mc = fmaxf(Mc, mm[i]);
+      const float keep = M > -INFINITY ? expf(M - Mc) : 0.0f;
+      L *= keep;
+      o *= keep;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float f = mm[i] > -INFINITY ? expf(mm[i] - Mc) : 0.0f;
+        L = fmaf(ll[i], f, L);
+        o = fmaf(aa[i], f, o);
+      }
+      M = Mc;
     }
-    for (; s2 < active; ++s2) o = fmaf(src[s2 * kHD], sf[s2][g], o);
+    if (L > 0.0f && isfinite(L)) o /= L;
     if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
     p.out16[h * kHD + d] = enc16<DT>(o);
   }
