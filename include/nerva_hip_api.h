@@ -498,6 +498,14 @@ int nerva_hip_memset(void *device_dst, int value, uint64_t bytes);
 int nerva_hip_stream_synchronize(void *stream);
 /* Counts hipMalloc/hipHostMalloc calls made by the library since load (hot-path allocation audit). */
 uint64_t nerva_hip_allocation_count(void);
+/* Operator timing (no reference counterpart). Between begin and end, device-pointer operator
+ * calls made with a null stream are recorded, not run; end turns them into one hipGraph, replays
+ * it `warmup_replays` + `timed_replays` times and reports the average device time of a replay
+ * (hipEvents on the library stream). Only launches may be issued in between: no copies, no
+ * allocation, no synchronisation. One recording at a time, one host thread. */
+int nerva_hip_timer_capture_begin(void);
+int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
+                                double *avg_replay_ns);
 /* Plain device-to-device copy kernel (16-byte aligned pointers and size): moves exactly `bytes`
  * in and `bytes` out, the known-size transfer memory counters are calibrated against. */
 int nerva_hip_copy_d2d(void *device_dst, const void *device_src, uint64_t bytes, void *stream);

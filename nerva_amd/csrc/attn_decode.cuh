@@ -55,6 +55,14 @@ struct AttnParams {
   uint32_t position, max_steps, append;
 };
 
+// Split-KV factor: every active split adds a partial for the last workgroup of its kv head to
+// merge, so the grid is kept to about 128 workgroups of 8 waves (kv_heads x splits).
+inline uint32_t attn_default_splits(uint32_t kv_heads, uint32_t block_count) {
+  uint32_t splits = (128 + kv_heads - 1) / (kv_heads == 0 ? 1 : kv_heads);
+  if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
+  if (splits > block_count) splits = block_count;
+  return splits == 0 ? 1 : splits;
+}
 uint64_t attn_workspace_bytes(uint32_t heads, uint32_t head_dim);
 // Carves part_acc/part_m/part_l/counters out of a workspace of attn_workspace_bytes().
 void attn_bind_workspace(AttnParams &p, void *workspace);

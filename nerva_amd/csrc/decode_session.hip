@@ -557,15 +557,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->planned_gpu_staged_weight_bytes = rq->planned_gpu_staged_weight_bytes;
   s->planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
   s->planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
-  // Split-KV factor of the decode attention. Every active split costs a device-scope
-  // release + an arrival ticket + one more partial for the last workgroup to merge
-  // (~0.4 us each, measured), so the grid is kept to ~128 workgroups of 8 waves.
-  {
-    uint32_t splits = (128 + rq->kv_heads - 1) / rq->kv_heads;
-    splits = std::min(splits, kAttnMaxSplits);
-    splits = std::min(splits, std::max(1u, block_count));
-    s->attn_splits = std::max(1u, splits);
-  }
+  s->attn_splits = attn_default_splits(rq->kv_heads, block_count);
 
   // ---- arena layout ------------------------------------------------------
   struct LayerOff {

@@ -202,6 +202,203 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Lean MoE kernels for the production shapes (hidden, inter multiples of 1024; block a
+// multiple of 16; 16-byte aligned weights). Same arithmetic as the kernels above; the
+// difference is the request pipeline: a wave walks a flat list of batches (one 1 KiB
+// chunk of each of its two rows, plus the two block scales) with four batches in
+// flight in four register buffers that are refilled as soon as they are consumed
+// (fully unrolled, no register copies), so rows, and in the down kernel experts,
+// follow each other without a bubble.
+// ---------------------------------------------------------------------------
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Params p) {
+  extern __shared__ __align__(16) float xsf[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const uint32_t units = slots * p.inter;
+  const uint32_t sc_cols = (p.hidden + p.block - 1) / p.block;
+  const uint64_t scale_stride = static_cast<uint64_t>((p.inter + p.block - 1) / p.block) * sc_cols;
+  const uint64_t w_stride = static_cast<uint64_t>(p.inter) * p.hidden;
+  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
+  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
+  const uint32_t bpr = p.hidden / 1024u;
+  const uint32_t my_units = wave_global < units ? (units - wave_global + wave_stride - 1) / wave_stride : 0u;
+  const uint32_t total = my_units * bpr;
+
+  uint32_t iu = wave_global, ib = 0;
+  const uint8_t *wg = nullptr, *wu = nullptr;
+  const float *sg = nullptr, *su = nullptr;
+  uint4 bg0, bg1, bg2, bg3, bu0, bu1, bu2, bu3;
+  float fg0, fg1, fg2, fg3, fu0, fu1, fu2, fu3;
+#define NV_GU_ISSUE(J)                                                                        \
+  do {                                                                                        \
+    if (ib == 0) {                                                                            \
+      const uint32_t k = iu / p.inter, i = iu % p.inter;                                      \
+      uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);     \
+      if (e >= p.num_experts) e = 0;                                                          \
+      const uint64_t row = e * w_stride + static_cast<uint64_t>(i) * p.hidden + lane * 16;    \
+      wg = p.w_gate + row;                                                                    \
+      wu = p.w_up + row;                                                                      \
+      const uint64_t srow = e * scale_stride + static_cast<uint64_t>(i / p.block) * sc_cols;  \
+      sg = p.s_gate + srow;                                                                   \
+      su = p.s_up + srow;                                                                     \
+    }                                                                                         \
+    bg##J = load_stream(wg + ib * 1024u);                                                     \
+    bu##J = load_stream(wu + ib * 1024u);                                                     \
+    fg##J = sg[(ib * 1024u + lane * 16) / p.block];                                           \
+    fu##J = su[(ib * 1024u + lane * 16) / p.block];                                           \
+    if (++ib == bpr) {                                                                        \
+      ib = 0;                                                                                 \
+      iu += wave_stride;                                                                      \
+    }                                                                                         \
+  } while (0)
+
+  uint32_t cu = wave_global, cb = 0;
+  float ag = 0.0f, au = 0.0f;
+#define NV_GU_CONSUME(J)                                                                      \
+  do {                                                                                        \
+    const float *xp = xsf + cb * 1024u + lane * 16;                                           \
+    ag = fmaf(fg##J, dot16_fp8(bg##J, xp), ag);                                               \
+    au = fmaf(fu##J, dot16_fp8(bu##J, xp), au);                                               \
+    if (++cb == bpr) {                                                                        \
+      cb = 0;                                                                                 \
+      const float g = wave_sum(ag), u = wave_sum(au);                                         \
+      if (lane == 0) p.act[cu] = silu(g) * u; /* act is [slot][inter] = flat unit index */    \
+      ag = 0.0f;                                                                              \
+      au = 0.0f;                                                                              \
+      cu += wave_stride;                                                                      \
+    }                                                                                         \
+  } while (0)
+
+  // requests first, then x -> LDS, then the ring
+  if (total > 0) NV_GU_ISSUE(0);
+  if (total > 1) NV_GU_ISSUE(1);
+  if (total > 2) NV_GU_ISSUE(2);
+  if (total > 3) NV_GU_ISSUE(3);
+  stage_x<DT>(xsf, p.x16, nullptr, p.hidden);
+  __syncthreads();
+  for (uint32_t t = 0; t < total; t += 4) {
+    NV_GU_CONSUME(0);
+    if (t + 4 < total) NV_GU_ISSUE(0);
+    if (t + 1 < total) {
+      NV_GU_CONSUME(1);
+      if (t + 5 < total) NV_GU_ISSUE(1);
+    }
+    if (t + 2 < total) {
+      NV_GU_CONSUME(2);
+      if (t + 6 < total) NV_GU_ISSUE(2);
+    }
+    if (t + 3 < total) {
+      NV_GU_CONSUME(3);
+      if (t + 7 < total) NV_GU_ISSUE(3);
+    }
+  }
+#undef NV_GU_ISSUE
+#undef NV_GU_CONSUME
+}
+
+// Down + combine, lean: the wave owns output rows 2u and 2u+1 and walks (expert, chunk)
+// batches; act[k] goes through a two-slot LDS buffer one expert ahead of its use.
+__global__ __launch_bounds__(kBlock, 4) void moe_down_lean_kernel(MoeFp8Params p) {
+  extern __shared__ __align__(16) float acts[];  // 2 x inter floats
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const uint32_t sc_cols = (p.inter + p.block - 1) / p.block;
+  const uint64_t scale_stride = static_cast<uint64_t>((p.hidden + p.block - 1) / p.block) * sc_cols;
+  const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * p.inter;
+  const uint32_t unit = blockIdx.x * kWavesPerBlock + wave;  // the grid covers all row pairs exactly
+  const uint32_t h0 = min(unit * 2, p.hidden - 1), h1 = min(unit * 2 + 1, p.hidden - 1);
+  const uint32_t bpe = p.inter / 1024u;       // batches per expert
+  const uint32_t total = slots * bpe;
+
+  uint32_t ik = 0, ib = 0;
+  const uint8_t *w0 = nullptr, *w1 = nullptr;
+  const float *s0 = nullptr, *s1 = nullptr;
+  uint4 ba0, ba1, ba2, ba3, bb0, bb1, bb2, bb3;
+  float fa0, fa1, fa2, fa3, fb0, fb1, fb2, fb3;
+#define NV_DN_ISSUE(J)                                                                        \
+  do {                                                                                        \
+    if (ib == 0) {                                                                            \
+      uint32_t e = ik < p.top_k ? p.expert_ids[ik] : static_cast<uint32_t>(p.shared_index);   \
+      if (e >= p.num_experts) e = 0;                                                          \
+      w0 = p.w_down + e * w_stride + static_cast<uint64_t>(h0) * p.inter + lane * 16;         \
+      w1 = p.w_down + e * w_stride + static_cast<uint64_t>(h1) * p.inter + lane * 16;         \
+      s0 = p.s_down + e * scale_stride + static_cast<uint64_t>(h0 / p.block) * sc_cols;       \
+      s1 = p.s_down + e * scale_stride + static_cast<uint64_t>(h1 / p.block) * sc_cols;       \
+    }                                                                                         \
+    ba##J = load_stream(w0 + ib * 1024u);                                                     \
+    bb##J = load_stream(w1 + ib * 1024u);                                                     \
+    fa##J = s0[(ib * 1024u + lane * 16) / p.block];                                           \
+    fb##J = s1[(ib * 1024u + lane * 16) / p.block];                                           \
+    if (++ib == bpe) {                                                                        \
+      ib = 0;                                                                                 \
+      ++ik;                                                                                   \
+    }                                                                                         \
+  } while (0)
+
+  uint32_t ck = 0, cb = 0;
+  float a0 = 0.0f, a1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
+#define NV_DN_STAGE(K)                                                                        \
+  do {                                                                                        \
+    float *dst_ = acts + ((K) & 1u) * p.inter;                                                \
+    for (uint32_t c = threadIdx.x * 4; c < p.inter; c += kBlock * 4)                          \
+      *reinterpret_cast<float4 *>(dst_ + c) =                                                 \
+          *reinterpret_cast<const float4 *>(p.act + static_cast<uint64_t>(K) * p.inter + c);  \
+  } while (0)
+#define NV_DN_CONSUME(J)                                                                      \
+  do {                                                                                        \
+    if (cb == 0) {                                                                            \
+      /* expert ck starts: its activations were staged one expert ago; stage the next */     \
+      __syncthreads();                                                                        \
+      if (ck + 1 < slots) NV_DN_STAGE(ck + 1);                                                \
+    }                                                                                         \
+    const float *xp = acts + (ck & 1u) * p.inter + cb * 1024u + lane * 16;                    \
+    a0 = fmaf(fa##J, dot16_fp8(ba##J, xp), a0);                                               \
+    a1 = fmaf(fb##J, dot16_fp8(bb##J, xp), a1);                                               \
+    if (++cb == bpe) {                                                                        \
+      cb = 0;                                                                                 \
+      const float weight = ck < p.top_k ? p.expert_weights[ck] : 1.0f;                        \
+      t0 = fmaf(weight, wave_sum(a0), t0);                                                    \
+      t1 = fmaf(weight, wave_sum(a1), t1);                                                    \
+      a0 = 0.0f;                                                                              \
+      a1 = 0.0f;                                                                              \
+      ++ck;                                                                                   \
+    }                                                                                         \
+  } while (0)
+
+  if (total > 0) NV_DN_ISSUE(0);
+  if (total > 1) NV_DN_ISSUE(1);
+  if (total > 2) NV_DN_ISSUE(2);
+  if (total > 3) NV_DN_ISSUE(3);
+  NV_DN_STAGE(0u);
+  for (uint32_t t = 0; t < total; t += 4) {
+    NV_DN_CONSUME(0);
+    if (t + 4 < total) NV_DN_ISSUE(0);
+    if (t + 1 < total) {
+      NV_DN_CONSUME(1);
+      if (t + 5 < total) NV_DN_ISSUE(1);
+    }
+    if (t + 2 < total) {
+      NV_DN_CONSUME(2);
+      if (t + 6 < total) NV_DN_ISSUE(2);
+    }
+    if (t + 3 < total) {
+      NV_DN_CONSUME(3);
+      if (t + 7 < total) NV_DN_ISSUE(3);
+    }
+  }
+#undef NV_DN_ISSUE
+#undef NV_DN_CONSUME
+#undef NV_DN_STAGE
+  if (lane == 0) {
+    if (unit * 2 < p.hidden) p.out[unit * 2] = t0;
+    if (unit * 2 + 1 < p.hidden) p.out[unit * 2 + 1] = t1;
+  }
+}
+
 // softmax over E logits, top-k by (probability desc, index asc), optional
 // renormalisation (precision/block/moe.rs:1107-1155,1254-1268,1303-1326).
 // One workgroup; E <= 1024. Selection is k rounds of a block-wide argmax.
@@ -325,7 +522,15 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t blocks =
         static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 32u));
     const size_t lds = static_cast<size_t>(p.hidden) * sizeof(float);
-    if (p.input_dtype == kBF16) {
+    if (fast_gu && aligned16(p.act)) {
+      // lean kernel: oversubscribed persistent-style grid, 8 workgroups per CU at most
+      const uint32_t lean_blocks =
+          static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u));
+      if (p.input_dtype == kBF16)
+        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kBF16>), dim3(lean_blocks), dim3(kBlock), lds, stream, p);
+      else
+        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kF16>), dim3(lean_blocks), dim3(kBlock), lds, stream, p);
+    } else if (p.input_dtype == kBF16) {
       if (fast_gu) hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
       else hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
     } else {
@@ -340,7 +545,9 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t units = (p.hidden + NR - 1) / NR;
     const uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
     const size_t lds = static_cast<size_t>(p.inter) * 2 * sizeof(float);
-    if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    if (fast_dn && aligned16(p.act) && p.inter % 4u == 0)
+      hipLaunchKernelGGL(moe_down_lean_kernel, dim3(blocks), dim3(kBlock), lds, stream, p);
+    else if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
     else hipLaunchKernelGGL((moe_down_kernel<NR, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
   }
   return hipGetLastError();

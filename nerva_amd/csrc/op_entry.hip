@@ -255,6 +255,57 @@ int nerva_hip_copy_d2d(void *device_dst, const void *device_src, uint64_t bytes,
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+// ---- operator timing: launches recorded between begin and end become one hipGraph ---------
+namespace {
+struct OpTimer {
+  bool capturing = false;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+} g_timer;
+void timer_drop_graph() {
+  if (g_timer.exec) (void)hipGraphExecDestroy(g_timer.exec);
+  if (g_timer.graph) (void)hipGraphDestroy(g_timer.graph);
+  g_timer.exec = nullptr;
+  g_timer.graph = nullptr;
+}
+}  // namespace
+
+int nerva_hip_timer_capture_begin(void) {
+  int32_t e = 0;
+  if (!device_ready(&e) || g_timer.capturing) return -1;
+  timer_drop_graph();
+  if (hipStreamSynchronize(library_stream()) != hipSuccess) return -1;
+  if (hipStreamBeginCapture(library_stream(), hipStreamCaptureModeThreadLocal) != hipSuccess) return -1;
+  g_timer.capturing = true;
+  return 0;
+}
+
+int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
+                                double *avg_replay_ns) {
+  if (!g_timer.capturing) return -1;
+  g_timer.capturing = false;
+  hipStream_t s = library_stream();
+  hipError_t err = hipStreamEndCapture(s, &g_timer.graph);
+  size_t count = 0;
+  if (err == hipSuccess) err = hipGraphGetNodes(g_timer.graph, nullptr, &count);
+  if (err == hipSuccess) err = hipGraphInstantiate(&g_timer.exec, g_timer.graph, nullptr, nullptr, 0);
+  if (err == hipSuccess && g_timer.e0 == nullptr) err = hipEventCreate(&g_timer.e0);
+  if (err == hipSuccess && g_timer.e1 == nullptr) err = hipEventCreate(&g_timer.e1);
+  for (uint32_t i = 0; err == hipSuccess && i < warmup_replays; ++i) err = hipGraphLaunch(g_timer.exec, s);
+  if (err == hipSuccess) err = hipEventRecord(g_timer.e0, s);
+  for (uint32_t i = 0; err == hipSuccess && i < timed_replays; ++i) err = hipGraphLaunch(g_timer.exec, s);
+  if (err == hipSuccess) err = hipEventRecord(g_timer.e1, s);
+  if (err == hipSuccess) err = hipEventSynchronize(g_timer.e1);
+  float ms = 0.0f;
+  if (err == hipSuccess) err = hipEventElapsedTime(&ms, g_timer.e0, g_timer.e1);
+  timer_drop_graph();
+  if (err != hipSuccess || timed_replays == 0) return -1;
+  if (nodes) *nodes = count;
+  if (avg_replay_ns) *avg_replay_ns = static_cast<double>(ms) * 1e6 / timed_replays;
+  return 0;
+}
+
 int nerva_hip_synth_fill_16(void *device_dst, uint32_t dtype, uint64_t seed, uint64_t tensor_id,
                             uint64_t count, float mean, float std) {
   hipStream_t s = library_stream();
@@ -370,7 +421,7 @@ int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *r, void *str
   p.out16 = r->output16;
   p.layer = r->layer;
   p.block_count = r->block_count;
-  p.splits = kAttnMaxSplits;
+  p.splits = attn_default_splits(r->kv_heads, r->block_count);
   p.eps = r->rms_eps;
   p.cursor = nullptr;
   p.position = r->position;

@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Operator-level measurements of the decode path on one MI355X:
+
+  1. q_proj GEMV 4096x4096 bf16
+  2. MLP block (RMSNorm -> gate/up GEMV -> SwiGLU -> down GEMV -> +residual), hidden 4096, MLP 12288
+  3. paged GQA decode attention, 32 q / 8 kv heads x 128, 4096 cached tokens + the new one
+  4. FP8 (e4m3, 128x128 block scales) MoE: 8 routed + 1 shared expert, hidden 7168, MLP 2048
+
+Each case is timed twice: "rotating" cycles through enough distinct copies of the weights / cache that
+the working set exceeds 1 GB (nothing is served from cache), "resident" repeats one copy. The launches
+of a case are recorded into one hipGraph and replayed; time is hipEvents around the replays. Bandwidth
+is algorithmic bytes (weights + vectors in and out, intermediates excluded) over time, against the
+8 TB/s HBM peak. Run: python -m nerva_amd.opbench
+"""
+import ctypes as C
+import os
+import sys
+import time
+
+import numpy as np
+
+from . import abi, runtime as R
+from .runtime import DeviceBuffer, Device
+
+BF16 = 1
+SEED = 0x4E45525641
+PEAK = 8000.0
+
+
+def log(*a):
+    print(*a, flush=True)
+
+
+def synth16(count, tid, mean=0.0, std=0.02):
+    buf = DeviceBuffer(count * 2)
+    assert abi.load().nerva_hip_synth_fill_16(buf.ptr, BF16, SEED, tid, count, mean, std) == 0
+    return buf
+
+
+def synth32(count, tid, std=1.0):
+    buf = DeviceBuffer(count * 4)
+    assert abi.load().nerva_hip_synth_fill_f32(buf.ptr, SEED, tid, count, 0.0, std) == 0
+    return buf
+
+
+def timed(enqueue, launches, warmup=3, replays=10):
+    """enqueue(i) issues the i-th launch group; returns average ns per group."""
+    lib = abi.load()
+    enqueue(0)                       # untimed: primes lazily built tables
+    Device.synchronize()
+    if os.environ.get("NERVA_OPBENCH_EAGER") == "1":
+        # kernel-tracing mode: plain launches (a profiler reports the per-kernel durations)
+        t0 = time.perf_counter()
+        for i in range(launches):
+            enqueue(i)
+        Device.synchronize()
+        return (time.perf_counter() - t0) * 1e9 / launches
+    assert lib.nerva_hip_timer_capture_begin() == 0
+    for i in range(launches):
+        enqueue(i)
+    nodes, ns = C.c_uint64(0), C.c_double(0.0)
+    assert lib.nerva_hip_timer_capture_end(warmup, replays, C.byref(nodes), C.byref(ns)) == 0
+    return ns.value / launches
+
+
+def report(name, variant, ns, nbytes):
+    gbs = nbytes / ns
+    log("%-34s %-9s %9.2f us  %8.1f GB/s  %5.1f%% of HBM peak   (ideal %.2f us)" % (
+        name, variant, ns / 1e3, gbs, 100 * gbs / PEAK, nbytes / PEAK / 1e3))
+
+
+def case_qproj():
+    rows = cols = 4096
+    copies = 40
+    w = synth16(copies * rows * cols, 11)
+    x = synth16(cols, 12, std=1.0)
+    y = DeviceBuffer(rows * 2)
+    nbytes = rows * cols * 2 + cols * 2 + rows * 2
+    for variant, n in (("rotating", copies), ("resident", 1)):
+        ns = timed(lambda i: R.gemv(BF16, w.at((i % n) * rows * cols * 2), rows, cols, input16=x, out16=y,
+                                    epilogue=3, sync=False), 80)
+        report("1 q_proj GEMV 4096x4096", variant, ns, nbytes)
+
+
+def case_mlp():
+    H, I = 4096, 12288
+    copies = 4
+    per = 3 * I * H
+    w = synth16(copies * per, 21)
+    gamma = synth16(H, 22, mean=1.0)
+    h = synth32(H, 23)
+    ff = DeviceBuffer(I * 2)
+    out = DeviceBuffer(H * 4)
+    nbytes = per * 2 + H * 2 + H * 2 + H * 2     # weights + gamma + h + out counted as 16-bit vectors
+
+    def enqueue(i, n):
+        base = (i % n) * per * 2
+        R.gemv(BF16, w.at(base), I, H, input_f32=h, gamma=gamma, eps=1e-6, out16=ff, epilogue=2, sync=False)
+        R.gemv(BF16, w.at(base + 2 * I * H * 2), H, I, input16=ff, residual=h, out_f32=out, epilogue=1, sync=False)
+    for variant, n in (("rotating", copies), ("resident", 1)):
+        ns = timed(lambda i: enqueue(i, n), 24)
+        report("2 MLP block 4096 -> 12288 -> 4096", variant, ns, nbytes)
+
+
+def case_attention():
+    heads, kvh, hd, tokens = 32, 8, 128, 4096
+    layers, blocks = 64, tokens // 16 + 1
+    rng = np.random.default_rng(3)
+    table = rng.permutation(blocks).astype(np.uint32)
+    cache = R.PagedKvCache(layers, blocks, kvh, hd, table)
+    lib = abi.load()
+    assert lib.nerva_hip_synth_fill_16(cache.k.ptr, BF16, SEED, 31, cache.elems, 0.0, 1.0) == 0
+    assert lib.nerva_hip_synth_fill_16(cache.v.ptr, BF16, SEED, 32, cache.elems, 0.0, 1.0) == 0
+    qkv = synth32((heads + 2 * kvh) * hd, 33)
+    qn, kn = synth16(hd, 34, mean=1.0), synth16(hd, 35, mean=1.0)
+    ws = R.attention_workspace(heads, hd)
+    out16, out32 = DeviceBuffer(heads * hd * 2), DeviceBuffer(heads * hd * 4)
+    kv_read = 2 * (tokens + 1) * kvh * hd * 2
+    nbytes = kv_read + (heads + 2 * kvh) * hd * 4 + (blocks * 4) + 2 * kvh * hd * 2 + heads * hd * 4
+    for variant, n in (("rotating", layers), ("resident", 1)):
+        ns = timed(lambda i: R.paged_attention(BF16, heads, kvh, hd, cache, i % n, tokens, qkv, ws, out16,
+                                               out_f32=out32, append=True, rope_theta=1e6, q_norm=qn, k_norm=kn,
+                                               sync=False), 128)
+        report("3 paged GQA attention, 4097 keys", variant, ns, nbytes)
+
+
+def case_moe():
+    H, I, E, K, blk = 7168, 2048, 96, 8, 128      # 96 experts resident: 12 disjoint routed sets of 8
+    lib = abi.load()
+    sH, sI = (H + blk - 1) // blk, (I + blk - 1) // blk
+    wg, wu, wd = (DeviceBuffer(E * I * H) for _ in range(3))
+    sg, su = DeviceBuffer(E * sI * sH * 4), DeviceBuffer(E * sI * sH * 4)
+    sd = DeviceBuffer(E * sH * sI * 4)
+    for e in range(E):
+        assert lib.nerva_hip_synth_fill_fp8_block(wg.ptr + e * I * H, sg.ptr + e * sI * sH * 4, SEED, 1000 + e, I, H, blk, 0.02) == 0
+        assert lib.nerva_hip_synth_fill_fp8_block(wu.ptr + e * I * H, su.ptr + e * sI * sH * 4, SEED, 2000 + e, I, H, blk, 0.02) == 0
+        assert lib.nerva_hip_synth_fill_fp8_block(wd.ptr + e * I * H, sd.ptr + e * sH * sI * 4, SEED, 3000 + e, H, I, blk, 0.02) == 0
+    x = synth16(H, 41, std=1.0)
+    sets = (E - 1) // K                            # expert E-1 is the shared expert
+    ids = [DeviceBuffer.from_numpy(np.arange(s * K, (s + 1) * K, dtype=np.uint32)) for s in range(sets)]
+    wts = DeviceBuffer.from_numpy(np.full(K, 1.0 / K, np.float32))
+    act = DeviceBuffer((K + 1) * I * 4)
+    out = DeviceBuffer(H * 4)
+    nbytes = 9 * (3 * I * H + 3 * sI * sH * 4) + H * 2 + H * 2
+    for variant, n in (("rotating", sets), ("resident", 1)):
+        ns = timed(lambda i: R.moe_fp8_experts(H, I, E, K, blk, x, ids[i % n], wts, wg, sg, wu, su, wd, sd, act, out,
+                                               shared_index=E - 1, sync=False), 33)
+        report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
+
+
+def main():
+    rc, smoke = Device.smoke()
+    if rc != 0:
+        print("no usable GPU (hip_error=%d): these operators have no CPU path" % smoke.hip_error, file=sys.stderr)
+        sys.exit(1)
+    log("device: %s" % smoke.gpu_name.decode())
+    case_qproj()
+    case_mlp()
+    case_attention()
+    case_moe()
+
+
+if __name__ == "__main__":
+    main()

@@ -482,3 +482,22 @@ def test_plain_copy_kernel_is_exact_and_rejects_unaligned():
         assert np.array_equal(b.numpy(np.uint8, nbytes), src)
     assert abi.load().nerva_hip_copy_d2d(b.ptr, a.ptr, 24, None) == -1
     assert abi.load().nerva_hip_copy_d2d(b.ptr + 4, a.ptr, 16, None) == -1
+
+
+def test_operator_timer_records_launches_into_a_graph():
+    import ctypes as C
+    rng = np.random.default_rng(5)
+    rows, cols = 256, 4096
+    w = O.encode16(BF16, rng.normal(0, 0.05, (rows, cols)))
+    x = O.encode16(BF16, rng.normal(0, 1, cols))
+    dw, dx, y = dev(w), dev(x), N.DeviceBuffer.zeros(rows * 4)
+    lib = abi.load()
+    nodes, ns = C.c_uint64(0), C.c_double(0.0)
+    assert lib.nerva_hip_timer_capture_end(1, 1, C.byref(nodes), C.byref(ns)) == -1   # nothing being recorded
+    assert lib.nerva_hip_timer_capture_begin() == 0
+    assert lib.nerva_hip_timer_capture_begin() == -1                                  # one recording at a time
+    for _ in range(5):
+        N.gemv(BF16, dw, rows, cols, input16=dx, out_f32=y, sync=False)
+    assert lib.nerva_hip_timer_capture_end(2, 4, C.byref(nodes), C.byref(ns)) == 0
+    assert nodes.value == 5 and ns.value > 0
+    assert rel_l2(y.numpy(np.float32), O.gemv(BF16, w, O.decode16(BF16, x))) <= REL_L2
