@@ -545,6 +545,11 @@ typedef struct NervaHipStepProfile {
   /* average device ns per launch when the `layers` launches of one kind run back to back
    * between a single hipEvent pair (no per-launch event gap): the kernel's own duration */
   uint64_t qkv_stream_ns, attention_stream_ns, o_stream_ns, gate_up_stream_ns, down_stream_ns;
+  /* persistent layer-chain launch (o + gate/up + down + next layer's qkv as phases of one kernel):
+   * when chain_enabled is 1 the o/gate_up/down figures above are zero and qkv counts the first
+   * layer's stand-alone launch only */
+  uint64_t chain_ns, chain_stream_ns, chain_bytes;
+  uint32_t chain_enabled, reserved;
 } NervaHipStepProfile;
 
 /* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT
@@ -553,6 +558,14 @@ typedef struct NervaHipStepProfile {
  * session_profile.inc.cu:35-56, session_decode_prefill.inc.cu:374-809). */
 int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uint32_t repeats,
                                    NervaHipStepProfile *out);
+
+/* Persistent layer-chain kernel of a session: *enabled = 1 when the session's shapes use it,
+ * *aborted = 1 when one of its bounded in-kernel waits ran out (the calls that covered those
+ * steps returned -1 with hip_error = hipErrorLaunchFailure; start() clears it). raise_abort != 0
+ * sets the abort word from the host first, which makes every such wait give up at once: the
+ * failure path can be exercised while all kernels still terminate normally. */
+int nerva_hip_session_chain_state(NervaHipHfDecodeSequenceSession *session, uint32_t raise_abort,
+                                  uint32_t *enabled, uint32_t *aborted);
 
 /* Reads back the f32 logits of the last sampled position (vocab_size floats) and
  * one KV row (kv_heads*head_dim 16-bit values each for K and V) for parity tests. */

@@ -25,6 +25,7 @@
 
 #include "argmax.cuh"
 #include "attn_decode.cuh"
+#include "decode_chain.cuh"
 #include "gemv_stream.cuh"
 #include "runtime_state.hpp"
 #include "synth_fill.cuh"
@@ -41,7 +42,7 @@ struct LayerDev {
 };
 
 enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
-enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLKinds };
+enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLKinds };
 
 struct StepProfiler {
   hipStream_t stream;
@@ -91,6 +92,10 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
   void *attn_ws = nullptr, *sample_ws = nullptr;
   uint32_t attn_splits = 1;
+  // persistent layer-chain kernel (o + gate/up + down + next qkv in one launch)
+  bool chain = false;
+  uint32_t *chain_flags = nullptr, *chain_abort = nullptr;
+  uint64_t *chain_trace = nullptr;  // NERVA_HIP_CHAIN_TRACE=1: per-layer timestamps of workgroup 0
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
   uint32_t *host_state = nullptr;
@@ -230,6 +235,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   }
   for (uint32_t l = 0; l < s->layers; ++l) {
     const LayerDev &w = s->layer[l];
+    if (!s->chain || l == 0)
     {
       GemvParams p{};
       p.w = w.wqkv;
@@ -271,6 +277,37 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.append = 1;
       NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
     }
+    if (s->chain) {
+      // o projection, gate/up, down and the next layer's qkv projection as one persistent launch
+      ChainParams c{};
+      c.wo = w.wo;
+      c.o_bias = w.o_bias;
+      c.rms_mlp = w.rms_mlp;
+      c.wgu = w.wgu;
+      c.wdown = w.wdown;
+      c.rms_next = l + 1 < s->layers ? s->layer[l + 1].rms_attn : nullptr;
+      c.wqkv_next = l + 1 < s->layers ? s->layer[l + 1].wqkv : nullptr;
+      c.attn16 = s->attn16;
+      c.x = s->x;
+      c.r = s->r;
+      c.ff16 = s->ff16;
+      c.qkv = s->qkv;
+      c.hidden = s->hidden;
+      c.attn_dim = A;
+      c.inter = s->intermediate;
+      c.qkv_rows = A + 2 * KV;
+      c.eps = s->eps;
+      c.round_out = mode == kDecodeStep ? 0u : 1u;
+      c.flags = s->chain_flags;
+      c.abort_flag = s->chain_abort;
+      c.cursor = s->state;
+      c.max_steps = s->max_ctx;
+      c.barrier_base = kChainMaxBarriers * l;
+      c.barriers_per_step = kChainMaxBarriers * s->layers;
+      c.trace = s->chain_trace != nullptr ? s->chain_trace + 32 * l : nullptr;
+      NV_STEP(kLChain, launch_decode_chain(s->dtype, c, st));
+      continue;
+    }
     {
       GemvParams p{};
       p.w = w.wo;
@@ -311,7 +348,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.max_steps = s->max_ctx;
       NV_STEP(kLDown, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
     }
-  }
+    }
   if (only >= 0) return hipSuccess;
   if (mode == kPromptStep) {
     if (prof) err = prof->before(kLAdvance);
@@ -394,7 +431,8 @@ hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *o
 hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
   if (eager_steps()) {
     hipError_t err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
-    if (err == hipSuccess) out->kernel_launches += (which == 0 ? 3 : 2) + 5ull * s->layers;
+    if (err == hipSuccess)
+      out->kernel_launches += s->chain ? (which == 0 ? 4 : 3) + 2ull * s->layers : (which == 0 ? 3 : 2) + 5ull * s->layers;
     return err;
   }
   hipError_t err = hipGraphLaunch(s->exec[which], s->stream);
@@ -464,6 +502,16 @@ bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
   return true;
 }
 
+// After a synchronisation: did a bounded wait of the chain kernel run out during the steps
+// just completed? Their tokens are then not to be trusted and the call fails.
+hipError_t chain_verdict(Session *s) {
+  if (!s->chain) return hipSuccess;
+  uint32_t aborted = 0;
+  const hipError_t err = hipMemcpy(&aborted, s->chain_abort, sizeof(aborted), hipMemcpyDeviceToHost);
+  if (err != hipSuccess) return err;
+  return aborted != 0 ? hipErrorLaunchFailure : hipSuccess;
+}
+
 hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t prompt_count,
                           NervaHipHfDecodeSequenceResult *out) {
   // Not on the per-token path: the prompt is copied synchronously (the caller's buffer may be
@@ -474,6 +522,8 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
                     hipMemcpyHostToDevice);
   if (err == hipSuccess)
     err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  // the chain kernel's barrier epochs grow with the position: a new sequence starts them over
+  if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count);
     err = hipGetLastError();
@@ -615,6 +665,8 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_rope_cs = c.take(HD * 4);
   const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
+  const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
+  const uint64_t off_chain_trace = c.take(static_cast<uint64_t>(rq->layer_count) * 32 * 8);
   s->arena_bytes = c.offset;
 
   if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
@@ -660,6 +712,22 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
   s->sample_ws = s->arena + off_sample_ws;
+  s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
+  s->chain_abort = reinterpret_cast<uint32_t *>(s->arena + off_chain + chain_flag_bytes());
+  {
+    // NERVA_HIP_CHAIN=1 runs o + gate/up + down + next qkv as one persistent launch per layer.
+    // Off by default: measured on MI355X it is about 4 % slower per step than one launch per
+    // GEMV (the in-kernel grid barriers cost as much as the kernel boundaries they replace, and
+    // a static split of the rows over 256 workgroups waits longer for its slowest member).
+    const char *want_chain = getenv("NERVA_HIP_CHAIN");
+    s->chain = want_chain != nullptr && want_chain[0] == '1' && rq->layer_count > 0 &&
+               chain_supported(rq->hidden, rq->heads * rq->head_dim, rq->intermediate,
+                               (rq->heads + 2 * rq->kv_heads) * rq->head_dim) &&
+               chain_prepare(rq->dtype) == hipSuccess;
+    const char *trace = getenv("NERVA_HIP_CHAIN_TRACE");
+    if (s->chain && trace != nullptr && trace[0] == '1')
+      s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
+  }
   s->layer.resize(L);
   for (uint32_t l = 0; l < L; ++l) {
     s->layer[l] = LayerDev{dev16(lo[l].rms_attn), dev16(lo[l].rms_mlp), dev16(lo[l].wqkv),
@@ -740,6 +808,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   }
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_workspace_bytes(rq->heads, rq->head_dim), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
@@ -852,7 +921,7 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
     err = launch_step(s, 1, out);
   }
   if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
-  if (err == hipSuccess) out->kernel_launches += 3 + 5ull * s->layers;
+  if (err == hipSuccess) out->kernel_launches += s->chain ? 4 + 2ull * s->layers : 3 + 5ull * s->layers;
   if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
@@ -921,6 +990,7 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
     err = hipStreamSynchronize(s->stream);
     out->sync_calls += 1;
   }
+  if (err == hipSuccess) err = chain_verdict(s);
   out->hot_path_allocations = allocation_count() - allocs_before;
   if (err == hipSuccess && run_count != 0) {
     float ms = 0.0f;
@@ -994,6 +1064,7 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
     err = hipStreamSynchronize(s->stream);
     out->sync_calls += 1;
   }
+  if (err == hipSuccess) err = chain_verdict(s);
   out->hot_path_allocations = allocation_count() - allocs_before;
   if (err == hipSuccess) {
     float ms = 0.0f;
@@ -1091,7 +1162,9 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {  // first pass is a warm-up
     prof.used = 0;
     prof.kinds.clear();
-    err = enqueue_step(s, kDecodeStep, &prof);
+    // the step is repeated at one position: the chain kernel's barrier epochs must start over
+    err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
+    if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, &prof);
     if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
     // undo the step: cursor and the published slot
     if (err == hipSuccess) err = hipMemcpy(s->state, &pos, 4, hipMemcpyHostToDevice);
@@ -1116,10 +1189,16 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // back-to-back pass: all `layers` launches of one kind between a single event pair, so the
   // figure is the kernel's own duration without the per-launch event gaps
   uint64_t stream_ns[kLKinds] = {0};
-  for (int kind = kLQkv; err == hipSuccess && kind <= kLDown; ++kind) {
+  for (int kind = kLQkv; err == hipSuccess && kind <= kLChain; ++kind) {
+    uint32_t launches = s->layers;
+    if (kind == kLHead || kind == kLAdvance) continue;
+    if (kind == kLQkv && s->chain) launches = 1;
+    if ((kind == kLO || kind == kLGateUp || kind == kLDown) && s->chain) continue;
+    if (kind == kLChain && !s->chain) continue;
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
-      err = hipEventRecord(s->ev0, s->stream);
+      err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
+      if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
       if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
       if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
       if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
@@ -1127,8 +1206,27 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
       if (err == hipSuccess) err = hipEventElapsedTime(&ms, s->ev0, s->ev1);
       if (rep > 0) acc += static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
     }
-    stream_ns[kind] = acc / (static_cast<uint64_t>(repeats) * s->layers);
+    stream_ns[kind] = acc / (static_cast<uint64_t>(repeats) * launches);
   }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    return -1;
+  }
+  if (s->chain_trace != nullptr) {
+    std::vector<uint64_t> tr(static_cast<size_t>(s->layers) * 32);
+    if (hipMemcpy(tr.data(), s->chain_trace, tr.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+      for (uint32_t l = 0; l < s->layers && l < 3; ++l) {
+        const uint64_t *t = tr.data() + 32 * l;
+        fprintf(stderr, "[chain trace] layer %u (10 ns ticks from the first barrier B):", l);
+        for (int i = 0; i < 22; ++i) fprintf(stderr, " %lld", static_cast<long long>(t[i]) - static_cast<long long>(t[1]));
+        fprintf(stderr, "\n");
+      }
+    }
+  }
+  // leave no epochs of this position behind: the sequence will run the step at `pos` for real
+  err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+  if (err == hipSuccess) err = chain_verdict(s);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     return -1;
@@ -1138,6 +1236,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->o_stream_ns = stream_ns[kLO];
   out->gate_up_stream_ns = stream_ns[kLGateUp];
   out->down_stream_ns = stream_ns[kLDown];
+  out->chain_stream_ns = stream_ns[kLChain];
   auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
   out->position = pos;
   out->embed_ns = avg(kLEmbed);
@@ -1147,6 +1246,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_ns = avg(kLGateUp);
   out->down_ns = avg(kLDown);
   out->lm_head_ns = avg(kLHead);
+  out->chain_ns = avg(kLChain);
   out->total_ns = total / repeats;
   const uint64_t H = s->hidden, A = static_cast<uint64_t>(s->heads) * s->head_dim,
                  KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim, I = s->intermediate, V = s->vocab;
@@ -1157,7 +1257,26 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_bytes = 2 * I * H * 2 + H * 4 + H * 2 + I * 2;
   out->down_bytes = H * I * 2 + I * 2 + H * 4 + H * 4;
   out->lm_head_bytes = V * H * 2 + H * 4 + H * 2 + V * 4;
+  // chain launch of a middle layer: o + gate/up + down + next qkv (the activations between them
+  // stay on the device and are counted once, as the phase that reads them)
+  out->chain_bytes = s->chain ? out->o_bytes + out->gate_up_bytes + out->down_bytes + out->qkv_bytes : 0;
+  out->chain_enabled = s->chain ? 1u : 0u;
   out->status = 0;
+  return 0;
+}
+
+int nerva_hip_session_chain_state(NervaHipHfDecodeSequenceSession *s, uint32_t raise_abort, uint32_t *enabled,
+                                  uint32_t *aborted) {
+  if (s == nullptr) return -1;
+  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
+  if (raise_abort != 0 && s->chain) {
+    const uint32_t one = 1;
+    if (hipMemcpy(s->chain_abort, &one, sizeof(one), hipMemcpyHostToDevice) != hipSuccess) return -1;
+  }
+  uint32_t flag = 0;
+  if (s->chain && hipMemcpy(&flag, s->chain_abort, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  if (enabled) *enabled = s->chain ? 1u : 0u;
+  if (aborted) *aborted = flag;
   return 0;
 }
 

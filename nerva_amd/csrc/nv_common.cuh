@@ -19,11 +19,11 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
 __device__ __forceinline__ uint16_t f32_to_bf16(float v) {
-  uint32_t bits = __float_as_uint(v);
-  if ((bits & 0x7f800000u) == 0x7f800000u && (bits & 0x007fffffu) != 0) {
-    return static_cast<uint16_t>((bits >> 16) | 1u);
-  }
-  return static_cast<uint16_t>((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+  const uint32_t bits = __float_as_uint(v);
+  // both results are computed and one is selected: no branch in the hot epilogues
+  const uint32_t rounded = (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+  const uint32_t nan = (bits >> 16) | 1u;
+  return static_cast<uint16_t>((bits & 0x7fffffffu) > 0x7f800000u ? nan : rounded);
 }
 __device__ __forceinline__ float f16_to_f32(uint16_t b) {
   return static_cast<float>(__builtin_bit_cast(_Float16, b));

@@ -136,6 +136,14 @@ class DecodeSession:
         rc = self.lib.nerva_hip_session_profile_step(self.handle, repeats, C.byref(res))
         return rc, res
 
+    def chain_state(self, raise_abort=False):
+        """(enabled, aborted) of the persistent layer-chain kernel; raise_abort sets the abort word."""
+        enabled, aborted = C.c_uint32(0), C.c_uint32(0)
+        rc = self.lib.nerva_hip_session_chain_state(self.handle, int(raise_abort), C.byref(enabled), C.byref(aborted))
+        if rc != 0:
+            raise RuntimeError("chain_state failed")
+        return bool(enabled.value), bool(aborted.value)
+
     def logits(self):
         out = np.empty(self.vocab, np.float32)
         if self.lib.nerva_hip_session_read_logits(self.handle, out.ctypes.data) != 0:

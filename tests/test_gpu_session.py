@@ -174,11 +174,23 @@ GEOMETRIES = [
     (F16, 256, 4, 2, 64, 520, 300, 2, 1e4, True, False),       # generic attention path, guarded GEMV
     (BF16, 96, 6, 2, 16, 200, 50, 2, 0, False, False),         # group 3, no RoPE, cols % 8 == 0 only
     (F16, 512, 4, 1, 128, 1024, 1000, 3, 1e6, True, False),    # fast attention path in f16
+    (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False), # shapes the persistent chain kernel accepts
+    (F16, 2048, 16, 16, 128, 2048, 700, 2, 1e4, False, True),  # same in f16, MHA, o bias
 ]
 
 
+@pytest.fixture(params=[False, True], ids=["launch-per-gemv", "chain-kernel"])
+def chain_mode(request, monkeypatch):
+    """Sessions created inside the test use the persistent layer-chain kernel when the shapes fit."""
+    if request.param:
+        monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
+    else:
+        monkeypatch.delenv("NERVA_HIP_CHAIN", raising=False)
+    return request.param
+
+
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_single_layer_short_prompt_is_tight(geom):
+def test_single_layer_short_prompt_is_tight(geom, chain_mode):
     """One layer and a 1- or 2-token prompt leave no room for 16-bit ties to compound: the whole
     step (embed, norms, GEMVs, RoPE, attention, LM head) must agree with the oracle at 1e-3 in
     f16. In bf16 a single value that sits within 1e-6 of a rounding boundary (attention output,
@@ -186,6 +198,8 @@ def test_single_layer_short_prompt_is_tight(geom):
     one activation by 2^-8 relative and the logits of this tiny model by up to ~3e-3: the bound
     is one such flip, 6e-3."""
     dtype, hidden, heads, kv, hd, inter, vocab, _, theta, qk_norm, bias = geom
+    if chain_mode and hidden % 2048:
+        pytest.skip("shapes do not fit the chain kernel: same path as launch-per-gemv")
     tol = REL_L2 if dtype == F16 else 6e-3
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, 1, hidden + 1, theta, qk_norm, bias)
     s = N.DecodeSession.create(weights, 32)
@@ -199,17 +213,24 @@ def test_single_layer_short_prompt_is_tight(geom):
         gk, gv = s.kv_row(0, len(prompt) - 1)
         rk, rv = ctx.read_kv16(0, len(prompt) - 1)
         # summation order may move a value across a 16-bit tie: at most one unit, on few elements
+        # (values near zero are compared by magnitude: one unit there is far below the f32 noise)
         for got, ref in ((gk, rk), (gv, rv)):
-            assert np.max(np.abs(got.astype(np.int32) - ref.astype(np.int32))) <= 1
-            assert np.mean(got != ref) <= 0.05
+            gf, rf = O.decode16(dtype, got), O.decode16(dtype, ref)
+            units = np.abs(got.astype(np.int32) - ref.astype(np.int32))
+            assert np.all((units <= 1) | (np.abs(gf - rf) <= 1e-4 * np.max(np.abs(rf))))
+            # one flipped element of the normalised input moves every K/V value by ~1e-5, which
+            # carries a few percent of them across their own 16-bit boundary
+            assert np.mean(got != ref) <= 0.10
         rc, res, tokens = s.advance(1)
         assert rc == 0 and tokens[0] == O.greedy_argmax(ctx.logits(), skip_nonfinite=True)
     s.destroy()
 
 
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_session_matches_oracle_logits_kv_and_stream(geom):
+def test_session_matches_oracle_logits_kv_and_stream(geom, chain_mode):
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
+    if chain_mode and hidden % 2048:
+        pytest.skip("shapes do not fit the chain kernel: same path as launch-per-gemv")
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, hidden, theta, qk_norm, bias)
     prompt = np.random.default_rng(1).integers(0, vocab, 21).astype(np.uint32)
     steps = 24
@@ -312,4 +333,61 @@ def test_synthetic_session_matches_oracle_weights():
     for i, t in enumerate(prompt):
         ctx2.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
     assert_streams_agree(tokens.tolist(), otokens.tolist(), margins, float(np.max(np.abs(ctx2.logits()))))
+    s.destroy()
+
+
+CHAIN_GEOM = (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False)
+
+
+def test_chain_kernel_is_used_and_agrees_with_one_launch_per_gemv(monkeypatch):
+    """Shapes that fit take the persistent layer-chain kernel (o + gate/up + down + next qkv in one
+    launch). Its dot products are summed in the same order as the stand-alone GEMV kernels; only
+    the RMSNorm sum of squares is grouped differently (one wave instead of four), so logits agree
+    to 16-bit-tie noise and the greedy streams of this model are identical."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = CHAIN_GEOM
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 77, theta, qk_norm, bias)
+    prompt = np.random.default_rng(2).integers(0, vocab, 19).astype(np.uint32)
+    monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
+    s = N.DecodeSession.create(weights, 64)
+    assert s.chain_state() == (True, False)
+    rc, res = s.start(prompt)
+    assert rc == 0
+    rc, res, chained = s.advance(12)
+    assert rc == 0 and res.graph_nodes == 4 + 2 * layers and res.hot_path_allocations == 0
+    logits_chain = s.logits()
+    rc, prof = s.profile_step(2)
+    assert rc == 0 and prof.chain_enabled == 1 and prof.launches == 4 + 2 * layers
+    assert prof.chain_ns > 0 and prof.chain_stream_ns > 0 and prof.o_ns == 0 and prof.chain_bytes > 0
+    rc, res, more = s.advance(4)                      # profiling did not disturb the sequence
+    assert rc == 0
+    s.destroy()
+    monkeypatch.delenv("NERVA_HIP_CHAIN")
+    s = N.DecodeSession.create(weights, 64)
+    assert s.chain_state() == (False, False)
+    s.start(prompt)
+    rc, res, plain = s.advance(12)
+    assert rc == 0 and res.graph_nodes == 3 + 5 * layers
+    assert rel_l2(logits_chain, s.logits()) <= E2E_REL_L2
+    rc, res, more_plain = s.advance(4)
+    assert chained.tolist() == plain.tolist() and more.tolist() == more_plain.tolist()
+    s.destroy()
+
+
+def test_chain_kernel_bounded_wait_gives_up_cleanly(monkeypatch):
+    """With the abort word raised from the host every in-kernel wait gives up at once: all kernels
+    still run to completion, the call reports the failure, and start() makes the session usable."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = CHAIN_GEOM
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 78, theta, qk_norm, bias)
+    monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
+    s = N.DecodeSession.create(weights, 32)
+    rc, res = s.start([1, 2, 3])
+    rc, res, good = s.advance(3)
+    assert rc == 0
+    assert s.chain_state(raise_abort=True) == (True, True)
+    rc, res, _ = s.advance(2)
+    assert rc == -1 and res.status == -1 and res.hip_error != 0
+    rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
+    assert rc == 0 and s.chain_state() == (True, False)
+    rc, res, again = s.advance(3)
+    assert rc == 0 and again.tolist() == good.tolist()
     s.destroy()
