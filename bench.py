@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one gate_up launch moves at the Qwen3-8B shape (24576x4096 bf16): FETCH_SIZE + WRITE_SIZE
 # per dispatch from two `rocprofv3 --pmc` runs, each scaled by what the counter reads for a plain
 # 256 MiB copy kernel (profiles/gate_up_gemv_hbm_traffic_pmc.txt). Not measurable in-process.
-GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201779003}
+GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201709220}
 # Same for one launch of the persistent layer-chain kernel (filled in from its counter profile).
 CHAIN_TRAFFIC_BYTES = {}
 SEED = 0x4E45525641
