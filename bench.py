@@ -134,7 +134,7 @@ def main():
         sys.exit(1)
     cfg = dict(N.Qwen3_8B)
     cfg["layers"] = args.layers
-    max_ctx = args.prompt + args.warmup + args.steps + 16
+    max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16
     t0 = time.time()
     session = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=WEIGHT_STD, qk_norm=True)
     log("[bench] %s: session created in %.1f s, arena %.2f GB (weights %.2f GB, KV %.2f GB)" % (
@@ -198,11 +198,25 @@ def main():
                     whole_step_bytes=bytes_step, whole_step_frac=round(bytes_step * tok_s / 1e9 / HBM_PEAK_GBS, 4),
                     per_kernel_frac={k: round(b / max(ns, 1) / HBM_PEAK_GBS, 4) for k, (ns, b) in per_kind.items()})
 
+    # host-observed latency of single tokens: one advance(1) call (graph launch + synchronisation +
+    # slot download) per token, which is how a caller that streams tokens out drives the session
+    lat = []
+    for _ in range(min(args.steps, 128)):
+        t1 = time.perf_counter()
+        rc, r1, last = session.advance(1)
+        lat.append(time.perf_counter() - t1)
+        assert rc == 0
+        tokens = last
+    lat_ms = np.sort(np.array(lat)) * 1e3
+    rank = lambda q: float(lat_ms[min(len(lat_ms) - 1, int(np.ceil(q * len(lat_ms))) - 1)])   # nearest rank
+    latency = dict(p50=round(rank(0.50), 4), p95=round(rank(0.95), 4), p99=round(rank(0.99), 4), tokens=len(lat_ms))
+    log("[bench] single-token advance(1) latency ms: p50 %.3f  p95 %.3f  p99 %.3f" % (latency["p50"], latency["p95"], latency["p99"]))
+
     cpu = None
     if not args.no_cpu:
         try:
             threads_all = min(os.cpu_count() or 1, 16)
-            position = args.prompt + args.warmup + args.steps      # tokens now in the KV cache
+            position = args.prompt + args.warmup + args.steps + len(lat)   # tokens now in the KV cache
             layers_sampled = min(args.cpu_layers, cfg["layers"])
             r = cpu_baseline(session, cfg, position, int(tokens[-1]), layers_sampled, threads_all)
             cpu = dict(value=round(r[1]["tok_s"], 5), unit="tok/s", cores=1, kind="port",
@@ -222,7 +236,7 @@ def main():
                                      % (cfg["layers"], args.prompt, args.steps),
                             prompt_tokens=args.prompt, context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
-                            gpu=smoke.gpu_name.decode()),
+                            per_token_latency_ms=latency, gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)
     print(json.dumps(line), flush=True)
 

@@ -1,0 +1,123 @@
+// Exercises the C++ host wrapper (nerva_amd/host/nerva_hip.hpp) the way the reference's Rust tests
+// exercise its safe wrappers (crates/nerva-cuda/src/tests/decode_sequence_session.rs:21-86,
+// decode_sequence.rs:123-223). Mode "cpu": everything that must hold without a device
+// (validation before the call, Unavailable when there is no GPU). Mode "gpu": the reference's
+// greedy-stream known-answer model through create / start / advance / run.
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "nerva_hip.hpp"
+
+using namespace nerva::hip;
+
+static int failures = 0;
+#define CHECK(cond)                                                       \
+  do {                                                                    \
+    if (!(cond)) {                                                        \
+      std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+      ++failures;                                                         \
+    }                                                                     \
+  } while (0)
+
+struct KatModel {
+  // hidden 2, vocab 4, f16: embeddings [1,0; 0,1; -1,0; 0,-1], layer matrices 0, lm_head [0,-1; 1,0; 0,1; -1,0]
+  std::vector<uint16_t> emb{0x3c00, 0x0000, 0x0000, 0x3c00, 0xbc00, 0x0000, 0x0000, 0xbc00};
+  std::vector<uint16_t> rms{0x3c00, 0x3c00};
+  std::vector<uint16_t> zero{0, 0, 0, 0};
+  std::vector<uint16_t> head{0x0000, 0xbc00, 0x3c00, 0x0000, 0x0000, 0x3c00, 0xbc00, 0x0000};
+  HipHfDecodeSequenceSessionConfig config() const {
+    HipHfDecodeSequenceSessionConfig c;
+    c.dtype = NERVA_HIP_DTYPE_F16;
+    c.hidden = 2;
+    c.heads = 1;
+    c.kv_heads = 1;
+    c.head_dim = 2;
+    c.intermediate = 2;
+    c.vocab_size = 4;
+    c.max_context_tokens = 16;
+    c.rms_eps = 1e-5f;
+    c.embeddings = emb;
+    c.final_norm_weight = rms;
+    c.lm_head = head;
+    HipHfDecodeChainLayer l;
+    l.rms_attn_weight = rms;
+    l.rms_mlp_weight = rms;
+    l.w_q = l.w_k = l.w_v = l.w_o = l.w_gate = l.w_up = l.w_down = zero;
+    c.layers.push_back(l);
+    return c;
+  }
+};
+
+static void cpu_checks() {
+  KatModel m;
+  // validation happens before any native call
+  HipHfDecodeSequenceSessionConfig bad = m.config();
+  bad.kv_heads = 0;
+  auto out = bad.create();
+  CHECK(out.summary.status == SmokeStatus::Failed && out.summary.error.has_value() && !out.session);
+  bad = m.config();
+  bad.layers[0].w_q = Span<uint16_t>(m.zero.data(), 3);
+  out = bad.create();
+  CHECK(out.summary.status == SmokeStatus::Failed && out.summary.error->find("wrong size") != std::string::npos);
+  HipHfDecodeSamplerConfig sampler;
+  sampler.top_p = 0.0f;
+  CHECK(sampler.validate().has_value());
+  CHECK(!HipHfDecodeSamplerConfig::greedy().validate().has_value());
+  std::vector<uint32_t> none, outside{7};
+  CHECK(detail::validate_loop_start(none, 4).has_value());
+  CHECK(detail::validate_loop_start(outside, 4).has_value());
+  // no device: Unavailable, never a crash, never a silent success
+  const HipDeviceSmokeSummary smoke = device_smoke();
+  if (smoke.status != SmokeStatus::Ok) {
+    CHECK(smoke.status == SmokeStatus::Unavailable);
+    out = m.config().create();
+    CHECK(out.summary.status == SmokeStatus::Unavailable && !out.session);
+    CHECK(out.summary.hip_error == NERVA_HIP_ERROR_NO_DEVICE);
+  }
+}
+
+static void gpu_checks() {
+  KatModel m;
+  CHECK(device_smoke().status == SmokeStatus::Ok);
+  auto created = m.config().create();
+  CHECK(created.summary.status == SmokeStatus::Ok && created.session);
+  if (!created.session) return;
+  CHECK(created.summary.hot_path_allocations == 0 && created.summary.resident_weight_bytes == 100);
+  HipHfDecodeSequenceSession &session = *created.session;
+  std::vector<uint32_t> prompt{0};
+  // one-call run: [1, 2, 3, 0]
+  HipHfDecodeSequenceSummary run = session.run(prompt, 4);
+  CHECK(run.status == SmokeStatus::Ok && run.tokens == std::vector<uint32_t>({1, 2, 3, 0}));
+  CHECK(run.graph_replays == 4 && run.sync_calls == 1 && run.hot_path_allocations == 0 && run.host_causality_edges == 0);
+  // with a stop token the stream ends at it
+  run = session.run(prompt, 4, 2u);
+  CHECK(run.status == SmokeStatus::Ok && run.tokens == std::vector<uint32_t>({1, 2}) && run.kv_tokens == 2);
+  // loop: start, then advance in pieces; a finished loop refuses to advance
+  auto started = HipHfDecodeSequenceLoop::start(session, prompt, 3u);
+  CHECK(started.summary.status == SmokeStatus::Ok && started.loop_state.has_value());
+  if (started.loop_state) {
+    HipHfDecodeSequenceSummary a = started.loop_state->advance(2);
+    CHECK(a.status == SmokeStatus::Ok && a.tokens == std::vector<uint32_t>({1, 2}));
+    HipHfDecodeSequenceSummary b = started.loop_state->advance(4);
+    CHECK(b.status == SmokeStatus::Ok && b.tokens == std::vector<uint32_t>({3}) && started.loop_state->finished());
+    CHECK(started.loop_state->advance(1).status == SmokeStatus::Failed);
+  }
+  // refusals: prompt outside the vocabulary (before the call), non-greedy sampling (by the library)
+  std::vector<uint32_t> outside{9};
+  CHECK(HipHfDecodeSequenceLoop::start(session, outside).summary.status == SmokeStatus::Failed);
+  HipHfDecodeSamplerConfig hot;
+  hot.temperature = 0.8f;
+  hot.top_k = 40;
+  auto refused = HipHfDecodeSequenceLoop::start_with_sampler(session, prompt, std::nullopt, hot);
+  CHECK(refused.summary.status == SmokeStatus::Failed && refused.summary.hip_error == NERVA_HIP_ERROR_NOT_SUPPORTED);
+}
+
+int main(int argc, char **argv) {
+  const std::string mode = argc > 1 ? argv[1] : "cpu";
+  cpu_checks();
+  if (mode == "gpu") gpu_checks();
+  std::printf("%s: %d failure(s)\n", mode.c_str(), failures);
+  return failures == 0 ? 0 : 1;
+}
