@@ -175,7 +175,15 @@ def main():
     assert rc == 0
     per_kind = {}
     chain = bool(prof.chain_enabled)
-    kinds = ("qkv", "attention", "chain", "lm_head") if chain else ("qkv", "attention", "o", "gate_up", "down", "lm_head")
+    front = int(prof.front_mode)   # 1: qkv + attention + o in one launch, 2: attention + o, 0: one launch per piece
+    if chain:
+        kinds = ("qkv", "attention", "chain", "lm_head")
+    elif front == 1:
+        kinds = ("front", "gate_up", "down", "lm_head")
+    elif front == 2:
+        kinds = ("qkv", "front", "gate_up", "down", "lm_head")
+    else:
+        kinds = ("qkv", "attention", "o", "gate_up", "down", "lm_head")
     for k in kinds:
         paired = getattr(prof, k + "_ns")
         ns = getattr(prof, k + "_stream_ns", 0) or paired

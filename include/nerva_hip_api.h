@@ -549,7 +549,11 @@ typedef struct NervaHipStepProfile {
    * when chain_enabled is 1 the o/gate_up/down figures above are zero and qkv counts the first
    * layer's stand-alone launch only */
   uint64_t chain_ns, chain_stream_ns, chain_bytes;
-  uint32_t chain_enabled, reserved;
+  uint32_t chain_enabled;
+  /* fused layer front (qkv + attention + o projection as roles of one launch). front_mode 1: all
+   * three (the qkv/attention/o figures above are zero), 2: attention + o only, 0: off */
+  uint32_t front_mode;
+  uint64_t front_ns, front_stream_ns, front_bytes;
 } NervaHipStepProfile;
 
 /* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT
@@ -559,13 +563,21 @@ typedef struct NervaHipStepProfile {
 int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uint32_t repeats,
                                    NervaHipStepProfile *out);
 
-/* Persistent layer-chain kernel of a session: *enabled = 1 when the session's shapes use it,
- * *aborted = 1 when one of its bounded in-kernel waits ran out (the calls that covered those
- * steps returned -1 with hip_error = hipErrorLaunchFailure; start() clears it). raise_abort != 0
- * sets the abort word from the host first, which makes every such wait give up at once: the
- * failure path can be exercised while all kernels still terminate normally. */
-int nerva_hip_session_chain_state(NervaHipHfDecodeSequenceSession *session, uint32_t raise_abort,
-                                  uint32_t *enabled, uint32_t *aborted);
+/* Kernels of a session that hand data between workgroups inside one launch. *mode says which
+ * the session's shapes and switches selected: the fused layer front (qkv + attention + o
+ * projection as roles of one launch, the default where the shapes fit), the same without the
+ * qkv role (NERVA_HIP_FRONT=2), the persistent layer-chain kernel (NERVA_HIP_CHAIN=1), or none
+ * (NERVA_HIP_FRONT=0 / shapes that do not fit). *aborted = 1 when one of their bounded in-kernel
+ * waits ran out (the calls that covered those steps returned -1 with hip_error =
+ * hipErrorLaunchFailure; start() clears it). raise_abort != 0 sets the abort word from the host
+ * first, which makes every such wait give up at once: the failure path can be exercised while
+ * all kernels still terminate normally. */
+#define NERVA_HIP_FUSED_NONE 0u
+#define NERVA_HIP_FUSED_CHAIN 1u
+#define NERVA_HIP_FUSED_FRONT 2u
+#define NERVA_HIP_FUSED_FRONT_ATTN_O 3u
+int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *session, uint32_t raise_abort,
+                                  uint32_t *mode, uint32_t *aborted);
 
 /* Reads back the f32 logits of the last sampled position (vocab_size floats) and
  * one KV row (kv_heads*head_dim 16-bit values each for K and V) for parity tests. */

@@ -26,6 +26,7 @@
 #include "argmax.cuh"
 #include "attn_decode.cuh"
 #include "decode_chain.cuh"
+#include "layer_front.cuh"
 #include "gemv_stream.cuh"
 #include "runtime_state.hpp"
 #include "synth_fill.cuh"
@@ -42,7 +43,7 @@ struct LayerDev {
 };
 
 enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
-enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLKinds };
+enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLFront, kLKinds };
 
 struct StepProfiler {
   hipStream_t stream;
@@ -86,7 +87,8 @@ struct NervaHipHfDecodeSequenceSession {
   const uint16_t *emb = nullptr, *final_norm = nullptr, *lm_head = nullptr;
   uint16_t *kc = nullptr, *vc = nullptr;
   uint32_t block_count = 0;
-  uint32_t *table = nullptr, *prompt = nullptr, *state = nullptr;  // state[0] cursor, state[1] prompt count
+  uint32_t *table = nullptr, *prompt = nullptr;
+  uint32_t *state = nullptr;  // state[0] cursor, state[1] prompt count, state[2] steps executed so far
   Slot *slots = nullptr;
   float *x = nullptr, *r = nullptr, *qkv = nullptr, *logits = nullptr, *rope_freq = nullptr, *rope_cs = nullptr;
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
@@ -96,6 +98,13 @@ struct NervaHipHfDecodeSequenceSession {
   bool chain = false;
   uint32_t *chain_flags = nullptr, *chain_abort = nullptr;
   uint64_t *chain_trace = nullptr;  // NERVA_HIP_CHAIN_TRACE=1: per-layer timestamps of workgroup 0
+  // fused layer front (qkv + attention + o in one launch): 0 off, 1 all three roles,
+  // 2 attention + o only (the qkv projection stays a launch of its own)
+  int front = 0;
+  uint32_t front_splits = 1;
+  uint32_t *front_flags = nullptr;
+  float *attn_f32 = nullptr;
+  uint64_t *front_trace = nullptr;  // NERVA_HIP_FRONT_TRACE=1: per-layer timestamps of selected workgroups
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
   uint32_t *host_state = nullptr;
@@ -120,12 +129,15 @@ namespace {
 
 template <uint32_t DT>
 __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, const uint32_t *prompt,
-                                                       const Slot *slots, const uint32_t *state,
+                                                       const Slot *slots, uint32_t *state,
                                                        uint32_t max_steps, uint32_t hidden,
                                                        uint32_t vocab, float *x, const float *rope_freq,
                                                        float *rope_cs, uint32_t half_dim) {
   const uint32_t pos = state[0];
   if (pos >= max_steps) return;
+  // steps executed so far: the epochs of in-launch hand-overs derive from it (nobody reads it
+  // in this launch)
+  if (blockIdx.x == 0 && threadIdx.x == 0) state[2] = state[2] + 1u;
   // this step's RoPE angles, once: cos at [i], sin at [half_dim + i] (f32 angle = pos / theta^(2i/d))
   if (rope_freq != nullptr && blockIdx.x == 0) {
     for (uint32_t i = threadIdx.x; i < half_dim; i += kBlock) {
@@ -235,7 +247,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   }
   for (uint32_t l = 0; l < s->layers; ++l) {
     const LayerDev &w = s->layer[l];
-    if (!s->chain || l == 0)
+    if (s->front != 0 ? s->front == 2 : (!s->chain || l == 0))
     {
       GemvParams p{};
       p.w = w.wqkv;
@@ -275,7 +287,30 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
       p.append = 1;
-      NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
+      if (s->front != 0) {
+        // qkv rows, attention splits and o rows as roles of one launch
+        FrontParams f{};
+        p.splits = s->front_splits;
+        f.attn = p;
+        f.wqkv = s->front == 1 ? w.wqkv : nullptr;
+        f.rms_attn = w.rms_attn;
+        f.x = s->x;
+        f.wo = w.wo;
+        f.o_bias = w.o_bias;
+        f.attn_f32 = s->attn_f32;
+        f.r = s->r;
+        f.hidden = s->hidden;
+        f.rms_eps = s->eps;
+        front_bind_flags(f, s->front_flags);
+        f.abort_flag = s->chain_abort;
+        f.step_counter = s->state + 2;
+        f.layer = l;
+        f.layers = s->layers;
+        f.trace = s->front_trace != nullptr ? s->front_trace + 32 * l : nullptr;
+        NV_STEP(kLFront, launch_layer_front(s->dtype, f, st));
+      } else {
+        NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
+      }
     }
     if (s->chain) {
       // o projection, gate/up, down and the next layer's qkv projection as one persistent launch
@@ -308,7 +343,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       NV_STEP(kLChain, launch_decode_chain(s->dtype, c, st));
       continue;
     }
-    {
+    if (s->front == 0) {
       GemvParams p{};
       p.w = w.wo;
       p.x16 = s->attn16;
@@ -391,6 +426,15 @@ bool eager_steps() {
   return eager;
 }
 
+// Kernel launches of one step (which = 0: decode step, 1: prompt step).
+uint64_t step_launches(const Session *s, int which) {
+  const uint64_t fixed = which == 0 ? 3 : 2;  // embed + (lm head + sampler | cursor advance)
+  if (s->chain) return fixed + 1 + 2ull * s->layers;
+  if (s->front == 1) return fixed + 3ull * s->layers;
+  if (s->front == 2) return fixed + 4ull * s->layers;
+  return fixed + 5ull * s->layers;
+}
+
 // Launch one step: graph replay, or the same kernels eagerly (tracing mode).
 hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out);
 
@@ -432,7 +476,7 @@ hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *ou
   if (eager_steps()) {
     hipError_t err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
     if (err == hipSuccess)
-      out->kernel_launches += s->chain ? (which == 0 ? 4 : 3) + 2ull * s->layers : (which == 0 ? 3 : 2) + 5ull * s->layers;
+      out->kernel_launches += step_launches(s, which);
     return err;
   }
   hipError_t err = hipGraphLaunch(s->exec[which], s->stream);
@@ -505,7 +549,7 @@ bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
 // After a synchronisation: did a bounded wait of the chain kernel run out during the steps
 // just completed? Their tokens are then not to be trusted and the call fails.
 hipError_t chain_verdict(Session *s) {
-  if (!s->chain) return hipSuccess;
+  if (!s->chain && s->front == 0) return hipSuccess;
   uint32_t aborted = 0;
   const hipError_t err = hipMemcpy(&aborted, s->chain_abort, sizeof(aborted), hipMemcpyDeviceToHost);
   if (err != hipSuccess) return err;
@@ -667,6 +711,9 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
   const uint64_t off_chain_trace = c.take(static_cast<uint64_t>(rq->layer_count) * 32 * 8);
+  const uint64_t front_flags_bytes = front_flag_bytes(rq->heads, rq->kv_heads);
+  const uint64_t off_front_flags = c.take(front_flags_bytes);
+  const uint64_t off_attn_f32 = c.take(A * 4);
   s->arena_bytes = c.offset;
 
   if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
@@ -727,6 +774,29 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
     const char *trace = getenv("NERVA_HIP_CHAIN_TRACE");
     if (s->chain && trace != nullptr && trace[0] == '1')
       s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
+  }
+  s->front_flags = reinterpret_cast<uint32_t *>(s->arena + off_front_flags);
+  s->attn_f32 = reinterpret_cast<float *>(s->arena + off_attn_f32);
+  {
+    // Fused layer front (layer_front.cuh). Default where the shapes allow: attention + o
+    // projection as roles of one launch (mode 2, measured 1 % faster per step than one launch
+    // per piece). NERVA_HIP_FRONT=1 adds the qkv projection as a third role (measured 1 %
+    // slower: its hand-over costs more than the kernel boundary it removes), =0 keeps one
+    // launch per piece.
+    const char *want = getenv("NERVA_HIP_FRONT");
+    int mode = 2;
+    if (want != nullptr && want[0] >= '0' && want[0] <= '2') mode = want[0] - '0';
+    if (s->chain || rq->layer_count == 0 || !front_supported(rq->hidden, rq->heads, rq->kv_heads, rq->head_dim))
+      mode = 0;
+    s->front = mode;
+    // one KV tile in flight per wave there, so twice the stand-alone kernel's splits
+    uint32_t splits = (256 + rq->kv_heads - 1) / rq->kv_heads;
+    if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
+    if (splits > block_count) splits = block_count;
+    s->front_splits = splits == 0 ? 1 : splits;
+    const char *trace = getenv("NERVA_HIP_FRONT_TRACE");
+    if (s->front != 0 && trace != nullptr && trace[0] == '1')
+      s->front_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
   }
   s->layer.resize(L);
   for (uint32_t l = 0; l < L; ++l) {
@@ -809,6 +879,9 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_workspace_bytes(rq->heads, rq->head_dim), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_flags, 0, front_flags_bytes, s->stream);
+  if (err == hipSuccess && rq->layer_count > 0)
+    err = hipMemsetAsync(s->arena + off_chain_trace, 0, static_cast<uint64_t>(rq->layer_count) * 32 * 8, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
@@ -921,7 +994,7 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
     err = launch_step(s, 1, out);
   }
   if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
-  if (err == hipSuccess) out->kernel_launches += s->chain ? 4 + 2ull * s->layers : 3 + 5ull * s->layers;
+  if (err == hipSuccess) out->kernel_launches += step_launches(s, 0);
   if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
@@ -1189,15 +1262,20 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // back-to-back pass: all `layers` launches of one kind between a single event pair, so the
   // figure is the kernel's own duration without the per-launch event gaps
   uint64_t stream_ns[kLKinds] = {0};
-  for (int kind = kLQkv; err == hipSuccess && kind <= kLChain; ++kind) {
+  for (int kind = kLQkv; err == hipSuccess && kind <= kLFront; ++kind) {
     uint32_t launches = s->layers;
     if (kind == kLHead || kind == kLAdvance) continue;
     if (kind == kLQkv && s->chain) launches = 1;
     if ((kind == kLO || kind == kLGateUp || kind == kLDown) && s->chain) continue;
     if (kind == kLChain && !s->chain) continue;
+    if (kind == kLFront && s->front == 0) continue;
+    if ((kind == kLAttn || kind == kLO) && s->front != 0) continue;
+    if (kind == kLQkv && s->front == 1) continue;
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
-      err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
+      // no embed launch here, so the step counter stands still: the hand-over epochs repeat
+      err = hipMemsetAsync(s->front_flags, 0, front_flag_bytes(s->heads, s->kv_heads), s->stream);
+      if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
       if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
       if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
       if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
@@ -1223,6 +1301,27 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
       }
     }
   }
+  if (s->front_trace != nullptr) {
+    // timestamps (10 ns ticks from the launch's earliest mark) of: qkv workgroup 0 [0..3] and the last
+    // one's end [4]; attention (kv head 0, split 0) [8..13]; the merging workgroup of kv head 0 [16..18];
+    // first [20..23] and last [24..27] o workgroup
+    std::vector<uint64_t> tr(static_cast<size_t>(s->layers) * 32);
+    if (hipMemcpy(tr.data(), s->front_trace, tr.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+      for (uint32_t l = 0; l < s->layers && l < 4; ++l) {
+        const uint64_t *t = tr.data() + 32 * l;
+        uint64_t first = ~uint64_t{0};
+        for (int i = 0; i < 28; ++i)
+          if (t[i] != 0 && t[i] < first) first = t[i];
+        fprintf(stderr, "[front trace] layer %u:", l);
+        for (int i = 0; i < 28; ++i) {
+          if (i == 8 || i == 16 || i == 20 || i == 24) fprintf(stderr, " |");
+          if (t[i] != 0) fprintf(stderr, " %lld", static_cast<long long>(t[i] - first));
+          else fprintf(stderr, " -");
+        }
+        fprintf(stderr, "\n");
+      }
+    }
+  }
   // leave no epochs of this position behind: the sequence will run the step at `pos` for real
   err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
   if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
@@ -1237,6 +1336,9 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_stream_ns = stream_ns[kLGateUp];
   out->down_stream_ns = stream_ns[kLDown];
   out->chain_stream_ns = stream_ns[kLChain];
+  out->front_stream_ns = stream_ns[kLFront];
+  out->front_ns = counts[kLFront] ? sums[kLFront] / counts[kLFront] : 0;
+  out->front_mode = static_cast<uint32_t>(s->front);
   auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
   out->position = pos;
   out->embed_ns = avg(kLEmbed);
@@ -1261,21 +1363,24 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // stay on the device and are counted once, as the phase that reads them)
   out->chain_bytes = s->chain ? out->o_bytes + out->gate_up_bytes + out->down_bytes + out->qkv_bytes : 0;
   out->chain_enabled = s->chain ? 1u : 0u;
+  // fused front: the pieces it replaces (their hand-over vectors stay on the device)
+  out->front_bytes = s->front == 0 ? 0 : out->attention_bytes + out->o_bytes + (s->front == 1 ? out->qkv_bytes : 0);
   out->status = 0;
   return 0;
 }
 
-int nerva_hip_session_chain_state(NervaHipHfDecodeSequenceSession *s, uint32_t raise_abort, uint32_t *enabled,
+int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *s, uint32_t raise_abort, uint32_t *mode,
                                   uint32_t *aborted) {
   if (s == nullptr) return -1;
   if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
-  if (raise_abort != 0 && s->chain) {
+  const bool fused = s->chain || s->front != 0;
+  if (raise_abort != 0 && fused) {
     const uint32_t one = 1;
     if (hipMemcpy(s->chain_abort, &one, sizeof(one), hipMemcpyHostToDevice) != hipSuccess) return -1;
   }
   uint32_t flag = 0;
-  if (s->chain && hipMemcpy(&flag, s->chain_abort, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  if (enabled) *enabled = s->chain ? 1u : 0u;
+  if (fused && hipMemcpy(&flag, s->chain_abort, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  if (mode) *mode = s->chain ? NERVA_HIP_FUSED_CHAIN : (s->front == 1 ? NERVA_HIP_FUSED_FRONT : (s->front == 2 ? NERVA_HIP_FUSED_FRONT_ATTN_O : NERVA_HIP_FUSED_NONE));
   if (aborted) *aborted = flag;
   return 0;
 }

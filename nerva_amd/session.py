@@ -136,13 +136,16 @@ class DecodeSession:
         rc = self.lib.nerva_hip_session_profile_step(self.handle, repeats, C.byref(res))
         return rc, res
 
-    def chain_state(self, raise_abort=False):
-        """(enabled, aborted) of the persistent layer-chain kernel; raise_abort sets the abort word."""
-        enabled, aborted = C.c_uint32(0), C.c_uint32(0)
-        rc = self.lib.nerva_hip_session_chain_state(self.handle, int(raise_abort), C.byref(enabled), C.byref(aborted))
+    FUSED_NONE, FUSED_CHAIN, FUSED_FRONT, FUSED_FRONT_ATTN_O = 0, 1, 2, 3
+
+    def fused_state(self, raise_abort=False):
+        """(mode, aborted) of the kernels that hand data between workgroups inside a launch (fused layer
+        front / layer chain); raise_abort sets the abort word so that their bounded waits give up."""
+        mode, aborted = C.c_uint32(0), C.c_uint32(0)
+        rc = self.lib.nerva_hip_session_fused_state(self.handle, int(raise_abort), C.byref(mode), C.byref(aborted))
         if rc != 0:
-            raise RuntimeError("chain_state failed")
-        return bool(enabled.value), bool(aborted.value)
+            raise RuntimeError("fused_state failed")
+        return int(mode.value), bool(aborted.value)
 
     def logits(self):
         out = np.empty(self.vocab, np.float32)

@@ -179,18 +179,42 @@ GEOMETRIES = [
 ]
 
 
-@pytest.fixture(params=[False, True], ids=["launch-per-gemv", "chain-kernel"])
-def chain_mode(request, monkeypatch):
-    """Sessions created inside the test use the persistent layer-chain kernel when the shapes fit."""
-    if request.param:
-        monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
-    else:
-        monkeypatch.delenv("NERVA_HIP_CHAIN", raising=False)
+STEP_MODES = {
+    # id: (NERVA_HIP_FRONT, NERVA_HIP_CHAIN, fused_state mode of a session whose shapes fit)
+    "launch-per-piece": ("0", None, N.DecodeSession.FUSED_NONE),
+    "fused-front": ("1", None, N.DecodeSession.FUSED_FRONT),
+    "fused-attn-o": (None, None, N.DecodeSession.FUSED_FRONT_ATTN_O),   # the default
+    "chain-kernel": (None, "1", N.DecodeSession.FUSED_CHAIN),
+}
+
+
+def set_step_mode(monkeypatch, name):
+    front, chain, _ = STEP_MODES[name]
+    for var, val in (("NERVA_HIP_FRONT", front), ("NERVA_HIP_CHAIN", chain)):
+        if val is None:
+            monkeypatch.delenv(var, raising=False)
+        else:
+            monkeypatch.setenv(var, val)
+
+
+def mode_fits(name, hidden, heads, kv, hd):
+    """Whether a session of these shapes actually takes the kernels the mode asks for."""
+    if name == "launch-per-piece":
+        return True
+    if name == "chain-kernel":
+        return hidden % 2048 == 0
+    return hd == 128 and heads == 4 * kv and hidden % 512 == 0 and hidden <= 4096 and heads * hd <= 4096
+
+
+@pytest.fixture(params=list(STEP_MODES), ids=list(STEP_MODES))
+def step_mode(request, monkeypatch):
+    """Sessions created inside the test build their step from these kernels when the shapes fit."""
+    set_step_mode(monkeypatch, request.param)
     return request.param
 
 
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_single_layer_short_prompt_is_tight(geom, chain_mode):
+def test_single_layer_short_prompt_is_tight(geom, step_mode):
     """One layer and a 1- or 2-token prompt leave no room for 16-bit ties to compound: the whole
     step (embed, norms, GEMVs, RoPE, attention, LM head) must agree with the oracle at 1e-3 in
     f16. In bf16 a single value that sits within 1e-6 of a rounding boundary (attention output,
@@ -198,11 +222,12 @@ def test_single_layer_short_prompt_is_tight(geom, chain_mode):
     one activation by 2^-8 relative and the logits of this tiny model by up to ~3e-3: the bound
     is one such flip, 6e-3."""
     dtype, hidden, heads, kv, hd, inter, vocab, _, theta, qk_norm, bias = geom
-    if chain_mode and hidden % 2048:
-        pytest.skip("shapes do not fit the chain kernel: same path as launch-per-gemv")
+    if not mode_fits(step_mode, hidden, heads, kv, hd):
+        pytest.skip("shapes do not fit this mode's kernels: same path as launch-per-piece")
     tol = REL_L2 if dtype == F16 else 6e-3
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, 1, hidden + 1, theta, qk_norm, bias)
     s = N.DecodeSession.create(weights, 32)
+    assert s.fused_state() == (STEP_MODES[step_mode][2], False)
     for prompt in ([3], [vocab - 1, 11]):
         ctx = O.Context(omodel, 32, staging=1)
         for i, t in enumerate(prompt):
@@ -227,10 +252,10 @@ def test_single_layer_short_prompt_is_tight(geom, chain_mode):
 
 
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_session_matches_oracle_logits_kv_and_stream(geom, chain_mode):
+def test_session_matches_oracle_logits_kv_and_stream(geom, step_mode):
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
-    if chain_mode and hidden % 2048:
-        pytest.skip("shapes do not fit the chain kernel: same path as launch-per-gemv")
+    if not mode_fits(step_mode, hidden, heads, kv, hd):
+        pytest.skip("shapes do not fit this mode's kernels: same path as launch-per-piece")
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, hidden, theta, qk_norm, bias)
     prompt = np.random.default_rng(1).integers(0, vocab, 21).astype(np.uint32)
     steps = 24
@@ -294,7 +319,8 @@ def test_eager_profile_pass_leaves_state_untouched():
     s.start(prompt)
     rc, res, a = s.advance(4)
     rc, prof = s.profile_step(2)
-    assert rc == 0 and prof.status == 0 and prof.launches == 3 + 5 * 2
+    assert rc == 0 and prof.status == 0 and prof.front_mode == 2 and prof.launches == 3 + 4 * 2
+    assert prof.front_ns > 0 and prof.front_stream_ns > 0 and prof.front_bytes > 0 and prof.attention_ns == 0
     assert prof.gate_up_ns > 0 and prof.lm_head_ns > 0 and prof.position == len(prompt) + 3
     rc, res, b = s.advance(6)
     s.start(prompt)
@@ -349,7 +375,7 @@ def test_chain_kernel_is_used_and_agrees_with_one_launch_per_gemv(monkeypatch):
     prompt = np.random.default_rng(2).integers(0, vocab, 19).astype(np.uint32)
     monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
     s = N.DecodeSession.create(weights, 64)
-    assert s.chain_state() == (True, False)
+    assert s.fused_state() == (s.FUSED_CHAIN, False)
     rc, res = s.start(prompt)
     assert rc == 0
     rc, res, chained = s.advance(12)
@@ -362,8 +388,9 @@ def test_chain_kernel_is_used_and_agrees_with_one_launch_per_gemv(monkeypatch):
     assert rc == 0
     s.destroy()
     monkeypatch.delenv("NERVA_HIP_CHAIN")
+    monkeypatch.setenv("NERVA_HIP_FRONT", "0")
     s = N.DecodeSession.create(weights, 64)
-    assert s.chain_state() == (False, False)
+    assert s.fused_state() == (s.FUSED_NONE, False)
     s.start(prompt)
     rc, res, plain = s.advance(12)
     assert rc == 0 and res.graph_nodes == 3 + 5 * layers
@@ -383,11 +410,65 @@ def test_chain_kernel_bounded_wait_gives_up_cleanly(monkeypatch):
     rc, res = s.start([1, 2, 3])
     rc, res, good = s.advance(3)
     assert rc == 0
-    assert s.chain_state(raise_abort=True) == (True, True)
+    assert s.fused_state(raise_abort=True) == (s.FUSED_CHAIN, True)
     rc, res, _ = s.advance(2)
     assert rc == -1 and res.status == -1 and res.hip_error != 0
     rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
-    assert rc == 0 and s.chain_state() == (True, False)
+    assert rc == 0 and s.fused_state() == (s.FUSED_CHAIN, False)
+    rc, res, again = s.advance(3)
+    assert rc == 0 and again.tolist() == good.tolist()
+    s.destroy()
+
+
+FRONT_GEOM = (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False)
+
+
+def test_fused_front_modes_agree_with_one_launch_per_piece(monkeypatch):
+    """Shapes that fit run qkv + attention + o as roles of one launch (3 launches per layer). The
+    GEMV roles sum in the same order as the stand-alone kernels and the attention role differs only
+    in how keys are grouped into splits, so logits agree to 16-bit-tie noise."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = FRONT_GEOM
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 91, theta, qk_norm, bias)
+    prompt = np.random.default_rng(5).integers(0, vocab, 37).astype(np.uint32)
+    results = {}
+    for name in ("fused-front", "fused-attn-o", "launch-per-piece"):
+        set_step_mode(monkeypatch, name)
+        s = N.DecodeSession.create(weights, 96)
+        assert s.fused_state() == (STEP_MODES[name][2], False)
+        rc, res = s.start(prompt)
+        assert rc == 0
+        rc, res, tokens = s.advance(40)               # crosses 16-token block boundaries
+        per_layer = {"fused-front": 3, "fused-attn-o": 4, "launch-per-piece": 5}[name]
+        assert rc == 0 and res.graph_nodes == 3 + per_layer * layers and res.hot_path_allocations == 0
+        rc, prof = s.profile_step(2)
+        assert rc == 0 and prof.launches == 3 + per_layer * layers
+        rc, res, more = s.advance(4)                  # profiling did not disturb the sequence
+        assert rc == 0
+        results[name] = (tokens.tolist() + more.tolist(), s.logits())
+        s.destroy()
+    ref_tokens, ref_logits = results["launch-per-piece"]
+    for name in ("fused-front", "fused-attn-o"):
+        tokens, logits = results[name]
+        assert rel_l2(logits, ref_logits) <= E2E_REL_L2
+        assert tokens[:8] == ref_tokens[:8]
+
+
+def test_fused_front_bounded_wait_gives_up_cleanly(monkeypatch):
+    """With the abort word raised from the host every in-kernel wait of the fused front gives up
+    at once: all kernels still run to completion, the call reports the failure, and start() makes
+    the session usable again."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = FRONT_GEOM
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 92, theta, qk_norm, bias)
+    set_step_mode(monkeypatch, "fused-front")
+    s = N.DecodeSession.create(weights, 32)
+    rc, res = s.start([1, 2, 3])
+    rc, res, good = s.advance(3)
+    assert rc == 0
+    assert s.fused_state(raise_abort=True) == (s.FUSED_FRONT, True)
+    rc, res, _ = s.advance(2)
+    assert rc == -1 and res.status == -1 and res.hip_error != 0
+    rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
+    assert rc == 0 and s.fused_state() == (s.FUSED_FRONT, False)
     rc, res, again = s.advance(3)
     assert rc == 0 and again.tolist() == good.tolist()
     s.destroy()
