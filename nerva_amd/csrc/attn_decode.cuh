@@ -53,12 +53,14 @@ struct AttnParams {
   float eps;
   const uint32_t *cursor;      // device position, or null -> `position`
   uint32_t position, max_steps, append;
+  uint64_t *trace;             // tuning aid: [32] device timestamps of selected workgroups' stages, or null
 };
 
-// Split-KV factor: every active split adds a partial for the last workgroup of its kv head to
-// merge, so the grid is kept to about 128 workgroups of 8 waves (kv_heads x splits).
+// Split-KV factor. The matrix-core kernel keeps one 8-wave workgroup per CU, so kv_heads x splits
+// stays within the 256 CUs (a second round of workgroups costs more than the shorter tile loops
+// save); within that, more splits mean fewer 16-token tiles per wave in a row.
 inline uint32_t attn_default_splits(uint32_t kv_heads, uint32_t block_count) {
-  uint32_t splits = (128 + kv_heads - 1) / (kv_heads == 0 ? 1 : kv_heads);
+  uint32_t splits = 256 / (kv_heads == 0 ? 1 : kv_heads);
   if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
   if (splits > block_count) splits = block_count;
   return splits == 0 ? 1 : splits;

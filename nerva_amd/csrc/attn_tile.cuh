@@ -18,19 +18,12 @@ constexpr int kAttnWaves = 8;   // waves per workgroup of the fast path (group 8
 // copy is stored too (K/V that go to the cache).
 // rope_cs (optional): cos at [i], sin at [64 + i] of this step's angles, computed once
 // per step; without it the angle pos / rope_freq[i] is evaluated here.
-template <uint32_t DT, bool COHERENT = false>
-__device__ __forceinline__ void prep_head128(const float *src, const uint16_t *bias,
+// (x0, x1) = raw projection values of dims (lane, lane + 64).
+template <uint32_t DT>
+__device__ __forceinline__ void prep_head128(float x0, float x1, const uint16_t *bias,
                                              const uint16_t *gamma, const float *rope_freq,
                                              const float *rope_cs, uint32_t pos, float eps, int lane,
                                              float *out, uint16_t *out16) {
-  float x0, x1;
-  if constexpr (COHERENT) {  // src was written by another workgroup of this launch
-    x0 = __hip_atomic_load(src + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    x1 = __hip_atomic_load(src + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  } else {
-    x0 = src[lane];
-    x1 = src[lane + 64];
-  }
   if (bias != nullptr) {
     x0 += dec16<DT>(bias[lane]);
     x1 += dec16<DT>(bias[lane + 64]);
@@ -106,11 +99,23 @@ __device__ __forceinline__ float row_shr(float v) {
 
 // v = hi + lo with hi, lo 16-bit: the pair carries 16 (bf16) / 22 (f16) mantissa bits, so a
 // matrix-core product against exact 16-bit K/V data loses nothing that matters to f32 math.
+// Finite inputs only (the hardware conversions round to nearest even like enc16; they differ
+// from it in the NaN bit pattern alone, and neither a scaled query nor a probability is NaN).
+template <uint32_t DT>
+__device__ __forceinline__ uint16_t enc16_finite(float v) {
+  if constexpr (DT == kBF16) return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));  // v_cvt_pk_bf16_f32
+  else return f32_to_f16(v);
+}
 template <uint32_t DT>
 __device__ __forceinline__ void split16(float v, uint16_t &hi, uint16_t &lo) {
-  hi = enc16<DT>(v);
-  lo = enc16<DT>(v - dec16<DT>(hi));
+  hi = enc16_finite<DT>(v);
+  lo = enc16_finite<DT>(v - dec16<DT>(hi));
 }
+// Softmax arithmetic runs in base 2: the query is pre-scaled by log2(e) / sqrt(d), so scores, the
+// running maxima m and every exchanged partial maximum are log2-domain numbers and
+// exp(s - m) is one v_exp_f32. exp2(-inf) = 0.
+__device__ __forceinline__ float attn_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+constexpr float kLog2e = 1.4426950408889634f;
 
 // Device-scope coherent accesses: written through / read around the XCD-local L2, so data
 // exchanged between workgroups inside one kernel needs no cache flush or invalidate.
@@ -190,12 +195,12 @@ __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], co
   mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
   mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
   const float m_new = fmaxf(m, mb);   // finite: every processed tile has a valid token
-  const float alpha = expf(m - m_new);
+  const float alpha = attn_exp2(m - m_new);
   uint32_t px[2];
   float psum = 0.0f;
 #pragma unroll
   for (int r = 0; r < 4; r += 2) {
-    const float p0 = expf(sc[r] - m_new), p1 = expf(sc[r + 1] - m_new);
+    const float p0 = attn_exp2(sc[r] - m_new), p1 = attn_exp2(sc[r + 1] - m_new);
     psum += p0 + p1;
     uint16_t h0, l0, h1, l1;
     split16<DT>(p0, h0, l0);
@@ -225,31 +230,105 @@ struct AttnShared {
   float wf[W][G];   // exp(m_w - M_g), 0 for idle waves
   float bM[G];
   uint32_t is_last;
-  alignas(16) uint4 qx_s[4][kWave];  // linked launches: the query operand of the first product
+  // linked launches: the query operand of the first product; m, l and exp(m - M) of the splits
+  alignas(16) uint4 qx_s[4][kWave];
+  float pm[G][kAttnMaxSplits], pl[G][kAttnMaxSplits], pf[G][kAttnMaxSplits];
 };
+
+// ---- hand-over between workgroups of one launch ------------------------------------------
+// A value that another workgroup of the same launch consumes travels as one 8-byte word
+// (f32 value, epoch): the consumer polls the word with device-coherent loads until the epoch is
+// the current one. A single aligned 8-byte store is indivisible, so a matching epoch proves
+// the value; no flag, no "stores performed" wait, no cache flush is needed on either side.
+// Epochs (step counter x layers + layer + 1) never repeat within a session.
+__device__ __forceinline__ void store_tagged(uint64_t *ptr, float v, uint32_t epoch) {
+  __hip_atomic_store(ptr, (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t load_tagged(const uint64_t *ptr) {
+  return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool tag_is(uint64_t word, uint32_t epoch) {
+  return static_cast<uint32_t>(word >> 32) == epoch;
+}
+__device__ __forceinline__ float tag_value(uint64_t word) { return __uint_as_float(static_cast<uint32_t>(word)); }
+
+// The attention output travels as (two 16-bit values, epoch) words: element pair (2i, 2i + 1) in
+// word i. `bits` = this lane's rounded element; lanes with an even element index store.
+__device__ __forceinline__ void store_tagged_pair16(uint64_t *out_words, uint32_t elem, uint32_t bits, uint32_t epoch) {
+  const uint32_t next = static_cast<uint32_t>(__shfl_down(static_cast<int>(bits), 1, kWave));
+  if ((elem & 1u) == 0u)
+    __hip_atomic_store(out_words + elem / 2, (static_cast<uint64_t>(epoch) << 32) | bits | (next << 16),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr uint32_t kLinkSpinLimit = 1u << 20;
+// One more unsuccessful poll: true when the wait has to be given up (limit reached, or the
+// abort word is up); raises the abort word then. Pauses the wave briefly otherwise.
+__device__ __forceinline__ bool link_give_up(uint32_t *abort_flag, uint32_t &spins) {
+  ++spins;
+  if (spins > kLinkSpinLimit || ((spins & 15u) == 0u && load_coherent(abort_flag) != 0u)) {
+    store_coherent(abort_flag, 1u);
+    return true;
+  }
+  __builtin_amdgcn_s_sleep(2);
+  return false;
+}
+
+constexpr int kTicketRound = 32;           // splits read per round by the last workgroup of the ticket protocol
+constexpr int kMergeRound = 16;            // splits polled per round by the merging workgroup
+constexpr uint32_t kPartRecord = kHD + 2;  // tagged words of one (head, split) partial: acc[128], m, l
 
 // Connections of an attention workgroup to the other roles of a fused launch.
 struct AttnLink {
-  const uint32_t *wait_flags;  // [wait_count <= 64] producer flags to wait for, or null
-  uint32_t wait_count;
-  uint32_t *done_flag;         // this kv head's flag, raised to `epoch` when its output is visible
-  float *out_coherent;         // [heads * 128] f32 output for the consumer role
+  const uint64_t *qkv_tagged;  // [A + 2 KV] q|k|v written by the qkv role of this launch, or null: p.qkv
+  uint64_t *part_tagged;       // [heads][splits][kPartRecord] split partials
+  uint64_t *out_tagged;        // [heads * 64] final output for the consumer role, two 16-bit elements per word
+  // hints for the consumers' cheap first wait: word [i * hint_stride + kvh] belongs to consumer
+  // workgroup i alone (a word polled by every consumer would make its memory channel the
+  // bottleneck of the whole launch); raised to `epoch` right before the output is stored
+  uint32_t *hints;
+  uint32_t hint_count, hint_stride;
+  uint32_t *split_hints;       // [kv_heads][kAttnMaxSplits] "this split's partial has been stored"
   uint32_t *abort_flag;        // raised when a bounded wait ran out
   uint32_t epoch;
   uint64_t *trace;             // tuning aid: device timestamps of this workgroup's stages, or null
   uint64_t *trace_merge;       // same for the workgroup that merges this kv head's splits
 };
+__device__ __forceinline__ void attn_raise_hints(const AttnLink &link, uint32_t kvh) {
+  for (uint32_t i = threadIdx.x; i < link.hint_count; i += blockDim.x)
+    store_coherent(link.hints + i * link.hint_stride + kvh, link.epoch);
+}
 __device__ __forceinline__ void link_mark(uint64_t *trace, int slot) {
   if (trace != nullptr && threadIdx.x == 0) trace[slot] = wall_clock64();
 }
-constexpr uint32_t kLinkSpinLimit = 1u << 20;
 
-// Every wave's output stores have to be performed before one lane raises the flag.
-__device__ __forceinline__ void attn_publish(const AttnLink &link, uint32_t kvh) {
-  wait_stores_performed();
-  __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(link.done_flag, link.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  (void)kvh;
+// Raw projection values (lane, lane + 64) of the 128-wide head that starts at element `off`.
+template <bool LINKED>
+__device__ __forceinline__ void load_head128(const float *qkv, const AttnLink &link, uint32_t off, int lane,
+                                             float &x0, float &x1) {
+  if constexpr (LINKED) {
+    if (link.qkv_tagged != nullptr) {
+      uint64_t r0, r1;
+      uint32_t spins = 0;
+      // a long wait: watch one word per wave (a single request), poll the whole head once it is there
+      while (!tag_is(load_tagged(link.qkv_tagged + off), link.epoch)) {
+        if (link_give_up(link.abort_flag, spins)) break;
+        __builtin_amdgcn_s_sleep(16);
+      }
+      for (;;) {
+        r0 = load_tagged(link.qkv_tagged + off + lane);
+        r1 = load_tagged(link.qkv_tagged + off + lane + 64);
+        if (__all(tag_is(r0, link.epoch) && tag_is(r1, link.epoch))) break;
+        if (link_give_up(link.abort_flag, spins)) break;
+      }
+      x0 = tag_value(r0);
+      x1 = tag_value(r1);
+      return;
+    }
+  }
+  x0 = qkv[off + lane];
+  x1 = qkv[off + lane + 64];
 }
 
 // W waves per workgroup. A workgroup owns one kv head and one contiguous range of
@@ -266,9 +345,9 @@ __device__ __forceinline__ void attn_publish(const AttnLink &link, uint32_t kvh)
 // 1 KiB instruction and lands in the registers the matrix core reads.
 //
 // LINKED = the workgroup is the attention role of a launch that also holds its producer and/or
-// consumer (AttnLink): it may wait for flags before it reads q/k/v (its first tiles are already
-// requested by then), reads q/k/v with device-coherent loads, publishes the final output with
-// device-coherent stores as well and raises the kv head's flag once they have been performed.
+// consumer (AttnLink). Its first tile is requested before it polls for q/k/v; partials and the
+// final output leave as tagged words; split 0 of a kv head merges (it polls the other splits'
+// partials instead of taking a ticket), so nobody waits for stores to be performed.
 template <uint32_t DT, int G, int W, bool LINKED>
 __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32_t pos, const uint32_t kvh,
                                                const uint32_t split, const uint32_t S, AttnShared<G, W> &sh,
@@ -285,6 +364,9 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
+  // tuning aid: stage timestamps of workgroup (kv head 0, split 0) and of kv head 0's merging workgroup
+  uint64_t *const tr = LINKED ? link.trace : (kvh == 0 && split == 0 ? p.trace : nullptr);
+  uint64_t *const trm = LINKED ? link.trace_merge : (kvh == 0 ? p.trace : nullptr);
   const uint32_t n_keys = pos + 1;
   const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
   // at least W tiles per active split so that every wave of a workgroup has work
@@ -306,44 +388,30 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   uint32_t b = b0 + wave;
   if (b < b1) attn_load_tile(p, b, kvh, lane, kreg, vreg);
 
-  if constexpr (LINKED) link_mark(link.trace, 8);
-  if constexpr (LINKED) {
-    // ---- the producer of q/k/v runs in the same launch: wait for its rows (bounded)
-    if (link.wait_flags != nullptr) {
-      if (wave == 0) {
-        uint32_t spins = 0;
-        bool ok = true;
-        for (;;) {
-          const bool mine = static_cast<uint32_t>(lane) >= link.wait_count ||
-                            static_cast<int32_t>(load_coherent(link.wait_flags + lane) - link.epoch) >= 0;
-          if (__all(mine)) break;
-          if (++spins > kLinkSpinLimit || load_coherent(link.abort_flag) != 0u) {
-            ok = false;
-            break;
-          }
-        }
-        if (!ok && lane == 0) store_coherent(link.abort_flag, 1u);
-      }
-      __syncthreads();
-    }
-    link_mark(link.trace, 9);
-  }
+  link_mark(tr, 8);
   // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
   for (int g = wave; g < G; g += W) {
     const uint32_t h = kvh * G + g;
-    prep_head128<DT, LINKED>(p.qkv + h * kHD, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq,
-                     p.rope_cs, pos, p.eps, lane, q_s[g], nullptr);
+    float x0, x1;
+    load_head128<LINKED>(p.qkv, link, h * kHD, lane, x0, x1);
+    prep_head128<DT>(x0, x1, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq, p.rope_cs, pos, p.eps,
+                     lane, q_s[g], nullptr);
   }
   if (owns_new) {
     if (wave == (G % W)) {
-      prep_head128<DT, LINKED>(p.qkv + A + kvh * kHD, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm,
-                       p.rope_freq, p.rope_cs, pos, p.eps, lane, nullptr, knew);
+      float x0, x1;
+      load_head128<LINKED>(p.qkv, link, A + kvh * kHD, lane, x0, x1);
+      prep_head128<DT>(x0, x1, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm, p.rope_freq, p.rope_cs, pos,
+                       p.eps, lane, nullptr, knew);
     } else if (wave == ((G + 1) % W)) {
-      prep_head128<DT, LINKED>(p.qkv + A + KV + kvh * kHD, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr,
-                       nullptr, nullptr, pos, p.eps, lane, nullptr, vnew);
+      float x0, x1;
+      load_head128<LINKED>(p.qkv, link, A + KV + kvh * kHD, lane, x0, x1);
+      prep_head128<DT>(x0, x1, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr, nullptr, nullptr, pos, p.eps,
+                       lane, nullptr, vnew);
     }
   }
   __syncthreads();
+  link_mark(tr, 9);
   if (owns_new && wave == 0) {
     // publish the rounded row to the cache in operand order
     const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[new_block], kvh);
@@ -359,7 +427,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   }
 
   const int col = lane & 15, grp = lane >> 4;
-  const float scale = 1.0f / sqrtf(static_cast<float>(kHD));
+  const float scale = kLog2e / sqrtf(static_cast<float>(kHD));
 
   // B operand of the first product: column `col` of Qx for dims j*32 + grp*8 .. +7
   uint4 qx[4];
@@ -387,7 +455,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     qx_lds = &sh.qx_s[0][lane];
   }
 
-  if constexpr (LINKED) link_mark(link.trace, 10);
+  link_mark(tr, 10);
   float m = -INFINITY, l = 0.0f;  // of column `col` (both copies of a head track the same values)
   f32x4_t acc[8];                  // O^T[dims s*16 + grp*4 .. +3][col]
 #pragma unroll
@@ -410,7 +478,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     }
   }
 
-  if constexpr (LINKED) link_mark(link.trace, 11);
+  link_mark(tr, 11);
   // ---- wave result: tokens of the four lane groups, then hi + lo columns; then the W waves
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
@@ -434,7 +502,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     float M = -INFINITY;
 #pragma unroll
     for (int w2 = 0; w2 < W; ++w2) M = fmaxf(M, wm[w2][g]);
-    wf[w][g] = wm[w][g] > -INFINITY ? expf(wm[w][g] - M) : 0.0f;
+    wf[w][g] = wm[w][g] > -INFINITY ? attn_exp2(wm[w][g] - M) : 0.0f;
     if (w == 0) bM[g] = M;
   }
   __syncthreads();
@@ -451,8 +519,16 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
       // a single split holds every key: this is the final result, nothing to exchange
       if (L > 0.0f && isfinite(L)) o /= L;
       if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
-      p.out16[h * kHD + d] = enc16<DT>(o);
-      if constexpr (LINKED) store_coherent(link.out_coherent + h * kHD + d, o);
+      const uint16_t o16 = enc16<DT>(o);
+      p.out16[h * kHD + d] = o16;
+      if constexpr (LINKED) store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
+    } else if constexpr (LINKED) {
+      uint64_t *rec = link.part_tagged + (static_cast<uint64_t>(h) * S + split) * kPartRecord;
+      store_tagged(rec + d, o, link.epoch);
+      if (d == 0) {
+        store_tagged(rec + kHD, bM[g], link.epoch);
+        store_tagged(rec + kHD + 1, L, link.epoch);
+      }
     } else {
       // The partial leaves through device-coherent stores (written through, no cache flush).
       store_coherent(p.part_acc + (static_cast<uint64_t>(h) * S + split) * kHD + d, o);
@@ -463,49 +539,155 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     }
   }
   if (active == 1) {
-    if constexpr (LINKED) attn_publish(link, kvh);
+    if constexpr (LINKED) {
+      attn_raise_hints(link, kvh);
+    }
+    return;
+  }
+  if constexpr (LINKED) {
+    // ---- split 0 merges: every thread owns one output element (g, d) and polls that element of
+    // every split's partial, kMergeRound splits per round; the first G * active threads also fetch the
+    // splits' m and l. Whatever has not arrived yet is simply polled again.
+    static_assert(!LINKED || G * kHD == kThreads, "one output element per thread");
+    // Tell the merging workgroup that this split's partial is in place: once the stores have
+    // been performed one word is raised. It is a hint (the tags decide), but a reliable one.
+    wait_stores_performed();
+    __syncthreads();
+    if (threadIdx.x == 0) store_coherent(link.split_hints + kvh * kAttnMaxSplits + split, link.epoch);
+    link_mark(tr, 12);
+    if (split != 0) return;
+    link_mark(trm, 16);
+    if (wave == 0) {
+      uint32_t spins = 0;
+      for (;;) {
+        const bool mine = static_cast<uint32_t>(lane) >= active ||
+                          load_coherent(link.split_hints + kvh * kAttnMaxSplits + lane) == link.epoch;
+        if (__all(mine)) break;
+        if (link_give_up(link.abort_flag, spins)) break;
+      }
+    }
+    __syncthreads();
+    link_mark(trm, 18);
+    const int g = threadIdx.x / kHD, d = threadIdx.x % kHD;
+    const uint32_t h = kvh * G + g;
+    const uint64_t *rec = link.part_tagged + static_cast<uint64_t>(h) * S * kPartRecord;
+    const bool has_ml = threadIdx.x < G * active;
+    const uint32_t g2 = has_ml ? threadIdx.x / active : 0u, s2 = has_ml ? threadIdx.x % active : 0u;
+    const uint64_t *rec_ml = link.part_tagged + (static_cast<uint64_t>(kvh * G + g2) * S + s2) * kPartRecord + kHD;
+    float o = 0.0f, L = 0.0f;
+    for (uint32_t s0 = 0; s0 < active; s0 += kMergeRound) {
+      // First through the ordinary load path: the splits of a kv head run on the XCD of the merging
+      // workgroup when workgroups are dealt to XCDs round robin and kv_heads is a multiple of the XCD
+      // count, so their written-through partials are current in the L2 these loads go to, and
+      // ordinary loads are many times faster than device-coherent ones (which this CU can only keep
+      // a few of in flight). The tags tell when that did not hold: then the round is polled again
+      // with device-coherent loads, which are right wherever the writers ran.
+      // Every load of a round is unconditional (indices past the last split are clamped to it):
+      // a load under a branch makes the compiler wait for all earlier loads at the join, which
+      // would turn the round into sixteen round trips in a row.
+      uint64_t av[kMergeRound], mv, lv;
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < kMergeRound; ++i)
+        av[i] = rec[static_cast<uint64_t>(min(s0 + i, active - 1)) * kPartRecord + d];
+      mv = rec_ml[0];
+      lv = rec_ml[1];
+#pragma unroll
+      for (int i = 0; i < kMergeRound; ++i) ok = ok & tag_is(av[i], link.epoch);
+      ok = ok & tag_is(mv, link.epoch) & tag_is(lv, link.epoch);
+      uint32_t spins = 0;
+      while (!__all(ok)) {
+        if (link_give_up(link.abort_flag, spins)) break;
+#pragma unroll
+        for (int i = 0; i < kMergeRound; ++i)
+          av[i] = load_tagged(rec + static_cast<uint64_t>(min(s0 + i, active - 1)) * kPartRecord + d);
+        mv = load_tagged(rec_ml);
+        lv = load_tagged(rec_ml + 1);
+        ok = true;
+#pragma unroll
+        for (int i = 0; i < kMergeRound; ++i) ok = ok & tag_is(av[i], link.epoch);
+        ok = ok & tag_is(mv, link.epoch) & tag_is(lv, link.epoch);
+      }
+      if (link.trace_merge != nullptr && threadIdx.x == 0) {
+        link.trace_merge[s0 == 0 ? 19 : 5] = wall_clock64();
+        link.trace_merge[s0 == 0 ? 6 : 7] = spins + 1;  // raw count (debugging aid)
+      }
+      if (s0 == 0) {
+        if (has_ml) {
+          sh.pm[g2][s2] = tag_value(mv);
+          sh.pl[g2][s2] = tag_value(lv);
+        }
+        __syncthreads();
+        if (has_ml) {
+          float M = -INFINITY;
+          for (uint32_t s = 0; s < active; ++s) M = fmaxf(M, sh.pm[g2][s]);
+          sh.pf[g2][s2] = attn_exp2(sh.pm[g2][s2] - M);  // every active split saw at least one key: m is finite
+        }
+        __syncthreads();
+        for (uint32_t s = 0; s < active; ++s) L = fmaf(sh.pl[g][s], sh.pf[g][s], L);
+      }
+#pragma unroll
+      for (int i = 0; i < kMergeRound; ++i)
+        if (s0 + i < active) o = fmaf(tag_value(av[i]), sh.pf[g][s0 + i], o);
+    }
+    if (L > 0.0f && isfinite(L)) o /= L;
+    // pollers of the output may start now: it follows within one store latency
+    attn_raise_hints(link, kvh);
+    if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
+    const uint16_t o16 = enc16<DT>(o);
+    p.out16[h * kHD + d] = o16;
+    store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
+    link_mark(trm, 17);
     return;
   }
   // Every wave waits until its own stores have been performed, the barrier collects the waves,
   // and only then one lane takes the arrival ticket of this kv head.
   wait_stores_performed();
   __syncthreads();
-  if constexpr (LINKED) link_mark(link.trace, 12);
+  link_mark(tr, 12);
   if (threadIdx.x == 0) {
     const uint32_t ticket =
         __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     sh.is_last = ticket == active - 1 ? 1u : 0u;
   }
   __syncthreads();
-  if constexpr (LINKED) link_mark(link.trace, 13);
+  link_mark(tr, 13);
   if (!sh.is_last) return;
-  if constexpr (LINKED) link_mark(link.trace_merge, 16);
+  link_mark(trm, 16);
   // ---- the last workgroup of this kv head merges the splits. Each thread owns (g, d) and reads
-  // the partials with device-coherent loads, sixteen splits per round trip, in split order.
+  // the partials with device-coherent loads, kTicketRound splits per round trip, in split order.
   for (int e = threadIdx.x; e < G * kHD; e += kThreads) {
     const int g = e / kHD, d = e % kHD;
     const uint32_t h = kvh * G + g;
     const float *pm = p.part_m + h * S, *pl = p.part_l + h * S;
     const float *src = p.part_acc + static_cast<uint64_t>(h) * S * kHD + d;
     float M = -INFINITY, L = 0.0f, o = 0.0f;
-    for (uint32_t s0 = 0; s0 < active; s0 += 16) {
-      float mm[16], ll[16], aa[16];
+    for (uint32_t s0 = 0; s0 < active; s0 += kTicketRound) {
+      float mm[kTicketRound], ll[kTicketRound], aa[kTicketRound];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < kTicketRound; ++i) {
+        // unconditional loads (index clamped): a load under a branch would serialise the round
+        const uint32_t si = min(s0 + i, active - 1);
+        mm[i] = load_coherent(pm + si);
+        ll[i] = load_coherent(pl + si);
+        aa[i] = load_coherent(src + static_cast<uint64_t>(si) * kHD);
+      }
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
         const bool on = s0 + i < active;
-        mm[i] = on ? load_coherent(pm + s0 + i) : -INFINITY;
-        ll[i] = on ? load_coherent(pl + s0 + i) : 0.0f;
-        aa[i] = on ? load_coherent(src + static_cast<uint64_t>(s0 + i) * kHD) : 0.0f;
+        mm[i] = on ? mm[i] : -INFINITY;
+        ll[i] = on ? ll[i] : 0.0f;
+        aa[i] = on ? aa[i] : 0.0f;
       }
       float Mc = M;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) Mc = fmaxf(Mc, mm[i]);
-      const float keep = M > -INFINITY ? expf(M - Mc) : 0.0f;
+      for (int i = 0; i < kTicketRound; ++i) Mc = fmaxf(Mc, mm[i]);
+      const float keep = M > -INFINITY ? attn_exp2(M - Mc) : 0.0f;
       L *= keep;
       o *= keep;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float f = mm[i] > -INFINITY ? expf(mm[i] - Mc) : 0.0f;
+      for (int i = 0; i < kTicketRound; ++i) {
+        const float f = mm[i] > -INFINITY ? attn_exp2(mm[i] - Mc) : 0.0f;
         L = fmaf(ll[i], f, L);
         o = fmaf(aa[i], f, o);
       }
@@ -514,14 +696,9 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     if (L > 0.0f && isfinite(L)) o /= L;
     if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
     p.out16[h * kHD + d] = enc16<DT>(o);
-    if constexpr (LINKED) store_coherent(link.out_coherent + h * kHD + d, o);
   }
   if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if constexpr (LINKED) {
-    link_mark(link.trace_merge, 17);
-    attn_publish(link, kvh);
-    link_mark(link.trace_merge, 18);
-  }
+  link_mark(trm, 17);
 }
 
 }  // namespace attn

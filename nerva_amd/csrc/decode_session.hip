@@ -102,8 +102,7 @@ struct NervaHipHfDecodeSequenceSession {
   // 2 attention + o only (the qkv projection stays a launch of its own)
   int front = 0;
   uint32_t front_splits = 1;
-  uint32_t *front_flags = nullptr;
-  float *attn_f32 = nullptr;
+  void *front_ws = nullptr;  // tagged hand-over buffers of the fused front
   uint64_t *front_trace = nullptr;  // NERVA_HIP_FRONT_TRACE=1: per-layer timestamps of selected workgroups
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
@@ -159,6 +158,10 @@ __global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prom
     state[0] = cursor;
     state[1] = prompt_count;
   }
+}
+
+__global__ void bump_step_counter_kernel(uint32_t *state) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) state[2] = state[2] + 1u;
 }
 
 __global__ void advance_cursor_kernel(uint32_t *state, uint32_t max_steps) {
@@ -287,6 +290,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
       p.append = 1;
+      p.trace = s->front == 0 && s->front_trace != nullptr ? s->front_trace + 32 * l : nullptr;
       if (s->front != 0) {
         // qkv rows, attention splits and o rows as roles of one launch
         FrontParams f{};
@@ -297,11 +301,10 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
         f.x = s->x;
         f.wo = w.wo;
         f.o_bias = w.o_bias;
-        f.attn_f32 = s->attn_f32;
         f.r = s->r;
         f.hidden = s->hidden;
         f.rms_eps = s->eps;
-        front_bind_flags(f, s->front_flags);
+        front_bind_workspace(f, s->front_ws);
         f.abort_flag = s->chain_abort;
         f.step_counter = s->state + 2;
         f.layer = l;
@@ -652,6 +655,11 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
   s->planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
   s->attn_splits = attn_default_splits(rq->kv_heads, block_count);
+  if (const char *v = getenv("NERVA_HIP_ATTN_SPLITS")) {  // tuning knob: split-KV factor of the stand-alone attention
+    const long want = strtol(v, nullptr, 10);
+    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits))
+      s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
+  }
 
   // ---- arena layout ------------------------------------------------------
   struct LayerOff {
@@ -711,9 +719,8 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
   const uint64_t off_chain_trace = c.take(static_cast<uint64_t>(rq->layer_count) * 32 * 8);
-  const uint64_t front_flags_bytes = front_flag_bytes(rq->heads, rq->kv_heads);
-  const uint64_t off_front_flags = c.take(front_flags_bytes);
-  const uint64_t off_attn_f32 = c.take(A * 4);
+  const uint64_t front_ws_bytes = front_workspace_bytes(rq->heads, rq->kv_heads);
+  const uint64_t off_front_ws = c.take(front_ws_bytes);
   s->arena_bytes = c.offset;
 
   if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
@@ -775,16 +782,16 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
     if (s->chain && trace != nullptr && trace[0] == '1')
       s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
   }
-  s->front_flags = reinterpret_cast<uint32_t *>(s->arena + off_front_flags);
-  s->attn_f32 = reinterpret_cast<float *>(s->arena + off_attn_f32);
+  s->front_ws = s->arena + off_front_ws;
   {
-    // Fused layer front (layer_front.cuh). Default where the shapes allow: attention + o
-    // projection as roles of one launch (mode 2, measured 1 % faster per step than one launch
-    // per piece). NERVA_HIP_FRONT=1 adds the qkv projection as a third role (measured 1 %
-    // slower: its hand-over costs more than the kernel boundary it removes), =0 keeps one
-    // launch per piece.
+    // Fused layer front (layer_front.cuh), opt-in: NERVA_HIP_FRONT=2 runs attention + o
+    // projection as roles of one launch, =1 adds the qkv projection as a third role. Off by
+    // default: measured on MI355X every hand-over between workgroups through memory costs
+    // 1.2-1.8 us (device-coherent store, poll, dependent load), about what the kernel boundary
+    // it replaces costs, and the attention role runs under a tighter register budget; the step is
+    // 3-6 % slower than with one launch per piece.
     const char *want = getenv("NERVA_HIP_FRONT");
-    int mode = 2;
+    int mode = 0;
     if (want != nullptr && want[0] >= '0' && want[0] <= '2') mode = want[0] - '0';
     if (s->chain || rq->layer_count == 0 || !front_supported(rq->hidden, rq->heads, rq->kv_heads, rq->head_dim))
       mode = 0;
@@ -795,7 +802,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
     if (splits > block_count) splits = block_count;
     s->front_splits = splits == 0 ? 1 : splits;
     const char *trace = getenv("NERVA_HIP_FRONT_TRACE");
-    if (s->front != 0 && trace != nullptr && trace[0] == '1')
+    if (!s->chain && rq->layer_count > 0 && trace != nullptr && trace[0] == '1')
       s->front_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
   }
   s->layer.resize(L);
@@ -879,7 +886,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_workspace_bytes(rq->heads, rq->head_dim), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_flags, 0, front_flags_bytes, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_ws, 0, front_ws_bytes, s->stream);
   if (err == hipSuccess && rq->layer_count > 0)
     err = hipMemsetAsync(s->arena + off_chain_trace, 0, static_cast<uint64_t>(rq->layer_count) * 32 * 8, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
@@ -1273,8 +1280,10 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
     if (kind == kLQkv && s->front == 1) continue;
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
-      // no embed launch here, so the step counter stands still: the hand-over epochs repeat
-      err = hipMemsetAsync(s->front_flags, 0, front_flag_bytes(s->heads, s->kv_heads), s->stream);
+      // no embed launch in this pass: advance the step counter here, so that the hand-over
+      // epochs of the fused front are fresh
+      hipLaunchKernelGGL(bump_step_counter_kernel, dim3(1), dim3(64), 0, s->stream, s->state);
+      err = hipGetLastError();
       if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
       if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
       if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
@@ -1311,11 +1320,12 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
         const uint64_t *t = tr.data() + 32 * l;
         uint64_t first = ~uint64_t{0};
         for (int i = 0; i < 28; ++i)
-          if (t[i] != 0 && t[i] < first) first = t[i];
+          if (t[i] > 1000000 && t[i] < first) first = t[i];
         fprintf(stderr, "[front trace] layer %u:", l);
         for (int i = 0; i < 28; ++i) {
           if (i == 8 || i == 16 || i == 20 || i == 24) fprintf(stderr, " |");
-          if (t[i] != 0) fprintf(stderr, " %lld", static_cast<long long>(t[i] - first));
+          if (t[i] > 1000000) fprintf(stderr, " %lld", static_cast<long long>(t[i] - first));
+          else if (t[i] != 0) fprintf(stderr, " #%lld", static_cast<long long>(t[i]));
           else fprintf(stderr, " -");
         }
         fprintf(stderr, "\n");

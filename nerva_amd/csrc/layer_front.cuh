@@ -7,10 +7,11 @@
 // attention output) have to wait. Roles are assigned by workgroup index in producer order -
 // qkv rows first, then attention splits, then o rows - so a workgroup only ever waits for
 // workgroups that were dispatched before it, and each role requests all of its weights / tiles
-// into registers before it waits. Hand-over between roles uses device-coherent stores and
-// loads plus epoch flags (no cache flush, no read-modify-write on the consumer side).
-// Every wait is bounded; a wait that runs out raises abort_flag and the step is reported as
-// failed by the host.
+// into registers before it waits. A value handed from one role to another travels as an
+// 8-byte (f32 value, epoch) word written and polled with device-coherent accesses: a matching
+// epoch proves the value, so there are no flags to order against, no cache flushes and no
+// read-modify-writes. Every wait is bounded; a wait that runs out raises abort_flag and the step
+// is reported as failed by the host.
 // Reference step order: launch_cublas_layer_session_step
 // (native/cuda/hf_decode_sequence/session_decode_prefill.inc.cu:74-372).
 #pragma once
@@ -21,7 +22,8 @@ namespace nv {
 
 constexpr uint32_t kFrontThreads = 512;      // 8 waves per workgroup in every role
 constexpr uint32_t kFrontRowsPerWg = 16;     // GEMV roles: two rows per wave
-constexpr uint32_t kFrontFlagStride = 16;    // u32 words between the per-kv-head flags (64 B)
+constexpr uint32_t kFrontFlagStride = 16;    // u32 words of one o workgroup's hint line (64 B): one word per kv head
+constexpr uint32_t kFrontMaxOWgs = 256;      // hidden <= 4096
 
 struct FrontParams {
   AttnParams attn;         // attention role (attn.qkv is what the qkv role writes)
@@ -30,22 +32,25 @@ struct FrontParams {
   const float *x;          // [hidden] layer input: RMSNorm source and the residual of the o projection
   const uint16_t *wo;      // [hidden][A]
   const uint16_t *o_bias;  // optional [hidden]
-  float *attn_f32;         // [A] attention output handed from the attention role to the o role
   float *r;                // [hidden] x + o projection (+ bias)
   uint32_t hidden;
   float rms_eps;
-  uint32_t *head_flags;    // [kv_heads * kFrontFlagStride] attention output of a kv head is visible
-  uint32_t *row_flags;     // [qkv workgroups] q/k/v rows of a workgroup are visible
+  // hand-over storage (front_bind_workspace): tagged words, zero before the first launch
+  uint64_t *qkv_tagged;    // [A + 2 KV] q|k|v from the qkv role to the attention role
+  uint64_t *part_tagged;   // [heads][kAttnMaxSplits][130] split partials
+  uint64_t *out_tagged;    // [A / 2] attention output (pairs of 16-bit values) from the attention role to the o role
+  uint32_t *head_hints;    // [o workgroups][kFrontFlagStride] "kv head's output is about to appear", a line per consumer
+  uint32_t *split_hints;   // [kv_heads][kAttnMaxSplits] "this split's partial has been stored"
   uint32_t *abort_flag;
   const uint32_t *step_counter;  // device word that grows by one per step; epochs derive from it
   uint32_t layer, layers;
   uint64_t *trace;         // optional [32] device timestamps of selected workgroups (tuning aid), or null
 };
 
-// Bytes of flag storage a caller provides (zeroed once; epochs only grow afterwards).
-uint64_t front_flag_bytes(uint32_t heads, uint32_t kv_heads);
-// Carves head_flags / row_flags out of a buffer of front_flag_bytes().
-void front_bind_flags(FrontParams &p, void *flags);
+// Bytes of hand-over storage a caller provides (zeroed once; epochs never repeat afterwards).
+uint64_t front_workspace_bytes(uint32_t heads, uint32_t kv_heads);
+// Carves the hand-over buffers out of a workspace of front_workspace_bytes() (needs p.attn dims).
+void front_bind_workspace(FrontParams &p, void *workspace);
 // True when the shapes fit the fused kernel (otherwise: one launch per piece).
 bool front_supported(uint32_t hidden, uint32_t heads, uint32_t kv_heads, uint32_t head_dim);
 // Number of workgroups of each role for these parameters.

@@ -36,10 +36,6 @@ struct GemvShared {
   float red[kFW];
 };
 
-__device__ __forceinline__ uint64_t load_coherent64(const void *ptr) {
-  return __hip_atomic_load(reinterpret_cast<const uint64_t *>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Requests row `row` of W[.][cols] (cols = nchunk * 512) into registers: 16 bytes per lane and chunk.
 __device__ __forceinline__ void request_row(const uint16_t *w, uint32_t row, uint32_t cols, uint32_t nchunk, int lane,
                                             uint4 (&buf)[kMaxChunks]) {
@@ -122,7 +118,6 @@ __device__ __forceinline__ void front_q_role(const FrontParams &p, uint32_t wg, 
   __syncthreads();
   link_mark(tr, 1);
 
-  float *out = const_cast<float *>(p.attn.qkv);
 #pragma unroll
   for (int r = 0; r < kQRowsPerWave; r += 2) {
     const float y0 = dot_row<DT>(w0, sh.xs, nchunk, lane);
@@ -130,14 +125,11 @@ __device__ __forceinline__ void front_q_role(const FrontParams &p, uint32_t wg, 
     const float y1 = dot_row<DT>(w1, sh.xs, nchunk, lane);
     if (r + 3 < kQRowsPerWave) request_row(p.wqkv, row0 + r + 3, cols, nchunk, lane, w1);
     if (lane == 0) {
-      store_coherent(out + row0 + r, y0);
-      store_coherent(out + row0 + r + 1, y1);
+      store_tagged(p.qkv_tagged + row0 + r, y0, epoch);
+      store_tagged(p.qkv_tagged + row0 + r + 1, y1, epoch);
     }
     if (r == 0) link_mark(tr, 2);
   }
-  wait_stores_performed();
-  __syncthreads();
-  if (threadIdx.x == 0) store_coherent(p.row_flags + wg, epoch);
   link_mark(tr, 3);
   if (p.trace != nullptr && wg + 1 == gridDim.x - p.attn.kv_heads * p.attn.splits - p.hidden / kFrontRowsPerWg)
     link_mark(p.trace, 4);
@@ -167,34 +159,38 @@ __device__ __forceinline__ void front_o_role(const FrontParams &p, uint32_t wg, 
     }
   }
 
-  // ---- wait until every kv head's attention output is visible (bounded)
+  // ---- a light wait first: one wave polls this workgroup's own hint words, one per kv head (the
+  // output itself is 16 KiB, too much for 256 workgroups to poll all along)
   if (wave == 0) {
     uint32_t spins = 0;
-    bool ok = true;
     for (;;) {
       const bool mine = static_cast<uint32_t>(lane) >= p.attn.kv_heads ||
-                        static_cast<int32_t>(load_coherent(p.head_flags + lane * kFrontFlagStride) - epoch) >= 0;
+                        load_coherent(p.head_hints + wg * kFrontFlagStride + lane) == epoch;
       if (__all(mine)) break;
-      if (++spins > kLinkSpinLimit || load_coherent(p.abort_flag) != 0u) {
-        ok = false;
-        break;
-      }
+      if (link_give_up(p.abort_flag, spins)) break;
     }
-    if (!ok && lane == 0) store_coherent(p.abort_flag, 1u);
   }
   __syncthreads();
   link_mark(tr, 1);
 
-  // ---- attention output: f32 (device-coherent source) -> 16 bit -> LDS
+  // ---- attention output: (two 16-bit values, epoch) words -> LDS; polled until every word is current
   const uint32_t c = threadIdx.x * 8;
   if (c < cols) {
-    const uint64_t v0 = load_coherent64(p.attn_f32 + c), v1 = load_coherent64(p.attn_f32 + c + 2);
-    const uint64_t v2 = load_coherent64(p.attn_f32 + c + 4), v3 = load_coherent64(p.attn_f32 + c + 6);
-    auto pack = [](uint64_t v) {
-      return static_cast<uint32_t>(enc16<DT>(__uint_as_float(static_cast<uint32_t>(v)))) |
-             (static_cast<uint32_t>(enc16<DT>(__uint_as_float(static_cast<uint32_t>(v >> 32)))) << 16);
-    };
-    *reinterpret_cast<uint4 *>(sh.xs + c) = make_uint4(pack(v0), pack(v1), pack(v2), pack(v3));
+    uint64_t v[4];
+    uint32_t spins = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = load_tagged(p.out_tagged + c / 2 + i);
+        ok = ok && tag_is(v[i], epoch);
+      }
+      if (__all(ok)) break;
+      if (link_give_up(p.abort_flag, spins)) break;
+      __builtin_amdgcn_s_sleep(8);
+    }
+    *reinterpret_cast<uint4 *>(sh.xs + c) = make_uint4(static_cast<uint32_t>(v[0]), static_cast<uint32_t>(v[1]),
+                                                       static_cast<uint32_t>(v[2]), static_cast<uint32_t>(v[3]));
   }
   __syncthreads();
   link_mark(tr, 2);
@@ -222,12 +218,14 @@ __global__ __launch_bounds__(kFrontThreads, 4) void layer_front_kernel(FrontPara
   } else if (b < q_wgs + a_wgs) {
     const uint32_t a = b - q_wgs;
     const uint32_t kvh = a % p.attn.kv_heads, split = a / p.attn.kv_heads;
-    constexpr uint32_t kWgsPerKvHead = (G + 2) * (kHD / kFrontQRowsPerWg);
     AttnLink link;
-    link.wait_flags = q_wgs != 0 ? p.row_flags + kvh * kWgsPerKvHead : nullptr;
-    link.wait_count = kWgsPerKvHead;
-    link.done_flag = p.head_flags + kvh * kFrontFlagStride;
-    link.out_coherent = p.attn_f32;
+    link.qkv_tagged = q_wgs != 0 ? p.qkv_tagged : nullptr;
+    link.part_tagged = p.part_tagged;
+    link.out_tagged = p.out_tagged;
+    link.hints = p.head_hints;
+    link.hint_count = p.hidden / kFrontRowsPerWg;
+    link.hint_stride = kFrontFlagStride;
+    link.split_hints = p.split_hints;
     link.abort_flag = p.abort_flag;
     link.epoch = epoch;
     link.trace = p.trace != nullptr && kvh == 0 && split == 0 ? p.trace : nullptr;
@@ -244,7 +242,7 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 bool front_supported(uint32_t hidden, uint32_t heads, uint32_t kv_heads, uint32_t head_dim) {
   if (head_dim != static_cast<uint32_t>(kHD) || kv_heads == 0 || heads != 4 * kv_heads) return false;
-  if (kv_heads > static_cast<uint32_t>(kWave)) return false;                 // one polling lane per kv head
+  if (kv_heads > kFrontFlagStride) return false;                             // one hint word per kv head in a 64-byte line
   if (hidden % kChunkCols != 0 || hidden > kMaxChunks * kChunkCols) return false;  // rows live in registers
   const uint32_t attn_dim = heads * head_dim;
   if (attn_dim > kMaxChunks * kChunkCols) return false;
@@ -258,24 +256,39 @@ void front_grid(const FrontParams &p, uint32_t *q_wgs, uint32_t *a_wgs, uint32_t
   *o_wgs = p.hidden / kFrontRowsPerWg;
 }
 
-uint64_t front_flag_bytes(uint32_t heads, uint32_t kv_heads) {
-  const uint64_t head_words = static_cast<uint64_t>(kv_heads) * kFrontFlagStride;
-  const uint64_t row_words = static_cast<uint64_t>(heads + 2 * kv_heads) * kHD / kFrontQRowsPerWg;
-  return ((head_words + row_words) * sizeof(uint32_t) + 255u) & ~static_cast<uint64_t>(255u);
+namespace {
+uint64_t round256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
+}  // namespace
+
+uint64_t front_workspace_bytes(uint32_t heads, uint32_t kv_heads) {
+  const uint64_t qkv = round256(static_cast<uint64_t>(heads + 2 * kv_heads) * kHD * 8);
+  const uint64_t part = round256(static_cast<uint64_t>(heads) * kAttnMaxSplits * kPartRecord * 8);
+  const uint64_t out = round256(static_cast<uint64_t>(heads) * kHD * 8);
+  const uint64_t hints = round256(static_cast<uint64_t>(kFrontMaxOWgs) * kFrontFlagStride * 4);
+  const uint64_t split_hints = round256(static_cast<uint64_t>(kv_heads) * kAttnMaxSplits * 4);
+  return qkv + part + out + hints + split_hints;
 }
 
-void front_bind_flags(FrontParams &p, void *flags) {
-  p.head_flags = static_cast<uint32_t *>(flags);
-  p.row_flags = p.head_flags + static_cast<uint64_t>(p.attn.kv_heads) * kFrontFlagStride;
+void front_bind_workspace(FrontParams &p, void *workspace) {
+  char *base = static_cast<char *>(workspace);
+  const uint32_t heads = p.attn.heads, kv_heads = p.attn.kv_heads;
+  p.qkv_tagged = reinterpret_cast<uint64_t *>(base);
+  base += round256(static_cast<uint64_t>(heads + 2 * kv_heads) * kHD * 8);
+  p.part_tagged = reinterpret_cast<uint64_t *>(base);
+  base += round256(static_cast<uint64_t>(heads) * kAttnMaxSplits * kPartRecord * 8);
+  p.out_tagged = reinterpret_cast<uint64_t *>(base);
+  base += round256(static_cast<uint64_t>(heads) * kHD * 8);
+  p.head_hints = reinterpret_cast<uint32_t *>(base);
+  base += round256(static_cast<uint64_t>(kFrontMaxOWgs) * kFrontFlagStride * 4);
+  p.split_hints = reinterpret_cast<uint32_t *>(base);
 }
 
 hipError_t launch_layer_front(uint32_t dtype, const FrontParams &p, hipStream_t stream) {
   const AttnParams &a = p.attn;
-  if (a.qkv == nullptr || a.k_cache == nullptr || a.v_cache == nullptr || a.table == nullptr || a.out16 == nullptr ||
-      a.part_acc == nullptr || a.counters == nullptr)
+  if (a.qkv == nullptr || a.k_cache == nullptr || a.v_cache == nullptr || a.table == nullptr || a.out16 == nullptr)
     return hipErrorInvalidValue;
-  if (p.x == nullptr || p.wo == nullptr || p.attn_f32 == nullptr || p.r == nullptr || p.head_flags == nullptr ||
-      p.row_flags == nullptr || p.abort_flag == nullptr || p.step_counter == nullptr)
+  if (p.x == nullptr || p.wo == nullptr || p.r == nullptr || p.qkv_tagged == nullptr || p.part_tagged == nullptr ||
+      p.out_tagged == nullptr || p.head_hints == nullptr || p.abort_flag == nullptr || p.step_counter == nullptr)
     return hipErrorInvalidValue;
   if (p.wqkv != nullptr && p.rms_attn == nullptr) return hipErrorInvalidValue;
   if (!front_supported(p.hidden, a.heads, a.kv_heads, a.head_dim)) return hipErrorInvalidValue;
@@ -285,7 +298,7 @@ hipError_t launch_layer_front(uint32_t dtype, const FrontParams &p, hipStream_t 
   if (a.cursor == nullptr &&
       static_cast<uint64_t>(a.position) >= static_cast<uint64_t>(a.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
-  if (!aligned16(p.x) || !aligned16(p.wo) || !aligned16(p.attn_f32) || !aligned16(a.qkv) ||
+  if (!aligned16(p.x) || !aligned16(p.wo) || !aligned16(p.out_tagged) || !aligned16(p.qkv_tagged) ||
       (p.wqkv != nullptr && (!aligned16(p.wqkv) || !aligned16(p.rms_attn))))
     return hipErrorInvalidValue;
   uint32_t q_wgs, a_wgs, o_wgs;

@@ -181,9 +181,9 @@ GEOMETRIES = [
 
 STEP_MODES = {
     # id: (NERVA_HIP_FRONT, NERVA_HIP_CHAIN, fused_state mode of a session whose shapes fit)
-    "launch-per-piece": ("0", None, N.DecodeSession.FUSED_NONE),
+    "launch-per-piece": (None, None, N.DecodeSession.FUSED_NONE),         # the default
     "fused-front": ("1", None, N.DecodeSession.FUSED_FRONT),
-    "fused-attn-o": (None, None, N.DecodeSession.FUSED_FRONT_ATTN_O),   # the default
+    "fused-attn-o": ("2", None, N.DecodeSession.FUSED_FRONT_ATTN_O),
     "chain-kernel": (None, "1", N.DecodeSession.FUSED_CHAIN),
 }
 
@@ -319,8 +319,7 @@ def test_eager_profile_pass_leaves_state_untouched():
     s.start(prompt)
     rc, res, a = s.advance(4)
     rc, prof = s.profile_step(2)
-    assert rc == 0 and prof.status == 0 and prof.front_mode == 2 and prof.launches == 3 + 4 * 2
-    assert prof.front_ns > 0 and prof.front_stream_ns > 0 and prof.front_bytes > 0 and prof.attention_ns == 0
+    assert rc == 0 and prof.status == 0 and prof.front_mode == 0 and prof.launches == 3 + 5 * 2
     assert prof.gate_up_ns > 0 and prof.lm_head_ns > 0 and prof.position == len(prompt) + 3
     rc, res, b = s.advance(6)
     s.start(prompt)
@@ -388,7 +387,6 @@ def test_chain_kernel_is_used_and_agrees_with_one_launch_per_gemv(monkeypatch):
     assert rc == 0
     s.destroy()
     monkeypatch.delenv("NERVA_HIP_CHAIN")
-    monkeypatch.setenv("NERVA_HIP_FRONT", "0")
     s = N.DecodeSession.create(weights, 64)
     assert s.fused_state() == (s.FUSED_NONE, False)
     s.start(prompt)
