@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one gate_up launch moves at the Qwen3-8B shape (24576x4096 bf16): FETCH_SIZE + WRITE_SIZE
 # per dispatch from two `rocprofv3 --pmc` runs, each scaled by what the counter reads for a plain
 # 256 MiB copy kernel (profiles/gate_up_gemv_hbm_traffic_pmc.txt). Not measurable in-process.
-GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201709220}
+GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201709978}
 # Same for one launch of the persistent layer-chain kernel (filled in from its counter profile).
 CHAIN_TRAFFIC_BYTES = {}
 SEED = 0x4E45525641
@@ -106,7 +106,24 @@ def cpu_baseline(session, cfg, position, token, layers_sampled, threads_all):
         result[threads] = dict(tok_s=1.0 / per_token, layers_s=t_layers, head_s=t_head)
         log("[cpu] %d thread(s): %d layers %.2f s, lm_head %.2f s -> %.4f tok/s (extrapolated)"
             % (threads, layers_sampled, t_layers, t_head, 1.0 / per_token))
+        if threads == 1:
+            oracle_rows = [ctx.read_kv16(l, position) for l in range(layers_sampled)]
         ctx.close()
+    # Full-size parity, checker only: the device now runs the same token at the same position, and the
+    # K/V rows it appends for the sampled layers are compared with the oracle's. Layer 0's row covers
+    # embedding, RMSNorm, the 6144x4096 qkv GEMV, QK-norm and RoPE; layer 1's row depends on layer 0's
+    # attention over the whole context, its o projection and its MLP, all at the workload's real sizes.
+    rc, _, _ = session.advance(1)
+    assert rc == 0
+    rel = lambda a, b: float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+    parity = {}
+    for l, (rk, rv) in enumerate(oracle_rows):
+        gk, gv = session.kv_row(l, position)
+        parity["layer%d_k" % l] = rel(O.decode16(dt, gk), O.decode16(dt, rk))
+        parity["layer%d_v" % l] = rel(O.decode16(dt, gv), O.decode16(dt, rv))
+    log("[cpu] device vs oracle K/V rows of the next token at position %d (relative L2): %s"
+        % (position, ", ".join("%s %.2e" % kv_ for kv_ in sorted(parity.items()))))
+    result["parity"] = parity
     return result
 
 
@@ -134,7 +151,7 @@ def main():
         sys.exit(1)
     cfg = dict(N.Qwen3_8B)
     cfg["layers"] = args.layers
-    max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16
+    max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16   # + the CPU leg's parity token
     t0 = time.time()
     session = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=WEIGHT_STD, qk_norm=True)
     log("[bench] %s: session created in %.1f s, arena %.2f GB (weights %.2f GB, KV %.2f GB)" % (
@@ -230,7 +247,9 @@ def main():
             cpu = dict(value=round(r[1]["tok_s"], 5), unit="tok/s", cores=1, kind="port",
                        sample="1 decode token at ctx %d: %d of %d layers + lm_head timed on the oracle, extrapolated to %d layers"
                               % (position, layers_sampled, cfg["layers"], cfg["layers"]),
-                       all_cores_value=round(r[threads_all]["tok_s"], 5), all_cores=threads_all)
+                       all_cores_value=round(r[threads_all]["tok_s"], 5), all_cores=threads_all,
+                       parity_rel_l2={k: float("%.3g" % v) for k, v in r["parity"].items()},
+                       parity_ok=all(v <= (2e-3 if k.startswith("layer0") else 2e-2) for k, v in r["parity"].items()))
         except Exception as e:  # the CPU leg never hides the GPU result
             log("[cpu] baseline failed: %r" % (e,))
     session.destroy()

@@ -28,9 +28,10 @@ using namespace attn;
 template <uint32_t DT, int G, int W>
 __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   __shared__ AttnShared<G, W> sh;
+  const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);  // before anything they could queue behind
   const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
   if (p.cursor != nullptr && pos >= p.max_steps) return;
-  attn_fast_body<DT, G, W, false>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{});
+  attn_fast_body<DT, G, W, false>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
 }
 
 // Any head_dim (even when RoPE is on) / any group size: one workgroup per query

@@ -18,30 +18,23 @@ constexpr int kAttnWaves = 8;   // waves per workgroup of the fast path (group 8
 // copy is stored too (K/V that go to the cache).
 // rope_cs (optional): cos at [i], sin at [64 + i] of this step's angles, computed once
 // per step; without it the angle pos / rope_freq[i] is evaluated here.
-// (x0, x1) = raw projection values of dims (lane, lane + 64).
+// (x0, x1) = raw projection values of dims (lane, lane + 64); bias / gamma / rotation of the
+// same two dims, already in registers.
 template <uint32_t DT>
-__device__ __forceinline__ void prep_head128(float x0, float x1, const uint16_t *bias,
-                                             const uint16_t *gamma, const float *rope_freq,
-                                             const float *rope_cs, uint32_t pos, float eps, int lane,
-                                             float *out, uint16_t *out16) {
-  if (bias != nullptr) {
-    x0 += dec16<DT>(bias[lane]);
-    x1 += dec16<DT>(bias[lane + 64]);
+__device__ __forceinline__ void prep_head128_core(float x0, float x1, bool has_bias, float b0, float b1,
+                                                  bool has_gamma, float g0, float g1, bool has_rope, float c,
+                                                  float s, float eps, int lane, float *out, uint16_t *out16) {
+  if (has_bias) {
+    x0 += b0;
+    x1 += b1;
   }
-  if (gamma != nullptr) {
+  if (has_gamma) {
     const float ss = wave_sum(x0 * x0 + x1 * x1);
     const float scale = 1.0f / sqrtf(ss / 128.0f + eps);
-    x0 *= scale * dec16<DT>(gamma[lane]);
-    x1 *= scale * dec16<DT>(gamma[lane + 64]);
+    x0 *= scale * g0;
+    x1 *= scale * g1;
   }
-  if (rope_freq != nullptr) {
-    float s, c;
-    if (rope_cs != nullptr) {
-      c = rope_cs[lane];
-      s = rope_cs[64 + lane];
-    } else {
-      sincosf(static_cast<float>(pos) / rope_freq[lane], &s, &c);
-    }
+  if (has_rope) {
     const float r0 = x0 * c - x1 * s;
     const float r1 = x1 * c + x0 * s;
     x0 = r0;
@@ -57,6 +50,32 @@ __device__ __forceinline__ void prep_head128(float x0, float x1, const uint16_t 
     out[lane] = x0;
     out[lane + 64] = x1;
   }
+}
+// Same with bias / gamma / rotation fetched here.
+template <uint32_t DT>
+__device__ __forceinline__ void prep_head128(float x0, float x1, const uint16_t *bias,
+                                             const uint16_t *gamma, const float *rope_freq,
+                                             const float *rope_cs, uint32_t pos, float eps, int lane,
+                                             float *out, uint16_t *out16) {
+  float b0 = 0.0f, b1 = 0.0f, g0 = 0.0f, g1 = 0.0f, c = 1.0f, s = 0.0f;
+  if (bias != nullptr) {
+    b0 = dec16<DT>(bias[lane]);
+    b1 = dec16<DT>(bias[lane + 64]);
+  }
+  if (gamma != nullptr) {
+    g0 = dec16<DT>(gamma[lane]);
+    g1 = dec16<DT>(gamma[lane + 64]);
+  }
+  if (rope_freq != nullptr) {
+    if (rope_cs != nullptr) {
+      c = rope_cs[lane];
+      s = rope_cs[64 + lane];
+    } else {
+      sincosf(static_cast<float>(pos) / rope_freq[lane], &s, &c);
+    }
+  }
+  prep_head128_core<DT>(x0, x1, bias != nullptr, b0, b1, gamma != nullptr, g0, g1, rope_freq != nullptr, c, s, eps,
+                        lane, out, out16);
 }
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -134,10 +153,10 @@ __device__ __forceinline__ uint32_t load_coherent(const uint32_t *ptr) {
 // Returns when every store this wave has issued has been performed.
 __device__ __forceinline__ void wait_stores_performed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-// Requests one (block, kv head) tile: four 1 KiB loads each for K and V.
-__device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t b, uint32_t kvh, int lane,
+// Requests one (physical block, kv head) tile: four 1 KiB loads each for K and V.
+__device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t physical_block, uint32_t kvh, int lane,
                                                uint4 (&k)[4], uint4 (&v)[4]) {
-  const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[b], kvh);
+  const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, physical_block, kvh);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     k[i] = load_stream(p.k_cache + tile + i * 512 + lane * 8);
@@ -331,6 +350,66 @@ __device__ __forceinline__ void load_head128(const float *qkv, const AttnLink &l
   x1 = qkv[off + lane + 64];
 }
 
+// Everything a wave needs to prepare its heads - raw projections of its query heads
+// (g = wave, wave + W, ...) and, on two designated waves, of the new key / value row, with the
+// bias, norm weight and rotation of the same dims - requested by the stand-alone kernel before
+// anything else and awaited before the first KV tile is requested: loads return in order, so a
+// value requested after the tiles could only be used once all of their data had arrived.
+struct HeadInputs {
+  float x0, x1;
+  uint16_t b0, b1;  // bias bits (valid when the bias pointer is set)
+};
+template <int G, int W>
+struct RawHeads {
+  HeadInputs q[(G + W - 1) / W];
+  HeadInputs e;                  // new key row (wave G % W) or new value row (wave (G + 1) % W)
+  uint16_t qg0, qg1, kg0, kg1;   // q_norm / k_norm weight bits
+  float rope_a, rope_b;          // cos, sin of this step; without a table: the frequency of the pair
+};
+template <int G, int W>
+__device__ __forceinline__ RawHeads<G, W> attn_request_raw(const AttnParams &p, uint32_t kvh) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
+  RawHeads<G, W> r{};
+#pragma unroll
+  for (int i = 0; i < (G + W - 1) / W; ++i) {
+    const uint32_t off = (kvh * G + min(wave + i * W, G - 1)) * kHD;  // clamped: the loads are unconditional
+    r.q[i].x0 = p.qkv[off + lane];
+    r.q[i].x1 = p.qkv[off + lane + 64];
+    if (p.q_bias != nullptr) {
+      r.q[i].b0 = p.q_bias[off + lane];
+      r.q[i].b1 = p.q_bias[off + lane + 64];
+    }
+  }
+  const bool value_wave = wave == ((G + 1) % W);
+  const uint32_t off = (value_wave ? A + KV : A) + kvh * kHD;
+  r.e.x0 = p.qkv[off + lane];
+  r.e.x1 = p.qkv[off + lane + 64];
+  const uint16_t *eb = value_wave ? p.v_bias : p.k_bias;
+  if (eb != nullptr) {
+    r.e.b0 = eb[kvh * kHD + lane];
+    r.e.b1 = eb[kvh * kHD + lane + 64];
+  }
+  if (p.q_norm != nullptr) {
+    r.qg0 = p.q_norm[lane];
+    r.qg1 = p.q_norm[lane + 64];
+  }
+  if (p.k_norm != nullptr) {
+    r.kg0 = p.k_norm[lane];
+    r.kg1 = p.k_norm[lane + 64];
+  }
+  if (p.rope_freq != nullptr) {
+    if (p.rope_cs != nullptr) {
+      r.rope_a = p.rope_cs[lane];
+      r.rope_b = p.rope_cs[64 + lane];
+    } else {
+      r.rope_a = p.rope_freq[lane];
+    }
+  }
+  return r;
+}
+
 // W waves per workgroup. A workgroup owns one kv head and one contiguous range of
 // 16-token tiles; wave w takes tiles b0+w, b0+w+W, ...  Both products of a tile run on
 // the matrix cores:
@@ -351,7 +430,7 @@ __device__ __forceinline__ void load_head128(const float *qkv, const AttnLink &l
 template <uint32_t DT, int G, int W, bool LINKED>
 __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32_t pos, const uint32_t kvh,
                                                const uint32_t split, const uint32_t S, AttnShared<G, W> &sh,
-                                               const AttnLink &link) {
+                                               const AttnLink &link, const RawHeads<G, W> &raw) {
   constexpr int kThreads = W * kWave;
   auto &q_s = sh.q_s;
   auto &knew = sh.knew;
@@ -363,7 +442,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   auto &bM = sh.bM;
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform: block-table reads stay scalar
   // tuning aid: stage timestamps of workgroup (kv head 0, split 0) and of kv head 0's merging workgroup
   uint64_t *const tr = LINKED ? link.trace : (kvh == 0 && split == 0 ? p.trace : nullptr);
   uint64_t *const trm = LINKED ? link.trace_merge : (kvh == 0 ? p.trace : nullptr);
@@ -381,33 +460,72 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
 
   // ---- first tile of every wave: issue its loads before anything else
-  // Two tiles in flight per wave (roles swap); a linked workgroup keeps one, to fit the register
-  // budget that lets two 8-wave workgroups share a CU, and its launch uses more splits instead.
-  constexpr int kInFlight = LINKED ? 1 : 2;
-  uint4 kreg[4], vreg[4], kreg1[kInFlight == 2 ? 4 : 1], vreg1[kInFlight == 2 ? 4 : 1];
+  // Up to four tiles in flight per wave (one 8-wave workgroup per CU leaves 256 registers a lane;
+  // at the default split factor a wave's whole share of an 8k context is requested at once). A
+  // linked workgroup keeps one, to fit the register budget that lets two 8-wave workgroups share
+  // a CU, and its launch uses more splits instead.
+  constexpr int kInFlight = LINKED ? 1 : 4;
+  uint4 kreg[kInFlight][4], vreg[kInFlight][4];
   uint32_t b = b0 + wave;
-  if (b < b1) attn_load_tile(p, b, kvh, lane, kreg, vreg);
+  // the block-table entries first, all of them, so that no tile request waits behind another tile's data
+  uint32_t phys[kInFlight];
+#pragma unroll
+  for (int f = 0; f < kInFlight; ++f) phys[f] = p.table[min(b + f * W, nblk - 1)];
+  // the head inputs requested at kernel start have to be in registers before the tiles go out
+  if constexpr (!LINKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int f = 0; f < kInFlight; ++f)
+    if (b + f * W < b1) attn_load_tile(p, phys[f], kvh, lane, kreg[f], vreg[f]);
 
   link_mark(tr, 8);
   // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
-  for (int g = wave; g < G; g += W) {
-    const uint32_t h = kvh * G + g;
-    float x0, x1;
-    load_head128<LINKED>(p.qkv, link, h * kHD, lane, x0, x1);
-    prep_head128<DT>(x0, x1, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq, p.rope_cs, pos, p.eps,
-                     lane, q_s[g], nullptr);
-  }
-  if (owns_new) {
-    if (wave == (G % W)) {
-      float x0, x1;
-      load_head128<LINKED>(p.qkv, link, A + kvh * kHD, lane, x0, x1);
-      prep_head128<DT>(x0, x1, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm, p.rope_freq, p.rope_cs, pos,
-                       p.eps, lane, nullptr, knew);
-    } else if (wave == ((G + 1) % W)) {
-      float x0, x1;
-      load_head128<LINKED>(p.qkv, link, A + KV + kvh * kHD, lane, x0, x1);
-      prep_head128<DT>(x0, x1, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr, nullptr, nullptr, pos, p.eps,
-                       lane, nullptr, vnew);
+  if constexpr (LINKED) {
+#pragma unroll
+    for (int i = 0; i < (G + W - 1) / W; ++i) {
+      const int g = wave + i * W;
+      if (g < G) {
+        const uint32_t h = kvh * G + g;
+        float x0, x1;
+        load_head128<LINKED>(p.qkv, link, h * kHD, lane, x0, x1);
+        prep_head128<DT>(x0, x1, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq, p.rope_cs, pos,
+                         p.eps, lane, q_s[g], nullptr);
+      }
+    }
+    if (owns_new) {
+      if (wave == (G % W)) {
+        float x0, x1;
+        load_head128<LINKED>(p.qkv, link, A + kvh * kHD, lane, x0, x1);
+        prep_head128<DT>(x0, x1, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm, p.rope_freq, p.rope_cs, pos,
+                         p.eps, lane, nullptr, knew);
+      } else if (wave == ((G + 1) % W)) {
+        float x0, x1;
+        load_head128<LINKED>(p.qkv, link, A + KV + kvh * kHD, lane, x0, x1);
+        prep_head128<DT>(x0, x1, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr, nullptr, nullptr, pos, p.eps,
+                         lane, nullptr, vnew);
+      }
+    }
+  } else {
+    // every input is in registers already: pure arithmetic while the tiles are in flight
+    const bool has_rope = p.rope_freq != nullptr;
+    float rc = raw.rope_a, rs = raw.rope_b;
+    if (has_rope && p.rope_cs == nullptr) sincosf(static_cast<float>(pos) / raw.rope_a, &rs, &rc);
+#pragma unroll
+    for (int i = 0; i < (G + W - 1) / W; ++i) {
+      const int g = wave + i * W;
+      if (g < G)
+        prep_head128_core<DT>(raw.q[i].x0, raw.q[i].x1, p.q_bias != nullptr, dec16<DT>(raw.q[i].b0),
+                              dec16<DT>(raw.q[i].b1), p.q_norm != nullptr, dec16<DT>(raw.qg0), dec16<DT>(raw.qg1),
+                              has_rope, rc, rs, p.eps, lane, q_s[g], nullptr);
+    }
+    if (owns_new) {
+      if (wave == (G % W)) {
+        prep_head128_core<DT>(raw.e.x0, raw.e.x1, p.k_bias != nullptr, dec16<DT>(raw.e.b0), dec16<DT>(raw.e.b1),
+                              p.k_norm != nullptr, dec16<DT>(raw.kg0), dec16<DT>(raw.kg1), has_rope, rc, rs, p.eps,
+                              lane, nullptr, knew);
+      } else if (wave == ((G + 1) % W)) {
+        prep_head128_core<DT>(raw.e.x0, raw.e.x1, p.v_bias != nullptr, dec16<DT>(raw.e.b0), dec16<DT>(raw.e.b1), false,
+                              0.0f, 0.0f, false, 1.0f, 0.0f, p.eps, lane, nullptr, vnew);
+      }
     }
   }
   __syncthreads();
@@ -461,20 +579,15 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
 #pragma unroll
   for (int s2 = 0; s2 < 8; ++s2) acc[s2] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-  if constexpr (kInFlight == 2) {
-    if (b + W < b1) attn_load_tile(p, b + W, kvh, lane, kreg1, vreg1);
-    for (; b < b1; b += 2 * W) {
-      attn_tile<DT, G, LINKED>(kreg, vreg, qx, qx_lds, b, n_keys, col, grp, owns_new && b == new_block, new_row, knew, vnew, m, l, acc);
-      if (b + 2 * W < b1) attn_load_tile(p, b + 2 * W, kvh, lane, kreg, vreg);
-      if (b + W < b1) {
-        attn_tile<DT, G, LINKED>(kreg1, vreg1, qx, qx_lds, b + W, n_keys, col, grp, owns_new && b + W == new_block, new_row, knew, vnew, m, l, acc);
-        if (b + 3 * W < b1) attn_load_tile(p, b + 3 * W, kvh, lane, kreg1, vreg1);
+  for (; b < b1; b += kInFlight * W) {
+#pragma unroll
+    for (int f = 0; f < kInFlight; ++f) {
+      const uint32_t bb = b + f * W;
+      if (bb < b1) {
+        attn_tile<DT, G, LINKED>(kreg[f], vreg[f], qx, qx_lds, bb, n_keys, col, grp, owns_new && bb == new_block, new_row,
+                                 knew, vnew, m, l, acc);
+        if (bb + kInFlight * W < b1) attn_load_tile(p, p.table[bb + kInFlight * W], kvh, lane, kreg[f], vreg[f]);
       }
-    }
-  } else {
-    for (; b < b1; b += W) {
-      attn_tile<DT, G, LINKED>(kreg, vreg, qx, qx_lds, b, n_keys, col, grp, owns_new && b == new_block, new_row, knew, vnew, m, l, acc);
-      if (b + W < b1) attn_load_tile(p, b + W, kvh, lane, kreg, vreg);
     }
   }
 

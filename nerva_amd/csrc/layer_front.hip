@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kFrontThreads, 4) void layer_front_kernel(FrontPara
     link.epoch = epoch;
     link.trace = p.trace != nullptr && kvh == 0 && split == 0 ? p.trace : nullptr;
     link.trace_merge = p.trace != nullptr && kvh == 0 ? p.trace : nullptr;
-    attn_fast_body<DT, G, kFW, true>(p.attn, pos, kvh, split, p.attn.splits, sh.attn, link);
+    attn_fast_body<DT, G, kFW, true>(p.attn, pos, kvh, split, p.attn.splits, sh.attn, link, RawHeads<G, kFW>{});
   } else {
     front_o_role<DT>(p, b - q_wgs - a_wgs, epoch, sh.gemv);
   }
