@@ -456,6 +456,24 @@ typedef struct NervaHipArgmaxRequest {
 int nerva_hip_argmax(const NervaHipArgmaxRequest *request, void *stream, int32_t *hip_error);
 uint64_t nerva_hip_argmax_workspace_bytes(void);
 
+typedef struct NervaHipSampleRequest {
+  uint32_t vocab;
+  uint32_t position;            /* sequence position of the sampled token: the random-number counter */
+  const float *logits;          /* device [vocab] */
+  NervaHipHfDecodeSamplerConfig sampler;
+  uint32_t *token;              /* device u32 */
+  void *workspace;              /* device, nerva_hip_sample_workspace_bytes(vocab) bytes */
+} NervaHipSampleRequest;
+
+/* One token from logits by the session's sampler (sampler.cu:66-392): greedy when
+ * !(temperature > 0) or top_k == 1; Gumbel-max over the whole vocabulary when top_k == 0 and
+ * top_p >= 0.999999; otherwise the k = (top_k == 0 ? 128 : min(top_k, 128)) best finite logits by
+ * (value desc, index asc), softmax with temperature in that order, nucleus top_p, one draw. Random
+ * numbers are a hash of (seed, position, index, salt), so equal inputs give equal tokens. The
+ * configuration is normalised like the reference's ABI does (sampler.cu:422-433), never refused. */
+int nerva_hip_sample(const NervaHipSampleRequest *request, void *stream, int32_t *hip_error);
+uint64_t nerva_hip_sample_workspace_bytes(uint32_t vocab);
+
 typedef struct NervaHipMoeFp8Request {
   uint32_t hidden, intermediate, num_experts, top_k, block, input_dtype;
   int32_t shared_index;         /* expert index of the always-on shared expert, or -1 */

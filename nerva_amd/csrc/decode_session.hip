@@ -27,6 +27,7 @@
 #include "attn_decode.cuh"
 #include "decode_chain.cuh"
 #include "layer_front.cuh"
+#include "sampler.cuh"
 #include "gemv_stream.cuh"
 #include "runtime_state.hpp"
 #include "synth_fill.cuh"
@@ -107,9 +108,15 @@ struct NervaHipHfDecodeSequenceSession {
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
   uint32_t *host_state = nullptr;
-  hipGraph_t graph[2] = {nullptr, nullptr};
-  hipGraphExec_t exec[2] = {nullptr, nullptr};
-  uint64_t graph_nodes[2] = {0, 0};
+  // captured steps: 0 decode step with the greedy finish, 1 prompt step, 2 decode step with the
+  // temperature / top-k / top-p sampler (its parameters live in device memory, so one capture
+  // serves every such configuration)
+  hipGraph_t graph[3] = {nullptr, nullptr, nullptr};
+  hipGraphExec_t exec[3] = {nullptr, nullptr, nullptr};
+  uint64_t graph_nodes[3] = {0, 0, 0};
+  SamplerDev sampler{};            // normalised configuration of the active sequence
+  SamplerDev *sampler_dev = nullptr;
+  uint64_t *sampler_keys = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   // echo of the caller's weight plan
   uint32_t planned_weight_blocks = 0, planned_gpu_resident_blocks = 0, planned_gpu_staged_blocks = 0,
@@ -204,7 +211,7 @@ bool layer_has_weights(const NervaHipHfDecodeChainLayer &l) {
 void destroy_session(Session *s) {
   if (s == nullptr) return;
   if (s->stream) (void)hipStreamSynchronize(s->stream);
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 3; ++i) {
     if (s->exec[i]) (void)hipGraphExecDestroy(s->exec[i]);
     if (s->graph[i]) (void)hipGraphDestroy(s->graph[i]);
   }
@@ -410,9 +417,22 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   p.sample.slots = s->slots;
   p.sample.cursor_rw = s->state;
   NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st));
-  // one small workgroup reduces the per-workgroup candidates, writes slot[pos], bumps the cursor
-  NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows, p.cols), s->state,
-                                          s->max_ctx, st));
+  if (s->sampler.mode == kSamplerGreedy) {
+    // one small workgroup reduces the per-workgroup candidates, writes slot[pos], bumps the cursor
+    NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows, p.cols), s->state,
+                                            s->max_ctx, st));
+  } else {
+    // temperature sampling from the logits (two launches), then slot[pos] and the cursor as above
+    SamplerParams sp{};
+    sp.logits = s->logits;
+    sp.vocab = s->vocab;
+    sp.config = s->sampler_dev;
+    sp.keys = s->sampler_keys;
+    sp.out = p.sample;
+    sp.cursor = s->state;
+    sp.max_steps = s->max_ctx;
+    NV_STEP(kLAdvance, launch_sampler(sp, st));
+  }
 #undef NV_STEP
   return hipSuccess;
 }
@@ -431,7 +451,8 @@ bool eager_steps() {
 
 // Kernel launches of one step (which = 0: decode step, 1: prompt step).
 uint64_t step_launches(const Session *s, int which) {
-  const uint64_t fixed = which == 0 ? 3 : 2;  // embed + (lm head + sampler | cursor advance)
+  // embed + (lm head + greedy finish | lm head + two sampler launches | cursor advance)
+  const uint64_t fixed = which == 1 ? 2 : (s->sampler.mode == kSamplerGreedy ? 3 : 4);
   if (s->chain) return fixed + 1 + 2ull * s->layers;
   if (s->front == 1) return fixed + 3ull * s->layers;
   if (s->front == 2) return fixed + 4ull * s->layers;
@@ -441,7 +462,10 @@ uint64_t step_launches(const Session *s, int which) {
 // Launch one step: graph replay, or the same kernels eagerly (tracing mode).
 hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out);
 
-// graph index 0: decode step, 1: prompt step
+// Index of the captured decode step for the active sampler.
+int decode_graph(const Session *s) { return s->sampler.mode == kSamplerGreedy ? 0 : 2; }
+
+// graph index 0 / 2: decode step (greedy finish / sampler), 1: prompt step
 hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
   if (eager_steps()) return hipSuccess;
   if (s->exec[which] != nullptr) {
@@ -454,7 +478,7 @@ hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *o
   hipGraph_t graph = nullptr;
   hipError_t err = hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal);
   if (err != hipSuccess) return err;
-  hipError_t step_err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
+  hipError_t step_err = enqueue_step(s, which == 1 ? kPromptStep : kDecodeStep, nullptr);
   err = hipStreamEndCapture(s->stream, &graph);
   if (step_err != hipSuccess) err = step_err;
   size_t nodes = 0;
@@ -477,7 +501,7 @@ hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *o
 
 hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
   if (eager_steps()) {
-    hipError_t err = enqueue_step(s, which == 0 ? kDecodeStep : kPromptStep, nullptr);
+    hipError_t err = enqueue_step(s, which == 1 ? kPromptStep : kDecodeStep, nullptr);
     if (err == hipSuccess)
       out->kernel_launches += step_launches(s, which);
     return err;
@@ -517,12 +541,12 @@ void fill_header(const Session *s, NervaHipHfDecodeSequenceResult *out, uint32_t
   out->planned_weight_descriptor_hash = s->planned_weight_descriptor_hash;
 }
 
-bool sampler_valid(const NervaHipHfDecodeSamplerConfig &c) {
-  return isfinite(c.temperature) && c.temperature >= 0.0f && isfinite(c.top_p) && c.top_p > 0.0f &&
-         c.top_p <= 1.0f;
-}
-bool sampler_greedy(const NervaHipHfDecodeSamplerConfig &c) {
-  return !(c.temperature > 0.0f) || c.top_k == 1;  // sampler.cu:89
+// The sampler of the sequence that is about to start: normalised the way the reference's ABI does
+// (sampler.cu:422-433; its callers validate before the call, the ABI itself never refuses a
+// configuration) and copied to the device words the sampler kernels read. Not on the per-token path.
+hipError_t set_sampler(Session *s, const NervaHipHfDecodeSamplerConfig &config) {
+  s->sampler = sampler_device_config(config);
+  return hipMemcpy(s->sampler_dev, &s->sampler, sizeof(SamplerDev), hipMemcpyHostToDevice);
 }
 
 uint32_t observed_count(uint32_t steps, uint32_t has_eos, uint32_t eos, const Slot *slots) {
@@ -717,6 +741,8 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_rope_cs = c.take(HD * 4);
   const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
+  const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
+  const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(rq->vocab_size));
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
   const uint64_t off_chain_trace = c.take(static_cast<uint64_t>(rq->layer_count) * 32 * 8);
   const uint64_t front_ws_bytes = front_workspace_bytes(rq->heads, rq->kv_heads);
@@ -766,6 +792,8 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
   s->sample_ws = s->arena + off_sample_ws;
+  s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
+  s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
   s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
   s->chain_abort = reinterpret_cast<uint32_t *>(s->arena + off_chain + chain_flag_bytes());
   {
@@ -979,21 +1007,17 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
                                                NervaHipHfDecodeSequenceResult *out) {
   if (!begin_result(out)) return -1;
   if (request == nullptr || request->session == nullptr || request->prompt_tokens == nullptr ||
-      request->prompt_token_count == 0 || !sampler_valid(request->sampler))
+      request->prompt_token_count == 0)
     return -1;
   Session *s = request->session;
   if (request->prompt_token_count > s->max_ctx) return -1;
   for (uint32_t i = 0; i < request->prompt_token_count; ++i)
     if (request->prompt_tokens[i] >= s->vocab) return -1;
-  if (!sampler_greedy(request->sampler)) {
-    out->device_count = 1;
-    out->hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED;
-    return -1;
-  }
   const uint32_t P = request->prompt_token_count;
   fill_header(s, out, 0, request->prompt_tokens[P - 1]);
   s->started = false;
-  hipError_t err = reset_sequence(s, request->prompt_tokens, P, out);
+  hipError_t err = set_sampler(s, request->sampler);   // session_api_lifecycle.inc.cu:1026
+  if (err == hipSuccess) err = reset_sequence(s, request->prompt_tokens, P, out);
   // prefill: P-1 prompt steps (graph replay) + one prompt step with the LM head and sampler
   if (err == hipSuccess && P > 1) err = ensure_graph(s, 1, out);
   if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
@@ -1041,11 +1065,11 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
   fill_header(s, out, request->steps, seed);
 
   hipError_t err = hipSuccess;
-  if (run_count != 0) err = ensure_graph(s, 0, out);
+  if (run_count != 0) err = ensure_graph(s, decode_graph(s), out);
   const uint64_t allocs_before = allocation_count();
   if (err == hipSuccess && run_count != 0) err = hipEventRecord(s->ev0, s->stream);
   for (uint32_t step = 0; err == hipSuccess && step < run_count; ++step) {
-    err = launch_step(s, 0, out);
+    err = launch_step(s, decode_graph(s), out);
     // With a stop token the host looks at each token so that it can stop launching
     // (session_api_lifecycle.inc.cu:1206-1234); without one the loop never syncs.
     if (err == hipSuccess && s->has_eos != 0) {
@@ -1110,7 +1134,6 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
       request->output_tokens == nullptr || request->steps == 0 || request->prompt_token_count == 0 ||
       request->output_token_capacity < request->steps ||
       request->prompt_tokens[request->prompt_token_count - 1u] != request->seed_token ||
-      !sampler_valid(request->sampler) ||
       request->prompt_token_count > UINT32_MAX - request->steps + 1u)
     return -1;
   Session *s = request->session;
@@ -1119,20 +1142,16 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
   if (context_steps > s->max_ctx) return -1;
   for (uint32_t i = 0; i < P; ++i)
     if (request->prompt_tokens[i] >= s->vocab) return -1;
-  if (!sampler_greedy(request->sampler)) {
-    out->device_count = 1;
-    out->hip_error = NERVA_HIP_ERROR_NOT_SUPPORTED;
-    return -1;
-  }
   fill_header(s, out, request->steps, request->seed_token);
   s->started = false;
-  hipError_t err = reset_sequence(s, request->prompt_tokens, P, out);
+  hipError_t err = set_sampler(s, request->sampler);   // session_api_lifecycle.inc.cu:770
+  if (err == hipSuccess) err = reset_sequence(s, request->prompt_tokens, P, out);
   // the decode-step graph walks every position, prompt included (session_api_lifecycle.inc.cu:748-990)
-  if (err == hipSuccess) err = ensure_graph(s, 0, out);
+  if (err == hipSuccess) err = ensure_graph(s, decode_graph(s), out);
   const uint64_t allocs_before = allocation_count();
   if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
   for (uint32_t step = 0; err == hipSuccess && step < context_steps; ++step) {
-    err = launch_step(s, 0, out);
+    err = launch_step(s, decode_graph(s), out);
   }
   if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
   const uint64_t slots_bytes = static_cast<uint64_t>(context_steps) * sizeof(Slot);

@@ -44,6 +44,25 @@ struct SampleParams {
   uint32_t *token_out;     // optional: plain token output (operator entry point)
 };
 
+// One lane: hands the step's token out - plain output word and/or slot[pos] in the reference's
+// slot format (nerva_cuda_api.h:29-37, sampler.cu:394-407) plus the cursor bump.
+__device__ __forceinline__ void publish_token(const SampleParams &s, uint32_t token) {
+  if (s.token_out != nullptr) *s.token_out = token;
+  if (s.slots != nullptr) {
+    const uint32_t pos = *s.cursor_rw;
+    NervaHipSyntheticTokenSlot slot;
+    slot.request_id = NERVA_HIP_SLOT_REQUEST_ID;
+    slot.sequence_id = NERVA_HIP_SLOT_SEQUENCE_ID;
+    slot.token_index = pos;
+    slot.token = token;
+    slot.version = static_cast<uint64_t>(pos) + 1u;
+    slot.completion = NERVA_HIP_SLOT_DEVICE_COMPLETE;
+    slot.host_copied = 0;
+    s.slots[pos] = slot;
+    *s.cursor_rw = pos + 1u;
+  }
+}
+
 struct GemvParams {
   const uint16_t *w;
   const uint16_t *x16;

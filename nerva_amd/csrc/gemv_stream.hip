@@ -46,21 +46,7 @@ __global__ __launch_bounds__(1024) void sample_finish_kernel(SampleParams s, uin
       Best o{red_v[w], red_i[w], red_h[w]};
       if (better(o, t)) t = o;
     }
-    const uint32_t token = t.has ? t.index : 0u;
-    if (s.token_out != nullptr) *s.token_out = token;
-    if (s.slots != nullptr) {
-      const uint32_t pos = *s.cursor_rw;
-      NervaHipSyntheticTokenSlot slot;
-      slot.request_id = NERVA_HIP_SLOT_REQUEST_ID;
-      slot.sequence_id = NERVA_HIP_SLOT_SEQUENCE_ID;
-      slot.token_index = pos;
-      slot.token = token;
-      slot.version = static_cast<uint64_t>(pos) + 1u;
-      slot.completion = NERVA_HIP_SLOT_DEVICE_COMPLETE;
-      slot.host_copied = 0;
-      s.slots[pos] = slot;
-      *s.cursor_rw = pos + 1u;
-    }
+    publish_token(s, t.has ? t.index : 0u);
   }
 }
 

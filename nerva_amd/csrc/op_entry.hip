@@ -11,6 +11,7 @@
 
 #include "argmax.cuh"
 #include "attn_decode.cuh"
+#include "sampler.cuh"
 #include "fp8_gemv.cuh"
 #include "gemv_stream.cuh"
 #include "nerva_hip_layout_check.hpp"
@@ -440,6 +441,38 @@ int nerva_hip_argmax(const NervaHipArgmaxRequest *r, void *stream, int32_t *hip_
   sample_bind_workspace(s, r->workspace);
   s.token_out = r->token;
   return finish(launch_argmax(r->logits, r->count, s, resolve_stream(stream)), hip_error);
+}
+
+__global__ void store_sampler_config_kernel(SamplerDev *dst, SamplerDev value) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *dst = value;
+}
+
+// workspace: sampler parameters (256 B), chunk candidates, chunk keys
+uint64_t nerva_hip_sample_workspace_bytes(uint32_t vocab) {
+  return 256u + ((sample_workspace_bytes() + 255u) & ~uint64_t{255}) + sampler_workspace_bytes(vocab);
+}
+
+int nerva_hip_sample(const NervaHipSampleRequest *r, void *stream, int32_t *hip_error) {
+  if (hip_error) *hip_error = 0;
+  if (r == nullptr || r->logits == nullptr || r->token == nullptr || r->workspace == nullptr || r->vocab == 0)
+    return finish(hipErrorInvalidValue, hip_error);
+  char *ws = static_cast<char *>(r->workspace);
+  const SamplerDev config = sampler_device_config(r->sampler);
+  hipStream_t st = resolve_stream(stream);
+  // the parameters travel as a kernel argument (a host-to-device copy of a stack variable could
+  // not be recorded into a graph)
+  hipLaunchKernelGGL(store_sampler_config_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<SamplerDev *>(ws), config);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return finish(err, hip_error);
+  SamplerParams p{};
+  p.logits = r->logits;
+  p.vocab = r->vocab;
+  p.config = reinterpret_cast<const SamplerDev *>(ws);
+  sample_bind_workspace(p.out, ws + 256);
+  p.out.token_out = r->token;
+  p.keys = reinterpret_cast<uint64_t *>(ws + 256 + ((sample_workspace_bytes() + 255u) & ~uint64_t{255}));
+  p.position = r->position;
+  return finish(launch_sampler(p, st), hip_error);
 }
 
 int nerva_hip_moe_fp8_experts(const NervaHipMoeFp8Request *r, void *stream, int32_t *hip_error) {

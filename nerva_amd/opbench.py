@@ -5,6 +5,7 @@
   2. MLP block (RMSNorm -> gate/up GEMV -> SwiGLU -> down GEMV -> +residual), hidden 4096, MLP 12288
   3. paged GQA decode attention, 32 q / 8 kv heads x 128, 4096 cached tokens + the new one
   4. FP8 (e4m3, 128x128 block scales) MoE: 8 routed + 1 shared expert, hidden 7168, MLP 2048
+  5. the token sampler over 151936 logits (greedy, temperature over the whole vocabulary, top-k / top-p)
 
 Each case is timed twice: "rotating" cycles through enough distinct copies of the weights / cache that
 the working set exceeds 1 GB (nothing is served from cache), "resident" repeats one copy. The launches
@@ -148,6 +149,28 @@ def case_moe():
         report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
 
 
+def case_sampler():
+    V = 151936
+    lib = abi.load()
+    logits = synth32(V, 51, std=3.0)
+    ws = DeviceBuffer.zeros(lib.nerva_hip_sample_workspace_bytes(V))
+    tok = DeviceBuffer.zeros(16)
+    nbytes = V * 4
+    for name, temperature, top_p, top_k in (("greedy", 0.0, 1.0, 0), ("T=0.7 whole vocabulary", 0.7, 1.0, 0),
+                                            ("T=0.7 top_p 0.9 (k=128)", 0.7, 0.9, 0), ("T=0.7 top_k 40", 0.7, 1.0, 40)):
+        req = abi.NervaHipSampleRequest()
+        req.vocab, req.logits, req.token, req.workspace = V, logits.ptr, tok.ptr, ws.ptr
+        req.sampler.temperature, req.sampler.top_p, req.sampler.top_k, req.sampler.seed = temperature, top_p, top_k, 1
+        err = C.c_int32(0)
+
+        def enqueue(i):
+            req.position = i
+            assert lib.nerva_hip_sample(C.byref(req), None, C.byref(err)) == 0
+        ns = timed(enqueue, 16)
+        report("5 sampler, 151936 logits", name[:9], ns, nbytes)
+        log("    (%s: two launches, after the LM head has left the logits in memory)" % name)
+
+
 def main():
     rc, smoke = Device.smoke()
     if rc != 0:
@@ -158,6 +181,7 @@ def main():
     case_mlp()
     case_attention()
     case_moe()
+    case_sampler()
 
 
 if __name__ == "__main__":

@@ -236,6 +236,20 @@ def argmax(logits_buf, count, workspace=None):
     return int(tok.numpy(np.uint32, 1)[0])
 
 
+def sample(logits_buf, vocab, temperature, top_p, top_k, seed, position, workspace=None):
+    """One token from device logits by the session's sampler rule (greedy / Gumbel-max / top-k + top-p)."""
+    lib = abi.load()
+    ws = workspace or DeviceBuffer.zeros(lib.nerva_hip_sample_workspace_bytes(vocab))
+    tok = DeviceBuffer.zeros(16)
+    req = abi.NervaHipSampleRequest()
+    req.vocab, req.position, req.logits, req.token, req.workspace = vocab, position, _ptr(logits_buf), tok.ptr, ws.ptr
+    req.sampler.temperature, req.sampler.top_p, req.sampler.top_k, req.sampler.seed = temperature, top_p, top_k, seed
+    err = C.c_int32(0)
+    _check(lib.nerva_hip_sample(C.byref(req), None, C.byref(err)), err, "nerva_hip_sample")
+    Device.synchronize()
+    return int(tok.numpy(np.uint32, 1)[0])
+
+
 def moe_route_softmax(logits, top_k, normalize=True):
     logits = np.ascontiguousarray(logits, np.float32)
     dl = DeviceBuffer.from_numpy(logits)

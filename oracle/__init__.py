@@ -84,6 +84,9 @@ _sig("nvo_attention_blockwise", C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, f32
 _sig("nvo_attention_paged16", C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32,
      f32p, u16p, u16p, u32p, C.c_uint64, C.c_uint64, C.c_uint64, f32p)
 _sig("nvo_greedy_argmax", C.c_int, f32p, C.c_uint64, C.c_int, u32p)
+_sig("nvo_sampler_mix64", C.c_uint64, C.c_uint64)
+_sig("nvo_sampler_uniform", C.c_float, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32)
+_sig("nvo_sample", C.c_int, f32p, C.c_uint32, C.c_float, C.c_float, C.c_uint32, C.c_uint64, C.c_uint32, u32p, f32p)
 _sig("nvo_moe_route_softmax", C.c_int, f32p, C.c_uint32, C.c_uint32, C.c_uint32, u32p, f32p)
 _sig("nvo_moe_forward_f32", C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32,
      C.c_float, f32p, u32p, f32p, f32p, f32p, f32p, C.c_uint32, f32p, f32p, f32p, f32p)
@@ -242,6 +245,25 @@ def greedy_argmax(logits, skip_nonfinite=False):
     if rc != 0:
         raise ValueError("greedy argmax rejected the logits")
     return out.value
+
+
+def sampler_mix64(value):
+    return int(lib.nvo_sampler_mix64(C.c_uint64(value & 0xFFFFFFFFFFFFFFFF)))
+
+
+def sampler_uniform(seed, position, token, salt):
+    return float(lib.nvo_sampler_uniform(C.c_uint64(seed), position, token, salt))
+
+
+def sample(logits, temperature, top_p, top_k, seed, position):
+    """(token, margin) of the device sampler's rule (greedy / Gumbel-max / top-k + top-p draw)."""
+    l = _f32(logits)
+    token, margin = C.c_uint32(0), C.c_float(0.0)
+    rc = lib.nvo_sample(_p(l, f32p), l.size, temperature, top_p, top_k, C.c_uint64(seed), position,
+                        C.byref(token), C.byref(margin))
+    if rc != 0:
+        raise ValueError("sampler rejected the logits")
+    return token.value, margin.value
 
 
 def moe_route_softmax(logits, top_k, normalize):

@@ -23,6 +23,10 @@
 //   moe route / experts        - reference closed-form KATs
 //   block forward              - reference output bits [16126, 17299] + FNV hash
 //   greedy loop                - reference token stream [1,2,3,0]
+//   sampler (non-greedy)       - the reference holds no golden vector for it (its tests compare two
+//                                of its own device paths); pinned by the published splitmix64 outputs
+//                                for seed 0 (hash), the closed form of the uniform, brute-force sorting
+//                                (top-k selection) and an f64 cumulative distribution (top-p and draw)
 //   synthetic generator        - not a reference function (defined by this build)
 // No function of this oracle is "parity unpinned".
 
@@ -759,6 +763,129 @@ NVO_API int nvo_ctx_forward_token(NvoContext *c, uint32_t token, int prompt_toke
 // embed(token) -> layers -> final norm -> lm_head -> argmax per step; stop after
 // emitting `eos_token` when has_eos. Returns the number of tokens written.
 // margins (optional, [steps]) receives top1-top2 logit margin per emitted token.
+// ---- sampler beyond greedy -------------------------------------------------------------------
+// sampler.cu:18-23 sampler_mix64: the splitmix64 output function applied to value + golden ratio.
+NVO_API uint64_t nvo_sampler_mix64(uint64_t value) {
+  value += 0x9e3779b97f4a7c15ull;
+  value = (value ^ (value >> 30)) * 0xbf58476d1ce4e5b9ull;
+  value = (value ^ (value >> 27)) * 0x94d049bb133111ebull;
+  return value ^ (value >> 31);
+}
+// sampler.cu:25-33 sampler_uniform_open: 24 hashed bits -> (0, 1).
+NVO_API float nvo_sampler_uniform(uint64_t seed, uint32_t position, uint32_t token, uint32_t salt) {
+  uint64_t value = seed ^ ((uint64_t)position << 32) ^ (uint64_t)token ^ ((uint64_t)salt << 48);
+  value = nvo_sampler_mix64(value);
+  const uint32_t mantissa = (uint32_t)((value >> 40) & 0x00ffffffu);
+  return ((float)mantissa + 1.0f) / 16777217.0f;
+}
+// sampler.cu:35-40 (value desc, index asc).
+static bool sampler_better(float lv, uint32_t li, float rv, uint32_t ri) {
+  return lv > rv || (lv == rv && li < ri);
+}
+// One sampled token (sampler.cu:66-392). Three branches, as there:
+//   greedy            !(temperature > 0) || top_k == 1: first maximum among finite logits
+//   whole vocabulary  top_k == 0 && top_p >= 0.999999: Gumbel-max, argmax of
+//                     logit / T - log(-log(u(seed, position, index, 0)))
+//   top-k / top-p     the k = (top_k == 0 ? 128 : min(top_k, 128)) best finite logits by (value desc,
+//                     index asc); softmax with temperature over them, summed in that order; the nucleus
+//                     is the shortest prefix whose share reaches top_p; one draw u(seed, position, 0, 1)
+//                     times the kept mass picks the first entry whose running sum reaches it.
+// `margin` (optional) tells how far the decision was from flipping, so that a caller comparing with
+// another implementation of expf/logf can set near-ties aside: greedy/Gumbel = best score minus
+// the runner-up's; top-k = distance of the draw to the nearest boundary of the chosen entry's
+// interval, as a fraction of the kept mass.
+NVO_API int nvo_sample(const float *logits, uint32_t vocab, float temperature, float top_p, uint32_t top_k,
+                       uint64_t seed, uint32_t position, uint32_t *token, float *margin) {
+  if (vocab == 0) return -1;
+  if (margin) *margin = INFINITY;
+  const bool greedy = !(temperature > 0.0f) || top_k == 1;
+  if (greedy || (top_k == 0 && top_p >= 0.999999f)) {
+    const float inv_t = greedy ? 1.0f : 1.0f / temperature;
+    float best = -INFINITY, second = -INFINITY;
+    uint32_t best_i = 0;
+    for (uint32_t i = 0; i < vocab; ++i) {
+      const float v = logits[i];
+      if (!isfinite(v)) continue;
+      float s = v;
+      if (!greedy) {
+        const float u = nvo_sampler_uniform(seed, position, i, 0);
+        s = v * inv_t + (-logf(-logf(u)));
+      }
+      if (sampler_better(s, i, best, best_i)) {
+        second = best;
+        best = s;
+        best_i = i;
+      } else if (s > second) {
+        second = s;
+      }
+    }
+    *token = best_i;
+    if (margin) *margin = best - second;
+    return 0;
+  }
+  const uint32_t requested = top_k == 0 ? 128u : (top_k < 128u ? top_k : 128u);
+  const uint32_t want = requested < vocab ? requested : vocab;
+  std::vector<std::pair<float, uint32_t>> cand;
+  cand.reserve(vocab);
+  for (uint32_t i = 0; i < vocab; ++i)
+    if (isfinite(logits[i])) cand.emplace_back(logits[i], i);
+  const uint32_t selected = (uint32_t)std::min<size_t>(want, cand.size());
+  std::partial_sort(cand.begin(), cand.begin() + selected, cand.end(),
+                    [](const std::pair<float, uint32_t> &a, const std::pair<float, uint32_t> &b) {
+                      return sampler_better(a.first, a.second, b.first, b.second);
+                    });
+  if (selected == 0) {
+    *token = 0;
+    return 0;
+  }
+  const float inv_t = 1.0f / temperature;
+  const float max_value = cand[0].first;
+  float total = 0.0f;
+  for (uint32_t i = 0; i < selected; ++i) total += expf((cand[i].first - max_value) * inv_t);
+  float kept_total = 0.0f;
+  uint32_t kept = selected;
+  float nucleus_gap = INFINITY;  // how close any examined prefix share came to top_p
+  if (top_p < 0.999999f) {
+    kept = 0;
+    for (uint32_t i = 0; i < selected; ++i) {
+      kept_total += expf((cand[i].first - max_value) * inv_t);
+      kept = i + 1;
+      if (total > 0.0f) nucleus_gap = fminf(nucleus_gap, fabsf(kept_total / total - top_p));
+      if (total > 0.0f && kept_total / total >= top_p) break;
+    }
+  } else {
+    kept_total = total;
+  }
+  if (kept_total <= 0.0f || kept == 0) {
+    *token = cand[0].second;
+    return 0;
+  }
+  const float draw = nvo_sampler_uniform(seed, position, 0, 1) * kept_total;
+  float cumulative = 0.0f;
+  uint32_t pick = kept - 1;
+  float lower = 0.0f, upper = kept_total;
+  bool found = false;
+  for (uint32_t i = 0; i < kept; ++i) {
+    const float before = cumulative;
+    cumulative += expf((cand[i].first - max_value) * inv_t);
+    if (draw <= cumulative) {
+      pick = i;
+      lower = before;
+      upper = cumulative;
+      found = true;
+      break;
+    }
+  }
+  if (!found) lower = cumulative;
+  *token = cand[pick].second;
+  if (margin) {
+    const float below = pick == 0 ? INFINITY : (draw - lower) / kept_total;       // flips to the entry before
+    const float above = pick + 1 == kept ? INFINITY : (upper - draw) / kept_total;  // the last entry also takes what is left
+    *margin = fminf(fminf(below, above), nucleus_gap);
+  }
+  return 0;
+}
+
 NVO_API int nvo_greedy_decode(NvoContext *c, const uint32_t *prompt, uint32_t prompt_count,
                               uint32_t steps, uint32_t has_eos, uint32_t eos_token,
                               uint32_t *out_tokens, float *margins) {

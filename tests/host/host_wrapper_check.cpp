@@ -104,14 +104,25 @@ static void gpu_checks() {
     CHECK(b.status == SmokeStatus::Ok && b.tokens == std::vector<uint32_t>({3}) && started.loop_state->finished());
     CHECK(started.loop_state->advance(1).status == SmokeStatus::Failed);
   }
-  // refusals: prompt outside the vocabulary (before the call), non-greedy sampling (by the library)
+  // refusal before the call: prompt outside the vocabulary
   std::vector<uint32_t> outside{9};
   CHECK(HipHfDecodeSequenceLoop::start(session, outside).summary.status == SmokeStatus::Failed);
+  // temperature sampling: served, reproducible for a seed, tokens inside the vocabulary
   HipHfDecodeSamplerConfig hot;
   hot.temperature = 0.8f;
   hot.top_k = 40;
-  auto refused = HipHfDecodeSequenceLoop::start_with_sampler(session, prompt, std::nullopt, hot);
-  CHECK(refused.summary.status == SmokeStatus::Failed && refused.summary.hip_error == NERVA_HIP_ERROR_NOT_SUPPORTED);
+  hot.seed = 11;
+  std::vector<uint32_t> first;
+  for (int round = 0; round < 2; ++round) {
+    auto sampled = HipHfDecodeSequenceLoop::start_with_sampler(session, prompt, std::nullopt, hot);
+    CHECK(sampled.summary.status == SmokeStatus::Ok && sampled.loop_state.has_value());
+    if (!sampled.loop_state) break;
+    HipHfDecodeSequenceSummary a = sampled.loop_state->advance(3);
+    CHECK(a.status == SmokeStatus::Ok && a.tokens.size() == 3);
+    for (uint32_t tok : a.tokens) CHECK(tok < 4);
+    if (round == 0) first = a.tokens;
+    else CHECK(a.tokens == first);
+  }
 }
 
 int main(int argc, char **argv) {

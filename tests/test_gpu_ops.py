@@ -393,6 +393,49 @@ def test_argmax_matches_oracle_rules():
         assert N.argmax(dev(l), l.size, ws) == 90000
 
 
+SAMPLER_CONFIGS = [(0.7, 0.9, 0), (1.0, 1.0, 0), (1.5, 0.5, 40), (0.3, 1.0, 3), (1.0, 0.8, 200), (0.0, 1.0, 0),
+                   (2.0, 0.9, 1), (0.9, 1.0, 128), (float("nan"), 2.0, 0)]
+
+
+def test_sampler_matches_oracle_rule():
+    """Same token as the oracle's restatement of the reference rule, at the full vocabulary and at ragged
+    small ones, with ties and non-finite logits. The selection is integer work and exact; the device's
+    exp/log may differ from the host's in the last bit, so a draw closer than 1e-5 (of the kept mass, or
+    of the runner-up's score) to a boundary is set aside - and such draws have to stay rare."""
+    rng = np.random.default_rng(5)
+    close = checked = 0
+    for n in (151936, 1000, 1025, 7, 1):
+        l = (rng.standard_normal(n) * 3).astype(np.float32)
+        if n > 100:
+            l[rng.integers(0, n, 4)] = l.max()               # exact ties at the top
+            l[rng.integers(0, n, 2)] = np.nan
+            l[rng.integers(0, n, 2)] = np.inf
+        buf = dev(l)
+        ws = N.DeviceBuffer.zeros(abi.load().nerva_hip_sample_workspace_bytes(n))
+        for temperature, top_p, top_k in SAMPLER_CONFIGS:
+            for position in (0, 1, 8191, 70000):
+                seed = int(rng.integers(0, 2 ** 62))
+                want, margin = O.sample(l, 0.0 if temperature != temperature else temperature,
+                                        1.0 if top_p > 1.0 else top_p, top_k, seed, position)
+                got = N.sample(buf, n, temperature, top_p, top_k, seed, position, ws)
+                checked += 1
+                if got != want:
+                    assert margin < 1e-5, (n, temperature, top_p, top_k, position, got, want, margin)
+                    close += 1
+    assert close <= checked // 50
+    # logits piled into the first chunks: the bound from the chunk maxima prunes nothing, and the
+    # selection takes its general route (radix selection over all chunk candidates)
+    l = (-1e-3 * np.arange(151936)).astype(np.float32)
+    l[5] = l[3]                                               # a tie inside the top
+    buf = dev(l)
+    ws = N.DeviceBuffer.zeros(abi.load().nerva_hip_sample_workspace_bytes(l.size))
+    for temperature, top_p, top_k in ((0.01, 1.0 - 1e-4, 0), (0.5, 0.9, 100), (5.0, 0.99, 7)):
+        for position in range(6):
+            want, margin = O.sample(l, temperature, top_p, top_k, 77, position)
+            got = N.sample(buf, l.size, temperature, top_p, top_k, 77, position, ws)
+            assert got == want or margin < 1e-5, (temperature, top_p, top_k, position, got, want, margin)
+
+
 def test_moe_route_matches_oracle():
     rng = np.random.default_rng(3)
     for e, k, norm in ((256, 8, True), (256, 8, False), (64, 6, True), (5, 5, True)):
