@@ -456,6 +456,30 @@ typedef struct NervaHipArgmaxRequest {
 int nerva_hip_argmax(const NervaHipArgmaxRequest *request, void *stream, int32_t *hip_error);
 uint64_t nerva_hip_argmax_workspace_bytes(void);
 
+typedef struct NervaHipGemmRowsRequest {
+  uint32_t dtype;            /* NERVA_HIP_DTYPE_* of weights and 16-bit vectors */
+  uint32_t rows, cols;       /* W is row-major [rows x cols] (epilogue 2: [2*rows x cols], gate rows first) */
+  uint32_t tokens;           /* 1..32 input rows */
+  uint32_t epilogue;         /* 0: f32 out; 1: f32 out = y + bias + residual; 2: out16 = round16(silu(gate)*up) */
+  uint32_t round_output;     /* epilogue 1: round the sum to 16 bits (prompt-token staging) */
+  const uint16_t *weights;
+  const uint16_t *input16;   /* [tokens][cols] */
+  const uint16_t *bias;      /* optional [rows] ([2*rows] for epilogue 2) */
+  const float *residual;     /* epilogue 1: [tokens][rows] */
+  float *output_f32;         /* epilogues 0, 1: [tokens][rows] */
+  uint16_t *output16;        /* epilogue 2: [tokens][rows] */
+} NervaHipGemmRowsRequest;
+
+/* Projection of a block of up to 32 token rows through one weight matrix on the matrix cores,
+ * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
+ * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
+ * prefill and projection batch (projection.cu:99-106, 297-300). rows % 16 == 0, cols % 2048 == 0. */
+int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *request, void *stream, int32_t *hip_error);
+/* out16[t] = round16(rmsnorm(x[t]) * gamma) for `tokens` rows of `cols` f32 values
+ * (rms_norm_encoded_into, ops.rs:31-50, once per row). */
+int nerva_hip_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
+                           uint32_t cols, uint16_t *out16, void *stream, int32_t *hip_error);
+
 typedef struct NervaHipSampleRequest {
   uint32_t vocab;
   uint32_t position;            /* sequence position of the sampled token: the random-number counter */

@@ -1,0 +1,46 @@
+// Multi-row projection on the matrix cores: Y[t][r] = sum_c W[r][c] * X[t][c] for a block of
+// T <= 32 token rows, streaming the weight matrix once for all of them. This is what a chunk of
+// prompt tokens (and a small batch of sequences) needs: the weight bytes are the same as for one
+// token, so the kernel is HBM-bound like the GEMV and T tokens cost about one.
+// Reference: the cuBLAS GEMM calls of the chunked prefill and of the projection batch
+// (native/cuda/hf_decode_sequence/projection.cu:99-106, 297-300; session_decode_prefill.inc.cu:
+// 1879-2243); arithmetic as mat_vec_encoded_row_major per token (precision/block/ops.rs:75-91).
+//
+// gfx950 mapping: a workgroup owns 16 weight rows (for SwiGLU: 16 gate rows and their 16 up
+// rows) over the full K; its 8 waves split K. A wave walks its K range in blocks of 256 columns:
+// the block of W is requested with coalesced loads (512 contiguous bytes per row and
+// instruction, like the GEMV), parked in a wave-private LDS tile and read back in matrix-operand
+// order; the X operand comes straight from global memory (L2), one 16-byte piece per lane, token
+// and K-step. v_mfma_f32_16x16x32 accumulates D[weight row][token] in f32, two token tiles per
+// wave; the waves' partial sums meet in LDS and are added in wave order (deterministic), then
+// the epilogue runs once per output element.
+#pragma once
+
+#include "nv_common.cuh"
+
+namespace nv {
+
+constexpr uint32_t kGemmMaxTokens = 32;
+enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
+
+struct GemmRowsParams {
+  const uint16_t *w;         // [rows][cols] row-major 16-bit (SwiGLU: [2*rows][cols], gate rows first)
+  const uint16_t *x16;       // [tokens][cols] 16-bit inputs
+  const uint16_t *bias;      // optional [rows] (SwiGLU: [2*rows])
+  const float *residual;     // kGemmResidual: [tokens][rows]
+  float *out_f32;            // kGemmF32 / kGemmResidual: [tokens][rows]
+  uint16_t *out16;           // kGemmSwiglu: [tokens][rows] = round16(silu(gate) * up)
+  uint32_t rows, cols, tokens;
+  uint32_t round_out;        // kGemmResidual: round the sum to 16 bit
+};
+
+// rows % 16 == 0, cols % 2048 == 0 (each of the 8 waves walks whole 256-column blocks),
+// 1 <= tokens <= kGemmMaxTokens, 16-byte aligned w and x16.
+bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens);
+hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream);
+
+// x16[t] = round16(x[t] * rsqrt(mean(x[t]^2) + eps) * gamma) for `tokens` rows of `cols` f32 values.
+hipError_t launch_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
+                               uint32_t cols, uint16_t *out16, hipStream_t stream);
+
+}  // namespace nv

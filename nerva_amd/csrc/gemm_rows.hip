@@ -1,0 +1,215 @@
+// Multi-row projection on the matrix cores (see gemm_rows.cuh).
+#include "gemm_rows.cuh"
+
+#include <mutex>
+
+namespace nv {
+
+namespace {
+
+constexpr int kGW = 8;                          // waves per workgroup: they split K
+constexpr int kGThreads = kGW * kWave;
+constexpr int kKB = 256;                        // columns per staged block (512 B per row)
+constexpr int kRowStride = kKB + 8;             // LDS row stride in elements: 16 B of padding keeps
+                                                // the 16 rows of an operand read on distinct banks
+constexpr int kTileElems = 16 * kRowStride;     // one 16-row block of W in LDS
+constexpr int kSteps = kKB / 32;                // matrix-core K-steps per block
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// D(16x16) += A(16x32) . B(32x16): lane l holds A[l%16][8*(l/16)..+7], B[8*(l/16)..+7][l%16] and
+// D[4*(l/16)..+3][l%16].
+template <uint32_t DT>
+__device__ __forceinline__ f32x4_t mfma_k32(const uint4 &a, const uint4 &b, f32x4_t c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                  0, 0);
+}
+
+template <int NR>
+constexpr size_t gemm_lds_bytes() {
+  const size_t tiles = static_cast<size_t>(kGW) * NR * kTileElems * sizeof(uint16_t);
+  const size_t partials = static_cast<size_t>(kGW) * NR * 16 * kGemmMaxTokens * sizeof(float);
+  return tiles > partials ? tiles : partials;
+}
+
+template <uint32_t DT, int EPI>
+__global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) {
+  constexpr int NR = EPI == kGemmSwiglu ? 2 : 1;  // SwiGLU: the gate rows and the up rows of the same outputs
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  uint16_t *tile = reinterpret_cast<uint16_t *>(smem) + static_cast<size_t>(wave) * NR * kTileElems;
+  const uint32_t cols = p.cols, T = p.tokens;
+  const uint32_t row0 = blockIdx.x * 16u;
+  const uint32_t kper = cols / kGW, nblk = kper / kKB, kbase = wave * kper;
+
+  // W block -> registers: instruction i covers rows 2i and 2i + 1, 32 lanes x 16 B each
+  const uint16_t *wp[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j)
+    wp[j] = p.w + static_cast<uint64_t>(row0 + j * p.rows + (lane >> 5)) * cols + kbase + (lane & 31) * 8;
+  uint4 areg[NR][8];
+#define NV_GEMM_REQUEST(BLK)                                                                        \
+  _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 8; ++i)      \
+      areg[j][i] = load_stream(wp[j] + static_cast<uint64_t>(2 * i) * cols + (BLK) * kKB)
+  uint16_t *park_at = tile + (lane >> 5) * kRowStride + (lane & 31) * 8;
+#define NV_GEMM_PARK()                                                                              \
+  _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 8; ++i)      \
+      *reinterpret_cast<uint4 *>(park_at + j * kTileElems + 2 * i * kRowStride) = areg[j][i]
+
+  // X operand: token of this lane in each of the two token tiles (clamped: columns past T are dropped later)
+  const uint32_t n = lane & 15, q = lane >> 4;
+  const uint16_t *xp0 = p.x16 + static_cast<uint64_t>(min(n, T - 1)) * cols + kbase + q * 8;
+  const uint16_t *xp1 = p.x16 + static_cast<uint64_t>(min(n + 16u, T - 1)) * cols + kbase + q * 8;
+  const uint16_t *a_read = tile + n * kRowStride + q * 8;
+
+  f32x4_t acc[NR][2];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) acc[j][0] = acc[j][1] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  uint4 breg[kSteps][2];
+#define NV_GEMM_LOAD_X(BLK)                                                                         \
+  _Pragma("unroll") for (int s = 0; s < kSteps; ++s) {                                              \
+    breg[s][0] = *reinterpret_cast<const uint4 *>(xp0 + (BLK) * kKB + s * 32);                      \
+    breg[s][1] = *reinterpret_cast<const uint4 *>(xp1 + (BLK) * kKB + s * 32);                      \
+  }
+#define NV_GEMM_COMPUTE()                                                                           \
+  _Pragma("unroll") for (int s = 0; s < kSteps; ++s) _Pragma("unroll") for (int j = 0; j < NR; ++j) { \
+    const uint4 a = *reinterpret_cast<const uint4 *>(a_read + j * kTileElems + s * 32);             \
+    acc[j][0] = mfma_k32<DT>(a, breg[s][0], acc[j][0]);                                             \
+    acc[j][1] = mfma_k32<DT>(a, breg[s][1], acc[j][1]);                                             \
+  }
+
+  // Order of requests per block: this block's X pieces, then the next block of W. Loads return in
+  // order, so the X pieces are usable while the next W block is still on its way. No request sits
+  // under a branch (the last block is peeled off), so the compiler's waits stay exact.
+  NV_GEMM_REQUEST(0);
+  uint32_t blk = 0;
+  for (; blk + 1 < nblk; ++blk) {
+    NV_GEMM_PARK();
+    NV_GEMM_LOAD_X(blk);
+    NV_GEMM_REQUEST(blk + 1);
+    NV_GEMM_COMPUTE();
+  }
+  NV_GEMM_PARK();
+  NV_GEMM_LOAD_X(blk);
+  NV_GEMM_COMPUTE();
+#undef NV_GEMM_REQUEST
+#undef NV_GEMM_PARK
+#undef NV_GEMM_LOAD_X
+#undef NV_GEMM_COMPUTE
+
+  // ---- partial sums of the 8 waves meet in LDS (the W tiles are done with)
+  __syncthreads();
+  float *red = reinterpret_cast<float *>(smem);  // [wave][j][row 16][token 32]
+#pragma unroll
+  for (int j = 0; j < NR; ++j)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        red[((wave * NR + j) * 16 + q * 4 + r) * kGemmMaxTokens + c * 16 + n] = acc[j][c][r];
+  __syncthreads();
+  // one thread per output element: 16 rows x 32 tokens, rows fastest (contiguous stores per token)
+  const uint32_t r = threadIdx.x & 15u, t = threadIdx.x >> 4;
+  if (t >= T) return;
+  float y[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kGW; ++w) sum += red[((w * NR + j) * 16 + r) * kGemmMaxTokens + t];
+    if (p.bias != nullptr) sum += dec16<DT>(p.bias[row0 + j * p.rows + r]);
+    y[j] = sum;
+  }
+  const uint64_t at = static_cast<uint64_t>(t) * p.rows + row0 + r;
+  if constexpr (EPI == kGemmF32) {
+    p.out_f32[at] = y[0];
+  } else if constexpr (EPI == kGemmResidual) {
+    float v = y[0] + p.residual[at];
+    if (p.round_out) v = round16<DT>(v);
+    p.out_f32[at] = v;
+  } else {
+    p.out16[at] = enc16<DT>(silu(y[0]) * y[NR - 1]);
+  }
+}
+
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock) void rmsnorm_rows_kernel(const float *x, const uint16_t *gamma, float eps,
+                                                              uint32_t cols, uint16_t *out16) {
+  __shared__ float red[kWavesPerBlock];
+  const float *row = x + static_cast<uint64_t>(blockIdx.x) * cols;
+  float ss = 0.0f;
+  for (uint32_t c = threadIdx.x; c < cols; c += kBlock) ss += row[c] * row[c];
+  ss = block_sum(ss, red);
+  const float scale = 1.0f / sqrtf(ss / static_cast<float>(cols) + eps);
+  uint16_t *out = out16 + static_cast<uint64_t>(blockIdx.x) * cols;
+  for (uint32_t c = threadIdx.x; c < cols; c += kBlock) out[c] = enc16<DT>(row[c] * scale * dec16<DT>(gamma[c]));
+}
+
+template <uint32_t DT, int EPI>
+hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
+  constexpr int NR = EPI == kGemmSwiglu ? 2 : 1;
+  constexpr size_t lds = gemm_lds_bytes<NR>();
+  if (lds > 64 * 1024) {
+    // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
+    static std::once_flag once;
+    static hipError_t raised = hipSuccess;
+    std::call_once(once, [] {
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    });
+    if (raised != hipSuccess) return raised;
+  }
+  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI>), dim3(p.rows / 16), dim3(kGThreads), lds, stream, p);
+  return hipGetLastError();
+}
+
+template <uint32_t DT>
+hipError_t launch_dt(int epilogue, const GemmRowsParams &p, hipStream_t stream) {
+  switch (epilogue) {
+    case kGemmF32: return launch_one<DT, kGemmF32>(p, stream);
+    case kGemmResidual: return launch_one<DT, kGemmResidual>(p, stream);
+    case kGemmSwiglu: return launch_one<DT, kGemmSwiglu>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+}  // namespace
+
+bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens) {
+  return rows != 0 && rows % 16 == 0 && cols != 0 && cols % (kGW * kKB) == 0 && tokens >= 1 &&
+         tokens <= kGemmMaxTokens;
+}
+
+hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream) {
+  if (p.w == nullptr || p.x16 == nullptr || !gemm_rows_supported(p.rows, p.cols, p.tokens)) return hipErrorInvalidValue;
+  if (!aligned16(p.w) || !aligned16(p.x16)) return hipErrorInvalidValue;
+  if ((epilogue == kGemmF32 || epilogue == kGemmResidual) && p.out_f32 == nullptr) return hipErrorInvalidValue;
+  if (epilogue == kGemmResidual && p.residual == nullptr) return hipErrorInvalidValue;
+  if (epilogue == kGemmSwiglu && p.out16 == nullptr) return hipErrorInvalidValue;
+  if (dtype == kBF16) return launch_dt<kBF16>(epilogue, p, stream);
+  if (dtype == kF16) return launch_dt<kF16>(epilogue, p, stream);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
+                               uint32_t cols, uint16_t *out16, hipStream_t stream) {
+  if (x == nullptr || gamma == nullptr || out16 == nullptr || tokens == 0 || cols == 0) return hipErrorInvalidValue;
+  if (dtype == kBF16)
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<kBF16>, dim3(tokens), dim3(kBlock), 0, stream, x, gamma, eps, cols, out16);
+  else if (dtype == kF16)
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<kF16>, dim3(tokens), dim3(kBlock), 0, stream, x, gamma, eps, cols, out16);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace nv

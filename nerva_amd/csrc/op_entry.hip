@@ -13,6 +13,7 @@
 #include "attn_decode.cuh"
 #include "sampler.cuh"
 #include "fp8_gemv.cuh"
+#include "gemm_rows.cuh"
 #include "gemv_stream.cuh"
 #include "nerva_hip_layout_check.hpp"
 #include "runtime_state.hpp"
@@ -441,6 +442,29 @@ int nerva_hip_argmax(const NervaHipArgmaxRequest *r, void *stream, int32_t *hip_
   sample_bind_workspace(s, r->workspace);
   s.token_out = r->token;
   return finish(launch_argmax(r->logits, r->count, s, resolve_stream(stream)), hip_error);
+}
+
+int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *r, void *stream, int32_t *hip_error) {
+  if (hip_error) *hip_error = 0;
+  if (r == nullptr || r->epilogue > 2) return finish(hipErrorInvalidValue, hip_error);
+  GemmRowsParams p{};
+  p.w = r->weights;
+  p.x16 = r->input16;
+  p.bias = r->bias;
+  p.residual = r->residual;
+  p.out_f32 = r->output_f32;
+  p.out16 = r->output16;
+  p.rows = r->rows;
+  p.cols = r->cols;
+  p.tokens = r->tokens;
+  p.round_out = r->round_output;
+  return finish(launch_gemm_rows(r->dtype, static_cast<int>(r->epilogue), p, resolve_stream(stream)), hip_error);
+}
+
+int nerva_hip_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
+                           uint32_t cols, uint16_t *out16, void *stream, int32_t *hip_error) {
+  if (hip_error) *hip_error = 0;
+  return finish(launch_rmsnorm_rows(dtype, x, gamma, eps, tokens, cols, out16, resolve_stream(stream)), hip_error);
 }
 
 __global__ void store_sampler_config_kernel(SamplerDev *dst, SamplerDev value) {

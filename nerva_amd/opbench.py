@@ -6,6 +6,7 @@
   3. paged GQA decode attention, 32 q / 8 kv heads x 128, 4096 cached tokens + the new one
   4. FP8 (e4m3, 128x128 block scales) MoE: 8 routed + 1 shared expert, hidden 7168, MLP 2048
   5. the token sampler over 151936 logits (greedy, temperature over the whole vocabulary, top-k / top-p)
+  6. multi-row projection (1, 8, 32 token rows through one weight stream) for the step's matrices
 
 Each case is timed twice: "rotating" cycles through enough distinct copies of the weights / cache that
 the working set exceeds 1 GB (nothing is served from cache), "resident" repeats one copy. The launches
@@ -149,6 +150,24 @@ def case_moe():
         report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
 
 
+def case_gemm_rows():
+    """Token blocks through the step's weight matrices on the matrix cores: the weights are streamed once
+    per block, so 32 tokens should cost about what one token costs."""
+    shapes = (("qkv 6144x4096", 6144, 4096, 0), ("gate_up 2x12288x4096 +SwiGLU", 12288, 4096, 2), ("down 4096x12288", 4096, 12288, 0))
+    for name, rows, cols, epi in shapes:
+        wrows = rows * (2 if epi == 2 else 1)
+        copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
+        w = synth16(copies * wrows * cols, 61)
+        for tokens in (1, 8, 32):
+            x = synth16(tokens * cols, 62, std=1.0)
+            y32 = DeviceBuffer(tokens * rows * 4)
+            y16 = DeviceBuffer(tokens * rows * 2)
+            nbytes = wrows * cols * 2 + tokens * cols * 2 + tokens * rows * (2 if epi == 2 else 4)
+            ns = timed(lambda i: R.gemm_rows(BF16, w.at((i % copies) * wrows * cols * 2), rows, cols, tokens, x, epilogue=epi,
+                                             out_f32=y32, out16=y16, sync=False), 2 * copies)
+            report("6 %s" % name, "T=%d" % tokens, ns, nbytes)
+
+
 def case_sampler():
     V = 151936
     lib = abi.load()
@@ -182,6 +201,7 @@ def main():
     case_attention()
     case_moe()
     case_sampler()
+    case_gemm_rows()
 
 
 if __name__ == "__main__":

@@ -236,6 +236,20 @@ def argmax(logits_buf, count, workspace=None):
     return int(tok.numpy(np.uint32, 1)[0])
 
 
+def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None, residual=None, out_f32=None,
+              out16=None, round_output=False, sync=True):
+    """Y[t] = W . X[t] for up to 32 token rows on the matrix cores (weights streamed once)."""
+    lib = abi.load()
+    req = abi.NervaHipGemmRowsRequest()
+    req.dtype, req.rows, req.cols, req.tokens, req.epilogue, req.round_output = dtype, rows, cols, tokens, epilogue, int(round_output)
+    req.weights, req.input16, req.bias, req.residual = _ptr(weights), _ptr(input16), _ptr(bias), _ptr(residual)
+    req.output_f32, req.output16 = _ptr(out_f32), _ptr(out16)
+    err = C.c_int32(0)
+    _check(lib.nerva_hip_gemm_rows(C.byref(req), None, C.byref(err)), err, "nerva_hip_gemm_rows")
+    if sync:
+        Device.synchronize()
+
+
 def sample(logits_buf, vocab, temperature, top_p, top_k, seed, position, workspace=None):
     """One token from device logits by the session's sampler rule (greedy / Gumbel-max / top-k + top-p)."""
     lib = abi.load()

@@ -120,6 +120,66 @@ def test_gemv_rmsnorm_prologue(dtype, cols, rows):
     assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
 
 
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 1), (48, 2048, 5), (32, 4096, 16), (16, 2048, 17),
+                                               (6144, 4096, 32), (4096, 12288, 31)])
+def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
+    """Multi-row projection on the matrix cores: every token row equals the oracle's GEMV of that row
+    (plain, and with bias + residual + 16-bit rounding as the prompt staging of the down projection uses)."""
+    if dtype == F16 and rows > 1000:
+        pytest.skip("full-size shapes once, in bf16")
+    rng = np.random.default_rng(rows + cols + tokens)
+    if rows * cols > 1 << 22:
+        w = O.synth_16(dtype, SEED, 300 + tokens, rows * cols, 0.0, 0.02).reshape(rows, cols)
+    else:
+        w = O.encode16(dtype, rng.normal(0, 0.02, (rows, cols)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, cols)))
+    bias = O.encode16(dtype, rng.normal(0, 0.1, rows))
+    res = rng.normal(0, 1, (tokens, rows)).astype(np.float32)
+    ref = np.stack([O.gemv_x16(dtype, w, x[t]) for t in range(tokens)])
+    dw, dx = dev(w), dev(x)
+    y = N.DeviceBuffer(tokens * rows * 4)
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dx, epilogue=0, out_f32=y)
+    got = y.numpy(np.float32).reshape(tokens, rows)
+    assert rel_l2(got, ref) <= REL_L2
+    assert max(rel_l2(got[t], ref[t]) for t in range(tokens)) <= REL_L2
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dx, epilogue=1, bias=dev(bias), residual=dev(res), out_f32=y,
+                round_output=True)
+    got = y.numpy(np.float32).reshape(tokens, rows)
+    want = O.decode16(dtype, O.encode16(dtype, (ref + O.decode16(dtype, bias)[None, :]) + res))
+    assert rel_l2(got, want) <= 4e-3                       # one 16-bit rounding of the sum
+    assert np.array_equal(O.encode16(dtype, got), O.encode16(dtype, got.astype(np.float32)))  # values are 16-bit numbers
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 3), (12288, 4096, 32)])
+def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
+    """Fused gate/up projection of a token block: out16 = round16(silu(gate) * up), gate rows first."""
+    if dtype == F16 and inter > 1000:
+        pytest.skip("full-size shape once, in bf16")
+    rng = np.random.default_rng(inter + tokens)
+    if inter > 1000:
+        w = O.synth_16(dtype, SEED, 310, 2 * inter * hidden, 0.0, 0.02).reshape(2 * inter, hidden)
+    else:
+        w = O.encode16(dtype, rng.normal(0, 0.05, (2 * inter, hidden)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, hidden)))
+    out = N.DeviceBuffer(tokens * inter * 2)
+    N.gemm_rows(dtype, dev(w), inter, hidden, tokens, dev(x), epilogue=2, out16=out)
+    got = O.decode16(dtype, out.numpy(np.uint16, tokens * inter)).reshape(tokens, inter)
+    for t in range(0, tokens, max(1, tokens // 4)):
+        gu = O.gemv_x16(dtype, w, x[t])
+        g, u = gu[:inter].astype(np.float64), gu[inter:].astype(np.float64)
+        want = O.decode16(dtype, O.encode16(dtype, (g / (1.0 + np.exp(-g)) * u).astype(np.float32)))
+        assert rel_l2(got[t], want) <= 4e-3
+
+
+def test_gemm_rows_rejects_unsupported_shapes():
+    w, x, y = N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16)
+    for rows, cols, tokens in ((24, 2048, 4), (16, 1024, 4), (16, 2048, 33), (16, 2048, 0)):
+        with pytest.raises(RuntimeError):
+            N.gemm_rows(BF16, w, rows, cols, tokens, x, out_f32=y)
+
+
 @pytest.mark.parametrize("full", [False, True])
 def test_mlp_block_matches_oracle(full):
     """Config 2: RMSNorm -> fused gate+up GEMV -> SiLU(gate)*up -> down GEMV -> residual add."""
