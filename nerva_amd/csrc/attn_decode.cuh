@@ -54,6 +54,14 @@ struct AttnParams {
   const uint32_t *cursor;      // device position, or null -> `position`
   uint32_t position, max_steps, append;
   uint64_t *trace;             // tuning aid: [32] device timestamps of selected workgroups' stages, or null
+  // A block of `tokens` consecutive positions in one launch (grid z; 0 or 1 = a single token).
+  // Token z works at position + z (the cursor is not used then) with its own q/k/v, output, rotation
+  // table and split workspace: the strides below are added z times.
+  uint32_t tokens;
+  uint32_t qkv_token_stride;   // f32 elements between tokens' q|k|v
+  uint32_t out_token_stride;   // elements between tokens' outputs (out16 and out_f32)
+  uint32_t rope_token_stride;  // f32 elements between tokens' cos|sin tables
+  uint64_t ws_token_stride;    // bytes between tokens' split workspaces (attn_workspace_bytes)
 };
 
 // Split-KV factor. The matrix-core kernel keeps one 8-wave workgroup per CU, so kv_heads x splits
@@ -69,5 +77,12 @@ uint64_t attn_workspace_bytes(uint32_t heads, uint32_t head_dim);
 // Carves part_acc/part_m/part_l/counters out of a workspace of attn_workspace_bytes().
 void attn_bind_workspace(AttnParams &p, void *workspace);
 hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t stream);
+
+// Prompt block: rounds and writes the K and V rows of `tokens` consecutive positions
+// (position .. position + tokens - 1) into the cache - bias, per-head RMSNorm (k_norm) and RoPE
+// as in the decode kernel - so that a following launch_attn_decode with append = 0 and the same
+// token block finds every row of the block in place. head_dim 128 only. Uses qkv, k_norm, k_bias,
+// v_bias, the caches and table, rope_freq / rope_cs and the token strides of `p`.
+hipError_t launch_kv_publish_rows(uint32_t dtype, const AttnParams &p, hipStream_t stream);
 
 }  // namespace nv

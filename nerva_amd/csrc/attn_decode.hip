@@ -24,10 +24,56 @@ namespace {
 
 using namespace attn;
 
-// Stand-alone launch of the matrix-core attention (attn_fast_body): grid (kv_heads, splits).
+// Parameters of token z of a block launch.
+__device__ __forceinline__ void token_view(AttnParams &p, uint32_t z) {
+  p.position += z;
+  p.qkv += static_cast<uint64_t>(z) * p.qkv_token_stride;
+  p.out16 += static_cast<uint64_t>(z) * p.out_token_stride;
+  if (p.out_f32 != nullptr) p.out_f32 += static_cast<uint64_t>(z) * p.out_token_stride;
+  if (p.rope_cs != nullptr) p.rope_cs += static_cast<uint64_t>(z) * p.rope_token_stride;
+  const uint64_t ws = z * p.ws_token_stride;
+  p.part_acc = reinterpret_cast<float *>(reinterpret_cast<char *>(p.part_acc) + ws);
+  p.part_m = reinterpret_cast<float *>(reinterpret_cast<char *>(p.part_m) + ws);
+  p.part_l = reinterpret_cast<float *>(reinterpret_cast<char *>(p.part_l) + ws);
+  p.counters = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(p.counters) + ws);
+}
+
+// K and V rows of a prompt block into the cache: grid (kv head, token), two waves (key, value).
+template <uint32_t DT>
+__global__ __launch_bounds__(2 * kWave) void kv_publish_rows_kernel(AttnParams p) {
+  __shared__ __align__(16) uint16_t row16[2][kHD];
+  const uint32_t kvh = blockIdx.x, z = blockIdx.y;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint32_t pos = p.position + z;
+  const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
+  const float *qkv = p.qkv + static_cast<uint64_t>(z) * p.qkv_token_stride;
+  const float *rope_cs = p.rope_cs != nullptr ? p.rope_cs + static_cast<uint64_t>(z) * p.rope_token_stride : nullptr;
+  const uint32_t off = (wave == 0 ? A : A + KV) + kvh * kHD;
+  const uint16_t *bias = wave == 0 ? p.k_bias : p.v_bias;
+  prep_head128<DT>(qkv[off + lane], qkv[off + lane + 64], bias ? bias + kvh * kHD : nullptr, wave == 0 ? p.k_norm : nullptr,
+                   wave == 0 ? p.rope_freq : nullptr, rope_cs, pos, p.eps, lane, nullptr, row16[wave]);
+  __syncthreads();
+  const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, p.table[pos / kKvBlockTokens], kvh);
+  const uint32_t row = pos % kKvBlockTokens;
+  if (wave == 0) {
+    if (lane < 16)  // K: 16 pieces of 8 consecutive dims
+      *reinterpret_cast<uint4 *>(p.k_cache + tile + kv_k_elem(kHD, row, lane * 8)) =
+          *reinterpret_cast<const uint4 *>(row16[0] + lane * 8);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {  // V: one 16-bit element per dim
+      const uint32_t d = lane + i * kWave;
+      p.v_cache[tile + kv_v_elem(kHD, row, d)] = row16[1][d];
+    }
+  }
+}
+
+// Stand-alone launch of the matrix-core attention (attn_fast_body): grid (kv_heads, splits[, tokens]).
 template <uint32_t DT, int G, int W>
 __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   __shared__ AttnShared<G, W> sh;
+  if (blockIdx.z != 0) token_view(p, blockIdx.z);
   const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);  // before anything they could queue behind
   const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
   if (p.cursor != nullptr && pos >= p.max_steps) return;
@@ -182,7 +228,7 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
   const bool fast = p.head_dim == kHD && (group == 1 || group == 2 || group == 4 || group == 8) &&
                     p.part_acc != nullptr && p.splits >= 1;
   if (fast) {
-    const dim3 grid(p.kv_heads, p.splits);
+    const dim3 grid(p.kv_heads, p.splits, p.tokens > 1 ? p.tokens : 1);
     switch (group) {
       case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
       case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
@@ -215,6 +261,19 @@ void attn_bind_workspace(AttnParams &p, void *workspace) {
   p.counters = reinterpret_cast<uint32_t *>(base + acc + 2 * ml);
 }
 
+hipError_t launch_kv_publish_rows(uint32_t dtype, const AttnParams &p, hipStream_t stream) {
+  if (p.qkv == nullptr || p.k_cache == nullptr || p.v_cache == nullptr || p.table == nullptr || p.tokens == 0 ||
+      p.head_dim != static_cast<uint32_t>(kHD) || p.kv_heads == 0)
+    return hipErrorInvalidValue;
+  if (static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+    return hipErrorInvalidValue;
+  const dim3 grid(p.kv_heads, p.tokens);
+  if (dtype == kBF16) hipLaunchKernelGGL(kv_publish_rows_kernel<kBF16>, grid, dim3(2 * kWave), 0, stream, p);
+  else if (dtype == kF16) hipLaunchKernelGGL(kv_publish_rows_kernel<kF16>, grid, dim3(2 * kWave), 0, stream, p);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
 hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t stream) {
   if (p.qkv == nullptr || p.k_cache == nullptr || p.v_cache == nullptr || p.table == nullptr ||
       p.out16 == nullptr)
@@ -227,6 +286,14 @@ hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t s
   if (p.cursor == nullptr &&
       static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
+  if (p.tokens > 1) {
+    // a block of positions: host-given positions, rows already in the cache, matrix-core kernel only
+    const uint32_t group = p.heads / p.kv_heads;
+    const bool fast = p.head_dim == 128 && (group == 1 || group == 2 || group == 4 || group == 8) && p.part_acc != nullptr;
+    if (p.cursor != nullptr || p.append != 0 || !fast || p.tokens > 65535 ||
+        static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+      return hipErrorInvalidValue;
+  }
   if (dtype == kBF16) return launch_dt<kBF16>(p, stream);
   if (dtype == kF16) return launch_dt<kF16>(p, stream);
   return hipErrorInvalidValue;

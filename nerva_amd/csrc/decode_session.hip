@@ -26,6 +26,7 @@
 #include "argmax.cuh"
 #include "attn_decode.cuh"
 #include "decode_chain.cuh"
+#include "gemm_rows.cuh"
 #include "layer_front.cuh"
 #include "sampler.cuh"
 #include "gemv_stream.cuh"
@@ -114,6 +115,13 @@ struct NervaHipHfDecodeSequenceSession {
   hipGraph_t graph[3] = {nullptr, nullptr, nullptr};
   hipGraphExec_t exec[3] = {nullptr, nullptr, nullptr};
   uint64_t graph_nodes[3] = {0, 0, 0};
+  // prompt blocks: up to kGemmMaxTokens prompt tokens per pass through the layers (weights streamed
+  // once per block on the matrix cores); false = one prompt step per token
+  bool block_prefill = false;
+  float *px = nullptr, *pr = nullptr, *pqkv = nullptr, *prope = nullptr;
+  uint16_t *pxn16 = nullptr, *pattn16 = nullptr, *pff16 = nullptr;
+  char *pattn_ws = nullptr;
+  uint64_t pattn_ws_stride = 0;
   SamplerDev sampler{};            // normalised configuration of the active sequence
   SamplerDev *sampler_dev = nullptr;
   uint64_t *sampler_keys = nullptr;
@@ -158,6 +166,26 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
   const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
   for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < hidden; i += gridDim.x * kBlock)
     x[i] = dec16<DT>(row[i]);
+}
+
+// Prompt block: embedding rows and rotation tables of positions first .. first + gridDim.x - 1.
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock) void embed_rows_kernel(const uint16_t *emb, const uint32_t *prompt, uint32_t first,
+                                                            uint32_t hidden, uint32_t vocab, float *x,
+                                                            const float *rope_freq, float *rope_cs, uint32_t half_dim) {
+  const uint32_t t = blockIdx.x, pos = first + t;
+  if (rope_freq != nullptr) {
+    for (uint32_t i = threadIdx.x; i < half_dim; i += kBlock) {
+      float sn, cs;
+      sincosf(static_cast<float>(pos) / rope_freq[i], &sn, &cs);
+      rope_cs[static_cast<uint64_t>(t) * 2 * half_dim + i] = cs;
+      rope_cs[static_cast<uint64_t>(t) * 2 * half_dim + half_dim + i] = sn;
+    }
+  }
+  uint32_t token = prompt[pos];
+  if (token >= vocab) token = 0;  // prompts are validated on the host
+  const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
+  for (uint32_t i = threadIdx.x; i < hidden; i += kBlock) x[static_cast<uint64_t>(t) * hidden + i] = dec16<DT>(row[i]);
 }
 
 __global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count) {
@@ -603,6 +631,114 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
   return err;
 }
 
+// Prompt tokens 0 .. count-1 through every layer in blocks of up to kGemmMaxTokens tokens, with the
+// prompt staging (16-bit hidden state between layers, prefill_kernels.cu:494-508): per block and
+// layer one RMSNorm launch, the qkv projection as a multi-row GEMM, the K/V rows of the block into the
+// cache, the attention of all its tokens in one launch (token z attends to keys 0 .. first + z), and
+// the o / gate-up / down projections as multi-row GEMMs. Leaves the cursor at `count`. The reference
+// prefills in chunks too (session_decode_prefill.inc.cu:1879-2243).
+hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, NervaHipHfDecodeSequenceResult *out) {
+  hipStream_t st = s->stream;
+  const uint32_t H = s->hidden, A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim, I = s->intermediate;
+  const float *rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
+  hipError_t err = hipSuccess;
+  for (uint32_t first = 0; err == hipSuccess && first < count; first += kGemmMaxTokens) {
+    const uint32_t T = std::min<uint32_t>(kGemmMaxTokens, count - first);
+    if (s->dtype == kBF16)
+      hipLaunchKernelGGL(embed_rows_kernel<kBF16>, dim3(T), dim3(kBlock), 0, st, s->emb, s->prompt, first, H, s->vocab,
+                         s->px, rope_freq, s->prope, s->head_dim / 2);
+    else
+      hipLaunchKernelGGL(embed_rows_kernel<kF16>, dim3(T), dim3(kBlock), 0, st, s->emb, s->prompt, first, H, s->vocab,
+                         s->px, rope_freq, s->prope, s->head_dim / 2);
+    err = hipGetLastError();
+    for (uint32_t l = 0; err == hipSuccess && l < s->layers; ++l) {
+      const LayerDev &w = s->layer[l];
+      err = launch_rmsnorm_rows(s->dtype, s->px, w.rms_attn, s->eps, T, H, s->pxn16, st);
+      GemmRowsParams g{};
+      g.tokens = T;
+      if (err == hipSuccess) {
+        g.w = w.wqkv;
+        g.x16 = s->pxn16;
+        g.out_f32 = s->pqkv;
+        g.rows = A + 2 * KV;
+        g.cols = H;
+        err = launch_gemm_rows(s->dtype, kGemmF32, g, st);
+      }
+      AttnParams a{};
+      a.heads = s->heads;
+      a.kv_heads = s->kv_heads;
+      a.head_dim = s->head_dim;
+      attn_bind_workspace(a, s->pattn_ws);
+      a.qkv = s->pqkv;
+      a.q_norm = w.q_norm;
+      a.k_norm = w.k_norm;
+      a.q_bias = w.q_bias;
+      a.k_bias = w.k_bias;
+      a.v_bias = w.v_bias;
+      a.k_cache = s->kc;
+      a.v_cache = s->vc;
+      a.table = s->table;
+      a.rope_freq = rope_freq;
+      a.rope_cs = rope_freq != nullptr ? s->prope : nullptr;
+      a.out16 = s->pattn16;
+      a.layer = l;
+      a.block_count = s->block_count;
+      a.splits = s->attn_splits;
+      a.eps = s->eps;
+      a.position = first;
+      a.tokens = T;
+      a.qkv_token_stride = A + 2 * KV;
+      a.out_token_stride = A;
+      a.rope_token_stride = s->head_dim;
+      a.ws_token_stride = s->pattn_ws_stride;
+      if (err == hipSuccess) err = launch_kv_publish_rows(s->dtype, a, st);
+      if (err == hipSuccess) err = launch_attn_decode(s->dtype, a, st);
+      if (err == hipSuccess) {
+        g = GemmRowsParams{};
+        g.tokens = T;
+        g.w = w.wo;
+        g.x16 = s->pattn16;
+        g.bias = w.o_bias;
+        g.residual = s->px;
+        g.out_f32 = s->pr;
+        g.rows = H;
+        g.cols = A;
+        err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
+      }
+      if (err == hipSuccess) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st);
+      if (err == hipSuccess) {
+        g = GemmRowsParams{};
+        g.tokens = T;
+        g.w = w.wgu;
+        g.x16 = s->pxn16;
+        g.out16 = s->pff16;
+        g.rows = I;
+        g.cols = H;
+        err = launch_gemm_rows(s->dtype, kGemmSwiglu, g, st);
+      }
+      if (err == hipSuccess) {
+        g = GemmRowsParams{};
+        g.tokens = T;
+        g.w = w.wdown;
+        g.x16 = s->pff16;
+        g.residual = s->pr;
+        g.out_f32 = s->px;
+        g.rows = H;
+        g.cols = I;
+        g.round_out = 1;  // prompt tokens carry a 16-bit hidden state between layers
+        err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
+      }
+    }
+    if (err == hipSuccess) out->kernel_launches += 1 + 9ull * s->layers;
+  }
+  if (err == hipSuccess) {
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, st, s->state, count, prompt_count);
+    err = hipGetLastError();
+    out->kernel_launches += 1;
+  }
+  return err;
+}
+
 int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool synthetic, uint64_t seed,
                 float weight_std, uint32_t with_qk_norm, NervaHipHfDecodeSequenceSessionCreateResult *out,
                 Session **session_out) {
@@ -741,6 +877,16 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_rope_cs = c.take(HD * 4);
   const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
+  const uint64_t pT = kGemmMaxTokens;
+  const uint64_t off_px = c.take(pT * H * 4);
+  const uint64_t off_pr = c.take(pT * H * 4);
+  const uint64_t off_pqkv = c.take(pT * (A + 2 * KV) * 4);
+  const uint64_t off_pxn16 = c.take(pT * H * 2);
+  const uint64_t off_pattn16 = c.take(pT * A * 2);
+  const uint64_t off_pff16 = c.take(pT * I * 2);
+  const uint64_t off_prope = c.take(pT * HD * 4);
+  const uint64_t pattn_ws_stride = (attn_workspace_bytes(rq->heads, rq->head_dim) + 255u) & ~uint64_t{255};
+  const uint64_t off_pattn_ws = c.take(pT * pattn_ws_stride);
   const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
   const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(rq->vocab_size));
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
@@ -792,6 +938,27 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
   s->sample_ws = s->arena + off_sample_ws;
+  s->px = reinterpret_cast<float *>(s->arena + off_px);
+  s->pr = reinterpret_cast<float *>(s->arena + off_pr);
+  s->pqkv = reinterpret_cast<float *>(s->arena + off_pqkv);
+  s->pxn16 = dev16(off_pxn16);
+  s->pattn16 = dev16(off_pattn16);
+  s->pff16 = dev16(off_pff16);
+  s->prope = reinterpret_cast<float *>(s->arena + off_prope);
+  s->pattn_ws = s->arena + off_pattn_ws;
+  s->pattn_ws_stride = pattn_ws_stride;
+  {
+    // Prompt blocks need the matrix-core attention (head_dim 128, GQA factor 1/2/4/8) and shapes the
+    // multi-row GEMM takes; NERVA_HIP_PREFILL=walk keeps one prompt step per token.
+    const char *mode = getenv("NERVA_HIP_PREFILL");
+    const uint32_t group = rq->heads / rq->kv_heads;
+    s->block_prefill = !(mode != nullptr && mode[0] == 'w') && rq->head_dim == 128 &&
+                       (group == 1 || group == 2 || group == 4 || group == 8) &&
+                       gemm_rows_supported(static_cast<uint32_t>(A + 2 * KV), rq->hidden, 1) &&
+                       gemm_rows_supported(rq->hidden, static_cast<uint32_t>(A), 1) &&
+                       gemm_rows_supported(rq->intermediate, rq->hidden, 1) &&
+                       gemm_rows_supported(rq->hidden, rq->intermediate, 1);
+  }
   s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
   s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
   s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
@@ -915,6 +1082,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_ws, 0, front_ws_bytes, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
   if (err == hipSuccess && rq->layer_count > 0)
     err = hipMemsetAsync(s->arena + off_chain_trace, 0, static_cast<uint64_t>(rq->layer_count) * 32 * 8, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
@@ -1018,11 +1186,14 @@ int nerva_hip_hf_decode_sequence_session_start(const NervaHipHfDecodeSequenceSes
   s->started = false;
   hipError_t err = set_sampler(s, request->sampler);   // session_api_lifecycle.inc.cu:1026
   if (err == hipSuccess) err = reset_sequence(s, request->prompt_tokens, P, out);
-  // prefill: P-1 prompt steps (graph replay) + one prompt step with the LM head and sampler
-  if (err == hipSuccess && P > 1) err = ensure_graph(s, 1, out);
+  // prefill: the first P-1 prompt tokens (in blocks on the matrix cores where the shapes allow,
+  // else one captured prompt step per token), then one prompt step with the LM head and sampler
+  if (err == hipSuccess && P > 1 && !s->block_prefill) err = ensure_graph(s, 1, out);
   if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
-  for (uint32_t i = 0; err == hipSuccess && i + 1 < P; ++i) {
-    err = launch_step(s, 1, out);
+  if (s->block_prefill) {
+    if (err == hipSuccess && P > 1) err = prefill_blocks(s, P - 1, P, out);
+  } else {
+    for (uint32_t i = 0; err == hipSuccess && i + 1 < P; ++i) err = launch_step(s, 1, out);
   }
   if (err == hipSuccess) err = enqueue_step(s, kPromptHeadStep, nullptr);
   if (err == hipSuccess) out->kernel_launches += step_launches(s, 0);

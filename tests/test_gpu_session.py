@@ -540,3 +540,42 @@ def test_session_temperature_sampling_follows_the_rule(temperature, top_p, top_k
     rc, res, greedy = s.advance(4)
     assert rc == 0 and res.graph_nodes == 3 + 5 * 2
     s.destroy()
+
+
+@pytest.mark.parametrize("geom", [GEOMETRIES[5], GEOMETRIES[6]])
+def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
+    """start() sends the prompt through the layers in blocks of up to 32 tokens (multi-row GEMMs, one
+    attention launch per block); NERVA_HIP_PREFILL=walk keeps one prompt step per token. Same staging,
+    so both agree with each other and with the oracle to the end-to-end tolerance, over three blocks."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
+    weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 1234, theta, qk_norm, bias)
+    prompt = np.random.default_rng(8).integers(0, vocab, 70).astype(np.uint32)
+    ctx = O.Context(omodel, 96, staging=1)
+    for i, tok in enumerate(prompt):
+        ctx.forward_token(int(tok), prompt_token=True, want_logits=(i == len(prompt) - 1))
+    ref_logits = ctx.logits()
+    results = {}
+    for mode in ("blocks", "walk"):
+        if mode == "walk":
+            monkeypatch.setenv("NERVA_HIP_PREFILL", "walk")
+        else:
+            monkeypatch.delenv("NERVA_HIP_PREFILL", raising=False)
+        s = N.DecodeSession.create(weights, 96)
+        rc, res = s.start(prompt)
+        assert rc == 0 and res.hot_path_allocations == 0
+        logits = s.logits()
+        assert rel_l2(logits, ref_logits) <= E2E_REL_L2
+        for layer in range(layers):
+            for token in (0, 15, 31, 32, 47, 68, 69):     # block edges included
+                gk, gv = s.kv_row(layer, token)
+                rk, rv = ctx.read_kv16(layer, token)
+                tol = 2e-3 if layer == 0 else E2E_REL_L2
+                assert rel_l2(O.decode16(dtype, gk), O.decode16(dtype, rk)) <= tol, (mode, layer, token)
+                assert rel_l2(O.decode16(dtype, gv), O.decode16(dtype, rv)) <= tol, (mode, layer, token)
+        rc, res, tokens = s.advance(6)
+        assert rc == 0
+        results[mode] = (logits, tokens.tolist(), res.kernel_launches)
+        s.destroy()
+    assert rel_l2(results["blocks"][0], results["walk"][0]) <= E2E_REL_L2
+    assert results["blocks"][1][0] == results["walk"][1][0] or \
+        np.sort(ref_logits)[-1] - np.sort(ref_logits)[-2] < E2E_REL_L2 * np.max(np.abs(ref_logits))
