@@ -163,7 +163,8 @@ def main():
     assert rc == 0, "start failed: hip_error=%d" % res.hip_error
     rc, res, first = session.advance(1)      # token 0 was sampled by the prefill; this only syncs
     assert rc == 0
-    log("[bench] prefill of %d tokens: %.1f s" % (args.prompt, time.time() - t0))
+    prefill_s = time.time() - t0
+    log("[bench] prefill of %d tokens: %.2f s (%.0f prompt tok/s)" % (args.prompt, prefill_s, args.prompt / prefill_s))
     if args.warmup:
         rc, res, _ = session.advance(args.warmup)
         assert rc == 0
@@ -261,7 +262,7 @@ def main():
                                      "32q/8kv x128, MLP 12288, vocab 151936, random-init bf16 N(0,0.02), batch 1, "
                                      "prompt %d prefilled, %d greedy tokens under hipGraph replay"
                                      % (cfg["layers"], args.prompt, args.steps),
-                            prompt_tokens=args.prompt, context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
+                            prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
                             per_token_latency_ms=latency, gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)

@@ -80,6 +80,15 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   attn_fast_body<DT, G, W, false>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
 }
 
+// Prompt-block launch of the same body (grid z = tokens): the lean variant, two workgroups per CU.
+template <uint32_t DT, int G, int W>
+__global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams p) {
+  __shared__ AttnShared<G, W> sh;
+  if (blockIdx.z != 0) token_view(p, blockIdx.z);
+  const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);
+  attn_fast_body<DT, G, W, false, 1>(p, p.position, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
+}
+
 // Any head_dim (even when RoPE is on) / any group size: one workgroup per query
 // head, waves stride over tokens, lanes over dims. Used for shapes the fast path
 // does not cover (the tiny known-answer models).
@@ -229,6 +238,15 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
                     p.part_acc != nullptr && p.splits >= 1;
   if (fast) {
     const dim3 grid(p.kv_heads, p.splits, p.tokens > 1 ? p.tokens : 1);
+    if (p.tokens > 1) {
+      switch (group) {
+        case 1: hipLaunchKernelGGL((attn_block_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL((attn_block_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+        case 4: hipLaunchKernelGGL((attn_block_kernel<DT, 4, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+        default: hipLaunchKernelGGL((attn_block_kernel<DT, 8, kAttnWaves / 2>), grid, dim3(kAttnWaves / 2 * kWave), 0, stream, p); break;
+      }
+      return hipGetLastError();
+    }
     switch (group) {
       case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
       case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;

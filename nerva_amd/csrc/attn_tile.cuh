@@ -427,7 +427,7 @@ __device__ __forceinline__ RawHeads<G, W> attn_request_raw(const AttnParams &p, 
 // consumer (AttnLink). Its first tile is requested before it polls for q/k/v; partials and the
 // final output leave as tagged words; split 0 of a kv head merges (it polls the other splits'
 // partials instead of taking a ticket), so nobody waits for stores to be performed.
-template <uint32_t DT, int G, int W, bool LINKED>
+template <uint32_t DT, int G, int W, bool LINKED, int IN_FLIGHT = (LINKED ? 1 : 4)>
 __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32_t pos, const uint32_t kvh,
                                                const uint32_t split, const uint32_t S, AttnShared<G, W> &sh,
                                                const AttnLink &link, const RawHeads<G, W> &raw) {
@@ -461,10 +461,12 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
 
   // ---- first tile of every wave: issue its loads before anything else
   // Up to four tiles in flight per wave (one 8-wave workgroup per CU leaves 256 registers a lane;
-  // at the default split factor a wave's whole share of an 8k context is requested at once). A
-  // linked workgroup keeps one, to fit the register budget that lets two 8-wave workgroups share
-  // a CU, and its launch uses more splits instead.
-  constexpr int kInFlight = LINKED ? 1 : 4;
+  // at the default split factor a wave's whole share of an 8k context is requested at once). The
+  // lean variant keeps one, to fit the 128 registers that let two 8-wave workgroups share a CU:
+  // linked workgroups (their launch uses more splits instead) and prompt blocks, whose launches
+  // hold thousands of workgroups and are bound by how many of them a CU can run at a time.
+  constexpr int kInFlight = IN_FLIGHT;
+  constexpr bool kLean = IN_FLIGHT == 1;  // 128-register budget: the query operand is parked in LDS
   uint4 kreg[kInFlight][4], vreg[kInFlight][4];
   uint32_t b = b0 + wave;
   // the block-table entries first, all of them, so that no tile request waits behind another tile's data
@@ -564,10 +566,10 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     }
     qx[j] = make_uint4(w[0], w[1], w[2], w[3]);
   }
-  // A linked workgroup runs under a tighter register budget: it parks the operand in LDS (every
-  // wave writes the same values, and reads them back after its own writes).
+  // Under the tighter register budget the operand is parked in LDS (every wave writes the same
+  // values, and reads them back after its own writes).
   const uint4 *qx_lds = nullptr;
-  if constexpr (LINKED) {
+  if constexpr (kLean) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) sh.qx_s[j][lane] = qx[j];
     qx_lds = &sh.qx_s[0][lane];
@@ -584,7 +586,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     for (int f = 0; f < kInFlight; ++f) {
       const uint32_t bb = b + f * W;
       if (bb < b1) {
-        attn_tile<DT, G, LINKED>(kreg[f], vreg[f], qx, qx_lds, bb, n_keys, col, grp, owns_new && bb == new_block, new_row,
+        attn_tile<DT, G, kLean>(kreg[f], vreg[f], qx, qx_lds, bb, n_keys, col, grp, owns_new && bb == new_block, new_row,
                                  knew, vnew, m, l, acc);
         if (bb + kInFlight * W < b1) attn_load_tile(p, p.table[bb + kInFlight * W], kvh, lane, kreg[f], vreg[f]);
       }

@@ -139,17 +139,46 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   }
 }
 
+// One workgroup of 1024 lanes per token row; a lane keeps its values in registers between the sum of
+// squares and the scaling (cols <= 16384), so the row is read once.
+constexpr int kNormThreads = 1024;
+constexpr int kNormPerLane = 4;  // float4 pieces per lane
 template <uint32_t DT>
-__global__ __launch_bounds__(kBlock) void rmsnorm_rows_kernel(const float *x, const uint16_t *gamma, float eps,
-                                                              uint32_t cols, uint16_t *out16) {
-  __shared__ float red[kWavesPerBlock];
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const float *x, const uint16_t *gamma, float eps,
+                                                                    uint32_t cols, uint16_t *out16) {
+  __shared__ float red[kNormThreads / kWave];
   const float *row = x + static_cast<uint64_t>(blockIdx.x) * cols;
+  float4 v[kNormPerLane];
   float ss = 0.0f;
-  for (uint32_t c = threadIdx.x; c < cols; c += kBlock) ss += row[c] * row[c];
-  ss = block_sum(ss, red);
-  const float scale = 1.0f / sqrtf(ss / static_cast<float>(cols) + eps);
+#pragma unroll
+  for (int i = 0; i < kNormPerLane; ++i) {
+    const uint32_t c = (i * kNormThreads + threadIdx.x) * 4;
+    v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (c < cols) v[i] = *reinterpret_cast<const float4 *>(row + c);
+    ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kNormThreads / kWave; ++w) total += red[w];
+  const float scale = 1.0f / sqrtf(total / static_cast<float>(cols) + eps);
   uint16_t *out = out16 + static_cast<uint64_t>(blockIdx.x) * cols;
-  for (uint32_t c = threadIdx.x; c < cols; c += kBlock) out[c] = enc16<DT>(row[c] * scale * dec16<DT>(gamma[c]));
+#pragma unroll
+  for (int i = 0; i < kNormPerLane; ++i) {
+    const uint32_t c = (i * kNormThreads + threadIdx.x) * 4;
+    if (c < cols) {
+      const uint2 g = *reinterpret_cast<const uint2 *>(gamma + c);
+      float g0, g1, g2, g3;
+      unpack2<DT>(g.x, g0, g1);
+      unpack2<DT>(g.y, g2, g3);
+      uint2 o;
+      o.x = enc16<DT>(v[i].x * scale * g0) | (static_cast<uint32_t>(enc16<DT>(v[i].y * scale * g1)) << 16);
+      o.y = enc16<DT>(v[i].z * scale * g2) | (static_cast<uint32_t>(enc16<DT>(v[i].w * scale * g3)) << 16);
+      *reinterpret_cast<uint2 *>(out + c) = o;
+    }
+  }
 }
 
 template <uint32_t DT, int EPI>
@@ -202,11 +231,14 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
 
 hipError_t launch_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
                                uint32_t cols, uint16_t *out16, hipStream_t stream) {
-  if (x == nullptr || gamma == nullptr || out16 == nullptr || tokens == 0 || cols == 0) return hipErrorInvalidValue;
+  if (x == nullptr || gamma == nullptr || out16 == nullptr || tokens == 0 || cols == 0 || cols % 4 != 0 ||
+      cols > static_cast<uint32_t>(kNormThreads * kNormPerLane * 4) || !aligned16(x) || (reinterpret_cast<uintptr_t>(gamma) & 7u) != 0 ||
+      (reinterpret_cast<uintptr_t>(out16) & 7u) != 0)
+    return hipErrorInvalidValue;
   if (dtype == kBF16)
-    hipLaunchKernelGGL(rmsnorm_rows_kernel<kBF16>, dim3(tokens), dim3(kBlock), 0, stream, x, gamma, eps, cols, out16);
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<kBF16>, dim3(tokens), dim3(kNormThreads), 0, stream, x, gamma, eps, cols, out16);
   else if (dtype == kF16)
-    hipLaunchKernelGGL(rmsnorm_rows_kernel<kF16>, dim3(tokens), dim3(kBlock), 0, stream, x, gamma, eps, cols, out16);
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<kF16>, dim3(tokens), dim3(kNormThreads), 0, stream, x, gamma, eps, cols, out16);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
