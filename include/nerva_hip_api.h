@@ -229,6 +229,48 @@ typedef struct NervaHipHfDecodeSequenceSessionAdvanceRequest {
   uint32_t output_token_capacity;
 } NervaHipHfDecodeSequenceSessionAdvanceRequest;
 
+/* mirrors NervaCudaHfDecodeSequenceSessionForkSharedWeightsRequest (nerva_cuda_api.h:689-692) */
+typedef struct NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest {
+  NervaHipHfDecodeSequenceSession *parent;
+  uint32_t detailed_profile;
+} NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest;
+
+/* reasons of a batch step (session_prelude.inc.cu:56-64) */
+#define NERVA_HIP_BATCH_READY 0u
+#define NERVA_HIP_BATCH_INVALID_REQUEST 1u
+#define NERVA_HIP_BATCH_NO_SESSIONS 2u
+#define NERVA_HIP_BATCH_NO_READY_SESSIONS 3u
+#define NERVA_HIP_BATCH_SHARED_WEIGHTS_UNPROVEN 4u
+#define NERVA_HIP_BATCH_INSUFFICIENT_COMPATIBLE_READY 5u
+#define NERVA_HIP_BATCH_MAX_BLOCK_TOKENS 32u /* types.cuh:63 */
+
+/* mirrors NervaCudaHfDecodeSequenceBatchAdvanceRequest (nerva_cuda_api.h:936-943) */
+typedef struct NervaHipHfDecodeSequenceBatchAdvanceRequest {
+  NervaHipHfDecodeSequenceSession **sessions;
+  uint32_t session_count, target_block_tokens, min_block_tokens;
+  uint32_t *output_tokens; /* [session_count], written at the index of each session that advanced */
+  uint32_t output_token_capacity;
+} NervaHipHfDecodeSequenceBatchAdvanceRequest;
+
+/* mirrors NervaCudaHfDecodeSequenceBatchAdvanceResult (nerva_cuda_api.h:945-976). The launch
+ * counters count this library's launches: pack = embedding and RMSNorm rows, projection = the
+ * multi-row GEMMs (or GEMVs), scatter = K/V rows into the caches, dependency = attention,
+ * sampling = sampler launches. *_elapsed_ns stay 0 except projection_elapsed_ns, which is the
+ * device time of the whole batch step (the projections are not timed apart from the rest).
+ * `shared_weight_stream` is 1 when one stream of the weights served every sequence of the step, 0
+ * when the model's shapes are outside the multi-row kernels and each sequence ran its own step. */
+typedef struct NervaHipHfDecodeSequenceBatchAdvanceResult {
+  int32_t status, hip_error, device_count;
+  uint32_t reason, exact, requested_session_count, eligible_session_count, block_tokens,
+      target_block_tokens, min_block_tokens, dtype, layer_count, observed_tokens, last_token;
+  uint64_t observed_token_hash, d2h_bytes, projection_elapsed_ns, qkv_elapsed_ns,
+      attention_output_elapsed_ns, gate_up_elapsed_ns, down_elapsed_ns, lm_head_elapsed_ns,
+      pack_kernel_launches, projection_kernel_launches, scatter_kernel_launches,
+      dependency_kernel_launches, experimental_rt_selector_launches, sampling_kernel_launches,
+      sync_calls, hot_path_allocations;
+  uint32_t shared_weight_stream;
+} NervaHipHfDecodeSequenceBatchAdvanceResult;
+
 /* mirrors NervaCudaDeepSeekQuantDequantResult (nerva_cuda_api.h:1338-1354) */
 typedef struct NervaHipDeepSeekQuantDequantResult {
   int32_t status, hip_error, device_count;
@@ -344,6 +386,26 @@ int nerva_hip_hf_decode_sequence_session_advance(
 /* replaces nerva_cuda_hf_decode_sequence_session_destroy (nerva_cuda_api.h:2216-2218) */
 int nerva_hip_hf_decode_sequence_session_destroy(NervaHipHfDecodeSequenceSession *session,
                                                  NervaHipHfDecodeSequenceSessionCreateResult *out);
+
+/* replaces nerva_cuda_hf_decode_sequence_session_fork_shared_weights (nerva_cuda_api.h:2212-2215):
+ * a second session on the parent's resident weights with a KV cache, token slots and cursor of its
+ * own. If the parent has a sequence under way (started, not finished), the child starts as a copy
+ * of it - prompt, slots, cursor, cache, sampler - and both go on independently. The weights are
+ * freed when the last session holding them is destroyed, in any order. */
+int nerva_hip_hf_decode_sequence_session_fork_shared_weights(
+    const NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest *request,
+    NervaHipHfDecodeSequenceSessionCreateResult *out, NervaHipHfDecodeSequenceSession **session);
+
+/* replaces nerva_cuda_hf_decode_sequence_batch_advance_one (nerva_cuda_api.h:2209-2211): one more
+ * token for each of up to 32 ready sessions of the same model through ONE stream of the weights.
+ * Ready = started, not finished, every token computed so far already handed out by advance
+ * (prompt + observed == cursor + 1). Sessions count as the same model when their weight
+ * descriptor hashes are non-zero and equal and their dimensions agree; the largest such group is
+ * taken in request order (status 0 with a reason other than READY means nothing ran). Each
+ * session samples with its own sampler and position. */
+int nerva_hip_hf_decode_sequence_batch_advance_one(
+    const NervaHipHfDecodeSequenceBatchAdvanceRequest *request,
+    NervaHipHfDecodeSequenceBatchAdvanceResult *out);
 
 /* replaces nerva_cuda_deepseek_quant_fp8_f32_scale_encoded_matvec (nerva_cuda_api.h:2245-2247) */
 int nerva_hip_deepseek_quant_fp8_f32_scale_encoded_matvec(
@@ -473,7 +535,8 @@ typedef struct NervaHipGemmRowsRequest {
 /* Projection of a block of up to 32 token rows through one weight matrix on the matrix cores,
  * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
  * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
- * prefill and projection batch (projection.cu:99-106, 297-300). rows % 16 == 0, cols % 2048 == 0. */
+ * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must
+ * not alias the output), cols % 2048 == 0. */
 int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *request, void *stream, int32_t *hip_error);
 /* out16[t] = round16(rmsnorm(x[t]) * gamma) for `tokens` rows of `cols` f32 values
  * (rms_norm_encoded_into, ops.rs:31-50, once per row). */

@@ -36,6 +36,13 @@ __host__ __device__ __forceinline__ uint32_t kv_v_elem(uint32_t head_dim, uint32
   return (slab / 2) * 512 + ((row / 4) * 16 + n) * 8 + (slab % 2) * 4 + row % 4;
 }
 
+// One sequence of a batch launch: the cache a token row belongs to and its position there.
+struct AttnSeq {
+  uint16_t *k_cache, *v_cache;
+  const uint32_t *table;
+  uint32_t block_count, position;
+};
+
 struct AttnParams {
   const float *qkv;            // [heads*hd | kv_heads*hd | kv_heads*hd] raw f32 projections
   const uint16_t *q_norm, *k_norm;           // optional [hd]
@@ -62,6 +69,10 @@ struct AttnParams {
   uint32_t out_token_stride;   // elements between tokens' outputs (out16 and out_f32)
   uint32_t rope_token_stride;  // f32 elements between tokens' cos|sin tables
   uint64_t ws_token_stride;    // bytes between tokens' split workspaces (attn_workspace_bytes)
+  // A batch of sequences instead of consecutive positions of one: token z belongs to seqs[z] (device
+  // memory, `tokens` entries), which replaces k_cache, v_cache, table, block_count and the position.
+  // Applies to z = 0 as well, and to a block of one token.
+  const AttnSeq *seqs;
 };
 
 // Split-KV factor. The matrix-core kernel keeps one 8-wave workgroup per CU, so kv_heads x splits

@@ -26,7 +26,16 @@ using namespace attn;
 
 // Parameters of token z of a block launch.
 __device__ __forceinline__ void token_view(AttnParams &p, uint32_t z) {
-  p.position += z;
+  if (p.seqs != nullptr) {
+    const AttnSeq seq = p.seqs[z];
+    p.k_cache = seq.k_cache;
+    p.v_cache = seq.v_cache;
+    p.table = seq.table;
+    p.block_count = seq.block_count;
+    p.position = seq.position;
+  } else {
+    p.position += z;
+  }
   p.qkv += static_cast<uint64_t>(z) * p.qkv_token_stride;
   p.out16 += static_cast<uint64_t>(z) * p.out_token_stride;
   if (p.out_f32 != nullptr) p.out_f32 += static_cast<uint64_t>(z) * p.out_token_stride;
@@ -45,7 +54,15 @@ __global__ __launch_bounds__(2 * kWave) void kv_publish_rows_kernel(AttnParams p
   const uint32_t kvh = blockIdx.x, z = blockIdx.y;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  const uint32_t pos = p.position + z;
+  uint32_t pos = p.position + z;
+  if (p.seqs != nullptr) {
+    const AttnSeq seq = p.seqs[z];
+    p.k_cache = seq.k_cache;
+    p.v_cache = seq.v_cache;
+    p.table = seq.table;
+    p.block_count = seq.block_count;
+    pos = seq.position;
+  }
   const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
   const float *qkv = p.qkv + static_cast<uint64_t>(z) * p.qkv_token_stride;
   const float *rope_cs = p.rope_cs != nullptr ? p.rope_cs + static_cast<uint64_t>(z) * p.rope_token_stride : nullptr;
@@ -84,7 +101,7 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
 template <uint32_t DT, int G, int W>
 __global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams p) {
   __shared__ AttnShared<G, W> sh;
-  if (blockIdx.z != 0) token_view(p, blockIdx.z);
+  if (blockIdx.z != 0 || p.seqs != nullptr) token_view(p, blockIdx.z);
   const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);
   attn_fast_body<DT, G, W, false, 1>(p, p.position, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
 }
@@ -238,7 +255,7 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
                     p.part_acc != nullptr && p.splits >= 1;
   if (fast) {
     const dim3 grid(p.kv_heads, p.splits, p.tokens > 1 ? p.tokens : 1);
-    if (p.tokens > 1) {
+    if (p.tokens > 1 || p.seqs != nullptr) {
       switch (group) {
         case 1: hipLaunchKernelGGL((attn_block_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
         case 2: hipLaunchKernelGGL((attn_block_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
@@ -280,10 +297,11 @@ void attn_bind_workspace(AttnParams &p, void *workspace) {
 }
 
 hipError_t launch_kv_publish_rows(uint32_t dtype, const AttnParams &p, hipStream_t stream) {
-  if (p.qkv == nullptr || p.k_cache == nullptr || p.v_cache == nullptr || p.table == nullptr || p.tokens == 0 ||
-      p.head_dim != static_cast<uint32_t>(kHD) || p.kv_heads == 0)
+  const bool caches = p.seqs != nullptr || (p.k_cache != nullptr && p.v_cache != nullptr && p.table != nullptr);
+  if (p.qkv == nullptr || !caches || p.tokens == 0 || p.head_dim != static_cast<uint32_t>(kHD) || p.kv_heads == 0)
     return hipErrorInvalidValue;
-  if (static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+  if (p.seqs == nullptr &&
+      static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
   const dim3 grid(p.kv_heads, p.tokens);
   if (dtype == kBF16) hipLaunchKernelGGL(kv_publish_rows_kernel<kBF16>, grid, dim3(2 * kWave), 0, stream, p);
@@ -293,23 +311,23 @@ hipError_t launch_kv_publish_rows(uint32_t dtype, const AttnParams &p, hipStream
 }
 
 hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t stream) {
-  if (p.qkv == nullptr || p.k_cache == nullptr || p.v_cache == nullptr || p.table == nullptr ||
-      p.out16 == nullptr)
-    return hipErrorInvalidValue;
+  const bool caches = p.seqs != nullptr || (p.k_cache != nullptr && p.v_cache != nullptr && p.table != nullptr);
+  if (p.qkv == nullptr || !caches || p.out16 == nullptr) return hipErrorInvalidValue;
   if (p.heads == 0 || p.kv_heads == 0 || p.head_dim == 0 || p.heads % p.kv_heads != 0 ||
-      p.block_count == 0 || p.kv_heads > 1024)
+      (p.seqs == nullptr && p.block_count == 0) || p.kv_heads > 1024)
     return hipErrorInvalidValue;
   if (p.rope_freq != nullptr && p.head_dim % 2 != 0) return hipErrorInvalidValue;
   if (p.splits > kAttnMaxSplits) return hipErrorInvalidValue;
-  if (p.cursor == nullptr &&
+  if (p.cursor == nullptr && p.seqs == nullptr &&
       static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
-  if (p.tokens > 1) {
+  if (p.tokens > 1 || p.seqs != nullptr) {
     // a block of positions: host-given positions, rows already in the cache, matrix-core kernel only
     const uint32_t group = p.heads / p.kv_heads;
     const bool fast = p.head_dim == 128 && (group == 1 || group == 2 || group == 4 || group == 8) && p.part_acc != nullptr;
-    if (p.cursor != nullptr || p.append != 0 || !fast || p.tokens > 65535 ||
-        static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+    if (p.cursor != nullptr || p.append != 0 || !fast || p.tokens == 0 || p.tokens > 65535 ||
+        (p.seqs == nullptr &&
+         static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens))
       return hipErrorInvalidValue;
   }
   if (dtype == kBF16) return launch_dt<kBF16>(p, stream);

@@ -21,6 +21,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <atomic>
 #include <vector>
 
 #include "argmax.cuh"
@@ -46,6 +47,21 @@ struct LayerDev {
 
 enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
 enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLFront, kLKinds };
+
+// The weight arena of a session and of every session forked from it (one stream of the weights can
+// then serve a token row of each of them); freed by the last of them to go.
+struct SharedWeights {
+  char *base = nullptr;
+  uint64_t bytes = 0;
+  std::atomic<uint32_t> refs{1};
+};
+
+// What a batch step needs to know of each of its sequences, in device memory: the cache and position
+// for the attention launches, the token slots for the embedding.
+struct BatchTable {
+  AttnSeq seq[kGemmMaxTokens];
+  const Slot *slots[kGemmMaxTokens];
+};
 
 struct StepProfiler {
   hipStream_t stream;
@@ -81,8 +97,10 @@ struct NervaHipHfDecodeSequenceSession {
            layers = 0, max_ctx = 0;
   float eps = 0.0f, theta = 0.0f;
   hipStream_t stream = nullptr;
-  char *arena = nullptr;
-  uint64_t arena_bytes = 0;
+  SharedWeights *weights = nullptr;  // shared with forks
+  char *arena = nullptr;             // everything but the weights: KV cache, sequence state, activations, workspaces
+  uint64_t state_bytes = 0;          // size of `arena`
+  uint64_t arena_bytes = 0;          // weights + state, as reported to the caller
   char *pinned = nullptr;
   uint64_t pinned_bytes = 0;
   std::vector<LayerDev> layer;
@@ -118,6 +136,10 @@ struct NervaHipHfDecodeSequenceSession {
   // prompt blocks: up to kGemmMaxTokens prompt tokens per pass through the layers (weights streamed
   // once per block on the matrix cores); false = one prompt step per token
   bool block_prefill = false;
+  // the multi-row kernels take this model's shapes (prompt blocks and batch steps need it)
+  bool rows_ready = false;
+  float *blogits = nullptr;          // [kGemmMaxTokens][vocab] logits of a batch step
+  BatchTable *btable = nullptr, *host_btable = nullptr;
   float *px = nullptr, *pr = nullptr, *pqkv = nullptr, *prope = nullptr;
   uint16_t *pxn16 = nullptr, *pattn16 = nullptr, *pff16 = nullptr;
   char *pattn_ws = nullptr;
@@ -188,6 +210,27 @@ __global__ __launch_bounds__(kBlock) void embed_rows_kernel(const uint16_t *emb,
   for (uint32_t i = threadIdx.x; i < hidden; i += kBlock) x[static_cast<uint64_t>(t) * hidden + i] = dec16<DT>(row[i]);
 }
 
+// Batch step: row t is the embedding of the token sequence t produced last (slot[position - 1]), and
+// the rotation table of its position.
+template <uint32_t DT>
+__global__ __launch_bounds__(kBlock) void embed_batch_kernel(const uint16_t *emb, const BatchTable *table, uint32_t hidden,
+                                                             uint32_t vocab, float *x, const float *rope_freq,
+                                                             float *rope_cs, uint32_t half_dim) {
+  const uint32_t t = blockIdx.x, pos = table->seq[t].position;
+  if (rope_freq != nullptr) {
+    for (uint32_t i = threadIdx.x; i < half_dim; i += kBlock) {
+      float sn, cs;
+      sincosf(static_cast<float>(pos) / rope_freq[i], &sn, &cs);
+      rope_cs[static_cast<uint64_t>(t) * 2 * half_dim + i] = cs;
+      rope_cs[static_cast<uint64_t>(t) * 2 * half_dim + half_dim + i] = sn;
+    }
+  }
+  uint32_t token = pos == 0 ? 0u : table->slots[t][pos - 1].token;
+  if (token >= vocab) token = 0;  // sampled ids are < vocab
+  const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
+  for (uint32_t i = threadIdx.x; i < hidden; i += kBlock) x[static_cast<uint64_t>(t) * hidden + i] = dec16<DT>(row[i]);
+}
+
 __global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     state[0] = cursor;
@@ -246,6 +289,10 @@ void destroy_session(Session *s) {
   if (s->ev0) (void)hipEventDestroy(s->ev0);
   if (s->ev1) (void)hipEventDestroy(s->ev1);
   if (s->arena) (void)hipFree(s->arena);
+  if (s->weights != nullptr && s->weights->refs.fetch_sub(1) == 1) {
+    if (s->weights->base) (void)hipFree(s->weights->base);
+    delete s->weights;
+  }
   if (s->pinned) (void)hipHostFree(s->pinned);
   if (s->stream) (void)hipStreamDestroy(s->stream);
   delete s;
@@ -739,6 +786,229 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   return err;
 }
 
+// Everything of a session that is not weights, from the dimensions already in `s`: stream, events,
+// the state arena (KV cache, block table, prompt, token slots, cursor words, activations and
+// workspaces), the pinned host mirrors, the step modes. Shared by create and fork.
+hipError_t setup_state(Session *s, int32_t *failure_stage) {
+  const uint64_t H = s->hidden, A = static_cast<uint64_t>(s->heads) * s->head_dim,
+                 KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim, I = s->intermediate, V = s->vocab,
+                 L = s->layers, HD = s->head_dim;
+  const uint32_t block_count = (s->max_ctx + kKvBlockTokens - 1) / kKvBlockTokens;
+  s->block_count = block_count;
+  s->attn_splits = attn_default_splits(s->kv_heads, block_count);
+  if (const char *v = getenv("NERVA_HIP_ATTN_SPLITS")) {  // tuning knob: split-KV factor of the stand-alone attention
+    const long want = strtol(v, nullptr, 10);
+    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits))
+      s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
+  }
+
+  Carver c;
+  const uint64_t kv_half = L * block_count * KV * kKvBlockTokens * 2;
+  const uint64_t off_kc = c.take(kv_half);
+  const uint64_t off_vc = c.take(kv_half);
+  s->kv_bytes = 2 * kv_half;
+  const uint64_t off_table = c.take(static_cast<uint64_t>(block_count) * 4);
+  const uint64_t off_prompt = c.take(static_cast<uint64_t>(s->max_ctx) * 4);
+  const uint64_t off_slots = c.take(static_cast<uint64_t>(s->max_ctx) * sizeof(Slot));
+  const uint64_t off_state = c.take(64);
+  const uint64_t off_x = c.take(H * 4);
+  const uint64_t off_r = c.take(H * 4);
+  const uint64_t off_qkv = c.take((A + 2 * KV) * 4);
+  const uint64_t off_logits = c.take(V * 4);
+  const uint64_t off_attn16 = c.take(A * 2);
+  const uint64_t off_ff16 = c.take(I * 2);
+  const uint64_t off_rope = c.take(HD * 4);
+  const uint64_t off_rope_cs = c.take(HD * 4);
+  const uint64_t attn_ws_bytes = attn_workspace_bytes(s->heads, s->head_dim);
+  const uint64_t off_attn_ws = c.take(attn_ws_bytes);
+  const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
+  const uint64_t pT = kGemmMaxTokens;
+  const uint64_t off_px = c.take(pT * H * 4);
+  const uint64_t off_pr = c.take(pT * H * 4);
+  const uint64_t off_pqkv = c.take(pT * (A + 2 * KV) * 4);
+  const uint64_t off_pxn16 = c.take(pT * H * 2);
+  const uint64_t off_pattn16 = c.take(pT * A * 2);
+  const uint64_t off_pff16 = c.take(pT * I * 2);
+  const uint64_t off_prope = c.take(pT * HD * 4);
+  const uint64_t pattn_ws_stride = (attn_ws_bytes + 255u) & ~uint64_t{255};
+  const uint64_t off_pattn_ws = c.take(pT * pattn_ws_stride);
+  const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
+  const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(s->vocab));
+  const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
+  const uint64_t off_chain_trace = c.take(L * 32 * 8);
+  const uint64_t front_ws_bytes = front_workspace_bytes(s->heads, s->kv_heads);
+  const uint64_t off_front_ws = c.take(front_ws_bytes);
+  {
+    // Prompt blocks and batch steps need the matrix-core attention (head_dim 128, GQA factor
+    // 1/2/4/8) and shapes the multi-row kernels take.
+    const uint32_t group = s->heads / s->kv_heads;
+    s->rows_ready = s->head_dim == 128 && (group == 1 || group == 2 || group == 4 || group == 8) && s->hidden <= 16384 &&
+                    gemm_rows_supported(static_cast<uint32_t>(A + 2 * KV), s->hidden, 1) &&
+                    gemm_rows_supported(s->hidden, static_cast<uint32_t>(A), 1) &&
+                    gemm_rows_supported(s->intermediate, s->hidden, 1) &&
+                    gemm_rows_supported(s->hidden, s->intermediate, 1);
+  }
+  const bool batch_head = s->rows_ready && gemm_rows_supported(s->vocab, s->hidden, 1);
+  const uint64_t off_blogits = batch_head ? c.take(pT * V * 4) : 0;
+  const uint64_t off_btable = c.take(sizeof(BatchTable));
+  s->state_bytes = c.offset;
+  s->arena_bytes = s->weights->bytes + s->state_bytes;
+
+  *failure_stage = 2;
+  hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
+  if (err == hipSuccess) err = counted_malloc(reinterpret_cast<void **>(&s->arena), s->state_bytes);
+  if (err != hipSuccess) return err;
+  *failure_stage = 3;
+  const uint64_t pinned_seq = (static_cast<uint64_t>(s->max_ctx) * (sizeof(Slot) + 4) + 256 + 255u) & ~uint64_t{255};
+  s->pinned_bytes = pinned_seq + sizeof(BatchTable);
+  err = counted_host_malloc(reinterpret_cast<void **>(&s->pinned), s->pinned_bytes);
+  if (err == hipSuccess) err = hipEventCreate(&s->ev0);
+  if (err == hipSuccess) err = hipEventCreate(&s->ev1);
+  if (err != hipSuccess) return err;
+  s->host_slots = reinterpret_cast<Slot *>(s->pinned);
+  s->host_prompt = reinterpret_cast<uint32_t *>(s->pinned + static_cast<uint64_t>(s->max_ctx) * sizeof(Slot));
+  s->host_state = s->host_prompt + s->max_ctx;
+  s->host_btable = reinterpret_cast<BatchTable *>(s->pinned + pinned_seq);
+
+  auto dev16 = [&](uint64_t off) { return reinterpret_cast<uint16_t *>(s->arena + off); };
+  s->kc = dev16(off_kc);
+  s->vc = dev16(off_vc);
+  s->table = reinterpret_cast<uint32_t *>(s->arena + off_table);
+  s->prompt = reinterpret_cast<uint32_t *>(s->arena + off_prompt);
+  s->slots = reinterpret_cast<Slot *>(s->arena + off_slots);
+  s->state = reinterpret_cast<uint32_t *>(s->arena + off_state);
+  s->x = reinterpret_cast<float *>(s->arena + off_x);
+  s->r = reinterpret_cast<float *>(s->arena + off_r);
+  s->qkv = reinterpret_cast<float *>(s->arena + off_qkv);
+  s->logits = reinterpret_cast<float *>(s->arena + off_logits);
+  s->attn16 = dev16(off_attn16);
+  s->ff16 = dev16(off_ff16);
+  s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
+  s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
+  s->attn_ws = s->arena + off_attn_ws;
+  s->sample_ws = s->arena + off_sample_ws;
+  s->px = reinterpret_cast<float *>(s->arena + off_px);
+  s->pr = reinterpret_cast<float *>(s->arena + off_pr);
+  s->pqkv = reinterpret_cast<float *>(s->arena + off_pqkv);
+  s->pxn16 = dev16(off_pxn16);
+  s->pattn16 = dev16(off_pattn16);
+  s->pff16 = dev16(off_pff16);
+  s->prope = reinterpret_cast<float *>(s->arena + off_prope);
+  s->pattn_ws = s->arena + off_pattn_ws;
+  s->pattn_ws_stride = pattn_ws_stride;
+  s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
+  s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
+  {
+    // NERVA_HIP_PREFILL=walk keeps one prompt step per token where prompt blocks would be possible.
+    const char *mode = getenv("NERVA_HIP_PREFILL");
+    s->block_prefill = s->rows_ready && !(mode != nullptr && mode[0] == 'w');
+  }
+  s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
+  s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
+  s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
+  s->chain_abort = reinterpret_cast<uint32_t *>(s->arena + off_chain + chain_flag_bytes());
+  {
+    // NERVA_HIP_CHAIN=1 runs o + gate/up + down + next qkv as one persistent launch per layer.
+    // Off by default: measured on MI355X it is about 4 % slower per step than one launch per
+    // GEMV (the in-kernel grid barriers cost as much as the kernel boundaries they replace, and
+    // a static split of the rows over 256 workgroups waits longer for its slowest member).
+    const char *want_chain = getenv("NERVA_HIP_CHAIN");
+    s->chain = want_chain != nullptr && want_chain[0] == '1' && s->layers > 0 &&
+               chain_supported(s->hidden, s->heads * s->head_dim, s->intermediate,
+                               (s->heads + 2 * s->kv_heads) * s->head_dim) &&
+               chain_prepare(s->dtype) == hipSuccess;
+    const char *trace = getenv("NERVA_HIP_CHAIN_TRACE");
+    if (s->chain && trace != nullptr && trace[0] == '1')
+      s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
+  }
+  s->front_ws = s->arena + off_front_ws;
+  {
+    // Fused layer front (layer_front.cuh), opt-in: NERVA_HIP_FRONT=2 runs attention + o
+    // projection as roles of one launch, =1 adds the qkv projection as a third role. Off by
+    // default: measured on MI355X every hand-over between workgroups through memory costs
+    // 1.2-1.8 us (device-coherent store, poll, dependent load), about what the kernel boundary
+    // it replaces costs, and the attention role runs under a tighter register budget; the step is
+    // 3-6 % slower than with one launch per piece.
+    const char *want = getenv("NERVA_HIP_FRONT");
+    int mode = 0;
+    if (want != nullptr && want[0] >= '0' && want[0] <= '2') mode = want[0] - '0';
+    if (s->chain || s->layers == 0 || !front_supported(s->hidden, s->heads, s->kv_heads, s->head_dim)) mode = 0;
+    s->front = mode;
+    // one KV tile in flight per wave there, so twice the stand-alone kernel's splits
+    uint32_t splits = (256 + s->kv_heads - 1) / s->kv_heads;
+    if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
+    if (splits > block_count) splits = block_count;
+    s->front_splits = splits == 0 ? 1 : splits;
+    const char *trace = getenv("NERVA_HIP_FRONT_TRACE");
+    if (!s->chain && s->layers > 0 && trace != nullptr && trace[0] == '1')
+      s->front_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
+  }
+
+  *failure_stage = 5;
+  {
+    std::vector<uint32_t> table(block_count);
+    for (uint32_t i = 0; i < block_count; ++i) table[i] = i;  // identity (kernels.cu:733-739)
+    err = hipMemcpy(s->table, table.data(), table.size() * 4, hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess && s->theta > 0.0f) {
+    // powf(theta, 2i/d) evaluated once on the host in f32 (common/rope.rs:69-70); the
+    // kernels divide the f32 position by it.
+    std::vector<float> freq(HD / 2);
+    for (uint32_t i = 0; i < HD / 2; ++i)
+      freq[i] = powf(s->theta, static_cast<float>(2 * i) / static_cast<float>(HD));
+    err = hipMemcpy(s->rope_freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_ws_bytes, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_ws, 0, front_ws_bytes, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
+  if (err == hipSuccess && L > 0) err = hipMemsetAsync(s->arena + off_chain_trace, 0, L * 32 * 8, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->sampler_dev, 0, sizeof(SamplerDev), s->stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+  return err;
+}
+
+void fill_create_result(const Session *s, NervaHipHfDecodeSequenceSessionCreateResult *out) {
+  out->device_count = 1;
+  out->dtype = s->dtype;
+  out->hidden = s->hidden;
+  out->heads = s->heads;
+  out->kv_heads = s->kv_heads;
+  out->head_dim = s->head_dim;
+  out->intermediate = s->intermediate;
+  out->vocab_size = s->vocab;
+  out->layer_count = s->layers;
+  out->max_context_tokens = s->max_ctx;
+  out->prefill_chunk_tokens = s->block_prefill ? kGemmMaxTokens : 1;
+  out->head_threads = kBlock;
+  out->resident_weight_bytes = s->resident_weight_bytes;
+  out->planned_weight_blocks = s->planned_weight_blocks;
+  out->planned_gpu_resident_blocks = s->planned_gpu_resident_blocks;
+  out->planned_gpu_staged_blocks = s->planned_gpu_staged_blocks;
+  out->planned_weight_bytes = s->planned_weight_bytes;
+  out->planned_gpu_resident_weight_bytes = s->planned_gpu_resident_weight_bytes;
+  out->planned_gpu_staged_weight_bytes = s->planned_gpu_staged_weight_bytes;
+  out->descriptor_gpu_resident_h2d_bytes = s->planned_gpu_resident_weight_bytes;
+  out->descriptor_gpu_staged_h2d_bytes = s->planned_gpu_staged_weight_bytes;
+  out->planned_weight_descriptor_count = s->planned_weight_descriptor_count;
+  out->planned_weight_descriptor_hash = s->planned_weight_descriptor_hash;
+  out->resident_kv_bytes = s->kv_bytes;
+  out->device_arena_bytes = s->arena_bytes;
+  out->pinned_host_bytes = s->pinned_bytes;
+  out->hot_path_allocations = 0;
+  {
+    // device-reported memory clock x bus width, like session_api_lifecycle.inc.cu:84-106
+    int clock_khz = 0, bus_bits = 0;
+    if (hipDeviceGetAttribute(&clock_khz, hipDeviceAttributeMemoryClockRate, 0) == hipSuccess &&
+        hipDeviceGetAttribute(&bus_bits, hipDeviceAttributeMemoryBusWidth, 0) == hipSuccess)
+      out->device_memory_bandwidth_bps = static_cast<uint64_t>(clock_khz) * 1000ull * 2ull * (static_cast<uint64_t>(bus_bits) / 8ull);
+  }
+}
+
 int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool synthetic, uint64_t seed,
                 float weight_std, uint32_t with_qk_norm, NervaHipHfDecodeSequenceSessionCreateResult *out,
                 Session **session_out) {
@@ -786,14 +1056,17 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   out->head_threads = kBlock;
   out->experimental_rt_decode_requested = rq->experimental_rt_decode;
 
-  const uint64_t allocs_before = allocation_count();
   const uint64_t H = rq->hidden, A = static_cast<uint64_t>(rq->heads) * rq->head_dim,
                  KV = static_cast<uint64_t>(rq->kv_heads) * rq->head_dim, I = rq->intermediate,
                  V = rq->vocab_size, L = rq->layer_count, HD = rq->head_dim;
-  const uint32_t block_count = (rq->max_context_tokens + kKvBlockTokens - 1) / kKvBlockTokens;
 
   Session *s = new (std::nothrow) Session();
   if (s == nullptr) return -1;
+  s->weights = new (std::nothrow) SharedWeights();
+  if (s->weights == nullptr) {
+    delete s;
+    return -1;
+  }
   s->dtype = rq->dtype;
   s->hidden = rq->hidden;
   s->heads = rq->heads;
@@ -805,7 +1078,6 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->max_ctx = rq->max_context_tokens;
   s->eps = rq->rms_eps;
   s->theta = rq->rope_theta;
-  s->block_count = block_count;
   s->planned_weight_blocks = rq->planned_weight_blocks;
   s->planned_gpu_resident_blocks = rq->planned_gpu_resident_blocks;
   s->planned_gpu_staged_blocks = rq->planned_gpu_staged_blocks;
@@ -814,14 +1086,8 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->planned_gpu_staged_weight_bytes = rq->planned_gpu_staged_weight_bytes;
   s->planned_weight_descriptor_count = rq->planned_weight_descriptor_count;
   s->planned_weight_descriptor_hash = rq->planned_weight_descriptor_hash;
-  s->attn_splits = attn_default_splits(rq->kv_heads, block_count);
-  if (const char *v = getenv("NERVA_HIP_ATTN_SPLITS")) {  // tuning knob: split-KV factor of the stand-alone attention
-    const long want = strtol(v, nullptr, 10);
-    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits))
-      s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
-  }
 
-  // ---- arena layout ------------------------------------------------------
+  // ---- weight arena layout -------------------------------------------------
   struct LayerOff {
     uint64_t rms_attn, rms_mlp, wqkv, q_norm, k_norm, q_bias, k_bias, v_bias, wo, o_bias, wgu, wdown;
   };
@@ -859,41 +1125,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   const uint64_t off_lm = c.take(V * H * 2);
   weight_elems += H + V * H;
   s->resident_weight_bytes = weight_elems * 2;
-  const uint64_t kv_half = L * block_count * KV * kKvBlockTokens * 2;
-  const uint64_t off_kc = c.take(kv_half);
-  const uint64_t off_vc = c.take(kv_half);
-  s->kv_bytes = 2 * kv_half;
-  const uint64_t off_table = c.take(static_cast<uint64_t>(block_count) * 4);
-  const uint64_t off_prompt = c.take(static_cast<uint64_t>(rq->max_context_tokens) * 4);
-  const uint64_t off_slots = c.take(static_cast<uint64_t>(rq->max_context_tokens) * sizeof(Slot));
-  const uint64_t off_state = c.take(64);
-  const uint64_t off_x = c.take(H * 4);
-  const uint64_t off_r = c.take(H * 4);
-  const uint64_t off_qkv = c.take((A + 2 * KV) * 4);
-  const uint64_t off_logits = c.take(V * 4);
-  const uint64_t off_attn16 = c.take(A * 2);
-  const uint64_t off_ff16 = c.take(I * 2);
-  const uint64_t off_rope = c.take(HD * 4);
-  const uint64_t off_rope_cs = c.take(HD * 4);
-  const uint64_t off_attn_ws = c.take(attn_workspace_bytes(rq->heads, rq->head_dim));
-  const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
-  const uint64_t pT = kGemmMaxTokens;
-  const uint64_t off_px = c.take(pT * H * 4);
-  const uint64_t off_pr = c.take(pT * H * 4);
-  const uint64_t off_pqkv = c.take(pT * (A + 2 * KV) * 4);
-  const uint64_t off_pxn16 = c.take(pT * H * 2);
-  const uint64_t off_pattn16 = c.take(pT * A * 2);
-  const uint64_t off_pff16 = c.take(pT * I * 2);
-  const uint64_t off_prope = c.take(pT * HD * 4);
-  const uint64_t pattn_ws_stride = (attn_workspace_bytes(rq->heads, rq->head_dim) + 255u) & ~uint64_t{255};
-  const uint64_t off_pattn_ws = c.take(pT * pattn_ws_stride);
-  const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
-  const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(rq->vocab_size));
-  const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
-  const uint64_t off_chain_trace = c.take(static_cast<uint64_t>(rq->layer_count) * 32 * 8);
-  const uint64_t front_ws_bytes = front_workspace_bytes(rq->heads, rq->kv_heads);
-  const uint64_t off_front_ws = c.take(front_ws_bytes);
-  s->arena_bytes = c.offset;
+  s->weights->bytes = c.offset;
 
   if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
     // session_api_oneshot.inc.cu: a weight plan that disagrees with the arena is rejected
@@ -901,111 +1133,26 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
     return -1;
   }
 
-  hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
   out->failure_stage = 2;
-  if (err == hipSuccess) err = counted_malloc(reinterpret_cast<void **>(&s->arena), s->arena_bytes);
-  out->failure_stage = 3;
-  s->pinned_bytes = static_cast<uint64_t>(rq->max_context_tokens) * (sizeof(Slot) + 4) + 256;
-  if (err == hipSuccess) err = counted_host_malloc(reinterpret_cast<void **>(&s->pinned), s->pinned_bytes);
-  if (err == hipSuccess) err = hipEventCreate(&s->ev0);
-  if (err == hipSuccess) err = hipEventCreate(&s->ev1);
+  hipError_t err = counted_malloc(reinterpret_cast<void **>(&s->weights->base), s->weights->bytes);
+  if (err == hipSuccess) err = setup_state(s, &out->failure_stage);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     destroy_session(s);
     return -1;
   }
-  s->host_slots = reinterpret_cast<Slot *>(s->pinned);
-  s->host_prompt = reinterpret_cast<uint32_t *>(s->pinned + static_cast<uint64_t>(rq->max_context_tokens) * sizeof(Slot));
-  s->host_state = s->host_prompt + rq->max_context_tokens;
 
-  auto dev16 = [&](uint64_t off) { return off == kNone ? nullptr : reinterpret_cast<uint16_t *>(s->arena + off); };
-  s->emb = dev16(off_emb);
-  s->final_norm = dev16(off_final);
-  s->lm_head = dev16(off_lm);
-  s->kc = dev16(off_kc);
-  s->vc = dev16(off_vc);
-  s->table = reinterpret_cast<uint32_t *>(s->arena + off_table);
-  s->prompt = reinterpret_cast<uint32_t *>(s->arena + off_prompt);
-  s->slots = reinterpret_cast<Slot *>(s->arena + off_slots);
-  s->state = reinterpret_cast<uint32_t *>(s->arena + off_state);
-  s->x = reinterpret_cast<float *>(s->arena + off_x);
-  s->r = reinterpret_cast<float *>(s->arena + off_r);
-  s->qkv = reinterpret_cast<float *>(s->arena + off_qkv);
-  s->logits = reinterpret_cast<float *>(s->arena + off_logits);
-  s->attn16 = dev16(off_attn16);
-  s->ff16 = dev16(off_ff16);
-  s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
-  s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
-  s->attn_ws = s->arena + off_attn_ws;
-  s->sample_ws = s->arena + off_sample_ws;
-  s->px = reinterpret_cast<float *>(s->arena + off_px);
-  s->pr = reinterpret_cast<float *>(s->arena + off_pr);
-  s->pqkv = reinterpret_cast<float *>(s->arena + off_pqkv);
-  s->pxn16 = dev16(off_pxn16);
-  s->pattn16 = dev16(off_pattn16);
-  s->pff16 = dev16(off_pff16);
-  s->prope = reinterpret_cast<float *>(s->arena + off_prope);
-  s->pattn_ws = s->arena + off_pattn_ws;
-  s->pattn_ws_stride = pattn_ws_stride;
-  {
-    // Prompt blocks need the matrix-core attention (head_dim 128, GQA factor 1/2/4/8) and shapes the
-    // multi-row GEMM takes; NERVA_HIP_PREFILL=walk keeps one prompt step per token.
-    const char *mode = getenv("NERVA_HIP_PREFILL");
-    const uint32_t group = rq->heads / rq->kv_heads;
-    s->block_prefill = !(mode != nullptr && mode[0] == 'w') && rq->head_dim == 128 &&
-                       (group == 1 || group == 2 || group == 4 || group == 8) &&
-                       gemm_rows_supported(static_cast<uint32_t>(A + 2 * KV), rq->hidden, 1) &&
-                       gemm_rows_supported(rq->hidden, static_cast<uint32_t>(A), 1) &&
-                       gemm_rows_supported(rq->intermediate, rq->hidden, 1) &&
-                       gemm_rows_supported(rq->hidden, rq->intermediate, 1);
-  }
-  s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
-  s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
-  s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
-  s->chain_abort = reinterpret_cast<uint32_t *>(s->arena + off_chain + chain_flag_bytes());
-  {
-    // NERVA_HIP_CHAIN=1 runs o + gate/up + down + next qkv as one persistent launch per layer.
-    // Off by default: measured on MI355X it is about 4 % slower per step than one launch per
-    // GEMV (the in-kernel grid barriers cost as much as the kernel boundaries they replace, and
-    // a static split of the rows over 256 workgroups waits longer for its slowest member).
-    const char *want_chain = getenv("NERVA_HIP_CHAIN");
-    s->chain = want_chain != nullptr && want_chain[0] == '1' && rq->layer_count > 0 &&
-               chain_supported(rq->hidden, rq->heads * rq->head_dim, rq->intermediate,
-                               (rq->heads + 2 * rq->kv_heads) * rq->head_dim) &&
-               chain_prepare(rq->dtype) == hipSuccess;
-    const char *trace = getenv("NERVA_HIP_CHAIN_TRACE");
-    if (s->chain && trace != nullptr && trace[0] == '1')
-      s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
-  }
-  s->front_ws = s->arena + off_front_ws;
-  {
-    // Fused layer front (layer_front.cuh), opt-in: NERVA_HIP_FRONT=2 runs attention + o
-    // projection as roles of one launch, =1 adds the qkv projection as a third role. Off by
-    // default: measured on MI355X every hand-over between workgroups through memory costs
-    // 1.2-1.8 us (device-coherent store, poll, dependent load), about what the kernel boundary
-    // it replaces costs, and the attention role runs under a tighter register budget; the step is
-    // 3-6 % slower than with one launch per piece.
-    const char *want = getenv("NERVA_HIP_FRONT");
-    int mode = 0;
-    if (want != nullptr && want[0] >= '0' && want[0] <= '2') mode = want[0] - '0';
-    if (s->chain || rq->layer_count == 0 || !front_supported(rq->hidden, rq->heads, rq->kv_heads, rq->head_dim))
-      mode = 0;
-    s->front = mode;
-    // one KV tile in flight per wave there, so twice the stand-alone kernel's splits
-    uint32_t splits = (256 + rq->kv_heads - 1) / rq->kv_heads;
-    if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
-    if (splits > block_count) splits = block_count;
-    s->front_splits = splits == 0 ? 1 : splits;
-    const char *trace = getenv("NERVA_HIP_FRONT_TRACE");
-    if (!s->chain && rq->layer_count > 0 && trace != nullptr && trace[0] == '1')
-      s->front_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
-  }
+  char *wbase = s->weights->base;
+  auto w16 = [&](uint64_t off) -> const uint16_t * { return off == kNone ? nullptr : reinterpret_cast<const uint16_t *>(wbase + off); };
+  s->emb = w16(off_emb);
+  s->final_norm = w16(off_final);
+  s->lm_head = w16(off_lm);
   s->layer.resize(L);
   for (uint32_t l = 0; l < L; ++l) {
-    s->layer[l] = LayerDev{dev16(lo[l].rms_attn), dev16(lo[l].rms_mlp), dev16(lo[l].wqkv),
-                           dev16(lo[l].q_norm),   dev16(lo[l].k_norm),  dev16(lo[l].q_bias),
-                           dev16(lo[l].k_bias),   dev16(lo[l].v_bias),  dev16(lo[l].wo),
-                           dev16(lo[l].o_bias),   dev16(lo[l].wgu),     dev16(lo[l].wdown)};
+    s->layer[l] = LayerDev{w16(lo[l].rms_attn), w16(lo[l].rms_mlp), w16(lo[l].wqkv),
+                           w16(lo[l].q_norm),   w16(lo[l].k_norm),  w16(lo[l].q_bias),
+                           w16(lo[l].k_bias),   w16(lo[l].v_bias),  w16(lo[l].wo),
+                           w16(lo[l].o_bias),   w16(lo[l].wgu),     w16(lo[l].wdown)};
   }
 
   // ---- weights -------------------------------------------------------------
@@ -1013,12 +1160,12 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   uint64_t h2d = 0;
   auto upload = [&](uint64_t off, const uint16_t *src, uint64_t elems) {
     if (err != hipSuccess || off == kNone) return;
-    err = hipMemcpy(s->arena + off, src, elems * 2, hipMemcpyHostToDevice);
+    err = hipMemcpy(wbase + off, src, elems * 2, hipMemcpyHostToDevice);
     h2d += elems * 2;
   };
   auto fill = [&](uint64_t off, uint64_t tensor_id, uint64_t elems, float mean) {
     if (err != hipSuccess || off == kNone) return;
-    err = launch_synth_16(s->arena + off, s->dtype, seed, tensor_id, elems, mean, weight_std, s->stream);
+    err = launch_synth_16(wbase + off, s->dtype, seed, tensor_id, elems, mean, weight_std, s->stream);
   };
   if (synthetic) {
     fill(off_emb, 1, V * H, 0.0f);
@@ -1038,6 +1185,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
       fill(lo[l].wgu + I * H * 2, base + 14, I * H, 0.0f);
       fill(lo[l].wdown, base + 15, H * I, 0.0f);
     }
+    if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
   } else {
     upload(off_emb, rq->embeddings, V * H);
     upload(off_final, rq->final_norm_weight, H);
@@ -1063,71 +1211,417 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
       upload(lo[l].wdown, src.w_down, H * I);
     }
   }
-  // ---- state ---------------------------------------------------------------
-  out->failure_stage = 5;
-  if (err == hipSuccess) {
-    std::vector<uint32_t> table(block_count);
-    for (uint32_t i = 0; i < block_count; ++i) table[i] = i;  // identity (kernels.cu:733-739)
-    err = hipMemcpy(s->table, table.data(), table.size() * 4, hipMemcpyHostToDevice);
-  }
-  if (err == hipSuccess && s->theta > 0.0f) {
-    // powf(theta, 2i/d) evaluated once on the host in f32 (common/rope.rs:69-70); the
-    // kernels divide the f32 position by it.
-    std::vector<float> freq(HD / 2);
-    for (uint32_t i = 0; i < HD / 2; ++i)
-      freq[i] = powf(s->theta, static_cast<float>(2 * i) / static_cast<float>(HD));
-    err = hipMemcpy(s->rope_freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
-  }
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_workspace_bytes(rq->heads, rq->head_dim), s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_ws, 0, front_ws_bytes, s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
-  if (err == hipSuccess && rq->layer_count > 0)
-    err = hipMemsetAsync(s->arena + off_chain_trace, 0, static_cast<uint64_t>(rq->layer_count) * 32 * 8, s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
-  if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     destroy_session(s);
     return -1;
   }
   out->failure_stage = 0;
-  out->resident_weight_bytes = s->resident_weight_bytes;
-  out->planned_weight_blocks = s->planned_weight_blocks;
-  out->planned_gpu_resident_blocks = s->planned_gpu_resident_blocks;
-  out->planned_gpu_staged_blocks = s->planned_gpu_staged_blocks;
-  out->planned_weight_bytes = s->planned_weight_bytes;
-  out->planned_gpu_resident_weight_bytes = s->planned_gpu_resident_weight_bytes;
-  out->planned_gpu_staged_weight_bytes = s->planned_gpu_staged_weight_bytes;
-  out->descriptor_gpu_resident_h2d_bytes = s->planned_gpu_resident_weight_bytes;
-  out->descriptor_gpu_staged_h2d_bytes = s->planned_gpu_staged_weight_bytes;
-  out->planned_weight_descriptor_count = s->planned_weight_descriptor_count;
-  out->planned_weight_descriptor_hash = s->planned_weight_descriptor_hash;
-  out->resident_kv_bytes = s->kv_bytes;
-  out->device_arena_bytes = s->arena_bytes;
-  out->pinned_host_bytes = s->pinned_bytes;
+  fill_create_result(s, out);
   out->h2d_bytes = h2d;
   out->sync_calls = 1;
-  out->hot_path_allocations = 0;
-  (void)allocs_before;
-  {
-    // device-reported memory clock x bus width, like session_api_lifecycle.inc.cu:84-106
-    int clock_khz = 0, bus_bits = 0;
-    if (hipDeviceGetAttribute(&clock_khz, hipDeviceAttributeMemoryClockRate, 0) == hipSuccess &&
-        hipDeviceGetAttribute(&bus_bits, hipDeviceAttributeMemoryBusWidth, 0) == hipSuccess)
-      out->device_memory_bandwidth_bps = static_cast<uint64_t>(clock_khz) * 1000ull * 2ull * (static_cast<uint64_t>(bus_bits) / 8ull);
-  }
   out->status = 0;
   *session_out = s;
   return 0;
 }
 
+
+// One decode step for `T` sequences on the weights and workspaces of `lead`: the token rows of all
+// sequences go through every projection as one multi-row GEMM (one stream of the weights for all),
+// attention runs per sequence on its own cache and position inside one launch, and every sequence
+// samples with its own sampler. Decode staging (f32 hidden state between layers), like enqueue_step.
+// Reference: session_api_layer_projection_batch.inc.cu (qkv, o, gate/up, down per layer) and
+// session_api_batch_fork_destroy.inc.cu:166-259 (layers, LM head, one sampler launch per session).
+hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
+                              NervaHipHfDecodeSequenceBatchAdvanceResult *out) {
+  hipStream_t st = lead->stream;
+  const uint32_t H = lead->hidden, A = lead->heads * lead->head_dim, KV = lead->kv_heads * lead->head_dim,
+                 I = lead->intermediate;
+  const float *rope_freq = lead->theta > 0.0f ? lead->rope_freq : nullptr;
+  BatchTable *host = lead->host_btable;
+  uint32_t min_blocks = ~0u;
+  for (uint32_t t = 0; t < T; ++t) {
+    const Session *q = seqs[t];
+    host->seq[t] = AttnSeq{q->kc, q->vc, q->table, q->block_count, q->cursor};
+    host->slots[t] = q->slots;
+    min_blocks = std::min(min_blocks, q->block_count);
+  }
+  hipError_t err = hipMemcpyAsync(lead->btable, host, sizeof(BatchTable), hipMemcpyHostToDevice, st);
+  if (err != hipSuccess) return err;
+  if (lead->dtype == kBF16)
+    hipLaunchKernelGGL(embed_batch_kernel<kBF16>, dim3(T), dim3(kBlock), 0, st, lead->emb, lead->btable, H, lead->vocab,
+                       lead->px, rope_freq, lead->prope, lead->head_dim / 2);
+  else
+    hipLaunchKernelGGL(embed_batch_kernel<kF16>, dim3(T), dim3(kBlock), 0, st, lead->emb, lead->btable, H, lead->vocab,
+                       lead->px, rope_freq, lead->prope, lead->head_dim / 2);
+  err = hipGetLastError();
+  out->pack_kernel_launches += 1;
+  for (uint32_t l = 0; err == hipSuccess && l < lead->layers; ++l) {
+    const LayerDev &w = lead->layer[l];
+    err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st);
+    GemmRowsParams g{};
+    if (err == hipSuccess) {
+      g.tokens = T;
+      g.w = w.wqkv;
+      g.x16 = lead->pxn16;
+      g.out_f32 = lead->pqkv;
+      g.rows = A + 2 * KV;
+      g.cols = H;
+      err = launch_gemm_rows(lead->dtype, kGemmF32, g, st);
+    }
+    AttnParams a{};
+    a.heads = lead->heads;
+    a.kv_heads = lead->kv_heads;
+    a.head_dim = lead->head_dim;
+    attn_bind_workspace(a, lead->pattn_ws);
+    a.qkv = lead->pqkv;
+    a.q_norm = w.q_norm;
+    a.k_norm = w.k_norm;
+    a.q_bias = w.q_bias;
+    a.k_bias = w.k_bias;
+    a.v_bias = w.v_bias;
+    a.rope_freq = rope_freq;
+    a.rope_cs = rope_freq != nullptr ? lead->prope : nullptr;
+    a.out16 = lead->pattn16;
+    a.layer = l;
+    a.splits = attn_default_splits(lead->kv_heads, min_blocks);
+    a.eps = lead->eps;
+    a.tokens = T;
+    a.qkv_token_stride = A + 2 * KV;
+    a.out_token_stride = A;
+    a.rope_token_stride = lead->head_dim;
+    a.ws_token_stride = lead->pattn_ws_stride;
+    a.seqs = lead->btable->seq;
+    if (err == hipSuccess) err = launch_kv_publish_rows(lead->dtype, a, st);
+    if (err == hipSuccess) err = launch_attn_decode(lead->dtype, a, st);
+    if (err == hipSuccess) {
+      g = GemmRowsParams{};
+      g.tokens = T;
+      g.w = w.wo;
+      g.x16 = lead->pattn16;
+      g.bias = w.o_bias;
+      g.residual = lead->px;
+      g.out_f32 = lead->pr;
+      g.rows = H;
+      g.cols = A;
+      err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
+    }
+    if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st);
+    if (err == hipSuccess) {
+      g = GemmRowsParams{};
+      g.tokens = T;
+      g.w = w.wgu;
+      g.x16 = lead->pxn16;
+      g.out16 = lead->pff16;
+      g.rows = I;
+      g.cols = H;
+      err = launch_gemm_rows(lead->dtype, kGemmSwiglu, g, st);
+    }
+    if (err == hipSuccess) {
+      g = GemmRowsParams{};
+      g.tokens = T;
+      g.w = w.wdown;
+      g.x16 = lead->pff16;
+      g.residual = lead->pr;
+      g.out_f32 = lead->px;
+      g.rows = H;
+      g.cols = I;
+      err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
+    }
+    out->pack_kernel_launches += 2;
+    out->projection_kernel_launches += 4;
+    out->scatter_kernel_launches += 1;
+    out->dependency_kernel_launches += 1;
+  }
+  if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st);
+  if (err == hipSuccess) {
+    GemmRowsParams g{};
+    g.tokens = T;
+    g.w = lead->lm_head;
+    g.x16 = lead->pxn16;
+    g.out_f32 = lead->blogits;
+    g.rows = lead->vocab;
+    g.cols = H;
+    err = launch_gemm_rows(lead->dtype, kGemmF32, g, st);
+    out->pack_kernel_launches += 1;
+    out->projection_kernel_launches += 1;
+  }
+  for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
+    // slot[position], cursor -> position + 1, with the sequence's own sampler and random-number counter
+    Session *q = seqs[t];
+    SamplerParams sp{};
+    sp.logits = lead->blogits + static_cast<uint64_t>(t) * lead->vocab;
+    sp.vocab = q->vocab;
+    sp.config = q->sampler_dev;
+    sp.keys = q->sampler_keys;
+    sample_bind_workspace(sp.out, q->sample_ws);
+    sp.out.slots = q->slots;
+    sp.out.cursor_rw = q->state;
+    sp.cursor = q->state;
+    sp.max_steps = q->max_ctx;
+    err = launch_sampler(sp, st);
+    out->sampling_kernel_launches += 2;
+  }
+  return err;
+}
+
 }  // namespace
 
 extern "C" {
+
+int nerva_hip_hf_decode_sequence_session_fork_shared_weights(
+    const NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest *request,
+    NervaHipHfDecodeSequenceSessionCreateResult *out, NervaHipHfDecodeSequenceSession **session_out) {
+  if (!begin_result(out)) return -1;
+  if (session_out == nullptr) return -1;
+  *session_out = nullptr;
+  out->failure_stage = 1;
+  if (request == nullptr || request->parent == nullptr || request->parent->weights == nullptr) return -1;
+  Session *parent = request->parent;
+  // session_api_batch_fork_destroy.inc.cu:331-333: a sequence under way is carried over
+  const bool clone = parent->started && !parent->finished && parent->prompt_count != 0;
+  if (!device_ready(&out->hip_error)) return -1;
+
+  Session *s = new (std::nothrow) Session();
+  if (s == nullptr) return -1;
+  s->dtype = parent->dtype;
+  s->hidden = parent->hidden;
+  s->heads = parent->heads;
+  s->kv_heads = parent->kv_heads;
+  s->head_dim = parent->head_dim;
+  s->intermediate = parent->intermediate;
+  s->vocab = parent->vocab;
+  s->layers = parent->layers;
+  s->max_ctx = parent->max_ctx;
+  s->eps = parent->eps;
+  s->theta = parent->theta;
+  s->planned_weight_blocks = parent->planned_weight_blocks;
+  s->planned_gpu_resident_blocks = parent->planned_gpu_resident_blocks;
+  s->planned_gpu_staged_blocks = parent->planned_gpu_staged_blocks;
+  s->planned_weight_bytes = parent->planned_weight_bytes;
+  s->planned_gpu_resident_weight_bytes = parent->planned_gpu_resident_weight_bytes;
+  s->planned_gpu_staged_weight_bytes = parent->planned_gpu_staged_weight_bytes;
+  s->planned_weight_descriptor_count = parent->planned_weight_descriptor_count;
+  s->planned_weight_descriptor_hash = parent->planned_weight_descriptor_hash;
+  s->resident_weight_bytes = parent->resident_weight_bytes;
+  s->weights = parent->weights;
+  s->weights->refs.fetch_add(1);
+  s->emb = parent->emb;
+  s->final_norm = parent->final_norm;
+  s->lm_head = parent->lm_head;
+  s->layer = parent->layer;
+
+  hipError_t err = setup_state(s, &out->failure_stage);
+  uint64_t syncs = 1;
+  if (err == hipSuccess && clone) {
+    err = hipStreamSynchronize(parent->stream);
+    syncs += 1;
+    memcpy(s->host_slots, parent->host_slots, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot));
+    const uint64_t kv_half = s->kv_bytes / 2;
+    auto copy = [&](void *dst, const void *src, uint64_t bytes) {
+      if (err == hipSuccess) err = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s->stream);
+    };
+    copy(s->prompt, parent->prompt, static_cast<uint64_t>(s->max_ctx) * 4);
+    copy(s->slots, parent->slots, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot));
+    copy(s->state, parent->state, 64);
+    copy(s->kc, parent->kc, kv_half);
+    copy(s->vc, parent->vc, kv_half);
+    copy(s->sampler_dev, parent->sampler_dev, sizeof(SamplerDev));
+    // the chain kernel's barrier epochs continue from where the sequence stands
+    if (s->chain && parent->chain) copy(s->chain_flags, parent->chain_flags, chain_flag_bytes());
+    s->sampler = parent->sampler;
+    s->prompt_count = parent->prompt_count;
+    s->has_eos = parent->has_eos;
+    s->eos = parent->eos;
+    s->seed_token = parent->seed_token;
+    s->observed = parent->observed;
+    s->cursor = parent->cursor;
+    s->started = parent->started;
+    s->finished = parent->finished;
+    if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
+  }
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    destroy_session(s);
+    return -1;
+  }
+  out->failure_stage = 0;
+  fill_create_result(s, out);
+  out->sync_calls = syncs;
+  out->status = 0;
+  *session_out = s;
+  return 0;
+}
+
+int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenceBatchAdvanceRequest *request,
+                                                   NervaHipHfDecodeSequenceBatchAdvanceResult *out) {
+  if (!begin_result(out)) return -1;
+  out->reason = NERVA_HIP_BATCH_INVALID_REQUEST;
+  if (request == nullptr) return -1;
+  out->requested_session_count = request->session_count;
+  out->target_block_tokens = request->target_block_tokens == 0 ? 1u : request->target_block_tokens;
+  out->min_block_tokens = request->min_block_tokens == 0 ? 1u : request->min_block_tokens;
+  if (request->session_count == 0) {
+    out->reason = NERVA_HIP_BATCH_NO_SESSIONS;
+    out->status = 0;
+    return 0;
+  }
+  if (request->sessions == nullptr || request->output_tokens == nullptr ||
+      request->output_token_capacity < request->session_count)
+    return -1;
+  if (!device_ready(&out->hip_error)) return -1;
+  out->device_count = 1;
+
+  // session_api_batch_fork_destroy.inc.cu:33-45: everything computed so far has been handed out
+  auto ready = [](const Session *q) {
+    return q != nullptr && q->started && !q->finished && q->prompt_count != 0 && q->cursor < q->max_ctx &&
+           static_cast<uint64_t>(q->prompt_count) + q->observed == static_cast<uint64_t>(q->cursor) + 1u;
+  };
+  // :46-61: same weights by descriptor hash, same dimensions
+  auto same_model = [](const Session *a, const Session *b) {
+    return a->planned_weight_descriptor_hash != 0 && a->planned_weight_descriptor_hash == b->planned_weight_descriptor_hash &&
+           a->dtype == b->dtype && a->hidden == b->hidden && a->heads == b->heads && a->kv_heads == b->kv_heads &&
+           a->head_dim == b->head_dim && a->intermediate == b->intermediate && a->vocab == b->vocab &&
+           a->layers == b->layers && a->resident_weight_bytes == b->resident_weight_bytes;
+  };
+  uint32_t ready_count = 0;
+  bool any_hash = false;
+  for (uint32_t i = 0; i < request->session_count; ++i) {
+    const Session *q = request->sessions[i];
+    if (!ready(q)) continue;
+    ready_count += 1;
+    any_hash = any_hash || q->planned_weight_descriptor_hash != 0;
+  }
+  if (ready_count == 0) {
+    out->reason = NERVA_HIP_BATCH_NO_READY_SESSIONS;
+    out->status = 0;
+    return 0;
+  }
+  if (!any_hash) {
+    out->reason = NERVA_HIP_BATCH_SHARED_WEIGHTS_UNPROVEN;
+    out->status = 0;
+    return 0;
+  }
+  Session *lead = nullptr;
+  uint32_t lead_count = 0;
+  for (uint32_t i = 0; i < request->session_count; ++i) {
+    Session *candidate = request->sessions[i];
+    if (!ready(candidate) || candidate->planned_weight_descriptor_hash == 0) continue;
+    uint32_t compatible = 0;
+    for (uint32_t j = 0; j < request->session_count; ++j)
+      if (ready(request->sessions[j]) && same_model(candidate, request->sessions[j])) compatible += 1;
+    if (compatible > lead_count) {
+      lead = candidate;
+      lead_count = compatible;
+    }
+  }
+  out->eligible_session_count = lead_count;
+  if (lead == nullptr || lead_count < out->min_block_tokens) {
+    out->reason = NERVA_HIP_BATCH_INSUFFICIENT_COMPATIBLE_READY;
+    out->status = 0;
+    return 0;
+  }
+  const uint32_t max_tokens = std::min<uint32_t>(out->target_block_tokens, NERVA_HIP_BATCH_MAX_BLOCK_TOKENS);
+  uint32_t picked[NERVA_HIP_BATCH_MAX_BLOCK_TOKENS];
+  Session *seqs[NERVA_HIP_BATCH_MAX_BLOCK_TOKENS];
+  uint32_t T = 0;
+  for (uint32_t i = 0; i < request->session_count && T < max_tokens; ++i) {
+    Session *q = request->sessions[i];
+    if (!ready(q) || !same_model(lead, q)) continue;
+    bool twice = false;  // a session listed twice advances once
+    for (uint32_t t = 0; t < T; ++t) twice = twice || seqs[t] == q;
+    if (twice) continue;
+    picked[T] = i;
+    seqs[T] = q;
+    T += 1;
+  }
+  if (T < out->min_block_tokens) {
+    out->reason = NERVA_HIP_BATCH_INSUFFICIENT_COMPATIBLE_READY;
+    out->status = 0;
+    return 0;
+  }
+  out->reason = NERVA_HIP_BATCH_READY;
+  out->exact = 1;
+  out->block_tokens = T;
+  out->dtype = lead->dtype;
+  out->layer_count = lead->layers;
+
+  const uint64_t allocs_before = allocation_count();
+  hipError_t err = hipSuccess;
+  // work the sequences queued on their own streams comes first
+  for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
+    if (seqs[t] == lead) continue;
+    err = hipStreamSynchronize(seqs[t]->stream);
+    out->sync_calls += 1;
+  }
+  const bool shared = lead->rows_ready && lead->blogits != nullptr;
+  out->shared_weight_stream = shared ? 1u : 0u;
+  if (err == hipSuccess && shared) {
+    err = hipEventRecord(lead->ev0, lead->stream);
+    if (err == hipSuccess) err = enqueue_batch_step(lead, seqs, T, out);
+    if (err == hipSuccess) err = hipEventRecord(lead->ev1, lead->stream);
+    for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
+      Session *q = seqs[t];
+      err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
+                           lead->stream);
+      out->d2h_bytes += sizeof(Slot);
+    }
+    if (err == hipSuccess) err = hipStreamSynchronize(lead->stream);
+    out->sync_calls += 1;
+    if (err == hipSuccess) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, lead->ev0, lead->ev1) == hipSuccess && ms > 0.0f)
+        out->projection_elapsed_ns = std::max<uint64_t>(1, static_cast<uint64_t>(static_cast<double>(ms) * 1e6));
+    }
+  } else if (err == hipSuccess) {
+    // shapes outside the multi-row kernels: every sequence runs its own captured step on its own stream
+    NervaHipHfDecodeSequenceResult scratch{};
+    for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
+      Session *q = seqs[t];
+      err = ensure_graph(q, decode_graph(q), &scratch);
+      if (err == hipSuccess) err = launch_step(q, decode_graph(q), &scratch);
+      if (err == hipSuccess)
+        err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
+                             q->stream);
+      out->d2h_bytes += sizeof(Slot);
+      out->pack_kernel_launches += 1;
+      out->projection_kernel_launches += 4ull * q->layers + 1;
+      out->dependency_kernel_launches += q->layers;
+      out->sampling_kernel_launches += q->sampler.mode == kSamplerGreedy ? 1 : 2;
+    }
+    for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
+      err = hipStreamSynchronize(seqs[t]->stream);
+      out->sync_calls += 1;
+      if (err == hipSuccess) err = chain_verdict(seqs[t]);
+    }
+  }
+  out->hot_path_allocations = allocation_count() - allocs_before;
+  if (err != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(err);
+    out->exact = 0;
+    return -1;
+  }
+  uint32_t observed[NERVA_HIP_BATCH_MAX_BLOCK_TOKENS];
+  for (uint32_t t = 0; t < T; ++t) {
+    Session *q = seqs[t];
+    const uint32_t at = q->cursor;  // = prompt_count - 1 + observed
+    const Slot &slot = q->host_slots[at];
+    if (!slots_consistent(&slot, 1, at)) {
+      out->status = -1;
+      return -1;
+    }
+    request->output_tokens[picked[t]] = slot.token;
+    observed[t] = slot.token;
+    out->last_token = slot.token;
+    q->observed += 1;
+    q->cursor += 1;
+    q->finished = (q->has_eos != 0 && slot.token == q->eos) || at + 1u >= q->max_ctx;
+    out->observed_tokens += 1;
+  }
+  out->observed_token_hash = fnv1a_bytes(observed, static_cast<size_t>(T) * 4);
+  out->status = out->observed_tokens == out->block_tokens ? 0 : -1;
+  return out->status == 0 ? 0 : -1;
+}
 
 int nerva_hip_hf_decode_sequence_session_create(const NervaHipHfDecodeSequenceSessionCreateRequest *request,
                                                 NervaHipHfDecodeSequenceSessionCreateResult *out,

@@ -34,8 +34,9 @@ struct GemmRowsParams {
   uint32_t round_out;        // kGemmResidual: round the sum to 16 bit
 };
 
-// rows % 16 == 0, cols % 2048 == 0 (each of the 8 waves walks whole 256-column blocks),
-// 1 <= tokens <= kGemmMaxTokens, 16-byte aligned w and x16.
+// rows >= 16 (any count: the last workgroup overlaps its neighbour, so with a row count that is no
+// multiple of 16 a residual must not be added in place), cols % 2048 == 0 (each of the 8 waves walks
+// whole 256-column blocks), 1 <= tokens <= kGemmMaxTokens, 16-byte aligned w and x16.
 bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens);
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream);
 

@@ -46,7 +46,9 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   uint16_t *tile = reinterpret_cast<uint16_t *>(smem) + static_cast<size_t>(wave) * NR * kTileElems;
   const uint32_t cols = p.cols, T = p.tokens;
-  const uint32_t row0 = blockIdx.x * 16u;
+  // the last workgroup of a row count that is no multiple of 16 moves back to the last 16 rows: the
+  // rows it shares with its neighbour are computed and stored twice, with the same value
+  const uint32_t row0 = min(blockIdx.x * 16u, p.rows - 16u);
   const uint32_t kper = cols / kGW, nblk = kper / kKB, kbase = wave * kper;
 
   // W block -> registers: instruction i covers rows 2i and 2i + 1, 32 lanes x 16 B each
@@ -195,7 +197,7 @@ hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI>), dim3(p.rows / 16), dim3(kGThreads), lds, stream, p);
+  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI>), dim3((p.rows + 15) / 16), dim3(kGThreads), lds, stream, p);
   return hipGetLastError();
 }
 
@@ -214,8 +216,7 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 }  // namespace
 
 bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens) {
-  return rows != 0 && rows % 16 == 0 && cols != 0 && cols % (kGW * kKB) == 0 && tokens >= 1 &&
-         tokens <= kGemmMaxTokens;
+  return rows >= 16 && cols != 0 && cols % (kGW * kKB) == 0 && tokens >= 1 && tokens <= kGemmMaxTokens;
 }
 
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream) {
@@ -223,6 +224,8 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
   if (!aligned16(p.w) || !aligned16(p.x16)) return hipErrorInvalidValue;
   if ((epilogue == kGemmF32 || epilogue == kGemmResidual) && p.out_f32 == nullptr) return hipErrorInvalidValue;
   if (epilogue == kGemmResidual && p.residual == nullptr) return hipErrorInvalidValue;
+  // rows shared by the last two workgroups are written twice: an in-place residual would be added twice
+  if (epilogue == kGemmResidual && p.rows % 16 != 0 && p.residual == p.out_f32) return hipErrorInvalidValue;
   if (epilogue == kGemmSwiglu && p.out16 == nullptr) return hipErrorInvalidValue;
   if (dtype == kBF16) return launch_dt<kBF16>(epilogue, p, stream);
   if (dtype == kF16) return launch_dt<kF16>(epilogue, p, stream);

@@ -81,13 +81,17 @@ class DecodeSession:
         return cls(handle, res, weights.vocab, weights.kv_heads * weights.head_dim)
 
     @classmethod
-    def create_synthetic(cls, cfg, max_context, seed=0x4E45525641, weight_std=0.02, qk_norm=True):
+    def create_synthetic(cls, cfg, max_context, seed=0x4E45525641, weight_std=0.02, qk_norm=True,
+                         weight_hash=0):
+        """Session over device-generated weights. `weight_hash` stands in for the weight-plan
+        descriptor hash by which batch steps recognise sessions of the same model."""
         lib = abi.load()
         req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
         req.dtype, req.hidden, req.heads, req.kv_heads = cfg["dtype"], cfg["hidden"], cfg["heads"], cfg["kv_heads"]
         req.head_dim, req.intermediate, req.vocab_size = cfg["head_dim"], cfg["intermediate"], cfg["vocab"]
         req.layer_count, req.max_context_tokens = cfg["layers"], max_context
         req.rms_eps, req.rope_theta = cfg["rms_eps"], cfg["rope_theta"] or 0.0
+        req.planned_weight_descriptor_hash = weight_hash
         res = abi.NervaHipHfDecodeSequenceSessionCreateResult()
         handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
         rc = lib.nerva_hip_bench_session_create_synthetic(C.byref(req), seed, weight_std, int(qk_norm),
@@ -96,6 +100,41 @@ class DecodeSession:
             raise RuntimeError("synthetic session_create failed: status=%d hip_error=%d stage=%d"
                                % (res.status, res.hip_error, res.failure_stage))
         return cls(handle, res, cfg["vocab"], cfg["kv_heads"] * cfg["head_dim"])
+
+    def fork_shared_weights(self, detailed_profile=False):
+        """A second session on this one's resident weights (request.rs:380-407); carries a sequence
+        that is under way over to the child."""
+        req = abi.NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest()
+        req.parent, req.detailed_profile = self.handle, int(detailed_profile)
+        res = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+        handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+        rc = self.lib.nerva_hip_hf_decode_sequence_session_fork_shared_weights(C.byref(req), C.byref(res),
+                                                                               C.byref(handle))
+        if rc != 0:
+            raise RuntimeError("session fork failed: status=%d hip_error=%d stage=%d"
+                               % (res.status, res.hip_error, res.failure_stage))
+        return DecodeSession(handle, res, self.vocab, self.kv_hidden)
+
+    BATCH_REASONS = ("ready", "invalid_request", "no_sessions", "no_ready_sessions", "shared_weights_unproven",
+                     "insufficient_compatible_ready")
+
+    @staticmethod
+    def batch_advance_one(sessions, target_block_tokens, min_block_tokens):
+        """One more token for every ready session of the same model (request.rs:575-597). Returns
+        (rc, result, tokens) with tokens[i] = 0xFFFFFFFF for sessions that did not advance."""
+        lib = abi.load()
+        handles = (C.POINTER(abi.NervaHipHfDecodeSequenceSession) * max(len(sessions), 1))()
+        for i, sess in enumerate(sessions):
+            handles[i] = sess.handle
+        tokens = np.full(max(len(sessions), 1), 0xFFFFFFFF, np.uint32)
+        req = abi.NervaHipHfDecodeSequenceBatchAdvanceRequest()
+        req.sessions = handles
+        req.session_count = len(sessions)
+        req.target_block_tokens, req.min_block_tokens = target_block_tokens, min_block_tokens
+        req.output_tokens, req.output_token_capacity = tokens.ctypes.data, len(sessions)
+        res = abi.NervaHipHfDecodeSequenceBatchAdvanceResult()
+        rc = lib.nerva_hip_hf_decode_sequence_batch_advance_one(C.byref(req), C.byref(res))
+        return rc, res, tokens[:len(sessions)]
 
     def start(self, prompt, eos=None, sampler=None):
         prompt = np.ascontiguousarray(prompt, np.uint32)

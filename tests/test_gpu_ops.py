@@ -122,6 +122,7 @@ def test_gemv_rmsnorm_prologue(dtype, cols, rows):
 
 @pytest.mark.parametrize("dtype", [BF16, F16])
 @pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 1), (48, 2048, 5), (32, 4096, 16), (16, 2048, 17),
+                                               (1000, 2048, 9), (25, 2048, 32),   # row counts off the 16-row grid
                                                (6144, 4096, 32), (4096, 12288, 31)])
 def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
     """Multi-row projection on the matrix cores: every token row equals the oracle's GEMV of that row
@@ -175,9 +176,11 @@ def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
 
 def test_gemm_rows_rejects_unsupported_shapes():
     w, x, y = N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16)
-    for rows, cols, tokens in ((24, 2048, 4), (16, 1024, 4), (16, 2048, 33), (16, 2048, 0)):
+    for rows, cols, tokens in ((8, 2048, 4), (16, 1024, 4), (16, 2048, 33), (16, 2048, 0)):
         with pytest.raises(RuntimeError):
             N.gemm_rows(BF16, w, rows, cols, tokens, x, out_f32=y)
+    with pytest.raises(RuntimeError):      # rows off the 16-row grid: no residual added in place
+        N.gemm_rows(BF16, w, 24, 2048, 4, x, epilogue=1, residual=y, out_f32=y)
 
 
 @pytest.mark.parametrize("full", [False, True])

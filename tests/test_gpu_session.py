@@ -579,3 +579,176 @@ def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
     assert rel_l2(results["blocks"][0], results["walk"][0]) <= E2E_REL_L2
     assert results["blocks"][1][0] == results["walk"][1][0] or \
         np.sort(ref_logits)[-1] - np.sort(ref_logits)[-2] < E2E_REL_L2 * np.max(np.abs(ref_logits))
+
+
+# ---- sessions on shared weights: fork, and one decode step for a batch of them -------------------
+
+WEIGHT_HASH = 0x5EED5EED
+
+
+def started(session, prompt, sampler=None):
+    """start + the advance(1) that hands out the token start computed: the state a batch step takes."""
+    rc, _ = session.start(prompt, sampler=sampler)
+    assert rc == 0
+    rc, _, first = session.advance(1)
+    assert rc == 0
+    return int(first[0])
+
+
+def oracle_follow(omodel, max_ctx, prompt, produced):
+    """Oracle context that walked the prompt (prompt staging) and then the tokens a device produced
+    (decode staging): its K/V rows and logits are what a device at the same history must hold."""
+    ctx = O.Context(omodel, max_ctx, staging=1)
+    for t in prompt:
+        ctx.forward_token(int(t), prompt_token=True, want_logits=False)
+    margins = []
+    for t in produced:
+        ctx.forward_token(int(t), prompt_token=False, want_logits=True)
+        top = np.sort(ctx.logits())
+        margins.append(float(top[-1] - top[-2]))
+    return ctx, margins
+
+
+@pytest.mark.parametrize("geom", [GEOMETRIES[5], GEOMETRIES[6]])
+def test_batch_advance_one_matches_solo_sessions_and_oracle(geom):
+    """Five sessions on one set of resident weights (a parent and four forks) at five different
+    positions advance together, one token per call through one stream of the weights. Every sequence
+    must come out as if it had advanced alone: same tokens as a solo session wherever the oracle's
+    margin is clear, and the K/V rows it appended equal to the oracle's for the same token history."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
+    weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 4321, theta, qk_norm, bias)
+    rng = np.random.default_rng(17)
+    prompts = [rng.integers(0, vocab, n).astype(np.uint32) for n in (1, 5, 17, 33, 40)]
+    steps, max_ctx = 6, 64
+    parent = N.DecodeSession.create(weights, max_ctx, planned_weight_descriptor_hash=WEIGHT_HASH)
+    sessions = [parent] + [parent.fork_shared_weights() for _ in range(4)]
+    for child in sessions[1:]:
+        assert child.create_result.resident_weight_bytes == parent.create_result.resident_weight_bytes
+        assert child.create_result.planned_weight_descriptor_hash == WEIGHT_HASH
+    streams = [[started(s, p)] for s, p in zip(sessions, prompts)]
+    for step in range(steps):
+        rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 32, 2)
+        assert rc == 0 and res.status == 0 and res.reason == abi.NERVA_HIP_BATCH_READY and res.exact == 1
+        assert res.block_tokens == 5 and res.eligible_session_count == 5 and res.observed_tokens == 5
+        assert res.shared_weight_stream == 1 and res.hot_path_allocations == 0
+        assert res.projection_kernel_launches == 4 * layers + 1 and res.dependency_kernel_launches == layers
+        assert res.scatter_kernel_launches == layers and res.sampling_kernel_launches == 2 * 5
+        assert res.observed_token_hash == O.fnv1a(tokens) and res.last_token == tokens[-1]
+        assert res.layer_count == layers and res.dtype == dtype and res.projection_elapsed_ns > 0
+        for stream, tok in zip(streams, tokens):
+            stream.append(int(tok))
+    # solo: a sixth session on the same weights walks each prompt alone
+    solo = parent.fork_shared_weights()
+    scale = None
+    for prompt, stream, sess in zip(prompts, streams, sessions):
+        rc, _ = solo.start(prompt)
+        assert rc == 0
+        rc, _, alone = solo.advance(steps + 1)
+        assert rc == 0
+        ctx, margins = oracle_follow(omodel, max_ctx, prompt, stream[:-1])
+        scale = float(np.max(np.abs(ctx.logits())))
+        for i in range(steps + 1):
+            if stream[i] != int(alone[i]):
+                # the histories part here; before that the oracle's margin must have been thin
+                assert i >= 1 and margins[i - 1] <= E2E_REL_L2 * scale, (len(prompt), i, stream, alone.tolist())
+                break
+        # K/V rows the batch steps appended (positions P .. P + steps - 1) against the oracle on this history
+        P = len(prompt)
+        for layer in range(layers):
+            for token in (P - 1, P, P + steps - 1):
+                gk, gv = sess.kv_row(layer, token)
+                rk, rv = ctx.read_kv16(layer, token)
+                tol = 2e-3 if layer == 0 else E2E_REL_L2
+                assert rel_l2(O.decode16(dtype, gk), O.decode16(dtype, rk)) <= tol, (P, layer, token)
+                assert rel_l2(O.decode16(dtype, gv), O.decode16(dtype, rv)) <= tol, (P, layer, token)
+        ctx.close()
+    # sessions go on alone after batch steps, and back
+    rc, res, more = sessions[2].advance(2)
+    assert rc == 0 and res.observed_tokens == 2
+    rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 32, 2)
+    assert rc == 0 and res.block_tokens == 5
+    solo.destroy()
+    for s in sessions[1:] + sessions[:1]:     # children first or last: the weights outlive the parent either way
+        s.destroy()
+
+
+def test_fork_carries_a_running_sequence_and_weights_outlive_the_parent():
+    """A fork taken in mid-sequence continues exactly like its parent (same cache, slots, cursor and
+    sampler), both independently; destroying the parent first leaves the child's weights in place."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[0]
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 99, theta, qk_norm, bias)
+    prompt = np.random.default_rng(3).integers(0, vocab, 9).astype(np.uint32)
+    cfg = abi.NervaHipHfDecodeSamplerConfig()
+    cfg.temperature, cfg.top_p, cfg.top_k, cfg.seed = 0.9, 0.95, 12, 777
+    parent = N.DecodeSession.create(weights, 48)
+    rc, _ = parent.start(prompt, sampler=cfg)
+    assert rc == 0
+    rc, _, head = parent.advance(5)
+    assert rc == 0
+    child = parent.fork_shared_weights()
+    rc, _, a = parent.advance(7)
+    assert rc == 0
+    parent.destroy()
+    rc, _, b = child.advance(7)
+    assert rc == 0
+    assert a.tolist() == b.tolist()           # same seed and positions: the same draws
+    # the child's cache holds the parent's rows
+    rc, _ = child.start(prompt)
+    assert rc == 0
+    child.destroy()
+
+
+def test_batch_advance_one_eligibility_and_reasons():
+    """The planning rules of the reference's batch step: what counts as ready, how sessions are
+    grouped, what is reported when nothing runs."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[0]
+    weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 5, theta, qk_norm, bias)
+    reasons = N.DecodeSession.BATCH_REASONS
+    rc, res, _ = N.DecodeSession.batch_advance_one([], 8, 2)
+    assert rc == 0 and res.status == 0 and reasons[res.reason] == "no_sessions"
+    hashed = N.DecodeSession.create(weights, 24, planned_weight_descriptor_hash=WEIGHT_HASH)
+    twin = hashed.fork_shared_weights()
+    other = N.DecodeSession.create(weights, 24, planned_weight_descriptor_hash=WEIGHT_HASH + 1)
+    plain = N.DecodeSession.create(weights, 24)
+    rc, res, _ = N.DecodeSession.batch_advance_one([hashed, twin], 8, 2)
+    assert rc == 0 and reasons[res.reason] == "no_ready_sessions"            # nothing started
+    rc, _ = hashed.start([1, 2, 3])
+    assert rc == 0
+    rc, res, _ = N.DecodeSession.batch_advance_one([hashed, twin], 8, 1)
+    assert reasons[res.reason] == "no_ready_sessions"                        # first token not handed out yet
+    rc, _, _ = hashed.advance(1)
+    first_plain = started(plain, [4, 5])
+    rc, res, _ = N.DecodeSession.batch_advance_one([plain], 8, 1)
+    assert rc == 0 and reasons[res.reason] == "shared_weights_unproven"      # no descriptor hash
+    rc, res, _ = N.DecodeSession.batch_advance_one([hashed, plain], 8, 2)
+    assert rc == 0 and reasons[res.reason] == "insufficient_compatible_ready" and res.eligible_session_count == 1
+    started(twin, [7])
+    started(other, [9, 9])
+    # shapes outside the multi-row kernels (hidden 512): every sequence runs its own step, same contract
+    rc, res, tokens = N.DecodeSession.batch_advance_one([other, plain, hashed, twin], 8, 2)
+    assert rc == 0 and reasons[res.reason] == "ready" and res.block_tokens == 2 and res.shared_weight_stream == 0
+    assert tokens[0] == 0xFFFFFFFF and tokens[1] == 0xFFFFFFFF and tokens[2] < vocab and tokens[3] < vocab
+    # the step is the one a solo advance would have made
+    ctx = O.Context(omodel, 24, staging=1)
+    otokens, margins = ctx.greedy_decode(np.array([1, 2, 3], np.uint32), 2)
+    scale = float(np.max(np.abs(ctx.logits())))
+    assert tokens[2] == otokens[1] or min(margins[0], margins[1]) <= E2E_REL_L2 * scale
+    # target_block_tokens caps the group in request order; a session listed twice advances once
+    rc, res, tokens = N.DecodeSession.batch_advance_one([hashed, hashed, twin], 1, 1)
+    assert rc == 0 and res.block_tokens == 1 and tokens[0] < vocab and tokens[2] == 0xFFFFFFFF
+    # capacity too small / null pointers
+    lib = abi.load()
+    req = abi.NervaHipHfDecodeSequenceBatchAdvanceRequest()
+    req.session_count = 2
+    out = abi.NervaHipHfDecodeSequenceBatchAdvanceResult()
+    assert lib.nerva_hip_hf_decode_sequence_batch_advance_one(C.byref(req), C.byref(out)) == -1
+    assert reasons[out.reason] == "invalid_request"
+    assert lib.nerva_hip_hf_decode_sequence_batch_advance_one(None, C.byref(out)) == -1
+    # a finished session (context full) drops out
+    for _ in range(40):
+        rc, res, _ = N.DecodeSession.batch_advance_one([hashed, twin], 8, 1)
+        if reasons[res.reason] != "ready":
+            break
+    assert reasons[res.reason] == "no_ready_sessions"
+    for s in (hashed, twin, other, plain):
+        s.destroy()
