@@ -136,6 +136,9 @@ def main():
     ap.add_argument("--layers", type=int, default=36, help="(debug) fewer layers = NOT the named workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-layers", type=int, default=2)
+    ap.add_argument("--batch-sessions", type=int, default=32,
+                    help="sessions advanced together in the shared-weights leg (0 = skip it)")
+    ap.add_argument("--batch-steps", type=int, default=24)
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also launch one plain copy kernel of this size (memory-counter calibration runs)")
     args = ap.parse_args()
@@ -153,7 +156,9 @@ def main():
     cfg["layers"] = args.layers
     max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16   # + the CPU leg's parity token
     t0 = time.time()
-    session = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=WEIGHT_STD, qk_norm=True)
+    max_ctx += args.batch_steps + 4
+    session = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=WEIGHT_STD, qk_norm=True,
+                                               weight_hash=SEED)
     log("[bench] %s: session created in %.1f s, arena %.2f GB (weights %.2f GB, KV %.2f GB)" % (
         smoke.gpu_name.decode(), time.time() - t0, session.create_result.device_arena_bytes / 1e9,
         session.create_result.resident_weight_bytes / 1e9, session.create_result.resident_kv_bytes / 1e9))
@@ -238,11 +243,45 @@ def main():
     latency = dict(p50=round(rank(0.50), 4), p95=round(rank(0.95), 4), p99=round(rank(0.99), 4), tokens=len(lat_ms))
     log("[bench] single-token advance(1) latency ms: p50 %.3f  p95 %.3f  p99 %.3f" % (latency["p50"], latency["p95"], latency["p99"]))
 
+    # Sequences on shared weights: forks of the session (each a copy of the running sequence, with a
+    # cache of its own) advance together, one token each per call, through one stream of the weights.
+    # Reported beside the headline figure, never as it: the metric is batch 1.
+    batch = None
+    if args.batch_sessions > 1:
+        t1 = time.time()
+        group = [session] + [session.fork_shared_weights() for _ in range(args.batch_sessions - 1)]
+        fork_s = time.time() - t1
+        for _ in range(3):
+            rc, bres, btok = N.DecodeSession.batch_advance_one(group, args.batch_sessions, 2)
+            assert rc == 0 and bres.block_tokens == len(group), (rc, bres.reason, bres.block_tokens)
+        t1 = time.perf_counter()
+        device_ns = 0
+        for _ in range(args.batch_steps):
+            rc, bres, btok = N.DecodeSession.batch_advance_one(group, args.batch_sessions, 2)
+            assert rc == 0 and bres.block_tokens == len(group) and bres.hot_path_allocations == 0
+            device_ns += bres.projection_elapsed_ns
+        b_elapsed = time.perf_counter() - t1
+        position = args.prompt + args.warmup + args.steps + len(lat) + 3 + args.batch_steps
+        batch = dict(sessions=len(group), context=position, steps=args.batch_steps,
+                     ms_per_step=round(1e3 * b_elapsed / args.batch_steps, 4),
+                     device_ms_per_step=round(device_ns / 1e6 / args.batch_steps, 4),
+                     tok_s=round(len(group) * args.batch_steps / b_elapsed, 1),
+                     shared_weight_stream=int(bres.shared_weight_stream), fork_s=round(fork_s, 2))
+        log("[bench] %d sessions on shared weights at context %d: %.3f ms per batch step (device %.3f) -> %.0f tok/s "
+            "aggregate (%.1fx the single sequence)" % (len(group), position, batch["ms_per_step"],
+                                                       batch["device_ms_per_step"], batch["tok_s"], batch["tok_s"] / tok_s))
+        for child in group[1:]:
+            child.destroy()
+        rc, r1, tokens = session.advance(1)   # the parent goes on alone
+        assert rc == 0
+
     cpu = None
     if not args.no_cpu:
         try:
             threads_all = min(os.cpu_count() or 1, 16)
             position = args.prompt + args.warmup + args.steps + len(lat)   # tokens now in the KV cache
+            if batch is not None:
+                position += 3 + args.batch_steps + 1
             layers_sampled = min(args.cpu_layers, cfg["layers"])
             r = cpu_baseline(session, cfg, position, int(tokens[-1]), layers_sampled, threads_all)
             cpu = dict(value=round(r[1]["tok_s"], 5), unit="tok/s", cores=1, kind="port",
@@ -264,7 +303,7 @@ def main():
                                      % (cfg["layers"], args.prompt, args.steps),
                             prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
-                            per_token_latency_ms=latency, gpu=smoke.gpu_name.decode()),
+                            per_token_latency_ms=latency, shared_weight_sessions=batch, gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)
     print(json.dumps(line), flush=True)
 

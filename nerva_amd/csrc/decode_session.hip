@@ -61,6 +61,7 @@ struct SharedWeights {
 struct BatchTable {
   AttnSeq seq[kGemmMaxTokens];
   const Slot *slots[kGemmMaxTokens];
+  SamplerParams sample[kGemmMaxTokens];
 };
 
 struct StepProfiler {
@@ -1244,7 +1245,28 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     const Session *q = seqs[t];
     host->seq[t] = AttnSeq{q->kc, q->vc, q->table, q->block_count, q->cursor};
     host->slots[t] = q->slots;
+    // slot[position], cursor -> position + 1, with the sequence's own sampler and random-number counter
+    SamplerParams &sp = host->sample[t];
+    sp = SamplerParams{};
+    sp.logits = lead->blogits + static_cast<uint64_t>(t) * lead->vocab;
+    sp.vocab = q->vocab;
+    sp.config = q->sampler_dev;
+    sp.keys = q->sampler_keys;
+    sample_bind_workspace(sp.out, q->sample_ws);
+    sp.out.slots = q->slots;
+    sp.out.cursor_rw = q->state;
+    sp.cursor = q->state;
+    sp.max_steps = q->max_ctx;
     min_blocks = std::min(min_blocks, q->block_count);
+  }
+  // kv_heads x T workgroups per split already fill the chip at T = 32; measured on MI355X (Qwen3-8B
+  // shapes, contexts 128 .. 8192) further splits only add merge work, so: as many as it takes to reach
+  // one workgroup per CU
+  uint32_t batch_splits = std::max<uint32_t>(1u, std::min<uint32_t>(attn_default_splits(lead->kv_heads, min_blocks),
+                                                                   (256u + lead->kv_heads * T - 1) / (lead->kv_heads * T)));
+  if (const char *v = getenv("NERVA_HIP_BATCH_SPLITS")) {
+    const long want = strtol(v, nullptr, 10);
+    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits)) batch_splits = std::min<uint32_t>(static_cast<uint32_t>(want), min_blocks);
   }
   hipError_t err = hipMemcpyAsync(lead->btable, host, sizeof(BatchTable), hipMemcpyHostToDevice, st);
   if (err != hipSuccess) return err;
@@ -1284,7 +1306,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     a.rope_cs = rope_freq != nullptr ? lead->prope : nullptr;
     a.out16 = lead->pattn16;
     a.layer = l;
-    a.splits = attn_default_splits(lead->kv_heads, min_blocks);
+    a.splits = batch_splits;
     a.eps = lead->eps;
     a.tokens = T;
     a.qkv_token_stride = A + 2 * KV;
@@ -1346,20 +1368,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     out->pack_kernel_launches += 1;
     out->projection_kernel_launches += 1;
   }
-  for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
-    // slot[position], cursor -> position + 1, with the sequence's own sampler and random-number counter
-    Session *q = seqs[t];
-    SamplerParams sp{};
-    sp.logits = lead->blogits + static_cast<uint64_t>(t) * lead->vocab;
-    sp.vocab = q->vocab;
-    sp.config = q->sampler_dev;
-    sp.keys = q->sampler_keys;
-    sample_bind_workspace(sp.out, q->sample_ws);
-    sp.out.slots = q->slots;
-    sp.out.cursor_rw = q->state;
-    sp.cursor = q->state;
-    sp.max_steps = q->max_ctx;
-    err = launch_sampler(sp, st);
+  if (err == hipSuccess) {
+    err = launch_sampler_batch(lead->btable->sample, T, lead->vocab, st);
     out->sampling_kernel_launches += 2;
   }
   return err;

@@ -60,5 +60,9 @@ struct SamplerParams {
 };
 // Both kernels on `stream`. vocab <= kSampleMaxBlocks * kSamplerChunk.
 hipError_t launch_sampler(const SamplerParams &p, hipStream_t stream);
+// The same two kernels for `count` sequences in one launch each: batch[i] (device memory) holds what
+// launch_sampler takes for sequence i - its own logits, configuration, workspaces, slots and cursor.
+// All of them over the same vocabulary size.
+hipError_t launch_sampler_batch(const SamplerParams *batch, uint32_t count, uint32_t vocab, hipStream_t stream);
 
 }  // namespace nv

@@ -67,7 +67,9 @@ __device__ __forceinline__ void sort_desc(uint64_t *keys, uint32_t count, uint32
   }
 }
 
-__global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerParams p) {
+// `batch` (device memory) replaces `p` by its entry blockIdx.y: one launch for several sequences.
+__global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerParams p, const SamplerParams *batch) {
+  if (batch != nullptr) p = batch[blockIdx.y];
   __shared__ uint64_t keys[kSamplerChunk];
   __shared__ float red_v[kChunkThreads / kWave];
   __shared__ uint32_t red_i[kChunkThreads / kWave];
@@ -133,7 +135,9 @@ __global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerPara
     p.keys[static_cast<uint64_t>(blockIdx.x) * kSamplerTopKMax + e] = e < want ? keys[e] : 0ull;
 }
 
-__global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerParams p, uint32_t chunks) {
+__global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerParams p, uint32_t chunks,
+                                                                      const SamplerParams *batch) {
+  if (batch != nullptr) p = batch[blockIdx.y];
   __shared__ uint32_t hist[kBins];
   __shared__ uint32_t scan[kSelectThreads];
   __shared__ uint64_t top[kSamplerTopKMax];
@@ -360,10 +364,21 @@ hipError_t launch_sampler(const SamplerParams &p, hipStream_t stream) {
     return hipErrorInvalidValue;
   const uint32_t chunks = sampler_chunks(p.vocab);
   if (chunks > kSampleMaxBlocks) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(sample_chunk_kernel, dim3(chunks), dim3(kChunkThreads), 0, stream, p);
+  hipLaunchKernelGGL(sample_chunk_kernel, dim3(chunks), dim3(kChunkThreads), 0, stream, p, nullptr);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(sample_select_kernel, dim3(1), dim3(kSelectThreads), 0, stream, p, chunks);
+  hipLaunchKernelGGL(sample_select_kernel, dim3(1), dim3(kSelectThreads), 0, stream, p, chunks, nullptr);
+  return hipGetLastError();
+}
+
+hipError_t launch_sampler_batch(const SamplerParams *batch, uint32_t count, uint32_t vocab, hipStream_t stream) {
+  if (batch == nullptr || count == 0 || count > 65535 || vocab == 0) return hipErrorInvalidValue;
+  const uint32_t chunks = sampler_chunks(vocab);
+  if (chunks > kSampleMaxBlocks) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(sample_chunk_kernel, dim3(chunks, count), dim3(kChunkThreads), 0, stream, SamplerParams{}, batch);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(sample_select_kernel, dim3(1, count), dim3(kSelectThreads), 0, stream, SamplerParams{}, chunks, batch);
   return hipGetLastError();
 }
 
