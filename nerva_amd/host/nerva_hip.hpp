@@ -169,6 +169,67 @@ inline std::optional<std::string> validate_loop_start(Span<uint32_t> prompt, uin
 }
 }  // namespace detail
 
+namespace detail {
+// helpers.rs create_summary_from_result: (return code, result struct) -> summary
+inline HipHfDecodeSequenceSessionCreateSummary create_summary_from_result(
+    int rc, const NervaHipHfDecodeSequenceSessionCreateResult &out, const char *what) {
+  HipHfDecodeSequenceSessionCreateSummary s;
+  s.status = status_from(rc, out.status, out.hip_error);
+  s.failure_stage = out.failure_stage;
+  s.hip_error = out.hip_error;
+  s.dtype = out.dtype;
+  s.hidden = out.hidden;
+  s.heads = out.heads;
+  s.kv_heads = out.kv_heads;
+  s.head_dim = out.head_dim;
+  s.intermediate = out.intermediate;
+  s.vocab_size = out.vocab_size;
+  s.layer_count = out.layer_count;
+  s.max_context_tokens = out.max_context_tokens;
+  s.resident_weight_bytes = out.resident_weight_bytes;
+  s.resident_kv_bytes = out.resident_kv_bytes;
+  s.device_arena_bytes = out.device_arena_bytes;
+  s.pinned_host_bytes = out.pinned_host_bytes;
+  s.h2d_bytes = out.h2d_bytes;
+  s.sync_calls = out.sync_calls;
+  s.hot_path_allocations = out.hot_path_allocations;
+  s.device_memory_bandwidth_bps = out.device_memory_bandwidth_bps;
+  if (s.status == SmokeStatus::Unavailable) s.error = "HIP device unavailable";
+  else if (s.status == SmokeStatus::Failed)
+    s.error = std::string("HIP HF decode sequence session ") + what + " failed (hip_error " + std::to_string(out.hip_error) + ")";
+  return s;
+}
+
+// request.rs:1290-1303 projection_batch_reason_name
+inline const char *projection_batch_reason_name(uint32_t reason) {
+  switch (reason) {
+    case NERVA_HIP_BATCH_READY: return "ready";
+    case NERVA_HIP_BATCH_INVALID_REQUEST: return "invalid_request";
+    case NERVA_HIP_BATCH_NO_SESSIONS: return "no_sessions";
+    case NERVA_HIP_BATCH_NO_READY_SESSIONS: return "no_ready_sessions";
+    case NERVA_HIP_BATCH_SHARED_WEIGHTS_UNPROVEN: return "shared_weights_unproven";
+    case NERVA_HIP_BATCH_INSUFFICIENT_COMPATIBLE_READY: return "insufficient_compatible_ready";
+    default: return "unknown";
+  }
+}
+}  // namespace detail
+
+// request.rs:217-248 CudaHfDecodeSequenceBatchAdvanceSummary. tokens[i] belongs to sessions[i] of the
+// call; UINT32_MAX marks a session that did not advance.
+struct HipHfDecodeSequenceBatchAdvanceSummary {
+  SmokeStatus status = SmokeStatus::Failed;
+  std::string reason;
+  bool exact = false, shared_weight_stream = false;
+  uint32_t requested_session_count = 0, eligible_session_count = 0, block_tokens = 0, target_block_tokens = 0,
+           min_block_tokens = 0, dtype = 0, layer_count = 0, observed_tokens = 0, last_token = 0;
+  uint64_t observed_token_hash = 0;
+  std::vector<uint32_t> tokens;
+  uint64_t d2h_bytes = 0, projection_elapsed_ns = 0, pack_kernel_launches = 0, projection_kernel_launches = 0,
+           scatter_kernel_launches = 0, dependency_kernel_launches = 0, sampling_kernel_launches = 0, sync_calls = 0,
+           hot_path_allocations = 0;
+  int32_t hip_error = 0;
+};
+
 class HipHfDecodeSequenceSession;
 
 struct HipHfDecodeSequenceSessionCreateOutput {
@@ -191,6 +252,55 @@ class HipHfDecodeSequenceSession {
   }
   const HipHfDecodeSequenceSessionCreateSummary &create_summary() const { return create_summary_; }
   NervaHipHfDecodeSequenceSession *raw_handle() { return handle_; }
+
+  // request.rs:380-407 fork_shared_weights: a second session on this one's resident weights; a
+  // sequence that is under way is carried over to the child
+  HipHfDecodeSequenceSessionCreateOutput fork_shared_weights(bool detailed_profile = false);
+
+  // request.rs:575-597 batch_advance_one: one more token for every ready session of the same model
+  static HipHfDecodeSequenceBatchAdvanceSummary batch_advance_one(const std::vector<HipHfDecodeSequenceSession *> &sessions,
+                                                                  uint32_t target_block_tokens, uint32_t min_block_tokens) {
+    std::vector<NervaHipHfDecodeSequenceSession *> handles;
+    handles.reserve(sessions.size());
+    for (HipHfDecodeSequenceSession *session : sessions) handles.push_back(session != nullptr ? session->raw_handle() : nullptr);
+    std::vector<uint32_t> tokens(handles.size(), UINT32_MAX);
+    NervaHipHfDecodeSequenceBatchAdvanceRequest rq{};
+    rq.sessions = handles.data();
+    rq.session_count = static_cast<uint32_t>(handles.size());
+    rq.target_block_tokens = target_block_tokens;
+    rq.min_block_tokens = min_block_tokens;
+    rq.output_tokens = tokens.data();
+    rq.output_token_capacity = static_cast<uint32_t>(tokens.size());
+    NervaHipHfDecodeSequenceBatchAdvanceResult out{};
+    const int rc = nerva_hip_hf_decode_sequence_batch_advance_one(&rq, &out);
+    HipHfDecodeSequenceBatchAdvanceSummary s;
+    s.status = rc == 0 && out.status == 0 ? SmokeStatus::Ok : SmokeStatus::Failed;   // request.rs:1251-1255
+    s.reason = detail::projection_batch_reason_name(out.reason);
+    s.exact = out.exact != 0;
+    s.shared_weight_stream = out.shared_weight_stream != 0;
+    s.requested_session_count = out.requested_session_count;
+    s.eligible_session_count = out.eligible_session_count;
+    s.block_tokens = out.block_tokens;
+    s.target_block_tokens = out.target_block_tokens;
+    s.min_block_tokens = out.min_block_tokens;
+    s.dtype = out.dtype;
+    s.layer_count = out.layer_count;
+    s.observed_tokens = out.observed_tokens;
+    s.last_token = out.last_token;
+    s.observed_token_hash = out.observed_token_hash;
+    s.tokens = std::move(tokens);
+    s.d2h_bytes = out.d2h_bytes;
+    s.projection_elapsed_ns = out.projection_elapsed_ns;
+    s.pack_kernel_launches = out.pack_kernel_launches;
+    s.projection_kernel_launches = out.projection_kernel_launches;
+    s.scatter_kernel_launches = out.scatter_kernel_launches;
+    s.dependency_kernel_launches = out.dependency_kernel_launches;
+    s.sampling_kernel_launches = out.sampling_kernel_launches;
+    s.sync_calls = out.sync_calls;
+    s.hot_path_allocations = out.hot_path_allocations;
+    s.hip_error = out.hip_error;
+    return s;
+  }
 
   // request.rs:412-457 run / run_with_sampler: prompt walk + `steps` tokens in one call
   HipHfDecodeSequenceSummary run(Span<uint32_t> prompt, size_t steps, std::optional<uint32_t> eos_token = std::nullopt,
@@ -230,6 +340,10 @@ struct HipHfDecodeSequenceSessionConfig {
   std::vector<HipHfDecodeChainLayer> layers;
   Span<uint16_t> final_norm_weight, lm_head;
   bool detailed_profile = false;
+  // Hash over the descriptors of the caller's weight plan (the reference derives it from
+  // weight_plan / weight_blocks, request.rs:96-99). Sessions whose hashes are non-zero and equal
+  // hold the same weights and may advance as one batch.
+  uint64_t planned_weight_descriptor_hash = 0;
 
   // validation.rs: every span must have exactly the size its shape implies
   std::optional<std::string> validate() const {
@@ -285,38 +399,30 @@ struct HipHfDecodeSequenceSessionConfig {
     rq.final_norm_weight = final_norm_weight.data;
     rq.lm_head = lm_head.data;
     rq.detailed_profile = detailed_profile ? 1u : 0u;
+    rq.planned_weight_descriptor_hash = planned_weight_descriptor_hash;
     NervaHipHfDecodeSequenceSessionCreateResult out{};
     NervaHipHfDecodeSequenceSession *handle = nullptr;
     const int rc = nerva_hip_hf_decode_sequence_session_create(&rq, &out, &handle);
-    HipHfDecodeSequenceSessionCreateSummary &s = result.summary;
-    s.status = status_from(rc, out.status, out.hip_error);
-    s.failure_stage = out.failure_stage;
-    s.hip_error = out.hip_error;
-    s.dtype = out.dtype;
-    s.hidden = out.hidden;
-    s.heads = out.heads;
-    s.kv_heads = out.kv_heads;
-    s.head_dim = out.head_dim;
-    s.intermediate = out.intermediate;
-    s.vocab_size = out.vocab_size;
-    s.layer_count = out.layer_count;
-    s.max_context_tokens = out.max_context_tokens;
-    s.resident_weight_bytes = out.resident_weight_bytes;
-    s.resident_kv_bytes = out.resident_kv_bytes;
-    s.device_arena_bytes = out.device_arena_bytes;
-    s.pinned_host_bytes = out.pinned_host_bytes;
-    s.h2d_bytes = out.h2d_bytes;
-    s.sync_calls = out.sync_calls;
-    s.hot_path_allocations = out.hot_path_allocations;
-    s.device_memory_bandwidth_bps = out.device_memory_bandwidth_bps;
-    if (s.status == SmokeStatus::Unavailable) s.error = "HIP device unavailable";
-    else if (s.status == SmokeStatus::Failed)
-      s.error = "HIP HF decode sequence session create failed (hip_error " + std::to_string(out.hip_error) + ")";
-    if (s.status == SmokeStatus::Ok && handle != nullptr)
-      result.session = std::make_unique<HipHfDecodeSequenceSession>(handle, s);
+    result.summary = detail::create_summary_from_result(rc, out, "create");
+    if (result.summary.status == SmokeStatus::Ok && handle != nullptr)
+      result.session = std::make_unique<HipHfDecodeSequenceSession>(handle, result.summary);
     return result;
   }
 };
+
+inline HipHfDecodeSequenceSessionCreateOutput HipHfDecodeSequenceSession::fork_shared_weights(bool detailed_profile) {
+  HipHfDecodeSequenceSessionCreateOutput result;
+  NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest rq{};
+  rq.parent = handle_;
+  rq.detailed_profile = detailed_profile ? 1u : 0u;
+  NervaHipHfDecodeSequenceSessionCreateResult out{};
+  NervaHipHfDecodeSequenceSession *handle = nullptr;
+  const int rc = nerva_hip_hf_decode_sequence_session_fork_shared_weights(&rq, &out, &handle);
+  result.summary = detail::create_summary_from_result(rc, out, "fork");
+  if (result.summary.status == SmokeStatus::Ok && handle != nullptr)
+    result.session = std::make_unique<HipHfDecodeSequenceSession>(handle, result.summary);
+  return result;
+}
 
 struct HipHfDecodeSequenceLoopStart;
 
@@ -366,6 +472,25 @@ class HipHfDecodeSequenceLoop {
     return s;
   }
   bool finished() const { return finished_; }
+
+  // stateful.rs:153-180: the sessions of these loops advance together; a loop whose new token is its
+  // stop token is finished afterwards
+  static HipHfDecodeSequenceBatchAdvanceSummary batch_advance_one(const std::vector<HipHfDecodeSequenceLoop *> &loops,
+                                                                  uint32_t target_block_tokens, uint32_t min_block_tokens) {
+    std::vector<HipHfDecodeSequenceSession *> sessions;
+    sessions.reserve(loops.size());
+    for (HipHfDecodeSequenceLoop *loop : loops) sessions.push_back(loop != nullptr ? loop->session_ : nullptr);
+    HipHfDecodeSequenceBatchAdvanceSummary summary =
+        HipHfDecodeSequenceSession::batch_advance_one(sessions, target_block_tokens, min_block_tokens);
+    if (summary.status == SmokeStatus::Ok) {
+      for (size_t i = 0; i < loops.size() && i < summary.tokens.size(); ++i) {
+        const uint32_t token = summary.tokens[i];
+        if (token != UINT32_MAX && loops[i] != nullptr)
+          loops[i]->finished_ = loops[i]->eos_token_.has_value() && token == *loops[i]->eos_token_;
+      }
+    }
+    return summary;
+  }
 
  private:
   HipHfDecodeSequenceLoop(HipHfDecodeSequenceSession &session, std::optional<uint32_t> eos_token)

@@ -68,6 +68,13 @@ static void cpu_checks() {
   std::vector<uint32_t> none, outside{7};
   CHECK(detail::validate_loop_start(none, 4).has_value());
   CHECK(detail::validate_loop_start(outside, 4).has_value());
+  // a batch step over nothing is answered without a device (decode_sequence_session.rs:61-86)
+  HipHfDecodeSequenceBatchAdvanceSummary nothing = HipHfDecodeSequenceSession::batch_advance_one({}, 8, 2);
+  CHECK(nothing.status == SmokeStatus::Ok && nothing.reason == "no_sessions" && !nothing.exact);
+  CHECK(nothing.requested_session_count == 0 && nothing.block_tokens == 0 && nothing.observed_tokens == 0);
+  CHECK(nothing.tokens.empty() && nothing.hot_path_allocations == 0);
+  nothing = HipHfDecodeSequenceLoop::batch_advance_one({}, 8, 2);
+  CHECK(nothing.status == SmokeStatus::Ok && nothing.reason == "no_sessions" && nothing.tokens.empty());
   // no device: Unavailable, never a crash, never a silent success
   const HipDeviceSmokeSummary smoke = device_smoke();
   if (smoke.status != SmokeStatus::Ok) {
@@ -125,10 +132,63 @@ static void gpu_checks() {
   }
 }
 
+// decode_sequence_session.rs:253-383, 506-628: two sessions of one model take their second token
+// together; forks share the parent's weights; a loop that meets its stop token in a batch step is
+// finished.
+static void gpu_batch_checks() {
+  KatModel m;
+  HipHfDecodeSequenceSessionConfig config = m.config();
+  config.planned_weight_descriptor_hash = 0x1234;
+  auto created_a = config.create();
+  auto created_b = config.create();
+  CHECK(created_a.session && created_b.session);
+  if (!created_a.session || !created_b.session) return;
+  std::vector<uint32_t> prompt_a{0}, prompt_b{1};
+  // what each sequence does alone: [1, 2, 3] after 0 and [2, 3, 0] after 1
+  CHECK(created_a.session->run(prompt_a, 3).tokens == std::vector<uint32_t>({1, 2, 3}));
+  CHECK(created_b.session->run(prompt_b, 3).tokens == std::vector<uint32_t>({2, 3, 0}));
+  auto loop_a = HipHfDecodeSequenceLoop::start(*created_a.session, prompt_a, std::nullopt);
+  auto loop_b = HipHfDecodeSequenceLoop::start(*created_b.session, prompt_b, 0u);   // stop token 0
+  CHECK(loop_a.loop_state.has_value() && loop_b.loop_state.has_value());
+  if (!loop_a.loop_state || !loop_b.loop_state) return;
+  std::vector<HipHfDecodeSequenceSession *> sessions{created_a.session.get(), created_b.session.get()};
+  // the first token has not been handed out yet: nothing is ready
+  HipHfDecodeSequenceBatchAdvanceSummary batch = HipHfDecodeSequenceSession::batch_advance_one(sessions, 2, 2);
+  CHECK(batch.status == SmokeStatus::Ok && batch.reason == "no_ready_sessions" && !batch.exact);
+  CHECK(loop_a.loop_state->advance(1).tokens == std::vector<uint32_t>({1}));
+  CHECK(loop_b.loop_state->advance(1).tokens == std::vector<uint32_t>({2}));
+  batch = HipHfDecodeSequenceSession::batch_advance_one(sessions, 2, 2);
+  CHECK(batch.status == SmokeStatus::Ok && batch.reason == "ready" && batch.exact);
+  CHECK(batch.block_tokens == 2 && batch.layer_count == 1 && batch.observed_tokens == 2);
+  CHECK(batch.tokens == std::vector<uint32_t>({2, 3}) && batch.last_token == 3 && batch.hot_path_allocations == 0);
+  // through the loops: b meets its stop token and is finished, a goes on
+  std::vector<HipHfDecodeSequenceLoop *> loops{&*loop_a.loop_state, &*loop_b.loop_state};
+  batch = HipHfDecodeSequenceLoop::batch_advance_one(loops, 2, 2);
+  CHECK(batch.status == SmokeStatus::Ok && batch.tokens == std::vector<uint32_t>({3, 0}));
+  CHECK(!loop_a.loop_state->finished() && loop_b.loop_state->finished());
+  batch = HipHfDecodeSequenceLoop::batch_advance_one(loops, 2, 2);
+  CHECK(batch.status == SmokeStatus::Ok && batch.reason == "insufficient_compatible_ready" && batch.eligible_session_count == 1);
+  batch = HipHfDecodeSequenceLoop::batch_advance_one(loops, 2, 1);
+  CHECK(batch.status == SmokeStatus::Ok && batch.reason == "ready" && batch.tokens == std::vector<uint32_t>({0, UINT32_MAX}));
+  // a fork taken in mid-sequence continues like its parent, on the same weights
+  auto forked = created_a.session->fork_shared_weights(false);
+  CHECK(forked.summary.status == SmokeStatus::Ok && forked.session);
+  if (!forked.session) return;
+  CHECK(forked.summary.resident_weight_bytes == created_a.summary.resident_weight_bytes);
+  std::vector<HipHfDecodeSequenceSession *> pair{created_a.session.get(), forked.session.get()};
+  batch = HipHfDecodeSequenceSession::batch_advance_one(pair, 8, 2);
+  CHECK(batch.status == SmokeStatus::Ok && batch.reason == "ready" && batch.tokens == std::vector<uint32_t>({1, 1}));
+  created_a.session.reset();   // the parent goes first: the child keeps the weights
+  CHECK(forked.session->run(prompt_a, 2).tokens == std::vector<uint32_t>({1, 2}));
+}
+
 int main(int argc, char **argv) {
   const std::string mode = argc > 1 ? argv[1] : "cpu";
   cpu_checks();
-  if (mode == "gpu") gpu_checks();
+  if (mode == "gpu") {
+    gpu_checks();
+    gpu_batch_checks();
+  }
   std::printf("%s: %d failure(s)\n", mode.c_str(), failures);
   return failures == 0 ? 0 : 1;
 }
