@@ -92,7 +92,18 @@ typedef struct NervaHipHfDecodeChainLayer {
       deepseek_swiglu_limit;
 } NervaHipHfDecodeChainLayer;
 
-/* mirrors NervaCudaHfDecodeSequenceWeightBlock (nerva_cuda_api.h:380-391) */
+/* mirrors NervaCudaHfDecodeSequenceWeightBlock (nerva_cuda_api.h:380-391): one block of a declared
+ * weight plan. The blocks tile the weight bytes [0, resident_weight_bytes) in the reference's arena
+ * order - embeddings; per layer rms_attn, w_q, [q_norm], w_k, [k_norm], w_v, w_o, rms_mlp, w_gate,
+ * w_up, w_down, [q_bias, k_bias, v_bias, o_bias]; final norm; LM head - and need not follow tensor
+ * boundaries. Source: host memory (host_source) or `bytes` bytes of a file at file_offset_begin
+ * (source_file, not NUL-terminated, source_file_len bytes). A request with planned_weight_blocks or
+ * planned_weight_bytes != 0 declares a plan: it must then hold one descriptor per block and the
+ * FNV-1a-64 hash over (block_id, block_version, offset_bytes, bytes: u64; strategy: u32) of all
+ * of them, the descriptors are THE source of the weights (weights.cu:411-467, 797-908), and the tensor
+ * pointers only mark which optional tensors exist (all others may be null). */
+#define NERVA_HIP_WEIGHT_STRATEGY_GPU_RESIDENT 1u /* weight_plan.rs:3 */
+#define NERVA_HIP_WEIGHT_STRATEGY_GPU_STAGED 2u   /* weight_plan.rs:4 */
 typedef struct NervaHipHfDecodeSequenceWeightBlock {
   const uint16_t *host_source;
   const char *source_file;
@@ -101,8 +112,9 @@ typedef struct NervaHipHfDecodeSequenceWeightBlock {
 } NervaHipHfDecodeSequenceWeightBlock;
 
 /* mirrors NervaCudaHfDecodeSamplerConfig (nerva_cuda_api.h:393-399).
- * Greedy <=> !(temperature > 0) || top_k == 1 (sampler.cu:89). Only greedy is
- * implemented: any other configuration fails start with NOT_SUPPORTED. */
+ * Greedy <=> !(temperature > 0) || top_k == 1 (sampler.cu:89); otherwise Gumbel-max over the whole
+ * vocabulary (top_k == 0 and top_p >= 0.999999) or top-k / top-p with the reference's hash random
+ * numbers. Out-of-range values are normalised like sampler.cu:422-433. */
 typedef struct NervaHipHfDecodeSamplerConfig {
   float temperature, top_p;
   uint32_t top_k, reserved;

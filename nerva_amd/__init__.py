@@ -8,8 +8,8 @@ importing a compute helper without the built library raises.
 from . import abi
 from .runtime import (DeviceBuffer, Device, device_available, gemv, fp8_gemv, paged_attention,
                       argmax, sample, gemm_rows, moe_fp8_experts, moe_route_softmax, PagedKvCache)
-from .session import DecodeSession, ModelWeights, Qwen3_8B
+from .session import DecodeSession, ModelWeights, Qwen3_8B, WeightPlan, hash_weight_blocks
 
 __all__ = ["abi", "DeviceBuffer", "Device", "device_available", "gemv", "fp8_gemv",
            "paged_attention", "argmax", "sample", "gemm_rows", "moe_fp8_experts", "moe_route_softmax", "PagedKvCache",
-           "DecodeSession", "ModelWeights", "Qwen3_8B"]
+           "DecodeSession", "ModelWeights", "Qwen3_8B", "WeightPlan", "hash_weight_blocks"]

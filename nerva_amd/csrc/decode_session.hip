@@ -21,6 +21,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <string>
 #include <atomic>
 #include <vector>
 
@@ -787,6 +788,130 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   return err;
 }
 
+// ---- weights from the caller's plan -----------------------------------------------------------
+// A declared weight plan (weights.cu:157-160) comes with descriptors that tile the weight bytes
+// [0, resident_weight_bytes) in the reference's arena order - embeddings, then per layer rms_attn,
+// w_q, [q_norm], w_k, [k_norm], w_v, w_o, rms_mlp, w_gate, w_up, w_down, [q/k/v/o bias], then the
+// final norm and the LM head (weights.cu:484-591, session_api_lifecycle.inc.cu:124-148) - each with a
+// host-memory or a file source. The descriptors are then THE source of the weights; the tensor
+// pointers of the request only say which optional tensors exist (weights.cu:18-23) and may be null
+// otherwise (weights.cu:237-243). This library keeps [q;k;v] and [gate;up] as row-concatenated
+// matrices elsewhere in its own arena, so a descriptor's byte range is cut along the tensor
+// boundaries of that order and every piece goes to its tensor's place.
+constexpr uint32_t kWeightStrategyGpuResident = 1, kWeightStrategyGpuStaged = 2;  // weight_plan.rs:3-4
+
+struct WeightSegment {
+  uint64_t logical, bytes;  // position in the reference's arena order
+  char *device;
+};
+
+template <typename Request>
+bool weight_plan_declared(const Request *rq) {
+  return rq->planned_weight_blocks != 0 || rq->planned_weight_bytes != 0;
+}
+
+void hash_le(uint64_t &hash, uint64_t value, int bytes) {
+  for (int i = 0; i < bytes; ++i) {
+    hash ^= (value >> (8 * i)) & 0xffu;
+    hash *= 0x00000100000001b3ull;
+  }
+}
+
+bool descriptor_has_file(const NervaHipHfDecodeSequenceWeightBlock &d) {
+  return d.source_file != nullptr && d.source_file_len != 0;
+}
+
+// weights.cu:411-467: contiguous from 0, even offsets and sizes, a source each, a known strategy, and
+// totals, counts and the FNV-1a hash over (block_id, block_version, offset_bytes, bytes, strategy)
+// equal to what the plan declares.
+bool validate_weight_descriptors(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, uint64_t resident_weight_bytes) {
+  uint64_t cursor = 0, hash = 0xcbf29ce484222325ull, resident_bytes = 0, staged_bytes = 0;
+  uint32_t resident_blocks = 0, staged_blocks = 0;
+  for (uint32_t i = 0; i < rq->planned_weight_descriptor_count; ++i) {
+    const NervaHipHfDecodeSequenceWeightBlock &d = rq->planned_weight_descriptors[i];
+    if (d.bytes == 0 || d.reserved != 0 || (d.host_source == nullptr && !descriptor_has_file(d)) ||
+        d.offset_bytes != cursor || d.offset_bytes % 2 != 0 || d.bytes % 2 != 0)
+      return false;
+    if (cursor + d.bytes < cursor) return false;
+    cursor += d.bytes;
+    hash_le(hash, d.block_id, 8);
+    hash_le(hash, d.block_version, 8);
+    hash_le(hash, d.offset_bytes, 8);
+    hash_le(hash, d.bytes, 8);
+    hash_le(hash, d.strategy, 4);
+    if (d.strategy == kWeightStrategyGpuResident) {
+      resident_blocks += 1;
+      resident_bytes += d.bytes;
+    } else if (d.strategy == kWeightStrategyGpuStaged) {
+      staged_blocks += 1;
+      staged_bytes += d.bytes;
+    } else {
+      return false;
+    }
+  }
+  return cursor == resident_weight_bytes && cursor == rq->planned_weight_bytes &&
+         hash == rq->planned_weight_descriptor_hash && resident_blocks == rq->planned_gpu_resident_blocks &&
+         staged_blocks == rq->planned_gpu_staged_blocks && resident_bytes == rq->planned_gpu_resident_weight_bytes &&
+         staged_bytes == rq->planned_gpu_staged_weight_bytes;
+}
+
+// weights.cu:797-908: every descriptor to the device, from memory directly or from its file through a
+// pinned staging buffer. `segments` is sorted and gapless in the reference's order.
+hipError_t copy_weight_descriptors(const NervaHipHfDecodeSequenceSessionCreateRequest *rq,
+                                   const std::vector<WeightSegment> &segments, hipStream_t stream, uint64_t *h2d_bytes,
+                                   uint64_t *sync_calls) {
+  constexpr uint64_t kStagingBytes = 64ull << 20;
+  char *staging = nullptr;
+  hipError_t err = hipSuccess;
+  size_t at = 0;  // descriptors ascend, so the segment cursor only moves forward
+  for (uint32_t i = 0; err == hipSuccess && i < rq->planned_weight_descriptor_count; ++i) {
+    const NervaHipHfDecodeSequenceWeightBlock &d = rq->planned_weight_descriptors[i];
+    FILE *file = nullptr;
+    if (d.host_source == nullptr) {
+      if (staging == nullptr) err = counted_host_malloc(reinterpret_cast<void **>(&staging), kStagingBytes);
+      if (err != hipSuccess) break;
+      const std::string path(d.source_file, d.source_file_len);
+      file = fopen(path.c_str(), "rb");
+      if (file == nullptr) {
+        err = hipErrorInvalidValue;
+        break;
+      }
+    }
+    uint64_t done = 0;
+    while (err == hipSuccess && done < d.bytes) {
+      const uint64_t logical = d.offset_bytes + done;
+      while (at < segments.size() && segments[at].logical + segments[at].bytes <= logical) ++at;
+      if (at == segments.size()) {
+        err = hipErrorInvalidValue;
+        break;
+      }
+      const WeightSegment &seg = segments[at];
+      const uint64_t inside = logical - seg.logical;
+      uint64_t piece = std::min(d.bytes - done, seg.bytes - inside);
+      if (file == nullptr) {
+        err = hipMemcpyAsync(seg.device + inside, reinterpret_cast<const char *>(d.host_source) + done, piece,
+                             hipMemcpyHostToDevice, stream);
+      } else {
+        piece = std::min(piece, kStagingBytes);
+        if (fseeko(file, static_cast<off_t>(d.file_offset_begin + done), SEEK_SET) != 0 ||
+            fread(staging, 1, piece, file) != piece) {
+          err = hipErrorInvalidValue;
+          break;
+        }
+        err = hipMemcpyAsync(seg.device + inside, staging, piece, hipMemcpyHostToDevice, stream);
+        if (err == hipSuccess) err = hipStreamSynchronize(stream);  // the one staging buffer is reused
+        *sync_calls += 1;
+      }
+      done += piece;
+    }
+    if (file != nullptr) fclose(file);
+    *h2d_bytes += done;
+  }
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  if (staging != nullptr) (void)hipHostFree(staging);
+  return err;
+}
+
 // Everything of a session that is not weights, from the dimensions already in `s`: stream, events,
 // the state arena (KV cache, block table, prompt, token slots, cursor words, activations and
 // workspaces), the pinned host mirrors, the step modes. Shared by create and fork.
@@ -1023,14 +1148,21 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
       !isfinite(rq->rms_eps) || !isfinite(rq->rope_theta))
     return -1;
   if (rq->rope_theta > 0.0f && rq->head_dim % 2 != 0) return -1;
+  // with a declared weight plan the descriptors are the source and the tensor pointers may be null
+  const bool declared = !synthetic && weight_plan_declared(rq);
   if (!synthetic) {
-    if (rq->embeddings == nullptr || rq->layers == nullptr || rq->final_norm_weight == nullptr ||
-        rq->lm_head == nullptr)
-      return -1;
-    for (uint32_t l = 0; l < rq->layer_count; ++l)
-      if (!layer_has_weights(rq->layers[l])) return -1;
+    if (rq->layers == nullptr) return -1;
+    if (!declared) {
+      if (rq->embeddings == nullptr || rq->final_norm_weight == nullptr || rq->lm_head == nullptr) return -1;
+      for (uint32_t l = 0; l < rq->layer_count; ++l)
+        if (!layer_has_weights(rq->layers[l])) return -1;
+    }
   }
   if (rq->planned_weight_descriptor_count != 0 && rq->planned_weight_descriptors == nullptr) return -1;
+  // session_api_lifecycle.inc.cu:48-55: a declared plan is complete - one descriptor per block, a hash
+  if (declared && (rq->planned_weight_blocks == 0 || rq->planned_weight_bytes == 0 || rq->planned_weight_descriptors == nullptr ||
+                   rq->planned_weight_descriptor_count != rq->planned_weight_blocks || rq->planned_weight_descriptor_hash == 0))
+    return -1;
   // explicit, never silent: features outside the dense full-attention path are refused
   bool supported = rq->experimental_rt_decode == 0 && rq->head_dim <= 512 &&
                    static_cast<uint64_t>(rq->intermediate) * 2 <= 60 * 1024 &&
@@ -1128,8 +1260,9 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   s->resident_weight_bytes = weight_elems * 2;
   s->weights->bytes = c.offset;
 
-  if (rq->planned_weight_blocks != 0 && rq->planned_weight_bytes != s->resident_weight_bytes) {
-    // session_api_oneshot.inc.cu: a weight plan that disagrees with the arena is rejected
+  if (declared && !validate_weight_descriptors(rq, s->resident_weight_bytes)) {
+    // session_api_lifecycle.inc.cu:156: a weight plan that disagrees with the arena or with its own
+    // descriptors is rejected before anything is allocated
     destroy_session(s);
     return -1;
   }
@@ -1168,7 +1301,39 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
     if (err != hipSuccess || off == kNone) return;
     err = launch_synth_16(wbase + off, s->dtype, seed, tensor_id, elems, mean, weight_std, s->stream);
   };
-  if (synthetic) {
+  uint64_t setup_syncs = 1;
+  if (declared) {
+    // the reference's arena order, piece by piece, onto this library's layout
+    std::vector<WeightSegment> segments;
+    uint64_t logical = 0;
+    auto segment = [&](uint64_t off, uint64_t elems) {
+      if (off == kNone) return;
+      segments.push_back(WeightSegment{logical, elems * 2, wbase + off});
+      logical += elems * 2;
+    };
+    segment(off_emb, V * H);
+    for (uint32_t l = 0; l < L; ++l) {
+      segment(lo[l].rms_attn, H);
+      segment(lo[l].wqkv, A * H);
+      segment(lo[l].q_norm, HD);
+      segment(lo[l].wqkv + A * H * 2, KV * H);
+      segment(lo[l].k_norm, HD);
+      segment(lo[l].wqkv + (A + KV) * H * 2, KV * H);
+      segment(lo[l].wo, H * A);
+      segment(lo[l].rms_mlp, H);
+      segment(lo[l].wgu, I * H);
+      segment(lo[l].wgu + I * H * 2, I * H);
+      segment(lo[l].wdown, H * I);
+      segment(lo[l].q_bias, A);
+      segment(lo[l].k_bias, KV);
+      segment(lo[l].v_bias, KV);
+      segment(lo[l].o_bias, H);
+    }
+    segment(off_final, H);
+    segment(off_lm, V * H);
+    err = logical == s->resident_weight_bytes ? copy_weight_descriptors(rq, segments, s->stream, &h2d, &setup_syncs)
+                                              : hipErrorInvalidValue;
+  } else if (synthetic) {
     fill(off_emb, 1, V * H, 0.0f);
     fill(off_final, 2, H, 1.0f);
     fill(off_lm, 3, V * H, 0.0f);
@@ -1220,7 +1385,7 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   out->failure_stage = 0;
   fill_create_result(s, out);
   out->h2d_bytes = h2d;
-  out->sync_calls = 1;
+  out->sync_calls = setup_syncs;
   out->status = 0;
   *session_out = s;
   return 0;

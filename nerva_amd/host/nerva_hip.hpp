@@ -95,6 +95,71 @@ struct HipHfDecodeChainLayer {
     l.o_bias = o_bias.data;
     return l;
   }
+  // hf_chain/layer.rs:352-399: with a declared weight plan the descriptors carry the data; the request
+  // only says which optional tensors exist
+  NervaHipHfDecodeChainLayer to_descriptor_layout_ffi() const {
+    NervaHipHfDecodeChainLayer l{};
+    l.q_norm_weight = q_norm_weight.data;
+    l.k_norm_weight = k_norm_weight.data;
+    l.q_bias = q_bias.data;
+    l.k_bias = k_bias.data;
+    l.v_bias = v_bias.data;
+    l.o_bias = o_bias.data;
+    return l;
+  }
+};
+
+// weight_plan.rs:3-4
+constexpr uint32_t HIP_HF_WEIGHT_STRATEGY_GPU_RESIDENT = 1, HIP_HF_WEIGHT_STRATEGY_GPU_STAGED = 2;
+using HipHfDecodeSequenceWeightBlock = NervaHipHfDecodeSequenceWeightBlock;   // weight_plan.rs:9-22
+
+// weight_plan.rs:102-126: FNV-1a-64 over (block_id, block_version, offset_bytes, bytes: u64; strategy:
+// u32), little endian, block after block
+inline uint64_t hash_weight_blocks(Span<HipHfDecodeSequenceWeightBlock> descriptors) {
+  uint64_t hash = 0xcbf29ce484222325ull;
+  auto mix = [&hash](uint64_t value, int bytes) {
+    for (int i = 0; i < bytes; ++i) {
+      hash ^= (value >> (8 * i)) & 0xffu;
+      hash *= 0x00000100000001b3ull;
+    }
+  };
+  for (size_t i = 0; i < descriptors.size; ++i) {
+    const HipHfDecodeSequenceWeightBlock &d = descriptors.data[i];
+    mix(d.block_id, 8);
+    mix(d.block_version, 8);
+    mix(d.offset_bytes, 8);
+    mix(d.bytes, 8);
+    mix(d.strategy, 4);
+  }
+  return hash;
+}
+
+// weight_plan.rs:24-100 CudaHfDecodeSequenceWeightPlan
+struct HipHfDecodeSequenceWeightPlan {
+  uint32_t blocks = 0, gpu_resident_blocks = 0, gpu_staged_blocks = 0;
+  uint64_t weight_bytes = 0, gpu_resident_weight_bytes = 0, gpu_staged_weight_bytes = 0, descriptor_hash = 0;
+  bool is_declared() const { return blocks != 0 || weight_bytes != 0; }
+  std::optional<std::string> validate() const {
+    if (!is_declared()) return std::nullopt;
+    if (blocks == 0 || weight_bytes == 0 || descriptor_hash == 0) return "HIP HF decode sequence weight plan is incomplete";
+    if (gpu_resident_blocks > blocks || gpu_staged_blocks > blocks - gpu_resident_blocks)
+      return "HIP HF decode sequence weight block counts are invalid";
+    if (gpu_resident_weight_bytes > weight_bytes || gpu_staged_weight_bytes > weight_bytes - gpu_resident_weight_bytes)
+      return "HIP HF decode sequence weight byte counts are invalid";
+    return std::nullopt;
+  }
+  std::optional<std::string> validate_descriptors(Span<HipHfDecodeSequenceWeightBlock> descriptors) const {
+    if (!is_declared()) return std::nullopt;
+    if (descriptors.size != blocks) return "HIP HF decode sequence weight descriptor count is invalid";
+    for (size_t i = 0; i < descriptors.size; ++i) {
+      const HipHfDecodeSequenceWeightBlock &d = descriptors.data[i];
+      if ((d.host_source == nullptr && (d.source_file == nullptr || d.source_file_len == 0)) || d.offset_bytes % 2 != 0 ||
+          d.bytes % 2 != 0)
+        return "HIP HF decode sequence weight descriptor source is invalid";
+    }
+    if (hash_weight_blocks(descriptors) != descriptor_hash) return "HIP HF decode sequence weight descriptor hash is invalid";
+    return std::nullopt;
+  }
 };
 
 // session/summary.rs: CudaHfDecodeSequenceSessionCreateSummary (fields this backend fills)
@@ -340,10 +405,11 @@ struct HipHfDecodeSequenceSessionConfig {
   std::vector<HipHfDecodeChainLayer> layers;
   Span<uint16_t> final_norm_weight, lm_head;
   bool detailed_profile = false;
-  // Hash over the descriptors of the caller's weight plan (the reference derives it from
-  // weight_plan / weight_blocks, request.rs:96-99). Sessions whose hashes are non-zero and equal
-  // hold the same weights and may advance as one batch.
-  uint64_t planned_weight_descriptor_hash = 0;
+  // request.rs:99-100: a declared plan makes weight_blocks the source of the weights (the tensor spans
+  // then only mark which optional tensors exist and may be empty otherwise). Sessions whose plans
+  // have the same descriptor hash hold the same weights and may advance as one batch.
+  std::optional<HipHfDecodeSequenceWeightPlan> weight_plan;
+  Span<HipHfDecodeSequenceWeightBlock> weight_blocks;
 
   // validation.rs: every span must have exactly the size its shape implies
   std::optional<std::string> validate() const {
@@ -352,6 +418,11 @@ struct HipHfDecodeSequenceSessionConfig {
     if (heads % kv_heads != 0) return "HIP HF decode sequence session requires heads divisible by kv_heads";
     if (max_context_tokens == 0) return "HIP HF decode sequence session requires max_context_tokens";
     if (dtype != NERVA_HIP_DTYPE_F16 && dtype != NERVA_HIP_DTYPE_BF16) return "HIP HF decode sequence session dtype must be f16 or bf16";
+    if (weight_plan.has_value()) {   // validation.rs:53-66: the plan and its descriptors, then no span lengths
+      if (auto e = weight_plan->validate()) return e;
+      if (auto e = weight_plan->validate_descriptors(weight_blocks)) return e;
+      if (weight_plan->is_declared()) return std::nullopt;
+    }
     const size_t a = heads * head_dim, kv = kv_heads * head_dim;
     if (embeddings.size != vocab_size * hidden) return "HIP HF decode sequence embeddings have the wrong size";
     if (lm_head.size != vocab_size * hidden) return "HIP HF decode sequence lm_head has the wrong size";
@@ -381,7 +452,9 @@ struct HipHfDecodeSequenceSessionConfig {
     }
     std::vector<NervaHipHfDecodeChainLayer> ffi_layers;
     ffi_layers.reserve(layers.size());
-    for (const HipHfDecodeChainLayer &l : layers) ffi_layers.push_back(l.to_ffi());
+    const HipHfDecodeSequenceWeightPlan plan = weight_plan.value_or(HipHfDecodeSequenceWeightPlan{});
+    const bool use_descriptors = plan.is_declared();
+    for (const HipHfDecodeChainLayer &l : layers) ffi_layers.push_back(use_descriptors ? l.to_descriptor_layout_ffi() : l.to_ffi());
     NervaHipHfDecodeSequenceSessionCreateRequest rq{};
     rq.dtype = dtype;
     rq.hidden = static_cast<uint32_t>(hidden);
@@ -394,12 +467,20 @@ struct HipHfDecodeSequenceSessionConfig {
     rq.max_context_tokens = static_cast<uint32_t>(max_context_tokens);
     rq.rms_eps = rms_eps;
     rq.rope_theta = rope_theta.value_or(0.0f);
-    rq.embeddings = embeddings.data;
+    rq.embeddings = use_descriptors ? nullptr : embeddings.data;   // helpers.rs:13-19 planned_ptr
     rq.layers = ffi_layers.data();
-    rq.final_norm_weight = final_norm_weight.data;
-    rq.lm_head = lm_head.data;
+    rq.final_norm_weight = use_descriptors ? nullptr : final_norm_weight.data;
+    rq.lm_head = use_descriptors ? nullptr : lm_head.data;
     rq.detailed_profile = detailed_profile ? 1u : 0u;
-    rq.planned_weight_descriptor_hash = planned_weight_descriptor_hash;
+    rq.planned_weight_blocks = plan.blocks;
+    rq.planned_gpu_resident_blocks = plan.gpu_resident_blocks;
+    rq.planned_gpu_staged_blocks = plan.gpu_staged_blocks;
+    rq.planned_weight_bytes = plan.weight_bytes;
+    rq.planned_gpu_resident_weight_bytes = plan.gpu_resident_weight_bytes;
+    rq.planned_gpu_staged_weight_bytes = plan.gpu_staged_weight_bytes;
+    rq.planned_weight_descriptors = weight_blocks.empty() ? nullptr : weight_blocks.data;
+    rq.planned_weight_descriptor_count = static_cast<uint32_t>(weight_blocks.size);
+    rq.planned_weight_descriptor_hash = plan.descriptor_hash;
     NervaHipHfDecodeSequenceSessionCreateResult out{};
     NervaHipHfDecodeSequenceSession *handle = nullptr;
     const int rc = nerva_hip_hf_decode_sequence_session_create(&rq, &out, &handle);

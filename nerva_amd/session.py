@@ -53,6 +53,100 @@ class ModelWeights:
         req.lm_head = self.lm_head.ctypes.data
 
 
+WEIGHT_STRATEGY_GPU_RESIDENT, WEIGHT_STRATEGY_GPU_STAGED = 1, 2    # weight_plan.rs:3-4
+
+_ARENA_ORDER = ("rms_attn", "w_q", "q_norm", "w_k", "k_norm", "w_v", "w_o", "rms_mlp", "w_gate", "w_up", "w_down",
+                "q_bias", "k_bias", "v_bias", "o_bias")
+
+
+def arena_order(weights):
+    """The model's tensors in the order the reference lays its weight arena out, which is the byte
+    space weight descriptors address (weights.cu:484-591, session_api_lifecycle.inc.cu:124-148)."""
+    out = [weights.embeddings]
+    for layer in weights.layers:
+        out += [layer[k] for k in _ARENA_ORDER if layer.get(k) is not None]
+    return out + [weights.final_norm, weights.lm_head]
+
+
+def hash_weight_blocks(blocks):
+    """FNV-1a-64 over (block_id, block_version, offset_bytes, bytes) as u64 and strategy as u32,
+    little endian, block after block (weight_plan.rs:102-126, weights.cu:90-111)."""
+    h = 0xcbf29ce484222325
+    for b in blocks:
+        for value, width in ((b.block_id, 8), (b.block_version, 8), (b.offset_bytes, 8), (b.bytes, 8), (b.strategy, 4)):
+            for i in range(width):
+                h = ((h ^ ((value >> (8 * i)) & 0xFF)) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+class WeightPlan:
+    """A declared weight plan: descriptors that tile the model's weight bytes in arena order, each
+    with a host-memory or a file source, and the totals the session checks them against
+    (weight_plan.rs:24-100)."""
+
+    def __init__(self, blocks, keepalive):
+        self.blocks = (abi.NervaHipHfDecodeSequenceWeightBlock * len(blocks))(*blocks)
+        self._keepalive = keepalive
+        self.descriptor_hash = hash_weight_blocks(blocks)
+
+    @classmethod
+    def from_weights(cls, weights, block_bytes=None, resident_blocks=None, path=None):
+        """block_bytes None: one block per tensor, sourced from the tensor's own memory. Otherwise the
+        arena is cut into blocks of block_bytes (even; the last one shorter) over one contiguous copy
+        of it - in memory, or in the file `path`, which is written here. The first `resident_blocks`
+        blocks are declared GPU-resident, the rest GPU-staged (both end up in device memory)."""
+        tensors = arena_order(weights)
+        keep, blocks, offset = [tensors], [], 0
+        if block_bytes is None:
+            pieces = [(t.ctypes.data, t.nbytes) for t in tensors]
+        else:
+            storage = np.concatenate([t.reshape(-1) for t in tensors])
+            keep.append(storage)
+            total = storage.nbytes
+            pieces = [(storage.ctypes.data + o, min(block_bytes, total - o)) for o in range(0, total, block_bytes)]
+            if path is not None:
+                storage.tofile(path)
+                keep.append(C.create_string_buffer(path.encode()))
+        for index, (address, nbytes) in enumerate(pieces):
+            b = abi.NervaHipHfDecodeSequenceWeightBlock()
+            if path is not None and block_bytes is not None:
+                b.source_file = C.cast(keep[-1], C.c_void_p).value
+                b.source_file_len = len(path.encode())
+                b.file_offset_begin = offset
+            else:
+                b.host_source = address
+            b.block_id, b.block_version, b.offset_bytes, b.bytes = index + 1, 0, offset, nbytes
+            resident = resident_blocks is None or index < resident_blocks
+            b.strategy = WEIGHT_STRATEGY_GPU_RESIDENT if resident else WEIGHT_STRATEGY_GPU_STAGED
+            blocks.append(b)
+            offset += nbytes
+        return cls(blocks, keep)
+
+    def fields(self):
+        resident = [b for b in self.blocks if b.strategy == WEIGHT_STRATEGY_GPU_RESIDENT]
+        staged = [b for b in self.blocks if b.strategy == WEIGHT_STRATEGY_GPU_STAGED]
+        return dict(planned_weight_blocks=len(self.blocks), planned_gpu_resident_blocks=len(resident),
+                    planned_gpu_staged_blocks=len(staged), planned_weight_bytes=sum(b.bytes for b in self.blocks),
+                    planned_gpu_resident_weight_bytes=sum(b.bytes for b in resident),
+                    planned_gpu_staged_weight_bytes=sum(b.bytes for b in staged),
+                    planned_weight_descriptors=self.blocks,
+                    planned_weight_descriptor_count=len(self.blocks),
+                    planned_weight_descriptor_hash=self.descriptor_hash)
+
+
+def descriptor_layout_layers(weights, req):
+    """What a request with a declared weight plan carries instead of tensor pointers
+    (hf_chain/layer.rs:352-399, helpers.rs:13-19): the layer array with only the pointers of the
+    optional tensors left, as markers that they exist; every other tensor pointer null."""
+    req.embeddings = req.final_norm_weight = req.lm_head = None
+    layers = (abi.NervaHipHfDecodeChainLayer * req.layer_count)()
+    for dst, src in zip(layers, weights.c_layers):
+        for field in ("q_norm_weight", "k_norm_weight", "q_bias", "k_bias", "v_bias", "o_bias"):
+            setattr(dst, field, getattr(src, field))
+    req.layers = layers
+    return layers
+
+
 def greedy_sampler():
     cfg = abi.NervaHipHfDecodeSamplerConfig()
     cfg.temperature, cfg.top_p, cfg.top_k, cfg.seed = 0.0, 1.0, 0, 0
@@ -65,11 +159,16 @@ class DecodeSession:
         self.lib = abi.load()
 
     @classmethod
-    def create(cls, weights, max_context, **extra):
+    def create(cls, weights, max_context, plan=None, tensor_pointers=True, **extra):
+        """plan: a WeightPlan whose descriptors then are the source of the weights; with
+        tensor_pointers=False the request carries no tensor pointers at all."""
         lib = abi.load()
         req = abi.NervaHipHfDecodeSequenceSessionCreateRequest()
         weights.fill_dims(req)
         req.max_context_tokens = max_context
+        keep = None if tensor_pointers else descriptor_layout_layers(weights, req)
+        for k, v in (plan.fields() if plan is not None else {}).items():
+            setattr(req, k, v)
         for k, v in extra.items():
             setattr(req, k, v)
         res = abi.NervaHipHfDecodeSequenceSessionCreateResult()

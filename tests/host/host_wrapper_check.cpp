@@ -48,6 +48,36 @@ struct KatModel {
     c.layers.push_back(l);
     return c;
   }
+  // decode_sequence_descriptor_blocks.rs:223-258: one block per tensor in arena order, the first six
+  // GPU-resident, the rest GPU-staged
+  std::vector<HipHfDecodeSequenceWeightBlock> blocks() const {
+    const uint64_t bytes[12] = {16, 4, 8, 8, 8, 8, 4, 8, 8, 8, 4, 16};
+    const std::vector<uint16_t> *sources[12] = {&emb, &rms, &zero, &zero, &zero, &zero, &rms, &zero, &zero, &zero, &rms, &head};
+    std::vector<HipHfDecodeSequenceWeightBlock> out;
+    uint64_t offset = 0;
+    for (int i = 0; i < 12; ++i) {
+      HipHfDecodeSequenceWeightBlock b{};
+      b.host_source = sources[i]->data();
+      b.block_id = static_cast<uint64_t>(i) + 1;
+      b.offset_bytes = offset;
+      b.bytes = bytes[i];
+      b.strategy = i < 6 ? HIP_HF_WEIGHT_STRATEGY_GPU_RESIDENT : HIP_HF_WEIGHT_STRATEGY_GPU_STAGED;
+      out.push_back(b);
+      offset += bytes[i];
+    }
+    return out;
+  }
+  static HipHfDecodeSequenceWeightPlan plan(const std::vector<HipHfDecodeSequenceWeightBlock> &blocks) {
+    HipHfDecodeSequenceWeightPlan p;
+    p.blocks = 12;
+    p.gpu_resident_blocks = 6;
+    p.gpu_staged_blocks = 6;
+    p.weight_bytes = 100;
+    p.gpu_resident_weight_bytes = 52;
+    p.gpu_staged_weight_bytes = 48;
+    p.descriptor_hash = hash_weight_blocks(blocks);
+    return p;
+  }
 };
 
 static void cpu_checks() {
@@ -68,6 +98,33 @@ static void cpu_checks() {
   std::vector<uint32_t> none, outside{7};
   CHECK(detail::validate_loop_start(none, 4).has_value());
   CHECK(detail::validate_loop_start(outside, 4).has_value());
+  // weight plan: validated before the call (weight_plan.rs:53-100)
+  {
+    const std::vector<HipHfDecodeSequenceWeightBlock> blocks = m.blocks();
+    HipHfDecodeSequenceSessionConfig planned = m.config();
+    planned.weight_plan = KatModel::plan(blocks);
+    planned.weight_blocks = blocks;
+    CHECK(!planned.validate().has_value());
+    planned.embeddings = Span<uint16_t>();          // with a declared plan the tensor spans are not looked at
+    CHECK(!planned.validate().has_value());
+    planned.weight_plan->descriptor_hash ^= 1;
+    CHECK(planned.validate().value_or("").find("hash") != std::string::npos);
+    planned.weight_plan = KatModel::plan(blocks);
+    planned.weight_plan->blocks = 11;
+    CHECK(planned.validate().value_or("").find("count") != std::string::npos);
+    planned.weight_plan = KatModel::plan(blocks);
+    planned.weight_plan->gpu_staged_blocks = 7;
+    CHECK(planned.validate().value_or("").find("block counts") != std::string::npos);
+    planned.weight_plan = KatModel::plan(blocks);
+    planned.weight_plan->descriptor_hash = 0;
+    CHECK(planned.validate().value_or("").find("incomplete") != std::string::npos);
+    std::vector<HipHfDecodeSequenceWeightBlock> sourceless = blocks;
+    sourceless[3].host_source = nullptr;
+    planned.weight_plan = KatModel::plan(sourceless);
+    planned.weight_blocks = sourceless;
+    CHECK(planned.validate().value_or("").find("source") != std::string::npos);
+    CHECK(hash_weight_blocks(Span<HipHfDecodeSequenceWeightBlock>()) == 0xcbf29ce484222325ull);
+  }
   // a batch step over nothing is answered without a device (decode_sequence_session.rs:61-86)
   HipHfDecodeSequenceBatchAdvanceSummary nothing = HipHfDecodeSequenceSession::batch_advance_one({}, 8, 2);
   CHECK(nothing.status == SmokeStatus::Ok && nothing.reason == "no_sessions" && !nothing.exact);
@@ -137,10 +194,17 @@ static void gpu_checks() {
 // finished.
 static void gpu_batch_checks() {
   KatModel m;
+  // both sessions from the same declared weight plan (decode_sequence_session.rs:305-333): the
+  // descriptors are the source of the weights, the tensor spans stay empty
+  const std::vector<HipHfDecodeSequenceWeightBlock> blocks = m.blocks();
   HipHfDecodeSequenceSessionConfig config = m.config();
-  config.planned_weight_descriptor_hash = 0x1234;
+  config.weight_plan = KatModel::plan(blocks);
+  config.weight_blocks = blocks;
+  config.embeddings = config.final_norm_weight = config.lm_head = Span<uint16_t>();
+  config.layers[0] = HipHfDecodeChainLayer{};
   auto created_a = config.create();
   auto created_b = config.create();
+  CHECK(created_a.summary.h2d_bytes == 100 && created_a.summary.resident_weight_bytes == 100);
   CHECK(created_a.session && created_b.session);
   if (!created_a.session || !created_b.session) return;
   std::vector<uint32_t> prompt_a{0}, prompt_b{1};

@@ -182,3 +182,58 @@ def test_python_package_has_no_cpu_fallback():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "from oracle" not in text, f
                 assert "libnerva_oracle" not in text and "nvo_" not in text, f
+
+
+def test_weight_plan_hash_and_totals_of_the_reference_twelve_block_plan():
+    """Host logic of the weight plan (weight_plan.rs:24-126): the known-answer model's tensors in arena
+    order give the reference's 12 blocks (decode_sequence_descriptor_blocks.rs:223-258), and the
+    descriptor hash is FNV-1a-64 over the little-endian bytes of (block_id, block_version,
+    offset_bytes, bytes: u64; strategy: u32) - checked against the oracle's byte hash, which the
+    reference's own hash vectors pin."""
+    import struct
+
+    import nerva_amd as N
+    import oracle as O
+
+    z4, r2 = np.zeros(4, np.uint16), np.full(2, 0x3C00, np.uint16)
+    layer = dict(rms_attn=r2, rms_mlp=r2, w_q=z4, w_k=z4, w_v=z4, w_o=z4, w_gate=z4, w_up=z4, w_down=z4)
+    weights = N.ModelWeights(0, 2, 1, 1, 2, 2, 4, 1e-5, 0.0, np.zeros(8, np.uint16), [layer], r2, np.zeros(8, np.uint16))
+    plan = N.WeightPlan.from_weights(weights, resident_blocks=6)
+    assert [b.bytes for b in plan.blocks] == [16, 4, 8, 8, 8, 8, 4, 8, 8, 8, 4, 16]
+    assert [b.offset_bytes for b in plan.blocks] == [0, 16, 20, 28, 36, 44, 52, 56, 64, 72, 80, 84]
+    assert [b.block_id for b in plan.blocks] == list(range(1, 13))
+    f = plan.fields()
+    assert (f["planned_weight_blocks"], f["planned_gpu_resident_blocks"], f["planned_gpu_staged_blocks"],
+            f["planned_weight_bytes"], f["planned_gpu_resident_weight_bytes"], f["planned_gpu_staged_weight_bytes"],
+            f["planned_weight_descriptor_count"]) == (12, 6, 6, 100, 52, 48, 12)
+    packed = b"".join(struct.pack("<QQQQI", b.block_id, b.block_version, b.offset_bytes, b.bytes, b.strategy)
+                      for b in plan.blocks)
+    assert plan.descriptor_hash == O.fnv1a(np.frombuffer(packed, np.uint8)) == f["planned_weight_descriptor_hash"]
+    assert N.hash_weight_blocks([]) == 0xCBF29CE484222325
+    # blocks cut across tensors: even sizes, gapless, the last one shorter
+    cut = N.WeightPlan.from_weights(weights, block_bytes=14)
+    assert [b.bytes for b in cut.blocks] == [14] * 7 + [2] and cut.fields()["planned_weight_bytes"] == 100
+    assert all(b.offset_bytes == 14 * i for i, b in enumerate(cut.blocks))
+
+
+def test_incomplete_weight_plan_is_refused_before_the_device(lib):
+    """session_api_lifecycle.inc.cu:48-55: a declared plan needs one descriptor per block and a hash;
+    refused as an invalid request (hip_error 0), with or without a GPU."""
+    req, layer, z = _tiny_request()
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    block = (abi.NervaHipHfDecodeSequenceWeightBlock * 1)()
+    block[0].host_source, block[0].bytes, block[0].strategy, block[0].block_id = z.ctypes.data, 100, 1, 1
+    cases = [dict(planned_weight_blocks=1),                                                     # no byte total
+             dict(planned_weight_bytes=100),                                                    # no block count
+             dict(planned_weight_blocks=1, planned_weight_bytes=100, planned_weight_descriptor_hash=7),   # no descriptors
+             dict(planned_weight_blocks=2, planned_weight_bytes=100, planned_weight_descriptor_hash=7,
+                  planned_weight_descriptors=block, planned_weight_descriptor_count=1),         # count != blocks
+             dict(planned_weight_blocks=1, planned_weight_bytes=100, planned_weight_descriptors=block,
+                  planned_weight_descriptor_count=1)]                                           # no hash
+    for fields in cases:
+        req, layer, z = _tiny_request()
+        for name, value in fields.items():
+            setattr(req, name, value)
+        assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1, fields
+        assert cres.status == -1 and cres.hip_error == 0 and cres.failure_stage == 1

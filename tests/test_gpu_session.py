@@ -55,19 +55,120 @@ def test_reference_greedy_stream_kat(kat, qk_norm):
     assert res.kv_tokens == k["kv_tokens_with_eos"] and res.graph_replays == 4
 
 
-def test_weight_plan_echo_and_mismatch(kat):
+def kat_plan(weights):
+    """The reference's 12-block plan of the known-answer model: one block per tensor, the first six
+    declared GPU-resident and the rest GPU-staged (decode_sequence_descriptor_blocks.rs:223-258)."""
+    plan = N.WeightPlan.from_weights(weights, resident_blocks=6)
+    assert [b.bytes for b in plan.blocks] == [16, 4, 8, 8, 8, 8, 4, 8, 8, 8, 4, 16]
+    return plan
+
+
+def test_weight_plan_descriptors_are_the_source_of_the_weights(kat):
+    """decode_sequence_descriptors.rs:2093-2181 (descriptors override poisoned tensor pointers) and
+    :2182-2187 with decode_sequence_descriptor_blocks.rs:41-97 (null tensor pointers): the stream is the
+    known-answer stream, the byte counters are the plan's."""
     weights, k = kat_models(kat, False)
-    plan = dict(planned_weight_blocks=12, planned_gpu_resident_blocks=6, planned_gpu_staged_blocks=6,
-                planned_weight_bytes=100, planned_gpu_resident_weight_bytes=52,
-                planned_gpu_staged_weight_bytes=48, planned_weight_descriptor_hash=1234)
-    rc, res, tokens = decode_sequence_oneshot(weights, k["prompt"], k["steps"], plan=plan)
+    plan = kat_plan(weights)
+    fields = plan.fields()
+    assert (fields["planned_weight_blocks"], fields["planned_gpu_resident_blocks"], fields["planned_gpu_staged_blocks"],
+            fields["planned_weight_bytes"], fields["planned_gpu_resident_weight_bytes"],
+            fields["planned_gpu_staged_weight_bytes"]) == (12, 6, 6, 100, 52, 48)
+    # poisoned tensor pointers: zero embeddings and head, all-ones matrices
+    one, zero = 0x3C00, 0x0000
+    bad_layer = {key: np.full(4, one, np.uint16) for key in ("w_q", "w_k", "w_v", "w_o", "w_gate", "w_up", "w_down")}
+    bad_layer.update(rms_attn=np.full(2, zero, np.uint16), rms_mlp=np.full(2, zero, np.uint16))
+    poisoned = N.ModelWeights(F16, k["hidden"], k["heads"], k["kv_heads"], k["head_dim"], k["intermediate"], k["vocab"],
+                              k["rms_eps"], k["rope_theta"], np.zeros(8, np.uint16), [bad_layer],
+                              np.zeros(2, np.uint16), np.zeros(8, np.uint16))
+    rc, res, tokens = decode_sequence_oneshot(poisoned, k["prompt"], k["steps"], plan=fields)
     assert rc == 0 and tokens.tolist() == k["tokens"]
     assert res.planned_weight_blocks == 12 and res.planned_weight_bytes == res.resident_weight_bytes == 100
-    assert res.planned_gpu_resident_weight_bytes == 52 and res.planned_gpu_staged_weight_bytes == 48
     assert res.descriptor_gpu_resident_h2d_bytes == 52 and res.descriptor_gpu_staged_h2d_bytes == 48
-    plan["planned_weight_bytes"] = 99  # a plan that disagrees with the arena is rejected
-    rc, res, _ = decode_sequence_oneshot(weights, k["prompt"], k["steps"], plan=plan)
-    assert rc == -1 and res.status == -1
+    assert res.planned_weight_descriptor_count == 12 and res.planned_weight_descriptor_hash == plan.descriptor_hash
+    # without the plan the poisoned pointers are what runs
+    rc, res, bad_tokens = decode_sequence_oneshot(poisoned, k["prompt"], k["steps"])
+    assert rc == 0 and bad_tokens.tolist() != k["tokens"]
+    # null tensor pointers
+    s = N.DecodeSession.create(weights, 16, plan=plan, tensor_pointers=False)
+    assert s.create_result.h2d_bytes == 100 and s.create_result.planned_weight_descriptor_hash == plan.descriptor_hash
+    rc, res, tokens = s.run(k["prompt"], k["steps"])
+    assert rc == 0 and tokens.tolist() == k["tokens"]
+    s.destroy()
+
+
+def test_weight_plan_validation(kat):
+    """weights.cu:411-467: what makes a declared plan unacceptable."""
+    weights, k = kat_models(kat, False)
+
+    def attempt(change=None, **override):
+        plan = kat_plan(weights)
+        if change is not None:
+            change(plan.blocks)
+        fields = plan.fields() if change is None else dict(plan.fields(), planned_weight_descriptor_hash=N.hash_weight_blocks(plan.blocks))
+        fields.update(override)
+        rc, res, _ = decode_sequence_oneshot(weights, k["prompt"], k["steps"], plan=fields)
+        return rc, res
+
+    assert attempt()[0] == 0
+    rc, res = attempt(planned_weight_bytes=99)
+    assert rc == -1 and res.status == -1                                        # totals disagree with the arena
+    assert attempt(planned_weight_descriptor_hash=1234)[0] == -1                # hash of the descriptors
+    assert attempt(planned_gpu_resident_blocks=5)[0] == -1                      # block counts
+    assert attempt(planned_gpu_resident_weight_bytes=50)[0] == -1               # byte counts
+    assert attempt(planned_weight_descriptor_count=11)[0] == -1                 # descriptors stop short of the arena
+    assert attempt(planned_weight_descriptor_count=0, planned_weight_descriptors=None)[0] == -1   # a plan without descriptors
+
+    def gap(blocks):
+        blocks[3].offset_bytes += 2
+    def odd(blocks):
+        blocks[2].bytes -= 1
+        blocks[3].offset_bytes -= 1
+        blocks[3].bytes += 1
+    def strategy(blocks):
+        blocks[4].strategy = 3
+    def reserved(blocks):
+        blocks[0].reserved = 1
+    def sourceless(blocks):
+        blocks[5].host_source = None
+    for change in (gap, odd, strategy, reserved, sourceless):
+        assert attempt(change)[0] == -1, change.__name__
+
+
+@pytest.mark.parametrize("source", ["memory", "file"])
+def test_weight_plan_blocks_cut_across_tensors(source, tmp_path):
+    """Descriptors need not follow tensor boundaries: the arena of a random model (q/k norms and biases
+    present, so every optional tensor of the order is exercised) is cut into 5000-byte blocks, from memory
+    or from a file, and the session must hold exactly the weights a pointer-fed session holds - same
+    logits bit for bit, same K/V rows, same stream."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers = BF16, 256, 4, 2, 64, 520, 300, 2
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 31, 1e4, qk_norm=True, bias=True)
+    path = str(tmp_path / "arena.bin") if source == "file" else None
+    plan = N.WeightPlan.from_weights(weights, block_bytes=5000, resident_blocks=40, path=path)
+    assert len(plan.blocks) > 100 and plan.fields()["planned_gpu_staged_blocks"] == len(plan.blocks) - 40
+    prompt = np.random.default_rng(2).integers(0, vocab, 11).astype(np.uint32)
+    outcome = []
+    for kwargs in (dict(), dict(plan=plan)):
+        s = N.DecodeSession.create(weights, 32, **kwargs)
+        rc, _ = s.start(prompt)
+        assert rc == 0
+        logits = s.logits()
+        rows = [s.kv_row(layer, 10) for layer in range(layers)]
+        rc, _, tokens = s.advance(8)
+        assert rc == 0
+        outcome.append((logits, rows, tokens.tolist(), s.create_result))
+        s.destroy()
+    (l0, r0, t0, c0), (l1, r1, t1, c1) = outcome
+    assert np.array_equal(l0, l1) and t0 == t1
+    for (k0, v0), (k1, v1) in zip(r0, r1):
+        assert np.array_equal(k0, k1) and np.array_equal(v0, v1)
+    assert c1.resident_weight_bytes == c0.resident_weight_bytes == c1.h2d_bytes == c1.planned_weight_bytes
+    assert c1.planned_weight_descriptor_count == len(plan.blocks)
+    if source == "file":
+        # a file that ends early is an error, not a silent short read
+        with open(path, "r+b") as f:
+            f.truncate(c1.planned_weight_bytes - 100)
+        with pytest.raises(RuntimeError):
+            N.DecodeSession.create(weights, 32, plan=plan)
 
 
 def test_session_lifecycle_kat(kat):
@@ -583,9 +684,6 @@ def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
 
 # ---- sessions on shared weights: fork, and one decode step for a batch of them -------------------
 
-WEIGHT_HASH = 0x5EED5EED
-
-
 def started(session, prompt, sampler=None):
     """start + the advance(1) that hands out the token start computed: the state a batch step takes."""
     rc, _ = session.start(prompt, sampler=sampler)
@@ -620,11 +718,12 @@ def test_batch_advance_one_matches_solo_sessions_and_oracle(geom):
     rng = np.random.default_rng(17)
     prompts = [rng.integers(0, vocab, n).astype(np.uint32) for n in (1, 5, 17, 33, 40)]
     steps, max_ctx = 6, 64
-    parent = N.DecodeSession.create(weights, max_ctx, planned_weight_descriptor_hash=WEIGHT_HASH)
+    plan = N.WeightPlan.from_weights(weights)        # a declared weight plan: its descriptor hash names the model
+    parent = N.DecodeSession.create(weights, max_ctx, plan=plan, tensor_pointers=False)
     sessions = [parent] + [parent.fork_shared_weights() for _ in range(4)]
     for child in sessions[1:]:
         assert child.create_result.resident_weight_bytes == parent.create_result.resident_weight_bytes
-        assert child.create_result.planned_weight_descriptor_hash == WEIGHT_HASH
+        assert child.create_result.planned_weight_descriptor_hash == plan.descriptor_hash != 0
     streams = [[started(s, p)] for s, p in zip(sessions, prompts)]
     for step in range(steps):
         rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 32, 2)
@@ -706,9 +805,9 @@ def test_batch_advance_one_eligibility_and_reasons():
     reasons = N.DecodeSession.BATCH_REASONS
     rc, res, _ = N.DecodeSession.batch_advance_one([], 8, 2)
     assert rc == 0 and res.status == 0 and reasons[res.reason] == "no_sessions"
-    hashed = N.DecodeSession.create(weights, 24, planned_weight_descriptor_hash=WEIGHT_HASH)
+    hashed = N.DecodeSession.create(weights, 24, plan=N.WeightPlan.from_weights(weights))
     twin = hashed.fork_shared_weights()
-    other = N.DecodeSession.create(weights, 24, planned_weight_descriptor_hash=WEIGHT_HASH + 1)
+    other = N.DecodeSession.create(weights, 24, plan=N.WeightPlan.from_weights(weights, block_bytes=4096))   # another plan
     plain = N.DecodeSession.create(weights, 24)
     rc, res, _ = N.DecodeSession.batch_advance_one([hashed, twin], 8, 2)
     assert rc == 0 and reasons[res.reason] == "no_ready_sessions"            # nothing started
