@@ -266,7 +266,7 @@ def main():
                      ms_per_step=round(1e3 * b_elapsed / args.batch_steps, 4),
                      device_ms_per_step=round(device_ns / 1e6 / args.batch_steps, 4),
                      tok_s=round(len(group) * args.batch_steps / b_elapsed, 1),
-                     shared_weight_stream=int(bres.shared_weight_stream), fork_s=round(fork_s, 2))
+                     shared_weight_stream=int(session.shares_weight_stream()), fork_s=round(fork_s, 2))
         log("[bench] %d sessions on shared weights at context %d: %.3f ms per batch step (device %.3f) -> %.0f tok/s "
             "aggregate (%.1fx the single sequence)" % (len(group), position, batch["ms_per_step"],
                                                        batch["device_ms_per_step"], batch["tok_s"], batch["tok_s"] / tok_s))

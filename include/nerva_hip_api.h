@@ -268,9 +268,7 @@ typedef struct NervaHipHfDecodeSequenceBatchAdvanceRequest {
  * counters count this library's launches: pack = embedding and RMSNorm rows, projection = the
  * multi-row GEMMs (or GEMVs), scatter = K/V rows into the caches, dependency = attention,
  * sampling = sampler launches. *_elapsed_ns stay 0 except projection_elapsed_ns, which is the
- * device time of the whole batch step (the projections are not timed apart from the rest).
- * `shared_weight_stream` is 1 when one stream of the weights served every sequence of the step, 0
- * when the model's shapes are outside the multi-row kernels and each sequence ran its own step. */
+ * device time of the whole batch step (the projections are not timed apart from the rest). */
 typedef struct NervaHipHfDecodeSequenceBatchAdvanceResult {
   int32_t status, hip_error, device_count;
   uint32_t reason, exact, requested_session_count, eligible_session_count, block_tokens,
@@ -280,7 +278,6 @@ typedef struct NervaHipHfDecodeSequenceBatchAdvanceResult {
       pack_kernel_launches, projection_kernel_launches, scatter_kernel_launches,
       dependency_kernel_launches, experimental_rt_selector_launches, sampling_kernel_launches,
       sync_calls, hot_path_allocations;
-  uint32_t shared_weight_stream;
 } NervaHipHfDecodeSequenceBatchAdvanceResult;
 
 /* mirrors NervaCudaDeepSeekQuantDequantResult (nerva_cuda_api.h:1338-1354) */
@@ -698,6 +695,10 @@ int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *session, uint
 
 /* Reads back the f32 logits of the last sampled position (vocab_size floats) and
  * one KV row (kv_heads*head_dim 16-bit values each for K and V) for parity tests. */
+/* 1 when a batch step led by this session streams the weights once for all its sequences (the
+ * model's shapes fit the multi-row kernels: head_dim 128, GQA factor 1/2/4/8, K dimensions multiples
+ * of 2048), 0 when every sequence of such a step runs its own decode step; -1 for a null session. */
+int nerva_hip_session_shares_weight_stream(NervaHipHfDecodeSequenceSession *session);
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *session, float *host_logits);
 int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *session, uint32_t layer, uint32_t token,
                               uint16_t *host_k, uint16_t *host_v);

@@ -23,6 +23,9 @@ NERVA_HIP_SIZE(NervaHipHfDecodeSequenceSessionCreateResult, 272);
 NERVA_HIP_SIZE(NervaHipHfDecodeSequenceSessionRunRequest, 80);
 NERVA_HIP_SIZE(NervaHipHfDecodeSequenceSessionStartRequest, 56);
 NERVA_HIP_SIZE(NervaHipHfDecodeSequenceSessionAdvanceRequest, 32);
+NERVA_HIP_SIZE(NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest, 16);
+NERVA_HIP_SIZE(NervaHipHfDecodeSequenceBatchAdvanceRequest, 40);
+NERVA_HIP_SIZE(NervaHipHfDecodeSequenceBatchAdvanceResult, 184);
 NERVA_HIP_SIZE(NervaHipDeepSeekQuantDequantResult, 96);
 NERVA_HIP_SIZE(NervaHipDeepSeekQuantFp8F32ScaleEncodedMatvecRequest, 56);
 NERVA_HIP_SIZE(NervaHipDeepSeekQuantFp8F32ScaleEncodedGemmTokensRequest, 56);
@@ -42,3 +45,6 @@ NERVA_HIP_OFF(NervaHipHfDecodeSequenceSessionCreateRequest, embeddings, 48);
 NERVA_HIP_OFF(NervaHipHfDecodeSequenceSessionCreateRequest, detailed_profile, 144);
 NERVA_HIP_OFF(NervaHipHfDecodeSequenceSessionCreateResult, device_memory_bandwidth_bps, 264);
 NERVA_HIP_OFF(NervaHipHfDecodeSequenceSessionStartRequest, sampler, 32);
+NERVA_HIP_OFF(NervaHipHfDecodeSequenceBatchAdvanceRequest, output_tokens, 24);
+NERVA_HIP_OFF(NervaHipHfDecodeSequenceBatchAdvanceResult, observed_token_hash, 56);
+NERVA_HIP_OFF(NervaHipHfDecodeSequenceBatchAdvanceResult, hot_path_allocations, 176);

@@ -1730,7 +1730,6 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
     out->sync_calls += 1;
   }
   const bool shared = lead->rows_ready && lead->blogits != nullptr;
-  out->shared_weight_stream = shared ? 1u : 0u;
   if (err == hipSuccess && shared) {
     err = hipEventRecord(lead->ev0, lead->stream);
     if (err == hipSuccess) err = enqueue_batch_step(lead, seqs, T, out);
@@ -2252,6 +2251,11 @@ int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *s, uint32_t r
   if (mode) *mode = s->chain ? NERVA_HIP_FUSED_CHAIN : (s->front == 1 ? NERVA_HIP_FUSED_FRONT : (s->front == 2 ? NERVA_HIP_FUSED_FRONT_ATTN_O : NERVA_HIP_FUSED_NONE));
   if (aborted) *aborted = flag;
   return 0;
+}
+
+int nerva_hip_session_shares_weight_stream(NervaHipHfDecodeSequenceSession *s) {
+  if (s == nullptr) return -1;
+  return s->rows_ready && s->blogits != nullptr ? 1 : 0;
 }
 
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *s, float *host_logits) {

@@ -284,7 +284,7 @@ inline const char *projection_batch_reason_name(uint32_t reason) {
 struct HipHfDecodeSequenceBatchAdvanceSummary {
   SmokeStatus status = SmokeStatus::Failed;
   std::string reason;
-  bool exact = false, shared_weight_stream = false;
+  bool exact = false;
   uint32_t requested_session_count = 0, eligible_session_count = 0, block_tokens = 0, target_block_tokens = 0,
            min_block_tokens = 0, dtype = 0, layer_count = 0, observed_tokens = 0, last_token = 0;
   uint64_t observed_token_hash = 0;
@@ -342,7 +342,6 @@ class HipHfDecodeSequenceSession {
     s.status = rc == 0 && out.status == 0 ? SmokeStatus::Ok : SmokeStatus::Failed;   // request.rs:1251-1255
     s.reason = detail::projection_batch_reason_name(out.reason);
     s.exact = out.exact != 0;
-    s.shared_weight_stream = out.shared_weight_stream != 0;
     s.requested_session_count = out.requested_session_count;
     s.eligible_session_count = out.eligible_session_count;
     s.block_tokens = out.block_tokens;

@@ -235,6 +235,10 @@ class DecodeSession:
         rc = lib.nerva_hip_hf_decode_sequence_batch_advance_one(C.byref(req), C.byref(res))
         return rc, res, tokens[:len(sessions)]
 
+    def shares_weight_stream(self):
+        """Whether a batch step led by this session streams the weights once for all its sequences."""
+        return self.lib.nerva_hip_session_shares_weight_stream(self.handle) == 1
+
     def start(self, prompt, eos=None, sampler=None):
         prompt = np.ascontiguousarray(prompt, np.uint32)
         req = abi.NervaHipHfDecodeSequenceSessionStartRequest()

@@ -729,7 +729,7 @@ def test_batch_advance_one_matches_solo_sessions_and_oracle(geom):
         rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 32, 2)
         assert rc == 0 and res.status == 0 and res.reason == abi.NERVA_HIP_BATCH_READY and res.exact == 1
         assert res.block_tokens == 5 and res.eligible_session_count == 5 and res.observed_tokens == 5
-        assert res.shared_weight_stream == 1 and res.hot_path_allocations == 0
+        assert parent.shares_weight_stream() and res.hot_path_allocations == 0
         assert res.projection_kernel_launches == 4 * layers + 1 and res.dependency_kernel_launches == layers
         assert res.scatter_kernel_launches == layers and res.sampling_kernel_launches == 2
         assert res.observed_token_hash == O.fnv1a(tokens) and res.last_token == tokens[-1]
@@ -825,7 +825,7 @@ def test_batch_advance_one_eligibility_and_reasons():
     started(other, [9, 9])
     # shapes outside the multi-row kernels (hidden 512): every sequence runs its own step, same contract
     rc, res, tokens = N.DecodeSession.batch_advance_one([other, plain, hashed, twin], 8, 2)
-    assert rc == 0 and reasons[res.reason] == "ready" and res.block_tokens == 2 and res.shared_weight_stream == 0
+    assert rc == 0 and reasons[res.reason] == "ready" and res.block_tokens == 2 and not hashed.shares_weight_stream()
     assert tokens[0] == 0xFFFFFFFF and tokens[1] == 0xFFFFFFFF and tokens[2] < vocab and tokens[3] < vocab
     # the step is the one a solo advance would have made
     ctx = O.Context(omodel, 24, staging=1)
