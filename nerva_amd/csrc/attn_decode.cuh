@@ -71,7 +71,8 @@ struct AttnParams {
   uint64_t ws_token_stride;    // bytes between tokens' split workspaces (attn_workspace_bytes)
   // A batch of sequences instead of consecutive positions of one: token z belongs to seqs[z] (device
   // memory, `tokens` entries), which replaces k_cache, v_cache, table, block_count and the position.
-  // Applies to z = 0 as well, and to a block of one token.
+  // Applies to z = 0 as well, and to a block of one token. With append = 1 every sequence's new row
+  // is written to its cache by the launch itself.
   const AttnSeq *seqs;
 };
 

@@ -322,10 +322,12 @@ hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t s
       static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
   if (p.tokens > 1 || p.seqs != nullptr) {
-    // a block of positions: host-given positions, rows already in the cache, matrix-core kernel only
+    // a block of positions or of sequences: host-given positions, matrix-core kernel only
     const uint32_t group = p.heads / p.kv_heads;
     const bool fast = p.head_dim == 128 && (group == 1 || group == 2 || group == 4 || group == 8) && p.part_acc != nullptr;
-    if (p.cursor != nullptr || p.append != 0 || !fast || p.tokens == 0 || p.tokens > 65535 ||
+    // (rows of consecutive positions have to be in the cache before the launch; rows of different
+    // sequences can be appended by the launch itself, as the single-token kernel does)
+    if (p.cursor != nullptr || (p.append != 0 && p.seqs == nullptr) || !fast || p.tokens == 0 || p.tokens > 65535 ||
         (p.seqs == nullptr &&
          static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens))
       return hipErrorInvalidValue;

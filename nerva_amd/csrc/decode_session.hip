@@ -1479,7 +1479,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     a.rope_token_stride = lead->head_dim;
     a.ws_token_stride = lead->pattn_ws_stride;
     a.seqs = lead->btable->seq;
-    if (err == hipSuccess) err = launch_kv_publish_rows(lead->dtype, a, st);
+    a.append = 1;  // each sequence's K/V row goes into its own cache inside the attention launch
     if (err == hipSuccess) err = launch_attn_decode(lead->dtype, a, st);
     if (err == hipSuccess) {
       g = GemmRowsParams{};
@@ -1517,7 +1517,6 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     }
     out->pack_kernel_launches += 2;
     out->projection_kernel_launches += 4;
-    out->scatter_kernel_launches += 1;
     out->dependency_kernel_launches += 1;
   }
   if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st);

@@ -1,6 +1,8 @@
 // Multi-row projection on the matrix cores (see gemm_rows.cuh).
 #include "gemm_rows.cuh"
 
+#include <stdlib.h>
+
 #include <mutex>
 
 namespace nv {
@@ -14,6 +16,7 @@ constexpr int kRowStride = kKB + 8;             // LDS row stride in elements: 1
                                                 // the 16 rows of an operand read on distinct banks
 constexpr int kTileElems = 16 * kRowStride;     // one 16-row block of W in LDS
 constexpr int kSteps = kKB / 32;                // matrix-core K-steps per block
+constexpr uint32_t kTwoTileMinWorkgroups = 512; // two row tiles per workgroup from this many workgroups on
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
@@ -38,9 +41,12 @@ constexpr size_t gemm_lds_bytes() {
   return tiles > partials ? tiles : partials;
 }
 
-template <uint32_t DT, int EPI>
+// RT: 16-row tiles of W per workgroup for the plain epilogues (the X pieces a wave fetches serve all of
+// them, so two tiles halve the X traffic per weight byte; the grid halves with it).
+template <uint32_t DT, int EPI, int RT>
 __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) {
-  constexpr int NR = EPI == kGemmSwiglu ? 2 : 1;  // SwiGLU: the gate rows and the up rows of the same outputs
+  constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;  // SwiGLU: the gate rows and the up rows of the same outputs
+  constexpr uint32_t kWgRows = EPI == kGemmSwiglu ? 16u : 16u * RT;
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -48,14 +54,15 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   const uint32_t cols = p.cols, T = p.tokens;
   // the last workgroup of a row count that is no multiple of 16 moves back to the last 16 rows: the
   // rows it shares with its neighbour are computed and stored twice, with the same value
-  const uint32_t row0 = min(blockIdx.x * 16u, p.rows - 16u);
+  const uint32_t row0 = min(blockIdx.x * kWgRows, p.rows - kWgRows);
+  const uint32_t tile_rows = EPI == kGemmSwiglu ? p.rows : 16u;   // rows between a wave's tiles
   const uint32_t kper = cols / kGW, nblk = kper / kKB, kbase = wave * kper;
 
   // W block -> registers: instruction i covers rows 2i and 2i + 1, 32 lanes x 16 B each
   const uint16_t *wp[NR];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
-    wp[j] = p.w + static_cast<uint64_t>(row0 + j * p.rows + (lane >> 5)) * cols + kbase + (lane & 31) * 8;
+    wp[j] = p.w + static_cast<uint64_t>(row0 + j * tile_rows + (lane >> 5)) * cols + kbase + (lane & 31) * 8;
   uint4 areg[NR][8];
 #define NV_GEMM_REQUEST(BLK)                                                                        \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 8; ++i)      \
@@ -126,18 +133,22 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
     float sum = 0.0f;
 #pragma unroll
     for (int w = 0; w < kGW; ++w) sum += red[((w * NR + j) * 16 + r) * kGemmMaxTokens + t];
-    if (p.bias != nullptr) sum += dec16<DT>(p.bias[row0 + j * p.rows + r]);
+    if (p.bias != nullptr) sum += dec16<DT>(p.bias[row0 + j * tile_rows + r]);
     y[j] = sum;
   }
   const uint64_t at = static_cast<uint64_t>(t) * p.rows + row0 + r;
-  if constexpr (EPI == kGemmF32) {
-    p.out_f32[at] = y[0];
-  } else if constexpr (EPI == kGemmResidual) {
-    float v = y[0] + p.residual[at];
-    if (p.round_out) v = round16<DT>(v);
-    p.out_f32[at] = v;
-  } else {
+  if constexpr (EPI == kGemmSwiglu) {
     p.out16[at] = enc16<DT>(silu(y[0]) * y[NR - 1]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < NR; ++j) {
+      float v = y[j];
+      if constexpr (EPI == kGemmResidual) {
+        v += p.residual[at + j * 16];
+        if (p.round_out) v = round16<DT>(v);
+      }
+      p.out_f32[at + j * 16] = v;
+    }
   }
 }
 
@@ -183,30 +194,43 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const float 
   }
 }
 
-template <uint32_t DT, int EPI>
+template <uint32_t DT, int EPI, int RT>
 hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
-  constexpr int NR = EPI == kGemmSwiglu ? 2 : 1;
+  constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;
+  constexpr uint32_t kWgRows = EPI == kGemmSwiglu ? 16u : 16u * RT;
   constexpr size_t lds = gemm_lds_bytes<NR>();
   if (lds > 64 * 1024) {
     // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI, RT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI>), dim3((p.rows + 15) / 16), dim3(kGThreads), lds, stream, p);
+  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI, RT>), dim3((p.rows + kWgRows - 1) / kWgRows), dim3(kGThreads), lds, stream, p);
   return hipGetLastError();
 }
 
 template <uint32_t DT>
 hipError_t launch_dt(int epilogue, const GemmRowsParams &p, hipStream_t stream) {
+  // Two row tiles per workgroup where that still leaves the chip full of workgroups and there are
+  // enough token rows for the X traffic to matter. Measured on MI355X at T = 1 / 8 / 32 (one tile vs
+  // two, microseconds): LM head 151936x4096 198 / 223 / 383 vs 207 / 218 / 314; qkv 6144x4096
+  // 12.4 / 14.1 / 23.6 vs 14.7 / 15.3 / 20.1; o and down (4096 rows: 128 workgroups with two tiles) lose.
+  static const int forced = [] {
+    const char *v = getenv("NERVA_HIP_GEMM_ROW_TILES");   // tuning knob: 1 or 2 for every plain projection
+    return v != nullptr && (v[0] == '1' || v[0] == '2') ? v[0] - '0' : 0;
+  }();
+  const bool two = forced != 0 ? forced == 2
+                               : (p.rows >= 32u * kTwoTileMinWorkgroups ? p.tokens >= 8 : (p.tokens > 16 && p.rows >= 32u * 192u));
+  const bool can_two = p.rows >= 32 && !(epilogue == kGemmResidual && p.rows % 32 != 0 && p.residual == p.out_f32);
   switch (epilogue) {
-    case kGemmF32: return launch_one<DT, kGemmF32>(p, stream);
-    case kGemmResidual: return launch_one<DT, kGemmResidual>(p, stream);
-    case kGemmSwiglu: return launch_one<DT, kGemmSwiglu>(p, stream);
+    case kGemmF32: return two && can_two ? launch_one<DT, kGemmF32, 2>(p, stream) : launch_one<DT, kGemmF32, 1>(p, stream);
+    case kGemmResidual:
+      return two && can_two ? launch_one<DT, kGemmResidual, 2>(p, stream) : launch_one<DT, kGemmResidual, 1>(p, stream);
+    case kGemmSwiglu: return launch_one<DT, kGemmSwiglu, 1>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

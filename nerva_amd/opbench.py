@@ -153,7 +153,9 @@ def case_moe():
 def case_gemm_rows():
     """Token blocks through the step's weight matrices on the matrix cores: the weights are streamed once
     per block, so 32 tokens should cost about what one token costs."""
-    shapes = (("qkv 6144x4096", 6144, 4096, 0), ("gate_up 2x12288x4096 +SwiGLU", 12288, 4096, 2), ("down 4096x12288", 4096, 12288, 0))
+    shapes = (("qkv 6144x4096", 6144, 4096, 0), ("o 4096x4096", 4096, 4096, 0),
+              ("gate_up 2x12288x4096 +SwiGLU", 12288, 4096, 2), ("down 4096x12288", 4096, 12288, 0),
+              ("lm_head 151936x4096", 151936, 4096, 0))
     for name, rows, cols, epi in shapes:
         wrows = rows * (2 if epi == 2 else 1)
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
@@ -191,17 +193,17 @@ def case_sampler():
 
 
 def main():
+    only = sys.argv[1:]
     rc, smoke = Device.smoke()
     if rc != 0:
         print("no usable GPU (hip_error=%d): these operators have no CPU path" % smoke.hip_error, file=sys.stderr)
         sys.exit(1)
     log("device: %s" % smoke.gpu_name.decode())
-    case_qproj()
-    case_mlp()
-    case_attention()
-    case_moe()
-    case_sampler()
-    case_gemm_rows()
+    cases = dict(qproj=case_qproj, mlp=case_mlp, attention=case_attention, moe=case_moe, sampler=case_sampler,
+                 gemm_rows=case_gemm_rows)
+    for name, case in cases.items():      # `python -m nerva_amd.opbench gemm_rows sampler` runs only those
+        if not only or name in only:
+            case()
 
 
 if __name__ == "__main__":
