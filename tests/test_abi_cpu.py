@@ -237,3 +237,24 @@ def test_incomplete_weight_plan_is_refused_before_the_device(lib):
             setattr(req, name, value)
         assert lib.nerva_hip_hf_decode_sequence_session_create(C.byref(req), C.byref(cres), C.byref(handle)) == -1, fields
         assert cres.status == -1 and cres.hip_error == 0 and cres.failure_stage == 1
+
+
+def test_batch_step_over_nothing_and_null_fork_need_no_device(lib):
+    """decode_sequence_session.rs:61-86: a batch step over no sessions answers "no_sessions" with
+    status 0 on any machine; null requests fail closed."""
+    import nerva_amd as N
+    rc, res, tokens = N.DecodeSession.batch_advance_one([], 8, 2)
+    assert rc == 0 and res.status == 0 and N.DecodeSession.BATCH_REASONS[res.reason] == "no_sessions"
+    assert res.exact == 0 and res.requested_session_count == 0 and res.block_tokens == 0 and res.observed_tokens == 0
+    assert res.target_block_tokens == 8 and res.min_block_tokens == 2 and res.hot_path_allocations == 0
+    out = abi.NervaHipHfDecodeSequenceBatchAdvanceResult()
+    assert lib.nerva_hip_hf_decode_sequence_batch_advance_one(None, C.byref(out)) == -1
+    assert out.status == -1 and out.reason == abi.NERVA_HIP_BATCH_INVALID_REQUEST
+    assert lib.nerva_hip_hf_decode_sequence_batch_advance_one(None, None) == -1
+    cres = abi.NervaHipHfDecodeSequenceSessionCreateResult()
+    handle = C.POINTER(abi.NervaHipHfDecodeSequenceSession)()
+    req = abi.NervaHipHfDecodeSequenceSessionForkSharedWeightsRequest()
+    assert lib.nerva_hip_hf_decode_sequence_session_fork_shared_weights(C.byref(req), C.byref(cres), C.byref(handle)) == -1
+    assert cres.status == -1 and cres.failure_stage == 1 and not handle
+    assert lib.nerva_hip_hf_decode_sequence_session_fork_shared_weights(None, C.byref(cres), C.byref(handle)) == -1
+    assert lib.nerva_hip_session_shares_weight_stream(None) == -1

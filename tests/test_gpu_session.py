@@ -851,3 +851,68 @@ def test_batch_advance_one_eligibility_and_reasons():
     assert reasons[res.reason] == "no_ready_sessions"
     for s in (hashed, twin, other, plain):
         s.destroy()
+
+
+@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65])
+def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
+    """Prompt lengths around the 32-token block size (the last prompt token always goes through the
+    ordinary head step, so length - 1 tokens are prefilled in blocks): logits, first token and K/V
+    rows agree with the token walk to the end-to-end tolerance; a context exactly as long as the
+    sequence needs is enough."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[5]
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 2718, theta, qk_norm, bias)
+    prompt = np.random.default_rng(length).integers(0, vocab, length).astype(np.uint32)
+    outcome = {}
+    for mode in ("blocks", "walk"):
+        if mode == "walk":
+            monkeypatch.setenv("NERVA_HIP_PREFILL", "walk")
+        else:
+            monkeypatch.delenv("NERVA_HIP_PREFILL", raising=False)
+        s = N.DecodeSession.create(weights, length + 2)          # room for the prompt and three tokens
+        rc, res = s.start(prompt)
+        assert rc == 0 and res.kv_tokens == length
+        logits = s.logits()
+        rows = [s.kv_row(layers - 1, t) for t in sorted({0, length // 2, length - 1})]
+        rc, res, tokens = s.advance(3)
+        assert rc == 0 and res.observed_tokens == 3
+        rc, _, _ = s.advance(1)                                   # the context is full now
+        assert rc == -1
+        outcome[mode] = (logits, rows, tokens.tolist())
+        s.destroy()
+    (lb, rb, tb), (lw, rw, tw) = outcome["blocks"], outcome["walk"]
+    assert rel_l2(lb, lw) <= E2E_REL_L2
+    for (kb, vb), (kw, vw) in zip(rb, rw):
+        assert rel_l2(O.decode16(dtype, kb), O.decode16(dtype, kw)) <= E2E_REL_L2
+        assert rel_l2(O.decode16(dtype, vb), O.decode16(dtype, vw)) <= E2E_REL_L2
+    top = np.sort(lw)
+    assert tb[0] == tw[0] or top[-1] - top[-2] < E2E_REL_L2 * np.max(np.abs(lw))
+
+
+def test_batch_advance_one_fills_contexts_to_the_last_slot():
+    """Sessions of different context sizes in one batch: each goes on until its own context is full,
+    finishes there (session_api_batch_fork_destroy.inc.cu:296-299), and the others continue."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[5]
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 161, theta, qk_norm, bias)
+    plan = N.WeightPlan.from_weights(weights)
+    small = N.DecodeSession.create(weights, 18, plan=plan)       # 17 blocks of context: crosses a 16-token tile
+    large = N.DecodeSession.create(weights, 40, plan=plan)
+    assert small.shares_weight_stream()
+    started(small, [3, 4, 5])
+    started(large, list(range(20)))
+    produced = {0: 1, 1: 1}
+    for step in range(30):
+        rc, res, tokens = N.DecodeSession.batch_advance_one([small, large], 32, 1)
+        assert rc == 0
+        if N.DecodeSession.BATCH_REASONS[res.reason] != "ready":
+            break
+        for i in (0, 1):
+            if tokens[i] != 0xFFFFFFFF:
+                assert tokens[i] < vocab
+                produced[i] += 1
+    assert N.DecodeSession.BATCH_REASONS[res.reason] == "no_ready_sessions"
+    # prompt + produced - 1 tokens are in the cache: exactly the context size
+    assert 3 + produced[0] - 1 == 18 and 20 + produced[1] - 1 == 40
+    rc, _, _ = small.advance(1)
+    assert rc == -1
+    small.destroy()
+    large.destroy()
