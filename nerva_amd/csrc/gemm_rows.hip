@@ -43,10 +43,15 @@ constexpr size_t gemm_lds_bytes() {
 
 // RT: 16-row tiles of W per workgroup for the plain epilogues (the X pieces a wave fetches serve all of
 // them, so two tiles halve the X traffic per weight byte; the grid halves with it).
-template <uint32_t DT, int EPI, int RT>
+// KW: waves of a workgroup along K (8, or 4: the workgroup then holds two row groups of four waves, and
+// the two waves that walk the same K range fetch the same X pieces at about the same time, so the
+// second fetch is served by the CU's own cache instead of L2).
+template <uint32_t DT, int EPI, int RT, int KW>
 __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) {
   constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;  // SwiGLU: the gate rows and the up rows of the same outputs
-  constexpr uint32_t kWgRows = EPI == kGemmSwiglu ? 16u : 16u * RT;
+  constexpr uint32_t kGroupRows = EPI == kGemmSwiglu ? 16u : 16u * RT;   // output rows of one row group
+  constexpr int kGroups = kGW / KW;
+  constexpr uint32_t kWgRows = kGroupRows * kGroups;
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -54,9 +59,10 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   const uint32_t cols = p.cols, T = p.tokens;
   // the last workgroup of a row count that is no multiple of 16 moves back to the last 16 rows: the
   // rows it shares with its neighbour are computed and stored twice, with the same value
-  const uint32_t row0 = min(blockIdx.x * kWgRows, p.rows - kWgRows);
+  const int kslice = wave % KW, group = wave / KW;
+  const uint32_t row0 = min(blockIdx.x * kWgRows, p.rows - kWgRows) + group * kGroupRows;
   const uint32_t tile_rows = EPI == kGemmSwiglu ? p.rows : 16u;   // rows between a wave's tiles
-  const uint32_t kper = cols / kGW, nblk = kper / kKB, kbase = wave * kper;
+  const uint32_t kper = cols / KW, nblk = kper / kKB, kbase = kslice * kper;
 
   // W block -> registers: instruction i covers rows 2i and 2i + 1, 32 lanes x 16 B each
   const uint16_t *wp[NR];
@@ -124,30 +130,36 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
       for (int r = 0; r < 4; ++r)
         red[((wave * NR + j) * 16 + q * 4 + r) * kGemmMaxTokens + c * 16 + n] = acc[j][c][r];
   __syncthreads();
-  // one thread per output element: 16 rows x 32 tokens, rows fastest (contiguous stores per token)
+  // one thread per output element of a row group: 16 rows x 32 tokens, rows fastest (contiguous stores
+  // per token); the row groups in turn
   const uint32_t r = threadIdx.x & 15u, t = threadIdx.x >> 4;
   if (t >= T) return;
-  float y[NR];
+  const uint32_t wg_row0 = row0 - group * kGroupRows;
 #pragma unroll
-  for (int j = 0; j < NR; ++j) {
-    float sum = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kGW; ++w) sum += red[((w * NR + j) * 16 + r) * kGemmMaxTokens + t];
-    if (p.bias != nullptr) sum += dec16<DT>(p.bias[row0 + j * tile_rows + r]);
-    y[j] = sum;
-  }
-  const uint64_t at = static_cast<uint64_t>(t) * p.rows + row0 + r;
-  if constexpr (EPI == kGemmSwiglu) {
-    p.out16[at] = enc16<DT>(silu(y[0]) * y[NR - 1]);
-  } else {
+  for (int gq = 0; gq < kGroups; ++gq) {
+    const uint32_t grow0 = wg_row0 + gq * kGroupRows;
+    float y[NR];
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      float v = y[j];
-      if constexpr (EPI == kGemmResidual) {
-        v += p.residual[at + j * 16];
-        if (p.round_out) v = round16<DT>(v);
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < KW; ++w) sum += red[(((gq * KW + w) * NR + j) * 16 + r) * kGemmMaxTokens + t];
+      if (p.bias != nullptr) sum += dec16<DT>(p.bias[grow0 + j * tile_rows + r]);
+      y[j] = sum;
+    }
+    const uint64_t at = static_cast<uint64_t>(t) * p.rows + grow0 + r;
+    if constexpr (EPI == kGemmSwiglu) {
+      p.out16[at] = enc16<DT>(silu(y[0]) * y[NR - 1]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NR; ++j) {
+        float v = y[j];
+        if constexpr (EPI == kGemmResidual) {
+          v += p.residual[at + j * 16];
+          if (p.round_out) v = round16<DT>(v);
+        }
+        p.out_f32[at + j * 16] = v;
       }
-      p.out_f32[at + j * 16] = v;
     }
   }
 }
@@ -194,22 +206,22 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const float 
   }
 }
 
-template <uint32_t DT, int EPI, int RT>
+template <uint32_t DT, int EPI, int RT, int KW>
 hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
   constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;
-  constexpr uint32_t kWgRows = EPI == kGemmSwiglu ? 16u : 16u * RT;
+  constexpr uint32_t kWgRows = (EPI == kGemmSwiglu ? 16u : 16u * RT) * (kGW / KW);
   constexpr size_t lds = gemm_lds_bytes<NR>();
   if (lds > 64 * 1024) {
     // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI, RT>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI, RT, KW>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI, RT>), dim3((p.rows + kWgRows - 1) / kWgRows), dim3(kGThreads), lds, stream, p);
+  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI, RT, KW>), dim3((p.rows + kWgRows - 1) / kWgRows), dim3(kGThreads), lds, stream, p);
   return hipGetLastError();
 }
 
@@ -226,11 +238,23 @@ hipError_t launch_dt(int epilogue, const GemmRowsParams &p, hipStream_t stream) 
   const bool two = forced != 0 ? forced == 2
                                : (p.rows >= 32u * kTwoTileMinWorkgroups ? p.tokens >= 8 : (p.tokens > 16 && p.rows >= 32u * 192u));
   const bool can_two = p.rows >= 32 && !(epilogue == kGemmResidual && p.rows % 32 != 0 && p.residual == p.out_f32);
+  static const int forced_kw = [] {
+    const char *v = getenv("NERVA_HIP_GEMM_K_WAVES");   // tuning knob: 8 or 4 waves along K
+    return v != nullptr && (v[0] == '4' || v[0] == '8') ? v[0] - '0' : 0;
+  }();
+  // Four waves along K (two row groups per workgroup): measured at T = 1 / 8 / 32 against eight, LM head
+  // 202 / 208 / 299 vs 199 / 219 / 315 us; gate_up 39.8 / 41.9 / 60.1 vs 36.5 / 38.3 / 53.1, down and o
+  // lose more (half the workgroups). So: only for matrices with thousands of row tiles.
+  const bool kw4 = (forced_kw != 0 ? forced_kw == 4 : (p.rows >= 32u * kTwoTileMinWorkgroups && p.tokens >= 8)) &&
+                   p.rows >= 64 && !(epilogue == kGemmResidual && p.residual == p.out_f32);
   switch (epilogue) {
-    case kGemmF32: return two && can_two ? launch_one<DT, kGemmF32, 2>(p, stream) : launch_one<DT, kGemmF32, 1>(p, stream);
+    case kGemmF32:
+      if (kw4) return two && can_two ? launch_one<DT, kGemmF32, 2, 4>(p, stream) : launch_one<DT, kGemmF32, 1, 4>(p, stream);
+      return two && can_two ? launch_one<DT, kGemmF32, 2, 8>(p, stream) : launch_one<DT, kGemmF32, 1, 8>(p, stream);
     case kGemmResidual:
-      return two && can_two ? launch_one<DT, kGemmResidual, 2>(p, stream) : launch_one<DT, kGemmResidual, 1>(p, stream);
-    case kGemmSwiglu: return launch_one<DT, kGemmSwiglu, 1>(p, stream);
+      if (kw4) return launch_one<DT, kGemmResidual, 1, 4>(p, stream);
+      return two && can_two ? launch_one<DT, kGemmResidual, 2, 8>(p, stream) : launch_one<DT, kGemmResidual, 1, 8>(p, stream);
+    case kGemmSwiglu: return kw4 ? launch_one<DT, kGemmSwiglu, 1, 4>(p, stream) : launch_one<DT, kGemmSwiglu, 1, 8>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }
