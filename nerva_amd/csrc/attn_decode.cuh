@@ -97,4 +97,11 @@ hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t s
 // v_bias, the caches and table, rope_freq / rope_cs and the token strides of `p`.
 hipError_t launch_kv_publish_rows(uint32_t dtype, const AttnParams &p, hipStream_t stream);
 
+// Attention of a prompt block with the K/V tiles of the prefix shared by the block's tokens
+// (attn_prompt.hip): same inputs and outputs as launch_attn_decode for a block (tokens consecutive
+// positions from `position`, rows already in the cache, append = 0, per-token strides, per-token split
+// workspaces, rotation tables per token row), head_dim 128 and GQA factor 1/2/4/8 only.
+// p.splits = 0 lets the launcher choose.
+hipError_t launch_attn_prompt(uint32_t dtype, const AttnParams &p, hipStream_t stream);
+
 }  // namespace nv

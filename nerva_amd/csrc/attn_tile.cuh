@@ -165,7 +165,11 @@ __device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t phy
 }
 
 // One 16-token tile against the G query heads of the kv head (see attn_fast_kernel).
-template <uint32_t DT, int G, bool QX_LDS>
+// n_keys may differ from lane to lane (by column: the prompt kernel's columns belong to tokens at
+// different positions). COLUMN_MASKS = a column may find a whole tile masked, even its first one: the
+// running maximum then stays at minus infinity, and the exponentials are taken against a finite stand-in
+// so that they come out as 0 instead of NaN.
+template <uint32_t DT, int G, bool QX_LDS, bool COLUMN_MASKS = false>
 __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], const uint4 (&qx)[4],
                                           const uint4 *qx_lds, uint32_t b,
                                           uint32_t n_keys, int col, int grp, bool splice, uint32_t new_row,
@@ -213,13 +217,14 @@ __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], co
   float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
   mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
   mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
-  const float m_new = fmaxf(m, mb);   // finite: every processed tile has a valid token
-  const float alpha = attn_exp2(m - m_new);
+  const float m_new = fmaxf(m, mb);   // finite: every processed tile has a valid token (without column masks)
+  const float m_ref = COLUMN_MASKS ? fmaxf(m_new, -3.0e38f) : m_new;
+  const float alpha = attn_exp2(m - m_ref);
   uint32_t px[2];
   float psum = 0.0f;
 #pragma unroll
   for (int r = 0; r < 4; r += 2) {
-    const float p0 = attn_exp2(sc[r] - m_new), p1 = attn_exp2(sc[r + 1] - m_new);
+    const float p0 = attn_exp2(sc[r] - m_ref), p1 = attn_exp2(sc[r + 1] - m_ref);
     psum += p0 + p1;
     uint16_t h0, l0, h1, l1;
     split16<DT>(p0, h0, l0);

@@ -691,6 +691,17 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   const uint32_t H = s->hidden, A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim, I = s->intermediate;
   const float *rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
   hipError_t err = hipSuccess;
+  // NERVA_HIP_PREFILL_ATTN=rows: the block's attention as one workgroup set per token (the batch step's
+  // kernel) instead of the prompt kernel that shares K/V tiles between tokens; for comparisons
+  static const bool rows_attention = [] {
+    const char *v = getenv("NERVA_HIP_PREFILL_ATTN");
+    return v != nullptr && v[0] == 'r';
+  }();
+  static const uint32_t prompt_splits = [] {
+    const char *v = getenv("NERVA_HIP_PROMPT_SPLITS");   // tuning knob: split factor of the prompt attention
+    const long want = v != nullptr ? strtol(v, nullptr, 10) : 0;
+    return want >= 1 && want <= static_cast<long>(kAttnMaxSplits) ? static_cast<uint32_t>(want) : 0u;
+  }();
   for (uint32_t first = 0; err == hipSuccess && first < count; first += kGemmMaxTokens) {
     const uint32_t T = std::min<uint32_t>(kGemmMaxTokens, count - first);
     if (s->dtype == kBF16)
@@ -741,7 +752,14 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
       a.rope_token_stride = s->head_dim;
       a.ws_token_stride = s->pattn_ws_stride;
       if (err == hipSuccess) err = launch_kv_publish_rows(s->dtype, a, st);
-      if (err == hipSuccess) err = launch_attn_decode(s->dtype, a, st);
+      if (err == hipSuccess) {
+        if (rows_attention) {
+          err = launch_attn_decode(s->dtype, a, st);   // every token streams the prefix itself
+        } else {
+          a.splits = prompt_splits;                    // K/V tiles shared by the tokens of the block (0: the launcher chooses)
+          err = launch_attn_prompt(s->dtype, a, st);
+        }
+      }
       if (err == hipSuccess) {
         g = GemmRowsParams{};
         g.tokens = T;
@@ -778,7 +796,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
     }
-    if (err == hipSuccess) out->kernel_launches += 1 + 9ull * s->layers;
+    if (err == hipSuccess) out->kernel_launches += 1 + (rows_attention ? 9ull : 10ull) * s->layers;
   }
   if (err == hipSuccess) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, st, s->state, count, prompt_count);

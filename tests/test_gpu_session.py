@@ -643,7 +643,15 @@ def test_session_temperature_sampling_follows_the_rule(temperature, top_p, top_k
     s.destroy()
 
 
-@pytest.mark.parametrize("geom", [GEOMETRIES[5], GEOMETRIES[6]])
+PREFILL_GEOMETRIES = [
+    GEOMETRIES[5],                                                # GQA factor 4: two tokens per wave of the prompt attention
+    GEOMETRIES[6],                                                # MHA: eight tokens per wave
+    (BF16, 2048, 16, 8, 128, 2048, 640, 2, 1e6, True, True),      # GQA factor 2: four tokens per wave
+    (F16, 2048, 16, 2, 128, 2048, 640, 2, 1e4, True, False),      # GQA factor 8: one token per wave
+]
+
+
+@pytest.mark.parametrize("geom", PREFILL_GEOMETRIES)
 def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
     """start() sends the prompt through the layers in blocks of up to 32 tokens (multi-row GEMMs, one
     attention launch per block); NERVA_HIP_PREFILL=walk keeps one prompt step per token. Same staging,
