@@ -541,7 +541,7 @@ typedef struct NervaHipGemmRowsRequest {
   uint16_t *output16;        /* epilogue 2: [tokens][rows] */
 } NervaHipGemmRowsRequest;
 
-/* Projection of a block of up to 32 token rows through one weight matrix on the matrix cores,
+/* Projection of a block of up to 64 token rows through one weight matrix on the matrix cores,
  * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
  * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must

@@ -1,4 +1,4 @@
-// Attention of a prompt block: up to 32 consecutive positions of one sequence in one launch, every
+// Attention of a prompt block: consecutive positions of one sequence (64 in the session's prefill) in one launch, every
 // K/V tile of the prefix fetched once per workgroup and used by all its tokens.
 // Reference: the chunked prefill's attention (session_decode_prefill.inc.cu:1879-2243) over the
 // arithmetic of exact_blockwise_attention_into (attention/exact/run.rs:13-127) per token; the rows

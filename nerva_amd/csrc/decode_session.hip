@@ -140,7 +140,7 @@ struct NervaHipHfDecodeSequenceSession {
   bool block_prefill = false;
   // the multi-row kernels take this model's shapes (prompt blocks and batch steps need it)
   bool rows_ready = false;
-  float *blogits = nullptr;          // [kGemmMaxTokens][vocab] logits of a batch step
+  float *blogits = nullptr;          // [NERVA_HIP_BATCH_MAX_BLOCK_TOKENS][vocab] logits of a batch step
   BatchTable *btable = nullptr, *host_btable = nullptr;
   float *px = nullptr, *pr = nullptr, *pqkv = nullptr, *prope = nullptr;
   uint16_t *pxn16 = nullptr, *pattn16 = nullptr, *pff16 = nullptr;
@@ -993,7 +993,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage) {
                     gemm_rows_supported(s->hidden, s->intermediate, 1);
   }
   const bool batch_head = s->rows_ready && gemm_rows_supported(s->vocab, s->hidden, 1);
-  const uint64_t off_blogits = batch_head ? c.take(pT * V * 4) : 0;
+  const uint64_t off_blogits = batch_head ? c.take(static_cast<uint64_t>(NERVA_HIP_BATCH_MAX_BLOCK_TOKENS) * V * 4) : 0;
   const uint64_t off_btable = c.take(sizeof(BatchTable));
   s->state_bytes = c.offset;
   s->arena_bytes = s->weights->bytes + s->state_bytes;

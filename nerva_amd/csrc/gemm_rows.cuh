@@ -1,5 +1,5 @@
 // Multi-row projection on the matrix cores: Y[t][r] = sum_c W[r][c] * X[t][c] for a block of
-// T <= 32 token rows, streaming the weight matrix once for all of them. This is what a chunk of
+// T <= 64 token rows, streaming the weight matrix once for all of them. This is what a chunk of
 // prompt tokens (and a small batch of sequences) needs: the weight bytes are the same as for one
 // token, so the kernel is HBM-bound like the GEMV and T tokens cost about one.
 // Reference: the cuBLAS GEMM calls of the chunked prefill and of the projection batch
@@ -20,7 +20,7 @@
 
 namespace nv {
 
-constexpr uint32_t kGemmMaxTokens = 32;
+constexpr uint32_t kGemmMaxTokens = 64;
 enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
 
 struct GemmRowsParams {

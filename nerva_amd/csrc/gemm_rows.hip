@@ -46,8 +46,11 @@ constexpr size_t gemm_lds_bytes() {
 // KW: waves of a workgroup along K (8, or 4: the workgroup then holds two row groups of four waves, and
 // the two waves that walk the same K range fetch the same X pieces at about the same time, so the
 // second fetch is served by the CU's own cache instead of L2).
-template <uint32_t DT, int EPI, int RT, int KW>
+// TT: 16-token tiles a wave keeps accumulators for (2: up to 32 token rows; 4: up to 64, every W operand
+// then serves four products).
+template <uint32_t DT, int EPI, int RT, int KW, int TT>
 __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) {
+  constexpr uint32_t kTokCap = 16u * TT;
   constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;  // SwiGLU: the gate rows and the up rows of the same outputs
   constexpr uint32_t kGroupRows = EPI == kGemmSwiglu ? 16u : 16u * RT;   // output rows of one row group
   constexpr int kGroups = kGW / KW;
@@ -78,26 +81,26 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 8; ++i)      \
       *reinterpret_cast<uint4 *>(park_at + j * kTileElems + 2 * i * kRowStride) = areg[j][i]
 
-  // X operand: token of this lane in each of the two token tiles (clamped: columns past T are dropped later)
+  // X operand: token of this lane in each of the token tiles (clamped: columns past T are dropped later)
   const uint32_t n = lane & 15, q = lane >> 4;
-  const uint16_t *xp0 = p.x16 + static_cast<uint64_t>(min(n, T - 1)) * cols + kbase + q * 8;
-  const uint16_t *xp1 = p.x16 + static_cast<uint64_t>(min(n + 16u, T - 1)) * cols + kbase + q * 8;
+  const uint16_t *xp[TT];
+#pragma unroll
+  for (int c = 0; c < TT; ++c) xp[c] = p.x16 + static_cast<uint64_t>(min(n + 16u * c, T - 1)) * cols + kbase + q * 8;
   const uint16_t *a_read = tile + n * kRowStride + q * 8;
 
-  f32x4_t acc[NR][2];
+  f32x4_t acc[NR][TT];
 #pragma unroll
-  for (int j = 0; j < NR; ++j) acc[j][0] = acc[j][1] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  uint4 breg[kSteps][2];
+  for (int j = 0; j < NR; ++j)
+#pragma unroll
+    for (int c = 0; c < TT; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  uint4 breg[kSteps][TT];
 #define NV_GEMM_LOAD_X(BLK)                                                                         \
-  _Pragma("unroll") for (int s = 0; s < kSteps; ++s) {                                              \
-    breg[s][0] = *reinterpret_cast<const uint4 *>(xp0 + (BLK) * kKB + s * 32);                      \
-    breg[s][1] = *reinterpret_cast<const uint4 *>(xp1 + (BLK) * kKB + s * 32);                      \
-  }
+  _Pragma("unroll") for (int s = 0; s < kSteps; ++s) _Pragma("unroll") for (int c = 0; c < TT; ++c)  \
+      breg[s][c] = *reinterpret_cast<const uint4 *>(xp[c] + (BLK) * kKB + s * 32)
 #define NV_GEMM_COMPUTE()                                                                           \
   _Pragma("unroll") for (int s = 0; s < kSteps; ++s) _Pragma("unroll") for (int j = 0; j < NR; ++j) { \
     const uint4 a = *reinterpret_cast<const uint4 *>(a_read + j * kTileElems + s * 32);             \
-    acc[j][0] = mfma_k32<DT>(a, breg[s][0], acc[j][0]);                                             \
-    acc[j][1] = mfma_k32<DT>(a, breg[s][1], acc[j][1]);                                             \
+    _Pragma("unroll") for (int c = 0; c < TT; ++c) acc[j][c] = mfma_k32<DT>(a, breg[s][c], acc[j][c]); \
   }
 
   // Order of requests per block: this block's X pieces, then the next block of W. Loads return in
@@ -121,20 +124,23 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
 
   // ---- partial sums of the 8 waves meet in LDS (the W tiles are done with)
   __syncthreads();
-  float *red = reinterpret_cast<float *>(smem);  // [wave][j][row 16][token 32]
+  float *red = reinterpret_cast<float *>(smem);  // [wave][j][row 16][token kTokCap]
 #pragma unroll
   for (int j = 0; j < NR; ++j)
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < TT; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        red[((wave * NR + j) * 16 + q * 4 + r) * kGemmMaxTokens + c * 16 + n] = acc[j][c][r];
+        red[((wave * NR + j) * 16 + q * 4 + r) * kTokCap + c * 16 + n] = acc[j][c][r];
   __syncthreads();
-  // one thread per output element of a row group: 16 rows x 32 tokens, rows fastest (contiguous stores
-  // per token); the row groups in turn
-  const uint32_t r = threadIdx.x & 15u, t = threadIdx.x >> 4;
-  if (t >= T) return;
+  // one thread per output element of a row group: 16 rows x 32 tokens at a time, rows fastest (contiguous
+  // stores per token); the row groups in turn
+  const uint32_t r = threadIdx.x & 15u;
   const uint32_t wg_row0 = row0 - group * kGroupRows;
+#pragma unroll
+  for (int half = 0; half < TT / 2; ++half) {
+  const uint32_t t = (threadIdx.x >> 4) + 32u * half;
+  if (t >= T) break;
 #pragma unroll
   for (int gq = 0; gq < kGroups; ++gq) {
     const uint32_t grow0 = wg_row0 + gq * kGroupRows;
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
     for (int j = 0; j < NR; ++j) {
       float sum = 0.0f;
 #pragma unroll
-      for (int w = 0; w < KW; ++w) sum += red[(((gq * KW + w) * NR + j) * 16 + r) * kGemmMaxTokens + t];
+      for (int w = 0; w < KW; ++w) sum += red[(((gq * KW + w) * NR + j) * 16 + r) * kTokCap + t];
       if (p.bias != nullptr) sum += dec16<DT>(p.bias[grow0 + j * tile_rows + r]);
       y[j] = sum;
     }
@@ -161,6 +167,7 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
         p.out_f32[at + j * 16] = v;
       }
     }
+  }
   }
 }
 
@@ -206,8 +213,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const float 
   }
 }
 
-template <uint32_t DT, int EPI, int RT, int KW>
-hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
+template <uint32_t DT, int EPI, int RT, int KW, int TT>
+hipError_t launch_tt(const GemmRowsParams &p, hipStream_t stream) {
   constexpr int NR = EPI == kGemmSwiglu ? 2 : RT;
   constexpr uint32_t kWgRows = (EPI == kGemmSwiglu ? 16u : 16u * RT) * (kGW / KW);
   constexpr size_t lds = gemm_lds_bytes<NR>();
@@ -216,13 +223,20 @@ hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI, RT, KW>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<DT, EPI, RT, KW, TT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI, RT, KW>), dim3((p.rows + kWgRows - 1) / kWgRows), dim3(kGThreads), lds, stream, p);
+  hipLaunchKernelGGL((gemm_rows_kernel<DT, EPI, RT, KW, TT>), dim3((p.rows + kWgRows - 1) / kWgRows), dim3(kGThreads), lds, stream, p);
   return hipGetLastError();
+}
+
+// More than 32 token rows: four token tiles (eight waves along K only).
+template <uint32_t DT, int EPI, int RT, int KW>
+hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
+  if (p.tokens > 32) return launch_tt<DT, EPI, RT, 8, 4>(p, stream);
+  return launch_tt<DT, EPI, RT, KW, 2>(p, stream);
 }
 
 template <uint32_t DT>

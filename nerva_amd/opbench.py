@@ -160,7 +160,7 @@ def case_gemm_rows():
         wrows = rows * (2 if epi == 2 else 1)
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
         w = synth16(copies * wrows * cols, 61)
-        for tokens in (1, 8, 32):
+        for tokens in (1, 8, 32, 64):
             x = synth16(tokens * cols, 62, std=1.0)
             y32 = DeviceBuffer(tokens * rows * 4)
             y16 = DeviceBuffer(tokens * rows * 2)

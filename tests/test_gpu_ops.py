@@ -123,7 +123,8 @@ def test_gemv_rmsnorm_prologue(dtype, cols, rows):
 @pytest.mark.parametrize("dtype", [BF16, F16])
 @pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 1), (48, 2048, 5), (32, 4096, 16), (16, 2048, 17),
                                                (1000, 2048, 9), (25, 2048, 32),   # row counts off the 16-row grid
-                                               (6144, 4096, 32), (4096, 12288, 31)])
+                                               (64, 2048, 33), (48, 4096, 49), (1000, 2048, 64),   # more than two token tiles
+                                               (6144, 4096, 32), (4096, 12288, 31), (6144, 4096, 64)])
 def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
     """Multi-row projection on the matrix cores: every token row equals the oracle's GEMV of that row
     (plain, and with bias + residual + 16-bit rounding as the prompt staging of the down projection uses)."""
@@ -153,7 +154,7 @@ def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
 
 
 @pytest.mark.parametrize("dtype", [BF16, F16])
-@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 3), (12288, 4096, 32)])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 3), (64, 2048, 57), (12288, 4096, 32), (12288, 4096, 64)])
 def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
     """Fused gate/up projection of a token block: out16 = round16(silu(gate) * up), gate rows first."""
     if dtype == F16 and inter > 1000:
@@ -176,7 +177,7 @@ def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
 
 def test_gemm_rows_rejects_unsupported_shapes():
     w, x, y = N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16)
-    for rows, cols, tokens in ((8, 2048, 4), (16, 1024, 4), (16, 2048, 33), (16, 2048, 0)):
+    for rows, cols, tokens in ((8, 2048, 4), (16, 1024, 4), (16, 2048, 65), (16, 2048, 0)):
         with pytest.raises(RuntimeError):
             N.gemm_rows(BF16, w, rows, cols, tokens, x, out_f32=y)
     with pytest.raises(RuntimeError):      # rows off the 16-row grid: no residual added in place

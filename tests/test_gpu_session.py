@@ -653,13 +653,13 @@ PREFILL_GEOMETRIES = [
 
 @pytest.mark.parametrize("geom", PREFILL_GEOMETRIES)
 def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
-    """start() sends the prompt through the layers in blocks of up to 32 tokens (multi-row GEMMs, one
+    """start() sends the prompt through the layers in blocks of up to 64 tokens (multi-row GEMMs, one
     attention launch per block); NERVA_HIP_PREFILL=walk keeps one prompt step per token. Same staging,
     so both agree with each other and with the oracle to the end-to-end tolerance, over three blocks."""
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 1234, theta, qk_norm, bias)
-    prompt = np.random.default_rng(8).integers(0, vocab, 70).astype(np.uint32)
-    ctx = O.Context(omodel, 96, staging=1)
+    prompt = np.random.default_rng(8).integers(0, vocab, 150).astype(np.uint32)
+    ctx = O.Context(omodel, 160, staging=1)
     for i, tok in enumerate(prompt):
         ctx.forward_token(int(tok), prompt_token=True, want_logits=(i == len(prompt) - 1))
     ref_logits = ctx.logits()
@@ -669,13 +669,13 @@ def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
             monkeypatch.setenv("NERVA_HIP_PREFILL", "walk")
         else:
             monkeypatch.delenv("NERVA_HIP_PREFILL", raising=False)
-        s = N.DecodeSession.create(weights, 96)
+        s = N.DecodeSession.create(weights, 160)
         rc, res = s.start(prompt)
         assert rc == 0 and res.hot_path_allocations == 0
         logits = s.logits()
         assert rel_l2(logits, ref_logits) <= E2E_REL_L2
         for layer in range(layers):
-            for token in (0, 15, 31, 32, 47, 68, 69):     # block edges included
+            for token in (0, 15, 31, 32, 47, 63, 64, 65, 127, 128, 129, 148, 149):     # block and tile edges included
                 gk, gv = s.kv_row(layer, token)
                 rk, rv = ctx.read_kv16(layer, token)
                 tol = 2e-3 if layer == 0 else E2E_REL_L2
@@ -861,9 +861,9 @@ def test_batch_advance_one_eligibility_and_reasons():
         s.destroy()
 
 
-@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65])
+@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65, 66, 129, 130])
 def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
-    """Prompt lengths around the 32-token block size (the last prompt token always goes through the
+    """Prompt lengths around the prefill block sizes (the last prompt token always goes through the
     ordinary head step, so length - 1 tokens are prefilled in blocks): logits, first token and K/V
     rows agree with the token walk to the end-to-end tolerance; a context exactly as long as the
     sequence needs is enough."""
