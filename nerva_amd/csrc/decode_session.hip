@@ -101,6 +101,7 @@ struct NervaHipHfDecodeSequenceSession {
   hipStream_t stream = nullptr;
   SharedWeights *weights = nullptr;  // shared with forks
   char *arena = nullptr;             // everything but the weights: KV cache, sequence state, activations, workspaces
+  bool arena_in_weights = false;     // `arena` lies behind the weights in their allocation (the creating session)
   uint64_t state_bytes = 0;          // size of `arena`
   uint64_t arena_bytes = 0;          // weights + state, as reported to the caller
   char *pinned = nullptr;
@@ -290,7 +291,7 @@ void destroy_session(Session *s) {
   }
   if (s->ev0) (void)hipEventDestroy(s->ev0);
   if (s->ev1) (void)hipEventDestroy(s->ev1);
-  if (s->arena) (void)hipFree(s->arena);
+  if (s->arena && !s->arena_in_weights) (void)hipFree(s->arena);
   if (s->weights != nullptr && s->weights->refs.fetch_sub(1) == 1) {
     if (s->weights->base) (void)hipFree(s->weights->base);
     delete s->weights;
@@ -933,7 +934,9 @@ hipError_t copy_weight_descriptors(const NervaHipHfDecodeSequenceSessionCreateRe
 // Everything of a session that is not weights, from the dimensions already in `s`: stream, events,
 // the state arena (KV cache, block table, prompt, token slots, cursor words, activations and
 // workspaces), the pinned host mirrors, the step modes. Shared by create and fork.
-hipError_t setup_state(Session *s, int32_t *failure_stage) {
+// with_weights: one allocation holds the weights (s->weights->bytes, not allocated yet) and, behind
+// them, this session's state; it lives as long as any session uses the weights.
+hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t H = s->hidden, A = static_cast<uint64_t>(s->heads) * s->head_dim,
                  KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim, I = s->intermediate, V = s->vocab,
                  L = s->layers, HD = s->head_dim;
@@ -1000,7 +1003,15 @@ hipError_t setup_state(Session *s, int32_t *failure_stage) {
 
   *failure_stage = 2;
   hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
-  if (err == hipSuccess) err = counted_malloc(reinterpret_cast<void **>(&s->arena), s->state_bytes);
+  if (err == hipSuccess && with_weights) {
+    err = counted_malloc(reinterpret_cast<void **>(&s->weights->base), s->weights->bytes + s->state_bytes);
+    if (err == hipSuccess) {
+      s->arena = s->weights->base + s->weights->bytes;
+      s->arena_in_weights = true;
+    }
+  } else if (err == hipSuccess) {
+    err = counted_malloc(reinterpret_cast<void **>(&s->arena), s->state_bytes);
+  }
   if (err != hipSuccess) return err;
   *failure_stage = 3;
   const uint64_t pinned_seq = (static_cast<uint64_t>(s->max_ctx) * (sizeof(Slot) + 4) + 256 + 255u) & ~uint64_t{255};
@@ -1286,8 +1297,14 @@ int create_impl(const NervaHipHfDecodeSequenceSessionCreateRequest *rq, bool syn
   }
 
   out->failure_stage = 2;
-  hipError_t err = counted_malloc(reinterpret_cast<void **>(&s->weights->base), s->weights->bytes);
-  if (err == hipSuccess) err = setup_state(s, &out->failure_stage);
+  // NERVA_HIP_SPLIT_ARENAS=1: weights and state of the creating session in two allocations (comparisons)
+  static const bool split_arenas = [] {
+    const char *v = getenv("NERVA_HIP_SPLIT_ARENAS");
+    return v != nullptr && v[0] == '1';
+  }();
+  hipError_t err = hipSuccess;
+  if (split_arenas) err = counted_malloc(reinterpret_cast<void **>(&s->weights->base), s->weights->bytes);
+  if (err == hipSuccess) err = setup_state(s, &out->failure_stage, !split_arenas);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     destroy_session(s);
@@ -1603,7 +1620,7 @@ int nerva_hip_hf_decode_sequence_session_fork_shared_weights(
   s->lm_head = parent->lm_head;
   s->layer = parent->layer;
 
-  hipError_t err = setup_state(s, &out->failure_stage);
+  hipError_t err = setup_state(s, &out->failure_stage, false);
   uint64_t syncs = 1;
   if (err == hipSuccess && clone) {
     err = hipStreamSynchronize(parent->stream);
