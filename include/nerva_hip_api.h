@@ -530,7 +530,7 @@ uint64_t nerva_hip_argmax_workspace_bytes(void);
 typedef struct NervaHipGemmRowsRequest {
   uint32_t dtype;            /* NERVA_HIP_DTYPE_* of weights and 16-bit vectors */
   uint32_t rows, cols;       /* W is row-major [rows x cols] (epilogue 2: [2*rows x cols], gate rows first) */
-  uint32_t tokens;           /* 1..32 input rows */
+  uint32_t tokens;           /* 1..64 input rows */
   uint32_t epilogue;         /* 0: f32 out; 1: f32 out = y + bias + residual; 2: out16 = round16(silu(gate)*up) */
   uint32_t round_output;     /* epilogue 1: round the sum to 16 bits (prompt-token staging) */
   const uint16_t *weights;
@@ -539,6 +539,11 @@ typedef struct NervaHipGemmRowsRequest {
   const float *residual;     /* epilogue 1: [tokens][rows] */
   float *output_f32;         /* epilogues 0, 1: [tokens][rows] */
   uint16_t *output16;        /* epilogue 2: [tokens][rows] */
+  /* != 0: input16 / output16 are in matrix-operand order instead of [tokens][cols] rows, the layout
+   * the kernel reads with full cache lines: element (token t, column k) at index
+   * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 above
+   * (slots past `tokens` are never looked at). */
+  uint32_t input_operand_order, output16_operand_order;
 } NervaHipGemmRowsRequest;
 
 /* Projection of a block of up to 64 token rows through one weight matrix on the matrix cores,
@@ -547,6 +552,9 @@ typedef struct NervaHipGemmRowsRequest {
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must
  * not alias the output), cols % 2048 == 0. */
 int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *request, void *stream, int32_t *hip_error);
+/* Index of element (token, column) of a block of `tokens` rows in matrix-operand order: for every 32
+ * columns and every 16 tokens, 64 pieces of 8 columns, piece (column % 32 / 8) * 16 + token % 16. */
+uint64_t nerva_hip_gemm_operand_index(uint32_t tokens, uint32_t token, uint32_t column);
 /* out16[t] = round16(rmsnorm(x[t]) * gamma) for `tokens` rows of `cols` f32 values
  * (rms_norm_encoded_into, ops.rs:31-50, once per row). */
 int nerva_hip_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,

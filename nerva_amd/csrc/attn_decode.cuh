@@ -74,7 +74,20 @@ struct AttnParams {
   // Applies to z = 0 as well, and to a block of one token. With append = 1 every sequence's new row
   // is written to its cache by the launch itself.
   const AttnSeq *seqs;
+  // Block launches only: != 0 writes out16 in the multi-row GEMM's operand order (gemm_x_packed_index)
+  // with this many token tiles, instead of [token][heads * head_dim] rows.
+  uint32_t out_packed_tiles;
 };
+
+// Index of output element e (= head * head_dim + dim) behind a token's out16 base.
+__host__ __device__ __forceinline__ uint32_t attn_out_elem(const AttnParams &p, uint32_t e) {
+  return p.out_packed_tiles != 0 ? (e / 32u) * p.out_packed_tiles * 512u + ((e % 32u) / 8u) * 128u + e % 8u : e;
+}
+// Offset of token z's out16 base.
+__host__ __device__ __forceinline__ uint64_t attn_out_token(const AttnParams &p, uint32_t z) {
+  return p.out_packed_tiles != 0 ? static_cast<uint64_t>(z / 16u) * 512u + (z % 16u) * 8u
+                                 : static_cast<uint64_t>(z) * p.out_token_stride;
+}
 
 // Split-KV factor. The matrix-core kernel keeps one 8-wave workgroup per CU, so kv_heads x splits
 // stays within the 256 CUs (a second round of workgroups costs more than the shorter tile loops

@@ -37,7 +37,7 @@ __device__ __forceinline__ void token_view(AttnParams &p, uint32_t z) {
     p.position += z;
   }
   p.qkv += static_cast<uint64_t>(z) * p.qkv_token_stride;
-  p.out16 += static_cast<uint64_t>(z) * p.out_token_stride;
+  p.out16 += attn_out_token(p, z);
   if (p.out_f32 != nullptr) p.out_f32 += static_cast<uint64_t>(z) * p.out_token_stride;
   if (p.rope_cs != nullptr) p.rope_cs += static_cast<uint64_t>(z) * p.rope_token_stride;
   const uint64_t ws = z * p.ws_token_stride;
@@ -320,6 +320,8 @@ hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t s
   if (p.splits > kAttnMaxSplits) return hipErrorInvalidValue;
   if (p.cursor == nullptr && p.seqs == nullptr &&
       static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
+    return hipErrorInvalidValue;
+  if (p.out_packed_tiles != 0 && (!(p.tokens > 1 || p.seqs != nullptr) || p.out_packed_tiles * 16u < p.tokens || p.out_f32 != nullptr))
     return hipErrorInvalidValue;
   if (p.tokens > 1 || p.seqs != nullptr) {
     // a block of positions or of sequences: host-given positions, matrix-core kernel only

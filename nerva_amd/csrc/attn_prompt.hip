@@ -156,7 +156,7 @@ __global__ __launch_bounds__(kPW *kWave) void attn_prompt_kernel(AttnParams p) {
       uint2 packed;
       packed.x = enc16<DT>(o.x * inv) | (static_cast<uint32_t>(enc16<DT>(o.y * inv)) << 16);
       packed.y = enc16<DT>(o.z * inv) | (static_cast<uint32_t>(enc16<DT>(o.w * inv)) << 16);
-      *reinterpret_cast<uint2 *>(p.out16 + static_cast<uint64_t>(tok) * p.out_token_stride + h * kHD + d) = packed;
+      *reinterpret_cast<uint2 *>(p.out16 + attn_out_token(p, tok) + attn_out_elem(p, h * kHD + d)) = packed;   // d % 4 == 0
     } else {
       *reinterpret_cast<float4 *>(reinterpret_cast<float *>(ws) + (static_cast<uint64_t>(h) * S + split) * kHD + d) = o;
     }
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(kHD) void attn_prompt_merge_kernel(AttnParams p, ui
     M = Mc;
   }
   if (L > 0.0f && isfinite(L)) o /= L;
-  p.out16[static_cast<uint64_t>(tok) * p.out_token_stride + h * kHD + d] = enc16<DT>(o);
+  p.out16[attn_out_token(p, tok) + attn_out_elem(p, h * kHD + d)] = enc16<DT>(o);
 }
 
 template <uint32_t DT>
@@ -246,6 +246,7 @@ hipError_t launch_attn_prompt(uint32_t dtype, const AttnParams &p, hipStream_t s
   if (static_cast<uint64_t>(p.position) + p.tokens > static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;
   if (p.rope_freq != nullptr && p.rope_cs == nullptr) return hipErrorInvalidValue;   // rotation tables per token row
+  if (p.out_packed_tiles != 0 && p.out_packed_tiles * 16u < p.tokens) return hipErrorInvalidValue;
   // enough splits of the prefix to spread the block over the chip, at least eight tiles each
   const uint32_t group_tokens = kPW * (kVG / group);
   const uint32_t groups = (p.tokens + group_tokens - 1) / group_tokens;

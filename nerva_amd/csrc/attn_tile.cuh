@@ -640,7 +640,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
       if (L > 0.0f && isfinite(L)) o /= L;
       if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
       const uint16_t o16 = enc16<DT>(o);
-      p.out16[h * kHD + d] = o16;
+      p.out16[attn_out_elem(p, h * kHD + d)] = o16;
       if constexpr (LINKED) store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
     } else if constexpr (LINKED) {
       uint64_t *rec = link.part_tagged + (static_cast<uint64_t>(h) * S + split) * kPartRecord;
@@ -755,7 +755,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     attn_raise_hints(link, kvh);
     if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
     const uint16_t o16 = enc16<DT>(o);
-    p.out16[h * kHD + d] = o16;
+    p.out16[attn_out_elem(p, h * kHD + d)] = o16;
     store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
     link_mark(trm, 17);
     return;
@@ -815,7 +815,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     }
     if (L > 0.0f && isfinite(L)) o /= L;
     if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
-    p.out16[h * kHD + d] = enc16<DT>(o);
+    p.out16[attn_out_elem(p, h * kHD + d)] = enc16<DT>(o);
   }
   if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   link_mark(trm, 17);

@@ -681,6 +681,17 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
   return err;
 }
 
+// Token blocks (prompt blocks, batch steps) keep their 16-bit activations - normalised rows, attention
+// output, SwiGLU output: the X operands of the multi-row GEMMs - in matrix-operand order, which the GEMM
+// reads with full cache lines. NERVA_HIP_BLOCK_LAYOUT=rows keeps them as [token][column] rows (comparisons).
+uint32_t block_operand_tiles(uint32_t tokens) {
+  static const bool rows = [] {
+    const char *v = getenv("NERVA_HIP_BLOCK_LAYOUT");
+    return v != nullptr && v[0] == 'r';
+  }();
+  return rows ? 0u : gemm_packed_tiles(tokens);
+}
+
 // Prompt tokens 0 .. count-1 through every layer in blocks of up to kGemmMaxTokens tokens, with the
 // prompt staging (16-bit hidden state between layers, prefill_kernels.cu:494-508): per block and
 // layer one RMSNorm launch, the qkv projection as a multi-row GEMM, the K/V rows of the block into the
@@ -705,6 +716,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   }();
   for (uint32_t first = 0; err == hipSuccess && first < count; first += kGemmMaxTokens) {
     const uint32_t T = std::min<uint32_t>(kGemmMaxTokens, count - first);
+    const uint32_t tiles = block_operand_tiles(T);
     if (s->dtype == kBF16)
       hipLaunchKernelGGL(embed_rows_kernel<kBF16>, dim3(T), dim3(kBlock), 0, st, s->emb, s->prompt, first, H, s->vocab,
                          s->px, rope_freq, s->prope, s->head_dim / 2);
@@ -714,12 +726,13 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
     err = hipGetLastError();
     for (uint32_t l = 0; err == hipSuccess && l < s->layers; ++l) {
       const LayerDev &w = s->layer[l];
-      err = launch_rmsnorm_rows(s->dtype, s->px, w.rms_attn, s->eps, T, H, s->pxn16, st);
+      err = launch_rmsnorm_rows(s->dtype, s->px, w.rms_attn, s->eps, T, H, s->pxn16, st, tiles);
       GemmRowsParams g{};
       g.tokens = T;
       if (err == hipSuccess) {
         g.w = w.wqkv;
         g.x16 = s->pxn16;
+        g.x_packed = tiles;
         g.out_f32 = s->pqkv;
         g.rows = A + 2 * KV;
         g.cols = H;
@@ -752,6 +765,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
       a.out_token_stride = A;
       a.rope_token_stride = s->head_dim;
       a.ws_token_stride = s->pattn_ws_stride;
+      a.out_packed_tiles = tiles;
       if (err == hipSuccess) err = launch_kv_publish_rows(s->dtype, a, st);
       if (err == hipSuccess) {
         if (rows_attention) {
@@ -766,6 +780,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.tokens = T;
         g.w = w.wo;
         g.x16 = s->pattn16;
+        g.x_packed = tiles;
         g.bias = w.o_bias;
         g.residual = s->px;
         g.out_f32 = s->pr;
@@ -773,13 +788,15 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.cols = A;
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
-      if (err == hipSuccess) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st);
+      if (err == hipSuccess) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st, tiles);
       if (err == hipSuccess) {
         g = GemmRowsParams{};
         g.tokens = T;
         g.w = w.wgu;
         g.x16 = s->pxn16;
+        g.x_packed = tiles;
         g.out16 = s->pff16;
+        g.out_packed_tiles = tiles;
         g.rows = I;
         g.cols = H;
         err = launch_gemm_rows(s->dtype, kGemmSwiglu, g, st);
@@ -789,6 +806,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.tokens = T;
         g.w = w.wdown;
         g.x16 = s->pff16;
+        g.x_packed = tiles;
         g.residual = s->pr;
         g.out_f32 = s->px;
         g.rows = H;
@@ -1439,6 +1457,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
   const uint32_t H = lead->hidden, A = lead->heads * lead->head_dim, KV = lead->kv_heads * lead->head_dim,
                  I = lead->intermediate;
   const float *rope_freq = lead->theta > 0.0f ? lead->rope_freq : nullptr;
+  const uint32_t tiles = block_operand_tiles(T);
   BatchTable *host = lead->host_btable;
   uint32_t min_blocks = ~0u;
   for (uint32_t t = 0; t < T; ++t) {
@@ -1480,12 +1499,13 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
   out->pack_kernel_launches += 1;
   for (uint32_t l = 0; err == hipSuccess && l < lead->layers; ++l) {
     const LayerDev &w = lead->layer[l];
-    err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st);
+    err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st, tiles);
     GemmRowsParams g{};
     if (err == hipSuccess) {
       g.tokens = T;
       g.w = w.wqkv;
       g.x16 = lead->pxn16;
+      g.x_packed = tiles;
       g.out_f32 = lead->pqkv;
       g.rows = A + 2 * KV;
       g.cols = H;
@@ -1514,6 +1534,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     a.rope_token_stride = lead->head_dim;
     a.ws_token_stride = lead->pattn_ws_stride;
     a.seqs = lead->btable->seq;
+    a.out_packed_tiles = tiles;
     a.append = 1;  // each sequence's K/V row goes into its own cache inside the attention launch
     if (err == hipSuccess) err = launch_attn_decode(lead->dtype, a, st);
     if (err == hipSuccess) {
@@ -1521,6 +1542,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.tokens = T;
       g.w = w.wo;
       g.x16 = lead->pattn16;
+      g.x_packed = tiles;
       g.bias = w.o_bias;
       g.residual = lead->px;
       g.out_f32 = lead->pr;
@@ -1528,13 +1550,15 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.cols = A;
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
-    if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st);
+    if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st, tiles);
     if (err == hipSuccess) {
       g = GemmRowsParams{};
       g.tokens = T;
       g.w = w.wgu;
       g.x16 = lead->pxn16;
+      g.x_packed = tiles;
       g.out16 = lead->pff16;
+      g.out_packed_tiles = tiles;
       g.rows = I;
       g.cols = H;
       err = launch_gemm_rows(lead->dtype, kGemmSwiglu, g, st);
@@ -1544,6 +1568,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.tokens = T;
       g.w = w.wdown;
       g.x16 = lead->pff16;
+      g.x_packed = tiles;
       g.residual = lead->pr;
       g.out_f32 = lead->px;
       g.rows = H;
@@ -1554,12 +1579,13 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     out->projection_kernel_launches += 4;
     out->dependency_kernel_launches += 1;
   }
-  if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st);
+  if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st, tiles);
   if (err == hipSuccess) {
     GemmRowsParams g{};
     g.tokens = T;
     g.w = lead->lm_head;
     g.x16 = lead->pxn16;
+    g.x_packed = tiles;
     g.out_f32 = lead->blogits;
     g.rows = lead->vocab;
     g.cols = H;

@@ -21,6 +21,16 @@
 namespace nv {
 
 constexpr uint32_t kGemmMaxTokens = 64;
+
+// Operand order of a block of token rows X[t][k] (16-bit), the layout the multi-row GEMM reads fastest:
+// for every K-step of 32 columns and every tile of 16 tokens the 64 lanes' 16-byte pieces in lane order,
+// lane = (k % 32 / 8) * 16 + t % 16 holding columns k - k % 8 .. + 7 of token t. `tiles` token tiles per
+// K-step; a buffer holds tiles * 16 token slots (slots past the block's tokens are never looked at).
+__host__ __device__ __forceinline__ uint64_t gemm_x_packed_index(uint32_t tiles, uint32_t t, uint32_t k) {
+  return (static_cast<uint64_t>(k / 32u) * tiles + t / 16u) * 512u + (((k % 32u) / 8u) * 16u + t % 16u) * 8u + k % 8u;
+}
+// Token tiles the GEMM works with for a block of `tokens` rows (its X buffer in operand order has as many).
+__host__ __device__ __forceinline__ uint32_t gemm_packed_tiles(uint32_t tokens) { return tokens > 32u ? 4u : 2u; }
 enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
 
 struct GemmRowsParams {
@@ -32,6 +42,9 @@ struct GemmRowsParams {
   uint16_t *out16;           // kGemmSwiglu: [tokens][rows] = round16(silu(gate) * up)
   uint32_t rows, cols, tokens;
   uint32_t round_out;        // kGemmResidual: round the sum to 16 bit
+  uint32_t x_packed;         // != 0: x16 is in matrix-operand order (gemm_x_packed_index) instead of [tokens][cols];
+                             // the value is its token-tile count and must be gemm_packed_tiles(tokens)
+  uint32_t out_packed_tiles; // kGemmSwiglu: != 0 writes out16 in operand order with this many token tiles
 };
 
 // rows >= 16 (any count: the last workgroup overlaps its neighbour, so with a row count that is no
@@ -41,7 +54,8 @@ bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens);
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream);
 
 // x16[t] = round16(x[t] * rsqrt(mean(x[t]^2) + eps) * gamma) for `tokens` rows of `cols` f32 values.
+// packed_tiles != 0: out16 in operand order (gemm_x_packed_index) with that many token tiles.
 hipError_t launch_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,
-                               uint32_t cols, uint16_t *out16, hipStream_t stream);
+                               uint32_t cols, uint16_t *out16, hipStream_t stream, uint32_t packed_tiles = 0);
 
 }  // namespace nv

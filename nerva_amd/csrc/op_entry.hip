@@ -458,7 +458,13 @@ int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *r, void *stream, int32_t 
   p.cols = r->cols;
   p.tokens = r->tokens;
   p.round_out = r->round_output;
+  p.x_packed = r->input_operand_order != 0 ? gemm_packed_tiles(r->tokens) : 0u;
+  p.out_packed_tiles = r->output16_operand_order != 0 ? gemm_packed_tiles(r->tokens) : 0u;
   return finish(launch_gemm_rows(r->dtype, static_cast<int>(r->epilogue), p, resolve_stream(stream)), hip_error);
+}
+
+uint64_t nerva_hip_gemm_operand_index(uint32_t tokens, uint32_t token, uint32_t column) {
+  return gemm_x_packed_index(gemm_packed_tiles(tokens), token, column);
 }
 
 int nerva_hip_rmsnorm_rows(uint32_t dtype, const float *x, const uint16_t *gamma, float eps, uint32_t tokens,

@@ -161,13 +161,16 @@ def case_gemm_rows():
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
         w = synth16(copies * wrows * cols, 61)
         for tokens in (1, 8, 32, 64):
-            x = synth16(tokens * cols, 62, std=1.0)
+            x = synth16(max(tokens, 64) * cols, 62, std=1.0)
             y32 = DeviceBuffer(tokens * rows * 4)
-            y16 = DeviceBuffer(tokens * rows * 2)
+            y16 = DeviceBuffer(max(tokens, 64) * rows * 2)
             nbytes = wrows * cols * 2 + tokens * cols * 2 + tokens * rows * (2 if epi == 2 else 4)
-            ns = timed(lambda i: R.gemm_rows(BF16, w.at((i % copies) * wrows * cols * 2), rows, cols, tokens, x, epilogue=epi,
-                                             out_f32=y32, out16=y16, sync=False), 2 * copies)
-            report("6 %s" % name, "T=%d" % tokens, ns, nbytes)
+            # "operand order": the activations in the layout token blocks keep inside the session
+            for packed in ((False,) if tokens < 32 else (False, True)):
+                ns = timed(lambda i: R.gemm_rows(BF16, w.at((i % copies) * wrows * cols * 2), rows, cols, tokens, x, epilogue=epi,
+                                                 out_f32=y32, out16=y16, sync=False, input_operand_order=packed,
+                                                 output16_operand_order=packed and epi == 2), 2 * copies)
+                report("6 %s" % name, "T=%d%s" % (tokens, " operand order" if packed else ""), ns, nbytes)
 
 
 def case_sampler():

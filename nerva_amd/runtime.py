@@ -236,11 +236,29 @@ def argmax(logits_buf, count, workspace=None):
     return int(tok.numpy(np.uint32, 1)[0])
 
 
+def gemm_operand_order(x, tokens=None):
+    """A [tokens][cols] block of 16-bit rows rearranged into the matrix-operand order the multi-row GEMM
+    reads fastest (index of every element from the library); slots past `tokens` stay zero."""
+    lib = abi.load()
+    x = np.ascontiguousarray(x, np.uint16)
+    tokens = x.shape[0] if tokens is None else tokens
+    cols = x.shape[1]
+    out = np.zeros((32 if tokens <= 32 else 64) * cols, np.uint16)
+    t, k = np.meshgrid(np.arange(tokens), np.arange(cols), indexing="ij")
+    # the index is affine in (token % 16, token // 16) and in the column's three digits: probe it once per digit
+    base = lambda tt, kk: int(lib.nerva_hip_gemm_operand_index(tokens, tt, kk))
+    idx = (np.array([base(i, 0) for i in range(tokens)])[t]
+           + np.array([base(0, j) for j in range(cols)])[k])
+    out[idx] = x[:tokens]
+    return out, idx
+
+
 def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None, residual=None, out_f32=None,
-              out16=None, round_output=False, sync=True):
-    """Y[t] = W . X[t] for up to 32 token rows on the matrix cores (weights streamed once)."""
+              out16=None, round_output=False, sync=True, input_operand_order=False, output16_operand_order=False):
+    """Y[t] = W . X[t] for up to 64 token rows on the matrix cores (weights streamed once)."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()
+    req.input_operand_order, req.output16_operand_order = int(input_operand_order), int(output16_operand_order)
     req.dtype, req.rows, req.cols, req.tokens, req.epilogue, req.round_output = dtype, rows, cols, tokens, epilogue, int(round_output)
     req.weights, req.input16, req.bias, req.residual = _ptr(weights), _ptr(input16), _ptr(bias), _ptr(residual)
     req.output_f32, req.output16 = _ptr(out_f32), _ptr(out16)

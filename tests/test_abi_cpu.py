@@ -258,3 +258,20 @@ def test_batch_step_over_nothing_and_null_fork_need_no_device(lib):
     assert cres.status == -1 and cres.failure_stage == 1 and not handle
     assert lib.nerva_hip_hf_decode_sequence_session_fork_shared_weights(None, C.byref(cres), C.byref(handle)) == -1
     assert lib.nerva_hip_session_shares_weight_stream(None) == -1
+
+
+def test_operand_order_index_is_the_matrix_core_operand_layout(lib):
+    """nerva_hip_gemm_operand_index (host arithmetic): per 32 columns and 16 tokens, 64 pieces of 8
+    columns in lane order, lane = (column % 32 / 8) * 16 + token % 16 - the B operand of a 16x16x32
+    matrix-core product; 2 token tiles per K-step up to 32 tokens, 4 above; a bijection onto the buffer."""
+    f = lib.nerva_hip_gemm_operand_index
+    for tokens, tiles in ((1, 2), (32, 2), (33, 4), (64, 4)):
+        cols = 96
+        seen = set()
+        for t in range(tiles * 16):
+            for k in range(cols):
+                i = f(tokens, t, k)
+                lane = (k % 32 // 8) * 16 + t % 16
+                assert i == ((k // 32) * tiles + t // 16) * 512 + lane * 8 + k % 8
+                seen.add(i)
+        assert seen == set(range(tiles * 16 * cols))

@@ -608,3 +608,30 @@ def test_operator_timer_records_launches_into_a_graph():
     assert lib.nerva_hip_timer_capture_end(2, 4, C.byref(nodes), C.byref(ns)) == 0
     assert nodes.value == 5 and ns.value > 0
     assert rel_l2(y.numpy(np.float32), O.gemv(BF16, w, O.decode16(BF16, x))) <= REL_L2
+
+
+@pytest.mark.parametrize("tokens,rows,cols", [(5, 48, 2048), (32, 1000, 2048), (33, 64, 4096), (64, 4096, 4096)])
+def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
+    """Inputs and SwiGLU outputs in matrix-operand order (what prompt blocks and batch steps keep between
+    their kernels) only change where bytes lie: the results are bit-identical to the row-major call."""
+    dtype = BF16
+    rng = np.random.default_rng(tokens * rows)
+    w = O.encode16(dtype, rng.normal(0, 0.05, (rows, cols)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, cols)))
+    packed, idx = N.gemm_operand_order(x)
+    assert np.array_equal(packed[idx], x) and len(np.unique(idx)) == idx.size      # a permutation into the buffer
+    dw = dev(w)
+    y0, y1 = N.DeviceBuffer(tokens * rows * 4), N.DeviceBuffer(tokens * rows * 4)
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dev(x), out_f32=y0)
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dev(packed), out_f32=y1, input_operand_order=True)
+    assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
+    if rows % 2 == 0 and (rows // 2) % 32 == 0:
+        inter = rows // 2                                                          # the same matrix as [gate; up]
+        o0 = N.DeviceBuffer(tokens * inter * 2)
+        o1 = N.DeviceBuffer.zeros((32 if tokens <= 32 else 64) * inter * 2)
+        N.gemm_rows(dtype, dw, inter, cols, tokens, dev(x), epilogue=2, out16=o0)
+        N.gemm_rows(dtype, dw, inter, cols, tokens, dev(packed), epilogue=2, out16=o1, input_operand_order=True,
+                    output16_operand_order=True)
+        rowmajor = o0.numpy(np.uint16, tokens * inter).reshape(tokens, inter)
+        _, oidx = N.gemm_operand_order(np.zeros((tokens, inter), np.uint16))
+        assert np.array_equal(o1.numpy(np.uint16)[oidx], rowmajor)
