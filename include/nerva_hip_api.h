@@ -530,7 +530,7 @@ uint64_t nerva_hip_argmax_workspace_bytes(void);
 typedef struct NervaHipGemmRowsRequest {
   uint32_t dtype;            /* NERVA_HIP_DTYPE_* of weights and 16-bit vectors */
   uint32_t rows, cols;       /* W is row-major [rows x cols] (epilogue 2: [2*rows x cols], gate rows first) */
-  uint32_t tokens;           /* 1..64 input rows */
+  uint32_t tokens;           /* 1..128 input rows */
   uint32_t epilogue;         /* 0: f32 out; 1: f32 out = y + bias + residual; 2: out16 = round16(silu(gate)*up) */
   uint32_t round_output;     /* epilogue 1: round the sum to 16 bits (prompt-token staging) */
   const uint16_t *weights;
@@ -541,12 +541,12 @@ typedef struct NervaHipGemmRowsRequest {
   uint16_t *output16;        /* epilogue 2: [tokens][rows] */
   /* != 0: input16 / output16 are in matrix-operand order instead of [tokens][cols] rows, the layout
    * the kernel reads with full cache lines: element (token t, column k) at index
-   * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 above
+   * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 for tokens <= 64, 128 above
    * (slots past `tokens` are never looked at). */
   uint32_t input_operand_order, output16_operand_order;
 } NervaHipGemmRowsRequest;
 
-/* Projection of a block of up to 64 token rows through one weight matrix on the matrix cores,
+/* Projection of a block of up to 128 token rows through one weight matrix on the matrix cores,
  * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
  * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must

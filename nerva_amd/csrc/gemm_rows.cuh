@@ -1,5 +1,5 @@
 // Multi-row projection on the matrix cores: Y[t][r] = sum_c W[r][c] * X[t][c] for a block of
-// T <= 64 token rows, streaming the weight matrix once for all of them. This is what a chunk of
+// T <= 128 token rows, streaming the weight matrix once for all of them. This is what a chunk of
 // prompt tokens (and a small batch of sequences) needs: the weight bytes are the same as for one
 // token, so the kernel is HBM-bound like the GEMV and T tokens cost about one.
 // Reference: the cuBLAS GEMM calls of the chunked prefill and of the projection batch
@@ -20,7 +20,7 @@
 
 namespace nv {
 
-constexpr uint32_t kGemmMaxTokens = 64;
+constexpr uint32_t kGemmMaxTokens = 128;
 
 // Operand order of a block of token rows X[t][k] (16-bit), the layout the multi-row GEMM reads fastest:
 // for every K-step of 32 columns and every tile of 16 tokens the 64 lanes' 16-byte pieces in lane order,
@@ -30,7 +30,9 @@ __host__ __device__ __forceinline__ uint64_t gemm_x_packed_index(uint32_t tiles,
   return (static_cast<uint64_t>(k / 32u) * tiles + t / 16u) * 512u + (((k % 32u) / 8u) * 16u + t % 16u) * 8u + k % 8u;
 }
 // Token tiles the GEMM works with for a block of `tokens` rows (its X buffer in operand order has as many).
-__host__ __device__ __forceinline__ uint32_t gemm_packed_tiles(uint32_t tokens) { return tokens > 32u ? 4u : 2u; }
+__host__ __device__ __forceinline__ uint32_t gemm_packed_tiles(uint32_t tokens) {
+  return tokens > 64u ? 8u : tokens > 32u ? 4u : 2u;
+}
 enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
 
 struct GemmRowsParams {

@@ -46,8 +46,8 @@ constexpr size_t gemm_lds_bytes() {
 // KW: waves of a workgroup along K (8, or 4: the workgroup then holds two row groups of four waves, and
 // the two waves that walk the same K range fetch the same X pieces at about the same time, so the
 // second fetch is served by the CU's own cache instead of L2).
-// TT: 16-token tiles a wave keeps accumulators for (2: up to 32 token rows; 4: up to 64, every W operand
-// then serves four products).
+// TT: 16-token tiles a wave keeps accumulators for (2: up to 32 token rows; 4: up to 64; 8: up to 128 -
+// every W operand then serves that many products).
 // XP: the X operand lies in matrix-operand order (gemm_x_packed_index with TT tiles) instead of row-major:
 // the 64 lanes' pieces of a (K-step, token tile) are then 1 KiB in a row and one load instruction
 // touches 8 full cache lines instead of 16 half lines of 16 different rows. Measured at 32 / 64 token
@@ -252,6 +252,7 @@ hipError_t launch_tt(const GemmRowsParams &p, hipStream_t stream) {
 // More than 32 token rows: four token tiles (eight waves along K only).
 template <uint32_t DT, int EPI, int RT, int KW>
 hipError_t launch_one(const GemmRowsParams &p, hipStream_t stream) {
+  if (p.tokens > 64) return launch_tt<DT, EPI, RT, 8, 8>(p, stream);
   if (p.tokens > 32) return launch_tt<DT, EPI, RT, 8, 4>(p, stream);
   return launch_tt<DT, EPI, RT, KW, 2>(p, stream);
 }

@@ -160,10 +160,10 @@ def case_gemm_rows():
         wrows = rows * (2 if epi == 2 else 1)
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
         w = synth16(copies * wrows * cols, 61)
-        for tokens in (1, 8, 32, 64):
-            x = synth16(max(tokens, 64) * cols, 62, std=1.0)
+        for tokens in (1, 8, 32, 64, 128):
+            x = synth16(max(tokens, 128) * cols, 62, std=1.0)
             y32 = DeviceBuffer(tokens * rows * 4)
-            y16 = DeviceBuffer(max(tokens, 64) * rows * 2)
+            y16 = DeviceBuffer(max(tokens, 128) * rows * 2)
             nbytes = wrows * cols * 2 + tokens * cols * 2 + tokens * rows * (2 if epi == 2 else 4)
             # "operand order": the activations in the layout token blocks keep inside the session
             for packed in ((False,) if tokens < 32 else (False, True)):

@@ -236,6 +236,11 @@ def argmax(logits_buf, count, workspace=None):
     return int(tok.numpy(np.uint32, 1)[0])
 
 
+def gemm_operand_slots(tokens):
+    """Token slots of a buffer in matrix-operand order for a block of `tokens` rows."""
+    return 32 if tokens <= 32 else 64 if tokens <= 64 else 128
+
+
 def gemm_operand_order(x, tokens=None):
     """A [tokens][cols] block of 16-bit rows rearranged into the matrix-operand order the multi-row GEMM
     reads fastest (index of every element from the library); slots past `tokens` stay zero."""
@@ -243,7 +248,7 @@ def gemm_operand_order(x, tokens=None):
     x = np.ascontiguousarray(x, np.uint16)
     tokens = x.shape[0] if tokens is None else tokens
     cols = x.shape[1]
-    out = np.zeros((32 if tokens <= 32 else 64) * cols, np.uint16)
+    out = np.zeros(gemm_operand_slots(tokens) * cols, np.uint16)
     t, k = np.meshgrid(np.arange(tokens), np.arange(cols), indexing="ij")
     # the index is affine in (token % 16, token // 16) and in the column's three digits: probe it once per digit
     base = lambda tt, kk: int(lib.nerva_hip_gemm_operand_index(tokens, tt, kk))
@@ -255,7 +260,7 @@ def gemm_operand_order(x, tokens=None):
 
 def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None, residual=None, out_f32=None,
               out16=None, round_output=False, sync=True, input_operand_order=False, output16_operand_order=False):
-    """Y[t] = W . X[t] for up to 64 token rows on the matrix cores (weights streamed once)."""
+    """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once)."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()
     req.input_operand_order, req.output16_operand_order = int(input_operand_order), int(output16_operand_order)

@@ -263,9 +263,9 @@ def test_batch_step_over_nothing_and_null_fork_need_no_device(lib):
 def test_operand_order_index_is_the_matrix_core_operand_layout(lib):
     """nerva_hip_gemm_operand_index (host arithmetic): per 32 columns and 16 tokens, 64 pieces of 8
     columns in lane order, lane = (column % 32 / 8) * 16 + token % 16 - the B operand of a 16x16x32
-    matrix-core product; 2 token tiles per K-step up to 32 tokens, 4 above; a bijection onto the buffer."""
+    matrix-core product; 2 token tiles per K-step up to 32 tokens, 4 up to 64, 8 above; a bijection onto the buffer."""
     f = lib.nerva_hip_gemm_operand_index
-    for tokens, tiles in ((1, 2), (32, 2), (33, 4), (64, 4)):
+    for tokens, tiles in ((1, 2), (32, 2), (33, 4), (64, 4), (65, 8), (128, 8)):
         cols = 96
         seen = set()
         for t in range(tiles * 16):

@@ -123,7 +123,7 @@ def test_gemv_rmsnorm_prologue(dtype, cols, rows):
 @pytest.mark.parametrize("dtype", [BF16, F16])
 @pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 1), (48, 2048, 5), (32, 4096, 16), (16, 2048, 17),
                                                (1000, 2048, 9), (25, 2048, 32),   # row counts off the 16-row grid
-                                               (64, 2048, 33), (48, 4096, 49), (1000, 2048, 64),   # more than two token tiles
+                                               (64, 2048, 33), (48, 4096, 49), (1000, 2048, 64), (64, 2048, 65), (1000, 2048, 128),   # more than two token tiles
                                                (6144, 4096, 32), (4096, 12288, 31), (6144, 4096, 64)])
 def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
     """Multi-row projection on the matrix cores: every token row equals the oracle's GEMV of that row
@@ -154,7 +154,7 @@ def test_gemm_rows_matches_oracle_per_token(dtype, rows, cols, tokens):
 
 
 @pytest.mark.parametrize("dtype", [BF16, F16])
-@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 3), (64, 2048, 57), (12288, 4096, 32), (12288, 4096, 64)])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 3), (64, 2048, 57), (64, 2048, 111), (12288, 4096, 32), (12288, 4096, 128)])
 def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
     """Fused gate/up projection of a token block: out16 = round16(silu(gate) * up), gate rows first."""
     if dtype == F16 and inter > 1000:
@@ -177,7 +177,7 @@ def test_gemm_rows_swiglu_matches_oracle(dtype, inter, hidden, tokens):
 
 def test_gemm_rows_rejects_unsupported_shapes():
     w, x, y = N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16), N.DeviceBuffer(1 << 16)
-    for rows, cols, tokens in ((8, 2048, 4), (16, 1024, 4), (16, 2048, 65), (16, 2048, 0)):
+    for rows, cols, tokens in ((8, 2048, 4), (16, 1024, 4), (16, 2048, 129), (16, 2048, 0)):
         with pytest.raises(RuntimeError):
             N.gemm_rows(BF16, w, rows, cols, tokens, x, out_f32=y)
     with pytest.raises(RuntimeError):      # rows off the 16-row grid: no residual added in place
@@ -610,7 +610,7 @@ def test_operator_timer_records_launches_into_a_graph():
     assert rel_l2(y.numpy(np.float32), O.gemv(BF16, w, O.decode16(BF16, x))) <= REL_L2
 
 
-@pytest.mark.parametrize("tokens,rows,cols", [(5, 48, 2048), (32, 1000, 2048), (33, 64, 4096), (64, 4096, 4096)])
+@pytest.mark.parametrize("tokens,rows,cols", [(5, 48, 2048), (32, 1000, 2048), (33, 64, 4096), (64, 4096, 4096), (65, 64, 2048), (128, 4096, 4096)])
 def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
     """Inputs and SwiGLU outputs in matrix-operand order (what prompt blocks and batch steps keep between
     their kernels) only change where bytes lie: the results are bit-identical to the row-major call."""
@@ -628,7 +628,7 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
     if rows % 2 == 0 and (rows // 2) % 32 == 0:
         inter = rows // 2                                                          # the same matrix as [gate; up]
         o0 = N.DeviceBuffer(tokens * inter * 2)
-        o1 = N.DeviceBuffer.zeros((32 if tokens <= 32 else 64) * inter * 2)
+        o1 = N.DeviceBuffer.zeros(N.gemm_operand_slots(tokens) * inter * 2)
         N.gemm_rows(dtype, dw, inter, cols, tokens, dev(x), epilogue=2, out16=o0)
         N.gemm_rows(dtype, dw, inter, cols, tokens, dev(packed), epilogue=2, out16=o1, input_operand_order=True,
                     output16_operand_order=True)
