@@ -87,14 +87,17 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
 
   // X operand: token of this lane in each of the token tiles (clamped: columns past T are dropped later)
   const uint32_t n = lane & 15, q = lane >> 4;
-  // Row-major X: lane (n, q) of token tile c reads 16 bytes of row n + 16c at column k + 8q (rows past T
-  // clamped: those columns are dropped later). Operand order: piece `lane` of (K-step, tile c).
+  // Row-major X: lane (n, q) of token tile c reads 16 bytes of row n + 16c at column k + 8q. Operand
+  // order: piece `lane` of (K-step, tile c). Either way rows past T are clamped to the last one (those
+  // columns are dropped later), so a small block touches few cache lines.
   const uint16_t *xp[TT];
   constexpr uint32_t x_step = XP ? TT * 512u : 32u;   // elements between K-steps
 #pragma unroll
-  for (int c = 0; c < TT; ++c)
-    xp[c] = XP ? p.x16 + (static_cast<uint64_t>(kbase / 32u) * TT + c) * 512u + lane * 8
-               : p.x16 + static_cast<uint64_t>(min(n + 16u * c, T - 1)) * cols + kbase + q * 8;
+  for (int c = 0; c < TT; ++c) {
+    const uint32_t tok = min(n + 16u * c, T - 1);   // lanes past the block's tokens re-read its last token
+    xp[c] = XP ? p.x16 + (static_cast<uint64_t>(kbase / 32u) * TT + tok / 16u) * 512u + (q * 16u + tok % 16u) * 8u
+               : p.x16 + static_cast<uint64_t>(tok) * cols + kbase + q * 8;
+  }
   const uint16_t *a_read = tile + n * kRowStride + q * 8;
 
   f32x4_t acc[NR][TT];
