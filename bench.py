@@ -301,7 +301,7 @@ def main():
                                      "32q/8kv x128, MLP 12288, vocab 151936, random-init bf16 N(0,0.02), batch 1, "
                                      "prompt %d prefilled, %d greedy tokens under hipGraph replay"
                                      % (cfg["layers"], args.prompt, args.steps),
-                            prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
+                            prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), prefill_tok_s=round(args.prompt / prefill_s, 1), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
                             per_token_latency_ms=latency, shared_weight_sessions=batch, gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)
