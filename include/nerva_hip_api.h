@@ -544,6 +544,11 @@ typedef struct NervaHipGemmRowsRequest {
    * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 for tokens <= 64, 128 above
    * (slots past `tokens` are never looked at). */
   uint32_t input_operand_order, output16_operand_order;
+  /* Optional device scratch of nerva_hip_gemm_rows_workspace_bytes(rows) bytes (rows doubled for
+   * epilogue 2). With more than 64 tokens in operand order the projections with few rows are split
+   * along K across workgroups, which leave f32 partial sums here; without it they run unsplit. */
+  void *workspace;
+  uint64_t workspace_bytes;
 } NervaHipGemmRowsRequest;
 
 /* Projection of a block of up to 128 token rows through one weight matrix on the matrix cores,
@@ -552,6 +557,7 @@ typedef struct NervaHipGemmRowsRequest {
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must
  * not alias the output), cols % 2048 == 0. */
 int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *request, void *stream, int32_t *hip_error);
+uint64_t nerva_hip_gemm_rows_workspace_bytes(uint32_t rows);
 /* Index of element (token, column) of a block of `tokens` rows in matrix-operand order: for every 32
  * columns and every 16 tokens, 64 pieces of 8 columns, piece (column % 32 / 8) * 16 + token % 16. */
 uint64_t nerva_hip_gemm_operand_index(uint32_t tokens, uint32_t token, uint32_t column);

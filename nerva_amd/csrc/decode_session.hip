@@ -147,6 +147,8 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *pxn16 = nullptr, *pattn16 = nullptr, *pff16 = nullptr;
   char *pattn_ws = nullptr;
   uint64_t pattn_ws_stride = 0;
+  char *pgemm_ws = nullptr;        // partial sums of the K-sliced projections of a prompt block
+  uint64_t pgemm_ws_bytes = 0;
   SamplerDev sampler{};            // normalised configuration of the active sequence
   SamplerDev *sampler_dev = nullptr;
   uint64_t *sampler_keys = nullptr;
@@ -740,6 +742,8 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.out_f32 = s->pqkv;
         g.rows = A + 2 * KV;
         g.cols = H;
+        g.workspace = s->pgemm_ws;
+        g.workspace_bytes = s->pgemm_ws_bytes;
         err = launch_gemm_rows(s->dtype, kGemmF32, g, st);
       }
       AttnParams a{};
@@ -790,6 +794,8 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.out_f32 = s->pr;
         g.rows = H;
         g.cols = A;
+        g.workspace = s->pgemm_ws;
+        g.workspace_bytes = s->pgemm_ws_bytes;
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
       if (err == hipSuccess) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st, tiles);
@@ -803,6 +809,8 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.out_packed_tiles = tiles;
         g.rows = I;
         g.cols = H;
+        g.workspace = s->pgemm_ws;
+        g.workspace_bytes = s->pgemm_ws_bytes;
         err = launch_gemm_rows(s->dtype, kGemmSwiglu, g, st);
       }
       if (err == hipSuccess) {
@@ -816,6 +824,8 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.rows = H;
         g.cols = I;
         g.round_out = 1;  // prompt tokens carry a 16-bit hidden state between layers
+        g.workspace = s->pgemm_ws;
+        g.workspace_bytes = s->pgemm_ws_bytes;
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
     }
@@ -1001,6 +1011,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_prope = c.take(pT * HD * 4);
   const uint64_t pattn_ws_stride = (attn_ws_bytes + 255u) & ~uint64_t{255};
   const uint64_t off_pattn_ws = c.take(pT * pattn_ws_stride);
+  const uint64_t pgemm_ws_bytes = gemm_block_workspace_bytes(static_cast<uint32_t>(std::max<uint64_t>(H, A + 2 * KV)));
+  const uint64_t off_pgemm_ws = c.take(pgemm_ws_bytes);
   const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
   const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(s->vocab));
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
@@ -1073,6 +1085,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->prope = reinterpret_cast<float *>(s->arena + off_prope);
   s->pattn_ws = s->arena + off_pattn_ws;
   s->pattn_ws_stride = pattn_ws_stride;
+  s->pgemm_ws = s->arena + off_pgemm_ws;
+  s->pgemm_ws_bytes = pgemm_ws_bytes;
   s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
   s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
   {

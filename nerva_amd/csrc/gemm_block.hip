@@ -1,0 +1,386 @@
+// Multi-row projection for large token blocks (65..128 rows, X in matrix-operand order): the X operand
+// is shared through LDS instead of being fetched by every wave (see gemm_rows.cuh).
+//
+// gemm_rows_kernel gives a workgroup 16 weight rows over the whole K and lets its 8 waves split K, so
+// every wave fetches its own X pieces from L2: per matrix instruction 0.6 vector-memory reads, and the
+// matrix cores are busy 8-13 % of the time. Here the waves of a workgroup split the ROWS and walk the
+// same K range, so a K-block of X (128 columns x 128 tokens = 32 KiB, contiguous in operand order) is
+// copied into LDS once per workgroup and read from there by all four waves as B operands; the weight
+// rows go from global memory straight into A-operand registers (16 rows x 64 bytes per request), two
+// K-blocks in flight per wave. A wave holds NR row tiles x 8 token tiles of f32 accumulators.
+// Projections with few rows get their parallelism from K: grid (row groups, K slices); with more than
+// one slice the workgroups write f32 partial sums and gemm_block_finish_kernel adds them in slice order
+// (deterministic) and applies the epilogue.
+#include "gemm_rows.cuh"
+
+#include <stdlib.h>
+
+#include <algorithm>
+#include <mutex>
+
+namespace nv {
+
+namespace {
+
+constexpr int kBW = 4;                       // waves per workgroup: they split the rows
+constexpr int kBThreads = kBW * kWave;
+constexpr int kBK = 128;                     // columns per K-block
+constexpr int kBSteps = kBK / 32;            // matrix-core K-steps per block
+constexpr int kBTiles = 8;                   // token tiles (X in operand order with 8 tiles)
+constexpr int kBStageVec = kBSteps * kBTiles * kWave;   // 16-byte pieces of one X block: 2048 = 32 KiB
+constexpr int kBFill = kBStageVec / kBThreads;          // pieces per thread and block: 8
+constexpr uint32_t kBTokCap = 16u * kBTiles;
+constexpr int kBRowStride = kBK + 8;         // LDS row stride of a W tile in elements: 16 B of padding keeps the
+                                             // 16 rows of an operand read on distinct banks
+constexpr int kBWTile = 16 * kBRowStride;    // one 16-row block of W in LDS
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // a 16-byte piece as a first-class value
+
+template <uint32_t DT>
+__device__ __forceinline__ f32x4_t mfma_k32(u32x4_t a, u32x4_t b, f32x4_t c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                  0, 0);
+}
+
+// Epilogue of four consecutive output rows (row .. row + 3) of token t. For SwiGLU `up` holds the up
+// rows' sums, otherwise it is unused.
+template <uint32_t DT, int EPI>
+__device__ __forceinline__ void block_epilogue(const GemmRowsParams &p, uint32_t t, uint32_t row, f32x4_t y, f32x4_t up) {
+  if (p.bias != nullptr) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      y[r] += dec16<DT>(p.bias[row + r]);
+      if constexpr (EPI == kGemmSwiglu) up[r] += dec16<DT>(p.bias[p.rows + row + r]);
+    }
+  }
+  const uint64_t at = static_cast<uint64_t>(t) * p.rows + row;
+  if constexpr (EPI == kGemmSwiglu) {
+    uint16_t h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] = enc16<DT>(silu(y[r]) * up[r]);
+    const uint64_t at16 = p.out_packed_tiles != 0 ? gemm_x_packed_index(p.out_packed_tiles, t, row) : at;
+    *reinterpret_cast<uint2 *>(p.out16 + at16) =
+        make_uint2(h[0] | (static_cast<uint32_t>(h[1]) << 16), h[2] | (static_cast<uint32_t>(h[3]) << 16));
+  } else {
+    if constexpr (EPI == kGemmResidual) {
+      const float4 res = *reinterpret_cast<const float4 *>(p.residual + at);
+      y[0] += res.x;
+      y[1] += res.y;
+      y[2] += res.z;
+      y[3] += res.w;
+      if (p.round_out) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[r] = round16<DT>(y[r]);
+      }
+    }
+    *reinterpret_cast<float4 *>(p.out_f32 + at) = make_float4(y[0], y[1], y[2], y[3]);
+  }
+}
+
+// Grid (row groups, K slices). NR: row tiles per wave (SwiGLU: 2 = the gate tile and its up tile).
+// cols / gridDim.y must be a multiple of 2 * kBK (the block loop is unrolled by two, loads never sit
+// under a branch).
+// WD: the weight rows go from global memory straight into A-operand registers (16 rows x 64 bytes per
+// request: half cache lines, 16 of them per quarter wave) instead of whole-line requests parked in LDS and
+// read back in operand order - less LDS traffic against more work for the vector-memory path.
+template <uint32_t DT, int EPI, int NR, bool WD>
+__global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams p, float *partials) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);   // [kBStageVec]: the X block, shared by the four waves
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  uint16_t *wtile = reinterpret_cast<uint16_t *>(smem + kBStageVec * sizeof(u32x4_t)) + wave * NR * kBWTile;   // wave-private
+  const uint32_t n = lane & 15, q = lane >> 4;
+  const uint32_t cols = p.cols, T = p.tokens;
+  const uint32_t kslices = gridDim.y, kper = cols / kslices, k0 = blockIdx.y * kper, nblk = kper / kBK;
+
+  // W row of tile j (index into W; for SwiGLU the up tile lies p.rows further down)
+  uint32_t trow[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j)
+    trow[j] = EPI == kGemmSwiglu ? j * p.rows + blockIdx.x * (16u * kBW) + wave * 16u
+                                 : blockIdx.x * (16u * kBW * NR) + (wave * NR + j) * 16u;
+  // W block -> registers: request i of a tile covers its rows 4i .. 4i + 3, 16 lanes x 16 B = 256 contiguous
+  // bytes per row (whole cache lines, like the GEMV's stream)
+  const uint16_t *wp[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j)
+    wp[j] = WD ? p.w + static_cast<uint64_t>(trow[j] + n) * cols + k0 + q * 8
+               : p.w + static_cast<uint64_t>(trow[j] + q) * cols + k0 + n * 8;
+  uint16_t *park_at = wtile + q * kBRowStride + n * 8;
+  const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
+  // X block b of this slice: kBStageVec pieces in a row
+  const u32x4_t *xsrc = reinterpret_cast<const u32x4_t *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kBTiles * kWave) + threadIdx.x;
+
+  u32x4_t areg[2][NR][4];
+  u32x4_t xreg[kBFill];
+  f32x4_t acc[NR][kBTiles];
+#pragma unroll
+  for (int j = 0; j < NR; ++j)
+#pragma unroll
+    for (int c = 0; c < kBTiles; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+#define NV_BLK_W(BUF, BLK)                                                                          \
+  _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
+      areg[BUF][j][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(               \
+          wp[j] + (WD ? static_cast<uint64_t>(i) * 32u : static_cast<uint64_t>(4 * i) * cols) +         \
+          static_cast<uint64_t>(BLK) * kBK))
+#define NV_BLK_WPARK(BUF)                                                                           \
+  if constexpr (!WD) {                                                                              \
+    _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)     \
+        *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]; \
+  }
+#define NV_BLK_X(BLK)                                                                               \
+  _Pragma("unroll") for (int i = 0; i < kBFill; ++i)                                                 \
+      xreg[i] = xsrc[static_cast<uint64_t>(BLK) * kBStageVec + i * kBThreads]
+#define NV_BLK_XPARK()                                                                              \
+  _Pragma("unroll") for (int i = 0; i < kBFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[i]
+  // LDS operand reads run one half K-step ahead of the products that use them: once the products of token
+  // tiles 0..3 have been issued their B registers take the next K-step's pieces, likewise tiles 4..7, so a
+  // read has the other half's products (128 cycles of matrix-core time per row tile) to arrive in. The
+  // scheduling barriers keep the compiler from folding this back into read-wait-multiply pairs.
+#define NV_BLK_READ_A(BUF, S, A)                                                                    \
+  _Pragma("unroll") for (int j = 0; j < NR; ++j) {                                                   \
+    if constexpr (WD) A[j] = areg[BUF][j][S];                                                       \
+    else A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32);                \
+  }
+#define NV_BLK_READ_B(S, C0)                                                                        \
+  _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c) b[c] = stage[((S) * kBTiles + c) * kWave + lane]
+#define NV_BLK_PRODUCTS(A, C0)                                                                      \
+  _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c)                                      \
+      _Pragma("unroll") for (int j = 0; j < NR; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
+#define NV_BLK_STEP(BUF, S, ACUR, ANEXT, LAST)                                                           \
+  if (!(LAST)) { NV_BLK_READ_A(BUF, (S) + 1, ANEXT); }                                                   \
+  NV_BLK_PRODUCTS(ACUR, 0);                                                                         \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  if (!(LAST)) { NV_BLK_READ_B((S) + 1, 0); }                                                       \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  NV_BLK_PRODUCTS(ACUR, kBTiles / 2);                                                               \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  if (!(LAST)) { NV_BLK_READ_B((S) + 1, kBTiles / 2); }                                             \
+  __builtin_amdgcn_sched_barrier(0)
+#define NV_BLK_COMPUTE(BUF)                                                                          \
+  do {                                                                                              \
+    u32x4_t a0[NR], a1[NR], b[kBTiles];                                                             \
+    NV_BLK_READ_A(BUF, 0, a0);                                                                           \
+    NV_BLK_READ_B(0, 0);                                                                            \
+    NV_BLK_READ_B(0, kBTiles / 2);                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    NV_BLK_STEP(BUF, 0, a0, a1, false);                                                                  \
+    NV_BLK_STEP(BUF, 1, a1, a0, false);                                                                  \
+    NV_BLK_STEP(BUF, 2, a0, a1, false);                                                                  \
+    NV_BLK_STEP(BUF, 3, a1, a0, true);                                                                   \
+  } while (0)
+  // One block: the wave parks its W rows (wave-private tile, read back in operand order), the workgroup
+  // swaps the X block in LDS (barrier: everyone has finished the previous block; barrier: the new block is
+  // complete), then the next requests go out and the products run. Requests per iteration: the next X block
+  // first, then the W block after next - loads return in order, and that is the order they are needed in.
+#define NV_BLK_ITER(BUF, XNEXT, WNEXT)                                                              \
+  NV_BLK_WPARK(BUF);                                                                                \
+  __syncthreads();                                                                                  \
+  NV_BLK_XPARK();                                                                                   \
+  __syncthreads();                                                                                  \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  XNEXT;                                                                                            \
+  __builtin_amdgcn_sched_barrier(0);   /* the request order is the order the data is waited for in */ \
+  if constexpr (!WD) { WNEXT; }        /* the registers are free once parked */                      \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  NV_BLK_COMPUTE(BUF);                                                                              \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  if constexpr (WD) { WNEXT; }         /* the registers were this block's operands */                \
+  __builtin_amdgcn_sched_barrier(0)
+
+  NV_BLK_W(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  NV_BLK_X(0);
+  __builtin_amdgcn_sched_barrier(0);
+  NV_BLK_W(1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t blk = 0;
+  for (; blk + 2 < nblk; blk += 2) {
+    NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 2));
+    NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 3));
+  }
+  NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
+  NV_BLK_ITER(1, (void)0, (void)0);
+#undef NV_BLK_W
+#undef NV_BLK_WPARK
+#undef NV_BLK_X
+#undef NV_BLK_XPARK
+#undef NV_BLK_COMPUTE
+#undef NV_BLK_READ_A
+#undef NV_BLK_READ_B
+#undef NV_BLK_PRODUCTS
+#undef NV_BLK_STEP
+#undef NV_BLK_ITER
+
+  // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
+  if (kslices == 1) {
+#pragma unroll
+    for (int c = 0; c < kBTiles; ++c) {
+      const uint32_t t = c * 16u + n;
+      if (t < T) {
+        if constexpr (EPI == kGemmSwiglu) {
+          block_epilogue<DT, EPI>(p, t, trow[0] + q * 4u, acc[0][c], acc[NR - 1][c]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < NR; ++j) block_epilogue<DT, EPI>(p, t, trow[j] + q * 4u, acc[j][c], acc[j][c]);
+        }
+      }
+    }
+  } else {
+    const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
+    float *part = partials + static_cast<uint64_t>(blockIdx.y) * kBTokCap * wrows;
+#pragma unroll
+    for (int c = 0; c < kBTiles; ++c) {
+      const uint32_t t = c * 16u + n;
+      if (t < T) {
+#pragma unroll
+        for (int j = 0; j < NR; ++j)
+          *reinterpret_cast<float4 *>(part + static_cast<uint64_t>(t) * wrows + trow[j] + q * 4u) =
+              make_float4(acc[j][c][0], acc[j][c][1], acc[j][c][2], acc[j][c][3]);
+      }
+    }
+  }
+}
+
+// One thread per token and four consecutive output rows: partial sums in slice order, then the epilogue.
+template <uint32_t DT, int EPI>
+__global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p, const float *partials, uint32_t kslices) {
+  const uint32_t quads = p.rows / 4u;
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= quads * p.tokens) return;
+  const uint32_t t = i / quads, row = (i % quads) * 4u;
+  const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
+  f32x4_t y = {0.0f, 0.0f, 0.0f, 0.0f}, up = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (uint32_t s = 0; s < kslices; ++s) {
+    const float *at = partials + (static_cast<uint64_t>(s) * kBTokCap + t) * wrows + row;
+    const float4 a = *reinterpret_cast<const float4 *>(at);
+    y[0] += a.x;
+    y[1] += a.y;
+    y[2] += a.z;
+    y[3] += a.w;
+    if constexpr (EPI == kGemmSwiglu) {
+      const float4 b = *reinterpret_cast<const float4 *>(at + p.rows);
+      up[0] += b.x;
+      up[1] += b.y;
+      up[2] += b.z;
+      up[3] += b.w;
+    }
+  }
+  block_epilogue<DT, EPI>(p, t, row, y, up);
+}
+
+template <int NR>
+constexpr size_t block_lds_bytes() {
+  return kBStageVec * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
+}
+
+template <uint32_t DT, int EPI, int NR, bool WD>
+hipError_t launch_block_wd(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kBW : 16u * kBW * NR;
+  constexpr size_t lds = block_lds_bytes<NR>();
+  if (lds > 64 * 1024) {
+    // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
+    static std::once_flag once;
+    static hipError_t raised = hipSuccess;
+    std::call_once(once, [] {
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR, WD>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    });
+    if (raised != hipSuccess) return raised;
+  }
+  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, WD>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
+                     p, partials);
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess && kslices > 1) {
+    const uint32_t threads = p.rows / 4u * p.tokens;
+    hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
+                       static_cast<const float *>(partials), kslices);
+    err = hipGetLastError();
+  }
+  return err;
+}
+
+template <uint32_t DT, int EPI, int NR>
+hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  static const bool direct = [] {
+    const char *v = getenv("NERVA_HIP_GEMM_BLOCK_W");   // tuning: "direct" = weights straight into operand registers
+    return v != nullptr && v[0] == 'd';
+  }();
+  return direct ? launch_block_wd<DT, EPI, NR, true>(p, partials, kslices, stream)
+                : launch_block_wd<DT, EPI, NR, false>(p, partials, kslices, stream);
+}
+
+template <uint32_t DT>
+hipError_t launch_block_dt(int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan, hipStream_t stream) {
+  float *partials = static_cast<float *>(p.workspace);
+  switch (epilogue) {
+    case kGemmF32:
+      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmF32, 2>(p, partials, plan.kslices, stream)
+                                 : launch_block_nr<DT, kGemmF32, 1>(p, partials, plan.kslices, stream);
+    case kGemmResidual:
+      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmResidual, 2>(p, partials, plan.kslices, stream)
+                                 : launch_block_nr<DT, kGemmResidual, 1>(p, partials, plan.kslices, stream);
+    case kGemmSwiglu: return launch_block_nr<DT, kGemmSwiglu, 2>(p, partials, plan.kslices, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int env_int(const char *name) {
+  const char *v = getenv(name);
+  return v != nullptr ? atoi(v) : 0;
+}
+
+}  // namespace
+
+GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
+  GemmBlockPlan plan{};
+  static const int mode = [] {
+    const char *v = getenv("NERVA_HIP_GEMM_BLOCK");   // 0: never use the shared-X kernel
+    return v != nullptr && v[0] == '0' ? 0 : 1;
+  }();
+  static const int want_slices = env_int("NERVA_HIP_GEMM_BLOCK_SLICES");   // tuning: K slices for every projection
+  static const int want_tiles = env_int("NERVA_HIP_GEMM_BLOCK_ROW_TILES"); // tuning: 1 or 2 row tiles per wave
+  if (mode == 0 || tokens <= 64 || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (2u * kBK) != 0) return plan;
+  const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
+  // Row tiles per wave: two where that still leaves a workgroup for most CUs.
+  uint32_t tiles = epilogue == kGemmSwiglu ? 2u : (rows / (16u * kBW * 2u) >= 96u && rows % (16u * kBW * 2u) == 0 ? 2u : 1u);
+  if (epilogue != kGemmSwiglu && (want_tiles == 1 || (want_tiles == 2 && rows % (16u * kBW * 2u) == 0))) tiles = want_tiles;
+  const uint32_t groups = rows / (epilogue == kGemmSwiglu ? 16u * kBW : 16u * kBW * tiles);
+  // K slices: enough workgroups for two per CU, each slice at least four K-blocks, an even number of them.
+  // (A sliced gate/up pair would write and re-read 12.6 MB of partial sums per slice: measured no faster.)
+  uint32_t slices = 1;
+  while (epilogue != kGemmSwiglu && groups * slices < 384u && cols % (slices * 2u * 2u * kBK) == 0 && cols / (slices * 2u) >= 4u * kBK) slices *= 2u;
+  if (want_slices > 0 && cols % (static_cast<uint32_t>(want_slices) * 2u * kBK) == 0) slices = want_slices;
+  if (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) {
+    // not enough room for the partial sums: as many slices as fit (a power of two), or none
+    while (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
+  }
+  plan.row_tiles = tiles;
+  plan.kslices = slices;
+  return plan;
+}
+
+uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {
+  // room for 8 slices of the widest plain projection or 2 of a gate/up pair of that width
+  return static_cast<uint64_t>(8) * kBTokCap * rows_max * sizeof(float);
+}
+
+hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,
+                             hipStream_t stream) {
+  if (plan.kslices == 0 || p.x_packed != kBTiles) return hipErrorInvalidValue;
+  if (plan.kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
+  if (dtype == kBF16) return launch_block_dt<kBF16>(epilogue, p, plan, stream);
+  if (dtype == kF16) return launch_block_dt<kF16>(epilogue, p, plan, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace nv

@@ -47,6 +47,8 @@ struct GemmRowsParams {
   uint32_t x_packed;         // != 0: x16 is in matrix-operand order (gemm_x_packed_index) instead of [tokens][cols];
                              // the value is its token-tile count and must be gemm_packed_tiles(tokens)
   uint32_t out_packed_tiles; // kGemmSwiglu: != 0 writes out16 in operand order with this many token tiles
+  void *workspace;           // optional: room for the f32 partial sums of the shared-X kernel's K slices
+  uint64_t workspace_bytes;  // (gemm_block_workspace_bytes; without it that kernel runs unsliced or not at all)
 };
 
 // rows >= 16 (any count: the last workgroup overlaps its neighbour, so with a row count that is no
@@ -54,6 +56,19 @@ struct GemmRowsParams {
 // whole 256-column blocks), 1 <= tokens <= kGemmMaxTokens, 16-byte aligned w and x16.
 bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens);
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream);
+
+// Blocks of more than 64 token rows with X in operand order: the kernel that shares the X operand through
+// LDS (gemm_block.hip). The plan says whether it takes a shape (kslices != 0) and how: row tiles per wave
+// and K slices (more than one needs slices x 128 x W rows f32 of workspace). launch_gemm_rows uses it by
+// itself where the plan allows.
+struct GemmBlockPlan {
+  uint32_t row_tiles, kslices;
+};
+GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
+// Workspace that lets every projection of up to `rows_max` output rows (a gate/up pair counts twice) use its plan.
+uint64_t gemm_block_workspace_bytes(uint32_t rows_max);
+hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,
+                             hipStream_t stream);
 
 // x16[t] = round16(x[t] * rsqrt(mean(x[t]^2) + eps) * gamma) for `tokens` rows of `cols` f32 values.
 // packed_tiles != 0: out16 in operand order (gemm_x_packed_index) with that many token tiles.

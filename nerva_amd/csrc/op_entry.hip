@@ -460,8 +460,12 @@ int nerva_hip_gemm_rows(const NervaHipGemmRowsRequest *r, void *stream, int32_t 
   p.round_out = r->round_output;
   p.x_packed = r->input_operand_order != 0 ? gemm_packed_tiles(r->tokens) : 0u;
   p.out_packed_tiles = r->output16_operand_order != 0 ? gemm_packed_tiles(r->tokens) : 0u;
+  p.workspace = r->workspace;
+  p.workspace_bytes = r->workspace != nullptr ? r->workspace_bytes : 0;
   return finish(launch_gemm_rows(r->dtype, static_cast<int>(r->epilogue), p, resolve_stream(stream)), hip_error);
 }
+
+uint64_t nerva_hip_gemm_rows_workspace_bytes(uint32_t rows) { return gemm_block_workspace_bytes(rows); }
 
 uint64_t nerva_hip_gemm_operand_index(uint32_t tokens, uint32_t token, uint32_t column) {
   return gemm_x_packed_index(gemm_packed_tiles(tokens), token, column);

@@ -259,10 +259,14 @@ def gemm_operand_order(x, tokens=None):
 
 
 def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None, residual=None, out_f32=None,
-              out16=None, round_output=False, sync=True, input_operand_order=False, output16_operand_order=False):
-    """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once)."""
+              out16=None, round_output=False, sync=True, input_operand_order=False, output16_operand_order=False,
+              workspace=None):
+    """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once).
+    `workspace`: optional DeviceBuffer of gemm_rows_workspace_bytes(rows) for the K-sliced large-block kernel."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()
+    if workspace is not None:
+        req.workspace, req.workspace_bytes = workspace.ptr, workspace.nbytes
     req.input_operand_order, req.output16_operand_order = int(input_operand_order), int(output16_operand_order)
     req.dtype, req.rows, req.cols, req.tokens, req.epilogue, req.round_output = dtype, rows, cols, tokens, epilogue, int(round_output)
     req.weights, req.input16, req.bias, req.residual = _ptr(weights), _ptr(input16), _ptr(bias), _ptr(residual)
@@ -271,6 +275,12 @@ def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None
     _check(lib.nerva_hip_gemm_rows(C.byref(req), None, C.byref(err)), err, "nerva_hip_gemm_rows")
     if sync:
         Device.synchronize()
+
+
+def gemm_rows_workspace_bytes(rows):
+    lib = abi.load()
+    lib.nerva_hip_gemm_rows_workspace_bytes.restype = C.c_uint64
+    return int(lib.nerva_hip_gemm_rows_workspace_bytes(C.c_uint32(rows)))
 
 
 def sample(logits_buf, vocab, temperature, top_p, top_k, seed, position, workspace=None):

@@ -624,7 +624,13 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
     y0, y1 = N.DeviceBuffer(tokens * rows * 4), N.DeviceBuffer(tokens * rows * 4)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(x), out_f32=y0)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(packed), out_f32=y1, input_operand_order=True)
-    assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
+    # blocks of more than 64 rows in operand order may take the kernel that shares X through LDS: the same
+    # products summed in another order
+    same_kernel = tokens <= 64 or rows % 64 != 0
+    if same_kernel:
+        assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
+    else:
+        assert rel_l2(y1.numpy(np.float32), y0.numpy(np.float32)) <= 1e-5
     if rows % 2 == 0 and (rows // 2) % 32 == 0:
         inter = rows // 2                                                          # the same matrix as [gate; up]
         o0 = N.DeviceBuffer(tokens * inter * 2)
@@ -634,4 +640,66 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
                     output16_operand_order=True)
         rowmajor = o0.numpy(np.uint16, tokens * inter).reshape(tokens, inter)
         _, oidx = N.gemm_operand_order(np.zeros((tokens, inter), np.uint16))
-        assert np.array_equal(o1.numpy(np.uint16)[oidx], rowmajor)
+        if same_kernel:
+            assert np.array_equal(o1.numpy(np.uint16)[oidx], rowmajor)
+        else:
+            assert rel_l2(O.decode16(dtype, o1.numpy(np.uint16)[oidx]), O.decode16(dtype, rowmajor)) <= 4e-3
+
+
+@pytest.mark.parametrize("sliced", [False, True])
+@pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 65), (192, 2048, 100), (4096, 4096, 128), (6144, 4096, 127),
+                                               (4096, 12288, 128)])
+def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
+    """More than 64 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
+    X from LDS. Every token row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
+    dtype = BF16
+    rng = np.random.default_rng(rows + cols + tokens)
+    if rows * cols > 1 << 22:
+        w = O.synth_16(dtype, SEED, 320 + tokens, rows * cols, 0.0, 0.02).reshape(rows, cols)
+    else:
+        w = O.encode16(dtype, rng.normal(0, 0.02, (rows, cols)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, cols)))
+    bias = O.encode16(dtype, rng.normal(0, 0.1, rows))
+    res = rng.normal(0, 1, (tokens, rows)).astype(np.float32)
+    step = 1 if rows * cols <= 1 << 22 else 9
+    picks = list(range(0, tokens, step)) + [tokens - 1]
+    ref = {t: O.gemv_x16(dtype, w, x[t]) for t in picks}
+    packed, _ = N.gemm_operand_order(x)
+    ws = N.DeviceBuffer(N.gemm_rows_workspace_bytes(rows)) if sliced else None
+    dw, dx = dev(w), dev(packed)
+    y = N.DeviceBuffer.zeros(tokens * rows * 4)
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dx, epilogue=0, out_f32=y, input_operand_order=True, workspace=ws)
+    got = y.numpy(np.float32).reshape(tokens, rows)
+    assert max(rel_l2(got[t], ref[t]) for t in picks) <= REL_L2
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dx, epilogue=1, bias=dev(bias), residual=dev(res), out_f32=y,
+                round_output=True, input_operand_order=True, workspace=ws)
+    got = y.numpy(np.float32).reshape(tokens, rows)
+    for t in picks:
+        want = O.decode16(dtype, O.encode16(dtype, (ref[t] + O.decode16(dtype, bias)) + res[t]))
+        assert rel_l2(got[t], want) <= 4e-3
+    assert np.array_equal(O.encode16(dtype, got), O.encode16(dtype, got.astype(np.float32)))
+
+
+@pytest.mark.parametrize("sliced", [False, True])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128)])
+def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
+    """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
+    dtype = BF16
+    rng = np.random.default_rng(inter + tokens)
+    if inter > 1000:
+        w = O.synth_16(dtype, SEED, 330, 2 * inter * hidden, 0.0, 0.02).reshape(2 * inter, hidden)
+    else:
+        w = O.encode16(dtype, rng.normal(0, 0.05, (2 * inter, hidden)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, hidden)))
+    packed, _ = N.gemm_operand_order(x)
+    ws = N.DeviceBuffer(N.gemm_rows_workspace_bytes(2 * inter)) if sliced else None
+    out = N.DeviceBuffer.zeros(N.gemm_operand_slots(tokens) * inter * 2)
+    N.gemm_rows(dtype, dev(w), inter, hidden, tokens, dev(packed), epilogue=2, out16=out, input_operand_order=True,
+                output16_operand_order=True, workspace=ws)
+    _, oidx = N.gemm_operand_order(np.zeros((tokens, inter), np.uint16))
+    got = O.decode16(dtype, out.numpy(np.uint16)[oidx]).reshape(tokens, inter)
+    for t in sorted({0, tokens // 3, tokens - 1}):
+        gu = O.gemv_x16(dtype, w, x[t])
+        g, u = gu[:inter].astype(np.float64), gu[inter:].astype(np.float64)
+        want = O.decode16(dtype, O.encode16(dtype, (g / (1.0 + np.exp(-g)) * u).astype(np.float32)))
+        assert rel_l2(got[t], want) <= 4e-3
