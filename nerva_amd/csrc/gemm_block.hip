@@ -26,6 +26,7 @@ constexpr int kBW = 4;                       // waves per workgroup: they split 
 constexpr int kBThreads = kBW * kWave;
 constexpr int kBK = 128;                     // columns per K-block
 constexpr int kBSteps = kBK / 32;            // matrix-core K-steps per block
+constexpr int kBRing = 4;                    // W blocks a wave requests ahead at most (two with one row tile per wave)
 constexpr int kBTiles = 8;                   // token tiles (X in operand order with 8 tiles)
 constexpr int kBStageVec = kBSteps * kBTiles * kWave;   // 16-byte pieces of one X block: 2048 = 32 KiB
 constexpr int kBFill = kBStageVec / kBThreads;          // pieces per thread and block: 8
@@ -85,13 +86,13 @@ __device__ __forceinline__ void block_epilogue(const GemmRowsParams &p, uint32_t
 }
 
 // Grid (row groups, K slices). NR: row tiles per wave (SwiGLU: 2 = the gate tile and its up tile).
-// cols / gridDim.y must be a multiple of 2 * kBK (the block loop is unrolled by two, loads never sit
-// under a branch).
-// WD: the weight rows go from global memory straight into A-operand registers (16 rows x 64 bytes per
-// request: half cache lines, 16 of them per quarter wave) instead of whole-line requests parked in LDS and
-// read back in operand order - less LDS traffic against more work for the vector-memory path.
-template <uint32_t DT, int EPI, int NR, bool WD>
-__global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams p, float *partials) {
+// cols / gridDim.y must be a multiple of kBRing * kBK (the block loop is unrolled by the ring depth, so
+// that no load sits under a branch and every register index is static).
+// One row tile per wave: two W blocks requested ahead, two workgroups share a CU. Two row tiles: a wave
+// takes more than 256 registers, a CU holds one workgroup, and four W blocks are requested ahead to make
+// up for it (measured: gate_up 62.5 -> 54.4 us with four; the one-tile projections lose 5-8 % with four).
+template <uint32_t DT, int EPI, int NR>
+__global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(GemmRowsParams p, float *partials) {
   extern __shared__ __align__(16) unsigned char smem[];
   u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);   // [kBStageVec]: the X block, shared by the four waves
   const int lane = threadIdx.x & (kWave - 1);
@@ -111,15 +112,14 @@ __global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams
   // bytes per row (whole cache lines, like the GEMV's stream)
   const uint16_t *wp[NR];
 #pragma unroll
-  for (int j = 0; j < NR; ++j)
-    wp[j] = WD ? p.w + static_cast<uint64_t>(trow[j] + n) * cols + k0 + q * 8
-               : p.w + static_cast<uint64_t>(trow[j] + q) * cols + k0 + n * 8;
+  for (int j = 0; j < NR; ++j) wp[j] = p.w + static_cast<uint64_t>(trow[j] + q) * cols + k0 + n * 8;
   uint16_t *park_at = wtile + q * kBRowStride + n * 8;
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
   // X block b of this slice: kBStageVec pieces in a row
   const u32x4_t *xsrc = reinterpret_cast<const u32x4_t *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kBTiles * kWave) + threadIdx.x;
 
-  u32x4_t areg[2][NR][4];
+  constexpr int kRing = NR == 1 ? 2 : kBRing;   // W blocks requested ahead: what the register budget holds
+  u32x4_t areg[kRing][NR][4];
   u32x4_t xreg[kBFill];
   f32x4_t acc[NR][kBTiles];
 #pragma unroll
@@ -130,13 +130,10 @@ __global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams
 #define NV_BLK_W(BUF, BLK)                                                                          \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       areg[BUF][j][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(               \
-          wp[j] + (WD ? static_cast<uint64_t>(i) * 32u : static_cast<uint64_t>(4 * i) * cols) +         \
-          static_cast<uint64_t>(BLK) * kBK))
+          wp[j] + static_cast<uint64_t>(4 * i) * cols + static_cast<uint64_t>(BLK) * kBK))
 #define NV_BLK_WPARK(BUF)                                                                           \
-  if constexpr (!WD) {                                                                              \
-    _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)     \
-        *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]; \
-  }
+  _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
+      *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]
 #define NV_BLK_X(BLK)                                                                               \
   _Pragma("unroll") for (int i = 0; i < kBFill; ++i)                                                 \
       xreg[i] = xsrc[static_cast<uint64_t>(BLK) * kBStageVec + i * kBThreads]
@@ -146,18 +143,16 @@ __global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams
   // tiles 0..3 have been issued their B registers take the next K-step's pieces, likewise tiles 4..7, so a
   // read has the other half's products (128 cycles of matrix-core time per row tile) to arrive in. The
   // scheduling barriers keep the compiler from folding this back into read-wait-multiply pairs.
-#define NV_BLK_READ_A(BUF, S, A)                                                                    \
-  _Pragma("unroll") for (int j = 0; j < NR; ++j) {                                                   \
-    if constexpr (WD) A[j] = areg[BUF][j][S];                                                       \
-    else A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32);                \
-  }
+#define NV_BLK_READ_A(S, A)                                                                         \
+  _Pragma("unroll") for (int j = 0; j < NR; ++j)                                                     \
+      A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32)
 #define NV_BLK_READ_B(S, C0)                                                                        \
   _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c) b[c] = stage[((S) * kBTiles + c) * kWave + lane]
 #define NV_BLK_PRODUCTS(A, C0)                                                                      \
   _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c)                                      \
       _Pragma("unroll") for (int j = 0; j < NR; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
-#define NV_BLK_STEP(BUF, S, ACUR, ANEXT, LAST)                                                           \
-  if (!(LAST)) { NV_BLK_READ_A(BUF, (S) + 1, ANEXT); }                                                   \
+#define NV_BLK_STEP(S, ACUR, ANEXT, LAST)                                                           \
+  if (!(LAST)) { NV_BLK_READ_A((S) + 1, ANEXT); }                                                   \
   NV_BLK_PRODUCTS(ACUR, 0);                                                                         \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   if (!(LAST)) { NV_BLK_READ_B((S) + 1, 0); }                                                       \
@@ -166,22 +161,23 @@ __global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams
   __builtin_amdgcn_sched_barrier(0);                                                                \
   if (!(LAST)) { NV_BLK_READ_B((S) + 1, kBTiles / 2); }                                             \
   __builtin_amdgcn_sched_barrier(0)
-#define NV_BLK_COMPUTE(BUF)                                                                          \
+#define NV_BLK_COMPUTE()                                                                            \
   do {                                                                                              \
     u32x4_t a0[NR], a1[NR], b[kBTiles];                                                             \
-    NV_BLK_READ_A(BUF, 0, a0);                                                                           \
+    NV_BLK_READ_A(0, a0);                                                                           \
     NV_BLK_READ_B(0, 0);                                                                            \
     NV_BLK_READ_B(0, kBTiles / 2);                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    NV_BLK_STEP(BUF, 0, a0, a1, false);                                                                  \
-    NV_BLK_STEP(BUF, 1, a1, a0, false);                                                                  \
-    NV_BLK_STEP(BUF, 2, a0, a1, false);                                                                  \
-    NV_BLK_STEP(BUF, 3, a1, a0, true);                                                                   \
+    NV_BLK_STEP(0, a0, a1, false);                                                                  \
+    NV_BLK_STEP(1, a1, a0, false);                                                                  \
+    NV_BLK_STEP(2, a0, a1, false);                                                                  \
+    NV_BLK_STEP(3, a1, a0, true);                                                                   \
   } while (0)
-  // One block: the wave parks its W rows (wave-private tile, read back in operand order), the workgroup
-  // swaps the X block in LDS (barrier: everyone has finished the previous block; barrier: the new block is
-  // complete), then the next requests go out and the products run. Requests per iteration: the next X block
-  // first, then the W block after next - loads return in order, and that is the order they are needed in.
+  // One block: the wave parks its W rows (wave-private tile, read back in operand order) and re-uses those
+  // registers for the block kBRing further on; the workgroup swaps the X block in LDS (barrier: everyone has
+  // finished the previous block; barrier: the new block is complete); the next X block is requested and the
+  // products run. Loads return in order, and the order of the requests is the order the data is waited for
+  // in (the scheduling barriers pin it): a wait for X never includes a W block requested after it.
 #define NV_BLK_ITER(BUF, XNEXT, WNEXT)                                                              \
   NV_BLK_WPARK(BUF);                                                                                \
   __syncthreads();                                                                                  \
@@ -189,27 +185,41 @@ __global__ __launch_bounds__(kBThreads, 2) void gemm_block_kernel(GemmRowsParams
   __syncthreads();                                                                                  \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   XNEXT;                                                                                            \
-  __builtin_amdgcn_sched_barrier(0);   /* the request order is the order the data is waited for in */ \
-  if constexpr (!WD) { WNEXT; }        /* the registers are free once parked */                      \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  NV_BLK_COMPUTE(BUF);                                                                              \
+  WNEXT;                                                                                            \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  if constexpr (WD) { WNEXT; }         /* the registers were this block's operands */                \
-  __builtin_amdgcn_sched_barrier(0)
+  NV_BLK_COMPUTE()
 
   NV_BLK_W(0, 0);
   __builtin_amdgcn_sched_barrier(0);
   NV_BLK_X(0);
   __builtin_amdgcn_sched_barrier(0);
-  NV_BLK_W(1, 1);
-  __builtin_amdgcn_sched_barrier(0);
   uint32_t blk = 0;
-  for (; blk + 2 < nblk; blk += 2) {
-    NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 2));
-    NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 3));
+  if constexpr (kRing == 4) {
+    NV_BLK_W(1, 1);
+    NV_BLK_W(2, 2);
+    NV_BLK_W(3, 3);
+    __builtin_amdgcn_sched_barrier(0);
+    for (; blk + 4 < nblk; blk += 4) {
+      NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 4));
+      NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 5));
+      NV_BLK_ITER(2, NV_BLK_X(blk + 3), NV_BLK_W(2, blk + 6));
+      NV_BLK_ITER(3, NV_BLK_X(blk + 4), NV_BLK_W(3, blk + 7));
+    }
+    NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
+    NV_BLK_ITER(1, NV_BLK_X(blk + 2), (void)0);
+    NV_BLK_ITER(2, NV_BLK_X(blk + 3), (void)0);
+    NV_BLK_ITER(3, (void)0, (void)0);
+  } else {
+    NV_BLK_W(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    for (; blk + 2 < nblk; blk += 2) {
+      NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 2));
+      NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 3));
+    }
+    NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
+    NV_BLK_ITER(1, (void)0, (void)0);
   }
-  NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
-  NV_BLK_ITER(1, (void)0, (void)0);
 #undef NV_BLK_W
 #undef NV_BLK_WPARK
 #undef NV_BLK_X
@@ -283,8 +293,8 @@ constexpr size_t block_lds_bytes() {
   return kBStageVec * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
 }
 
-template <uint32_t DT, int EPI, int NR, bool WD>
-hipError_t launch_block_wd(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+template <uint32_t DT, int EPI, int NR>
+hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
   const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kBW : 16u * kBW * NR;
   constexpr size_t lds = block_lds_bytes<NR>();
   if (lds > 64 * 1024) {
@@ -292,12 +302,12 @@ hipError_t launch_block_wd(const GemmRowsParams &p, float *partials, uint32_t ks
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR, WD>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, WD>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
+  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
                      p, partials);
   hipError_t err = hipGetLastError();
   if (err == hipSuccess && kslices > 1) {
@@ -307,16 +317,6 @@ hipError_t launch_block_wd(const GemmRowsParams &p, float *partials, uint32_t ks
     err = hipGetLastError();
   }
   return err;
-}
-
-template <uint32_t DT, int EPI, int NR>
-hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
-  static const bool direct = [] {
-    const char *v = getenv("NERVA_HIP_GEMM_BLOCK_W");   // tuning: "direct" = weights straight into operand registers
-    return v != nullptr && v[0] == 'd';
-  }();
-  return direct ? launch_block_wd<DT, EPI, NR, true>(p, partials, kslices, stream)
-                : launch_block_wd<DT, EPI, NR, false>(p, partials, kslices, stream);
 }
 
 template <uint32_t DT>
@@ -349,17 +349,17 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   }();
   static const int want_slices = env_int("NERVA_HIP_GEMM_BLOCK_SLICES");   // tuning: K slices for every projection
   static const int want_tiles = env_int("NERVA_HIP_GEMM_BLOCK_ROW_TILES"); // tuning: 1 or 2 row tiles per wave
-  if (mode == 0 || tokens <= 64 || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (2u * kBK) != 0) return plan;
+  if (mode == 0 || tokens <= 64 || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (kBRing * kBK) != 0) return plan;
   const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
   // Row tiles per wave: two where that still leaves a workgroup for most CUs.
   uint32_t tiles = epilogue == kGemmSwiglu ? 2u : (rows / (16u * kBW * 2u) >= 96u && rows % (16u * kBW * 2u) == 0 ? 2u : 1u);
   if (epilogue != kGemmSwiglu && (want_tiles == 1 || (want_tiles == 2 && rows % (16u * kBW * 2u) == 0))) tiles = want_tiles;
   const uint32_t groups = rows / (epilogue == kGemmSwiglu ? 16u * kBW : 16u * kBW * tiles);
-  // K slices: enough workgroups for two per CU, each slice at least four K-blocks, an even number of them.
+  // K slices: enough workgroups for two per CU, each slice a whole number of rings of K-blocks.
   // (A sliced gate/up pair would write and re-read 12.6 MB of partial sums per slice: measured no faster.)
   uint32_t slices = 1;
-  while (epilogue != kGemmSwiglu && groups * slices < 384u && cols % (slices * 2u * 2u * kBK) == 0 && cols / (slices * 2u) >= 4u * kBK) slices *= 2u;
-  if (want_slices > 0 && cols % (static_cast<uint32_t>(want_slices) * 2u * kBK) == 0) slices = want_slices;
+  while (epilogue != kGemmSwiglu && groups * slices < 384u && cols % (slices * 2u * kBRing * kBK) == 0) slices *= 2u;
+  if (want_slices > 0 && cols % (static_cast<uint32_t>(want_slices) * kBRing * kBK) == 0) slices = want_slices;
   if (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) {
     // not enough room for the partial sums: as many slices as fit (a power of two), or none
     while (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
