@@ -14,6 +14,8 @@
 // and K-step. v_mfma_f32_16x16x32 accumulates D[weight row][token] in f32, two token tiles per
 // wave; the waves' partial sums meet in LDS and are added in wave order (deterministic), then
 // the epilogue runs once per output element.
+// Blocks of more than 64 rows with X in operand order take another kernel (gemm_block.hip) in which the
+// waves of a workgroup split the rows instead and share each K-block of X through LDS.
 #pragma once
 
 #include "nv_common.cuh"
