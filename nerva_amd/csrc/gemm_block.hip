@@ -110,17 +110,22 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
                                  : blockIdx.x * (16u * kBW * NR) + (wave * NR + j) * 16u;
   // W block -> registers: request i of a tile covers its rows 4i .. 4i + 3, 16 lanes x 16 B = 256 contiguous
   // bytes per row (whole cache lines, like the GEMV's stream)
-  const uint16_t *wp[NR];
+  // Addresses are a wave-uniform 64-bit base (scalar registers, scalar arithmetic) plus a 32-bit per-lane
+  // offset that never changes, so a request costs no vector ALU work.
+  const char *wbase[NR];
 #pragma unroll
-  for (int j = 0; j < NR; ++j) wp[j] = p.w + static_cast<uint64_t>(trow[j] + q) * cols + k0 + n * 8;
+  for (int j = 0; j < NR; ++j)
+    wbase[j] = reinterpret_cast<const char *>(p.w) + (static_cast<uint64_t>(trow[j]) * cols + k0) * sizeof(uint16_t);
+  const uint32_t wlane = (q * cols + n * 8u) * static_cast<uint32_t>(sizeof(uint16_t));
   uint16_t *park_at = wtile + q * kBRowStride + n * 8;
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
   // X block b of this slice: kBStageVec pieces in a row
-  const u32x4_t *xsrc = reinterpret_cast<const u32x4_t *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kBTiles * kWave) + threadIdx.x;
+  const char *xbase = reinterpret_cast<const char *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kBTiles * kWave) * sizeof(u32x4_t);
+  const uint32_t xlane = threadIdx.x * static_cast<uint32_t>(sizeof(u32x4_t));
 
   constexpr int kRing = NR == 1 ? 2 : kBRing;   // W blocks requested ahead: what the register budget holds
   u32x4_t areg[kRing][NR][4];
-  u32x4_t xreg[kBFill];
+  u32x4_t xreg[2][kBFill];   // the X blocks one and two ahead
   f32x4_t acc[NR][kBTiles];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
@@ -130,15 +135,16 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 #define NV_BLK_W(BUF, BLK)                                                                          \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       areg[BUF][j][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(               \
-          wp[j] + static_cast<uint64_t>(4 * i) * cols + static_cast<uint64_t>(BLK) * kBK))
+          wbase[j] + (static_cast<uint64_t>(4 * i) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
 #define NV_BLK_WPARK(BUF)                                                                           \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]
-#define NV_BLK_X(BLK)                                                                               \
+#define NV_BLK_X(XB, BLK)                                                                           \
   _Pragma("unroll") for (int i = 0; i < kBFill; ++i)                                                 \
-      xreg[i] = xsrc[static_cast<uint64_t>(BLK) * kBStageVec + i * kBThreads]
-#define NV_BLK_XPARK()                                                                              \
-  _Pragma("unroll") for (int i = 0; i < kBFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[i]
+      xreg[XB][i] = *reinterpret_cast<const u32x4_t *>(                                              \
+          xbase + (static_cast<uint64_t>(BLK) * kBStageVec + i * kBThreads) * sizeof(u32x4_t) + xlane)
+#define NV_BLK_XPARK(XB)                                                                            \
+  _Pragma("unroll") for (int i = 0; i < kBFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[XB][i]
   // LDS operand reads run one half K-step ahead of the products that use them: once the products of token
   // tiles 0..3 have been issued their B registers take the next K-step's pieces, likewise tiles 4..7, so a
   // read has the other half's products (128 cycles of matrix-core time per row tile) to arrive in. The
@@ -174,14 +180,16 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
     NV_BLK_STEP(3, a1, a0, true);                                                                   \
   } while (0)
   // One block: the wave parks its W rows (wave-private tile, read back in operand order) and re-uses those
-  // registers for the block kBRing further on; the workgroup swaps the X block in LDS (barrier: everyone has
-  // finished the previous block; barrier: the new block is complete); the next X block is requested and the
-  // products run. Loads return in order, and the order of the requests is the order the data is waited for
-  // in (the scheduling barriers pin it): a wait for X never includes a W block requested after it.
-#define NV_BLK_ITER(BUF, XNEXT, WNEXT)                                                              \
+  // registers for the block kRing further on; the workgroup swaps the X block in LDS (barrier: everyone has
+  // finished the previous block; barrier: the new block is complete) and requests the X block after next;
+  // then the products run. Loads return in order, so the order of the requests is pinned (scheduling
+  // barriers) to the order their data is awaited in, and X is requested TWO blocks ahead: an X block comes
+  // from L2 but queues behind the W block requested an iteration earlier, which comes from HBM - requested
+  // one block ahead, every X wait was a wait for that W block's HBM latency.
+#define NV_BLK_ITER(BUF, XB, XNEXT, WNEXT)                                                          \
   NV_BLK_WPARK(BUF);                                                                                \
   __syncthreads();                                                                                  \
-  NV_BLK_XPARK();                                                                                   \
+  NV_BLK_XPARK(XB);                                                                                 \
   __syncthreads();                                                                                  \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   XNEXT;                                                                                            \
@@ -192,7 +200,9 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 
   NV_BLK_W(0, 0);
   __builtin_amdgcn_sched_barrier(0);
-  NV_BLK_X(0);
+  NV_BLK_X(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  NV_BLK_X(1, 1);
   __builtin_amdgcn_sched_barrier(0);
   uint32_t blk = 0;
   if constexpr (kRing == 4) {
@@ -201,24 +211,24 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
     NV_BLK_W(3, 3);
     __builtin_amdgcn_sched_barrier(0);
     for (; blk + 4 < nblk; blk += 4) {
-      NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 4));
-      NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 5));
-      NV_BLK_ITER(2, NV_BLK_X(blk + 3), NV_BLK_W(2, blk + 6));
-      NV_BLK_ITER(3, NV_BLK_X(blk + 4), NV_BLK_W(3, blk + 7));
+      NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), NV_BLK_W(0, blk + 4));
+      NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), NV_BLK_W(1, blk + 5));
+      NV_BLK_ITER(2, 0, NV_BLK_X(0, blk + 4), NV_BLK_W(2, blk + 6));
+      NV_BLK_ITER(3, 1, NV_BLK_X(1, blk + 5), NV_BLK_W(3, blk + 7));
     }
-    NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
-    NV_BLK_ITER(1, NV_BLK_X(blk + 2), (void)0);
-    NV_BLK_ITER(2, NV_BLK_X(blk + 3), (void)0);
-    NV_BLK_ITER(3, (void)0, (void)0);
+    NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), (void)0);
+    NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), (void)0);
+    NV_BLK_ITER(2, 0, (void)0, (void)0);
+    NV_BLK_ITER(3, 1, (void)0, (void)0);
   } else {
     NV_BLK_W(1, 1);
     __builtin_amdgcn_sched_barrier(0);
     for (; blk + 2 < nblk; blk += 2) {
-      NV_BLK_ITER(0, NV_BLK_X(blk + 1), NV_BLK_W(0, blk + 2));
-      NV_BLK_ITER(1, NV_BLK_X(blk + 2), NV_BLK_W(1, blk + 3));
+      NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), NV_BLK_W(0, blk + 2));
+      NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), NV_BLK_W(1, blk + 3));
     }
-    NV_BLK_ITER(0, NV_BLK_X(blk + 1), (void)0);
-    NV_BLK_ITER(1, (void)0, (void)0);
+    NV_BLK_ITER(0, 0, (void)0, (void)0);
+    NV_BLK_ITER(1, 1, (void)0, (void)0);
   }
 #undef NV_BLK_W
 #undef NV_BLK_WPARK
