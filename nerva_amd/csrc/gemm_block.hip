@@ -157,46 +157,62 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 #define NV_BLK_PRODUCTS(A, C0)                                                                      \
   _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c)                                      \
       _Pragma("unroll") for (int j = 0; j < NR; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
-#define NV_BLK_STEP(S, ACUR, ANEXT, LAST)                                                           \
+  // The requests for the blocks ahead go out between the products, two per half K-step (first the X pieces,
+  // then the W rows: the order they are awaited in): the CU's vector-memory path takes 64 bytes a cycle, and
+  // four waves handing it their 16 requests at once spent 550-1000 cycles issuing them before any product ran.
+#define NV_BLK_W1(BUF, BLK, J, I)                                                                   \
+  areg[BUF][J][I] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(                   \
+      wbase[J] + (static_cast<uint64_t>(4 * (I)) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
+#define NV_BLK_X1(XB, BLK, I)                                                                       \
+  xreg[XB][I] = *reinterpret_cast<const u32x4_t *>(                                                  \
+      xbase + (static_cast<uint64_t>(BLK) * kBStageVec + (I) * kBThreads) * sizeof(u32x4_t) + xlane)
+#define NV_BLK_SLOT(K, BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
+  if constexpr ((K) < 4) {                                                                          \
+    if constexpr (XEN) {                                                                            \
+      NV_BLK_X1(XB, XBLK, 2 * (K));                                                                 \
+      NV_BLK_X1(XB, XBLK, 2 * (K) + 1);                                                             \
+    }                                                                                               \
+  } else if constexpr (WEN && 2 * ((K) - 4) < NR * 4) {                                             \
+    NV_BLK_W1(BUF, WBLK, (2 * ((K) - 4)) / 4, (2 * ((K) - 4)) % 4);                                 \
+    NV_BLK_W1(BUF, WBLK, (2 * ((K) - 4) + 1) / 4, (2 * ((K) - 4) + 1) % 4);                         \
+  }
+#define NV_BLK_STEP(S, ACUR, ANEXT, LAST, BUF, XB, XEN, XBLK, WEN, WBLK)                            \
   if (!(LAST)) { NV_BLK_READ_A((S) + 1, ANEXT); }                                                   \
   NV_BLK_PRODUCTS(ACUR, 0);                                                                         \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   if (!(LAST)) { NV_BLK_READ_B((S) + 1, 0); }                                                       \
+  NV_BLK_SLOT(2 * (S), BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   NV_BLK_PRODUCTS(ACUR, kBTiles / 2);                                                               \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   if (!(LAST)) { NV_BLK_READ_B((S) + 1, kBTiles / 2); }                                             \
+  NV_BLK_SLOT(2 * (S) + 1, BUF, XB, XEN, XBLK, WEN, WBLK)                                           \
   __builtin_amdgcn_sched_barrier(0)
-#define NV_BLK_COMPUTE()                                                                            \
+#define NV_BLK_COMPUTE(BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   do {                                                                                              \
     u32x4_t a0[NR], a1[NR], b[kBTiles];                                                             \
     NV_BLK_READ_A(0, a0);                                                                           \
     NV_BLK_READ_B(0, 0);                                                                            \
     NV_BLK_READ_B(0, kBTiles / 2);                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    NV_BLK_STEP(0, a0, a1, false);                                                                  \
-    NV_BLK_STEP(1, a1, a0, false);                                                                  \
-    NV_BLK_STEP(2, a0, a1, false);                                                                  \
-    NV_BLK_STEP(3, a1, a0, true);                                                                   \
+    NV_BLK_STEP(0, a0, a1, false, BUF, XB, XEN, XBLK, WEN, WBLK);                                   \
+    NV_BLK_STEP(1, a1, a0, false, BUF, XB, XEN, XBLK, WEN, WBLK);                                   \
+    NV_BLK_STEP(2, a0, a1, false, BUF, XB, XEN, XBLK, WEN, WBLK);                                   \
+    NV_BLK_STEP(3, a1, a0, true, BUF, XB, XEN, XBLK, WEN, WBLK);                                    \
   } while (0)
   // One block: the wave parks its W rows (wave-private tile, read back in operand order) and re-uses those
   // registers for the block kRing further on; the workgroup swaps the X block in LDS (barrier: everyone has
-  // finished the previous block; barrier: the new block is complete) and requests the X block after next;
-  // then the products run. Loads return in order, so the order of the requests is pinned (scheduling
-  // barriers) to the order their data is awaited in, and X is requested TWO blocks ahead: an X block comes
-  // from L2 but queues behind the W block requested an iteration earlier, which comes from HBM - requested
-  // one block ahead, every X wait was a wait for that W block's HBM latency.
-#define NV_BLK_ITER(BUF, XB, XNEXT, WNEXT)                                                          \
+  // finished the previous block; barrier: the new block is complete); then the products run, with the
+  // requests for the X block after next (XEN: block XBLK) and the W block kRing ahead (WEN: block WBLK)
+  // between them. Loads return in order, so the order of the requests is pinned (scheduling barriers) to
+  // the order their data is awaited in.
+#define NV_BLK_ITER(BUF, XB, XEN, XBLK, WEN, WBLK)                                                  \
   NV_BLK_WPARK(BUF);                                                                                \
   __syncthreads();                                                                                  \
   NV_BLK_XPARK(XB);                                                                                 \
   __syncthreads();                                                                                  \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  XNEXT;                                                                                            \
-  __builtin_amdgcn_sched_barrier(0);                                                                \
-  WNEXT;                                                                                            \
-  __builtin_amdgcn_sched_barrier(0);                                                                \
-  NV_BLK_COMPUTE()
+  NV_BLK_COMPUTE(BUF, XB, XEN, XBLK, WEN, WBLK)
 
   NV_BLK_W(0, 0);
   __builtin_amdgcn_sched_barrier(0);
@@ -211,24 +227,24 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
     NV_BLK_W(3, 3);
     __builtin_amdgcn_sched_barrier(0);
     for (; blk + 4 < nblk; blk += 4) {
-      NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), NV_BLK_W(0, blk + 4));
-      NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), NV_BLK_W(1, blk + 5));
-      NV_BLK_ITER(2, 0, NV_BLK_X(0, blk + 4), NV_BLK_W(2, blk + 6));
-      NV_BLK_ITER(3, 1, NV_BLK_X(1, blk + 5), NV_BLK_W(3, blk + 7));
+      NV_BLK_ITER(0, 0, true, blk + 2, true, blk + 4);
+      NV_BLK_ITER(1, 1, true, blk + 3, true, blk + 5);
+      NV_BLK_ITER(2, 0, true, blk + 4, true, blk + 6);
+      NV_BLK_ITER(3, 1, true, blk + 5, true, blk + 7);
     }
-    NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), (void)0);
-    NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), (void)0);
-    NV_BLK_ITER(2, 0, (void)0, (void)0);
-    NV_BLK_ITER(3, 1, (void)0, (void)0);
+    NV_BLK_ITER(0, 0, true, blk + 2, false, 0);
+    NV_BLK_ITER(1, 1, true, blk + 3, false, 0);
+    NV_BLK_ITER(2, 0, false, 0, false, 0);
+    NV_BLK_ITER(3, 1, false, 0, false, 0);
   } else {
     NV_BLK_W(1, 1);
     __builtin_amdgcn_sched_barrier(0);
     for (; blk + 2 < nblk; blk += 2) {
-      NV_BLK_ITER(0, 0, NV_BLK_X(0, blk + 2), NV_BLK_W(0, blk + 2));
-      NV_BLK_ITER(1, 1, NV_BLK_X(1, blk + 3), NV_BLK_W(1, blk + 3));
+      NV_BLK_ITER(0, 0, true, blk + 2, true, blk + 2);
+      NV_BLK_ITER(1, 1, true, blk + 3, true, blk + 3);
     }
-    NV_BLK_ITER(0, 0, (void)0, (void)0);
-    NV_BLK_ITER(1, 1, (void)0, (void)0);
+    NV_BLK_ITER(0, 0, false, 0, false, 0);
+    NV_BLK_ITER(1, 1, false, 0, false, 0);
   }
 #undef NV_BLK_W
 #undef NV_BLK_WPARK
@@ -239,6 +255,9 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 #undef NV_BLK_READ_B
 #undef NV_BLK_PRODUCTS
 #undef NV_BLK_STEP
+#undef NV_BLK_SLOT
+#undef NV_BLK_W1
+#undef NV_BLK_X1
 #undef NV_BLK_ITER
 
   // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
