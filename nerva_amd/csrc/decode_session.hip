@@ -1527,6 +1527,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.out_f32 = lead->pqkv;
       g.rows = A + 2 * KV;
       g.cols = H;
+      g.workspace = lead->pgemm_ws;
+      g.workspace_bytes = lead->pgemm_ws_bytes;
       err = launch_gemm_rows(lead->dtype, kGemmF32, g, st);
     }
     AttnParams a{};
@@ -1566,6 +1568,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.out_f32 = lead->pr;
       g.rows = H;
       g.cols = A;
+      g.workspace = lead->pgemm_ws;
+      g.workspace_bytes = lead->pgemm_ws_bytes;
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
     if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st, tiles);
@@ -1579,6 +1583,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.out_packed_tiles = tiles;
       g.rows = I;
       g.cols = H;
+      g.workspace = lead->pgemm_ws;
+      g.workspace_bytes = lead->pgemm_ws_bytes;
       err = launch_gemm_rows(lead->dtype, kGemmSwiglu, g, st);
     }
     if (err == hipSuccess) {
@@ -1591,6 +1597,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.out_f32 = lead->px;
       g.rows = H;
       g.cols = I;
+      g.workspace = lead->pgemm_ws;
+      g.workspace_bytes = lead->pgemm_ws_bytes;
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
     out->pack_kernel_launches += 2;
@@ -1607,6 +1615,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     g.out_f32 = lead->blogits;
     g.rows = lead->vocab;
     g.cols = H;
+    g.workspace = lead->pgemm_ws;
+    g.workspace_bytes = lead->pgemm_ws_bytes;
     err = launch_gemm_rows(lead->dtype, kGemmF32, g, st);
     out->pack_kernel_launches += 1;
     out->projection_kernel_launches += 1;

@@ -1,5 +1,5 @@
-// Multi-row projection for large token blocks (65..128 rows, X in matrix-operand order): the X operand
-// is shared through LDS instead of being fetched by every wave (see gemm_rows.cuh).
+// Multi-row projection for token blocks of 17..128 rows with X in matrix-operand order: the X operand is
+// shared through LDS instead of being fetched by every wave (see gemm_rows.cuh).
 //
 // gemm_rows_kernel gives a workgroup 16 weight rows over the whole K and lets its 8 waves split K, so
 // every wave fetches its own X pieces from L2: per matrix instruction 0.6 vector-memory reads, and the
@@ -27,10 +27,7 @@ constexpr int kBThreads = kBW * kWave;
 constexpr int kBK = 128;                     // columns per K-block
 constexpr int kBSteps = kBK / 32;            // matrix-core K-steps per block
 constexpr int kBRing = 4;                    // W blocks a wave requests ahead at most (two with one row tile per wave)
-constexpr int kBTiles = 8;                   // token tiles (X in operand order with 8 tiles)
-constexpr int kBStageVec = kBSteps * kBTiles * kWave;   // 16-byte pieces of one X block: 2048 = 32 KiB
-constexpr int kBFill = kBStageVec / kBThreads;          // pieces per thread and block: 8
-constexpr uint32_t kBTokCap = 16u * kBTiles;
+constexpr uint32_t kBTokCap = 128;           // token rows at most; also the token stride of the partial sums
 constexpr int kBRowStride = kBK + 8;         // LDS row stride of a W tile in elements: 16 B of padding keeps the
                                              // 16 rows of an operand read on distinct banks
 constexpr int kBWTile = 16 * kBRowStride;    // one 16-row block of W in LDS
@@ -91,13 +88,16 @@ __device__ __forceinline__ void block_epilogue(const GemmRowsParams &p, uint32_t
 // One row tile per wave: two W blocks requested ahead, two workgroups share a CU. Two row tiles: a wave
 // takes more than 256 registers, a CU holds one workgroup, and four W blocks are requested ahead to make
 // up for it (measured: gate_up 62.5 -> 54.4 us with four; the one-tile projections lose 5-8 % with four).
-template <uint32_t DT, int EPI, int NR>
+template <uint32_t DT, int EPI, int NR, int TT>
 __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(GemmRowsParams p, float *partials) {
+  constexpr int kTiles = TT;                              // 16-token tiles of the block (X in operand order with TT tiles)
+  constexpr int kStageVec = kBSteps * kTiles * kWave;     // 16-byte pieces of one X block (TT = 8: 2048 = 32 KiB)
+  constexpr int kFill = kStageVec / kBThreads;            // pieces per thread and block
   extern __shared__ __align__(16) unsigned char smem[];
-  u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);   // [kBStageVec]: the X block, shared by the four waves
+  u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);   // [kStageVec]: the X block, shared by the four waves
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  uint16_t *wtile = reinterpret_cast<uint16_t *>(smem + kBStageVec * sizeof(u32x4_t)) + wave * NR * kBWTile;   // wave-private
+  uint16_t *wtile = reinterpret_cast<uint16_t *>(smem + kStageVec * sizeof(u32x4_t)) + wave * NR * kBWTile;   // wave-private
   const uint32_t n = lane & 15, q = lane >> 4;
   const uint32_t cols = p.cols, T = p.tokens;
   const uint32_t kslices = gridDim.y, kper = cols / kslices, k0 = blockIdx.y * kper, nblk = kper / kBK;
@@ -119,18 +119,18 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   const uint32_t wlane = (q * cols + n * 8u) * static_cast<uint32_t>(sizeof(uint16_t));
   uint16_t *park_at = wtile + q * kBRowStride + n * 8;
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
-  // X block b of this slice: kBStageVec pieces in a row
-  const char *xbase = reinterpret_cast<const char *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kBTiles * kWave) * sizeof(u32x4_t);
+  // X block b of this slice: kStageVec pieces in a row
+  const char *xbase = reinterpret_cast<const char *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kTiles * kWave) * sizeof(u32x4_t);
   const uint32_t xlane = threadIdx.x * static_cast<uint32_t>(sizeof(u32x4_t));
 
   constexpr int kRing = NR == 1 ? 2 : kBRing;   // W blocks requested ahead: what the register budget holds
   u32x4_t areg[kRing][NR][4];
-  u32x4_t xreg[2][kBFill];   // the X blocks one and two ahead
-  f32x4_t acc[NR][kBTiles];
+  u32x4_t xreg[2][kFill];   // the X blocks one and two ahead
+  f32x4_t acc[NR][kTiles];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
 #pragma unroll
-    for (int c = 0; c < kBTiles; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = 0; c < kTiles; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
 #define NV_BLK_W(BUF, BLK)                                                                          \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
@@ -140,11 +140,11 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]
 #define NV_BLK_X(XB, BLK)                                                                           \
-  _Pragma("unroll") for (int i = 0; i < kBFill; ++i)                                                 \
+  _Pragma("unroll") for (int i = 0; i < kFill; ++i)                                                 \
       xreg[XB][i] = *reinterpret_cast<const u32x4_t *>(                                              \
-          xbase + (static_cast<uint64_t>(BLK) * kBStageVec + i * kBThreads) * sizeof(u32x4_t) + xlane)
+          xbase + (static_cast<uint64_t>(BLK) * kStageVec + i * kBThreads) * sizeof(u32x4_t) + xlane)
 #define NV_BLK_XPARK(XB)                                                                            \
-  _Pragma("unroll") for (int i = 0; i < kBFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[XB][i]
+  _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[XB][i]
   // LDS operand reads run one half K-step ahead of the products that use them: once the products of token
   // tiles 0..3 have been issued their B registers take the next K-step's pieces, likewise tiles 4..7, so a
   // read has the other half's products (128 cycles of matrix-core time per row tile) to arrive in. The
@@ -153,9 +153,9 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   _Pragma("unroll") for (int j = 0; j < NR; ++j)                                                     \
       A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32)
 #define NV_BLK_READ_B(S, C0)                                                                        \
-  _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c) b[c] = stage[((S) * kBTiles + c) * kWave + lane]
+  _Pragma("unroll") for (int c = C0; c < C0 + kTiles / 2; ++c) b[c] = stage[((S) * kTiles + c) * kWave + lane]
 #define NV_BLK_PRODUCTS(A, C0)                                                                      \
-  _Pragma("unroll") for (int c = C0; c < C0 + kBTiles / 2; ++c)                                      \
+  _Pragma("unroll") for (int c = C0; c < C0 + kTiles / 2; ++c)                                      \
       _Pragma("unroll") for (int j = 0; j < NR; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
   // The requests for the blocks ahead go out between the products, two per half K-step (first the X pieces,
   // then the W rows: the order they are awaited in): the CU's vector-memory path takes 64 bytes a cycle, and
@@ -165,10 +165,10 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
       wbase[J] + (static_cast<uint64_t>(4 * (I)) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
 #define NV_BLK_X1(XB, BLK, I)                                                                       \
   xreg[XB][I] = *reinterpret_cast<const u32x4_t *>(                                                  \
-      xbase + (static_cast<uint64_t>(BLK) * kBStageVec + (I) * kBThreads) * sizeof(u32x4_t) + xlane)
+      xbase + (static_cast<uint64_t>(BLK) * kStageVec + (I) * kBThreads) * sizeof(u32x4_t) + xlane)
 #define NV_BLK_SLOT(K, BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   if constexpr ((K) < 4) {                                                                          \
-    if constexpr (XEN) {                                                                            \
+    if constexpr (XEN && 2 * (K) < kFill) {                                                         \
       NV_BLK_X1(XB, XBLK, 2 * (K));                                                                 \
       NV_BLK_X1(XB, XBLK, 2 * (K) + 1);                                                             \
     }                                                                                               \
@@ -183,17 +183,17 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   if (!(LAST)) { NV_BLK_READ_B((S) + 1, 0); }                                                       \
   NV_BLK_SLOT(2 * (S), BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  NV_BLK_PRODUCTS(ACUR, kBTiles / 2);                                                               \
+  NV_BLK_PRODUCTS(ACUR, kTiles / 2);                                                               \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  if (!(LAST)) { NV_BLK_READ_B((S) + 1, kBTiles / 2); }                                             \
+  if (!(LAST)) { NV_BLK_READ_B((S) + 1, kTiles / 2); }                                             \
   NV_BLK_SLOT(2 * (S) + 1, BUF, XB, XEN, XBLK, WEN, WBLK)                                           \
   __builtin_amdgcn_sched_barrier(0)
 #define NV_BLK_COMPUTE(BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   do {                                                                                              \
-    u32x4_t a0[NR], a1[NR], b[kBTiles];                                                             \
+    u32x4_t a0[NR], a1[NR], b[kTiles];                                                             \
     NV_BLK_READ_A(0, a0);                                                                           \
     NV_BLK_READ_B(0, 0);                                                                            \
-    NV_BLK_READ_B(0, kBTiles / 2);                                                                  \
+    NV_BLK_READ_B(0, kTiles / 2);                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                              \
     NV_BLK_STEP(0, a0, a1, false, BUF, XB, XEN, XBLK, WEN, WBLK);                                   \
     NV_BLK_STEP(1, a1, a0, false, BUF, XB, XEN, XBLK, WEN, WBLK);                                   \
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
   if (kslices == 1) {
 #pragma unroll
-    for (int c = 0; c < kBTiles; ++c) {
+    for (int c = 0; c < kTiles; ++c) {
       const uint32_t t = c * 16u + n;
       if (t < T) {
         if constexpr (EPI == kGemmSwiglu) {
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
     const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
     float *part = partials + static_cast<uint64_t>(blockIdx.y) * kBTokCap * wrows;
 #pragma unroll
-    for (int c = 0; c < kBTiles; ++c) {
+    for (int c = 0; c < kTiles; ++c) {
       const uint32_t t = c * 16u + n;
       if (t < T) {
 #pragma unroll
@@ -317,26 +317,26 @@ __global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p
   block_epilogue<DT, EPI>(p, t, row, y, up);
 }
 
-template <int NR>
+template <int NR, int TT>
 constexpr size_t block_lds_bytes() {
-  return kBStageVec * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
+  return static_cast<size_t>(kBSteps) * TT * kWave * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
 }
 
-template <uint32_t DT, int EPI, int NR>
-hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+template <uint32_t DT, int EPI, int NR, int TT>
+hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
   const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kBW : 16u * kBW * NR;
-  constexpr size_t lds = block_lds_bytes<NR>();
+  constexpr size_t lds = block_lds_bytes<NR, TT>();
   if (lds > 64 * 1024) {
     // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR, TT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
+  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, TT>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
                      p, partials);
   hipError_t err = hipGetLastError();
   if (err == hipSuccess && kslices > 1) {
@@ -346,6 +346,16 @@ hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t ks
     err = hipGetLastError();
   }
   return err;
+}
+
+template <uint32_t DT, int EPI, int NR>
+hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  switch (p.x_packed) {   // token tiles of the block = tiles of its operand-order layout
+    case 2: return launch_block_tt<DT, EPI, NR, 2>(p, partials, kslices, stream);
+    case 4: return launch_block_tt<DT, EPI, NR, 4>(p, partials, kslices, stream);
+    case 8: return launch_block_tt<DT, EPI, NR, 8>(p, partials, kslices, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <uint32_t DT>
@@ -378,7 +388,11 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   }();
   static const int want_slices = env_int("NERVA_HIP_GEMM_BLOCK_SLICES");   // tuning: K slices for every projection
   static const int want_tiles = env_int("NERVA_HIP_GEMM_BLOCK_ROW_TILES"); // tuning: 1 or 2 row tiles per wave
-  if (mode == 0 || tokens <= 64 || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (kBRing * kBK) != 0) return plan;
+  static const uint32_t min_tokens = [] {
+    const int v = env_int("NERVA_HIP_GEMM_BLOCK_MIN_TOKENS");   // tuning: smallest block this kernel takes
+    return v > 0 ? static_cast<uint32_t>(v) : 17u;
+  }();
+  if (mode == 0 || tokens < min_tokens || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (kBRing * kBK) != 0) return plan;
   const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
   // Row tiles per wave: two where that still leaves a workgroup for most CUs.
   uint32_t tiles = epilogue == kGemmSwiglu ? 2u : (rows / (16u * kBW * 2u) >= 96u && rows % (16u * kBW * 2u) == 0 ? 2u : 1u);
@@ -388,6 +402,10 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   // (A sliced gate/up pair would write and re-read 12.6 MB of partial sums per slice: measured no faster.)
   uint32_t slices = 1;
   while (epilogue != kGemmSwiglu && groups * slices < 384u && cols % (slices * 2u * kBRing * kBK) == 0) slices *= 2u;
+  // A projection that would need eight or more slices of four K-blocks each (the o projection, 4096 x 4096)
+  // stays with gemm_rows_kernel: pipelines that short plus the second launch measured 12.6 / 15.9 / 20.0 us
+  // against 10.4 / 13.9 / 19.5 at 32 / 64 / 128 rows.
+  if (want_slices == 0 && slices >= 8 && cols / slices <= 4u * kBK) return plan;
   if (want_slices > 0 && cols % (static_cast<uint32_t>(want_slices) * kBRing * kBK) == 0) slices = want_slices;
   if (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) {
     // not enough room for the partial sums: as many slices as fit (a power of two), or none
@@ -405,7 +423,7 @@ uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {
 
 hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,
                              hipStream_t stream) {
-  if (plan.kslices == 0 || p.x_packed != kBTiles) return hipErrorInvalidValue;
+  if (plan.kslices == 0 || p.x_packed == 0 || p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;
   if (plan.kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
   if (dtype == kBF16) return launch_block_dt<kBF16>(epilogue, p, plan, stream);
   if (dtype == kF16) return launch_block_dt<kF16>(epilogue, p, plan, stream);

@@ -624,9 +624,9 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
     y0, y1 = N.DeviceBuffer(tokens * rows * 4), N.DeviceBuffer(tokens * rows * 4)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(x), out_f32=y0)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(packed), out_f32=y1, input_operand_order=True)
-    # blocks of more than 64 rows in operand order may take the kernel that shares X through LDS: the same
+    # blocks of more than 16 rows in operand order may take the kernel that shares X through LDS: the same
     # products summed in another order
-    same_kernel = tokens <= 64 or rows % 64 != 0
+    same_kernel = tokens <= 16 or rows % 64 != 0 or cols % 512 != 0
     if same_kernel:
         assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
     else:
@@ -648,10 +648,11 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
 
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 65), (192, 2048, 100), (4096, 4096, 128), (6144, 4096, 127),
-                                               (4096, 12288, 128)])
+                                               (4096, 12288, 128), (192, 2048, 17), (64, 2048, 33), (4096, 4096, 32),
+                                               (6144, 4096, 48), (4096, 12288, 64)])
 def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
-    """More than 64 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
-    X from LDS. Every token row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
+    """More than 16 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
+    X from LDS (2, 4 or 8 token tiles). Every token row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
     dtype = BF16
     rng = np.random.default_rng(rows + cols + tokens)
     if rows * cols > 1 << 22:
@@ -681,7 +682,7 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
 
 
 @pytest.mark.parametrize("sliced", [False, True])
-@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128)])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
