@@ -784,13 +784,22 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
     float M = -INFINITY, L = 0.0f, o = 0.0f;
     for (uint32_t s0 = 0; s0 < active; s0 += kTicketRound) {
       float mm[kTicketRound], ll[kTicketRound], aa[kTicketRound];
+      // m and l of this head's splits: the head is the same for all lanes of a wave, so lane i fetches
+      // m of split s0 + i and lane kTicketRound + i its l (one load a lane instead of two per split),
+      // and the values are handed round with lane reads below.
+      static_assert(2 * kTicketRound == kWave && kHD % kWave == 0, "one (m, l) pair per lane pair, one head per wave");
+      const uint32_t si_ml = min(s0 + static_cast<uint32_t>(lane & (kTicketRound - 1)), active - 1);
+      const float ml = load_coherent((lane < kTicketRound ? pm : pl) + si_ml);
 #pragma unroll
       for (int i = 0; i < kTicketRound; ++i) {
         // unconditional loads (index clamped): a load under a branch would serialise the round
         const uint32_t si = min(s0 + i, active - 1);
-        mm[i] = load_coherent(pm + si);
-        ll[i] = load_coherent(pl + si);
         aa[i] = load_coherent(src + static_cast<uint64_t>(si) * kHD);
+      }
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
+        mm[i] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ml), i));
+        ll[i] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ml), kTicketRound + i));
       }
 #pragma unroll
       for (int i = 0; i < kTicketRound; ++i) {
