@@ -171,6 +171,52 @@ def test_weight_plan_blocks_cut_across_tensors(source, tmp_path):
             N.DecodeSession.create(weights, 32, plan=plan)
 
 
+@pytest.mark.parametrize("model_type,shards,qk_norm,bias,tied", [("qwen3", 2, True, False, False),
+                                                                 ("llama", 1, False, True, False),
+                                                                 ("qwen3", 3, True, False, True)])
+def test_session_from_checkpoint_files(model_type, shards, qk_norm, bias, tied, tmp_path):
+    """The checkpoint planner end to end: a random model written out as config.json + safetensors shards
+    (tensors shuffled across the files) gives, through file-backed descriptors alone, the session a
+    pointer-fed create gives - same logits bit for bit, same K/V rows, same stream, same byte counts."""
+    from checkpoint_files import write_checkpoint
+    from nerva_amd import checkpoint as ckpt
+    dtype, hidden, heads, kv, hd, inter, vocab, layers = BF16, 256, 4, 2, 64, 520, 300, 2
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 47, 1e4, qk_norm=qk_norm, bias=bias)
+    if tied:
+        weights = N.ModelWeights(dtype, hidden, heads, kv, hd, inter, vocab, 1e-6, 1e4, weights.embeddings,
+                                 weights.layers, weights.final_norm, weights.embeddings)
+    write_checkpoint(str(tmp_path), weights, model_type, shards=shards, seed=shards, tied=tied,
+                     extra_config=dict(attention_bias=True) if bias else None)
+    prompt = np.random.default_rng(3).integers(0, vocab, 11).astype(np.uint32)
+    outcome = []
+    for from_files in (False, True):
+        plan = None
+        if from_files:
+            s, plan = ckpt.create_session(str(tmp_path), 32)
+        else:
+            s = N.DecodeSession.create(weights, 32)
+        rc, _ = s.start(prompt)
+        assert rc == 0
+        logits = s.logits()
+        rows = [s.kv_row(layer, 10) for layer in range(layers)]
+        rc, _, tokens = s.advance(8)
+        assert rc == 0
+        outcome.append((logits, rows, tokens.tolist(), s.create_result))
+        s.destroy()
+    (l0, r0, t0, c0), (l1, r1, t1, c1) = outcome
+    assert np.array_equal(l0, l1) and t0 == t1
+    for (k0, v0), (k1, v1) in zip(r0, r1):
+        assert np.array_equal(k0, k1) and np.array_equal(v0, v1)
+    assert c1.resident_weight_bytes == c0.resident_weight_bytes == c1.h2d_bytes == c1.planned_weight_bytes
+    assert c1.planned_weight_descriptor_count == len(plan.blocks) and c1.planned_weight_descriptor_hash == plan.descriptor_hash
+    # a shard that ends early is an error, not a silent short read
+    name, shard, begin, nbytes = plan.entries[-1]
+    with open(str(tmp_path / shard), "r+b") as f:
+        f.truncate(begin + nbytes - 64)
+    with pytest.raises((RuntimeError, ckpt.CheckpointError)):
+        ckpt.create_session(str(tmp_path), 32)
+
+
 def test_session_lifecycle_kat(kat):
     """create -> start -> advance in pieces; token accounting of the reference
     (session_api_lifecycle.inc.cu:992-1311): the first advance(n) does n-1 replays."""
