@@ -35,6 +35,65 @@ __device__ __forceinline__ float dot16_fp8(const uint4 &w, const float *x) {
   return acc;
 }
 
+// Lean-kernel operand order in LDS. A lane owns 16 consecutive columns of every 1024-column chunk
+// (the 16 weights of its 16-byte request). Stored column after column, the lanes of a wave would read
+// 16-byte pieces 64 bytes apart (32 for 16-bit values) and collide on the banks; instead a chunk is
+// kept as planes of one 16-byte piece per lane - piece j of lane l at [chunk][j][l] - so that a wave's
+// read of piece j is 1 KiB in a row.
+//   f32 values: 4 planes of 4 columns; 16-bit values: 2 planes of 8 columns.
+__device__ __forceinline__ uint32_t lean_slot_f32(uint32_t c) {
+  const uint32_t i = c & 15u, lane = (c >> 4) & 63u;
+  return (c & ~1023u) + (i >> 2) * 256u + lane * 4u + (i & 3u);
+}
+__device__ __forceinline__ uint32_t lean_slot_16(uint32_t c) {
+  const uint32_t i = c & 15u, lane = (c >> 4) & 63u;
+  return (c & ~1023u) + (i >> 3) * 512u + lane * 8u + (i & 7u);
+}
+
+// 16 e4m3fn weights times the lane's 16 f32 activations in lean order (xp -> piece 0 of the lane).
+__device__ __forceinline__ float dot16_fp8_lean(const uint4 &w, const float *xp) {
+  float f[4];
+  float acc = 0.0f;
+  const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    fp8x4_to_f32(words[i], f);
+    const float4 xv = *reinterpret_cast<const float4 *>(xp + 256 * i);
+    acc = fmaf(f[0], xv.x, acc);
+    acc = fmaf(f[1], xv.y, acc);
+    acc = fmaf(f[2], xv.z, acc);
+    acc = fmaf(f[3], xv.w, acc);
+  }
+  return acc;
+}
+
+// The same against 16-bit activations: e4m3fn values are exact in bf16 and in f16, so two weights
+// become one packed 16-bit pair (gfx950 scaled conversion, scale 1) and meet their activation pair in
+// one dot2 with f32 accumulation - half the instructions and half the LDS bytes of the f32 route.
+typedef __bf16 lean_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 lean_f16x2_t __attribute__((ext_vector_type(2)));
+template <uint32_t DT>
+__device__ __forceinline__ float dot4_fp8_x16(uint32_t w, uint32_t x01, uint32_t x23, float acc) {
+  if constexpr (DT == kBF16) {
+    const lean_bf16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+    const lean_bf16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(lo, __builtin_bit_cast(lean_bf16x2_t, x01), acc, false);
+    return __builtin_amdgcn_fdot2_f32_bf16(hi, __builtin_bit_cast(lean_bf16x2_t, x23), acc, false);
+  } else {
+    const lean_f16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    const lean_f16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+    acc = __builtin_amdgcn_fdot2(lo, __builtin_bit_cast(lean_f16x2_t, x01), acc, false);
+    return __builtin_amdgcn_fdot2(hi, __builtin_bit_cast(lean_f16x2_t, x23), acc, false);
+  }
+}
+template <uint32_t DT>
+__device__ __forceinline__ float dot16_fp8_x16(const uint4 &w, const uint4 &xa, const uint4 &xb) {
+  float acc = dot4_fp8_x16<DT>(w.x, xa.x, xa.y, 0.0f);
+  acc = dot4_fp8_x16<DT>(w.y, xa.z, xa.w, acc);
+  acc = dot4_fp8_x16<DT>(w.z, xb.x, xb.y, acc);
+  return dot4_fp8_x16<DT>(w.w, xb.z, xb.w, acc);
+}
+
 // Stage x (16-bit or f32) into LDS as f32.
 template <uint32_t DT>
 __device__ __forceinline__ void stage_x(float *xs, const uint16_t *x16, const float *xf, uint32_t cols) {
@@ -213,7 +272,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
 // ---------------------------------------------------------------------------
 template <uint32_t DT>
 __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Params p) {
-  extern __shared__ __align__(16) float xsf[];
+  extern __shared__ __align__(16) uint16_t xs16[];  // the 16-bit activations as they came, in lean order
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
@@ -259,9 +318,11 @@ __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Param
   float ag = 0.0f, au = 0.0f;
 #define NV_GU_CONSUME(J)                                                                      \
   do {                                                                                        \
-    const float *xp = xsf + cb * 1024u + lane * 16;                                           \
-    ag = fmaf(fg##J, dot16_fp8(bg##J, xp), ag);                                               \
-    au = fmaf(fu##J, dot16_fp8(bu##J, xp), au);                                               \
+    const uint16_t *xp = xs16 + cb * 1024u + lane * 8;                                        \
+    const uint4 xa = *reinterpret_cast<const uint4 *>(xp);                                    \
+    const uint4 xb = *reinterpret_cast<const uint4 *>(xp + 512);                              \
+    ag = fmaf(fg##J, dot16_fp8_x16<DT>(bg##J, xa, xb), ag);                                   \
+    au = fmaf(fu##J, dot16_fp8_x16<DT>(bu##J, xa, xb), au);                                   \
     if (++cb == bpr) {                                                                        \
       cb = 0;                                                                                 \
       const float g = wave_sum(ag), u = wave_sum(au);                                         \
@@ -277,7 +338,8 @@ __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Param
   if (total > 1) NV_GU_ISSUE(1);
   if (total > 2) NV_GU_ISSUE(2);
   if (total > 3) NV_GU_ISSUE(3);
-  stage_x<DT>(xsf, p.x16, nullptr, p.hidden);
+  for (uint32_t c = threadIdx.x * 8; c < p.hidden; c += kBlock * 8)  // 8 columns = one piece of one lane
+    *reinterpret_cast<uint4 *>(xs16 + lean_slot_16(c)) = *reinterpret_cast<const uint4 *>(p.x16 + c);
   __syncthreads();
   for (uint32_t t = 0; t < total; t += 4) {
     NV_GU_CONSUME(0);
@@ -299,68 +361,122 @@ __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Param
 #undef NV_GU_CONSUME
 }
 
-// Down + combine, lean: the wave owns output rows 2u and 2u+1 and walks (expert, chunk)
-// batches; act[k] goes through a two-slot LDS buffer one expert ahead of its use.
-__global__ __launch_bounds__(kBlock, 4) void moe_down_lean_kernel(MoeFp8Params p) {
-  extern __shared__ __align__(16) float acts[];  // 2 x inter floats
+// Down + combine, lean. Four consumer waves each own output rows 2u and 2u+1 and walk (expert, chunk)
+// batches through a ring of four request buffers; a fifth wave does nothing but move act[k] into a
+// two-slot LDS buffer one expert ahead (lean order) - loads return in order, so a consumer that
+// fetched activations itself would have to wait for every weight batch it had requested before them,
+// once per expert. Expert ids and weights sit in LDS from the start for the same reason: the loop of a
+// consumer holds no vector load besides the ring's. P = inter / 1024 chunks per expert and row; P
+// divides the ring, so which ring slot starts or ends an expert is known at compile time and the
+// steady-state loop body is straight-line code: the compiler can count exactly how many younger
+// requests may stay in flight at each use instead of waiting for all of them.
+constexpr int kDownLeanThreads = kBlock + kWave;
+constexpr uint32_t kDownLeanMaxSlots = 65;  // top_k <= 64 routed experts + the shared one
+template <int P>
+__global__ __launch_bounds__(kDownLeanThreads, 5) void moe_down_lean_kernel(MoeFp8Params p) {
+  static_assert(P == 1 || P == 2 || P == 4, "P must divide the ring of four");
+  extern __shared__ __align__(16) float acts[];  // 2 x inter floats, lean order
+  __shared__ uint32_t sh_expert[kDownLeanMaxSlots];
+  __shared__ float sh_weight[kDownLeanMaxSlots];
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
-  const uint32_t sc_cols = (p.inter + p.block - 1) / p.block;
+  constexpr uint32_t inter = P * 1024u;
+  if (threadIdx.x < slots) {
+    uint32_t e = threadIdx.x < p.top_k ? p.expert_ids[threadIdx.x] : static_cast<uint32_t>(p.shared_index);
+    if (e >= p.num_experts) e = 0;
+    sh_expert[threadIdx.x] = e;
+    sh_weight[threadIdx.x] = threadIdx.x < p.top_k ? p.expert_weights[threadIdx.x] : 1.0f;
+  }
+  if (wave == kWavesPerBlock) {
+    // ---- the staging wave: act[k] -> LDS slot k & 1, published by the barrier that starts expert k
+    for (uint32_t k = 0; k < slots; ++k) {
+      float4 st[P * 4];
+#pragma unroll
+      for (int i = 0; i < P * 4; ++i)
+        st[i] = *reinterpret_cast<const float4 *>(p.act + static_cast<uint64_t>(k) * inter + (i * kWave + lane) * 4);
+      float *dst = acts + (k & 1u) * inter;
+#pragma unroll
+      for (int i = 0; i < P * 4; ++i)
+        *reinterpret_cast<float4 *>(dst + lean_slot_f32((i * kWave + lane) * 4)) = st[i];
+      __syncthreads();  // barrier k: expert k may be read; everyone has left slot (k + 1) & 1
+    }
+    return;
+  }
+  __syncthreads();  // barrier 0 (also publishes the expert table)
+  const uint32_t sc_cols = (inter + p.block - 1) / p.block;
   const uint64_t scale_stride = static_cast<uint64_t>((p.hidden + p.block - 1) / p.block) * sc_cols;
-  const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * p.inter;
+  const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * inter;
   const uint32_t unit = blockIdx.x * kWavesPerBlock + wave;  // the grid covers all row pairs exactly
   const uint32_t h0 = min(unit * 2, p.hidden - 1), h1 = min(unit * 2 + 1, p.hidden - 1);
-  const uint32_t bpe = p.inter / 1024u;       // batches per expert
-  const uint32_t total = slots * bpe;
+  const uint32_t total = slots * P;
 
-  uint32_t ik = 0, ib = 0;
+  uint32_t ik = 0;  // expert slot of the next request
   const uint8_t *w0 = nullptr, *w1 = nullptr;
   const float *s0 = nullptr, *s1 = nullptr;
-  uint4 ba0, ba1, ba2, ba3, bb0, bb1, bb2, bb3;
+  // The ring's requests are asynchronous loads issued by hand, and each batch is awaited with an
+  // explicit outstanding-request count just before its use (requests return in issue order: with
+  // four requests a batch, "at most 4 n outstanding" means the batch is complete once n newer batches
+  // have been requested). Left to the compiler's own bookkeeping the loop waited for the whole ring at
+  // every batch. These waves issue no other vector-memory instruction inside the loop.
+  typedef uint32_t dn_u32x4_t __attribute__((ext_vector_type(4)));
+  dn_u32x4_t ba0, ba1, ba2, ba3, bb0, bb1, bb2, bb3;
   float fa0, fa1, fa2, fa3, fb0, fb1, fb2, fb3;
+  // ring slot J always carries chunk J % P of an expert
 #define NV_DN_ISSUE(J)                                                                        \
   do {                                                                                        \
-    if (ib == 0) {                                                                            \
-      uint32_t e = ik < p.top_k ? p.expert_ids[ik] : static_cast<uint32_t>(p.shared_index);   \
-      if (e >= p.num_experts) e = 0;                                                          \
-      w0 = p.w_down + e * w_stride + static_cast<uint64_t>(h0) * p.inter + lane * 16;         \
-      w1 = p.w_down + e * w_stride + static_cast<uint64_t>(h1) * p.inter + lane * 16;         \
+    constexpr uint32_t ib_ = (J) % P;                                                         \
+    if constexpr (ib_ == 0) {                                                                 \
+      const uint32_t e = sh_expert[ik];                                                       \
+      w0 = p.w_down + e * w_stride + static_cast<uint64_t>(h0) * inter + lane * 16;           \
+      w1 = p.w_down + e * w_stride + static_cast<uint64_t>(h1) * inter + lane * 16;           \
       s0 = p.s_down + e * scale_stride + static_cast<uint64_t>(h0 / p.block) * sc_cols;       \
       s1 = p.s_down + e * scale_stride + static_cast<uint64_t>(h1 / p.block) * sc_cols;       \
     }                                                                                         \
-    ba##J = load_stream(w0 + ib * 1024u);                                                     \
-    bb##J = load_stream(w1 + ib * 1024u);                                                     \
-    fa##J = s0[(ib * 1024u + lane * 16) / p.block];                                           \
-    fb##J = s1[(ib * 1024u + lane * 16) / p.block];                                           \
-    if (++ib == bpe) {                                                                        \
-      ib = 0;                                                                                 \
-      ++ik;                                                                                   \
-    }                                                                                         \
+    const uint8_t *q0_ = w0 + ib_ * 1024u, *q1_ = w1 + ib_ * 1024u;                           \
+    const float *r0_ = s0 + (ib_ * 1024u + lane * 16) / p.block;                              \
+    const float *r1_ = s1 + (ib_ * 1024u + lane * 16) / p.block;                              \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(ba##J) : "v"(q0_) : "memory");   \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(bb##J) : "v"(q1_) : "memory");   \
+    asm volatile("global_load_dword %0, %1, off" : "=v"(fa##J) : "v"(r0_) : "memory");        \
+    asm volatile("global_load_dword %0, %1, off" : "=v"(fb##J) : "v"(r1_) : "memory");        \
+    if constexpr (ib_ == P - 1) ++ik;                                                         \
   } while (0)
-
-  uint32_t ck = 0, cb = 0;
-  float a0 = 0.0f, a1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
-#define NV_DN_STAGE(K)                                                                        \
+  // The wait and the hand-over of a batch to compiler-visible registers are one asm statement: the
+  // moves read the request's destination registers after the wait whatever registers the compiler
+  // picks for either side (a wait with the registers as in/out operands leaves it free to copy them
+  // before the wait).
+  dn_u32x4_t ua, ub;
+  float ga, gb;
+#define NV_DN_TAKE(WAIT, J)                                                                   \
+  asm volatile(WAIT "\n\tv_mov_b32 %0, %10\n\tv_mov_b32 %1, %11\n\tv_mov_b32 %2, %12\n\tv_mov_b32 %3, %13" \
+               "\n\tv_mov_b32 %4, %14\n\tv_mov_b32 %5, %15\n\tv_mov_b32 %6, %16\n\tv_mov_b32 %7, %17"     \
+               "\n\tv_mov_b32 %8, %18\n\tv_mov_b32 %9, %19"                                       \
+               : "=&v"(ua.x), "=&v"(ua.y), "=&v"(ua.z), "=&v"(ua.w), "=&v"(ub.x), "=&v"(ub.y),     \
+                 "=&v"(ub.z), "=&v"(ub.w), "=&v"(ga), "=&v"(gb)                                    \
+               : "v"(ba##J.x), "v"(ba##J.y), "v"(ba##J.z), "v"(ba##J.w), "v"(bb##J.x),             \
+                 "v"(bb##J.y), "v"(bb##J.z), "v"(bb##J.w), "v"(fa##J), "v"(fb##J)                  \
+               : "memory")
+#define NV_DN_AWAIT(J, NEWER)                                                                 \
   do {                                                                                        \
-    float *dst_ = acts + ((K) & 1u) * p.inter;                                                \
-    for (uint32_t c = threadIdx.x * 4; c < p.inter; c += kBlock * 4)                          \
-      *reinterpret_cast<float4 *>(dst_ + c) =                                                 \
-          *reinterpret_cast<const float4 *>(p.act + static_cast<uint64_t>(K) * p.inter + c);  \
+    if ((NEWER) >= 3u) NV_DN_TAKE("s_waitcnt vmcnt(12)", J);                                  \
+    else NV_DN_TAKE("s_waitcnt vmcnt(0)", J);                                                 \
   } while (0)
+#define NV_DN_U4(V) make_uint4((V).x, (V).y, (V).z, (V).w)
+
+  uint32_t ck = 0;  // expert slot being consumed
+  float a0 = 0.0f, a1 = 0.0f, t0 = 0.0f, t1 = 0.0f;
 #define NV_DN_CONSUME(J)                                                                      \
   do {                                                                                        \
-    if (cb == 0) {                                                                            \
-      /* expert ck starts: its activations were staged one expert ago; stage the next */     \
-      __syncthreads();                                                                        \
-      if (ck + 1 < slots) NV_DN_STAGE(ck + 1);                                                \
+    constexpr uint32_t cb_ = (J) % P;                                                         \
+    if constexpr (cb_ == 0) {                                                                 \
+      if (ck != 0) __syncthreads(); /* barrier ck; barrier 0 was taken above */               \
     }                                                                                         \
-    const float *xp = acts + (ck & 1u) * p.inter + cb * 1024u + lane * 16;                    \
-    a0 = fmaf(fa##J, dot16_fp8(ba##J, xp), a0);                                               \
-    a1 = fmaf(fb##J, dot16_fp8(bb##J, xp), a1);                                               \
-    if (++cb == bpe) {                                                                        \
-      cb = 0;                                                                                 \
-      const float weight = ck < p.top_k ? p.expert_weights[ck] : 1.0f;                        \
+    const float *xp = acts + (ck & 1u) * inter + cb_ * 1024u + lane * 4;                      \
+    a0 = fmaf(ga, dot16_fp8_lean(NV_DN_U4(ua), xp), a0);                                      \
+    a1 = fmaf(gb, dot16_fp8_lean(NV_DN_U4(ub), xp), a1);                                      \
+    if constexpr (cb_ == P - 1) {                                                             \
+      const float weight = sh_weight[ck];                                                     \
       t0 = fmaf(weight, wave_sum(a0), t0);                                                    \
       t1 = fmaf(weight, wave_sum(a1), t1);                                                    \
       a0 = 0.0f;                                                                              \
@@ -373,26 +489,46 @@ __global__ __launch_bounds__(kBlock, 4) void moe_down_lean_kernel(MoeFp8Params p
   if (total > 1) NV_DN_ISSUE(1);
   if (total > 2) NV_DN_ISSUE(2);
   if (total > 3) NV_DN_ISSUE(3);
-  NV_DN_STAGE(0u);
-  for (uint32_t t = 0; t < total; t += 4) {
+  uint32_t t = 0;
+  for (; t + 8 <= total; t += 4) {  // steady state: three newer batches behind every use
+    NV_DN_AWAIT(0, 3u);
+    NV_DN_CONSUME(0);
+    NV_DN_ISSUE(0);
+    NV_DN_AWAIT(1, 3u);
+    NV_DN_CONSUME(1);
+    NV_DN_ISSUE(1);
+    NV_DN_AWAIT(2, 3u);
+    NV_DN_CONSUME(2);
+    NV_DN_ISSUE(2);
+    NV_DN_AWAIT(3, 3u);
+    NV_DN_CONSUME(3);
+    NV_DN_ISSUE(3);
+  }
+  for (; t < total; t += 4) {       // the last four to seven batches wait for everything requested
+    NV_DN_AWAIT(0, 0u);
     NV_DN_CONSUME(0);
     if (t + 4 < total) NV_DN_ISSUE(0);
     if (t + 1 < total) {
+      NV_DN_AWAIT(1, 0u);
       NV_DN_CONSUME(1);
       if (t + 5 < total) NV_DN_ISSUE(1);
     }
     if (t + 2 < total) {
+      NV_DN_AWAIT(2, 0u);
       NV_DN_CONSUME(2);
       if (t + 6 < total) NV_DN_ISSUE(2);
     }
     if (t + 3 < total) {
+      NV_DN_AWAIT(3, 0u);
       NV_DN_CONSUME(3);
       if (t + 7 < total) NV_DN_ISSUE(3);
     }
   }
+#undef NV_DN_AWAIT
+#undef NV_DN_TAKE
+#undef NV_DN_U4
 #undef NV_DN_ISSUE
 #undef NV_DN_CONSUME
-#undef NV_DN_STAGE
   if (lane == 0) {
     if (unit * 2 < p.hidden) p.out[unit * 2] = t0;
     if (unit * 2 + 1 < p.hidden) p.out[unit * 2 + 1] = t1;
@@ -522,7 +658,7 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t blocks =
         static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 32u));
     const size_t lds = static_cast<size_t>(p.hidden) * sizeof(float);
-    if (fast_gu && aligned16(p.act)) {
+    if (fast_gu && aligned16(p.act) && aligned16(p.x16)) {
       // lean kernel: oversubscribed persistent-style grid, 8 workgroups per CU at most
       const uint32_t lean_blocks =
           static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u));
@@ -545,8 +681,13 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t units = (p.hidden + NR - 1) / NR;
     const uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
     const size_t lds = static_cast<size_t>(p.inter) * 2 * sizeof(float);
-    if (fast_dn && aligned16(p.act) && p.inter % 4u == 0)
-      hipLaunchKernelGGL(moe_down_lean_kernel, dim3(blocks), dim3(kBlock), lds, stream, p);
+    const bool lean_dn = fast_dn && aligned16(p.act) && slots <= kDownLeanMaxSlots;  // whole experts per ring of four 1024-column chunks
+    if (lean_dn && p.inter == 1024u)
+      hipLaunchKernelGGL(moe_down_lean_kernel<1>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
+    else if (lean_dn && p.inter == 2048u)
+      hipLaunchKernelGGL(moe_down_lean_kernel<2>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
+    else if (lean_dn && p.inter == 4096u)
+      hipLaunchKernelGGL(moe_down_lean_kernel<4>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
     else if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
     else hipLaunchKernelGGL((moe_down_kernel<NR, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
   }

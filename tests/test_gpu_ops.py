@@ -545,6 +545,41 @@ def test_moe_fp8_experts_match_oracle(hidden, inter, experts, top_k):
     assert rel_l2(out.numpy(np.float32), ref2) <= REL_L2
 
 
+@pytest.mark.parametrize("dtype", [BF16, F16])
+def test_moe_lean_kernels_decode_every_fp8_code(dtype):
+    """The production-shape MoE kernels turn pairs of e4m3fn weights into packed 16-bit pairs with the
+    hardware conversion (gate/up) or into f32 (down) and read the activations in their own LDS order. Here
+    every output meets exactly one weight code: gate row i holds code i % 256 in column i and the
+    activation vector is all ones, the up rows pick a 1, so act[i] = silu(value of the code) - every finite
+    code in four different lanes and pieces; down row h holds code h % 256 in column h, so out[h] =
+    value(code) * act[h]. Exact up to f32 rounding of silu."""
+    hidden = inter = 1024
+    B = 128
+    codes = np.arange(256, dtype=np.uint8)
+    codes[[0x7f, 0xff]] = 0                                  # the two NaN codes
+    values = O.decode_fp8(codes).astype(np.float64)
+    wg = np.zeros((1, inter, hidden), np.uint8)
+    wu = np.zeros_like(wg)
+    wd = np.zeros((1, hidden, inter), np.uint8)
+    idx = np.arange(inter)
+    wg[0, idx, idx] = codes[idx % 256]
+    wu[0, idx, (idx * 7 + 3) % hidden] = 0x38                # 1.0
+    wd[0, idx, idx] = codes[(idx + 64) % 256]
+    ones = np.ones((1, inter // B, hidden // B), np.float32)
+    x16 = O.encode16(dtype, np.ones(hidden))
+    ids, wts = np.zeros(1, np.uint32), np.ones(1, np.float32)
+    act = N.DeviceBuffer(inter * 4)
+    out = N.DeviceBuffer(hidden * 4)
+    N.moe_fp8_experts(hidden, inter, 1, 1, B, dev(x16), dev(ids), dev(wts), dev(wg), dev(ones), dev(wu), dev(ones),
+                      dev(wd), dev(ones), act, out, input_dtype=dtype)
+    g = values[idx % 256]
+    want_act = g / (1.0 + np.exp(-g))
+    got_act = act.numpy(np.float32).astype(np.float64)
+    assert np.allclose(got_act, want_act, rtol=2e-6, atol=1e-9)
+    want_out = values[(idx + 64) % 256] * got_act
+    assert np.allclose(out.numpy(np.float32), want_out, rtol=1e-6, atol=1e-12)
+
+
 def test_moe_forward_f32_kat_host_pointer_abi(kat):
     import ctypes as C
     k = kat["moe_routed_clamp"]
