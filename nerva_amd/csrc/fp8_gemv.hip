@@ -370,10 +370,11 @@ __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Param
 // divides the ring, so which ring slot starts or ends an expert is known at compile time and the
 // steady-state loop body is straight-line code: the compiler can count exactly how many younger
 // requests may stay in flight at each use instead of waiting for all of them.
-constexpr int kDownLeanThreads = kBlock + kWave;
+constexpr int kDownLeanMaxConsumers = 7;    // consumer waves of a workgroup (+ 1 staging wave: 512 threads at most)
+constexpr int kDownLeanMaxThreads = (kDownLeanMaxConsumers + 1) * kWave;
 constexpr uint32_t kDownLeanMaxSlots = 65;  // top_k <= 64 routed experts + the shared one
 template <int P>
-__global__ __launch_bounds__(kDownLeanThreads, 5) void moe_down_lean_kernel(MoeFp8Params p) {
+__global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(MoeFp8Params p) {
   static_assert(P == 1 || P == 2 || P == 4, "P must divide the ring of four");
   extern __shared__ __align__(16) float acts[];  // 2 x inter floats, lean order
   __shared__ uint32_t sh_expert[kDownLeanMaxSlots];
@@ -388,7 +389,8 @@ __global__ __launch_bounds__(kDownLeanThreads, 5) void moe_down_lean_kernel(MoeF
     sh_expert[threadIdx.x] = e;
     sh_weight[threadIdx.x] = threadIdx.x < p.top_k ? p.expert_weights[threadIdx.x] : 1.0f;
   }
-  if (wave == kWavesPerBlock) {
+  const int consumers = static_cast<int>(blockDim.x) / kWave - 1;  // the last wave stages
+  if (wave == consumers) {
     // ---- the staging wave: act[k] -> LDS slot k & 1, published by the barrier that starts expert k
     for (uint32_t k = 0; k < slots; ++k) {
       float4 st[P * 4];
@@ -407,7 +409,7 @@ __global__ __launch_bounds__(kDownLeanThreads, 5) void moe_down_lean_kernel(MoeF
   const uint32_t sc_cols = (inter + p.block - 1) / p.block;
   const uint64_t scale_stride = static_cast<uint64_t>((p.hidden + p.block - 1) / p.block) * sc_cols;
   const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * inter;
-  const uint32_t unit = blockIdx.x * kWavesPerBlock + wave;  // the grid covers all row pairs exactly
+  const uint32_t unit = blockIdx.x * consumers + wave;  // the grid covers all row pairs
   const uint32_t h0 = min(unit * 2, p.hidden - 1), h1 = min(unit * 2 + 1, p.hidden - 1);
   const uint32_t total = slots * P;
 
@@ -681,13 +683,28 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t units = (p.hidden + NR - 1) / NR;
     const uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
     const size_t lds = static_cast<size_t>(p.inter) * 2 * sizeof(float);
-    const bool lean_dn = fast_dn && aligned16(p.act) && slots <= kDownLeanMaxSlots;  // whole experts per ring of four 1024-column chunks
-    if (lean_dn && p.inter == 1024u)
-      hipLaunchKernelGGL(moe_down_lean_kernel<1>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
-    else if (lean_dn && p.inter == 2048u)
-      hipLaunchKernelGGL(moe_down_lean_kernel<2>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
-    else if (lean_dn && p.inter == 4096u)
-      hipLaunchKernelGGL(moe_down_lean_kernel<4>, dim3(blocks), dim3(kDownLeanThreads), lds, stream, p);
+    const bool lean_dn = fast_dn && aligned16(p.act) && slots <= kDownLeanMaxSlots &&
+                         (p.inter == 1024u || p.inter == 2048u || p.inter == 4096u);  // whole experts per ring of four chunks
+    if (lean_dn) {
+      // Consumer waves per workgroup: the count that puts the fewest row pairs on the busiest CU while
+      // every workgroup is resident at once (20 waves a CU at this kernel's register budget); hidden 7168
+      // = 14 pairs a CU = two workgroups of 7 + 1 waves.
+      uint32_t consumers = 4, best = ~0u;
+      for (uint32_t c = kDownLeanMaxConsumers; c >= 1; --c) {
+        const uint32_t wgs = (units + c - 1) / c, per_cu = 20u / (c + 1);
+        if (wgs > 256u * per_cu) continue;
+        const uint32_t load = (wgs + 255u) / 256u * c;
+        if (load < best) {
+          best = load;
+          consumers = c;
+        }
+      }
+      const uint32_t wgs = (units + consumers - 1) / consumers;
+      const dim3 block((consumers + 1) * kWave);
+      if (p.inter == 1024u) hipLaunchKernelGGL(moe_down_lean_kernel<1>, dim3(wgs), block, lds, stream, p);
+      else if (p.inter == 2048u) hipLaunchKernelGGL(moe_down_lean_kernel<2>, dim3(wgs), block, lds, stream, p);
+      else hipLaunchKernelGGL(moe_down_lean_kernel<4>, dim3(wgs), block, lds, stream, p);
+    }
     else if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
     else hipLaunchKernelGGL((moe_down_kernel<NR, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
   }
