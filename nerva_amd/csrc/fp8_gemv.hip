@@ -94,18 +94,26 @@ __device__ __forceinline__ float dot16_fp8_x16(const uint4 &w, const uint4 &xa, 
   return dot4_fp8_x16<DT>(w.w, xb.z, xb.w, acc);
 }
 
-// Stage x (16-bit or f32) into LDS as f32.
-template <uint32_t DT>
+// Stage x (16-bit or f32) into LDS. ORDER 0: f32, column after column; 1: f32 in lean order; 2: the
+// 16-bit values as they came, in lean order (x16 only, 16-byte aligned, cols % 8 == 0).
+constexpr int kXColumns = 0, kXLeanF32 = 1, kXLean16 = 2;
+template <uint32_t DT, int ORDER = kXColumns>
 __device__ __forceinline__ void stage_x(float *xs, const uint16_t *x16, const float *xf, uint32_t cols) {
-  if (x16 != nullptr) {
-    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) xs[c] = dec16<DT>(x16[c]);
+  if constexpr (ORDER == kXLean16) {
+    uint16_t *xs16 = reinterpret_cast<uint16_t *>(xs);
+    for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8)
+      *reinterpret_cast<uint4 *>(xs16 + lean_slot_16(c)) = *reinterpret_cast<const uint4 *>(x16 + c);
+  } else if (x16 != nullptr) {
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock)
+      xs[ORDER == kXLeanF32 ? lean_slot_f32(c) : c] = dec16<DT>(x16[c]);
   } else {
-    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) xs[c] = xf[c];
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) xs[ORDER == kXLeanF32 ? lean_slot_f32(c) : c] = xf[c];
   }
 }
 
-// UU consecutive 1024-column chunks of NR rows, all loads issued before the first use.
-template <int NR, int UU>
+// UU consecutive 1024-column chunks of NR rows, all loads issued before the first use. XT says how the
+// activations lie in LDS (lean orders: see lean_slot_f32 / lean_slot_16).
+template <uint32_t DT, int NR, int UU, int XT>
 __device__ __forceinline__ void fp8_chunks(const uint8_t *const (&wrow)[NR], const float *const (&srow)[NR],
                                            const float *xs, uint32_t chunk, uint32_t block_cols,
                                            int lane, float (&acc)[NR]) {
@@ -119,26 +127,38 @@ __device__ __forceinline__ void fp8_chunks(const uint8_t *const (&wrow)[NR], con
   for (int u = 0; u < UU; ++u) {
     const uint32_t c = c0 + u * 1024u;
     const uint32_t sidx = c / block_cols;
+    if constexpr (XT == kXLean16) {
+      const uint16_t *xp = reinterpret_cast<const uint16_t *>(xs) + (chunk + u) * 1024u + lane * 8;
+      const uint4 xa = *reinterpret_cast<const uint4 *>(xp), xb = *reinterpret_cast<const uint4 *>(xp + 512);
 #pragma unroll
-    for (int k = 0; k < NR; ++k) acc[k] = fmaf(srow[k][sidx], dot16_fp8(wv[k][u], xs + c), acc[k]);
+      for (int k = 0; k < NR; ++k) acc[k] = fmaf(srow[k][sidx], dot16_fp8_x16<DT>(wv[k][u], xa, xb), acc[k]);
+    } else if constexpr (XT == kXLeanF32) {
+      const float *xp = xs + (chunk + u) * 1024u + lane * 4;
+#pragma unroll
+      for (int k = 0; k < NR; ++k) acc[k] = fmaf(srow[k][sidx], dot16_fp8_lean(wv[k][u], xp), acc[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < NR; ++k) acc[k] = fmaf(srow[k][sidx], dot16_fp8(wv[k][u], xs + c), acc[k]);
+    }
   }
 }
 
 // NR rows x all columns for one wave; FAST: cols % 1024 == 0, block_cols % 16 == 0,
-// 16-byte aligned rows.
-template <int NR, bool FAST>
+// 16-byte aligned rows, activations in a lean order (XT); otherwise column order.
+template <uint32_t DT, int NR, bool FAST, int XT>
 __device__ __forceinline__ void fp8_rows(const uint8_t *const (&wrow)[NR], const float *const (&srow)[NR],
                                          const float *xs, uint32_t cols, uint32_t block_cols, int lane,
                                          float (&acc)[NR]) {
+  static_assert(FAST ? XT != kXColumns : XT == kXColumns, "lean orders belong to the chunked path");
   if constexpr (FAST) {
     const uint32_t nchunks = cols / 1024u;
     uint32_t chunk = 0;
-    for (; chunk + 4 <= nchunks; chunk += 4) fp8_chunks<NR, 4>(wrow, srow, xs, chunk, block_cols, lane, acc);
+    for (; chunk + 4 <= nchunks; chunk += 4) fp8_chunks<DT, NR, 4, XT>(wrow, srow, xs, chunk, block_cols, lane, acc);
     if (chunk + 2 <= nchunks) {
-      fp8_chunks<NR, 2>(wrow, srow, xs, chunk, block_cols, lane, acc);
+      fp8_chunks<DT, NR, 2, XT>(wrow, srow, xs, chunk, block_cols, lane, acc);
       chunk += 2;
     }
-    if (chunk < nchunks) fp8_chunks<NR, 1>(wrow, srow, xs, chunk, block_cols, lane, acc);
+    if (chunk < nchunks) fp8_chunks<DT, NR, 1, XT>(wrow, srow, xs, chunk, block_cols, lane, acc);
   } else {
     for (uint32_t c = lane; c < cols; c += kWave) {
 #pragma unroll
@@ -150,15 +170,15 @@ __device__ __forceinline__ void fp8_rows(const uint8_t *const (&wrow)[NR], const
   }
 }
 
-template <uint32_t DT, int NR, bool FAST>
+template <uint32_t DT, int NR, bool FAST, int XT = FAST ? kXLeanF32 : kXColumns>
 __global__ __launch_bounds__(kBlock) void fp8_gemv_kernel(Fp8GemvParams p) {
   extern __shared__ __align__(16) float xsf[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   for (uint32_t token = 0; token < p.tokens; ++token) {
     if (token != 0) __syncthreads();
-    stage_x<DT>(xsf, p.x16 ? p.x16 + static_cast<uint64_t>(token) * p.cols : nullptr,
-                p.xf ? p.xf + static_cast<uint64_t>(token) * p.cols : nullptr, p.cols);
+    stage_x<DT, XT>(xsf, p.x16 ? p.x16 + static_cast<uint64_t>(token) * p.cols : nullptr,
+                    p.xf ? p.xf + static_cast<uint64_t>(token) * p.cols : nullptr, p.cols);
     __syncthreads();
     const uint32_t scale_cols = (p.cols + p.block_cols - 1) / p.block_cols;
     const uint32_t units = (p.rows + NR - 1) / NR;
@@ -174,7 +194,7 @@ __global__ __launch_bounds__(kBlock) void fp8_gemv_kernel(Fp8GemvParams p) {
         srow[k] = p.scales + static_cast<uint64_t>(r / p.block_rows) * scale_cols;
         acc[k] = 0.0f;
       }
-      fp8_rows<NR, FAST>(wrow, srow, xsf, p.cols, p.block_cols, lane, acc);
+      fp8_rows<DT, NR, FAST, XT>(wrow, srow, xsf, p.cols, p.block_cols, lane, acc);
 #pragma unroll
       for (int k = 0; k < NR; ++k) {
         const float y = wave_sum(acc[k]);
@@ -192,7 +212,7 @@ __global__ __launch_bounds__(kBlock) void moe_gate_up_kernel(MoeFp8Params p) {
   extern __shared__ __align__(16) float xsf[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  stage_x<DT>(xsf, p.x16, nullptr, p.hidden);
+  stage_x<DT, FAST ? kXLeanF32 : kXColumns>(xsf, p.x16, nullptr, p.hidden);
   __syncthreads();
   const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
   const uint32_t units = slots * p.inter;
@@ -209,7 +229,7 @@ __global__ __launch_bounds__(kBlock) void moe_gate_up_kernel(MoeFp8Params p) {
     const float *srow[2] = {p.s_gate + e * scale_stride + static_cast<uint64_t>(i / p.block) * sc,
                             p.s_up + e * scale_stride + static_cast<uint64_t>(i / p.block) * sc};
     float acc[2] = {0.0f, 0.0f};
-    fp8_rows<2, FAST>(wrow, srow, xsf, p.hidden, p.block, lane, acc);
+    fp8_rows<DT, 2, FAST, FAST ? kXLeanF32 : kXColumns>(wrow, srow, xsf, p.hidden, p.block, lane, acc);
     const float g = wave_sum(acc[0]);
     const float u = wave_sum(acc[1]);
     if (lane == 0) p.act[static_cast<uint64_t>(k) * p.inter + i] = silu(g) * u;
@@ -235,7 +255,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
   for (uint32_t k = 0; k < slots; ++k) {
     float *buf = acts + (k & 1u) * p.inter;
     for (uint32_t c = threadIdx.x; c < p.inter; c += kBlock)
-      buf[c] = p.act[static_cast<uint64_t>(k) * p.inter + c];
+      buf[FAST ? lean_slot_f32(c) : c] = p.act[static_cast<uint64_t>(k) * p.inter + c];
     __syncthreads();  // double buffer: the previous expert's readers are at most one step behind
     uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);
     if (e >= p.num_experts) e = 0;
@@ -250,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
       srow[r] = p.s_down + e * scale_stride + static_cast<uint64_t>(h / p.block) * sc;
       acc[r] = 0.0f;
     }
-    fp8_rows<NR, FAST>(wrow, srow, buf, p.inter, p.block, lane, acc);
+    fp8_rows<kBF16, NR, FAST, FAST ? kXLeanF32 : kXColumns>(wrow, srow, buf, p.inter, p.block, lane, acc);
 #pragma unroll
     for (int r = 0; r < NR; ++r) total[r] = fmaf(weight, wave_sum(acc[r]), total[r]);
   }
@@ -611,29 +631,30 @@ hipError_t launch_fp8_gemv(const Fp8GemvParams &p, hipStream_t stream) {
   if (p.rows == 0 || p.cols == 0 || p.block_rows == 0 || p.block_cols == 0 || p.tokens == 0)
     return hipErrorInvalidValue;
   if (p.input_dtype > kBF16) return hipErrorInvalidValue;
-  const size_t lds = static_cast<size_t>(p.cols) * sizeof(float);
-  if (lds > 60 * 1024) return hipErrorInvalidValue;
   const bool fast = p.cols % 1024u == 0 && p.block_cols % 16u == 0 && aligned16(p.w);
+  // 16-bit activations stay 16 bit in LDS on the chunked path (half the bytes, and K up to 30720)
+  const bool x16_lean = fast && p.x16 != nullptr && aligned16(p.x16);
+  const size_t lds = static_cast<size_t>(p.cols) * (x16_lean ? sizeof(uint16_t) : sizeof(float));
+  if (lds > 60 * 1024) return hipErrorInvalidValue;
+  const bool bf = p.input_dtype == kBF16;
   if (fast) {
     // short rows: more rows per wave to keep the same number of bytes in flight
-    if (p.cols <= 2048u) {
-      const uint32_t units = (p.rows + 3) / 4;
-      const uint32_t blocks = std::min<uint32_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
-      if (p.input_dtype == kBF16)
-        hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 4, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
-      else
-        hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 4, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+    const bool four = p.cols <= 2048u;
+    const uint32_t units = four ? (p.rows + 3) / 4 : (p.rows + 1) / 2;
+    const uint32_t blocks = std::min<uint32_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
+#define NV_FP8_GEMV_LAUNCH(DT, NR, XT) \
+  hipLaunchKernelGGL((fp8_gemv_kernel<DT, NR, true, XT>), dim3(blocks), dim3(kBlock), lds, stream, p)
+    if (x16_lean) {
+      if (four) { if (bf) NV_FP8_GEMV_LAUNCH(kBF16, 4, kXLean16); else NV_FP8_GEMV_LAUNCH(kF16, 4, kXLean16); }
+      else { if (bf) NV_FP8_GEMV_LAUNCH(kBF16, 2, kXLean16); else NV_FP8_GEMV_LAUNCH(kF16, 2, kXLean16); }
     } else {
-      const uint32_t units = (p.rows + 1) / 2;
-      const uint32_t blocks = std::min<uint32_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
-      if (p.input_dtype == kBF16)
-        hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 2, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
-      else
-        hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 2, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
+      if (four) { if (bf) NV_FP8_GEMV_LAUNCH(kBF16, 4, kXLeanF32); else NV_FP8_GEMV_LAUNCH(kF16, 4, kXLeanF32); }
+      else { if (bf) NV_FP8_GEMV_LAUNCH(kBF16, 2, kXLeanF32); else NV_FP8_GEMV_LAUNCH(kF16, 2, kXLeanF32); }
     }
+#undef NV_FP8_GEMV_LAUNCH
   } else {
     const uint32_t blocks = std::min<uint32_t>((p.rows + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u);
-    if (p.input_dtype == kBF16)
+    if (bf)
       hipLaunchKernelGGL((fp8_gemv_kernel<kBF16, 1, false>), dim3(blocks), dim3(kBlock), lds, stream, p);
     else
       hipLaunchKernelGGL((fp8_gemv_kernel<kF16, 1, false>), dim3(blocks), dim3(kBlock), lds, stream, p);

@@ -150,6 +150,27 @@ def case_moe():
         report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
 
 
+def case_fp8_gemv():
+    """One FP8 block-scaled GEMV at DeepSeek-V3's dense shapes (o projection 7168x16384, dense-layer gate
+    18432x7168): e4m3fn weights, 128x128 f32 scales, bf16 activations, f32 output."""
+    lib = abi.load()
+    blk = 128
+    for name, rows, cols, copies in (("o 7168x16384", 7168, 16384, 10), ("gate 18432x7168", 18432, 7168, 9)):
+        sr, sc = (rows + blk - 1) // blk, (cols + blk - 1) // blk
+        w = DeviceBuffer(copies * rows * cols)
+        s = DeviceBuffer(copies * sr * sc * 4)
+        for i in range(copies):
+            assert lib.nerva_hip_synth_fill_fp8_block(w.ptr + i * rows * cols, s.ptr + i * sr * sc * 4, SEED, 4000 + i,
+                                                      rows, cols, blk, 0.02) == 0
+        x = synth16(cols, 43, std=1.0)
+        y = DeviceBuffer(rows * 4)
+        nbytes = rows * cols + sr * sc * 4 + cols * 2 + rows * 4
+        for variant, n in (("rotating", copies), ("resident", 1)):
+            ns = timed(lambda i: R.fp8_gemv(w.ptr + (i % n) * rows * cols, s.ptr + (i % n) * sr * sc * 4, rows, cols,
+                                            blk, blk, y, input16=x, sync=False), 3 * copies)
+            report("7 FP8 GEMV " + name, variant, ns, nbytes)
+
+
 def case_gemm_rows():
     """Token blocks through the step's weight matrices on the matrix cores: the weights are streamed once
     per block, so 32 tokens should cost about what one token costs."""
@@ -203,7 +224,8 @@ def main():
         print("no usable GPU (hip_error=%d): these operators have no CPU path" % smoke.hip_error, file=sys.stderr)
         sys.exit(1)
     log("device: %s" % smoke.gpu_name.decode())
-    cases = dict(qproj=case_qproj, mlp=case_mlp, attention=case_attention, moe=case_moe, sampler=case_sampler,
+    cases = dict(qproj=case_qproj, mlp=case_mlp, attention=case_attention, moe=case_moe, fp8_gemv=case_fp8_gemv,
+                 sampler=case_sampler,
                  gemm_rows=case_gemm_rows)
     for name, case in cases.items():      # `python -m nerva_amd.opbench gemm_rows sampler` runs only those
         if not only or name in only:
