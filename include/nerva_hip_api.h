@@ -530,6 +530,20 @@ typedef struct NervaHipArgmaxRequest {
 int nerva_hip_argmax(const NervaHipArgmaxRequest *request, void *stream, int32_t *hip_error);
 uint64_t nerva_hip_argmax_workspace_bytes(void);
 
+/* nerva_hip_argmax for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same rule and same
+ * result as nerva_hip_argmax; the per-workgroup candidates live in a 6 KiB array inside the
+ * library's device image instead of a caller workspace, and the call performs no hipMalloc, hipFree
+ * or other allocating routine: two kernel launches on `stream` (pass the caller's stream; NULL
+ * uses the library's stream, which exists once nerva_hip_device_smoke has run). `logits` and
+ * `token` are device pointers. count > NERVA_HIP_ARGMAX_STATIC_MAX_COUNT fails with
+ * hipErrorInvalidValue and launches nothing. All calls on one GPU share the array: calls that
+ * overlap on one GPU (different streams, or graphs replayed concurrently) race. The array's address
+ * is resolved at the first call on a device, or by nerva_hip_device_smoke. */
+#define NERVA_HIP_ARGMAX_STATIC_MAX_COUNT 16777216u
+int nerva_hip_argmax_static(const float *logits, uint32_t count, uint32_t *token, void *stream,
+                            int32_t *hip_error);
+
 typedef struct NervaHipGemmRowsRequest {
   uint32_t dtype;            /* NERVA_HIP_DTYPE_* of weights and 16-bit vectors */
   uint32_t rows, cols;       /* W is row-major [rows x cols] (epilogue 2: [2*rows x cols], gate rows first) */

@@ -3,11 +3,43 @@
 // to the lowest index (sampler.cu:35-40,89-119; common/token.rs:33-58).
 #include "argmax.cuh"
 
+#include <mutex>
+
 #include "gemv_stream.cuh"
+#include "runtime_state.hpp"
 
 namespace nv {
 
 namespace {
+
+// Candidate storage of nerva_hip_argmax_static: one (value, index, has) triple per workgroup of the
+// first launch, kept in the library's own device image so the call never allocates. Every GPU holds
+// its own copy at its own address; host code only ever uses the address that hipGetSymbolAddress
+// returned for the current device (static_scratch), never the array's name.
+constexpr uint32_t kArgmaxBlocks = 512;  // workgroups of the first launch (they loop over the logits)
+static __device__ __align__(256) uint32_t scratch[3 * kArgmaxBlocks];
+
+constexpr int kMaxDevices = 16;
+std::mutex g_scratch_mutex;
+uint32_t *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, resolved once per device.
+hipError_t static_scratch(uint32_t **out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return err;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void *ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (ptr == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = static_cast<uint32_t *>(ptr);
+  }
+  *out = g_scratch_ptr[device];
+  return hipSuccess;
+}
 
 __global__ __launch_bounds__(kBlock) void argmax_kernel(const float *logits, uint32_t count,
                                                         SampleParams s) {
@@ -55,7 +87,7 @@ hipError_t launch_argmax(const float *logits, uint32_t count, const SampleParams
                          hipStream_t stream) {
   if (logits == nullptr || count == 0 || s.part_value == nullptr) return hipErrorInvalidValue;
   uint32_t blocks = (count + kBlock * 8 - 1) / (kBlock * 8);
-  if (blocks > 512) blocks = 512;
+  if (blocks > kArgmaxBlocks) blocks = kArgmaxBlocks;
   if (blocks == 0) blocks = 1;
   hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(kBlock), 0, stream, logits, count, s);
   hipError_t err = hipGetLastError();
@@ -63,4 +95,39 @@ hipError_t launch_argmax(const float *logits, uint32_t count, const SampleParams
   return launch_sample_finish(s, blocks, nullptr, 0, stream);
 }
 
+hipError_t argmax_static_setup() {
+  uint32_t *ptr = nullptr;
+  return static_scratch(&ptr);
+}
+
 }  // namespace nv
+
+extern "C" {
+
+int nerva_hip_argmax_static(const float *logits, uint32_t count, uint32_t *token, void *stream,
+                            int32_t *hip_error) {
+  using namespace nv;
+  auto done = [&](hipError_t err) {
+    if (hip_error) *hip_error = static_cast<int32_t>(err);
+    return err == hipSuccess ? 0 : -1;
+  };
+  if (hip_error) *hip_error = 0;
+  if (logits == nullptr || token == nullptr || count == 0 || count > NERVA_HIP_ARGMAX_STATIC_MAX_COUNT)
+    return done(hipErrorInvalidValue);
+  // With a caller's stream nothing is created here; the library's own stream exists after
+  // nerva_hip_device_smoke (or any earlier call that used it).
+  hipStream_t s = resolve_stream(stream);
+  if (s == nullptr) return done(hipErrorInvalidResourceHandle);
+  uint32_t *base = nullptr;
+  hipError_t err = static_scratch(&base);
+  if (err != hipSuccess) return done(err);
+  SampleParams p{};
+  p.part_value = reinterpret_cast<float *>(base);
+  p.part_index = base + kArgmaxBlocks;
+  p.part_has = base + 2 * kArgmaxBlocks;
+  p.token_out = token;
+  // Both launches write every candidate they later read, so nothing has to be cleared between calls.
+  return done(launch_argmax(logits, count, p, s));
+}
+
+}  // extern "C"

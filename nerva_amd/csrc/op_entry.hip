@@ -204,6 +204,11 @@ int nerva_hip_device_smoke(NervaHipDeviceSmokeResult *out) {
   strncpy(out->gpu_name, prop.name[0] != '\0' ? prop.name : prop.gcnArchName, sizeof(out->gpu_name) - 1);
   char bus[32] = {0};
   if (hipDeviceGetPCIBusId(bus, sizeof(bus), 0) == hipSuccess) strncpy(out->pci_bus_id, bus, sizeof(out->pci_bus_id) - 1);
+  // set-up of the entry point that allocates nothing: its stream and its candidate array's address
+  if (library_stream() == nullptr || argmax_static_setup() != hipSuccess) {
+    out->hip_error = static_cast<int32_t>(hipErrorNotInitialized);
+    return -1;
+  }
   out->status = value == probe ? 0 : -1;
   return out->status;
 }

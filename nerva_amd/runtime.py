@@ -236,6 +236,16 @@ def argmax(logits_buf, count, workspace=None):
     return int(tok.numpy(np.uint32, 1)[0])
 
 
+def argmax_static(logits_buf, count, token_buf):
+    """nerva_hip_argmax_static: launches only, no allocation inside the library; the caller owns the
+    logits and the token word. Returns (rc, hip_error); synchronises when rc == 0."""
+    err = C.c_int32(0)
+    rc = abi.load().nerva_hip_argmax_static(_ptr(logits_buf), count, _ptr(token_buf), None, C.byref(err))
+    if rc == 0:
+        Device.synchronize()
+    return rc, err.value
+
+
 def gemm_operand_slots(tokens):
     """Token slots of a buffer in matrix-operand order for a block of `tokens` rows."""
     return 32 if tokens <= 32 else 64 if tokens <= 64 else 128
