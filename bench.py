@@ -54,41 +54,17 @@ def step_bytes(cfg, ctx_tokens):
 def cpu_baseline(session, cfg, position, token, layers_sampled, threads_all):
     """Time the oracle on `layers_sampled` layers + LM head of one decode step at `position`,
     on 1 core and on all cores, with the device's own weights (regenerated bit-identically on
-    the host) and the KV cache downloaded from the device prefill."""
+    the host) and the KV cache downloaded from the device prefill. Then, checker only, the device
+    runs that token with its step traced and every kernel of the sampled layers and of the head is
+    compared with the oracle operator on the device's own input (oracle/links.py)."""
     import oracle as O
-    H, A = cfg["hidden"], cfg["heads"] * cfg["head_dim"]
-    KV, I, V, HD, dt = cfg["kv_heads"] * cfg["head_dim"], cfg["intermediate"], cfg["vocab"], cfg["head_dim"], cfg["dtype"]
-
-    def gen(tid, n, mean=0.0):
-        chunk = 1 << 24
-        out = np.empty(n, np.uint16)
-
-        def work(start):
-            m = min(chunk, n - start)
-            out[start:start + m] = O.synth_16(dt, SEED, tid, m, mean, WEIGHT_STD, offset=start)
-        with concurrent.futures.ThreadPoolExecutor(max_workers=threads_all) as pool:
-            list(pool.map(work, range(0, n, chunk)))
-        return out
-
+    from oracle.links import check_step_links
+    dt = cfg["dtype"]
     t0 = time.time()
-    layers = []
-    for l in range(layers_sampled):
-        b = 16 * (l + 1)
-        layers.append(dict(rms_attn=gen(b, H, 1.0), rms_mlp=gen(b + 1, H, 1.0), w_q=gen(b + 2, A * H).reshape(A, H),
-                           w_k=gen(b + 4, KV * H).reshape(KV, H), q_norm=gen(b + 5, HD, 1.0), k_norm=gen(b + 6, HD, 1.0),
-                           w_v=gen(b + 7, KV * H).reshape(KV, H), w_o=gen(b + 8, H * A).reshape(H, A),
-                           w_gate=gen(b + 13, I * H).reshape(I, H), w_up=gen(b + 14, I * H).reshape(I, H),
-                           w_down=gen(b + 15, H * I).reshape(H, I)))
-    emb = np.zeros((token + 1, H), np.uint16)
-    emb[token] = O.synth_16(dt, SEED, 1, H, 0.0, WEIGHT_STD, offset=token * H)
-    lm_head = gen(3, V * H).reshape(V, H)
-    final_norm = gen(2, H, 1.0)
-    model = O.Model(dt, H, cfg["heads"], cfg["kv_heads"], HD, I, V, cfg["rms_eps"], cfg["rope_theta"], emb, layers,
-                    final_norm, lm_head)
+    model = O.synthetic_model(cfg, SEED, WEIGHT_STD, layers=layers_sampled, embedding_rows=[token], threads=threads_all)
     kv = [session.kv_range(l, 0, position) for l in range(layers_sampled)]
     log("[cpu] host weights + KV ready in %.1f s" % (time.time() - t0))
     result = {}
-    logits = None
     for threads in (1, threads_all):
         os.environ["OMP_NUM_THREADS"] = str(threads)
         ctx = O.Context(model, position + 2, staging=1, threads=threads)
@@ -99,31 +75,33 @@ def cpu_baseline(session, cfg, position, token, layers_sampled, threads_all):
         hidden = ctx.forward_token(token, prompt_token=False, want_logits=False)
         t_layers = time.time() - t0
         t0 = time.time()
-        normed = O.decode16(dt, O.encode16(dt, O.rms_norm(dt, hidden, final_norm, cfg["rms_eps"])))
-        logits = O.gemv(dt, lm_head, normed, threads=threads)
+        normed = O.decode16(dt, O.encode16(dt, O.rms_norm(dt, hidden, model.final_norm, cfg["rms_eps"])))
+        O.gemv(dt, model.lm_head, normed, threads=threads)
         t_head = time.time() - t0
         per_token = t_layers * cfg["layers"] / layers_sampled + t_head
         result[threads] = dict(tok_s=1.0 / per_token, layers_s=t_layers, head_s=t_head)
         log("[cpu] %d thread(s): %d layers %.2f s, lm_head %.2f s -> %.4f tok/s (extrapolated)"
             % (threads, layers_sampled, t_layers, t_head, 1.0 / per_token))
-        if threads == 1:
-            oracle_rows = [ctx.read_kv16(l, position) for l in range(layers_sampled)]
         ctx.close()
-    # Full-size parity, checker only: the device now runs the same token at the same position, and the
-    # K/V rows it appends for the sampled layers are compared with the oracle's. Layer 0's row covers
-    # embedding, RMSNorm, the 6144x4096 qkv GEMV, QK-norm and RoPE; layer 1's row depends on layer 0's
-    # attention over the whole context, its o projection and its MLP, all at the workload's real sizes.
-    rc, _, _ = session.advance(1)
-    assert rc == 0
-    rel = lambda a, b: float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
-    parity = {}
-    for l, (rk, rv) in enumerate(oracle_rows):
-        gk, gv = session.kv_row(l, position)
-        parity["layer%d_k" % l] = rel(O.decode16(dt, gk), O.decode16(dt, rk))
-        parity["layer%d_v" % l] = rel(O.decode16(dt, gv), O.decode16(dt, rv))
-    log("[cpu] device vs oracle K/V rows of the next token at position %d (relative L2): %s"
-        % (position, ", ".join("%s %.2e" % kv_ for kv_ in sorted(parity.items()))))
-    result["parity"] = parity
+    # Full-size parity, checker only: the traced step at the workload's real sizes and context. Layers
+    # 0..layers_sampled-1 (norms, 6144x4096 qkv, attention over the whole context, o, gate/up, down) and
+    # the head (final norm, 151936x4096 logits, greedy token) link by link on the device's own inputs.
+    rc, _, out, trace = session.traced_advance()
+    assert rc == 0 and trace is not None
+    k_rows, v_rows = [], []
+    for l, (k, v) in enumerate(kv):
+        rk, rv = session.kv_row(l, position)
+        k_rows.append(np.vstack([k, rk[None]]))
+        v_rows.append(np.vstack([v, rv[None]]))
+    try:
+        links = check_step_links(model, trace, position, token, int(out[0]), k_rows, v_rows, threads=threads_all)
+        result["parity_ok"] = True
+    except AssertionError as e:
+        links = {"failed": str(e)}
+        result["parity_ok"] = False
+    log("[cpu] device kernels vs oracle operators on the device's own inputs at position %d: %s"
+        % (position, ", ".join("%s %.1e" % kv_ for kv_ in sorted(links.items()) if not isinstance(kv_[1], str)) or links))
+    result["links"] = links
     return result
 
 
@@ -198,13 +176,8 @@ def main():
     assert rc == 0
     per_kind = {}
     chain = bool(prof.chain_enabled)
-    front = int(prof.front_mode)   # 1: qkv + attention + o in one launch, 2: attention + o, 0: one launch per piece
     if chain:
         kinds = ("qkv", "attention", "chain", "lm_head")
-    elif front == 1:
-        kinds = ("front", "gate_up", "down", "lm_head")
-    elif front == 2:
-        kinds = ("qkv", "front", "gate_up", "down", "lm_head")
     else:
         kinds = ("qkv", "attention", "o", "gate_up", "down", "lm_head")
     for k in kinds:
@@ -288,8 +261,10 @@ def main():
                        sample="1 decode token at ctx %d: %d of %d layers + lm_head timed on the oracle, extrapolated to %d layers"
                               % (position, layers_sampled, cfg["layers"], cfg["layers"]),
                        all_cores_value=round(r[threads_all]["tok_s"], 5), all_cores=threads_all,
-                       parity_rel_l2={k: float("%.3g" % v) for k, v in r["parity"].items()},
-                       parity_ok=all(v <= (2e-3 if k.startswith("layer0") else 2e-2) for k, v in r["parity"].items()))
+                       parity="traced step at ctx %d: every kernel of layers 0..%d and the head against the oracle operator on "
+                              "the device's own input, 1e-3 on the value before any 16-bit rounding" % (position, layers_sampled - 1),
+                       parity_links={k: (v if isinstance(v, str) else float("%.3g" % v)) for k, v in r["links"].items()},
+                       parity_ok=r["parity_ok"])
         except Exception as e:  # the CPU leg never hides the GPU result
             log("[cpu] baseline failed: %r" % (e,))
     session.destroy()

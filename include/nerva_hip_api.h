@@ -502,6 +502,7 @@ typedef struct NervaHipPagedAttentionRequest {
   void *workspace;              /* nerva_hip_paged_attention_workspace_bytes() bytes, zero-initialised once */
   float *output_f32;            /* optional [heads*hd] */
   uint16_t *output16;           /* [heads*hd] rounded */
+  uint32_t splits;              /* 0: the library's split-KV factor; 1..64 (and <= block_count): this one (tests) */
 } NervaHipPagedAttentionRequest;
 
 /* Fused per-head RMSNorm + RoPE + KV append + paged GQA split-KV decode attention
@@ -617,7 +618,9 @@ typedef struct NervaHipMoeFp8Request {
 
 /* out = sum_k w_k * Wd_e(swiglu(Wg_e x, Wu_e x)) + shared(x) with FP8 block-scaled
  * expert weights (reference/moe.rs:76-166, precision/block/moe.rs:744-859;
- * kernels_sparse_moe.inc.cu:323-397,787-946). */
+ * kernels_sparse_moe.inc.cu:323-397,787-946). The expert ids are device data, so the host cannot
+ * refuse them: an id >= num_experts makes every output element NaN (no memory outside the bank is
+ * read), never a plausible result from another expert. */
 int nerva_hip_moe_fp8_experts(const NervaHipMoeFp8Request *request, void *stream, int32_t *hip_error);
 
 typedef struct NervaHipMoeRouteRequest {
@@ -695,10 +698,6 @@ typedef struct NervaHipStepProfile {
    * layer's stand-alone launch only */
   uint64_t chain_ns, chain_stream_ns, chain_bytes;
   uint32_t chain_enabled;
-  /* fused layer front (qkv + attention + o projection as roles of one launch). front_mode 1: all
-   * three (the qkv/attention/o figures above are zero), 2: attention + o only, 0: off */
-  uint32_t front_mode;
-  uint64_t front_ns, front_stream_ns, front_bytes;
 } NervaHipStepProfile;
 
 /* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT
@@ -709,20 +708,21 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
                                    NervaHipStepProfile *out);
 
 /* Kernels of a session that hand data between workgroups inside one launch. *mode says which
- * the session's shapes and switches selected: the fused layer front (qkv + attention + o
- * projection as roles of one launch, the default where the shapes fit), the same without the
- * qkv role (NERVA_HIP_FRONT=2), the persistent layer-chain kernel (NERVA_HIP_CHAIN=1), or none
- * (NERVA_HIP_FRONT=0 / shapes that do not fit). *aborted = 1 when one of their bounded in-kernel
+ * the session's shapes and switches selected: the persistent layer-chain kernel
+ * (NERVA_HIP_CHAIN=1 where the shapes fit), or none. *aborted = 1 when one of its bounded in-kernel
  * waits ran out (the calls that covered those steps returned -1 with hip_error =
  * hipErrorLaunchFailure; start() clears it). raise_abort != 0 sets the abort word from the host
  * first, which makes every such wait give up at once: the failure path can be exercised while
  * all kernels still terminate normally. */
 #define NERVA_HIP_FUSED_NONE 0u
 #define NERVA_HIP_FUSED_CHAIN 1u
-#define NERVA_HIP_FUSED_FRONT 2u
-#define NERVA_HIP_FUSED_FRONT_ATTN_O 3u
 int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *session, uint32_t raise_abort,
                                   uint32_t *mode, uint32_t *aborted);
+
+/* 1 when this process launches its steps kernel by kernel instead of replaying captured graphs:
+ * NERVA_HIP_EAGER_STEPS=1, or the ROCm profiler's environment was found at the first call (a traced
+ * process must not reach hipGraphLaunch on this stack). Decided once per process. */
+int nerva_hip_steps_are_eager(void);
 
 /* Reads back the f32 logits of the last sampled position (vocab_size floats) and
  * one KV row (kv_heads*head_dim 16-bit values each for K and V) for parity tests. */
@@ -731,6 +731,20 @@ int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *session, uint
  * of 2048), 0 when every sequence of such a step runs its own decode step; -1 for a null session. */
 int nerva_hip_session_shares_weight_stream(NervaHipHfDecodeSequenceSession *session);
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *session, float *host_logits);
+/* Test hook (no counterpart): arms a trace of the NEXT decode step the session launches (through
+ * advance): that one step runs kernel by kernel instead of as a graph replay, and after each kernel
+ * its output vector is copied into `device_buffer`, one 256-byte-aligned slot behind the other, in
+ * this order: x after the embedding [hidden f32]; per layer the attention RMSNorm's output as the qkv
+ * rows are multiplied with it [hidden 16-bit], qkv [(heads + 2 kv_heads) * head_dim f32], attention
+ * output [heads * head_dim 16-bit], r after the o projection [hidden f32], the MLP RMSNorm's output
+ * [hidden 16-bit], SwiGLU output [intermediate 16-bit], x after the down projection [hidden f32]; then
+ * the final RMSNorm's output [hidden 16-bit] and the logits [vocab f32].
+ * The step is otherwise the ordinary one (same kernels, same launch shapes, token slot, cursor).
+ * Greedy sessions on the launch-per-piece step only; -1 otherwise or when the buffer is smaller than
+ * nerva_hip_session_step_trace_bytes(). A NULL buffer disarms a trace that has not run yet. */
+uint64_t nerva_hip_session_step_trace_bytes(NervaHipHfDecodeSequenceSession *session);
+int nerva_hip_session_trace_next_step(NervaHipHfDecodeSequenceSession *session, void *device_buffer,
+                                      uint64_t bytes);
 int nerva_hip_session_read_kv(NervaHipHfDecodeSequenceSession *session, uint32_t layer, uint32_t token,
                               uint16_t *host_k, uint16_t *host_v);
 /* Same for tokens [first_token, first_token + token_count): host_k / host_v receive

@@ -1,8 +1,7 @@
 // Device-side building blocks of the matrix-core decode attention (head_dim 128): head
 // preparation (bias, per-head RMSNorm, RoPE), operand helpers, coherent accesses for data
 // exchanged between workgroups of one launch, and the 16-token tile step. Shared by the
-// stand-alone attention kernel (attn_decode.hip) and the fused layer-front kernel
-// (layer_front.hip).
+// decode attention kernel (attn_decode.hip) and the prompt-block kernel (attn_prompt.hip).
 #pragma once
 
 #include "attn_decode.cuh"

@@ -19,6 +19,7 @@
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <string>
@@ -29,7 +30,6 @@
 #include "attn_decode.cuh"
 #include "decode_chain.cuh"
 #include "gemm_rows.cuh"
-#include "layer_front.cuh"
 #include "sampler.cuh"
 #include "gemv_stream.cuh"
 #include "runtime_state.hpp"
@@ -47,7 +47,7 @@ struct LayerDev {
 };
 
 enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
-enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLFront, kLKinds };
+enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLKinds };
 
 // The weight arena of a session and of every session forked from it (one stream of the weights can
 // then serve a token row of each of them); freed by the last of them to go.
@@ -121,12 +121,7 @@ struct NervaHipHfDecodeSequenceSession {
   bool chain = false;
   uint32_t *chain_flags = nullptr, *chain_abort = nullptr;
   uint64_t *chain_trace = nullptr;  // NERVA_HIP_CHAIN_TRACE=1: per-layer timestamps of workgroup 0
-  // fused layer front (qkv + attention + o in one launch): 0 off, 1 all three roles,
-  // 2 attention + o only (the qkv projection stays a launch of its own)
-  int front = 0;
-  uint32_t front_splits = 1;
-  void *front_ws = nullptr;  // tagged hand-over buffers of the fused front
-  uint64_t *front_trace = nullptr;  // NERVA_HIP_FRONT_TRACE=1: per-layer timestamps of selected workgroups
+  uint64_t *attn_trace = nullptr;  // NERVA_HIP_ATTN_TRACE=1: per-layer stage timestamps of selected attention workgroups
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
   uint32_t *host_state = nullptr;
@@ -153,6 +148,10 @@ struct NervaHipHfDecodeSequenceSession {
   SamplerDev *sampler_dev = nullptr;
   uint64_t *sampler_keys = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  // test hook: the next decode step is launched kernel by kernel and every intermediate vector is
+  // copied behind the previous one into this caller-owned device buffer (step_trace_bytes)
+  char *trace_buf = nullptr;
+  uint64_t trace_used = 0;
   // echo of the caller's weight plan
   uint32_t planned_weight_blocks = 0, planned_gpu_resident_blocks = 0, planned_gpu_staged_blocks = 0,
            planned_weight_descriptor_count = 0;
@@ -309,6 +308,20 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   hipStream_t st = s->stream;
   const uint32_t A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim;
   hipError_t err = hipSuccess;
+  // armed trace: copy an intermediate vector behind the ones already recorded (256-byte slots)
+  const bool tracing = s->trace_buf != nullptr && mode == kDecodeStep && only < 0 && prof == nullptr;
+  auto snap = [&](const void *src, uint64_t bytes) {
+    if (!tracing || err != hipSuccess) return;
+    err = hipMemcpyAsync(s->trace_buf + s->trace_used, src, bytes, hipMemcpyDeviceToDevice, st);
+    s->trace_used += (bytes + 255u) & ~uint64_t{255};
+  };
+  // the next trace slot as a destination a kernel writes itself (the RMSNorm prologue's 16-bit vector)
+  auto snap_slot = [&](uint64_t bytes) -> uint16_t * {
+    if (!tracing) return nullptr;
+    uint16_t *at = reinterpret_cast<uint16_t *>(s->trace_buf + s->trace_used);
+    s->trace_used += (bytes + 255u) & ~uint64_t{255};
+    return at;
+  };
 #define NV_STEP(kind, expr)                         \
   do {                                              \
     if (only >= 0 && only != (kind)) break;         \
@@ -334,11 +347,11 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
     err = hipGetLastError();
     if (prof && err == hipSuccess) err = prof->after();
     if (err != hipSuccess) return err;
+    snap(s->x, static_cast<uint64_t>(s->hidden) * sizeof(float));
   }
   for (uint32_t l = 0; l < s->layers; ++l) {
     const LayerDev &w = s->layer[l];
-    if (s->front != 0 ? s->front == 2 : (!s->chain || l == 0))
-    {
+    if (!s->chain || l == 0) {
       GemvParams p{};
       p.w = w.wqkv;
       p.xf = s->x;
@@ -349,7 +362,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.eps = s->eps;
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
+      p.x16_dump = snap_slot(static_cast<uint64_t>(s->hidden) * sizeof(uint16_t));
       NV_STEP(kLQkv, launch_gemv(s->dtype, kProRmsNorm, kEpiF32, p, st));
+      snap(s->qkv, static_cast<uint64_t>(A + 2 * KV) * sizeof(float));
     }
     {
       AttnParams p{};
@@ -377,30 +392,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
       p.append = 1;
-      p.trace = s->front == 0 && s->front_trace != nullptr ? s->front_trace + 32 * l : nullptr;
-      if (s->front != 0) {
-        // qkv rows, attention splits and o rows as roles of one launch
-        FrontParams f{};
-        p.splits = s->front_splits;
-        f.attn = p;
-        f.wqkv = s->front == 1 ? w.wqkv : nullptr;
-        f.rms_attn = w.rms_attn;
-        f.x = s->x;
-        f.wo = w.wo;
-        f.o_bias = w.o_bias;
-        f.r = s->r;
-        f.hidden = s->hidden;
-        f.rms_eps = s->eps;
-        front_bind_workspace(f, s->front_ws);
-        f.abort_flag = s->chain_abort;
-        f.step_counter = s->state + 2;
-        f.layer = l;
-        f.layers = s->layers;
-        f.trace = s->front_trace != nullptr ? s->front_trace + 32 * l : nullptr;
-        NV_STEP(kLFront, launch_layer_front(s->dtype, f, st));
-      } else {
-        NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
-      }
+      p.trace = s->attn_trace != nullptr ? s->attn_trace + 32 * l : nullptr;
+      NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
+      snap(s->attn16, static_cast<uint64_t>(A) * sizeof(uint16_t));
     }
     if (s->chain) {
       // o projection, gate/up, down and the next layer's qkv projection as one persistent launch
@@ -433,7 +427,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       NV_STEP(kLChain, launch_decode_chain(s->dtype, c, st));
       continue;
     }
-    if (s->front == 0) {
+    {
       GemvParams p{};
       p.w = w.wo;
       p.x16 = s->attn16;
@@ -445,6 +439,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
       NV_STEP(kLO, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
+      snap(s->r, static_cast<uint64_t>(s->hidden) * sizeof(float));
     }
     {
       GemvParams p{};
@@ -457,7 +452,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.eps = s->eps;
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
+      p.x16_dump = snap_slot(static_cast<uint64_t>(s->hidden) * sizeof(uint16_t));
       NV_STEP(kLGateUp, launch_gemv(s->dtype, kProRmsNorm, kEpiSwiglu, p, st));
+      snap(s->ff16, static_cast<uint64_t>(s->intermediate) * sizeof(uint16_t));
     }
     {
       GemvParams p{};
@@ -472,6 +469,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
       NV_STEP(kLDown, launch_gemv(s->dtype, kProX16, kEpiResidual, p, st));
+      snap(s->x, static_cast<uint64_t>(s->hidden) * sizeof(float));
     }
     }
   if (only >= 0) return hipSuccess;
@@ -496,11 +494,13 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   sample_bind_workspace(p.sample, s->sample_ws);
   p.sample.slots = s->slots;
   p.sample.cursor_rw = s->state;
-  NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st));
+  p.x16_dump = snap_slot(static_cast<uint64_t>(s->hidden) * sizeof(uint16_t));
+  uint32_t head_blocks = 0;  // workgroups of the LM-head launch = candidates it leaves
+  NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st, nullptr, &head_blocks));
+  snap(s->logits, static_cast<uint64_t>(s->vocab) * sizeof(float));
   if (s->sampler.mode == kSamplerGreedy) {
     // one small workgroup reduces the per-workgroup candidates, writes slot[pos], bumps the cursor
-    NV_STEP(kLAdvance, launch_sample_finish(p.sample, gemv_sample_blocks(p.rows, p.cols), s->state,
-                                            s->max_ctx, st));
+    NV_STEP(kLAdvance, launch_sample_finish(p.sample, head_blocks, s->state, s->max_ctx, st));
   } else {
     // temperature sampling from the logits (two launches), then slot[pos] and the cursor as above
     SamplerParams sp{};
@@ -517,14 +517,28 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   return hipSuccess;
 }
 
-// NERVA_HIP_EAGER_STEPS=1 launches every step kernel by kernel instead of replaying the
-// captured graph. It exists for kernel tracing only: replaying a hipGraph under
-// `rocprofv3 --kernel-trace` crashes inside the runtime on this stack. Results and
-// per-kernel durations are the same; the graph counters then report zero replays.
+// Steps are launched kernel by kernel instead of as graph replays when NERVA_HIP_EAGER_STEPS=1 is
+// set, or when the process runs under the ROCm profiler: with ROCm 7.2 a process traced by
+// rocprofv3 --kernel-trace died inside the HIP runtime at its first hipGraphLaunch (no message of its
+// own; the tool reported the abort), so a traced process must never reach that call. The profiler is
+// recognised by what it puts into the environment of the process it starts (its tool library in
+// LD_PRELOAD / ROCP_TOOL_LIBRARIES, ROCPROF_* settings). Results and per-kernel durations are the
+// same; the graph counters then report zero replays.
+bool profiler_in_environment() {
+  for (char **e = ::environ; e != nullptr && *e != nullptr; ++e) {
+    const char *v = *e;
+    if (strncmp(v, "ROCPROF", 7) == 0 || strncmp(v, "ROCP_TOOL_LIBRARIES=", 20) == 0 ||
+        strncmp(v, "ROCPROFILER_", 12) == 0)
+      return true;
+    if (strncmp(v, "LD_PRELOAD=", 11) == 0 && (strstr(v, "rocprofiler") != nullptr || strstr(v, "rocprof") != nullptr))
+      return true;
+  }
+  return false;
+}
 bool eager_steps() {
   static const bool eager = [] {
     const char *v = getenv("NERVA_HIP_EAGER_STEPS");
-    return v != nullptr && v[0] == '1';
+    return (v != nullptr && v[0] == '1') || profiler_in_environment();
   }();
   return eager;
 }
@@ -534,8 +548,6 @@ uint64_t step_launches(const Session *s, int which) {
   // embed + (lm head + greedy finish | lm head + two sampler launches | cursor advance)
   const uint64_t fixed = which == 1 ? 2 : (s->sampler.mode == kSamplerGreedy ? 3 : 4);
   if (s->chain) return fixed + 1 + 2ull * s->layers;
-  if (s->front == 1) return fixed + 3ull * s->layers;
-  if (s->front == 2) return fixed + 4ull * s->layers;
   return fixed + 5ull * s->layers;
 }
 
@@ -580,6 +592,14 @@ hipError_t ensure_graph(Session *s, int which, NervaHipHfDecodeSequenceResult *o
 }
 
 hipError_t launch_step(Session *s, int which, NervaHipHfDecodeSequenceResult *out) {
+  if (s->trace_buf != nullptr && which != 1) {
+    // armed by nerva_hip_session_trace_next_step: this one step runs kernel by kernel with copies
+    s->trace_used = 0;
+    hipError_t err = enqueue_step(s, kDecodeStep, nullptr);
+    s->trace_buf = nullptr;
+    if (err == hipSuccess) out->kernel_launches += step_launches(s, which);
+    return err;
+  }
   if (eager_steps()) {
     hipError_t err = enqueue_step(s, which == 1 ? kPromptStep : kDecodeStep, nullptr);
     if (err == hipSuccess)
@@ -656,7 +676,7 @@ bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
 // After a synchronisation: did a bounded wait of the chain kernel run out during the steps
 // just completed? Their tokens are then not to be trusted and the call fails.
 hipError_t chain_verdict(Session *s) {
-  if (!s->chain && s->front == 0) return hipSuccess;
+  if (!s->chain) return hipSuccess;
   uint32_t aborted = 0;
   const hipError_t err = hipMemcpy(&aborted, s->chain_abort, sizeof(aborted), hipMemcpyDeviceToHost);
   if (err != hipSuccess) return err;
@@ -1017,8 +1037,6 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(s->vocab));
   const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
   const uint64_t off_chain_trace = c.take(L * 32 * 8);
-  const uint64_t front_ws_bytes = front_workspace_bytes(s->heads, s->kv_heads);
-  const uint64_t off_front_ws = c.take(front_ws_bytes);
   {
     // Prompt blocks and batch steps need the matrix-core attention (head_dim 128, GQA factor
     // 1/2/4/8) and shapes the multi-row kernels take.
@@ -1112,27 +1130,10 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
     if (s->chain && trace != nullptr && trace[0] == '1')
       s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
   }
-  s->front_ws = s->arena + off_front_ws;
   {
-    // Fused layer front (layer_front.cuh), opt-in: NERVA_HIP_FRONT=2 runs attention + o
-    // projection as roles of one launch, =1 adds the qkv projection as a third role. Off by
-    // default: measured on MI355X every hand-over between workgroups through memory costs
-    // 1.2-1.8 us (device-coherent store, poll, dependent load), about what the kernel boundary
-    // it replaces costs, and the attention role runs under a tighter register budget; the step is
-    // 3-6 % slower than with one launch per piece.
-    const char *want = getenv("NERVA_HIP_FRONT");
-    int mode = 0;
-    if (want != nullptr && want[0] >= '0' && want[0] <= '2') mode = want[0] - '0';
-    if (s->chain || s->layers == 0 || !front_supported(s->hidden, s->heads, s->kv_heads, s->head_dim)) mode = 0;
-    s->front = mode;
-    // one KV tile in flight per wave there, so twice the stand-alone kernel's splits
-    uint32_t splits = (256 + s->kv_heads - 1) / s->kv_heads;
-    if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
-    if (splits > block_count) splits = block_count;
-    s->front_splits = splits == 0 ? 1 : splits;
-    const char *trace = getenv("NERVA_HIP_FRONT_TRACE");
+    const char *trace = getenv("NERVA_HIP_ATTN_TRACE");
     if (!s->chain && s->layers > 0 && trace != nullptr && trace[0] == '1')
-      s->front_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
+      s->attn_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
   }
 
   *failure_stage = 5;
@@ -1152,7 +1153,6 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_ws_bytes, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_front_ws, 0, front_ws_bytes, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
   if (err == hipSuccess && L > 0) err = hipMemsetAsync(s->arena + off_chain_trace, 0, L * 32 * 8, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
@@ -1846,6 +1846,12 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
         err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
                              q->stream);
       out->d2h_bytes += sizeof(Slot);
+      // A chain step keeps one workgroup resident on every CU and its workgroups wait for each other:
+      // two of them must never share the machine, so such sessions run one after the other.
+      if (err == hipSuccess && q->chain) {
+        err = hipStreamSynchronize(q->stream);
+        out->sync_calls += 1;
+      }
       out->pack_kernel_launches += 1;
       out->projection_kernel_launches += 4ull * q->layers + 1;
       out->dependency_kernel_launches += q->layers;
@@ -2015,7 +2021,7 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
   if (err == hipSuccess) {
     err = hipMemcpyAsync(s->host_slots + slot_start, s->slots + slot_start, slots_bytes,
                          hipMemcpyDeviceToHost, s->stream);
-    out->d2h_bytes = slots_bytes;
+    out->d2h_bytes += slots_bytes;
   }
   if (err == hipSuccess) {
     err = hipStreamSynchronize(s->stream);
@@ -2215,19 +2221,15 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // back-to-back pass: all `layers` launches of one kind between a single event pair, so the
   // figure is the kernel's own duration without the per-launch event gaps
   uint64_t stream_ns[kLKinds] = {0};
-  for (int kind = kLQkv; err == hipSuccess && kind <= kLFront; ++kind) {
+  for (int kind = kLQkv; err == hipSuccess && kind <= kLChain; ++kind) {
     uint32_t launches = s->layers;
     if (kind == kLHead || kind == kLAdvance) continue;
     if (kind == kLQkv && s->chain) launches = 1;
     if ((kind == kLO || kind == kLGateUp || kind == kLDown) && s->chain) continue;
     if (kind == kLChain && !s->chain) continue;
-    if (kind == kLFront && s->front == 0) continue;
-    if ((kind == kLAttn || kind == kLO) && s->front != 0) continue;
-    if (kind == kLQkv && s->front == 1) continue;
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
-      // no embed launch in this pass: advance the step counter here, so that the hand-over
-      // epochs of the fused front are fresh
+      // no embed launch in this pass: advance the step counter here
       hipLaunchKernelGGL(bump_step_counter_kernel, dim3(1), dim3(64), 0, s->stream, s->state);
       err = hipGetLastError();
       if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
@@ -2256,18 +2258,18 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
       }
     }
   }
-  if (s->front_trace != nullptr) {
+  if (s->attn_trace != nullptr) {
     // timestamps (10 ns ticks from the launch's earliest mark) of: qkv workgroup 0 [0..3] and the last
     // one's end [4]; attention (kv head 0, split 0) [8..13]; the merging workgroup of kv head 0 [16..18];
     // first [20..23] and last [24..27] o workgroup
     std::vector<uint64_t> tr(static_cast<size_t>(s->layers) * 32);
-    if (hipMemcpy(tr.data(), s->front_trace, tr.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+    if (hipMemcpy(tr.data(), s->attn_trace, tr.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
       for (uint32_t l = 0; l < s->layers && l < 4; ++l) {
         const uint64_t *t = tr.data() + 32 * l;
         uint64_t first = ~uint64_t{0};
         for (int i = 0; i < 28; ++i)
           if (t[i] > 1000000 && t[i] < first) first = t[i];
-        fprintf(stderr, "[front trace] layer %u:", l);
+        fprintf(stderr, "[attention trace] layer %u:", l);
         for (int i = 0; i < 28; ++i) {
           if (i == 8 || i == 16 || i == 20 || i == 24) fprintf(stderr, " |");
           if (t[i] > 1000000) fprintf(stderr, " %lld", static_cast<long long>(t[i] - first));
@@ -2292,9 +2294,6 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_stream_ns = stream_ns[kLGateUp];
   out->down_stream_ns = stream_ns[kLDown];
   out->chain_stream_ns = stream_ns[kLChain];
-  out->front_stream_ns = stream_ns[kLFront];
-  out->front_ns = counts[kLFront] ? sums[kLFront] / counts[kLFront] : 0;
-  out->front_mode = static_cast<uint32_t>(s->front);
   auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
   out->position = pos;
   out->embed_ns = avg(kLEmbed);
@@ -2319,8 +2318,6 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // stay on the device and are counted once, as the phase that reads them)
   out->chain_bytes = s->chain ? out->o_bytes + out->gate_up_bytes + out->down_bytes + out->qkv_bytes : 0;
   out->chain_enabled = s->chain ? 1u : 0u;
-  // fused front: the pieces it replaces (their hand-over vectors stay on the device)
-  out->front_bytes = s->front == 0 ? 0 : out->attention_bytes + out->o_bytes + (s->front == 1 ? out->qkv_bytes : 0);
   out->status = 0;
   return 0;
 }
@@ -2329,14 +2326,14 @@ int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *s, uint32_t r
                                   uint32_t *aborted) {
   if (s == nullptr) return -1;
   if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
-  const bool fused = s->chain || s->front != 0;
+  const bool fused = s->chain;
   if (raise_abort != 0 && fused) {
     const uint32_t one = 1;
     if (hipMemcpy(s->chain_abort, &one, sizeof(one), hipMemcpyHostToDevice) != hipSuccess) return -1;
   }
   uint32_t flag = 0;
   if (fused && hipMemcpy(&flag, s->chain_abort, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  if (mode) *mode = s->chain ? NERVA_HIP_FUSED_CHAIN : (s->front == 1 ? NERVA_HIP_FUSED_FRONT : (s->front == 2 ? NERVA_HIP_FUSED_FRONT_ATTN_O : NERVA_HIP_FUSED_NONE));
+  if (mode) *mode = s->chain ? NERVA_HIP_FUSED_CHAIN : NERVA_HIP_FUSED_NONE;
   if (aborted) *aborted = flag;
   return 0;
 }
@@ -2344,6 +2341,30 @@ int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *s, uint32_t r
 int nerva_hip_session_shares_weight_stream(NervaHipHfDecodeSequenceSession *s) {
   if (s == nullptr) return -1;
   return s->rows_ready && s->blogits != nullptr ? 1 : 0;
+}
+
+int nerva_hip_steps_are_eager(void) { return eager_steps() ? 1 : 0; }
+
+uint64_t nerva_hip_session_step_trace_bytes(NervaHipHfDecodeSequenceSession *s) {
+  if (s == nullptr) return 0;
+  auto slot = [](uint64_t bytes) { return (bytes + 255u) & ~uint64_t{255}; };
+  const uint64_t A = static_cast<uint64_t>(s->heads) * s->head_dim, KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim;
+  const uint64_t per_layer = slot(s->hidden * 2ull) + slot((A + 2 * KV) * 4) + slot(A * 2) + slot(s->hidden * 4ull) +
+                             slot(s->hidden * 2ull) + slot(s->intermediate * 2ull) + slot(s->hidden * 4ull);
+  return slot(s->hidden * 4ull) + per_layer * s->layers + slot(s->hidden * 2ull) + slot(s->vocab * 4ull);
+}
+
+int nerva_hip_session_trace_next_step(NervaHipHfDecodeSequenceSession *s, void *device_buffer, uint64_t bytes) {
+  if (s == nullptr) return -1;
+  if (device_buffer == nullptr) {  // disarm
+    s->trace_buf = nullptr;
+    return 0;
+  }
+  if (bytes < nerva_hip_session_step_trace_bytes(s)) return -1;
+  if (s->chain || s->sampler.mode != kSamplerGreedy) return -1;  // the launch-per-piece greedy step only
+  s->trace_buf = static_cast<char *>(device_buffer);
+  s->trace_used = 0;
+  return 0;
 }
 
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *s, float *host_logits) {

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void moe_gate_up_kernel(MoeFp8Params p) {
        unit += gridDim.x * kWavesPerBlock) {
     const uint32_t k = unit / p.inter, i = unit % p.inter;
     uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);
-    if (e >= p.num_experts) e = 0;  // ids are validated on the host when they are host-visible
+    if (e >= p.num_experts) e = 0;  // stay in bounds; the down kernel turns such a slot into NaN outputs
     const uint8_t *wrow[2] = {p.w_gate + e * w_stride + static_cast<uint64_t>(i) * p.hidden,
                               p.w_up + e * w_stride + static_cast<uint64_t>(i) * p.hidden};
     const float *srow[2] = {p.s_gate + e * scale_stride + static_cast<uint64_t>(i / p.block) * sc,
@@ -258,8 +258,11 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
       buf[FAST ? lean_slot_f32(c) : c] = p.act[static_cast<uint64_t>(k) * p.inter + c];
     __syncthreads();  // double buffer: the previous expert's readers are at most one step behind
     uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);
-    if (e >= p.num_experts) e = 0;
-    const float weight = k < p.top_k ? p.expert_weights[k] : 1.0f;
+    float weight = k < p.top_k ? p.expert_weights[k] : 1.0f;
+    if (e >= p.num_experts) {  // an id outside the bank: read expert 0 (in bounds), poison the result
+      e = 0;
+      weight = __builtin_nanf("");
+    }
     const uint8_t *wrow[NR];
     const float *srow[NR];
     float acc[NR];
@@ -405,9 +408,13 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   constexpr uint32_t inter = P * 1024u;
   if (threadIdx.x < slots) {
     uint32_t e = threadIdx.x < p.top_k ? p.expert_ids[threadIdx.x] : static_cast<uint32_t>(p.shared_index);
-    if (e >= p.num_experts) e = 0;
+    float weight = threadIdx.x < p.top_k ? p.expert_weights[threadIdx.x] : 1.0f;
+    if (e >= p.num_experts) {  // an id outside the bank: read expert 0 (in bounds), poison the result
+      e = 0;
+      weight = __builtin_nanf("");
+    }
     sh_expert[threadIdx.x] = e;
-    sh_weight[threadIdx.x] = threadIdx.x < p.top_k ? p.expert_weights[threadIdx.x] : 1.0f;
+    sh_weight[threadIdx.x] = weight;
   }
   const int consumers = static_cast<int>(blockDim.x) / kWave - 1;  // the last wave stages
   if (wave == consumers) {

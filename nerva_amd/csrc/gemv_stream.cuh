@@ -79,6 +79,9 @@ struct GemvParams {
   const uint32_t *cursor;  // optional step guard: skip when *cursor >= max_steps
   uint32_t max_steps;
   SampleParams sample;
+  // test hook of the RMSNorm prologue: when set, workgroup 0 also writes the 16-bit vector the rows
+  // are multiplied with (the prologue's output, which otherwise exists in LDS only) to [cols]
+  uint16_t *x16_dump;
 };
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -243,6 +246,10 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
     }
   }
   __syncthreads();
+  if constexpr (PRO == kProRmsNorm) {
+    if (p.x16_dump != nullptr && blockIdx.x == 0)
+      for (uint32_t c = threadIdx.x; c < cols; c += kBlock) p.x16_dump[c] = xs[c];
+  }
 
   // ---- main loop: each wave owns NR rows per iteration -------------------
   Best best{0.0f, 0u, 0u};
@@ -516,6 +523,10 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
     }
   }
   __syncthreads();
+  if constexpr (PRO == kProRmsNorm) {
+    if (p.x16_dump != nullptr && blockIdx.x == 0)
+      for (uint32_t c = threadIdx.x; c < cols; c += kBlock) p.x16_dump[c] = xs[c];
+  }
 
   // ---- 5. main loop
   Best best{0.0f, 0u, 0u};
@@ -603,8 +614,10 @@ struct GemvTuning {
   bool force_generic = false;  // never take the lean production-shape kernel
 };
 
+// `blocks_used`, when given, receives the number of workgroups launched: an LM-head launch leaves
+// exactly that many sampler candidates, so the finishing launch takes its count from here.
 hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvParams &p,
-                       hipStream_t stream, const GemvTuning *tuning = nullptr);
+                       hipStream_t stream, const GemvTuning *tuning = nullptr, uint32_t *blocks_used = nullptr);
 // Kernel variant and grid of a launch (shared by the launcher and by callers that size
 // per-workgroup outputs). `vec16` = every pointer is 16-byte aligned.
 struct GemvPlan {
@@ -614,8 +627,6 @@ struct GemvPlan {
 constexpr int kFast = 3;  // the lean production-shape kernel
 GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,
                    const struct GemvTuning *tuning);
-// Number of workgroups (= sampler candidates) an LM-head launch over [rows x cols] uses.
-uint32_t gemv_sample_blocks(uint32_t rows, uint32_t cols);
 // Reduce `count` per-workgroup candidates and publish the token (one workgroup).
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,
                                 uint32_t max_steps, hipStream_t stream);

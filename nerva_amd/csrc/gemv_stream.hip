@@ -130,7 +130,8 @@ GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, boo
 }
 
 hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvParams &p,
-                       hipStream_t stream, const GemvTuning *tuning) {
+                       hipStream_t stream, const GemvTuning *tuning, uint32_t *blocks_used) {
+  if (blocks_used) *blocks_used = 0;
   if (p.w == nullptr || p.rows == 0 || p.cols == 0) return hipErrorInvalidValue;
   if (prologue == kProX16 && p.x16 == nullptr) return hipErrorInvalidValue;
   if (prologue == kProRmsNorm && (p.xf == nullptr || p.gamma == nullptr)) return hipErrorInvalidValue;
@@ -150,6 +151,7 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
   const GemvPlan plan = gemv_plan(prologue, epilogue, p.rows, p.cols, vec16, tuning);
   const int mode = plan.mode;
   const uint32_t blocks = plan.blocks;
+  if (blocks_used) *blocks_used = blocks;
   if (dtype == kBF16) {
     if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, blocks, lds, stream);
     if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
@@ -160,11 +162,6 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
   if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
   if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream);
   return launch_pro<kF16, kScalar>(prologue, epilogue, p, blocks, lds, stream);
-}
-
-uint32_t gemv_sample_blocks(uint32_t rows, uint32_t cols) {
-  // session buffers come from a 256-byte-granular arena, so the aligned plan is the one launched
-  return gemv_plan(kProRmsNorm, kEpiArgmax, rows, cols, true, nullptr).blocks;
 }
 
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,

@@ -203,8 +203,9 @@ class PagedKvCache:
 
 def paged_attention(dtype, heads, kv_heads, head_dim, cache, layer, position, qkv_f32, workspace, out16,
                     *, out_f32=None, append=True, eps=1e-6, rope_theta=0.0, q_norm=None, k_norm=None,
-                    q_bias=None, k_bias=None, v_bias=None, sync=True):
+                    q_bias=None, k_bias=None, v_bias=None, sync=True, splits=0):
     req = abi.NervaHipPagedAttentionRequest()
+    req.splits = splits
     req.dtype, req.heads, req.kv_heads, req.head_dim = dtype, heads, kv_heads, head_dim
     req.layer, req.block_count, req.position, req.append = layer, cache.block_count, position, int(append)
     req.rms_eps, req.rope_theta = eps, rope_theta

@@ -278,16 +278,54 @@ class DecodeSession:
         rc = self.lib.nerva_hip_session_profile_step(self.handle, repeats, C.byref(res))
         return rc, res
 
-    FUSED_NONE, FUSED_CHAIN, FUSED_FRONT, FUSED_FRONT_ATTN_O = 0, 1, 2, 3
+    FUSED_NONE, FUSED_CHAIN = 0, 1
 
     def fused_state(self, raise_abort=False):
-        """(mode, aborted) of the kernels that hand data between workgroups inside a launch (fused layer
-        front / layer chain); raise_abort sets the abort word so that their bounded waits give up."""
+        """(mode, aborted) of the kernel that hands data between workgroups inside a launch (the layer
+        chain); raise_abort sets the abort word so that its bounded waits give up."""
         mode, aborted = C.c_uint32(0), C.c_uint32(0)
         rc = self.lib.nerva_hip_session_fused_state(self.handle, int(raise_abort), C.byref(mode), C.byref(aborted))
         if rc != 0:
             raise RuntimeError("fused_state failed")
         return int(mode.value), bool(aborted.value)
+
+    def traced_advance(self):
+        """advance(1) with the step's intermediates read back (nerva_hip_session_trace_next_step).
+
+        Returns (rc, result, tokens, trace); trace = {"x0": f32[hidden], "layers": [{"a16", "qkv", "attn16",
+        "r", "m16", "ff16", "x"}...], "h16", "logits": f32[vocab]} - the output vector of every kernel of
+        that step, and the 16-bit outputs of the RMSNorm prologues (a16, m16, h16),
+        or None when the call launched no step (the first advance hands out the token start() made)."""
+        from .runtime import DeviceBuffer
+        cr = self.create_result
+        nbytes = int(self.lib.nerva_hip_session_step_trace_bytes(self.handle))
+        buf = DeviceBuffer.zeros(nbytes)
+        if self.lib.nerva_hip_session_trace_next_step(self.handle, buf.ptr, nbytes) != 0:
+            raise RuntimeError("trace_next_step refused")
+        rc, res, tokens = self.advance(1)
+        if rc != 0 or res.kernel_launches == 0:
+            self.lib.nerva_hip_session_trace_next_step(self.handle, None, 0)  # disarm
+            return rc, res, tokens, None
+        raw = buf.numpy(np.uint8)
+        at = [0]
+
+        def take(count, dtype):
+            n = count * np.dtype(dtype).itemsize
+            a = raw[at[0]:at[0] + n].view(dtype).copy()
+            at[0] += (n + 255) & ~255
+            return a
+
+        A, KV = cr.heads * cr.head_dim, cr.kv_heads * cr.head_dim
+        trace = {"x0": take(cr.hidden, np.float32), "layers": []}
+        for _ in range(cr.layer_count):
+            trace["layers"].append({"a16": take(cr.hidden, np.uint16), "qkv": take(A + 2 * KV, np.float32),
+                                    "attn16": take(A, np.uint16), "r": take(cr.hidden, np.float32),
+                                    "m16": take(cr.hidden, np.uint16), "ff16": take(cr.intermediate, np.uint16),
+                                    "x": take(cr.hidden, np.float32)})
+        trace["h16"] = take(cr.hidden, np.uint16)
+        trace["logits"] = take(cr.vocab_size, np.float32)
+        assert at[0] == nbytes
+        return rc, res, tokens, trace
 
     def logits(self):
         out = np.empty(self.vocab, np.float32)

@@ -364,6 +364,47 @@ class Model:
                           _p(self.final_norm, u16p), _p(self.lm_head, u16p))
 
 
+def synthetic_model(cfg, seed, weight_std, layers=None, embedding_rows=None, threads=8):
+    """Host copy of the weights nerva_hip_bench_session_create_synthetic generates on the device
+    (same counter-based generator, same tensor ids), as a Model. `layers` keeps the first n layers;
+    `embedding_rows` keeps only those rows of the embedding table (the others stay zero)."""
+    import concurrent.futures
+    dt, H, HD = cfg["dtype"], cfg["hidden"], cfg["head_dim"]
+    A, KV, I, V = cfg["heads"] * HD, cfg["kv_heads"] * HD, cfg["intermediate"], cfg["vocab"]
+    layers = cfg["layers"] if layers is None else layers
+
+    def gen(tid, n, mean=0.0):
+        chunk = 1 << 24
+        out = np.empty(n, np.uint16)
+
+        def work(start):
+            m = min(chunk, n - start)
+            out[start:start + m] = synth_16(dt, seed, tid, m, mean, weight_std, offset=start)
+        if n <= chunk:
+            work(0)
+        else:
+            with concurrent.futures.ThreadPoolExecutor(max_workers=threads) as pool:
+                list(pool.map(work, range(0, n, chunk)))
+        return out
+
+    ls = []
+    for l in range(layers):
+        b = 16 * (l + 1)
+        ls.append(dict(rms_attn=gen(b, H, 1.0), rms_mlp=gen(b + 1, H, 1.0), w_q=gen(b + 2, A * H).reshape(A, H),
+                       w_k=gen(b + 4, KV * H).reshape(KV, H), q_norm=gen(b + 5, HD, 1.0), k_norm=gen(b + 6, HD, 1.0),
+                       w_v=gen(b + 7, KV * H).reshape(KV, H), w_o=gen(b + 8, H * A).reshape(H, A),
+                       w_gate=gen(b + 13, I * H).reshape(I, H), w_up=gen(b + 14, I * H).reshape(I, H),
+                       w_down=gen(b + 15, H * I).reshape(H, I)))
+    if embedding_rows is None:
+        emb = gen(1, V * H).reshape(V, H)
+    else:
+        emb = np.zeros((V, H), np.uint16)
+        for t in embedding_rows:
+            emb[t] = synth_16(dt, seed, 1, H, 0.0, weight_std, offset=int(t) * H)
+    return Model(dt, H, cfg["heads"], cfg["kv_heads"], HD, I, V, cfg["rms_eps"], cfg["rope_theta"], emb, ls,
+                 gen(2, H, 1.0), gen(3, V * H).reshape(V, H))
+
+
 class Context:
     def __init__(self, model, max_ctx, staging=1, threads=1):
         self.model = model

@@ -275,3 +275,19 @@ def test_operand_order_index_is_the_matrix_core_operand_layout(lib):
                 assert i == ((k // 32) * tiles + t // 16) * 512 + lane * 8 + k % 8
                 seen.add(i)
         assert seen == set(range(tiles * 16 * cols))
+
+
+def test_profiled_processes_never_replay_graphs():
+    """A process started by the ROCm profiler carries its tool library and settings in the
+    environment; such a process must launch its steps kernel by kernel (a traced hipGraphLaunch
+    took the process down on this stack). Decided at the first call, so each case is a process."""
+    import subprocess
+    import sys
+    code = "import nerva_amd.abi as a; print(a.load().nerva_hip_steps_are_eager())"
+    cases = [({}, "0"), ({"NERVA_HIP_EAGER_STEPS": "1"}, "1"), ({"ROCP_TOOL_LIBRARIES": ""}, "1"),
+             ({"ROCPROF_KERNEL_TRACE": "1"}, "1"), ({"ROCPROF_OUTPUT_PATH": "/tmp/x"}, "1")]
+    for extra, want in cases:
+        env = {k: v for k, v in os.environ.items() if not k.startswith(("ROCPROF", "ROCP_", "NERVA_HIP_"))}
+        env.update(extra)
+        out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True)
+        assert out.returncode == 0 and out.stdout.strip() == want, (extra, out.stdout, out.stderr)

@@ -423,6 +423,48 @@ def test_paged_attention_permutation_invariance_and_repeatability():
     assert np.array_equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("tokens", [17, 255, 4096, 8191])
+def test_paged_attention_split_merge_is_stable_over_many_launches(tokens):
+    """The cross-split merge (partials written by every split's workgroup, one ticket per workgroup,
+    the last arriver of a kv head merges in split order) must not depend on arrival order or timing:
+    for split factors 2, 8, 32 and 64, 200 launches in a row give the bits of the first launch, and
+    those are within tolerance of the oracle. Stops at the first mismatch."""
+    c = _attention_case(BF16, 32, 8, 128, tokens, 1e6, True, 5000 + tokens)
+    ref, _, _ = _attention_oracle(c)
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
+    cache.fill(c["layer"], c["k_rows"], c["v_rows"])
+    ws = attention_workspace(32, 128)
+    out16, out32 = N.DeviceBuffer(4096 * 2), N.DeviceBuffer(4096 * 4)
+    qkv, qn, kn = dev(c["qkv"]), dev(c["qn"]), dev(c["kn"])
+    outs = {}
+    for splits in (2, 8, 32, 64):
+        if splits > c["n_blocks"]:
+            continue
+        first = None
+        for launch in range(200):
+            N.paged_attention(BF16, 32, 8, 128, cache, c["layer"], tokens, qkv, ws, out16, out_f32=out32, append=True,
+                              rope_theta=1e6, q_norm=qn, k_norm=kn, splits=splits)
+            bits = out32.numpy(np.uint32)
+            if first is None:
+                first = bits
+                assert rel_l2(first.view(np.float32), ref) <= REL_L2, (tokens, splits)
+            assert np.array_equal(bits, first), "context %d, %d splits: launch %d differs from the first" % (tokens, splits, launch)
+        outs[splits] = first.view(np.float32)
+    # different split factors are different (each deterministic) summation orders of the same sums
+    for splits, out in outs.items():
+        assert rel_l2(out, outs[min(outs)]) <= 1e-5, splits
+
+
+def test_paged_attention_split_override_is_validated():
+    c = _attention_case(BF16, 32, 8, 128, 40, 1e6, True, 3)
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
+    ws = attention_workspace(32, 128)
+    out16 = N.DeviceBuffer(4096 * 2)
+    for bad in (65, c["n_blocks"] + 1):
+        with pytest.raises(RuntimeError):
+            N.paged_attention(BF16, 32, 8, 128, cache, 0, 40, dev(c["qkv"]), ws, out16, splits=bad)
+
+
 def test_paged_attention_no_append_reads_cache_only():
     c = _attention_case(BF16, 32, 8, 128, 200, 1e6, True, 9)
     cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
@@ -547,6 +589,47 @@ def test_moe_fp8_experts_match_oracle(hidden, inter, experts, top_k):
     N.moe_fp8_experts(hidden, inter, experts, top_k, B, dev(x16), dids, dwts, dev(wg), dev(sg), dev(wu),
                       dev(su), dev(wd), dev(sd), act, out, shared_index=-1)
     assert rel_l2(out.numpy(np.float32), ref2) <= REL_L2
+
+
+def test_moe_fp8_experts_in_a_256_expert_bank():
+    """Config 4's address space: 256 routed experts + the shared one (index 256), hidden 7168,
+    intermediate 2048. Only the experts the route selects hold data (ids 3, 131, 254, 255 among them:
+    expert stride x 255 is a 64-bit product), everything else in the 11 GB bank is never touched. The
+    oracle sees the same nine experts as a compact bank with the ids renumbered - the same sums in the
+    same order. An id outside the bank must poison the output, not pick another expert."""
+    hidden, inter, experts, top_k, B = 7168, 2048, 257, 8, 128
+    chosen = np.array([3, 131, 254, 255, 0, 77, 128, 200], np.uint32)
+    wts = np.random.default_rng(4).dirichlet(np.ones(top_k)).astype(np.float32)
+    bank = list(chosen) + [256]
+    wg = np.empty((len(bank), inter, hidden), np.uint8)
+    wu = np.empty_like(wg)
+    wd = np.empty((len(bank), hidden, inter), np.uint8)
+    sg = np.empty((len(bank), inter // B, hidden // B), np.float32)
+    su = np.empty_like(sg)
+    sd = np.empty((len(bank), hidden // B, inter // B), np.float32)
+    for j, e in enumerate(bank):
+        wg[j], sg[j] = O.synth_fp8_block(SEED, 3000 + int(e), inter, hidden, B, 0.02)
+        wu[j], su[j] = O.synth_fp8_block(SEED, 4000 + int(e), inter, hidden, B, 0.02)
+        wd[j], sd[j] = O.synth_fp8_block(SEED, 5000 + int(e), hidden, inter, B, 0.02)
+    x16 = O.synth_16(BF16, SEED, 12, hidden, 0.0, 1.0)
+    ref = O.moe_fp8_forward(hidden, inter, len(bank), B, x16, np.arange(top_k, dtype=np.uint32), wts, wg, sg, wu, su,
+                            wd, sd, shared_index=top_k)
+    dwg, dwu, dwd = (N.DeviceBuffer(experts * inter * hidden) for _ in range(3))
+    dsg, dsu, dsd = (N.DeviceBuffer(experts * (inter // B) * (hidden // B) * 4) for _ in range(3))
+    for j, e in enumerate(bank):
+        e = int(e)
+        for buf, arr in ((dwg, wg), (dwu, wu), (dwd, wd), (dsg, sg), (dsu, su), (dsd, sd)):
+            buf.upload(arr[j], offset=e * arr[j].nbytes)
+    act = N.DeviceBuffer((top_k + 1) * inter * 4)
+    out = N.DeviceBuffer(hidden * 4)
+    N.moe_fp8_experts(hidden, inter, experts, top_k, B, dev(x16), dev(chosen), dev(wts), dwg, dsg, dwu, dsu, dwd, dsd,
+                      act, out, shared_index=256)
+    assert rel_l2(out.numpy(np.float32), ref) <= REL_L2
+    bad = chosen.copy()
+    bad[2] = 257
+    N.moe_fp8_experts(hidden, inter, experts, top_k, B, dev(x16), dev(bad), dev(wts), dwg, dsg, dwu, dsu, dwd, dsd,
+                      act, out, shared_index=256)
+    assert np.all(np.isnan(out.numpy(np.float32)))
 
 
 @pytest.mark.parametrize("dtype", [BF16, F16])

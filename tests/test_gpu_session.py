@@ -11,6 +11,7 @@ import oracle as O
 from conftest import hx
 from nerva_amd import abi
 from nerva_amd.session import decode_sequence_oneshot
+from oracle.links import assert_stream_follows_oracle, chain_budget, run_traced_stream
 
 pytestmark = pytest.mark.gpu
 
@@ -295,23 +296,17 @@ def random_model(dtype, hidden, heads, kv_heads, hd, inter, vocab, layers, seed,
     return N.ModelWeights(*args), O.Model(*args)
 
 
-# End-to-end tolerance. Every operator is checked on its own at relative L2 <= 1e-3
-# (tests/test_gpu_ops.py). Through a whole model the 16-bit staging points amplify
-# f32 summation-order noise: one bf16 rounding that lands on the other side of a tie
-# moves that element by 2^-8 relative, and every later layer sees it. Measured on these
-# models: device vs oracle logits differ by 2e-3..6e-3 relative L2, the same size as the
-# reference's own two stagings differ from each other (oracle staging 0 vs 1: 3e-3..7e-3).
-E2E_REL_L2 = 2e-2
+# End-to-end numbers. Every operator is held to relative L2 <= 1e-3 on its own (tests/test_gpu_ops.py)
+# and inside a running session on the device's own inputs (tests/test_gpu_parity_links.py: measured
+# <= 1.1e-5 for every link). Through a whole model the 16-bit staging points amplify f32
+# summation-order noise: one bf16 rounding that lands on the other side of a boundary moves that
+# element by 2^-8 relative, and every later layer sees it. So the logits of a whole step are held to
+# the chain's budget - one operator tolerance per 16-bit staging point, oracle.links.chain_budget -
+# and the measured figure (2e-3..8e-3 on these models, the size by which the reference's own two
+# stagings differ from each other) is only reported.
 
 
-def assert_streams_agree(device_tokens, oracle_tokens, margins, logit_scale):
-    """Identical greedy streams wherever the oracle's top-2 margin exceeds the end-to-end tolerance."""
-    n = min(len(device_tokens), len(oracle_tokens))
-    for i in range(n):
-        if device_tokens[i] != oracle_tokens[i]:
-            assert margins[i] <= E2E_REL_L2 * logit_scale, (i, device_tokens[i], oracle_tokens[i], margins[i])
-            return i
-    return n
+E2E_REL_L2 = chain_budget(3)   # no model here is deeper than 3 layers
 
 
 GEOMETRIES = [
@@ -327,17 +322,15 @@ GEOMETRIES = [
 
 
 STEP_MODES = {
-    # id: (NERVA_HIP_FRONT, NERVA_HIP_CHAIN, fused_state mode of a session whose shapes fit)
-    "launch-per-piece": (None, None, N.DecodeSession.FUSED_NONE),         # the default
-    "fused-front": ("1", None, N.DecodeSession.FUSED_FRONT),
-    "fused-attn-o": ("2", None, N.DecodeSession.FUSED_FRONT_ATTN_O),
-    "chain-kernel": (None, "1", N.DecodeSession.FUSED_CHAIN),
+    # id: (NERVA_HIP_CHAIN, fused_state mode of a session whose shapes fit)
+    "launch-per-piece": (None, N.DecodeSession.FUSED_NONE),         # the default
+    "chain-kernel": ("1", N.DecodeSession.FUSED_CHAIN),
 }
 
 
 def set_step_mode(monkeypatch, name):
-    front, chain, _ = STEP_MODES[name]
-    for var, val in (("NERVA_HIP_FRONT", front), ("NERVA_HIP_CHAIN", chain)):
+    chain, _ = STEP_MODES[name]
+    for var, val in (("NERVA_HIP_CHAIN", chain),):
         if val is None:
             monkeypatch.delenv(var, raising=False)
         else:
@@ -348,9 +341,7 @@ def mode_fits(name, hidden, heads, kv, hd):
     """Whether a session of these shapes actually takes the kernels the mode asks for."""
     if name == "launch-per-piece":
         return True
-    if name == "chain-kernel":
-        return hidden % 2048 == 0
-    return hd == 128 and heads == 4 * kv and hidden % 512 == 0 and hidden <= 4096 and heads * hd <= 4096
+    return hidden % 2048 == 0
 
 
 @pytest.fixture(params=list(STEP_MODES), ids=list(STEP_MODES))
@@ -374,7 +365,7 @@ def test_single_layer_short_prompt_is_tight(geom, step_mode):
     tol = REL_L2 if dtype == F16 else 6e-3
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, 1, hidden + 1, theta, qk_norm, bias)
     s = N.DecodeSession.create(weights, 32)
-    assert s.fused_state() == (STEP_MODES[step_mode][2], False)
+    assert s.fused_state() == (STEP_MODES[step_mode][1], False)
     for prompt in ([3], [vocab - 1, 11]):
         ctx = O.Context(omodel, 32, staging=1)
         for i, t in enumerate(prompt):
@@ -406,8 +397,6 @@ def test_session_matches_oracle_logits_kv_and_stream(geom, step_mode):
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, hidden, theta, qk_norm, bias)
     prompt = np.random.default_rng(1).integers(0, vocab, 21).astype(np.uint32)
     steps = 24
-    ctx = O.Context(omodel, 64, staging=1)
-    otokens, margins = ctx.greedy_decode(prompt, steps)
     s = N.DecodeSession.create(weights, 64)
     rc, res = s.start(prompt)
     assert rc == 0
@@ -417,21 +406,25 @@ def test_session_matches_oracle_logits_kv_and_stream(geom, step_mode):
         ctx2.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
     ref_logits = ctx2.logits()
     got_logits = s.logits()
-    assert rel_l2(got_logits, ref_logits) <= E2E_REL_L2
+    assert rel_l2(got_logits, ref_logits) <= chain_budget(layers)
     for layer in range(layers):
         for token in (0, 7, len(prompt) - 1):
             gk, gv = s.kv_row(layer, token)
             rk, rv = ctx2.read_kv16(layer, token)
             # layer 0 rows depend on one embedding row only: at most a few 16-bit ties differ
-            tol = 2e-3 if layer == 0 else E2E_REL_L2
+            tol = 2e-3 if layer == 0 else chain_budget(layer)
             assert rel_l2(O.decode16(dtype, gk), O.decode16(dtype, rk)) <= tol
             assert rel_l2(O.decode16(dtype, gv), O.decode16(dtype, rv)) <= tol
+    # the stream token by token: every step's logits and token against the oracle that follows the
+    # device's tokens (in every step mode; the launch-per-piece step is also traced link by link in
+    # tests/test_gpu_parity_links.py)
+    stepwise, _, e2e = run_traced_stream(s, omodel, prompt, steps, 64, trace_links=False)
+    # the same stream from one call: graph replays back to back, no allocation, one synchronisation
+    rc, _ = s.start(prompt)
     rc, res, tokens = s.advance(steps)
     assert rc == 0 and res.observed_tokens == steps and res.graph_replays == steps - 1
     assert res.hot_path_allocations == 0 and res.host_causality_edges == 0 and res.sync_calls == 1
-    scale = float(np.max(np.abs(ref_logits)))
-    agreed = assert_streams_agree(tokens.tolist(), otokens.tolist(), margins, scale)
-    assert agreed >= 1
+    assert tokens.tolist() == stepwise
     assert res.observed_token_hash == O.fnv1a(tokens)
     # determinism: the same prompt again gives the same stream and hash
     rc, _ = s.start(prompt)
@@ -466,7 +459,7 @@ def test_eager_profile_pass_leaves_state_untouched():
     s.start(prompt)
     rc, res, a = s.advance(4)
     rc, prof = s.profile_step(2)
-    assert rc == 0 and prof.status == 0 and prof.front_mode == 0 and prof.launches == 3 + 5 * 2
+    assert rc == 0 and prof.status == 0 and prof.launches == 3 + 5 * 2
     assert prof.gate_up_ns > 0 and prof.lm_head_ns > 0 and prof.position == len(prompt) + 3
     rc, res, b = s.advance(6)
     s.start(prompt)
@@ -495,16 +488,11 @@ def test_synthetic_session_matches_oracle_weights():
     omodel = O.Model(BF16, H, 4, 1, HD, I, V, 1e-6, 1e6, g(1, V * H).reshape(V, H), layers, g(2, H, 1.0),
                      g(3, V * H).reshape(V, H))
     prompt = O.synth_tokens(seed, 1000, 12, V)
-    ctx = O.Context(omodel, 64, staging=1)
-    otokens, margins = ctx.greedy_decode(prompt, 8)
     rc, res = s.start(prompt)
     assert rc == 0
     rc, res, tokens = s.advance(8)
     assert rc == 0
-    ctx2 = O.Context(omodel, 64, staging=1)
-    for i, t in enumerate(prompt):
-        ctx2.forward_token(int(t), prompt_token=True, want_logits=(i == len(prompt) - 1))
-    assert_streams_agree(tokens.tolist(), otokens.tolist(), margins, float(np.max(np.abs(ctx2.logits()))))
+    assert_stream_follows_oracle(omodel, prompt, tokens, 64)
     s.destroy()
 
 
@@ -560,60 +548,6 @@ def test_chain_kernel_bounded_wait_gives_up_cleanly(monkeypatch):
     assert rc == -1 and res.status == -1 and res.hip_error != 0
     rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
     assert rc == 0 and s.fused_state() == (s.FUSED_CHAIN, False)
-    rc, res, again = s.advance(3)
-    assert rc == 0 and again.tolist() == good.tolist()
-    s.destroy()
-
-
-FRONT_GEOM = (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False)
-
-
-def test_fused_front_modes_agree_with_one_launch_per_piece(monkeypatch):
-    """Shapes that fit run qkv + attention + o as roles of one launch (3 launches per layer). The
-    GEMV roles sum in the same order as the stand-alone kernels and the attention role differs only
-    in how keys are grouped into splits, so logits agree to 16-bit-tie noise."""
-    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = FRONT_GEOM
-    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 91, theta, qk_norm, bias)
-    prompt = np.random.default_rng(5).integers(0, vocab, 37).astype(np.uint32)
-    results = {}
-    for name in ("fused-front", "fused-attn-o", "launch-per-piece"):
-        set_step_mode(monkeypatch, name)
-        s = N.DecodeSession.create(weights, 96)
-        assert s.fused_state() == (STEP_MODES[name][2], False)
-        rc, res = s.start(prompt)
-        assert rc == 0
-        rc, res, tokens = s.advance(40)               # crosses 16-token block boundaries
-        per_layer = {"fused-front": 3, "fused-attn-o": 4, "launch-per-piece": 5}[name]
-        assert rc == 0 and res.graph_nodes == 3 + per_layer * layers and res.hot_path_allocations == 0
-        rc, prof = s.profile_step(2)
-        assert rc == 0 and prof.launches == 3 + per_layer * layers
-        rc, res, more = s.advance(4)                  # profiling did not disturb the sequence
-        assert rc == 0
-        results[name] = (tokens.tolist() + more.tolist(), s.logits())
-        s.destroy()
-    ref_tokens, ref_logits = results["launch-per-piece"]
-    for name in ("fused-front", "fused-attn-o"):
-        tokens, logits = results[name]
-        assert rel_l2(logits, ref_logits) <= E2E_REL_L2
-        assert tokens[:8] == ref_tokens[:8]
-
-
-def test_fused_front_bounded_wait_gives_up_cleanly(monkeypatch):
-    """With the abort word raised from the host every in-kernel wait of the fused front gives up
-    at once: all kernels still run to completion, the call reports the failure, and start() makes
-    the session usable again."""
-    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = FRONT_GEOM
-    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 92, theta, qk_norm, bias)
-    set_step_mode(monkeypatch, "fused-front")
-    s = N.DecodeSession.create(weights, 32)
-    rc, res = s.start([1, 2, 3])
-    rc, res, good = s.advance(3)
-    assert rc == 0
-    assert s.fused_state(raise_abort=True) == (s.FUSED_FRONT, True)
-    rc, res, _ = s.advance(2)
-    assert rc == -1 and res.status == -1 and res.hip_error != 0
-    rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
-    assert rc == 0 and s.fused_state() == (s.FUSED_FRONT, False)
     rc, res, again = s.advance(3)
     assert rc == 0 and again.tolist() == good.tolist()
     s.destroy()
