@@ -106,6 +106,332 @@ __global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams 
   attn_fast_body<DT, G, W, false, 1>(p, p.position, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The decode step's launch: one token, grid (kv_heads, splits), 8 waves, G = 1, 2 or 4 query heads per
+// kv head. Same arithmetic as attn_fast_body (same tile step, same merges); what differs is the order
+// in which a wave asks for things, because at decode sizes - a wave owns two or three 8 KiB tiles of an
+// 8k-token context - the launch is one burst of requests and a chain of latencies, not a stream:
+//   1. the head inputs (raw q / k / v, bias, norm weights, rotation) are requested first but NOT
+//      awaited; 2. position and block-table entries come through the scalar path; 3. the wave's tiles
+//      (up to four) are requested right behind the inputs; 4. the wave waits for the inputs only:
+//      loads return in request order, so "at most 8 x tiles requests outstanding" means the inputs have
+//      arrived while every tile is still in flight. All of these requests are issued by hand with
+//      explicit outstanding-request counts: a count the compiler derives stops at the first
+//      conditional request and falls back to waiting for everything.
+//   5. head preparation (bias, RMSNorm, RoPE, scaling, hi/lo split) runs under the tiles' flight; the
+//      query operand of the first product is written to LDS once per workgroup, as 16-bit hi and lo
+//      rows, and every wave reads its operand registers back with four 16-byte LDS reads.
+//   6. tiles are consumed in request order with counted waits; a wave with more than four tiles
+//      re-requests into the registers it has just consumed. A wait is a bare instruction chosen by a
+//      scalar branch on the number of tiles requested behind the awaited one; the statement that hands
+//      the awaited registers to the compiler comes after the branch has joined, so nothing that reads
+//      them (not even a register copy) can precede the wait.
+// A split takes ceil(blocks / splits) blocks - not rounded up to a multiple of the wave count: at 8k
+// tokens that keeps 31 of 32 splits busy instead of 22 - and a wave without a tile simply contributes
+// nothing to the merge.
+// ---------------------------------------------------------------------------------------------
+// Loads through the scalar path (position, block-table entries: the same for every lane, and read-only
+// while the launch runs). The compiler takes the vector path for them - it cannot prove that the
+// launch does not write there - and a vector load would have to be awaited with everything requested
+// before it.
+__device__ __forceinline__ uint32_t sload(const uint32_t *ptr) {
+  uint32_t v;
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ptr) : "memory");
+  return v;
+}
+__device__ __forceinline__ void sload4(const uint32_t *p0, const uint32_t *p1, const uint32_t *p2, const uint32_t *p3,
+                                       uint32_t (&v)[4]) {
+  asm volatile(
+      "s_load_dword %0, %4, 0x0\n\ts_load_dword %1, %5, 0x0\n\ts_load_dword %2, %6, 0x0\n\ts_load_dword %3, %7, 0x0\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(v[0]), "=&s"(v[1]), "=&s"(v[2]), "=&s"(v[3])
+      : "s"(p0), "s"(p1), "s"(p2), "s"(p3)
+      : "memory");
+}
+
+template <int G>
+struct StepShared {
+  static constexpr int kRow = kHD + 8;     // 272-byte rows: the operand reads of a lane group spread over the banks
+  alignas(16) uint16_t qhl[2 * G][kRow];   // Qx columns: rows 0..G-1 the hi halves of the scaled query heads, G..2G-1 the lo halves
+  alignas(16) uint16_t knew[kHD];
+  alignas(16) uint16_t vnew[kHD];
+  float wm[8][G], wl[8][G];
+  alignas(16) float wacc[8][G][kHD];
+  uint32_t is_last;
+};
+
+#define NV_AT_LD32(DST, PTR, OFF) asm volatile("global_load_dword %0, %1, off offset:" #OFF : "=v"(DST) : "v"(PTR) : "memory")
+#define NV_AT_LD16(DST, PTR, OFF) asm volatile("global_load_ushort %0, %1, off offset:" #OFF : "=v"(DST) : "v"(PTR) : "memory")
+#define NV_AT_TILE_LOAD(F, PHYS)                                                                                 \
+  do {                                                                                                           \
+    const uint64_t t_ = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, (PHYS), kvh) + lane * 8;          \
+    const uint16_t *kp_ = p.k_cache + t_, *vp_ = p.v_cache + t_;                                                  \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(kr[F][0]) : "v"(kp_) : "memory");                    \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:1024 nt" : "=v"(kr[F][1]) : "v"(kp_) : "memory");        \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:2048 nt" : "=v"(kr[F][2]) : "v"(kp_) : "memory");        \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:3072 nt" : "=v"(kr[F][3]) : "v"(kp_) : "memory");        \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(vr[F][0]) : "v"(vp_) : "memory");                    \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:1024 nt" : "=v"(vr[F][1]) : "v"(vp_) : "memory");        \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:2048 nt" : "=v"(vr[F][2]) : "v"(vp_) : "memory");        \
+    asm volatile("global_load_dwordx4 %0, %1, off offset:3072 nt" : "=v"(vr[F][3]) : "v"(vp_) : "memory");        \
+  } while (0)
+// Waits until at most 8 * TILES of this wave's requests are outstanding (TILES uniform, 0..4).
+#define NV_AT_WAIT_BEHIND(TILES)                                                \
+  do {                                                                          \
+    switch (TILES) {                                                            \
+      case 0u: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;          \
+      case 1u: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;          \
+      case 2u: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;         \
+      case 3u: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;         \
+      default: asm volatile("s_waitcnt vmcnt(32)" ::: "memory"); break;         \
+    }                                                                           \
+  } while (0)
+// Hands registers that a wait has just covered to the compiler: every later use depends on this statement.
+#define NV_AT_TAKE_INPUTS()                                                                                        \
+  asm volatile(""                                                                                                  \
+               : "+v"(qx0), "+v"(qx1), "+v"(ex0), "+v"(ex1), "+v"(qb0), "+v"(qb1), "+v"(eb0), "+v"(eb1), "+v"(qg0), \
+                 "+v"(qg1), "+v"(kg0), "+v"(kg1), "+v"(ra), "+v"(rb))
+#define NV_AT_TAKE_TILE(F)                                                                                         \
+  asm volatile(""                                                                                                  \
+               : "+v"(kr[F][0]), "+v"(kr[F][1]), "+v"(kr[F][2]), "+v"(kr[F][3]), "+v"(vr[F][0]), "+v"(vr[F][1]),   \
+                 "+v"(vr[F][2]), "+v"(vr[F][3]))
+#define NV_AT_U4(V) make_uint4((V).x, (V).y, (V).z, (V).w)
+
+template <uint32_t DT, int G>
+__global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
+  constexpr int W = 8;
+  constexpr int kThreads = W * kWave;
+  __shared__ StepShared<G> sh;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t kvh = blockIdx.x, split = blockIdx.y, S = gridDim.y;
+  const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
+  uint64_t *const tr = kvh == 0 && split == 0 ? p.trace : nullptr;
+  uint64_t *const trm = kvh == 0 ? p.trace : nullptr;
+  link_mark(tr, 7);
+
+  // ---- 1. head inputs, every one of them requested unconditionally (a missing bias / weight / table
+  // reads a stand-in address inside the projection vector and is ignored below)
+  const bool q_wave = wave < G, key_wave = wave == (G % W), value_wave = wave == ((G + 1) % W);
+  const uint32_t qoff = (kvh * G + (q_wave ? wave : 0)) * kHD;
+  const uint32_t eoff = (value_wave ? A + KV : A) + kvh * kHD;
+  const uint16_t *stand_in = reinterpret_cast<const uint16_t *>(p.qkv);
+  const uint16_t *ebias = value_wave ? p.v_bias : p.k_bias;
+  const float *qp = p.qkv + qoff + lane, *ep = p.qkv + eoff + lane;
+  const uint16_t *qbp = (p.q_bias != nullptr ? p.q_bias + qoff : stand_in) + lane;
+  const uint16_t *ebp = (ebias != nullptr ? ebias + kvh * kHD : stand_in) + lane;
+  const uint16_t *qgp = (p.q_norm != nullptr ? p.q_norm : stand_in) + lane;
+  const uint16_t *kgp = (p.k_norm != nullptr ? p.k_norm : stand_in) + lane;
+  const float *rap = (p.rope_cs != nullptr ? p.rope_cs : (p.rope_freq != nullptr ? p.rope_freq : p.qkv)) + lane;
+  const float *rbp = p.rope_cs != nullptr ? p.rope_cs + 64 + lane : rap;
+  float qx0, qx1, ex0, ex1, ra, rb;
+  uint32_t qb0, qb1, eb0, eb1, qg0, qg1, kg0, kg1;
+  NV_AT_LD32(qx0, qp, 0);
+  NV_AT_LD32(qx1, qp, 256);
+  NV_AT_LD32(ex0, ep, 0);
+  NV_AT_LD32(ex1, ep, 256);
+  NV_AT_LD16(qb0, qbp, 0);
+  NV_AT_LD16(qb1, qbp, 128);
+  NV_AT_LD16(eb0, ebp, 0);
+  NV_AT_LD16(eb1, ebp, 128);
+  NV_AT_LD16(qg0, qgp, 0);
+  NV_AT_LD16(qg1, qgp, 128);
+  NV_AT_LD16(kg0, kgp, 0);
+  NV_AT_LD16(kg1, kgp, 128);
+  NV_AT_LD32(ra, rap, 0);
+  NV_AT_LD32(rb, rbp, 0);
+
+  // ---- 2. position, this split's blocks, this wave's tiles (scalar path)
+  const uint32_t pos = p.cursor != nullptr ? sload(p.cursor) : p.position;
+  if (p.cursor != nullptr && pos >= p.max_steps) return;
+  const uint32_t n_keys = pos + 1;
+  const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
+  const uint32_t bps = (nblk + S - 1) / S;
+  const uint32_t active = (nblk + bps - 1) / bps;
+  if (split >= active) return;  // idle splits neither store a partial nor take a ticket
+  const uint32_t b0 = split * bps;
+  const uint32_t b1 = min(nblk, b0 + bps);
+  const uint32_t first = b0 + wave;
+  const uint32_t nt = first < b1 ? (b1 - first + W - 1) / W : 0u;  // tiles first, first + W, ...
+  const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
+  const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
+  uint32_t phys[4];
+  sload4(p.table + min(first, nblk - 1), p.table + min(first + W, nblk - 1), p.table + min(first + 2 * W, nblk - 1),
+         p.table + min(first + 3 * W, nblk - 1), phys);
+
+  // ---- 3. the wave's first four tiles
+  u32x4_t kr[4][4], vr[4][4];
+  if (nt > 0) NV_AT_TILE_LOAD(0, phys[0]);
+  if (nt > 1) NV_AT_TILE_LOAD(1, phys[1]);
+  if (nt > 2) NV_AT_TILE_LOAD(2, phys[2]);
+  if (nt > 3) NV_AT_TILE_LOAD(3, phys[3]);
+  link_mark(tr, 8);
+
+  // ---- 4. the inputs have arrived once at most the tile requests are outstanding
+  NV_AT_WAIT_BEHIND(min(nt, 4u));
+  NV_AT_TAKE_INPUTS();
+  link_mark(tr, 14);
+
+  // ---- 5. head preparation under the tiles' flight
+  const bool has_rope = p.rope_freq != nullptr;
+  float rc = ra, rs = rb;
+  if (has_rope && p.rope_cs == nullptr) sincosf(static_cast<float>(pos) / ra, &rs, &rc);
+  if (q_wave) {
+    float x0 = qx0, x1 = qx1;
+    head_values<DT>(x0, x1, p.q_bias != nullptr, dec16<DT>(static_cast<uint16_t>(qb0)), dec16<DT>(static_cast<uint16_t>(qb1)),
+                    p.q_norm != nullptr, dec16<DT>(static_cast<uint16_t>(qg0)), dec16<DT>(static_cast<uint16_t>(qg1)),
+                    has_rope, rc, rs, p.eps);
+    // softmax runs in base 2 on scores scaled by 1/sqrt(d): both folded into the query
+    const float scale = kLog2e / sqrtf(static_cast<float>(kHD));
+    uint16_t h0, l0, h1, l1;
+    split16<DT>(x0 * scale, h0, l0);
+    split16<DT>(x1 * scale, h1, l1);
+    sh.qhl[wave][lane] = h0;
+    sh.qhl[wave][lane + 64] = h1;
+    sh.qhl[G + wave][lane] = l0;
+    sh.qhl[G + wave][lane + 64] = l1;
+  }
+  if (owns_new && (key_wave || value_wave)) {
+    float x0 = ex0, x1 = ex1;
+    const bool norm = key_wave && p.k_norm != nullptr;
+    head_values<DT>(x0, x1, ebias != nullptr, dec16<DT>(static_cast<uint16_t>(eb0)), dec16<DT>(static_cast<uint16_t>(eb1)), norm,
+                    dec16<DT>(static_cast<uint16_t>(kg0)), dec16<DT>(static_cast<uint16_t>(kg1)), key_wave && has_rope, rc, rs,
+                    p.eps);
+    uint16_t *row = key_wave ? sh.knew : sh.vnew;
+    row[lane] = enc16<DT>(x0);
+    row[lane + 64] = enc16<DT>(x1);
+  }
+  link_mark(tr, 15);
+  __syncthreads();
+  link_mark(tr, 9);
+  if (owns_new && wave == W - 1) {
+    // publish the rounded row to the cache in operand order
+    const uint64_t tile = kv_tile_offset(p.block_count, p.kv_heads, kHD, p.layer, sload(p.table + new_block), kvh);
+    if (lane < 16)  // K: 16 pieces of 8 consecutive dims
+      *reinterpret_cast<uint4 *>(p.k_cache + tile + kv_k_elem(kHD, new_row, lane * 8)) =
+          *reinterpret_cast<const uint4 *>(sh.knew + lane * 8);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {  // V: one 16-bit element per dim
+      const uint32_t d = lane + i * kWave;
+      p.v_cache[tile + kv_v_elem(kHD, new_row, d)] = sh.vnew[d];
+    }
+  }
+
+  // ---- B operand of the first product: column `col` of Qx for dims j*32 + grp*8 .. +7
+  const int col = lane & 15, grp = lane >> 4;
+  uint4 qx[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(&sh.qhl[col < 2 * G ? col : 0][j * 32 + grp * 8]);
+    qx[j] = col < 2 * G ? v : make_uint4(0u, 0u, 0u, 0u);
+  }
+  link_mark(tr, 10);
+
+  // ---- 6. tiles in request order
+  float m = -INFINITY, l = 0.0f;  // of column `col` (both copies of a head track the same values)
+  f32x4_t acc[8];                  // O^T[dims s*16 + grp*4 .. +3][col]
+#pragma unroll
+  for (int s2 = 0; s2 < 8; ++s2) acc[s2] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#define NV_AT_STEP(F)                                                                                              \
+  do {                                                                                                             \
+    const uint32_t t_idx = done + F;                                                                               \
+    if (t_idx < nt) {                                                                                              \
+      /* tiles requested behind this one and not yet consumed: at most three */                                   \
+      NV_AT_WAIT_BEHIND(min(nt - t_idx - 1u, 3u));                                                                 \
+      NV_AT_TAKE_TILE(F);                                                                                          \
+      uint4 kk[4], vv[4];                                                                                          \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                              \
+        kk[j] = NV_AT_U4(kr[F][j]);                                                                                \
+        vv[j] = NV_AT_U4(vr[F][j]);                                                                                \
+      }                                                                                                            \
+      const uint32_t bb = first + t_idx * W;                                                                       \
+      attn_tile<DT, G, false>(kk, vv, qx, nullptr, bb, n_keys, col, grp, owns_new && bb == new_block, new_row,     \
+                              sh.knew, sh.vnew, m, l, acc);                                                        \
+      if (t_idx + 4u < nt) NV_AT_TILE_LOAD(F, sload(p.table + first + (t_idx + 4u) * W));                          \
+    }                                                                                                              \
+  } while (0)
+  for (uint32_t done = 0; done < nt; done += 4) {
+    NV_AT_STEP(0);
+    NV_AT_STEP(1);
+    NV_AT_STEP(2);
+    NV_AT_STEP(3);
+  }
+#undef NV_AT_STEP
+  link_mark(tr, 11);
+
+  // ---- 7. wave result: tokens of the four lane groups, then hi + lo columns; then the W waves
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+#pragma unroll
+  for (int s2 = 0; s2 < 8; ++s2) {
+    float4 o;
+    o.x = acc[s2][0] + row_shl<G>(acc[s2][0]);
+    o.y = acc[s2][1] + row_shl<G>(acc[s2][1]);
+    o.z = acc[s2][2] + row_shl<G>(acc[s2][2]);
+    o.w = acc[s2][3] + row_shl<G>(acc[s2][3]);
+    if (col < G) *reinterpret_cast<float4 *>(&sh.wacc[wave][col][s2 * 16 + grp * 4]) = o;
+  }
+  if (lane < G) {
+    sh.wm[wave][lane] = m;
+    sh.wl[wave][lane] = l;
+  }
+  __syncthreads();
+  // every thread owns output elements (g, d): the W waves' scale factors are recomputed per thread
+  // (eight exponentials) instead of being shared through another barrier
+  for (int e = threadIdx.x; e < G * kHD; e += kThreads) {
+    const int g = e / kHD, d = e % kHD;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < W; ++w) M = fmaxf(M, sh.wm[w][g]);
+    float L = 0.0f, o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      const float mw = sh.wm[w][g];
+      const float f = mw > -INFINITY ? attn_exp2(mw - M) : 0.0f;  // a wave without a tile contributes nothing
+      L = fmaf(sh.wl[w][g], f, L);
+      o = fmaf(sh.wacc[w][g][d], f, o);
+    }
+    const uint32_t h = kvh * G + g;
+    if (active == 1) {
+      // a single split holds every key: this is the final result, nothing to exchange
+      if (L > 0.0f && isfinite(L)) o /= L;
+      if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
+      p.out16[attn_out_elem(p, h * kHD + d)] = enc16<DT>(o);
+    } else {
+      // The partial leaves through device-coherent stores (written through, no cache flush).
+      store_coherent(p.part_acc + (static_cast<uint64_t>(h) * S + split) * kHD + d, o);
+      if (d == 0) {
+        store_coherent(p.part_m + h * S + split, M);
+        store_coherent(p.part_l + h * S + split, L);
+      }
+    }
+  }
+  if (active == 1) return;
+  // Every wave waits until its own stores have been performed, the barrier collects the waves,
+  // and only then one lane takes the arrival ticket of this kv head.
+  wait_stores_performed();
+  __syncthreads();
+  link_mark(tr, 12);
+  if (threadIdx.x == 0) {
+    const uint32_t ticket = __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.is_last = ticket == active - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  link_mark(tr, 13);
+  if (!sh.is_last) return;
+  link_mark(trm, 16);
+  merge_splits<DT, G, kThreads>(p, kvh, S, active, lane);
+  if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  link_mark(trm, 17);
+}
+#undef NV_AT_LD32
+#undef NV_AT_LD16
+#undef NV_AT_TILE_LOAD
+#undef NV_AT_WAIT_BEHIND
+#undef NV_AT_TAKE_INPUTS
+#undef NV_AT_TAKE_TILE
+#undef NV_AT_U4
+
 // Any head_dim (even when RoPE is on) / any group size: one workgroup per query
 // head, waves stride over tokens, lanes over dims. Used for shapes the fast path
 // does not cover (the tiny known-answer models).
@@ -265,9 +591,9 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
       return hipGetLastError();
     }
     switch (group) {
-      case 1: hipLaunchKernelGGL((attn_fast_kernel<DT, 1, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
-      case 2: hipLaunchKernelGGL((attn_fast_kernel<DT, 2, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
-      case 4: hipLaunchKernelGGL((attn_fast_kernel<DT, 4, kAttnWaves>), grid, dim3(kAttnWaves * kWave), 0, stream, p); break;
+      case 1: hipLaunchKernelGGL((attn_step_kernel<DT, 1>), grid, dim3(8 * kWave), 0, stream, p); break;
+      case 2: hipLaunchKernelGGL((attn_step_kernel<DT, 2>), grid, dim3(8 * kWave), 0, stream, p); break;
+      case 4: hipLaunchKernelGGL((attn_step_kernel<DT, 4>), grid, dim3(8 * kWave), 0, stream, p); break;
       default: hipLaunchKernelGGL((attn_fast_kernel<DT, 8, kAttnWaves / 2>), grid, dim3(kAttnWaves / 2 * kWave), 0, stream, p); break;
     }
   } else {

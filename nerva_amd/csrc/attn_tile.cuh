@@ -50,6 +50,27 @@ __device__ __forceinline__ void prep_head128_core(float x0, float x1, bool has_b
     out[lane + 64] = x1;
   }
 }
+// The same arithmetic on values that stay in registers: (x0, x1) = dims (lane, lane + 64) of one head.
+template <uint32_t DT>
+__device__ __forceinline__ void head_values(float &x0, float &x1, bool has_bias, float b0, float b1, bool has_gamma,
+                                            float g0, float g1, bool has_rope, float c, float s, float eps) {
+  if (has_bias) {
+    x0 += b0;
+    x1 += b1;
+  }
+  if (has_gamma) {
+    const float ss = wave_sum(x0 * x0 + x1 * x1);
+    const float scale = 1.0f / sqrtf(ss / 128.0f + eps);
+    x0 *= scale * g0;
+    x1 *= scale * g1;
+  }
+  if (has_rope) {
+    const float r0 = x0 * c - x1 * s;
+    const float r1 = x1 * c + x0 * s;
+    x0 = r0;
+    x1 = r1;
+  }
+}
 // Same with bias / gamma / rotation fetched here.
 template <uint32_t DT>
 __device__ __forceinline__ void prep_head128(float x0, float x1, const uint16_t *bias,
@@ -298,7 +319,6 @@ __device__ __forceinline__ bool link_give_up(uint32_t *abort_flag, uint32_t &spi
   return false;
 }
 
-constexpr int kTicketRound = 32;           // splits read per round by the last workgroup of the ticket protocol
 constexpr int kMergeRound = 16;            // splits polled per round by the merging workgroup
 constexpr uint32_t kPartRecord = kHD + 2;  // tagged words of one (head, split) partial: acc[128], m, l
 
@@ -412,6 +432,64 @@ __device__ __forceinline__ RawHeads<G, W> attn_request_raw(const AttnParams &p, 
     }
   }
   return r;
+}
+
+constexpr int kTicketRound = 32;           // splits read per round by the last workgroup of the ticket protocol
+// The last workgroup of a kv head merges the splits' partials. Each thread owns output elements (g, d)
+// and reads the partials with device-coherent loads, kTicketRound splits per round trip, in split
+// order, so the result does not depend on which workgroup arrived last.
+template <uint32_t DT, int G, int THREADS>
+__device__ __forceinline__ void merge_splits(const AttnParams &p, uint32_t kvh, uint32_t S, uint32_t active, int lane) {
+  for (int e = threadIdx.x; e < G * kHD; e += THREADS) {
+    const int g = e / kHD, d = e % kHD;
+    const uint32_t h = kvh * G + g;
+    const float *pm = p.part_m + h * S, *pl = p.part_l + h * S;
+    const float *src = p.part_acc + static_cast<uint64_t>(h) * S * kHD + d;
+    float M = -INFINITY, L = 0.0f, o = 0.0f;
+    for (uint32_t s0 = 0; s0 < active; s0 += kTicketRound) {
+      float mm[kTicketRound], ll[kTicketRound], aa[kTicketRound];
+      // m and l of this head's splits: the head is the same for all lanes of a wave, so lane i fetches
+      // m of split s0 + i and lane kTicketRound + i its l (one load a lane instead of two per split),
+      // and the values are handed round with lane reads below.
+      static_assert(2 * kTicketRound == kWave && kHD % kWave == 0, "one (m, l) pair per lane pair, one head per wave");
+      const uint32_t si_ml = min(s0 + static_cast<uint32_t>(lane & (kTicketRound - 1)), active - 1);
+      const float ml = load_coherent((lane < kTicketRound ? pm : pl) + si_ml);
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
+        // unconditional loads (index clamped): a load under a branch would serialise the round
+        const uint32_t si = min(s0 + i, active - 1);
+        aa[i] = load_coherent(src + static_cast<uint64_t>(si) * kHD);
+      }
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
+        mm[i] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ml), i));
+        ll[i] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ml), kTicketRound + i));
+      }
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
+        const bool on = s0 + i < active;
+        mm[i] = on ? mm[i] : -INFINITY;
+        ll[i] = on ? ll[i] : 0.0f;
+        aa[i] = on ? aa[i] : 0.0f;
+      }
+      float Mc = M;
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) Mc = fmaxf(Mc, mm[i]);
+      const float keep = M > -INFINITY ? attn_exp2(M - Mc) : 0.0f;
+      L *= keep;
+      o *= keep;
+#pragma unroll
+      for (int i = 0; i < kTicketRound; ++i) {
+        const float f = mm[i] > -INFINITY ? attn_exp2(mm[i] - Mc) : 0.0f;
+        L = fmaf(ll[i], f, L);
+        o = fmaf(aa[i], f, o);
+      }
+      M = Mc;
+    }
+    if (L > 0.0f && isfinite(L)) o /= L;
+    if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
+    p.out16[attn_out_elem(p, h * kHD + d)] = enc16<DT>(o);
+  }
 }
 
 // W waves per workgroup. A workgroup owns one kv head and one contiguous range of
