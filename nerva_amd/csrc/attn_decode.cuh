@@ -77,7 +77,46 @@ struct AttnParams {
   // Block launches only: != 0 writes out16 in the multi-row GEMM's operand order (gemm_x_packed_index)
   // with this many token tiles, instead of [token][heads * head_dim] rows.
   uint32_t out_packed_tiles;
+  // Decode step only, optional: this step's split plan (attn_plan_fill), written once per step for
+  // all layers - position, split geometry and every wave's first physical blocks - so that a launch
+  // reaches its tile requests through one scalar read instead of position -> block table -> tiles.
+  // Valid for launches with `splits` = the plan's split factor and 8 waves per workgroup.
+  const uint32_t *plan;
 };
+
+// ---- per-step split plan of the decode attention ---------------------------------------------
+// words [0..7]: position, blocks, blocks per split, active splits, 4 spare;
+// then one 8-word entry per (split, wave): tiles of the wave, its first block, the physical blocks
+// of its first four tiles (clamped), 2 spare.
+constexpr uint32_t kAttnPlanHeader = 8, kAttnPlanEntry = 8, kAttnPlanWaves = 8;
+__host__ __device__ __forceinline__ uint64_t attn_plan_bytes(uint32_t splits) {
+  return (kAttnPlanHeader + static_cast<uint64_t>(splits) * kAttnPlanWaves * kAttnPlanEntry) * sizeof(uint32_t);
+}
+// Split geometry shared by the kernel and the plan: a split takes ceil(blocks / splits) blocks.
+__host__ __device__ __forceinline__ void attn_split_geometry(uint32_t pos, uint32_t splits, uint32_t &nblk, uint32_t &bps,
+                                                             uint32_t &active) {
+  nblk = (pos + 1 + kKvBlockTokens - 1) / kKvBlockTokens;
+  bps = (nblk + splits - 1) / splits;
+  active = (nblk + bps - 1) / bps;
+}
+// One thread per (split, wave) entry (`entry` < splits * 8); entry 0 also writes the header.
+__device__ __forceinline__ void attn_plan_fill(uint32_t *plan, const uint32_t *table, uint32_t pos, uint32_t splits,
+                                               uint32_t entry) {
+  uint32_t nblk, bps, active;
+  attn_split_geometry(pos, splits, nblk, bps, active);
+  if (entry == 0) {
+    plan[0] = pos;
+    plan[1] = nblk;
+    plan[2] = bps;
+    plan[3] = active;
+  }
+  const uint32_t split = entry / kAttnPlanWaves, wave = entry % kAttnPlanWaves;
+  const uint32_t b0 = split * bps, b1 = min(nblk, b0 + bps), first = b0 + wave;
+  uint32_t *e = plan + kAttnPlanHeader + entry * kAttnPlanEntry;
+  e[0] = first < b1 ? (b1 - first + kAttnPlanWaves - 1) / kAttnPlanWaves : 0u;
+  e[1] = first;
+  for (uint32_t f = 0; f < 4; ++f) e[2 + f] = table[min(first + f * kAttnPlanWaves, nblk - 1)];
+}
 
 // Index of output element e (= head * head_dim + dim) behind a token's out16 base.
 __host__ __device__ __forceinline__ uint32_t attn_out_elem(const AttnParams &p, uint32_t e) {

@@ -149,6 +149,14 @@ __device__ __forceinline__ void sload4(const uint32_t *p0, const uint32_t *p1, c
       : "memory");
 }
 
+typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ void sload8x2(const uint32_t *a, const uint32_t *b, u32x8_t &va, u32x8_t &vb) {
+  asm volatile("s_load_dwordx8 %0, %2, 0x0\n\ts_load_dwordx8 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(va), "=&s"(vb)
+               : "s"(a), "s"(b)
+               : "memory");
+}
+
 template <int G>
 struct StepShared {
   static constexpr int kRow = kHD + 8;     // 272-byte rows: the operand reads of a lane group spread over the banks
@@ -242,24 +250,35 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   NV_AT_LD32(rb, rbp, 0);
 
   // ---- 2. position, this split's blocks, this wave's tiles (scalar path)
-  const uint32_t pos = p.cursor != nullptr ? sload(p.cursor) : p.position;
-  if (p.cursor != nullptr && pos >= p.max_steps) return;
-  const uint32_t n_keys = pos + 1;
-  const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
-  const uint32_t bps = (nblk + S - 1) / S;
-  const uint32_t active = (nblk + bps - 1) / bps;
+  uint32_t pos, nblk, bps, active, first, nt, phys[4];
+  if (p.plan != nullptr) {
+    // this step's plan: everything above in one round trip
+    u32x8_t head, mine;
+    sload8x2(p.plan, p.plan + kAttnPlanHeader + (split * W + wave) * kAttnPlanEntry, head, mine);
+    pos = head[0], nblk = head[1], bps = head[2], active = head[3];
+    nt = mine[0], first = mine[1];
+    phys[0] = mine[2], phys[1] = mine[3], phys[2] = mine[4], phys[3] = mine[5];
+    if (pos >= p.max_steps) return;
+  } else {
+    pos = p.cursor != nullptr ? sload(p.cursor) : p.position;
+    if (p.cursor != nullptr && pos >= p.max_steps) return;
+    attn_split_geometry(pos, S, nblk, bps, active);
+    first = split * bps + wave;
+    const uint32_t end = min(nblk, split * bps + bps);
+    nt = first < end ? (end - first + W - 1) / W : 0u;  // tiles first, first + W, ...
+    if (split < active)
+      sload4(p.table + min(first, nblk - 1), p.table + min(first + W, nblk - 1), p.table + min(first + 2 * W, nblk - 1),
+             p.table + min(first + 3 * W, nblk - 1), phys);
+  }
   if (split >= active) return;  // idle splits neither store a partial nor take a ticket
+  const uint32_t n_keys = pos + 1;
   const uint32_t b0 = split * bps;
   const uint32_t b1 = min(nblk, b0 + bps);
-  const uint32_t first = b0 + wave;
-  const uint32_t nt = first < b1 ? (b1 - first + W - 1) / W : 0u;  // tiles first, first + W, ...
   const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
-  uint32_t phys[4];
-  sload4(p.table + min(first, nblk - 1), p.table + min(first + W, nblk - 1), p.table + min(first + 2 * W, nblk - 1),
-         p.table + min(first + 3 * W, nblk - 1), phys);
 
   // ---- 3. the wave's first four tiles
+  link_mark(tr, 6);
   u32x4_t kr[4][4], vr[4][4];
   if (nt > 0) NV_AT_TILE_LOAD(0, phys[0]);
   if (nt > 1) NV_AT_TILE_LOAD(1, phys[1]);

@@ -117,6 +117,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
   void *attn_ws = nullptr, *sample_ws = nullptr;
   uint32_t attn_splits = 1;
+  uint32_t *attn_plan = nullptr;     // this step's split plan of the decode attention (attn_plan_fill), or null
   // persistent layer-chain kernel (o + gate/up + down + next qkv in one launch)
   bool chain = false;
   uint32_t *chain_flags = nullptr, *chain_abort = nullptr;
@@ -172,9 +173,17 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
                                                        const Slot *slots, uint32_t *state,
                                                        uint32_t max_steps, uint32_t hidden,
                                                        uint32_t vocab, float *x, const float *rope_freq,
-                                                       float *rope_cs, uint32_t half_dim) {
+                                                       float *rope_cs, uint32_t half_dim, uint32_t *attn_plan,
+                                                       const uint32_t *table, uint32_t attn_splits) {
   const uint32_t pos = state[0];
+  // the position goes into the attention plan even past the last step: the attention launches take
+  // their step guard from there
+  if (attn_plan != nullptr && blockIdx.x == 0 && threadIdx.x == 0) attn_plan[0] = pos;
   if (pos >= max_steps) return;
+  // this step's split plan of the decode attention, once for all layers
+  if (attn_plan != nullptr && blockIdx.x == 0)
+    for (uint32_t e = threadIdx.x; e < attn_splits * kAttnPlanWaves; e += kBlock)
+      attn_plan_fill(attn_plan, table, pos, attn_splits, e);
   // steps executed so far: the epochs of in-launch hand-overs derive from it (nobody reads it
   // in this launch)
   if (blockIdx.x == 0 && threadIdx.x == 0) state[2] = state[2] + 1u;
@@ -339,11 +348,11 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
     if (s->dtype == kBF16)
       hipLaunchKernelGGL(embed_kernel<kBF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
                          s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
-                         s->head_dim / 2);
+                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits);
     else
       hipLaunchKernelGGL(embed_kernel<kF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
                          s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
-                         s->head_dim / 2);
+                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits);
     err = hipGetLastError();
     if (prof && err == hipSuccess) err = prof->after();
     if (err != hipSuccess) return err;
@@ -393,6 +402,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.max_steps = s->max_ctx;
       p.append = 1;
       p.trace = s->attn_trace != nullptr ? s->attn_trace + 32 * l : nullptr;
+      // (a pass of attention launches alone - profiling - follows full steps at the same position, whose
+      // embedding launch left the plan of that position)
+      p.plan = s->attn_plan;
       NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
       snap(s->attn16, static_cast<uint64_t>(A) * sizeof(uint16_t));
     }
@@ -1020,6 +1032,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_rope_cs = c.take(HD * 4);
   const uint64_t attn_ws_bytes = attn_workspace_bytes(s->heads, s->head_dim);
   const uint64_t off_attn_ws = c.take(attn_ws_bytes);
+  const uint64_t off_attn_plan = c.take(attn_plan_bytes(kAttnMaxSplits));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
   const uint64_t pT = kGemmMaxTokens;
   const uint64_t off_px = c.take(pT * H * 4);
@@ -1093,6 +1106,12 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
   s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
+  {
+    // the plan serves the step kernel (head_dim 128, 1, 2 or 4 query heads per kv head, 8 waves)
+    const uint32_t group = s->kv_heads != 0 ? s->heads / s->kv_heads : 0;
+    if (s->head_dim == 128 && (group == 1 || group == 2 || group == 4))
+      s->attn_plan = reinterpret_cast<uint32_t *>(s->arena + off_attn_plan);
+  }
   s->sample_ws = s->arena + off_sample_ws;
   s->px = reinterpret_cast<float *>(s->arena + off_px);
   s->pr = reinterpret_cast<float *>(s->arena + off_pr);
@@ -1151,6 +1170,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
     err = hipMemcpy(s->rope_freq, freq.data(), freq.size() * 4, hipMemcpyHostToDevice);
   }
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_ws_bytes, s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_plan, 0, attn_plan_bytes(kAttnMaxSplits), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
