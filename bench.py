@@ -114,6 +114,7 @@ def main():
     ap.add_argument("--layers", type=int, default=36, help="(debug) fewer layers = NOT the named workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-layers", type=int, default=2)
+    ap.add_argument("--no-operators", action="store_true", help="skip the operator rows (configs 1-4)")
     ap.add_argument("--batch-sessions", type=int, default=32,
                     help="sessions advanced together in the shared-weights leg (0 = skip it)")
     ap.add_argument("--batch-steps", type=int, default=24)
@@ -269,6 +270,23 @@ def main():
             log("[cpu] baseline failed: %r" % (e,))
     session.destroy()
 
+    # The operator configurations (1: q_proj GEMV, 2: MLP block, 3: paged GQA attention at 4096 keys,
+    # 4: FP8 MoE experts), each over a rotating working set above 1 GB: the "GEMV HBM GB/s as % of
+    # peak" half of the metric. Recorded into one hipGraph per case and timed with hipEvents.
+    operators = None
+    if not args.no_operators:
+        from nerva_amd import opbench
+        operators = {}
+        for key, case in (("configs[0] q_proj GEMV 4096x4096 bf16", opbench.case_qproj),
+                          ("configs[1] MLP block 4096-12288-4096 (2 launches)", opbench.case_mlp),
+                          ("configs[2] paged GQA decode attention 32q/8kv x128, 4097 keys", opbench.case_attention),
+                          ("configs[3] FP8 MoE 8 routed + 1 shared, 7168/2048 (2 launches)", opbench.case_moe)):
+            try:
+                operators[key] = case()
+            except Exception as e:  # an operator row never hides the headline figure
+                log("[bench] operator case %s failed: %r" % (key, e))
+                operators[key] = {"failed": repr(e)}
+
     line = dict(metric="decode tok/s Qwen3-8B bs1", value=round(tok_s, 2), unit="tok/s", n_gpus=1,
                 steps=args.steps, warmup=args.warmup, ms_per_step=round(1e3 * elapsed / args.steps, 4),
                 higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
@@ -278,7 +296,8 @@ def main():
                                      % (cfg["layers"], args.prompt, args.steps),
                             prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), prefill_tok_s=round(args.prompt / prefill_s, 1), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
-                            per_token_latency_ms=latency, shared_weight_sessions=batch, gpu=smoke.gpu_name.decode()),
+                            per_token_latency_ms=latency, shared_weight_sessions=batch, operators=operators,
+                            gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)
     print(json.dumps(line), flush=True)
 

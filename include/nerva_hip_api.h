@@ -614,6 +614,8 @@ typedef struct NervaHipMoeFp8Request {
   const float *s_down;          /* [E][ceil(H/block)][ceil(I/block)] */
   float *activation;            /* scratch f32 [(top_k+1) * intermediate] */
   float *output;                /* f32 [hidden] */
+  uint32_t phases;              /* 0: the whole operator (two launches); 1: gate/up + SwiGLU only (fills
+                                   `activation`); 2: down + combine only (reads `activation`) - timing */
 } NervaHipMoeFp8Request;
 
 /* out = sum_k w_k * Wd_e(swiglu(Wg_e x, Wu_e x)) + shared(x) with FP8 block-scaled

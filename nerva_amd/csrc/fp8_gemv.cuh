@@ -24,6 +24,7 @@ struct MoeFp8Params {
   float *out;   // [hidden]
   uint32_t hidden, inter, num_experts, top_k, block, input_dtype;
   int32_t shared_index;
+  uint32_t phases;   // 0: both launches; 1: gate/up only; 2: down only (act holds an earlier gate/up result)
 };
 
 struct MoeRouteParams {

@@ -683,7 +683,8 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     return hipErrorInvalidValue;
   const bool fast_gu = p.hidden % 1024u == 0 && p.block % 16u == 0 && aligned16(p.w_gate) && aligned16(p.w_up);
   const bool fast_dn = p.inter % 1024u == 0 && p.block % 16u == 0 && aligned16(p.w_down);
-  {
+  if (p.phases > 2) return hipErrorInvalidValue;
+  if (p.phases != 2) {
     const uint64_t units = static_cast<uint64_t>(slots) * p.inter;
     const uint32_t blocks =
         static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 32u));
@@ -706,7 +707,7 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
-  {
+  if (p.phases != 1) {
     constexpr int NR = 2;
     const uint32_t units = (p.hidden + NR - 1) / NR;
     const uint32_t blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;

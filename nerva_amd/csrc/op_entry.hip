@@ -540,6 +540,7 @@ int nerva_hip_moe_fp8_experts(const NervaHipMoeFp8Request *r, void *stream, int3
   p.block = r->block;
   p.input_dtype = r->input_dtype;
   p.shared_index = r->shared_index;
+  p.phases = r->phases;
   return finish(launch_moe_fp8(p, resolve_stream(stream)), hip_error);
 }
 

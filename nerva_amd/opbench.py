@@ -66,9 +66,11 @@ def timed(enqueue, launches, warmup=3, replays=10):
 
 
 def report(name, variant, ns, nbytes):
+    """Prints one row and returns it: {"us", "GB/s", "frac" of the 8 TB/s peak, "bytes"}."""
     gbs = nbytes / ns
     log("%-34s %-9s %9.2f us  %8.1f GB/s  %5.1f%% of HBM peak   (ideal %.2f us)" % (
         name, variant, ns / 1e3, gbs, 100 * gbs / PEAK, nbytes / PEAK / 1e3))
+    return {"us": round(ns / 1e3, 2), "GB/s": round(gbs, 1), "frac": round(gbs / PEAK, 4), "bytes": int(nbytes)}
 
 
 def case_qproj():
@@ -78,10 +80,12 @@ def case_qproj():
     x = synth16(cols, 12, std=1.0)
     y = DeviceBuffer(rows * 2)
     nbytes = rows * cols * 2 + cols * 2 + rows * 2
+    rows_out = {}
     for variant, n in (("rotating", copies), ("resident", 1)):
         ns = timed(lambda i: R.gemv(BF16, w.at((i % n) * rows * cols * 2), rows, cols, input16=x, out16=y,
                                     epilogue=3, sync=False), 80)
-        report("1 q_proj GEMV 4096x4096", variant, ns, nbytes)
+        rows_out[variant] = report("1 q_proj GEMV 4096x4096", variant, ns, nbytes)
+    return rows_out
 
 
 def case_mlp():
@@ -99,9 +103,11 @@ def case_mlp():
         base = (i % n) * per * 2
         R.gemv(BF16, w.at(base), I, H, input_f32=h, gamma=gamma, eps=1e-6, out16=ff, epilogue=2, sync=False)
         R.gemv(BF16, w.at(base + 2 * I * H * 2), H, I, input16=ff, residual=h, out_f32=out, epilogue=1, sync=False)
+    rows_out = {}
     for variant, n in (("rotating", copies), ("resident", 1)):
         ns = timed(lambda i: enqueue(i, n), 24)
-        report("2 MLP block 4096 -> 12288 -> 4096", variant, ns, nbytes)
+        rows_out[variant] = report("2 MLP block 4096 -> 12288 -> 4096", variant, ns, nbytes)
+    return rows_out
 
 
 def case_attention():
@@ -119,11 +125,13 @@ def case_attention():
     out16, out32 = DeviceBuffer(heads * hd * 2), DeviceBuffer(heads * hd * 4)
     kv_read = 2 * (tokens + 1) * kvh * hd * 2
     nbytes = kv_read + (heads + 2 * kvh) * hd * 4 + (blocks * 4) + 2 * kvh * hd * 2 + heads * hd * 4
+    rows_out = {}
     for variant, n in (("rotating", layers), ("resident", 1)):
         ns = timed(lambda i: R.paged_attention(BF16, heads, kvh, hd, cache, i % n, tokens, qkv, ws, out16,
                                                out_f32=out32, append=True, rope_theta=1e6, q_norm=qn, k_norm=kn,
                                                sync=False), 128)
-        report("3 paged GQA attention, 4097 keys", variant, ns, nbytes)
+        rows_out[variant] = report("3 paged GQA attention, 4097 keys", variant, ns, nbytes)
+    return rows_out
 
 
 def case_moe():
@@ -144,10 +152,17 @@ def case_moe():
     act = DeviceBuffer((K + 1) * I * 4)
     out = DeviceBuffer(H * 4)
     nbytes = 9 * (3 * I * H + 3 * sI * sH * 4) + H * 2 + H * 2
+    rows_out = {}
     for variant, n in (("rotating", sets), ("resident", 1)):
         ns = timed(lambda i: R.moe_fp8_experts(H, I, E, K, blk, x, ids[i % n], wts, wg, sg, wu, su, wd, sd, act, out,
                                                shared_index=E - 1, sync=False), 33)
-        report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
+        rows_out[variant] = report("4 FP8 MoE, 8 routed + 1 shared", variant, ns, nbytes)
+    # the two launches on their own (rotating): gate/up + SwiGLU (two thirds of the weights), down + combine
+    for phase, label, part in ((1, "gate_up", 9 * (2 * I * H + 2 * sI * sH * 4) + H * 2), (2, "down", 9 * (I * H + sI * sH * 4) + H * 4)):
+        ns = timed(lambda i: R.moe_fp8_experts(H, I, E, K, blk, x, ids[i % sets], wts, wg, sg, wu, su, wd, sd, act, out,
+                                               shared_index=E - 1, sync=False, phases=phase), 33)
+        rows_out[label] = report("4 FP8 MoE, %s launch" % label, "rotating", ns, part)
+    return rows_out
 
 
 def case_fp8_gemv():

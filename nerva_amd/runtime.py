@@ -324,8 +324,9 @@ def moe_route_softmax(logits, top_k, normalize=True):
 
 
 def moe_fp8_experts(hidden, inter, num_experts, top_k, block, x16, ids, weights, w_gate, s_gate, w_up,
-                    s_up, w_down, s_down, act, out, *, shared_index=-1, input_dtype=BF16, sync=True):
+                    s_up, w_down, s_down, act, out, *, shared_index=-1, input_dtype=BF16, sync=True, phases=0):
     req = abi.NervaHipMoeFp8Request()
+    req.phases = phases
     req.hidden, req.intermediate, req.num_experts, req.top_k = hidden, inter, num_experts, top_k
     req.block, req.input_dtype, req.shared_index = block, input_dtype, shared_index
     req.input16, req.expert_ids, req.expert_weights = _ptr(x16), _ptr(ids), _ptr(weights)
