@@ -276,6 +276,7 @@ def main():
     operators = None
     if not args.no_operators:
         from nerva_amd import opbench
+        opbench.OUT = sys.stderr
         operators = {}
         for key, case in (("configs[0] q_proj GEMV 4096x4096 bf16", opbench.case_qproj),
                           ("configs[1] MLP block 4096-12288-4096 (2 launches)", opbench.case_mlp),

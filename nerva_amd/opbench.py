@@ -29,8 +29,11 @@ SEED = 0x4E45525641
 PEAK = 8000.0
 
 
+OUT = sys.stdout   # a caller that keeps stdout for its own result (bench.py) points this at stderr
+
+
 def log(*a):
-    print(*a, flush=True)
+    print(*a, flush=True, file=OUT)
 
 
 def synth16(count, tid, mean=0.0, std=0.02):
