@@ -54,6 +54,9 @@ struct AttnParams {
   float *part_acc;             // [heads][splits][hd]  un-normalised partial outputs
   float *part_m, *part_l;      // [heads][splits]
   uint32_t *counters;          // [kv_heads] arrival counters, zero between launches
+  // Decode step kernel: the splits' partials as (f32 value, tag) 8-byte words, [heads][splits][head_dim + 2]
+  // (accumulators, then m and l), all tags zero between launches (attn_step_workspace_bytes)
+  uint64_t *part_tagged;
   float *out_f32;              // optional [heads*hd]
   uint16_t *out16;             // [heads*hd]
   uint32_t heads, kv_heads, head_dim, layer, block_count, splits;
@@ -138,6 +141,8 @@ inline uint32_t attn_default_splits(uint32_t kv_heads, uint32_t block_count) {
   return splits == 0 ? 1 : splits;
 }
 uint64_t attn_workspace_bytes(uint32_t heads, uint32_t head_dim);
+// Bytes of AttnParams::part_tagged (head_dim 128), zero-initialised once.
+uint64_t attn_step_workspace_bytes(uint32_t heads);
 // Carves part_acc/part_m/part_l/counters out of a workspace of attn_workspace_bytes().
 void attn_bind_workspace(AttnParams &p, void *workspace);
 hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t stream);

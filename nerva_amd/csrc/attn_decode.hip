@@ -94,7 +94,7 @@ __global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
   const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);  // before anything they could queue behind
   const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
   if (p.cursor != nullptr && pos >= p.max_steps) return;
-  attn_fast_body<DT, G, W, false>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
+  attn_fast_body<DT, G, W>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, raw);
 }
 
 // Prompt-block launch of the same body (grid z = tokens): the lean variant, two workgroups per CU.
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams 
   __shared__ AttnShared<G, W> sh;
   if (blockIdx.z != 0 || p.seqs != nullptr) token_view(p, blockIdx.z);
   const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);
-  attn_fast_body<DT, G, W, false, 1>(p, p.position, blockIdx.x, blockIdx.y, gridDim.y, sh, AttnLink{}, raw);
+  attn_fast_body<DT, G, W, 1>(p, p.position, blockIdx.x, blockIdx.y, gridDim.y, sh, raw);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -147,6 +147,91 @@ __device__ __forceinline__ void sload4(const uint32_t *p0, const uint32_t *p1, c
       : "=&s"(v[0]), "=&s"(v[1]), "=&s"(v[2]), "=&s"(v[3])
       : "s"(p0), "s"(p1), "s"(p2), "s"(p3)
       : "memory");
+}
+
+// The splits' partials of the step kernel, as (f32 value, tag) words. One (head, split) record is cut
+// into kStepParts parts of 32 dims, each followed by its own copy of the split's m and l, so that a part
+// is read - and its tags cleared - by exactly one merging workgroup.
+constexpr uint32_t kStepParts = 4, kStepPartDims = kHD / kStepParts, kStepPartWords = kStepPartDims + 2;
+constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
+// One part (32 dims of one head) merged by one workgroup of 512 threads. Thread (dl = t % 32,
+// q = t / 32) takes the splits q, q + 16, q + 32, q + 48: it polls their accumulator word and their m
+// and l words until every tag is up and folds them in split order; the sixteen groups meet in LDS in
+// group order - a fixed order, whatever the arrival order was. A CU sustains only a few hundred
+// device-coherent cache lines per microsecond, which is why a head is spread over several merging
+// workgroups. Afterwards every word that was read gets its tag cleared for the next launch (launches
+// are ordered by the stream). A wait that runs out (a split that never stored: cannot happen on a
+// healthy device) ends after kMergeSpinLimit polls and the output is then not to be trusted.
+constexpr uint32_t kMergeSpinLimit = 1u << 20;
+template <uint32_t DT, int G>
+__device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t kvh, uint32_t g, uint32_t part, uint32_t S,
+                                                  uint32_t active, float *lds_o, float *lds_m, float *lds_l) {
+  constexpr uint32_t kGroups = 16, kPer = kAttnMaxSplits / kGroups;  // 4 splits per thread at most
+  const uint32_t h = kvh * G + g;
+  uint64_t *rec = p.part_tagged + static_cast<uint64_t>(h) * S * kStepRecord + part * kStepPartWords;
+  const uint32_t dl = threadIdx.x % kStepPartDims, q = threadIdx.x / kStepPartDims;
+  uint64_t av[kPer], mv[kPer], lv[kPer];
+  uint32_t spins = 0;
+  for (;;) {
+    bool ok = true;
+#pragma unroll
+    for (uint32_t i = 0; i < kPer; ++i) {
+      // unconditional loads (index clamped): a load under a branch would serialise the round
+      const uint64_t *r = rec + static_cast<uint64_t>(min(q + i * kGroups, active - 1)) * kStepRecord;
+      av[i] = load_tagged(r + dl);
+      mv[i] = load_tagged(r + kStepPartDims);
+      lv[i] = load_tagged(r + kStepPartDims + 1);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPer; ++i)  // (a clamped repeat of the last split belongs to another thread: not awaited)
+      if (q + i * kGroups < active) ok = ok && tag_is(av[i], 1u) && tag_is(mv[i], 1u) && tag_is(lv[i], 1u);
+    if (__all(ok) || ++spins > kMergeSpinLimit) break;
+  }
+  float M = -INFINITY, L = 0.0f, o = 0.0f;
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; ++i)
+    if (q + i * kGroups < active) M = fmaxf(M, tag_value(mv[i]));
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; ++i) {
+    if (q + i * kGroups < active) {
+      const float f = attn_exp2(tag_value(mv[i]) - M);  // every active split saw a key: its m is finite
+      L = fmaf(tag_value(lv[i]), f, L);
+      o = fmaf(tag_value(av[i]), f, o);
+    }
+  }
+  __syncthreads();  // the LDS arrays below were read by the wave merge (or by the previous part's merge)
+  // Every thread has taken what it needs: the words can be cleared for the next launch (a split's m and
+  // l words are read by all 32 threads of a group, so nobody may clear them before this barrier).
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; ++i) {
+    if (q + i * kGroups < active) {
+      uint64_t *r = rec + static_cast<uint64_t>(q + i * kGroups) * kStepRecord;
+      __hip_atomic_store(r + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (dl < 2) __hip_atomic_store(r + kStepPartDims + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  lds_o[q * kStepPartDims + dl] = o;
+  if (dl == 0) {
+    lds_m[q] = M;
+    lds_l[q] = L;
+  }
+  __syncthreads();
+  if (q == 0) {
+    float Mt = -INFINITY;
+#pragma unroll
+    for (uint32_t k = 0; k < kGroups; ++k) Mt = fmaxf(Mt, lds_m[k]);
+    float Lt = 0.0f, ot = 0.0f;
+#pragma unroll
+    for (uint32_t k = 0; k < kGroups; ++k) {
+      const float f = lds_m[k] > -INFINITY ? attn_exp2(lds_m[k] - Mt) : 0.0f;  // a group without a split
+      Lt = fmaf(lds_l[k], f, Lt);
+      ot = fmaf(lds_o[k * kStepPartDims + dl], f, ot);
+    }
+    if (Lt > 0.0f && isfinite(Lt)) ot /= Lt;
+    const uint32_t e = h * kHD + part * kStepPartDims + dl;
+    if (p.out_f32 != nullptr) p.out_f32[e] = ot;
+    p.out16[attn_out_elem(p, e)] = enc16<DT>(ot);
+  }
 }
 
 typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
@@ -417,31 +502,29 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
       if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
       p.out16[attn_out_elem(p, h * kHD + d)] = enc16<DT>(o);
     } else {
-      // The partial leaves through device-coherent stores (written through, no cache flush).
-      store_coherent(p.part_acc + (static_cast<uint64_t>(h) * S + split) * kHD + d, o);
-      if (d == 0) {
-        store_coherent(p.part_m + h * S + split, M);
-        store_coherent(p.part_l + h * S + split, L);
+      // The partial leaves as tagged words through device-coherent stores (written through, no cache
+      // flush, nobody waits for them to be performed).
+      const uint32_t part = d / kStepPartDims, dl = d % kStepPartDims;
+      uint64_t *rec = p.part_tagged + (static_cast<uint64_t>(h) * S + split) * kStepRecord + part * kStepPartWords;
+      store_tagged(rec + dl, o, 1u);
+      if (dl == 0) {
+        store_tagged(rec + kStepPartDims, M, 1u);
+        store_tagged(rec + kStepPartDims + 1, L, 1u);
       }
     }
   }
   if (active == 1) return;
-  // Every wave waits until its own stores have been performed, the barrier collects the waves,
-  // and only then one lane takes the arrival ticket of this kv head.
-  wait_stores_performed();
-  __syncthreads();
   link_mark(tr, 12);
-  if (threadIdx.x == 0) {
-    const uint32_t ticket = __hip_atomic_fetch_add(p.counters + kvh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    sh.is_last = ticket == active - 1 ? 1u : 0u;
+  // ---- 8. the splits' merge: part j = (head g, 32 dims) of this kv head is merged by split j (mod the
+  // active splits), which polls the other splits' words until every tag is up - two memory round
+  // trips after the slowest split's tiles (store, then the poll that finds it), where a ticket taken
+  // after the stores have been performed and a merge by the last arriver needed four.
+  for (uint32_t j = split; j < G * kStepParts; j += active) {
+    link_mark(trm, 16);
+    float *lds = sh.wacc[0][0];  // at least 1024 floats, free once the wave merge has been read
+    merge_part_tagged<DT, G>(p, kvh, j % G, j / G, S, active, lds, lds + 512, lds + 528);
+    link_mark(trm, 17);
   }
-  __syncthreads();
-  link_mark(tr, 13);
-  if (!sh.is_last) return;
-  link_mark(trm, 16);
-  merge_splits<DT, G, kThreads>(p, kvh, S, active, lane);
-  if (threadIdx.x == 0) __hip_atomic_store(p.counters + kvh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  link_mark(trm, 17);
 }
 #undef NV_AT_LD32
 #undef NV_AT_LD16
@@ -609,6 +692,7 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
       }
       return hipGetLastError();
     }
+    if (group != 8 && p.part_tagged == nullptr) return hipErrorInvalidValue;
     switch (group) {
       case 1: hipLaunchKernelGGL((attn_step_kernel<DT, 1>), grid, dim3(8 * kWave), 0, stream, p); break;
       case 2: hipLaunchKernelGGL((attn_step_kernel<DT, 2>), grid, dim3(8 * kWave), 0, stream, p); break;
@@ -624,6 +708,10 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
 }
 
 }  // namespace
+
+uint64_t attn_step_workspace_bytes(uint32_t heads) {
+  return static_cast<uint64_t>(heads) * kAttnMaxSplits * kStepRecord * sizeof(uint64_t);
+}
 
 uint64_t attn_workspace_bytes(uint32_t heads, uint32_t head_dim) {
   const uint64_t acc = static_cast<uint64_t>(heads) * kAttnMaxSplits * head_dim * sizeof(float);

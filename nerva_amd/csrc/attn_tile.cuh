@@ -274,17 +274,15 @@ struct AttnShared {
   float wf[W][G];   // exp(m_w - M_g), 0 for idle waves
   float bM[G];
   uint32_t is_last;
-  // linked launches: the query operand of the first product; m, l and exp(m - M) of the splits
-  alignas(16) uint4 qx_s[4][kWave];
-  float pm[G][kAttnMaxSplits], pl[G][kAttnMaxSplits], pf[G][kAttnMaxSplits];
+  alignas(16) uint4 qx_s[4][kWave];  // lean variant: the query operand of the first product
 };
 
 // ---- hand-over between workgroups of one launch ------------------------------------------
 // A value that another workgroup of the same launch consumes travels as one 8-byte word
-// (f32 value, epoch): the consumer polls the word with device-coherent loads until the epoch is
-// the current one. A single aligned 8-byte store is indivisible, so a matching epoch proves
-// the value; no flag, no "stores performed" wait, no cache flush is needed on either side.
-// Epochs (step counter x layers + layer + 1) never repeat within a session.
+// (f32 value, tag): the consumer polls the word with device-coherent loads until the tag is the
+// expected one. A single aligned 8-byte store is indivisible, so a matching tag proves the value;
+// no flag, no "stores performed" wait, no cache flush is needed on either side. The consumer
+// clears the tag once it has taken the value (launches are ordered by the stream).
 __device__ __forceinline__ void store_tagged(uint64_t *ptr, float v, uint32_t epoch) {
   __hip_atomic_store(ptr, (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(v), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
@@ -297,81 +295,8 @@ __device__ __forceinline__ bool tag_is(uint64_t word, uint32_t epoch) {
 }
 __device__ __forceinline__ float tag_value(uint64_t word) { return __uint_as_float(static_cast<uint32_t>(word)); }
 
-// The attention output travels as (two 16-bit values, epoch) words: element pair (2i, 2i + 1) in
-// word i. `bits` = this lane's rounded element; lanes with an even element index store.
-__device__ __forceinline__ void store_tagged_pair16(uint64_t *out_words, uint32_t elem, uint32_t bits, uint32_t epoch) {
-  const uint32_t next = static_cast<uint32_t>(__shfl_down(static_cast<int>(bits), 1, kWave));
-  if ((elem & 1u) == 0u)
-    __hip_atomic_store(out_words + elem / 2, (static_cast<uint64_t>(epoch) << 32) | bits | (next << 16),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-constexpr uint32_t kLinkSpinLimit = 1u << 20;
-// One more unsuccessful poll: true when the wait has to be given up (limit reached, or the
-// abort word is up); raises the abort word then. Pauses the wave briefly otherwise.
-__device__ __forceinline__ bool link_give_up(uint32_t *abort_flag, uint32_t &spins) {
-  ++spins;
-  if (spins > kLinkSpinLimit || ((spins & 15u) == 0u && load_coherent(abort_flag) != 0u)) {
-    store_coherent(abort_flag, 1u);
-    return true;
-  }
-  __builtin_amdgcn_s_sleep(2);
-  return false;
-}
-
-constexpr int kMergeRound = 16;            // splits polled per round by the merging workgroup
-constexpr uint32_t kPartRecord = kHD + 2;  // tagged words of one (head, split) partial: acc[128], m, l
-
-// Connections of an attention workgroup to the other roles of a fused launch.
-struct AttnLink {
-  const uint64_t *qkv_tagged;  // [A + 2 KV] q|k|v written by the qkv role of this launch, or null: p.qkv
-  uint64_t *part_tagged;       // [heads][splits][kPartRecord] split partials
-  uint64_t *out_tagged;        // [heads * 64] final output for the consumer role, two 16-bit elements per word
-  // hints for the consumers' cheap first wait: word [i * hint_stride + kvh] belongs to consumer
-  // workgroup i alone (a word polled by every consumer would make its memory channel the
-  // bottleneck of the whole launch); raised to `epoch` right before the output is stored
-  uint32_t *hints;
-  uint32_t hint_count, hint_stride;
-  uint32_t *split_hints;       // [kv_heads][kAttnMaxSplits] "this split's partial has been stored"
-  uint32_t *abort_flag;        // raised when a bounded wait ran out
-  uint32_t epoch;
-  uint64_t *trace;             // tuning aid: device timestamps of this workgroup's stages, or null
-  uint64_t *trace_merge;       // same for the workgroup that merges this kv head's splits
-};
-__device__ __forceinline__ void attn_raise_hints(const AttnLink &link, uint32_t kvh) {
-  for (uint32_t i = threadIdx.x; i < link.hint_count; i += blockDim.x)
-    store_coherent(link.hints + i * link.hint_stride + kvh, link.epoch);
-}
 __device__ __forceinline__ void link_mark(uint64_t *trace, int slot) {
   if (trace != nullptr && threadIdx.x == 0) trace[slot] = wall_clock64();
-}
-
-// Raw projection values (lane, lane + 64) of the 128-wide head that starts at element `off`.
-template <bool LINKED>
-__device__ __forceinline__ void load_head128(const float *qkv, const AttnLink &link, uint32_t off, int lane,
-                                             float &x0, float &x1) {
-  if constexpr (LINKED) {
-    if (link.qkv_tagged != nullptr) {
-      uint64_t r0, r1;
-      uint32_t spins = 0;
-      // a long wait: watch one word per wave (a single request), poll the whole head once it is there
-      while (!tag_is(load_tagged(link.qkv_tagged + off), link.epoch)) {
-        if (link_give_up(link.abort_flag, spins)) break;
-        __builtin_amdgcn_s_sleep(16);
-      }
-      for (;;) {
-        r0 = load_tagged(link.qkv_tagged + off + lane);
-        r1 = load_tagged(link.qkv_tagged + off + lane + 64);
-        if (__all(tag_is(r0, link.epoch) && tag_is(r1, link.epoch))) break;
-        if (link_give_up(link.abort_flag, spins)) break;
-      }
-      x0 = tag_value(r0);
-      x1 = tag_value(r1);
-      return;
-    }
-  }
-  x0 = qkv[off + lane];
-  x1 = qkv[off + lane + 64];
 }
 
 // Everything a wave needs to prepare its heads - raw projections of its query heads
@@ -504,15 +429,10 @@ __device__ __forceinline__ void merge_splits(const AttnParams &p, uint32_t kvh, 
 // accumulators are indexed by the same column, so m, l and the rescale never cross lanes.
 // The cache stores tiles in operand order (kv_k_elem / kv_v_elem): every load is one coalesced
 // 1 KiB instruction and lands in the registers the matrix core reads.
-//
-// LINKED = the workgroup is the attention role of a launch that also holds its producer and/or
-// consumer (AttnLink). Its first tile is requested before it polls for q/k/v; partials and the
-// final output leave as tagged words; split 0 of a kv head merges (it polls the other splits'
-// partials instead of taking a ticket), so nobody waits for stores to be performed.
-template <uint32_t DT, int G, int W, bool LINKED, int IN_FLIGHT = (LINKED ? 1 : 4)>
+template <uint32_t DT, int G, int W, int IN_FLIGHT = 4>
 __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32_t pos, const uint32_t kvh,
                                                const uint32_t split, const uint32_t S, AttnShared<G, W> &sh,
-                                               const AttnLink &link, const RawHeads<G, W> &raw) {
+                                               const RawHeads<G, W> &raw) {
   constexpr int kThreads = W * kWave;
   auto &q_s = sh.q_s;
   auto &knew = sh.knew;
@@ -526,8 +446,8 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform: block-table reads stay scalar
   // tuning aid: stage timestamps of workgroup (kv head 0, split 0) and of kv head 0's merging workgroup
-  uint64_t *const tr = LINKED ? link.trace : (kvh == 0 && split == 0 ? p.trace : nullptr);
-  uint64_t *const trm = LINKED ? link.trace_merge : (kvh == 0 ? p.trace : nullptr);
+  uint64_t *const tr = kvh == 0 && split == 0 ? p.trace : nullptr;
+  uint64_t *const trm = kvh == 0 ? p.trace : nullptr;
   const uint32_t n_keys = pos + 1;
   const uint32_t nblk = (n_keys + kKvBlockTokens - 1) / kKvBlockTokens;
   // at least W tiles per active split so that every wave of a workgroup has work
@@ -556,39 +476,14 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
 #pragma unroll
   for (int f = 0; f < kInFlight; ++f) phys[f] = p.table[min(b + f * W, nblk - 1)];
   // the head inputs requested at kernel start have to be in registers before the tiles go out
-  if constexpr (!LINKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int f = 0; f < kInFlight; ++f)
     if (b + f * W < b1) attn_load_tile(p, phys[f], kvh, lane, kreg[f], vreg[f]);
 
   link_mark(tr, 8);
   // ---- q (all workgroups) and the new K/V row (the workgroup whose range holds pos)
-  if constexpr (LINKED) {
-#pragma unroll
-    for (int i = 0; i < (G + W - 1) / W; ++i) {
-      const int g = wave + i * W;
-      if (g < G) {
-        const uint32_t h = kvh * G + g;
-        float x0, x1;
-        load_head128<LINKED>(p.qkv, link, h * kHD, lane, x0, x1);
-        prep_head128<DT>(x0, x1, p.q_bias ? p.q_bias + h * kHD : nullptr, p.q_norm, p.rope_freq, p.rope_cs, pos,
-                         p.eps, lane, q_s[g], nullptr);
-      }
-    }
-    if (owns_new) {
-      if (wave == (G % W)) {
-        float x0, x1;
-        load_head128<LINKED>(p.qkv, link, A + kvh * kHD, lane, x0, x1);
-        prep_head128<DT>(x0, x1, p.k_bias ? p.k_bias + kvh * kHD : nullptr, p.k_norm, p.rope_freq, p.rope_cs, pos,
-                         p.eps, lane, nullptr, knew);
-      } else if (wave == ((G + 1) % W)) {
-        float x0, x1;
-        load_head128<LINKED>(p.qkv, link, A + KV + kvh * kHD, lane, x0, x1);
-        prep_head128<DT>(x0, x1, p.v_bias ? p.v_bias + kvh * kHD : nullptr, nullptr, nullptr, nullptr, pos, p.eps,
-                         lane, nullptr, vnew);
-      }
-    }
-  } else {
+  {
     // every input is in registers already: pure arithmetic while the tiles are in flight
     const bool has_rope = p.rope_freq != nullptr;
     float rc = raw.rope_a, rs = raw.rope_b;
@@ -718,14 +613,6 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
       if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
       const uint16_t o16 = enc16<DT>(o);
       p.out16[attn_out_elem(p, h * kHD + d)] = o16;
-      if constexpr (LINKED) store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
-    } else if constexpr (LINKED) {
-      uint64_t *rec = link.part_tagged + (static_cast<uint64_t>(h) * S + split) * kPartRecord;
-      store_tagged(rec + d, o, link.epoch);
-      if (d == 0) {
-        store_tagged(rec + kHD, bM[g], link.epoch);
-        store_tagged(rec + kHD + 1, L, link.epoch);
-      }
     } else {
       // The partial leaves through device-coherent stores (written through, no cache flush).
       store_coherent(p.part_acc + (static_cast<uint64_t>(h) * S + split) * kHD + d, o);
@@ -735,108 +622,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
       }
     }
   }
-  if (active == 1) {
-    if constexpr (LINKED) {
-      attn_raise_hints(link, kvh);
-    }
-    return;
-  }
-  if constexpr (LINKED) {
-    // ---- split 0 merges: every thread owns one output element (g, d) and polls that element of
-    // every split's partial, kMergeRound splits per round; the first G * active threads also fetch the
-    // splits' m and l. Whatever has not arrived yet is simply polled again.
-    static_assert(!LINKED || G * kHD == kThreads, "one output element per thread");
-    // Tell the merging workgroup that this split's partial is in place: once the stores have
-    // been performed one word is raised. It is a hint (the tags decide), but a reliable one.
-    wait_stores_performed();
-    __syncthreads();
-    if (threadIdx.x == 0) store_coherent(link.split_hints + kvh * kAttnMaxSplits + split, link.epoch);
-    link_mark(tr, 12);
-    if (split != 0) return;
-    link_mark(trm, 16);
-    if (wave == 0) {
-      uint32_t spins = 0;
-      for (;;) {
-        const bool mine = static_cast<uint32_t>(lane) >= active ||
-                          load_coherent(link.split_hints + kvh * kAttnMaxSplits + lane) == link.epoch;
-        if (__all(mine)) break;
-        if (link_give_up(link.abort_flag, spins)) break;
-      }
-    }
-    __syncthreads();
-    link_mark(trm, 18);
-    const int g = threadIdx.x / kHD, d = threadIdx.x % kHD;
-    const uint32_t h = kvh * G + g;
-    const uint64_t *rec = link.part_tagged + static_cast<uint64_t>(h) * S * kPartRecord;
-    const bool has_ml = threadIdx.x < G * active;
-    const uint32_t g2 = has_ml ? threadIdx.x / active : 0u, s2 = has_ml ? threadIdx.x % active : 0u;
-    const uint64_t *rec_ml = link.part_tagged + (static_cast<uint64_t>(kvh * G + g2) * S + s2) * kPartRecord + kHD;
-    float o = 0.0f, L = 0.0f;
-    for (uint32_t s0 = 0; s0 < active; s0 += kMergeRound) {
-      // First through the ordinary load path: the splits of a kv head run on the XCD of the merging
-      // workgroup when workgroups are dealt to XCDs round robin and kv_heads is a multiple of the XCD
-      // count, so their written-through partials are current in the L2 these loads go to, and
-      // ordinary loads are many times faster than device-coherent ones (which this CU can only keep
-      // a few of in flight). The tags tell when that did not hold: then the round is polled again
-      // with device-coherent loads, which are right wherever the writers ran.
-      // Every load of a round is unconditional (indices past the last split are clamped to it):
-      // a load under a branch makes the compiler wait for all earlier loads at the join, which
-      // would turn the round into sixteen round trips in a row.
-      uint64_t av[kMergeRound], mv, lv;
-      bool ok = true;
-#pragma unroll
-      for (int i = 0; i < kMergeRound; ++i)
-        av[i] = rec[static_cast<uint64_t>(min(s0 + i, active - 1)) * kPartRecord + d];
-      mv = rec_ml[0];
-      lv = rec_ml[1];
-#pragma unroll
-      for (int i = 0; i < kMergeRound; ++i) ok = ok & tag_is(av[i], link.epoch);
-      ok = ok & tag_is(mv, link.epoch) & tag_is(lv, link.epoch);
-      uint32_t spins = 0;
-      while (!__all(ok)) {
-        if (link_give_up(link.abort_flag, spins)) break;
-#pragma unroll
-        for (int i = 0; i < kMergeRound; ++i)
-          av[i] = load_tagged(rec + static_cast<uint64_t>(min(s0 + i, active - 1)) * kPartRecord + d);
-        mv = load_tagged(rec_ml);
-        lv = load_tagged(rec_ml + 1);
-        ok = true;
-#pragma unroll
-        for (int i = 0; i < kMergeRound; ++i) ok = ok & tag_is(av[i], link.epoch);
-        ok = ok & tag_is(mv, link.epoch) & tag_is(lv, link.epoch);
-      }
-      if (link.trace_merge != nullptr && threadIdx.x == 0) {
-        link.trace_merge[s0 == 0 ? 19 : 5] = wall_clock64();
-        link.trace_merge[s0 == 0 ? 6 : 7] = spins + 1;  // raw count (debugging aid)
-      }
-      if (s0 == 0) {
-        if (has_ml) {
-          sh.pm[g2][s2] = tag_value(mv);
-          sh.pl[g2][s2] = tag_value(lv);
-        }
-        __syncthreads();
-        if (has_ml) {
-          float M = -INFINITY;
-          for (uint32_t s = 0; s < active; ++s) M = fmaxf(M, sh.pm[g2][s]);
-          sh.pf[g2][s2] = attn_exp2(sh.pm[g2][s2] - M);  // every active split saw at least one key: m is finite
-        }
-        __syncthreads();
-        for (uint32_t s = 0; s < active; ++s) L = fmaf(sh.pl[g][s], sh.pf[g][s], L);
-      }
-#pragma unroll
-      for (int i = 0; i < kMergeRound; ++i)
-        if (s0 + i < active) o = fmaf(tag_value(av[i]), sh.pf[g][s0 + i], o);
-    }
-    if (L > 0.0f && isfinite(L)) o /= L;
-    // pollers of the output may start now: it follows within one store latency
-    attn_raise_hints(link, kvh);
-    if (p.out_f32 != nullptr) p.out_f32[h * kHD + d] = o;
-    const uint16_t o16 = enc16<DT>(o);
-    p.out16[attn_out_elem(p, h * kHD + d)] = o16;
-    store_tagged_pair16(link.out_tagged, h * kHD + d, o16, link.epoch);
-    link_mark(trm, 17);
-    return;
-  }
+  if (active == 1) return;
   // Every wave waits until its own stores have been performed, the barrier collects the waves,
   // and only then one lane takes the arrival ticket of this kv head.
   wait_stores_performed();

@@ -117,6 +117,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
   void *attn_ws = nullptr, *sample_ws = nullptr;
   uint32_t attn_splits = 1;
+  uint64_t *attn_tagged = nullptr;   // tagged split partials of the decode step kernel
   uint32_t *attn_plan = nullptr;     // this step's split plan of the decode attention (attn_plan_fill), or null
   // persistent layer-chain kernel (o + gate/up + down + next qkv in one launch)
   bool chain = false;
@@ -405,6 +406,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       // (a pass of attention launches alone - profiling - follows full steps at the same position, whose
       // embedding launch left the plan of that position)
       p.plan = s->attn_plan;
+      p.part_tagged = s->attn_tagged;
       NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
       snap(s->attn16, static_cast<uint64_t>(A) * sizeof(uint16_t));
     }
@@ -1033,6 +1035,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t attn_ws_bytes = attn_workspace_bytes(s->heads, s->head_dim);
   const uint64_t off_attn_ws = c.take(attn_ws_bytes);
   const uint64_t off_attn_plan = c.take(attn_plan_bytes(kAttnMaxSplits));
+  const uint64_t off_attn_tagged = c.take(attn_step_workspace_bytes(s->heads));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
   const uint64_t pT = kGemmMaxTokens;
   const uint64_t off_px = c.take(pT * H * 4);
@@ -1106,6 +1109,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->rope_freq = reinterpret_cast<float *>(s->arena + off_rope);
   s->rope_cs = reinterpret_cast<float *>(s->arena + off_rope_cs);
   s->attn_ws = s->arena + off_attn_ws;
+  s->attn_tagged = reinterpret_cast<uint64_t *>(s->arena + off_attn_tagged);
   {
     // the plan serves the step kernel (head_dim 128, 1, 2 or 4 query heads per kv head, 8 waves)
     const uint32_t group = s->kv_heads != 0 ? s->heads / s->kv_heads : 0;
@@ -1171,6 +1175,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   }
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_ws, 0, attn_ws_bytes, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_plan, 0, attn_plan_bytes(kAttnMaxSplits), s->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_tagged, 0, attn_step_workspace_bytes(s->heads), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);

@@ -375,7 +375,9 @@ int nerva_hip_fp8_gemv(const NervaHipFp8GemvRequest *r, void *stream, int32_t *h
 }
 
 uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim) {
-  return attn_workspace_bytes(heads, head_dim) + static_cast<uint64_t>(head_dim) * sizeof(float);
+  // split workspace, RoPE frequency table (256-byte slot), tagged partials of the decode step kernel
+  return attn_workspace_bytes(heads, head_dim) + ((static_cast<uint64_t>(head_dim) * sizeof(float) + 255u) & ~uint64_t{255}) +
+         attn_step_workspace_bytes(heads);
 }
 
 uint64_t nerva_hip_kv_cache_offset(uint32_t block_count, uint32_t kv_heads, uint32_t head_dim,
@@ -398,6 +400,8 @@ int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *r, void *str
   p.kv_heads = r->kv_heads;
   p.head_dim = r->head_dim;
   attn_bind_workspace(p, r->workspace);
+  p.part_tagged = reinterpret_cast<uint64_t *>(static_cast<char *>(r->workspace) + attn_workspace_bytes(r->heads, r->head_dim) +
+                                               ((static_cast<uint64_t>(r->head_dim) * sizeof(float) + 255u) & ~uint64_t{255}));
   float *rope_table =
       reinterpret_cast<float *>(static_cast<char *>(r->workspace) + attn_workspace_bytes(r->heads, r->head_dim));
   if (r->rope_theta > 0.0f) {
