@@ -160,7 +160,7 @@ def main():
     t0 = time.perf_counter()
     rc, res, tokens = session.advance(args.steps)
     elapsed = time.perf_counter() - t0
-    eager = os.environ.get("NERVA_HIP_EAGER_STEPS") == "1"   # kernel-tracing mode, see decode_session.hip
+    eager = N.Device.steps_are_eager()   # kernel-tracing mode (asked for, or a profiler is attached)
     assert rc == 0 and res.observed_tokens == args.steps and (eager or res.graph_replays == args.steps)
     assert res.hot_path_allocations == 0 and N.Device.allocation_count() == allocs
     tok_s = args.steps / elapsed

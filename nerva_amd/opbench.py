@@ -53,8 +53,9 @@ def timed(enqueue, launches, warmup=3, replays=10):
     lib = abi.load()
     enqueue(0)                       # untimed: primes lazily built tables
     Device.synchronize()
-    if os.environ.get("NERVA_OPBENCH_EAGER") == "1":
-        # kernel-tracing mode: plain launches (a profiler reports the per-kernel durations)
+    if os.environ.get("NERVA_OPBENCH_EAGER") == "1" or Device.steps_are_eager():
+        # kernel-tracing mode (asked for, or a profiler is attached): plain launches, the profiler
+        # reports the per-kernel durations
         t0 = time.perf_counter()
         for i in range(launches):
             enqueue(i)
@@ -113,8 +114,8 @@ def case_mlp():
     return rows_out
 
 
-def case_attention():
-    heads, kvh, hd, tokens = 32, 8, 128, 4096
+def case_attention(tokens=4096, label="3 paged GQA attention, 4097 keys"):
+    heads, kvh, hd = 32, 8, 128
     layers, blocks = 64, tokens // 16 + 1
     rng = np.random.default_rng(3)
     table = rng.permutation(blocks).astype(np.uint32)
@@ -133,8 +134,21 @@ def case_attention():
         ns = timed(lambda i: R.paged_attention(BF16, heads, kvh, hd, cache, i % n, tokens, qkv, ws, out16,
                                                out_f32=out32, append=True, rope_theta=1e6, q_norm=qn, k_norm=kn,
                                                sync=False), 128)
-        rows_out[variant] = report("3 paged GQA attention, 4097 keys", variant, ns, nbytes)
+        rows_out[variant] = report(label, variant, ns, nbytes)
     return rows_out
+
+
+def case_attention_8k():
+    """The decode step's attention at the bench's context (8192 cached tokens + the new one)."""
+    return case_attention(8192, "paged GQA attention, 8193 keys")
+
+
+def case_copy_probe(mib=256):
+    """One plain device copy of known size: the launch a counter run reads its byte scale from."""
+    src, dst = (DeviceBuffer.zeros(mib << 20) for _ in range(2))
+    Device.copy(dst, src, mib << 20)
+    Device.synchronize()
+    log("copy probe: %d MiB read, %d MiB written by one plain_copy_kernel launch" % (mib, mib))
 
 
 def case_moe():
@@ -242,7 +256,8 @@ def main():
         print("no usable GPU (hip_error=%d): these operators have no CPU path" % smoke.hip_error, file=sys.stderr)
         sys.exit(1)
     log("device: %s" % smoke.gpu_name.decode())
-    cases = dict(qproj=case_qproj, mlp=case_mlp, attention=case_attention, moe=case_moe, fp8_gemv=case_fp8_gemv,
+    cases = dict(qproj=case_qproj, mlp=case_mlp, attention=case_attention, attention_8k=case_attention_8k, copy_probe=case_copy_probe,
+                 moe=case_moe, fp8_gemv=case_fp8_gemv,
                  sampler=case_sampler,
                  gemm_rows=case_gemm_rows)
     for name, case in cases.items():      # `python -m nerva_amd.opbench gemm_rows sampler` runs only those

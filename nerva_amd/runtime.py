@@ -32,6 +32,12 @@ class Device:
         return int(abi.load().nerva_hip_allocation_count())
 
     @staticmethod
+    def steps_are_eager():
+        """True when sessions launch a step's kernels one by one instead of replaying the captured
+        graph: asked for through NERVA_HIP_EAGER_STEPS=1, or forced because a profiler is attached."""
+        return bool(abi.load().nerva_hip_steps_are_eager())
+
+    @staticmethod
     def copy(dst, src, nbytes):
         """Plain device copy kernel of a known size (memory-counter calibration)."""
         if abi.load().nerva_hip_copy_d2d(dst.ptr, src.ptr, nbytes, None) != 0:
