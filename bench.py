@@ -28,9 +28,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one gate_up launch moves at the Qwen3-8B shape (24576x4096 bf16): FETCH_SIZE + WRITE_SIZE
 # per dispatch from two `rocprofv3 --pmc` runs, each scaled by what the counter reads for a plain
 # 256 MiB copy kernel (profiles/gate_up_gemv_hbm_traffic_pmc.txt). Not measurable in-process.
-GATE_UP_TRAFFIC_BYTES = {(4096, 12288): 201709978}
-# Same for one launch of the persistent layer-chain kernel (filled in from its counter profile).
-CHAIN_TRAFFIC_BYTES = {}
+# Keyed to the launch shape the figure was measured for - (hidden, intermediate, kernel variant,
+# workgroups) as nerva_hip_gemv_launch_shape reports them - so that a changed plan reports null
+# instead of a stale number.
+GATE_UP_TRAFFIC_BYTES = {(4096, 12288, 3, 2048): 201709978}
 SEED = 0x4E45525641
 WEIGHT_STD = 0.02
 
@@ -176,26 +177,17 @@ def main():
     rc, prof = session.profile_step(3)
     assert rc == 0
     per_kind = {}
-    chain = bool(prof.chain_enabled)
-    if chain:
-        kinds = ("qkv", "attention", "chain", "lm_head")
-    else:
-        kinds = ("qkv", "attention", "o", "gate_up", "down", "lm_head")
+    kinds = ("qkv", "attention", "o", "gate_up", "down", "lm_head")
     for k in kinds:
         paired = getattr(prof, k + "_ns")
         ns = getattr(prof, k + "_stream_ns", 0) or paired
         per_kind[k] = (ns, getattr(prof, k + "_bytes"))
         log("[profile] %-9s %8.2f us (event pair per launch %8.2f us)  %7.1f GB/s  (%.1f%% of HBM peak)" % (
             k, ns / 1e3, paired / 1e3, per_kind[k][1] / max(ns, 1), 100 * per_kind[k][1] / max(ns, 1) / HBM_PEAK_GBS))
-    if chain:
-        dom_ns, dom_bytes = per_kind["chain"]
-        dom_name = ("decode_chain_kernel<bf16>: o 4096x4096 + gate_up 24576x4096 + down 4096x12288 + next qkv 6144x4096 "
-                    "as phases of one persistent launch")
-        traffic = CHAIN_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"]))
-    else:
-        dom_ns, dom_bytes = per_kind["gate_up"]
-        dom_name = "gemv_fast_kernel<bf16, rmsnorm prologue, swiglu epilogue> (gate_up 24576x4096)"
-        traffic = GATE_UP_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"]))
+    dom_ns, dom_bytes = per_kind["gate_up"]
+    dom_name = "gemv_fast_kernel<bf16, rmsnorm prologue, swiglu epilogue> (gate_up 24576x4096)"
+    traffic = GATE_UP_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"]) + N.gemv_launch_shape(
+        1, 2, cfg["intermediate"], cfg["hidden"]))
     roofline = dict(bound="hbm", kernel=dom_name,
                     achieved=round(dom_bytes / dom_ns, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(dom_bytes / dom_ns / HBM_PEAK_GBS, 4), traffic=traffic,

@@ -774,10 +774,6 @@ pub struct NervaHipStepProfile {
     pub o_stream_ns: u64,
     pub gate_up_stream_ns: u64,
     pub down_stream_ns: u64,
-    pub chain_ns: u64,
-    pub chain_stream_ns: u64,
-    pub chain_bytes: u64,
-    pub chain_enabled: u32,
 }
 
 unsafe extern "C" {
@@ -795,6 +791,7 @@ unsafe extern "C" {
     pub fn nerva_hip_projection_bench(request: *const NervaHipProjectionBenchRequest, out: *mut NervaHipProjectionBenchResult) -> c_int;
     pub fn nerva_hip_deepseek_moe_forward(request: *const NervaHipDeepSeekMoeForwardRequest, out: *mut NervaHipDeepSeekMoeForwardResult) -> c_int;
     pub fn nerva_hip_gemv(request: *const NervaHipGemvRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
+    pub fn nerva_hip_gemv_launch_shape(prologue: u32, epilogue: u32, rows: u32, cols: u32, kernel: *mut u32, workgroups: *mut u32) -> c_int;
     pub fn nerva_hip_fp8_gemv(request: *const NervaHipFp8GemvRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_paged_gqa_decode(request: *const NervaHipPagedAttentionRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_paged_attention_workspace_bytes(heads: u32, head_dim: u32) -> u64;
@@ -825,7 +822,7 @@ unsafe extern "C" {
     pub fn nerva_hip_synth_fill_fp8_block(device_weights: *mut c_void, device_scales: *mut c_void, seed: u64, tensor_id: u64, rows: u64, cols: u64, block: u64, std: f32) -> c_int;
     pub fn nerva_hip_bench_session_create_synthetic(request: *const NervaHipHfDecodeSequenceSessionCreateRequest, seed: u64, weight_std: f32, with_qk_norm: u32, out: *mut NervaHipHfDecodeSequenceSessionCreateResult, session: *mut *mut NervaHipHfDecodeSequenceSession) -> c_int;
     pub fn nerva_hip_session_profile_step(session: *mut NervaHipHfDecodeSequenceSession, repeats: u32, out: *mut NervaHipStepProfile) -> c_int;
-    pub fn nerva_hip_session_fused_state(session: *mut NervaHipHfDecodeSequenceSession, raise_abort: u32, mode: *mut u32, aborted: *mut u32) -> c_int;
+    pub fn nerva_hip_test_set_tuning(name: *const c_char, value: i32) -> c_int;
     pub fn nerva_hip_steps_are_eager() -> c_int;
     pub fn nerva_hip_session_shares_weight_stream(session: *mut NervaHipHfDecodeSequenceSession) -> c_int;
     pub fn nerva_hip_session_read_logits(session: *mut NervaHipHfDecodeSequenceSession, host_logits: *mut f32) -> c_int;

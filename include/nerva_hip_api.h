@@ -471,6 +471,13 @@ typedef struct NervaHipGemvRequest {
  * decode step (device_ops.cuh:317-332, kernels.cu:577-612,651-668). */
 int nerva_hip_gemv(const NervaHipGemvRequest *request, void *stream, int32_t *hip_error);
 
+/* The launch shape nerva_hip_gemv (and the session's step) chooses for a request of these sizes with
+ * 16-byte-aligned pointers: *kernel = 0 scalar, 1 guarded vector, 2 full vector, 3 the lean
+ * production-shape kernel; *workgroups = the grid. Host arithmetic only (no device is touched):
+ * measurements taken for one launch shape (counter profiles) are keyed to it. No counterpart. */
+int nerva_hip_gemv_launch_shape(uint32_t prologue, uint32_t epilogue, uint32_t rows, uint32_t cols,
+                                uint32_t *kernel, uint32_t *workgroups);
+
 typedef struct NervaHipFp8GemvRequest {
   uint32_t rows, cols, block_rows, block_cols;
   uint32_t input_dtype;      /* dtype of input16 */
@@ -695,11 +702,6 @@ typedef struct NervaHipStepProfile {
   /* average device ns per launch when the `layers` launches of one kind run back to back
    * between a single hipEvent pair (no per-launch event gap): the kernel's own duration */
   uint64_t qkv_stream_ns, attention_stream_ns, o_stream_ns, gate_up_stream_ns, down_stream_ns;
-  /* persistent layer-chain launch (o + gate/up + down + next layer's qkv as phases of one kernel):
-   * when chain_enabled is 1 the o/gate_up/down figures above are zero and qkv counts the first
-   * layer's stand-alone launch only */
-  uint64_t chain_ns, chain_stream_ns, chain_bytes;
-  uint32_t chain_enabled;
 } NervaHipStepProfile;
 
 /* Runs `repeats` decode steps eagerly at the session's current cursor WITHOUT
@@ -709,17 +711,13 @@ typedef struct NervaHipStepProfile {
 int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uint32_t repeats,
                                    NervaHipStepProfile *out);
 
-/* Kernels of a session that hand data between workgroups inside one launch. *mode says which
- * the session's shapes and switches selected: the persistent layer-chain kernel
- * (NERVA_HIP_CHAIN=1 where the shapes fit), or none. *aborted = 1 when one of its bounded in-kernel
- * waits ran out (the calls that covered those steps returned -1 with hip_error =
- * hipErrorLaunchFailure; start() clears it). raise_abort != 0 sets the abort word from the host
- * first, which makes every such wait give up at once: the failure path can be exercised while
- * all kernels still terminate normally. */
-#define NERVA_HIP_FUSED_NONE 0u
-#define NERVA_HIP_FUSED_CHAIN 1u
-int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *session, uint32_t raise_abort,
-                                  uint32_t *mode, uint32_t *aborted);
+/* Test and measurement hook (no counterpart): overrides one launch-shape choice for the whole process;
+ * value 0 restores the built-in choice. Names: "attn_splits" (split-KV factor of a session's decode
+ * attention, read when a session is created), "batch_splits", "prompt_splits" (the batch step's and the
+ * prompt blocks' attention), "gemm_row_tiles" (1|2), "gemm_k_waves" (8|4), "gemm_block_slices",
+ * "gemm_block_row_tiles" (1|2), "gemm_block_min_tokens" (the multi-row projections). Values a kernel
+ * cannot take are ignored where they are read. -1 for an unknown name. */
+int nerva_hip_test_set_tuning(const char *name, int32_t value);
 
 /* 1 when this process launches its steps kernel by kernel instead of replaying captured graphs:
  * NERVA_HIP_EAGER_STEPS=1, or the ROCm profiler's environment was found at the first call (a traced

@@ -15,7 +15,7 @@ OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libnerva_hip.so")
 
 SOURCES = ["gemv_stream.hip", "fp8_gemv.hip", "attn_decode.hip", "attn_prompt.hip", "argmax.hip", "synth_fill.hip",
-           "decode_chain.hip", "sampler.hip", "gemm_rows.hip", "gemm_block.hip", "op_entry.hip", "decode_session.hip"]
+           "sampler.hip", "gemm_rows.hip", "gemm_block.hip", "op_entry.hip", "decode_session.hip"]
 
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # packed fp32 VALU ops are kept off for every device function of this library

@@ -161,7 +161,8 @@ constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
 // device-coherent cache lines per microsecond, which is why a head is spread over several merging
 // workgroups. Afterwards every word that was read gets its tag cleared for the next launch (launches
 // are ordered by the stream). A wait that runs out (a split that never stored: cannot happen on a
-// healthy device) ends after kMergeSpinLimit polls and the output is then not to be trusted.
+// healthy device) ends after kMergeSpinLimit polls and the outputs it feeds become NaN: a failure that
+// shows in the logits instead of a plausible wrong number.
 constexpr uint32_t kMergeSpinLimit = 1u << 20;
 template <uint32_t DT, int G>
 __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t kvh, uint32_t g, uint32_t part, uint32_t S,
@@ -187,6 +188,7 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
       if (q + i * kGroups < active) ok = ok && tag_is(av[i], 1u) && tag_is(mv[i], 1u) && tag_is(lv[i], 1u);
     if (__all(ok) || ++spins > kMergeSpinLimit) break;
   }
+  const bool gave_up = spins > kMergeSpinLimit;  // per wave; poisons the outputs this wave contributes to
   float M = -INFINITY, L = 0.0f, o = 0.0f;
 #pragma unroll
   for (uint32_t i = 0; i < kPer; ++i)
@@ -210,7 +212,7 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
       if (dl < 2) __hip_atomic_store(r + kStepPartDims + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  lds_o[q * kStepPartDims + dl] = o;
+  lds_o[q * kStepPartDims + dl] = gave_up ? NAN : o;
   if (dl == 0) {
     lds_m[q] = M;
     lds_l[q] = L;

@@ -28,7 +28,6 @@
 
 #include "argmax.cuh"
 #include "attn_decode.cuh"
-#include "decode_chain.cuh"
 #include "gemm_rows.cuh"
 #include "sampler.cuh"
 #include "gemv_stream.cuh"
@@ -47,7 +46,7 @@ struct LayerDev {
 };
 
 enum StepMode { kDecodeStep = 0, kPromptStep = 1, kPromptHeadStep = 2 };
-enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLChain, kLKinds };
+enum LaunchKind { kLEmbed = 0, kLQkv, kLAttn, kLO, kLGateUp, kLDown, kLHead, kLAdvance, kLKinds };
 
 // The weight arena of a session and of every session forked from it (one stream of the weights can
 // then serve a token row of each of them); freed by the last of them to go.
@@ -119,10 +118,6 @@ struct NervaHipHfDecodeSequenceSession {
   uint32_t attn_splits = 1;
   uint64_t *attn_tagged = nullptr;   // tagged split partials of the decode step kernel
   uint32_t *attn_plan = nullptr;     // this step's split plan of the decode attention (attn_plan_fill), or null
-  // persistent layer-chain kernel (o + gate/up + down + next qkv in one launch)
-  bool chain = false;
-  uint32_t *chain_flags = nullptr, *chain_abort = nullptr;
-  uint64_t *chain_trace = nullptr;  // NERVA_HIP_CHAIN_TRACE=1: per-layer timestamps of workgroup 0
   uint64_t *attn_trace = nullptr;  // NERVA_HIP_ATTN_TRACE=1: per-layer stage timestamps of selected attention workgroups
   Slot *host_slots = nullptr;
   uint32_t *host_prompt = nullptr;
@@ -361,7 +356,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   }
   for (uint32_t l = 0; l < s->layers; ++l) {
     const LayerDev &w = s->layer[l];
-    if (!s->chain || l == 0) {
+    {
       GemvParams p{};
       p.w = w.wqkv;
       p.xf = s->x;
@@ -409,37 +404,6 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.part_tagged = s->attn_tagged;
       NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
       snap(s->attn16, static_cast<uint64_t>(A) * sizeof(uint16_t));
-    }
-    if (s->chain) {
-      // o projection, gate/up, down and the next layer's qkv projection as one persistent launch
-      ChainParams c{};
-      c.wo = w.wo;
-      c.o_bias = w.o_bias;
-      c.rms_mlp = w.rms_mlp;
-      c.wgu = w.wgu;
-      c.wdown = w.wdown;
-      c.rms_next = l + 1 < s->layers ? s->layer[l + 1].rms_attn : nullptr;
-      c.wqkv_next = l + 1 < s->layers ? s->layer[l + 1].wqkv : nullptr;
-      c.attn16 = s->attn16;
-      c.x = s->x;
-      c.r = s->r;
-      c.ff16 = s->ff16;
-      c.qkv = s->qkv;
-      c.hidden = s->hidden;
-      c.attn_dim = A;
-      c.inter = s->intermediate;
-      c.qkv_rows = A + 2 * KV;
-      c.eps = s->eps;
-      c.round_out = mode == kDecodeStep ? 0u : 1u;
-      c.flags = s->chain_flags;
-      c.abort_flag = s->chain_abort;
-      c.cursor = s->state;
-      c.max_steps = s->max_ctx;
-      c.barrier_base = kChainMaxBarriers * l;
-      c.barriers_per_step = kChainMaxBarriers * s->layers;
-      c.trace = s->chain_trace != nullptr ? s->chain_trace + 32 * l : nullptr;
-      NV_STEP(kLChain, launch_decode_chain(s->dtype, c, st));
-      continue;
     }
     {
       GemvParams p{};
@@ -561,7 +525,6 @@ bool eager_steps() {
 uint64_t step_launches(const Session *s, int which) {
   // embed + (lm head + greedy finish | lm head + two sampler launches | cursor advance)
   const uint64_t fixed = which == 1 ? 2 : (s->sampler.mode == kSamplerGreedy ? 3 : 4);
-  if (s->chain) return fixed + 1 + 2ull * s->layers;
   return fixed + 5ull * s->layers;
 }
 
@@ -687,16 +650,6 @@ bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
   return true;
 }
 
-// After a synchronisation: did a bounded wait of the chain kernel run out during the steps
-// just completed? Their tokens are then not to be trusted and the call fails.
-hipError_t chain_verdict(Session *s) {
-  if (!s->chain) return hipSuccess;
-  uint32_t aborted = 0;
-  const hipError_t err = hipMemcpy(&aborted, s->chain_abort, sizeof(aborted), hipMemcpyDeviceToHost);
-  if (err != hipSuccess) return err;
-  return aborted != 0 ? hipErrorLaunchFailure : hipSuccess;
-}
-
 hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t prompt_count,
                           NervaHipHfDecodeSequenceResult *out) {
   // Not on the per-token path: the prompt is copied synchronously (the caller's buffer may be
@@ -707,8 +660,6 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
                     hipMemcpyHostToDevice);
   if (err == hipSuccess)
     err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
-  // the chain kernel's barrier epochs grow with the position: a new sequence starts them over
-  if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count);
     err = hipGetLastError();
@@ -749,11 +700,10 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
     const char *v = getenv("NERVA_HIP_PREFILL_ATTN");
     return v != nullptr && v[0] == 'r';
   }();
-  static const uint32_t prompt_splits = [] {
-    const char *v = getenv("NERVA_HIP_PROMPT_SPLITS");   // tuning knob: split factor of the prompt attention
-    const long want = v != nullptr ? strtol(v, nullptr, 10) : 0;
-    return want >= 1 && want <= static_cast<long>(kAttnMaxSplits) ? static_cast<uint32_t>(want) : 0u;
-  }();
+  const int want_prompt_splits = tuning(kTunePromptSplits);
+  const uint32_t prompt_splits = want_prompt_splits >= 1 && want_prompt_splits <= static_cast<int>(kAttnMaxSplits)
+                                     ? static_cast<uint32_t>(want_prompt_splits)
+                                     : 0u;
   for (uint32_t first = 0; err == hipSuccess && first < count; first += kGemmMaxTokens) {
     const uint32_t T = std::min<uint32_t>(kGemmMaxTokens, count - first);
     const uint32_t tiles = block_operand_tiles(T);
@@ -1009,11 +959,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint32_t block_count = (s->max_ctx + kKvBlockTokens - 1) / kKvBlockTokens;
   s->block_count = block_count;
   s->attn_splits = attn_default_splits(s->kv_heads, block_count);
-  if (const char *v = getenv("NERVA_HIP_ATTN_SPLITS")) {  // tuning knob: split-KV factor of the stand-alone attention
-    const long want = strtol(v, nullptr, 10);
-    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits))
-      s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
-  }
+  if (const int want = tuning(kTuneAttnSplits); want >= 1 && want <= static_cast<int>(kAttnMaxSplits))
+    s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
 
   Carver c;
   const uint64_t kv_half = L * block_count * KV * kKvBlockTokens * 2;
@@ -1051,8 +998,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_pgemm_ws = c.take(pgemm_ws_bytes);
   const uint64_t off_sampler_dev = c.take(sizeof(SamplerDev));
   const uint64_t off_sampler_keys = c.take(sampler_workspace_bytes(s->vocab));
-  const uint64_t off_chain = c.take(chain_flag_bytes() + 256);  // arrival flags, then the abort word
-  const uint64_t off_chain_trace = c.take(L * 32 * 8);
+  const uint64_t off_attn_trace = c.take(L * 32 * 8);
   {
     // Prompt blocks and batch steps need the matrix-core attention (head_dim 128, GQA factor
     // 1/2/4/8) and shapes the multi-row kernels take.
@@ -1137,26 +1083,10 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   }
   s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
   s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
-  s->chain_flags = reinterpret_cast<uint32_t *>(s->arena + off_chain);
-  s->chain_abort = reinterpret_cast<uint32_t *>(s->arena + off_chain + chain_flag_bytes());
-  {
-    // NERVA_HIP_CHAIN=1 runs o + gate/up + down + next qkv as one persistent launch per layer.
-    // Off by default: measured on MI355X it is about 4 % slower per step than one launch per
-    // GEMV (the in-kernel grid barriers cost as much as the kernel boundaries they replace, and
-    // a static split of the rows over 256 workgroups waits longer for its slowest member).
-    const char *want_chain = getenv("NERVA_HIP_CHAIN");
-    s->chain = want_chain != nullptr && want_chain[0] == '1' && s->layers > 0 &&
-               chain_supported(s->hidden, s->heads * s->head_dim, s->intermediate,
-                               (s->heads + 2 * s->kv_heads) * s->head_dim) &&
-               chain_prepare(s->dtype) == hipSuccess;
-    const char *trace = getenv("NERVA_HIP_CHAIN_TRACE");
-    if (s->chain && trace != nullptr && trace[0] == '1')
-      s->chain_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);
-  }
   {
     const char *trace = getenv("NERVA_HIP_ATTN_TRACE");
-    if (!s->chain && s->layers > 0 && trace != nullptr && trace[0] == '1')
-      s->attn_trace = reinterpret_cast<uint64_t *>(s->arena + off_chain_trace);  // the chain kernel is off then
+    if (s->layers > 0 && trace != nullptr && trace[0] == '1')
+      s->attn_trace = reinterpret_cast<uint64_t *>(s->arena + off_attn_trace);
   }
 
   *failure_stage = 5;
@@ -1177,9 +1107,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_plan, 0, attn_plan_bytes(kAttnMaxSplits), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_attn_tagged, 0, attn_step_workspace_bytes(s->heads), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_sample_ws, 0, sample_workspace_bytes(), s->stream);
-  if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_chain, 0, chain_flag_bytes() + 256, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_pattn_ws, 0, pT * pattn_ws_stride, s->stream);
-  if (err == hipSuccess && L > 0) err = hipMemsetAsync(s->arena + off_chain_trace, 0, L * 32 * 8, s->stream);
+  if (err == hipSuccess && L > 0) err = hipMemsetAsync(s->arena + off_attn_trace, 0, L * 32 * 8, s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->arena + off_kc, 0, 2 * ((kv_half + 255) & ~uint64_t{255}), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
   if (err == hipSuccess) err = hipMemsetAsync(s->state, 0, 64, s->stream);
@@ -1526,10 +1455,8 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
   // one workgroup per CU
   uint32_t batch_splits = std::max<uint32_t>(1u, std::min<uint32_t>(attn_default_splits(lead->kv_heads, min_blocks),
                                                                    (256u + lead->kv_heads * T - 1) / (lead->kv_heads * T)));
-  if (const char *v = getenv("NERVA_HIP_BATCH_SPLITS")) {
-    const long want = strtol(v, nullptr, 10);
-    if (want >= 1 && want <= static_cast<long>(kAttnMaxSplits)) batch_splits = std::min<uint32_t>(static_cast<uint32_t>(want), min_blocks);
-  }
+  if (const int want = tuning(kTuneBatchSplits); want >= 1 && want <= static_cast<int>(kAttnMaxSplits))
+    batch_splits = std::min<uint32_t>(static_cast<uint32_t>(want), min_blocks);
   hipError_t err = hipMemcpyAsync(lead->btable, host, sizeof(BatchTable), hipMemcpyHostToDevice, st);
   if (err != hipSuccess) return err;
   if (lead->dtype == kBF16)
@@ -1715,8 +1642,6 @@ int nerva_hip_hf_decode_sequence_session_fork_shared_weights(
     copy(s->kc, parent->kc, kv_half);
     copy(s->vc, parent->vc, kv_half);
     copy(s->sampler_dev, parent->sampler_dev, sizeof(SamplerDev));
-    // the chain kernel's barrier epochs continue from where the sequence stands
-    if (s->chain && parent->chain) copy(s->chain_flags, parent->chain_flags, chain_flag_bytes());
     s->sampler = parent->sampler;
     s->prompt_count = parent->prompt_count;
     s->has_eos = parent->has_eos;
@@ -1871,12 +1796,6 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
         err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
                              q->stream);
       out->d2h_bytes += sizeof(Slot);
-      // A chain step keeps one workgroup resident on every CU and its workgroups wait for each other:
-      // two of them must never share the machine, so such sessions run one after the other.
-      if (err == hipSuccess && q->chain) {
-        err = hipStreamSynchronize(q->stream);
-        out->sync_calls += 1;
-      }
       out->pack_kernel_launches += 1;
       out->projection_kernel_launches += 4ull * q->layers + 1;
       out->dependency_kernel_launches += q->layers;
@@ -1885,7 +1804,6 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
     for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
       err = hipStreamSynchronize(seqs[t]->stream);
       out->sync_calls += 1;
-      if (err == hipSuccess) err = chain_verdict(seqs[t]);
     }
   }
   out->hot_path_allocations = allocation_count() - allocs_before;
@@ -2052,7 +1970,6 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
     err = hipStreamSynchronize(s->stream);
     out->sync_calls += 1;
   }
-  if (err == hipSuccess) err = chain_verdict(s);
   out->hot_path_allocations = allocation_count() - allocs_before;
   if (err == hipSuccess && run_count != 0) {
     float ms = 0.0f;
@@ -2121,7 +2038,6 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
     err = hipStreamSynchronize(s->stream);
     out->sync_calls += 1;
   }
-  if (err == hipSuccess) err = chain_verdict(s);
   out->hot_path_allocations = allocation_count() - allocs_before;
   if (err == hipSuccess) {
     float ms = 0.0f;
@@ -2219,9 +2135,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {  // first pass is a warm-up
     prof.used = 0;
     prof.kinds.clear();
-    // the step is repeated at one position: the chain kernel's barrier epochs must start over
-    err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
-    if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, &prof);
+    err = enqueue_step(s, kDecodeStep, &prof);
     if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
     // undo the step: cursor and the published slot
     if (err == hipSuccess) err = hipMemcpy(s->state, &pos, 4, hipMemcpyHostToDevice);
@@ -2246,18 +2160,13 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   // back-to-back pass: all `layers` launches of one kind between a single event pair, so the
   // figure is the kernel's own duration without the per-launch event gaps
   uint64_t stream_ns[kLKinds] = {0};
-  for (int kind = kLQkv; err == hipSuccess && kind <= kLChain; ++kind) {
-    uint32_t launches = s->layers;
-    if (kind == kLHead || kind == kLAdvance) continue;
-    if (kind == kLQkv && s->chain) launches = 1;
-    if ((kind == kLO || kind == kLGateUp || kind == kLDown) && s->chain) continue;
-    if (kind == kLChain && !s->chain) continue;
+  for (int kind = kLQkv; err == hipSuccess && kind <= kLDown; ++kind) {
+    const uint32_t launches = s->layers;
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
       // no embed launch in this pass: advance the step counter here
       hipLaunchKernelGGL(bump_step_counter_kernel, dim3(1), dim3(64), 0, s->stream, s->state);
       err = hipGetLastError();
-      if (err == hipSuccess) err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
       if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
       if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
       if (err == hipSuccess) err = hipEventRecord(s->ev1, s->stream);
@@ -2271,17 +2180,6 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     return -1;
-  }
-  if (s->chain_trace != nullptr) {
-    std::vector<uint64_t> tr(static_cast<size_t>(s->layers) * 32);
-    if (hipMemcpy(tr.data(), s->chain_trace, tr.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-      for (uint32_t l = 0; l < s->layers && l < 3; ++l) {
-        const uint64_t *t = tr.data() + 32 * l;
-        fprintf(stderr, "[chain trace] layer %u (10 ns ticks from the first barrier B):", l);
-        for (int i = 0; i < 22; ++i) fprintf(stderr, " %lld", static_cast<long long>(t[i]) - static_cast<long long>(t[1]));
-        fprintf(stderr, "\n");
-      }
-    }
   }
   if (s->attn_trace != nullptr) {
     // timestamps (10 ns ticks from the launch's earliest mark) of: qkv workgroup 0 [0..3] and the last
@@ -2305,10 +2203,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
       }
     }
   }
-  // leave no epochs of this position behind: the sequence will run the step at `pos` for real
-  err = hipMemsetAsync(s->chain_flags, 0, chain_flag_bytes(), s->stream);
-  if (err == hipSuccess) err = hipStreamSynchronize(s->stream);
-  if (err == hipSuccess) err = chain_verdict(s);
+  err = hipStreamSynchronize(s->stream);
   if (err != hipSuccess) {
     out->hip_error = static_cast<int32_t>(err);
     return -1;
@@ -2318,7 +2213,6 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->o_stream_ns = stream_ns[kLO];
   out->gate_up_stream_ns = stream_ns[kLGateUp];
   out->down_stream_ns = stream_ns[kLDown];
-  out->chain_stream_ns = stream_ns[kLChain];
   auto avg = [&](int k) { return counts[k] ? sums[k] / counts[k] : 0; };
   out->position = pos;
   out->embed_ns = avg(kLEmbed);
@@ -2328,7 +2222,6 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_ns = avg(kLGateUp);
   out->down_ns = avg(kLDown);
   out->lm_head_ns = avg(kLHead);
-  out->chain_ns = avg(kLChain);
   out->total_ns = total / repeats;
   const uint64_t H = s->hidden, A = static_cast<uint64_t>(s->heads) * s->head_dim,
                  KV = static_cast<uint64_t>(s->kv_heads) * s->head_dim, I = s->intermediate, V = s->vocab;
@@ -2339,27 +2232,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
   out->gate_up_bytes = 2 * I * H * 2 + H * 4 + H * 2 + I * 2;
   out->down_bytes = H * I * 2 + I * 2 + H * 4 + H * 4;
   out->lm_head_bytes = V * H * 2 + H * 4 + H * 2 + V * 4;
-  // chain launch of a middle layer: o + gate/up + down + next qkv (the activations between them
-  // stay on the device and are counted once, as the phase that reads them)
-  out->chain_bytes = s->chain ? out->o_bytes + out->gate_up_bytes + out->down_bytes + out->qkv_bytes : 0;
-  out->chain_enabled = s->chain ? 1u : 0u;
   out->status = 0;
-  return 0;
-}
-
-int nerva_hip_session_fused_state(NervaHipHfDecodeSequenceSession *s, uint32_t raise_abort, uint32_t *mode,
-                                  uint32_t *aborted) {
-  if (s == nullptr) return -1;
-  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
-  const bool fused = s->chain;
-  if (raise_abort != 0 && fused) {
-    const uint32_t one = 1;
-    if (hipMemcpy(s->chain_abort, &one, sizeof(one), hipMemcpyHostToDevice) != hipSuccess) return -1;
-  }
-  uint32_t flag = 0;
-  if (fused && hipMemcpy(&flag, s->chain_abort, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  if (mode) *mode = s->chain ? NERVA_HIP_FUSED_CHAIN : NERVA_HIP_FUSED_NONE;
-  if (aborted) *aborted = flag;
   return 0;
 }
 
@@ -2386,7 +2259,7 @@ int nerva_hip_session_trace_next_step(NervaHipHfDecodeSequenceSession *s, void *
     return 0;
   }
   if (bytes < nerva_hip_session_step_trace_bytes(s)) return -1;
-  if (s->chain || s->sampler.mode != kSamplerGreedy) return -1;  // the launch-per-piece greedy step only
+  if (s->sampler.mode != kSamplerGreedy) return -1;  // the greedy step only
   s->trace_buf = static_cast<char *>(device_buffer);
   s->trace_used = 0;
   return 0;

@@ -373,11 +373,6 @@ hipError_t launch_block_dt(int epilogue, const GemmRowsParams &p, const GemmBloc
   }
 }
 
-int env_int(const char *name) {
-  const char *v = getenv(name);
-  return v != nullptr ? atoi(v) : 0;
-}
-
 }  // namespace
 
 GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
@@ -386,12 +381,9 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
     const char *v = getenv("NERVA_HIP_GEMM_BLOCK");   // 0: never use the shared-X kernel
     return v != nullptr && v[0] == '0' ? 0 : 1;
   }();
-  static const int want_slices = env_int("NERVA_HIP_GEMM_BLOCK_SLICES");   // tuning: K slices for every projection
-  static const int want_tiles = env_int("NERVA_HIP_GEMM_BLOCK_ROW_TILES"); // tuning: 1 or 2 row tiles per wave
-  static const uint32_t min_tokens = [] {
-    const int v = env_int("NERVA_HIP_GEMM_BLOCK_MIN_TOKENS");   // tuning: smallest block this kernel takes
-    return v > 0 ? static_cast<uint32_t>(v) : 17u;
-  }();
+  const int want_slices = tuning(kTuneGemmBlockSlices);
+  const int want_tiles = tuning(kTuneGemmBlockRowTiles);
+  const uint32_t min_tokens = tuning(kTuneGemmBlockMinTokens) > 0 ? static_cast<uint32_t>(tuning(kTuneGemmBlockMinTokens)) : 17u;
   if (mode == 0 || tokens < min_tokens || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (kBRing * kBK) != 0) return plan;
   const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
   // Row tiles per wave: two where that still leaves a workgroup for most CUs.

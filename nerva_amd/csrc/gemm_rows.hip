@@ -266,17 +266,11 @@ hipError_t launch_dt(int epilogue, const GemmRowsParams &p, hipStream_t stream) 
   // enough token rows for the X traffic to matter. Measured on MI355X at T = 1 / 8 / 32 (one tile vs
   // two, microseconds): LM head 151936x4096 198 / 223 / 383 vs 207 / 218 / 314; qkv 6144x4096
   // 12.4 / 14.1 / 23.6 vs 14.7 / 15.3 / 20.1; o and down (4096 rows: 128 workgroups with two tiles) lose.
-  static const int forced = [] {
-    const char *v = getenv("NERVA_HIP_GEMM_ROW_TILES");   // tuning knob: 1 or 2 for every plain projection
-    return v != nullptr && (v[0] == '1' || v[0] == '2') ? v[0] - '0' : 0;
-  }();
+  const int forced = tuning(kTuneGemmRowTiles) == 1 || tuning(kTuneGemmRowTiles) == 2 ? tuning(kTuneGemmRowTiles) : 0;
   const bool two = forced != 0 ? forced == 2
                                : (p.rows >= 32u * kTwoTileMinWorkgroups ? p.tokens >= 8 : (p.tokens > 16 && p.rows >= 32u * 192u));
   const bool can_two = p.rows >= 32 && !(epilogue == kGemmResidual && p.rows % 32 != 0 && p.residual == p.out_f32);
-  static const int forced_kw = [] {
-    const char *v = getenv("NERVA_HIP_GEMM_K_WAVES");   // tuning knob: 8 or 4 waves along K
-    return v != nullptr && (v[0] == '4' || v[0] == '8') ? v[0] - '0' : 0;
-  }();
+  const int forced_kw = tuning(kTuneGemmKWaves) == 4 || tuning(kTuneGemmKWaves) == 8 ? tuning(kTuneGemmKWaves) : 0;
   // Four waves along K (two row groups per workgroup): measured at T = 1 / 8 / 32 against eight, LM head
   // 202 / 208 / 299 vs 199 / 219 / 315 us; gate_up 39.8 / 41.9 / 60.1 vs 36.5 / 38.3 / 53.1, down and o
   // lose more (half the workgroups). So: only for matrices with thousands of row tiles.

@@ -109,6 +109,21 @@ __device__ __forceinline__ Best wave_best(Best b) {
   return b;
 }
 
+// Launch-shape overrides for measurements and tests, set through nerva_hip_test_set_tuning (0 = the
+// built-in choice). The product path never reads the environment for these.
+enum TuningKnob : int {
+  kTuneAttnSplits = 0,       // split-KV factor of a session's decode attention (read at session create)
+  kTuneBatchSplits,          // split factor of the batch step's attention
+  kTunePromptSplits,         // split factor of the prompt-block attention
+  kTuneGemmRowTiles,         // multi-row GEMM: 1 or 2 row tiles per wave for every plain projection
+  kTuneGemmKWaves,           // multi-row GEMM: 8 or 4 waves along K
+  kTuneGemmBlockSlices,      // shared-X GEMM: K slices for every projection
+  kTuneGemmBlockRowTiles,    // shared-X GEMM: 1 or 2 row tiles per wave
+  kTuneGemmBlockMinTokens,   // shared-X GEMM: smallest token block it takes
+  kTuneKnobs
+};
+int tuning(TuningKnob knob);
+
 // 16-byte streaming load that does not pollute the caches with single-use weights.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 load_stream(const void *p) {

@@ -2,6 +2,7 @@
 // (FP8 matvec, f32 MoE forward, projection bench). The decode session lives in
 // decode_session.hip.
 #include <math.h>
+#include <string.h>
 
 #include <algorithm>
 #include <atomic>
@@ -25,7 +26,13 @@ namespace {
 std::atomic<uint64_t> g_allocations{0};
 std::once_flag g_stream_once;
 hipStream_t g_stream = nullptr;
+std::atomic<int> g_tuning[kTuneKnobs];
+constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_splits",       "prompt_splits",
+                                                  "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
+                                                  "gemm_block_row_tiles", "gemm_block_min_tokens"};
 }  // namespace
+
+int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }
 
 bool device_ready(int32_t *hip_error) {
   int count = 0;
@@ -333,6 +340,26 @@ int nerva_hip_synth_fill_fp8_block(void *device_weights, void *device_scales, ui
       hipSuccess)
     return -1;
   return hipStreamSynchronize(s) == hipSuccess ? 0 : -1;
+}
+
+int nerva_hip_test_set_tuning(const char *name, int32_t value) {
+  if (name == nullptr) return -1;
+  for (int k = 0; k < kTuneKnobs; ++k) {
+    if (strcmp(name, kTuningNames[k]) == 0) {
+      g_tuning[k].store(value, std::memory_order_relaxed);
+      return 0;
+    }
+  }
+  return -1;
+}
+
+int nerva_hip_gemv_launch_shape(uint32_t prologue, uint32_t epilogue, uint32_t rows, uint32_t cols, uint32_t *kernel,
+                                uint32_t *workgroups) {
+  if (prologue > 1 || epilogue > 4 || rows == 0 || cols == 0) return -1;
+  const GemvPlan plan = gemv_plan(static_cast<int>(prologue), static_cast<int>(epilogue), rows, cols, true, nullptr);
+  if (kernel) *kernel = static_cast<uint32_t>(plan.mode);
+  if (workgroups) *workgroups = plan.blocks;
+  return 0;
 }
 
 int nerva_hip_gemv(const NervaHipGemvRequest *r, void *stream, int32_t *hip_error) {

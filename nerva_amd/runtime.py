@@ -32,6 +32,13 @@ class Device:
         return int(abi.load().nerva_hip_allocation_count())
 
     @staticmethod
+    def set_tuning(name, value):
+        """Overrides one launch-shape choice for the process (0 restores the built-in one): a hook for
+        measurements and tests, see nerva_hip_test_set_tuning."""
+        if abi.load().nerva_hip_test_set_tuning(name.encode(), int(value)) != 0:
+            raise ValueError("unknown tuning name %r" % name)
+
+    @staticmethod
     def steps_are_eager():
         """True when sessions launch a step's kernels one by one instead of replaying the captured
         graph: asked for through NERVA_HIP_EAGER_STEPS=1, or forced because a profiler is attached."""
@@ -126,6 +133,14 @@ def gemv(dtype, weights, rows, cols, *, input16=None, input_f32=None, gamma=None
     _check(abi.load().nerva_hip_gemv(C.byref(req), None, C.byref(err)), err, "nerva_hip_gemv")
     if sync:
         Device.synchronize()
+
+
+def gemv_launch_shape(prologue, epilogue, rows, cols):
+    """(kernel variant, workgroups) of the launch nerva_hip_gemv chooses for these sizes (host arithmetic)."""
+    kernel, groups = C.c_uint32(0), C.c_uint32(0)
+    if abi.load().nerva_hip_gemv_launch_shape(prologue, epilogue, rows, cols, C.byref(kernel), C.byref(groups)) != 0:
+        raise ValueError("no launch shape for these sizes")
+    return int(kernel.value), int(groups.value)
 
 
 def fp8_gemv(weights, scales, rows, cols, block_rows, block_cols, out, *, input16=None, input_f32=None,

@@ -278,17 +278,6 @@ class DecodeSession:
         rc = self.lib.nerva_hip_session_profile_step(self.handle, repeats, C.byref(res))
         return rc, res
 
-    FUSED_NONE, FUSED_CHAIN = 0, 1
-
-    def fused_state(self, raise_abort=False):
-        """(mode, aborted) of the kernel that hands data between workgroups inside a launch (the layer
-        chain); raise_abort sets the abort word so that its bounded waits give up."""
-        mode, aborted = C.c_uint32(0), C.c_uint32(0)
-        rc = self.lib.nerva_hip_session_fused_state(self.handle, int(raise_abort), C.byref(mode), C.byref(aborted))
-        if rc != 0:
-            raise RuntimeError("fused_state failed")
-        return int(mode.value), bool(aborted.value)
-
     def traced_advance(self):
         """advance(1) with the step's intermediates read back (nerva_hip_session_trace_next_step).
 

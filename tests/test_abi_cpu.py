@@ -291,3 +291,27 @@ def test_profiled_processes_never_replay_graphs():
         env.update(extra)
         out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True)
         assert out.returncode == 0 and out.stdout.strip() == want, (extra, out.stdout, out.stderr)
+
+
+def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
+    """The GEMV launch shape is decided on the host (measurements are keyed to it), and launch-shape
+    overrides go through a named hook, not through the environment."""
+    import nerva_amd as N
+    # the decode step's launches at Qwen3-8B widths: every one the lean kernel
+    assert N.gemv_launch_shape(1, 2, 12288, 4096) == (3, 2048)     # gate_up: oversubscribed long launch
+    assert N.gemv_launch_shape(1, 0, 6144, 4096) == (3, 768)       # qkv: two rows per wave in one round
+    assert N.gemv_launch_shape(0, 1, 4096, 4096) == (3, 1024)      # o: every row on the machine at once
+    assert N.gemv_launch_shape(1, 4, 151936, 4096)[0] == 3         # LM head
+    assert N.gemv_launch_shape(0, 0, 100, 520)[0] == 1             # 520 columns: the guarded vector kernel
+    with pytest.raises(ValueError):
+        N.gemv_launch_shape(0, 0, 0, 64)
+    for name in ("attn_splits", "batch_splits", "prompt_splits", "gemm_row_tiles", "gemm_k_waves",
+                 "gemm_block_slices", "gemm_block_row_tiles", "gemm_block_min_tokens"):
+        N.Device.set_tuning(name, 2)
+        N.Device.set_tuning(name, 0)
+    with pytest.raises(ValueError):
+        N.Device.set_tuning("NERVA_HIP_ATTN_SPLITS", 2)
+    csrc = os.path.join(ROOT, "nerva_amd", "csrc")
+    src = "".join(open(os.path.join(csrc, f)).read() for f in os.listdir(csrc) if f.endswith((".hip", ".cuh", ".hpp")))
+    for knob in ("_SPLITS", "_ROW_TILES", "_K_WAVES", "_SLICES", "_MIN_TOKENS"):
+        assert knob + '")' not in src, knob    # no getenv("NERVA_HIP_..._SPLITS") and the like

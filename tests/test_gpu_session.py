@@ -316,43 +316,13 @@ GEOMETRIES = [
     (F16, 256, 4, 2, 64, 520, 300, 2, 1e4, True, False),       # generic attention path, guarded GEMV
     (BF16, 96, 6, 2, 16, 200, 50, 2, 0, False, False),         # group 3, no RoPE, cols % 8 == 0 only
     (F16, 512, 4, 1, 128, 1024, 1000, 3, 1e6, True, False),    # fast attention path in f16
-    (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False), # shapes the persistent chain kernel accepts
+    (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False), # 2048-wide, group 4: the lean GEMV kernel on every projection
     (F16, 2048, 16, 16, 128, 2048, 700, 2, 1e4, False, True),  # same in f16, MHA, o bias
 ]
 
 
-STEP_MODES = {
-    # id: (NERVA_HIP_CHAIN, fused_state mode of a session whose shapes fit)
-    "launch-per-piece": (None, N.DecodeSession.FUSED_NONE),         # the default
-    "chain-kernel": ("1", N.DecodeSession.FUSED_CHAIN),
-}
-
-
-def set_step_mode(monkeypatch, name):
-    chain, _ = STEP_MODES[name]
-    for var, val in (("NERVA_HIP_CHAIN", chain),):
-        if val is None:
-            monkeypatch.delenv(var, raising=False)
-        else:
-            monkeypatch.setenv(var, val)
-
-
-def mode_fits(name, hidden, heads, kv, hd):
-    """Whether a session of these shapes actually takes the kernels the mode asks for."""
-    if name == "launch-per-piece":
-        return True
-    return hidden % 2048 == 0
-
-
-@pytest.fixture(params=list(STEP_MODES), ids=list(STEP_MODES))
-def step_mode(request, monkeypatch):
-    """Sessions created inside the test build their step from these kernels when the shapes fit."""
-    set_step_mode(monkeypatch, request.param)
-    return request.param
-
-
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_single_layer_short_prompt_is_tight(geom, step_mode):
+def test_single_layer_short_prompt_is_tight(geom):
     """One layer and a 1- or 2-token prompt leave no room for 16-bit ties to compound: the whole
     step (embed, norms, GEMVs, RoPE, attention, LM head) must agree with the oracle at 1e-3 in
     f16. In bf16 a single value that sits within 1e-6 of a rounding boundary (attention output,
@@ -360,12 +330,9 @@ def test_single_layer_short_prompt_is_tight(geom, step_mode):
     one activation by 2^-8 relative and the logits of this tiny model by up to ~3e-3: the bound
     is one such flip, 6e-3."""
     dtype, hidden, heads, kv, hd, inter, vocab, _, theta, qk_norm, bias = geom
-    if not mode_fits(step_mode, hidden, heads, kv, hd):
-        pytest.skip("shapes do not fit this mode's kernels: same path as launch-per-piece")
     tol = REL_L2 if dtype == F16 else 6e-3
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, 1, hidden + 1, theta, qk_norm, bias)
     s = N.DecodeSession.create(weights, 32)
-    assert s.fused_state() == (STEP_MODES[step_mode][1], False)
     for prompt in ([3], [vocab - 1, 11]):
         ctx = O.Context(omodel, 32, staging=1)
         for i, t in enumerate(prompt):
@@ -390,10 +357,8 @@ def test_single_layer_short_prompt_is_tight(geom, step_mode):
 
 
 @pytest.mark.parametrize("geom", GEOMETRIES)
-def test_session_matches_oracle_logits_kv_and_stream(geom, step_mode):
+def test_session_matches_oracle_logits_kv_and_stream(geom):
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
-    if not mode_fits(step_mode, hidden, heads, kv, hd):
-        pytest.skip("shapes do not fit this mode's kernels: same path as launch-per-piece")
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, hidden, theta, qk_norm, bias)
     prompt = np.random.default_rng(1).integers(0, vocab, 21).astype(np.uint32)
     steps = 24
@@ -468,6 +433,30 @@ def test_eager_profile_pass_leaves_state_untouched():
     s.destroy()
 
 
+def test_session_split_factor_override_changes_only_the_summation_order():
+    """The split-KV factor of a session's decode attention is a launch-shape choice: sessions created
+    under the override hook with 1, 3 and 64 splits of a 700-token context give the default session's
+    logits up to the order in which the splits' partial sums meet, and the same greedy tokens."""
+    weights, omodel = random_model(BF16, 512, 4, 1, 128, 1024, 500, 2, 6)
+    prompt = np.random.default_rng(8).integers(0, 500, 700).astype(np.uint32)
+    runs = {}
+    try:
+        for splits in (0, 1, 3, 64):
+            N.Device.set_tuning("attn_splits", splits)
+            s = N.DecodeSession.create(weights, 768)
+            rc, res = s.start(prompt)
+            assert rc == 0
+            rc, res, toks = s.advance(6)
+            assert rc == 0 and res.graph_replays == 5
+            runs[splits] = (toks.tolist(), s.logits())
+            s.destroy()
+    finally:
+        N.Device.set_tuning("attn_splits", 0)
+    for splits in (1, 3, 64):
+        assert runs[splits][0] == runs[0][0], splits
+        assert rel_l2(runs[splits][1], runs[0][1]) <= chain_budget(2), splits
+
+
 def test_synthetic_session_matches_oracle_weights():
     """Device-generated weights (benchmark path) equal the oracle's generator bit for bit, so the
     CPU baseline can rebuild the same model on the host."""
@@ -493,63 +482,6 @@ def test_synthetic_session_matches_oracle_weights():
     rc, res, tokens = s.advance(8)
     assert rc == 0
     assert_stream_follows_oracle(omodel, prompt, tokens, 64)
-    s.destroy()
-
-
-CHAIN_GEOM = (BF16, 2048, 16, 4, 128, 4096, 1000, 3, 1e6, True, False)
-
-
-def test_chain_kernel_is_used_and_agrees_with_one_launch_per_gemv(monkeypatch):
-    """Shapes that fit take the persistent layer-chain kernel (o + gate/up + down + next qkv in one
-    launch). Its dot products are summed in the same order as the stand-alone GEMV kernels; only
-    the RMSNorm sum of squares is grouped differently (one wave instead of four), so logits agree
-    to 16-bit-tie noise and the greedy streams of this model are identical."""
-    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = CHAIN_GEOM
-    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 77, theta, qk_norm, bias)
-    prompt = np.random.default_rng(2).integers(0, vocab, 19).astype(np.uint32)
-    monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
-    s = N.DecodeSession.create(weights, 64)
-    assert s.fused_state() == (s.FUSED_CHAIN, False)
-    rc, res = s.start(prompt)
-    assert rc == 0
-    rc, res, chained = s.advance(12)
-    assert rc == 0 and res.graph_nodes == 4 + 2 * layers and res.hot_path_allocations == 0
-    logits_chain = s.logits()
-    rc, prof = s.profile_step(2)
-    assert rc == 0 and prof.chain_enabled == 1 and prof.launches == 4 + 2 * layers
-    assert prof.chain_ns > 0 and prof.chain_stream_ns > 0 and prof.o_ns == 0 and prof.chain_bytes > 0
-    rc, res, more = s.advance(4)                      # profiling did not disturb the sequence
-    assert rc == 0
-    s.destroy()
-    monkeypatch.delenv("NERVA_HIP_CHAIN")
-    s = N.DecodeSession.create(weights, 64)
-    assert s.fused_state() == (s.FUSED_NONE, False)
-    s.start(prompt)
-    rc, res, plain = s.advance(12)
-    assert rc == 0 and res.graph_nodes == 3 + 5 * layers
-    assert rel_l2(logits_chain, s.logits()) <= E2E_REL_L2
-    rc, res, more_plain = s.advance(4)
-    assert chained.tolist() == plain.tolist() and more.tolist() == more_plain.tolist()
-    s.destroy()
-
-
-def test_chain_kernel_bounded_wait_gives_up_cleanly(monkeypatch):
-    """With the abort word raised from the host every in-kernel wait gives up at once: all kernels
-    still run to completion, the call reports the failure, and start() makes the session usable."""
-    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = CHAIN_GEOM
-    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 78, theta, qk_norm, bias)
-    monkeypatch.setenv("NERVA_HIP_CHAIN", "1")
-    s = N.DecodeSession.create(weights, 32)
-    rc, res = s.start([1, 2, 3])
-    rc, res, good = s.advance(3)
-    assert rc == 0
-    assert s.fused_state(raise_abort=True) == (s.FUSED_CHAIN, True)
-    rc, res, _ = s.advance(2)
-    assert rc == -1 and res.status == -1 and res.hip_error != 0
-    rc, res = s.start([1, 2, 3])                      # a new sequence clears the abort word
-    assert rc == 0 and s.fused_state() == (s.FUSED_CHAIN, False)
-    rc, res, again = s.advance(3)
-    assert rc == 0 and again.tolist() == good.tolist()
     s.destroy()
 
 
