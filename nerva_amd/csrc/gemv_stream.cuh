@@ -399,7 +399,12 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
 constexpr int fast_waves_per_simd(int prologue) { return prologue == kProRmsNorm ? 5 : 6; }
 constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per lane
 
-template <uint32_t DT, int PRO, int EPI, int NR, int B>
+// EXACT (short launches: a wave's whole share is the two batches requested up front, so the start-up is
+// the launch): the first two batches and the residual element are requested unconditionally - a wave
+// without a row asks for the last row's data and drops it - so that the compiler can count the requests
+// behind the activation loads and waits for exactly those before the prologue, which then runs under
+// the weights' latency. With the requests under `if (total > n)` it waits for everything.
+template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false>
 __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
   extern __shared__ __align__(16) uint16_t xs[];
   __shared__ float red[kWavesPerBlock];
@@ -444,7 +449,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
   }
 
   // ---- 2. weight request state + the first two batches
-  uint32_t iu = wave_global, ib = 0;  // next batch to request: unit, batch within the row
+  uint32_t iu = EXACT ? min(wave_global, units - 1) : wave_global, ib = 0;  // next batch to request: unit, batch within the row
   const uint16_t *wp[NR];
   uint4 buf0[NR][B], buf1[NR][B];
   float res0 = 0.0f, res1 = 0.0f;     // residual element requested with a row's first batch
@@ -454,7 +459,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
       _Pragma("unroll") for (int k = 0; k < NR; ++k)                                              \
         wp[k] = p.w + static_cast<uint64_t>(iu + k * p.rows) * cols + lane * 8;                   \
       if constexpr (EPI == kEpiResidual) {                                                        \
-        if (lane == 0) RES = p.residual[iu];                                                      \
+        if (EXACT || lane == 0) RES = p.residual[iu];                                             \
       }                                                                                           \
     }                                                                                             \
     _Pragma("unroll") for (int u = 0; u < B; ++u)                                                 \
@@ -465,8 +470,13 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
       iu += wave_stride;                                                                          \
     }                                                                                             \
   } while (0)
-  if (total > 0) NV_FAST_ISSUE(buf0, res0);
-  if (total > 1) NV_FAST_ISSUE(buf1, res1);
+  if constexpr (EXACT) {  // the launcher guarantees two batches per row at least
+    NV_FAST_ISSUE(buf0, res0);
+    NV_FAST_ISSUE(buf1, res1);
+  } else {
+    if (total > 0) NV_FAST_ISSUE(buf0, res0);
+    if (total > 1) NV_FAST_ISSUE(buf1, res1);
+  }
 
   // ---- 3. step guard (after the requests: they do not depend on it and are always in bounds)
   if (p.cursor != nullptr && *p.cursor >= p.max_steps) return;

@@ -54,8 +54,25 @@ template <uint32_t DT, int PRO, int EPI, int MODE>
 hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream) {
   constexpr int NR = EPI == kEpiSwiglu ? 2 : kDefaultNR;  // swiglu: the gate row and the up row
   if constexpr (MODE == kFast) {
-    hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR>), dim3(blocks), dim3(kBlock), lds,
-                       stream, p);
+    // Launches whose waves own ONE row that is exactly the two batches requested up front (the step's o
+    // projection at 4096 columns) take the variant with exact start-up waits: measured 7.8 -> 7.6 us there.
+    // It needs two batches per row at least. Measured with it forced on: qkv (two rows a wave) 10.7 -> 10.8 us,
+    // down (six batches a row) 17.5 -> 18.1 us - so the rule is narrow; the "gemv_exact_start" override
+    // (1 = wherever it can run, 2 = nowhere) exists to measure that.
+    constexpr bool kShortShapes = EPI == kEpiF32 || EPI == kEpiResidual;
+    constexpr uint32_t kBatchCols = kWave * 8u * (4 / NR);
+    const uint32_t units_per_wave = (p.rows + blocks * kWavesPerBlock - 1) / (blocks * kWavesPerBlock);
+    const int forced = tuning(kTuneGemvExactStart);
+    const bool can = kShortShapes && p.cols >= 2u * kBatchCols;
+    const bool want = forced == 1 || (forced == 0 && units_per_wave == 1 && p.cols == 2u * kBatchCols);
+    if (can && want) {
+      if constexpr (kShortShapes)
+        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, true>), dim3(blocks), dim3(kBlock), lds,
+                           stream, p);
+    } else {
+      hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR>), dim3(blocks), dim3(kBlock), lds,
+                         stream, p);
+    }
   } else if constexpr (MODE == kVecFull) {
     hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, kDefaultU / NR, kVecFull, kDefaultDot2>),
                        dim3(blocks), dim3(kBlock), lds, stream, p);

@@ -120,6 +120,7 @@ enum TuningKnob : int {
   kTuneGemmBlockSlices,      // shared-X GEMM: K slices for every projection
   kTuneGemmBlockRowTiles,    // shared-X GEMM: 1 or 2 row tiles per wave
   kTuneGemmBlockMinTokens,   // shared-X GEMM: smallest token block it takes
+  kTuneGemvExactStart,       // lean GEMV: 1 = exact start-up waits wherever they can run, 2 = nowhere
   kTuneKnobs
 };
 int tuning(TuningKnob knob);
