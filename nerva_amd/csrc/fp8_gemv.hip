@@ -404,11 +404,18 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   __shared__ float sh_weight[kDownLeanMaxSlots];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const bool has_shared = p.shared_index >= 0;
+  const uint32_t slots = p.top_k + (has_shared ? 1u : 0u);
   constexpr uint32_t inter = P * 1024u;
+  // Slot order: the shared expert FIRST, then the routed ones in their order. The shared expert's index is a
+  // launch argument, so every wave can request its first weights at once; the routed ids are a dependent read
+  // from memory (a microsecond at the start of a launch) which then arrives under those weights' latency.
+  // source(slot): where the slot's activations and routing entry sit in the caller's order (routed.., shared).
+  const uint32_t first_routed = has_shared ? 1u : 0u;
   if (threadIdx.x < slots) {
-    uint32_t e = threadIdx.x < p.top_k ? p.expert_ids[threadIdx.x] : static_cast<uint32_t>(p.shared_index);
-    float weight = threadIdx.x < p.top_k ? p.expert_weights[threadIdx.x] : 1.0f;
+    const bool routed = threadIdx.x >= first_routed;
+    uint32_t e = routed ? p.expert_ids[threadIdx.x - first_routed] : static_cast<uint32_t>(p.shared_index);
+    float weight = routed ? p.expert_weights[threadIdx.x - first_routed] : 1.0f;
     if (e >= p.num_experts) {  // an id outside the bank: read expert 0 (in bounds), poison the result
       e = 0;
       weight = __builtin_nanf("");
@@ -423,7 +430,8 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
       float4 st[P * 4];
 #pragma unroll
       for (int i = 0; i < P * 4; ++i)
-        st[i] = *reinterpret_cast<const float4 *>(p.act + static_cast<uint64_t>(k) * inter + (i * kWave + lane) * 4);
+        st[i] = *reinterpret_cast<const float4 *>(p.act + static_cast<uint64_t>(has_shared ? (k == 0 ? p.top_k : k - 1) : k) * inter +
+                                                  (i * kWave + lane) * 4);
       float *dst = acts + (k & 1u) * inter;
 #pragma unroll
       for (int i = 0; i < P * 4; ++i)
@@ -432,7 +440,6 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     }
     return;
   }
-  __syncthreads();  // barrier 0 (also publishes the expert table)
   const uint32_t sc_cols = (inter + p.block - 1) / p.block;
   const uint64_t scale_stride = static_cast<uint64_t>((p.hidden + p.block - 1) / p.block) * sc_cols;
   const uint64_t w_stride = static_cast<uint64_t>(p.hidden) * inter;
@@ -441,6 +448,10 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   const uint32_t total = slots * P;
 
   uint32_t ik = 0;  // expert slot of the next request
+  // slot 0's expert without the table: the shared expert's index is an argument; without a shared expert
+  // it is the first routed id, read here directly (the same dependent read the table would have waited for)
+  uint32_t first_e = has_shared ? static_cast<uint32_t>(p.shared_index) : p.expert_ids[0];
+  if (first_e >= p.num_experts) first_e = 0;   // (the table entry carries the NaN weight for this case)
   const uint8_t *w0 = nullptr, *w1 = nullptr;
   const float *s0 = nullptr, *s1 = nullptr;
   // The ring's requests are asynchronous loads issued by hand, and each batch is awaited with an
@@ -456,7 +467,7 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   do {                                                                                        \
     constexpr uint32_t ib_ = (J) % P;                                                         \
     if constexpr (ib_ == 0) {                                                                 \
-      const uint32_t e = sh_expert[ik];                                                       \
+      const uint32_t e = ik == 0 ? first_e : sh_expert[ik];                                   \
       w0 = p.w_down + e * w_stride + static_cast<uint64_t>(h0) * inter + lane * 16;           \
       w1 = p.w_down + e * w_stride + static_cast<uint64_t>(h1) * inter + lane * 16;           \
       s0 = p.s_down + e * scale_stride + static_cast<uint64_t>(h0 / p.block) * sc_cols;       \
@@ -514,10 +525,24 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     }                                                                                         \
   } while (0)
 
-  if (total > 0) NV_DN_ISSUE(0);
-  if (total > 1) NV_DN_ISSUE(1);
-  if (total > 2) NV_DN_ISSUE(2);
-  if (total > 3) NV_DN_ISSUE(3);
+  // the shared expert's batches (the first P of the ring) go out before anything is awaited; barrier 0 then
+  // publishes the expert table and the first activations, and the rest of the ring follows
+  // (every ring register has ONE place where it is requested first: two places would meet in a copy of a
+  // register whose data is still on its way)
+  NV_DN_ISSUE(0);
+  if constexpr (P >= 2) NV_DN_ISSUE(1);
+  if constexpr (P == 4) {
+    NV_DN_ISSUE(2);
+    NV_DN_ISSUE(3);
+  }
+  __syncthreads();  // barrier 0
+  if constexpr (P == 1) {
+    if (total > 1) NV_DN_ISSUE(1);
+  }
+  if constexpr (P <= 2) {
+    if (total > 2) NV_DN_ISSUE(2);
+    if (total > 3) NV_DN_ISSUE(3);
+  }
   uint32_t t = 0;
   for (; t + 8 <= total; t += 4) {  // steady state: three newer batches behind every use
     NV_DN_AWAIT(0, 3u);
