@@ -25,6 +25,7 @@ struct MoeFp8Params {
   uint32_t hidden, inter, num_experts, top_k, block, input_dtype;
   int32_t shared_index;
   uint32_t phases;   // 0: both launches; 1: gate/up only; 2: down only (act holds an earlier gate/up result)
+  uint32_t shared_last;  // set by the launcher: lean down kernel walks the shared expert last (measurements)
 };
 
 struct MoeRouteParams {

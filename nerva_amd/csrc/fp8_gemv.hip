@@ -404,8 +404,8 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   __shared__ float sh_weight[kDownLeanMaxSlots];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const bool has_shared = p.shared_index >= 0;
-  const uint32_t slots = p.top_k + (has_shared ? 1u : 0u);
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  const bool has_shared = p.shared_index >= 0 && p.shared_last == 0;   // "the shared expert is slot 0"
   constexpr uint32_t inter = P * 1024u;
   // Slot order: the shared expert FIRST, then the routed ones in their order. The shared expert's index is a
   // launch argument, so every wave can request its first weights at once; the routed ids are a dependent read
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
   // source(slot): where the slot's activations and routing entry sit in the caller's order (routed.., shared).
   const uint32_t first_routed = has_shared ? 1u : 0u;
   if (threadIdx.x < slots) {
-    const bool routed = threadIdx.x >= first_routed;
+    const bool routed = threadIdx.x >= first_routed && threadIdx.x < first_routed + p.top_k;
     uint32_t e = routed ? p.expert_ids[threadIdx.x - first_routed] : static_cast<uint32_t>(p.shared_index);
     float weight = routed ? p.expert_weights[threadIdx.x - first_routed] : 1.0f;
     if (e >= p.num_experts) {  // an id outside the bank: read expert 0 (in bounds), poison the result
@@ -755,9 +755,11 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
       }
       const uint32_t wgs = (units + consumers - 1) / consumers;
       const dim3 block((consumers + 1) * kWave);
-      if (p.inter == 1024u) hipLaunchKernelGGL(moe_down_lean_kernel<1>, dim3(wgs), block, lds, stream, p);
-      else if (p.inter == 2048u) hipLaunchKernelGGL(moe_down_lean_kernel<2>, dim3(wgs), block, lds, stream, p);
-      else hipLaunchKernelGGL(moe_down_lean_kernel<4>, dim3(wgs), block, lds, stream, p);
+      MoeFp8Params q = p;
+      q.shared_last = tuning(kTuneMoeDownSharedFirst) == 2 ? 1u : 0u;
+      if (p.inter == 1024u) hipLaunchKernelGGL(moe_down_lean_kernel<1>, dim3(wgs), block, lds, stream, q);
+      else if (p.inter == 2048u) hipLaunchKernelGGL(moe_down_lean_kernel<2>, dim3(wgs), block, lds, stream, q);
+      else hipLaunchKernelGGL(moe_down_lean_kernel<4>, dim3(wgs), block, lds, stream, q);
     }
     else if (fast_dn) hipLaunchKernelGGL((moe_down_kernel<NR, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
     else hipLaunchKernelGGL((moe_down_kernel<NR, false>), dim3(blocks), dim3(kBlock), lds, stream, p);

@@ -121,6 +121,7 @@ enum TuningKnob : int {
   kTuneGemmBlockRowTiles,    // shared-X GEMM: 1 or 2 row tiles per wave
   kTuneGemmBlockMinTokens,   // shared-X GEMM: smallest token block it takes
   kTuneGemvExactStart,       // lean GEMV: 1 = exact start-up waits wherever they can run, 2 = nowhere
+  kTuneMoeDownSharedFirst,   // lean MoE down: 2 = walk the shared expert last, as the caller orders the slots
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

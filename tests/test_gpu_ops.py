@@ -105,6 +105,40 @@ def test_gemv_linearity_and_unit_vectors_full_size():
     assert rel_l2(outs[2], outs[0] + outs[1]) < 1e-5
 
 
+@pytest.mark.parametrize("shape", ["o", "qkv", "down", "ragged rows"])
+def test_gemv_start_up_variants_are_the_same_function(shape):
+    """The lean GEMV has two start-up orders (requests under branches, or unconditional with exact waits;
+    the launcher picks per shape). Forced on and forced off they must give bit-identical results - the
+    arithmetic and its order are the same - at the step's shapes, with the residual epilogue and with a
+    row count that leaves waves without a row."""
+    rows, cols, pro, epi = {"o": (4096, 4096, 0, 1), "qkv": (6144, 4096, 1, 0), "down": (4096, 12288, 0, 1),
+                            "ragged rows": (4090, 4096, 0, 1)}[shape]
+    rng = np.random.default_rng(rows + cols)
+    w = O.synth_16(BF16, SEED, 140, rows * cols, 0.0, 0.02).reshape(rows, cols)
+    x16 = O.encode16(BF16, rng.normal(0, 1, cols).astype(np.float32))
+    xf = rng.normal(0, 1, cols).astype(np.float32)
+    gamma = O.encode16(BF16, rng.normal(1, 0.1, cols).astype(np.float32))
+    res = rng.normal(0, 1, rows).astype(np.float32)
+    dw, y = dev(w), N.DeviceBuffer(rows * 4)
+    outs = {}
+    try:
+        for mode in (2, 1, 0):
+            N.Device.set_tuning("gemv_exact_start", mode)
+            if pro == 0:
+                N.gemv(BF16, dw, rows, cols, input16=dev(x16), residual=dev(res), out_f32=y, epilogue=epi)
+            else:
+                N.gemv(BF16, dw, rows, cols, input_f32=dev(xf), gamma=dev(gamma), eps=1e-6, out_f32=y, epilogue=epi)
+            outs[mode] = y.numpy(np.float32).copy()
+    finally:
+        N.Device.set_tuning("gemv_exact_start", 0)
+    assert np.array_equal(outs[1], outs[2]) and np.array_equal(outs[0], outs[2])
+    if pro == 0:
+        ref = O.gemv_x16(BF16, w, x16) + res
+    else:
+        ref = O.gemv_x16(BF16, w, O.encode16(BF16, O.rms_norm(BF16, xf, gamma, 1e-6)))
+    assert rel_l2(outs[0], ref) <= REL_L2
+
+
 @pytest.mark.parametrize("dtype", [BF16, F16])
 @pytest.mark.parametrize("cols,rows", [(4096, 6144), (520, 64), (6, 3)])
 def test_gemv_rmsnorm_prologue(dtype, cols, rows):
