@@ -404,33 +404,37 @@ constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per la
 // without a row asks for the last row's data and drops it - so that the compiler can count the requests
 // behind the activation loads and waits for exactly those before the prologue, which then runs under
 // the weights' latency. With the requests under `if (total > n)` it waits for everything.
-template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false>
-__global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
+// WG: waves per workgroup (4 or 16). Every workgroup fetches the whole input vector (and for the RMSNorm
+// prologue the norm weights) for itself, so fewer, larger workgroups move that much less through the L2s ahead of
+// the weights; the waves' work is the same whatever the size (wave_global = workgroup x WG + wave).
+template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false, int WG = kWavesPerBlock>
+__global__ __launch_bounds__(WG *kWave, fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
+  constexpr int TB = WG * kWave;
   extern __shared__ __align__(16) uint16_t xs[];
-  __shared__ float red[kWavesPerBlock];
-  __shared__ uint32_t red_i[kWavesPerBlock];
-  __shared__ uint32_t red_h[kWavesPerBlock];
+  __shared__ float red[WG];
+  __shared__ uint32_t red_i[WG];
+  __shared__ uint32_t red_h[WG];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint32_t cols = p.cols;
   const uint32_t units = p.rows;  // NR == 1: rows; kEpiSwiglu (NR == 2): gate/up pairs
-  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
-  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
+  const uint32_t wave_global = blockIdx.x * WG + wave;
+  const uint32_t wave_stride = gridDim.x * WG;
   const uint32_t bpr = cols / (kWave * 8 * B);  // request batches per row
   const uint32_t my_units = wave_global < units ? (units - wave_global + wave_stride - 1) / wave_stride : 0u;
   const uint32_t total = my_units * bpr;
 
   // ---- 1. activation loads (L2 hits), kept in registers until the weights are requested
-  constexpr int kXV = kFastMaxCols / (kBlock * 8);  // 6
+  constexpr int kXV = (kFastMaxCols + TB * 8 - 1) / (TB * 8);  // 6 with four waves
   uint4 xraw[PRO == kProX16 ? kXV : 1];
   float4 xa[PRO == kProRmsNorm ? 2 : 1], xb[PRO == kProRmsNorm ? 2 : 1];
   uint4 gw[PRO == kProRmsNorm ? 2 : 1];
-  const bool norm_in_regs = cols <= kBlock * 16;
+  const bool norm_in_regs = cols <= TB * 16;
   if constexpr (PRO == kProX16) {
 #pragma unroll
     for (int i = 0; i < kXV; ++i) {
-      const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+      const uint32_t c = (i * TB + threadIdx.x) * 8;
       xraw[i] = make_uint4(0u, 0u, 0u, 0u);
       if (c < cols) xraw[i] = *reinterpret_cast<const uint4 *>(p.x16 + c);
     }
@@ -438,7 +442,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
     if (norm_in_regs) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        const uint32_t c = (i * TB + threadIdx.x) * 8;
         if (c < cols) {
           xa[i] = *reinterpret_cast<const float4 *>(p.xf + c);
           xb[i] = *reinterpret_cast<const float4 *>(p.xf + c + 4);
@@ -485,7 +489,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
   if constexpr (PRO == kProX16) {
 #pragma unroll
     for (int i = 0; i < kXV; ++i) {
-      const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+      const uint32_t c = (i * TB + threadIdx.x) * 8;
       if (c < cols) *reinterpret_cast<uint4 *>(xs + c) = xraw[i];
     }
   } else {
@@ -493,19 +497,19 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
     if (norm_in_regs) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        const uint32_t c = (i * TB + threadIdx.x) * 8;
         if (c < cols)
           ss += xa[i].x * xa[i].x + xa[i].y * xa[i].y + xa[i].z * xa[i].z + xa[i].w * xa[i].w +
                 xb[i].x * xb[i].x + xb[i].y * xb[i].y + xb[i].z * xb[i].z + xb[i].w * xb[i].w;
       }
     } else {
-      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8) {
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += TB * 8) {
         const float4 a = *reinterpret_cast<const float4 *>(p.xf + c);
         const float4 b = *reinterpret_cast<const float4 *>(p.xf + c + 4);
         ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
       }
     }
-    ss = block_sum(ss, red);
+    ss = block_sum_n<WG>(ss, red);
     const float scale = 1.0f / sqrtf(ss / static_cast<float>(cols) + p.eps);
     auto emit = [&](uint32_t c, const float4 &a, const float4 &b, const uint4 &g) {
       float g0, g1, g2, g3, g4, g5, g6, g7;
@@ -523,11 +527,11 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
     if (norm_in_regs) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const uint32_t c = (i * kBlock + threadIdx.x) * 8;
+        const uint32_t c = (i * TB + threadIdx.x) * 8;
         if (c < cols) emit(c, xa[i], xb[i], gw[i]);
       }
     } else {
-      for (uint32_t c = threadIdx.x * 8; c < cols; c += kBlock * 8)
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += TB * 8)
         emit(c, *reinterpret_cast<const float4 *>(p.xf + c), *reinterpret_cast<const float4 *>(p.xf + c + 4),
              *reinterpret_cast<const uint4 *>(p.gamma + c));
     }
@@ -535,7 +539,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
   __syncthreads();
   if constexpr (PRO == kProRmsNorm) {
     if (p.x16_dump != nullptr && blockIdx.x == 0)
-      for (uint32_t c = threadIdx.x; c < cols; c += kBlock) p.x16_dump[c] = xs[c];
+      for (uint32_t c = threadIdx.x; c < cols; c += TB) p.x16_dump[c] = xs[c];
   }
 
   // ---- 5. main loop
@@ -607,7 +611,7 @@ __global__ __launch_bounds__(kBlock, fast_waves_per_simd(PRO)) void gemv_fast_ke
     __syncthreads();
     if (threadIdx.x == 0) {
       Best block_best{red[0], red_i[0], red_h[0]};
-      for (int w = 1; w < kWavesPerBlock; ++w) {
+      for (int w = 1; w < WG; ++w) {
         Best o{red[w], red_i[w], red_h[w]};
         if (better(o, block_best)) block_best = o;
       }
@@ -632,7 +636,9 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
 // per-workgroup outputs). `vec16` = every pointer is 16-byte aligned.
 struct GemvPlan {
   int mode;         // kScalar / kVecGuarded / kVecFull / kFast
-  uint32_t blocks;
+  uint32_t blocks;  // four-wave workgroups' worth of waves
+  int wg_waves;     // waves per workgroup the launch uses (kFast: 4 or 16)
+  uint32_t grid;    // workgroups launched: ceil(blocks * 4 / wg_waves)
 };
 constexpr int kFast = 3;  // the lean production-shape kernel
 GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,

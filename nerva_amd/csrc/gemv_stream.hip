@@ -51,7 +51,7 @@ __global__ __launch_bounds__(1024) void sample_finish_kernel(SampleParams s, uin
 }
 
 template <uint32_t DT, int PRO, int EPI, int MODE>
-hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream) {
+hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream, int wg) {
   constexpr int NR = EPI == kEpiSwiglu ? 2 : kDefaultNR;  // swiglu: the gate row and the up row
   if constexpr (MODE == kFast) {
     // Launches whose waves own ONE row that is exactly the two batches requested up front (the step's o
@@ -65,14 +65,21 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
     const int forced = tuning(kTuneGemvExactStart);
     const bool can = kShortShapes && p.cols >= 2u * kBatchCols;
     const bool want = forced == 1 || (forced == 0 && units_per_wave == 1 && p.cols == 2u * kBatchCols);
+    // Waves per workgroup: the same waves in fewer workgroups (see the kernel).
+    const uint32_t waves = blocks * kWavesPerBlock;
+#define NV_GEMV_LAUNCH(EX, W)                                                                                  \
+  hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, EX, W>), dim3((waves + W - 1) / W), dim3(W * kWave), lds, \
+                     stream, p)
     if (can && want) {
-      if constexpr (kShortShapes)
-        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, true>), dim3(blocks), dim3(kBlock), lds,
-                           stream, p);
+      if constexpr (kShortShapes) {
+        if (wg == 16) NV_GEMV_LAUNCH(true, 16);
+        else NV_GEMV_LAUNCH(true, 4);
+      }
     } else {
-      hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR>), dim3(blocks), dim3(kBlock), lds,
-                         stream, p);
+      if (wg == 16) NV_GEMV_LAUNCH(false, 16);
+      else NV_GEMV_LAUNCH(false, 4);
     }
+#undef NV_GEMV_LAUNCH
   } else if constexpr (MODE == kVecFull) {
     hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, kDefaultU / NR, kVecFull, kDefaultDot2>),
                        dim3(blocks), dim3(kBlock), lds, stream, p);
@@ -88,26 +95,36 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
 
 template <uint32_t DT, int PRO, int MODE>
 hipError_t launch_epi(int epilogue, const GemvParams &p, uint32_t blocks, size_t lds,
-                      hipStream_t stream) {
+                      hipStream_t stream, int wg) {
   switch (epilogue) {
-    case kEpiF32: return launch_one<DT, PRO, kEpiF32, MODE>(p, blocks, lds, stream);
-    case kEpiResidual: return launch_one<DT, PRO, kEpiResidual, MODE>(p, blocks, lds, stream);
-    case kEpiSwiglu: return launch_one<DT, PRO, kEpiSwiglu, MODE>(p, blocks, lds, stream);
-    case kEpiOut16: return launch_one<DT, PRO, kEpiOut16, MODE>(p, blocks, lds, stream);
-    case kEpiArgmax: return launch_one<DT, PRO, kEpiArgmax, MODE>(p, blocks, lds, stream);
+    case kEpiF32: return launch_one<DT, PRO, kEpiF32, MODE>(p, blocks, lds, stream, wg);
+    case kEpiResidual: return launch_one<DT, PRO, kEpiResidual, MODE>(p, blocks, lds, stream, wg);
+    case kEpiSwiglu: return launch_one<DT, PRO, kEpiSwiglu, MODE>(p, blocks, lds, stream, wg);
+    case kEpiOut16: return launch_one<DT, PRO, kEpiOut16, MODE>(p, blocks, lds, stream, wg);
+    case kEpiArgmax: return launch_one<DT, PRO, kEpiArgmax, MODE>(p, blocks, lds, stream, wg);
     default: return hipErrorInvalidValue;
   }
 }
 
 template <uint32_t DT, int MODE>
 hipError_t launch_pro(int prologue, int epilogue, const GemvParams &p, uint32_t blocks, size_t lds,
-                      hipStream_t stream) {
-  if (prologue == kProX16) return launch_epi<DT, kProX16, MODE>(epilogue, p, blocks, lds, stream);
-  if (prologue == kProRmsNorm) return launch_epi<DT, kProRmsNorm, MODE>(epilogue, p, blocks, lds, stream);
+                      hipStream_t stream, int wg) {
+  if (prologue == kProX16) return launch_epi<DT, kProX16, MODE>(epilogue, p, blocks, lds, stream, wg);
+  if (prologue == kProRmsNorm) return launch_epi<DT, kProRmsNorm, MODE>(epilogue, p, blocks, lds, stream, wg);
   return hipErrorInvalidValue;
 }
 
 bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+// Waves per workgroup the lean kernel is launched with (4 or 16), per shape. Every workgroup fetches the input
+// vector and the norm weights for itself (24 KiB at 4096 columns); the LM head's 2048 looping workgroups move
+// 49 MB of that ahead of their weights, as 512 workgroups of 16 waves 12 MB: 197 -> 190 us. The step's other
+// launches measured the same (qkv, o, down: within 0.1 us) or worse (gate_up 32.8 -> 34.6 us: one workgroup of
+// 16 waves per CU instead of five of 4) with 16.
+int fast_workgroup_waves(int prologue, int epilogue, uint32_t rows, uint32_t cols) {
+  (void)cols;
+  return prologue == kProRmsNorm && epilogue == kEpiArgmax && rows >= 65536u ? 16 : kWavesPerBlock;
+}
 
 }  // namespace
 
@@ -143,6 +160,12 @@ GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, boo
   }
   if (epilogue == kEpiArgmax && blocks > kSampleMaxBlocks) blocks = kSampleMaxBlocks;
   plan.blocks = blocks == 0 ? 1 : blocks;
+  plan.wg_waves = kWavesPerBlock;
+  if (plan.mode == kFast) {
+    plan.wg_waves = nv::tuning(kTuneGemvWorkgroupWaves);
+    if (plan.wg_waves != 4 && plan.wg_waves != 16) plan.wg_waves = fast_workgroup_waves(prologue, epilogue, rows, cols);
+  }
+  plan.grid = (plan.blocks * kWavesPerBlock + plan.wg_waves - 1) / plan.wg_waves;
   return plan;
 }
 
@@ -168,17 +191,19 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
   const GemvPlan plan = gemv_plan(prologue, epilogue, p.rows, p.cols, vec16, tuning);
   const int mode = plan.mode;
   const uint32_t blocks = plan.blocks;
-  if (blocks_used) *blocks_used = blocks;
+  // (the plan counts four-wave workgroups; the lean kernel may launch the same waves as fewer, larger ones)
+  const int wg = plan.wg_waves;
+  if (blocks_used) *blocks_used = plan.grid;
   if (dtype == kBF16) {
-    if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, blocks, lds, stream);
-    if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
-    if (mode == kVecGuarded) return launch_pro<kBF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream);
-    return launch_pro<kBF16, kScalar>(prologue, epilogue, p, blocks, lds, stream);
+    if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, blocks, lds, stream, wg);
+    if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream, wg);
+    if (mode == kVecGuarded) return launch_pro<kBF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream, wg);
+    return launch_pro<kBF16, kScalar>(prologue, epilogue, p, blocks, lds, stream, wg);
   }
-  if (mode == kFast) return launch_pro<kF16, kFast>(prologue, epilogue, p, blocks, lds, stream);
-  if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream);
-  if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream);
-  return launch_pro<kF16, kScalar>(prologue, epilogue, p, blocks, lds, stream);
+  if (mode == kFast) return launch_pro<kF16, kFast>(prologue, epilogue, p, blocks, lds, stream, wg);
+  if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream, wg);
+  if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream, wg);
+  return launch_pro<kF16, kScalar>(prologue, epilogue, p, blocks, lds, stream, wg);
 }
 
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,

@@ -83,6 +83,20 @@ __device__ __forceinline__ float block_sum(float v, float *scratch) {
   return total;
 }
 
+// The same for a workgroup of WG waves (`scratch`: WG floats).
+template <int WG>
+__device__ __forceinline__ float block_sum_n(float v, float *scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < WG; ++w) total += scratch[w];
+  return total;
+}
+
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
 // (value desc, index asc) among finite candidates; `has` false = no candidate yet
@@ -122,6 +136,7 @@ enum TuningKnob : int {
   kTuneGemmBlockMinTokens,   // shared-X GEMM: smallest token block it takes
   kTuneGemvExactStart,       // lean GEMV: 1 = exact start-up waits wherever they can run, 2 = nowhere
   kTuneMoeDownSharedFirst,   // lean MoE down: 2 = walk the shared expert last, as the caller orders the slots
+  kTuneGemvWorkgroupWaves,   // lean GEMV: waves per workgroup for every launch (4 or 16)
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

@@ -30,7 +30,7 @@ std::atomic<int> g_tuning[kTuneKnobs];
 constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_splits",       "prompt_splits",
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
-                                                  "moe_down_shared_first"};
+                                                  "moe_down_shared_first", "gemv_workgroup_waves"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }
@@ -359,7 +359,7 @@ int nerva_hip_gemv_launch_shape(uint32_t prologue, uint32_t epilogue, uint32_t r
   if (prologue > 1 || epilogue > 4 || rows == 0 || cols == 0) return -1;
   const GemvPlan plan = gemv_plan(static_cast<int>(prologue), static_cast<int>(epilogue), rows, cols, true, nullptr);
   if (kernel) *kernel = static_cast<uint32_t>(plan.mode);
-  if (workgroups) *workgroups = plan.blocks;
+  if (workgroups) *workgroups = plan.grid;
   return 0;
 }
 
