@@ -7,7 +7,7 @@ use std::path::{Path, PathBuf};
 use std::process::Command;
 
 const SOURCES: &[&str] = &[
-    "gemv_stream", "fp8_gemv", "attn_decode", "attn_prompt", "argmax", "synth_fill", "decode_chain",
+    "gemv_stream", "fp8_gemv", "attn_decode", "attn_prompt", "argmax", "synth_fill",
     "sampler", "gemm_rows", "gemm_block", "op_entry", "decode_session",
 ];
 

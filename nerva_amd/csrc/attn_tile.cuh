@@ -465,8 +465,8 @@ __device__ __forceinline__ void attn_fast_body(const AttnParams &p, const uint32
   // Up to four tiles in flight per wave (one 8-wave workgroup per CU leaves 256 registers a lane;
   // at the default split factor a wave's whole share of an 8k context is requested at once). The
   // lean variant keeps one, to fit the 128 registers that let two 8-wave workgroups share a CU:
-  // linked workgroups (their launch uses more splits instead) and prompt blocks, whose launches
-  // hold thousands of workgroups and are bound by how many of them a CU can run at a time.
+  // prompt blocks, whose launches hold thousands of workgroups and are bound by how many of them a
+  // CU can run at a time.
   constexpr int kInFlight = IN_FLIGHT;
   constexpr bool kLean = IN_FLIGHT == 1;  // 128-register budget: the query operand is parked in LDS
   uint4 kreg[kInFlight][4], vreg[kInFlight][4];

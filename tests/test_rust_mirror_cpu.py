@@ -107,3 +107,13 @@ def test_safe_wrappers_name_only_what_exists():
     contracts = open(os.path.join(CRATE, "src", "contracts.rs")).read()
     for name in re.findall(r'name: "(hip_\w+)"', contracts):
         assert '+            name: "%s",' % name in rows
+
+
+def test_build_script_lists_the_sources_that_exist():
+    """build.rs compiles nerva_amd/csrc/<name>.hip for every name in SOURCES: the list is the library's."""
+    import re
+    text = open(os.path.join(ROOT, "crates", "nerva-hip", "build.rs")).read()
+    block = re.search(r"const SOURCES: &\[&str\] = &\[(.*?)\];", text, re.S).group(1)
+    names = re.findall(r'"([a-z0-9_]+)"', block)
+    csrc = os.path.join(ROOT, "nerva_amd", "csrc")
+    assert sorted(names) == sorted(f[:-4] for f in os.listdir(csrc) if f.endswith(".hip"))
