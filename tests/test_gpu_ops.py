@@ -105,6 +105,22 @@ def test_gemv_linearity_and_unit_vectors_full_size():
     assert rel_l2(outs[2], outs[0] + outs[1]) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", [BF16, F16])
+def test_gemv_keeps_16_bit_denormals(dtype):
+    """The lean GEMV multiplies 16-bit pairs with the packed dot instruction (f32 accumulation): weights that
+    are denormal in their 16-bit type must count in full (no flush to zero) - every weight of this matrix is a
+    denormal, the activations are large, and the result equals the oracle's exactly."""
+    rows = cols = 4096
+    w = np.full((rows, cols), 0x0001, np.uint16)                     # the smallest denormal of either type
+    w[1::2] = 0x03FF if dtype == F16 else 0x007F                     # the largest
+    x = O.encode16(dtype, np.full(cols, 1024.0 if dtype == F16 else 2.0 ** 100, np.float32))
+    ref = O.gemv_x16(dtype, w, x)
+    assert np.all(ref > 0)
+    y = N.DeviceBuffer(rows * 4)
+    N.gemv(dtype, dev(w), rows, cols, input16=dev(x), out_f32=y)
+    assert np.array_equal(y.numpy(np.float32), ref)
+
+
 @pytest.mark.parametrize("shape", ["o", "qkv", "down", "ragged rows"])
 def test_gemv_start_up_variants_are_the_same_function(shape):
     """The lean GEMV has two start-up orders (requests under branches, or unconditional with exact waits;
