@@ -54,17 +54,17 @@ template <uint32_t DT, int PRO, int EPI, int MODE>
 hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream, int wg) {
   constexpr int NR = EPI == kEpiSwiglu ? 2 : kDefaultNR;  // swiglu: the gate row and the up row
   if constexpr (MODE == kFast) {
-    // Launches whose waves own ONE row that is exactly the two batches requested up front (the step's o
-    // projection at 4096 columns) take the variant with exact start-up waits: measured 7.8 -> 7.6 us there.
-    // It needs two batches per row at least. Measured with it forced on: qkv (two rows a wave) 10.7 -> 10.8 us,
-    // down (six batches a row) 17.5 -> 18.1 us - so the rule is narrow; the "gemv_exact_start" override
-    // (1 = wherever it can run, 2 = nowhere) exists to measure that.
+    // Launches whose waves own one or two rows of exactly two batches each (the step's o and qkv projections at
+    // 4096 columns) take the variant with exact start-up waits: o 7.5 -> 7.2 us, qkv 10.6 -> 10.25 us in the step.
+    // It needs two batches per row at least. Measured with it forced on elsewhere ("gemv_exact_start" override:
+    // 1 = wherever it can run, 2 = nowhere): down (six batches a row) 17.1 -> 17.6 us; the gate/up pair and the
+    // LM head do not move, so only the plain and residual epilogues have the variant.
     constexpr bool kShortShapes = EPI == kEpiF32 || EPI == kEpiResidual;
     constexpr uint32_t kBatchCols = kWave * 8u * (4 / NR);
     const uint32_t units_per_wave = (p.rows + blocks * kWavesPerBlock - 1) / (blocks * kWavesPerBlock);
     const int forced = tuning(kTuneGemvExactStart);
     const bool can = kShortShapes && p.cols >= 2u * kBatchCols;
-    const bool want = forced == 1 || (forced == 0 && units_per_wave == 1 && p.cols == 2u * kBatchCols);
+    const bool want = forced == 1 || (forced == 0 && units_per_wave <= 2 && p.cols == 2u * kBatchCols);
     // Waves per workgroup: the same waves in fewer workgroups (see the kernel).
     const uint32_t waves = blocks * kWavesPerBlock;
 #define NV_GEMV_LAUNCH(EX, W)                                                                                  \

@@ -301,7 +301,7 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
     assert N.gemv_launch_shape(1, 2, 12288, 4096) == (3, 2048)     # gate_up: oversubscribed long launch
     assert N.gemv_launch_shape(1, 0, 6144, 4096) == (3, 768)       # qkv: two rows per wave in one round
     assert N.gemv_launch_shape(0, 1, 4096, 4096) == (3, 1024)      # o: every row on the machine at once
-    assert N.gemv_launch_shape(1, 4, 151936, 4096)[0] == 3         # LM head
+    assert N.gemv_launch_shape(1, 4, 151936, 4096) == (3, 512)     # LM head: 16-wave workgroups
     assert N.gemv_launch_shape(0, 0, 100, 520)[0] == 1             # 520 columns: the guarded vector kernel
     with pytest.raises(ValueError):
         N.gemv_launch_shape(0, 0, 0, 64)
