@@ -411,9 +411,15 @@ constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per la
 // WG: waves per workgroup (4 or 16). Every workgroup fetches the whole input vector (and for the RMSNorm
 // prologue the norm weights) for itself, so fewer, larger workgroups move that much less through the L2s ahead of
 // the weights; the waves' work is the same whatever the size (wave_global = workgroup x WG + wave).
-template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false, int WG = kWavesPerBlock>
-__global__ __launch_bounds__(WG *kWave, fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
+// XREG (4096 columns only): a lane's share of the input vector - the eight 16-byte pieces that meet its eight
+// weight pieces of a row - is read from LDS once, right after the prologue, and kept in registers, so the
+// products behind a batch's arrival do not wait for LDS reads (a wave gets one 1 KiB LDS read through every
+// ~30 cycles: eight of them a row were twice the time of the row's 32 dot instructions). Costs 32 registers:
+// one wave per SIMD less.
+template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false, int WG = kWavesPerBlock, bool XREG = false>
+__global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
   constexpr int TB = WG * kWave;
+  constexpr uint32_t kXregBpr = 8 / B;   // batches per 4096-column row
   extern __shared__ __align__(16) uint16_t xs[];
   __shared__ float red[WG];
   __shared__ uint32_t red_i[WG];
@@ -547,6 +553,11 @@ __global__ __launch_bounds__(WG *kWave, fast_waves_per_simd(PRO)) void gemv_fast
   }
 
   // ---- 5. main loop
+  uint4 xr[XREG ? 8 : 1];
+  if constexpr (XREG) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = *reinterpret_cast<const uint4 *>(xs + i * (kWave * 8) + lane * 8);
+  }
   Best best{0.0f, 0u, 0u};
   uint32_t cu = wave_global, cb = 0;  // batch being consumed: unit, batch within the row
   float acc[NR];
@@ -559,10 +570,12 @@ __global__ __launch_bounds__(WG *kWave, fast_waves_per_simd(PRO)) void gemv_fast
     }                                                                                             \
     const uint32_t c0 = cb * (B * kWave * 8) + lane * 8;                                          \
     _Pragma("unroll") for (int u = 0; u < B; ++u) {                                               \
-      const uint4 xv = *reinterpret_cast<const uint4 *>(xs + c0 + u * (kWave * 8));               \
+      uint4 xv;                                                                                   \
+      if constexpr (XREG) xv = xr[cb * B + u]; /* cb is a constant at every use in this mode */   \
+      else xv = *reinterpret_cast<const uint4 *>(xs + c0 + u * (kWave * 8));                      \
       _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = dot8<DT, true>(SRC[k][u], xv, acc[k]);  \
     }                                                                                             \
-    if (++cb == bpr) {                                                                            \
+    if (++cb == (XREG ? kXregBpr : bpr)) {                                                        \
       cb = 0;                                                                                     \
       _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = wave_sum(acc[k]);                   \
       if (lane == 0) {                                                                            \
@@ -595,12 +608,32 @@ __global__ __launch_bounds__(WG *kWave, fast_waves_per_simd(PRO)) void gemv_fast
     }                                                                                             \
   } while (0)
 
-  for (uint32_t t = 0; t < total; t += 2) {
-    NV_FAST_CONSUME(buf0, res0);
-    if (t + 2 < total) NV_FAST_ISSUE(buf0, res0);
-    if (t + 1 < total) {
+  if constexpr (XREG) {
+    // one unit per turn: its batches alternate between the two buffers, the batch index is a constant
+    for (uint32_t t = 0; t < total; t += kXregBpr) {
+      cb = 0;
+      NV_FAST_CONSUME(buf0, res0);
+      if (t + 2 < total) NV_FAST_ISSUE(buf0, res0);
+      cb = 1;
       NV_FAST_CONSUME(buf1, res1);
       if (t + 3 < total) NV_FAST_ISSUE(buf1, res1);
+      if constexpr (kXregBpr == 4) {
+        cb = 2;
+        NV_FAST_CONSUME(buf0, res0);
+        if (t + 4 < total) NV_FAST_ISSUE(buf0, res0);
+        cb = 3;
+        NV_FAST_CONSUME(buf1, res1);
+        if (t + 5 < total) NV_FAST_ISSUE(buf1, res1);
+      }
+    }
+  } else {
+    for (uint32_t t = 0; t < total; t += 2) {
+      NV_FAST_CONSUME(buf0, res0);
+      if (t + 2 < total) NV_FAST_ISSUE(buf0, res0);
+      if (t + 1 < total) {
+        NV_FAST_CONSUME(buf1, res1);
+        if (t + 3 < total) NV_FAST_ISSUE(buf1, res1);
+      }
     }
   }
 #undef NV_FAST_ISSUE

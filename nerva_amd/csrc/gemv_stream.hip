@@ -67,17 +67,24 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
     const bool want = forced == 1 || (forced == 0 && units_per_wave <= 2 && p.cols == 2u * kBatchCols);
     // Waves per workgroup: the same waves in fewer workgroups (see the kernel).
     const uint32_t waves = blocks * kWavesPerBlock;
-#define NV_GEMV_LAUNCH(EX, W)                                                                                  \
-  hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, EX, W>), dim3((waves + W - 1) / W), dim3(W * kWave), lds, \
-                     stream, p)
+    // The input vector in registers (see the kernel): measured o 7.25 -> 7.05 us; qkv unchanged, gate_up
+    // 31.8 -> 33.5 us, LM head 187 -> 189 us (one wave per SIMD less) - so only the short launches with a
+    // 16-bit input take it.
+    const bool xreg = PRO == kProX16 && p.cols == 4096u && tuning(kTuneGemvXRegisters) != 2;
+#define NV_GEMV_LAUNCH(EX, W, XR)                                                                              \
+  hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, EX, W, XR>), dim3((waves + W - 1) / W),         \
+                     dim3(W * kWave), lds, stream, p)
     if (can && want) {
       if constexpr (kShortShapes) {
-        if (wg == 16) NV_GEMV_LAUNCH(true, 16);
-        else NV_GEMV_LAUNCH(true, 4);
+        if (wg == 16) NV_GEMV_LAUNCH(true, 16, false);
+        else if constexpr (PRO == kProX16) {
+          if (xreg) NV_GEMV_LAUNCH(true, 4, true);
+          else NV_GEMV_LAUNCH(true, 4, false);
+        } else NV_GEMV_LAUNCH(true, 4, false);
       }
     } else {
-      if (wg == 16) NV_GEMV_LAUNCH(false, 16);
-      else NV_GEMV_LAUNCH(false, 4);
+      if (wg == 16) NV_GEMV_LAUNCH(false, 16, false);
+      else NV_GEMV_LAUNCH(false, 4, false);
     }
 #undef NV_GEMV_LAUNCH
   } else if constexpr (MODE == kVecFull) {

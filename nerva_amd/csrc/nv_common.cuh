@@ -137,6 +137,7 @@ enum TuningKnob : int {
   kTuneGemvExactStart,       // lean GEMV: 1 = exact start-up waits wherever they can run, 2 = nowhere
   kTuneMoeDownSharedFirst,   // lean MoE down: 2 = walk the shared expert last, as the caller orders the slots
   kTuneGemvWorkgroupWaves,   // lean GEMV: waves per workgroup for every launch (4 or 16)
+  kTuneGemvXRegisters,       // lean GEMV: 2 = never keep the input vector in registers
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

@@ -30,7 +30,8 @@ std::atomic<int> g_tuning[kTuneKnobs];
 constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_splits",       "prompt_splits",
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
-                                                  "moe_down_shared_first", "gemv_workgroup_waves"};
+                                                  "moe_down_shared_first", "gemv_workgroup_waves",
+                                                  "gemv_x_registers"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }

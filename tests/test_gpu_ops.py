@@ -140,6 +140,7 @@ def test_gemv_start_up_variants_are_the_same_function(shape):
     try:
         for mode in (2, 1, 0):
             N.Device.set_tuning("gemv_exact_start", mode)
+            N.Device.set_tuning("gemv_x_registers", 2 if mode == 1 else 0)   # (1: exact start without the register copy of x)
             if pro == 0:
                 N.gemv(BF16, dw, rows, cols, input16=dev(x16), residual=dev(res), out_f32=y, epilogue=epi)
             else:
@@ -147,6 +148,7 @@ def test_gemv_start_up_variants_are_the_same_function(shape):
             outs[mode] = y.numpy(np.float32).copy()
     finally:
         N.Device.set_tuning("gemv_exact_start", 0)
+        N.Device.set_tuning("gemv_x_registers", 0)
     assert np.array_equal(outs[1], outs[2]) and np.array_equal(outs[0], outs[2])
     if pro == 0:
         ref = O.gemv_x16(BF16, w, x16) + res
