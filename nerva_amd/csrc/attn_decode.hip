@@ -159,7 +159,7 @@ constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
 // and l words until every tag is up and folds them in split order; the sixteen groups meet in LDS in
 // group order - a fixed order, whatever the arrival order was. A CU sustains only a few hundred
 // device-coherent cache lines per microsecond, which is why a head is spread over several merging
-// workgroups. Afterwards every word that was read gets its tag cleared for the next launch (launches
+// workgroups. Last of all every word that was read gets its tag cleared for the next launch (launches
 // are ordered by the stream). A wait that runs out (a split that never stored: cannot happen on a
 // healthy device) ends after kMergeSpinLimit polls and the outputs it feeds become NaN: a failure that
 // shows in the logits instead of a plausible wrong number.
@@ -202,16 +202,6 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
     }
   }
   __syncthreads();  // the LDS arrays below were read by the wave merge (or by the previous part's merge)
-  // Every thread has taken what it needs: the words can be cleared for the next launch (a split's m and
-  // l words are read by all 32 threads of a group, so nobody may clear them before this barrier).
-#pragma unroll
-  for (uint32_t i = 0; i < kPer; ++i) {
-    if (q + i * kGroups < active) {
-      uint64_t *r = rec + static_cast<uint64_t>(q + i * kGroups) * kStepRecord;
-      __hip_atomic_store(r + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (dl < 2) __hip_atomic_store(r + kStepPartDims + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
   lds_o[q * kStepPartDims + dl] = gave_up ? NAN : o;
   if (dl == 0) {
     lds_m[q] = M;
@@ -233,6 +223,17 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
     const uint32_t e = h * kHD + part * kStepPartDims + dl;
     if (p.out_f32 != nullptr) p.out_f32[e] = ot;
     p.out16[attn_out_elem(p, e)] = enc16<DT>(ot);
+  }
+  // Every thread has taken what it needs (a split's m and l words are read by all 32 threads of a group, so
+  // nobody may clear them before a barrier that follows the reads: the one above): the words are cleared for
+  // the next launch - behind the output, which the next kernel waits for, while nothing waits for these.
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; ++i) {
+    if (q + i * kGroups < active) {
+      uint64_t *r = rec + static_cast<uint64_t>(q + i * kGroups) * kStepRecord;
+      __hip_atomic_store(r + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (dl < 2) __hip_atomic_store(r + kStepPartDims + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
@@ -364,17 +365,18 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
 
-  // ---- 3. the wave's first four tiles
+  // ---- 3. the wave's first tile. Only the first: at long contexts the launch is one burst of requests, the
+  // memory path fills up, and a wave that goes on requesting sits in its request instructions until the burst
+  // has drained enough (3 us at 8k tokens) - with its head inputs long there and its head preparation not
+  // started. So: one tile out, the head preparation under its flight, then the rest (the burst takes its
+  // 4-5 us either way; what is requested a microsecond later is not served later).
   link_mark(tr, 6);
   u32x4_t kr[4][4], vr[4][4];
   if (nt > 0) NV_AT_TILE_LOAD(0, phys[0]);
-  if (nt > 1) NV_AT_TILE_LOAD(1, phys[1]);
-  if (nt > 2) NV_AT_TILE_LOAD(2, phys[2]);
-  if (nt > 3) NV_AT_TILE_LOAD(3, phys[3]);
   link_mark(tr, 8);
 
-  // ---- 4. the inputs have arrived once at most the tile requests are outstanding
-  NV_AT_WAIT_BEHIND(min(nt, 4u));
+  // ---- 4. the inputs have arrived once at most the first tile's requests are outstanding
+  NV_AT_WAIT_BEHIND(min(nt, 1u));
   NV_AT_TAKE_INPUTS();
   link_mark(tr, 14);
 
@@ -407,6 +409,10 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
     row[lane] = enc16<DT>(x0);
     row[lane + 64] = enc16<DT>(x1);
   }
+  // the wave's other tiles of the first four, behind its own head work and before it waits for the others'
+  if (nt > 1) NV_AT_TILE_LOAD(1, phys[1]);
+  if (nt > 2) NV_AT_TILE_LOAD(2, phys[2]);
+  if (nt > 3) NV_AT_TILE_LOAD(3, phys[3]);
   link_mark(tr, 15);
   __syncthreads();
   link_mark(tr, 9);
