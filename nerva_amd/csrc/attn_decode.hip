@@ -350,7 +350,7 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   } else {
     pos = p.cursor != nullptr ? sload(p.cursor) : p.position;
     if (p.cursor != nullptr && pos >= p.max_steps) return;
-    attn_split_geometry(pos, S, nblk, bps, active);
+    attn_split_geometry(pos, S, p.single_split_blocks, nblk, bps, active);
     first = split * bps + wave;
     const uint32_t end = min(nblk, split * bps + bps);
     nt = first < end ? (end - first + W - 1) / W : 0u;  // tiles first, first + W, ...

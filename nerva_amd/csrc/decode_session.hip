@@ -116,6 +116,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
   void *attn_ws = nullptr, *sample_ws = nullptr;
   uint32_t attn_splits = 1;
+  uint32_t attn_single_blocks = 0;   // contexts of up to this many blocks go to one split (0 with a forced split factor)
   uint64_t *attn_tagged = nullptr;   // tagged split partials of the decode step kernel
   uint32_t *attn_plan = nullptr;     // this step's split plan of the decode attention (attn_plan_fill), or null
   uint64_t *attn_trace = nullptr;  // NERVA_HIP_ATTN_TRACE=1: per-layer stage timestamps of selected attention workgroups
@@ -170,7 +171,8 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
                                                        uint32_t max_steps, uint32_t hidden,
                                                        uint32_t vocab, float *x, const float *rope_freq,
                                                        float *rope_cs, uint32_t half_dim, uint32_t *attn_plan,
-                                                       const uint32_t *table, uint32_t attn_splits) {
+                                                       const uint32_t *table, uint32_t attn_splits,
+                                                       uint32_t attn_single_blocks) {
   const uint32_t pos = state[0];
   // the position goes into the attention plan even past the last step: the attention launches take
   // their step guard from there
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
   // this step's split plan of the decode attention, once for all layers
   if (attn_plan != nullptr && blockIdx.x == 0)
     for (uint32_t e = threadIdx.x; e < attn_splits * kAttnPlanWaves; e += kBlock)
-      attn_plan_fill(attn_plan, table, pos, attn_splits, e);
+      attn_plan_fill(attn_plan, table, pos, attn_splits, attn_single_blocks, e);
   // steps executed so far: the epochs of in-launch hand-overs derive from it (nobody reads it
   // in this launch)
   if (blockIdx.x == 0 && threadIdx.x == 0) state[2] = state[2] + 1u;
@@ -344,11 +346,11 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
     if (s->dtype == kBF16)
       hipLaunchKernelGGL(embed_kernel<kBF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
                          s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
-                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits);
+                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits, s->attn_single_blocks);
     else
       hipLaunchKernelGGL(embed_kernel<kF16>, dim3(blocks), dim3(kBlock), 0, st, s->emb, s->prompt,
                          s->slots, s->state, s->max_ctx, s->hidden, s->vocab, s->x, rope_freq, s->rope_cs,
-                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits);
+                         s->head_dim / 2, s->attn_plan, s->table, s->attn_splits, s->attn_single_blocks);
     err = hipGetLastError();
     if (prof && err == hipSuccess) err = prof->after();
     if (err != hipSuccess) return err;
@@ -393,6 +395,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       p.layer = l;
       p.block_count = s->block_count;
       p.splits = s->attn_splits;
+      p.single_split_blocks = s->attn_single_blocks;
       p.eps = s->eps;
       p.cursor = s->state;
       p.max_steps = s->max_ctx;
@@ -959,8 +962,11 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint32_t block_count = (s->max_ctx + kKvBlockTokens - 1) / kKvBlockTokens;
   s->block_count = block_count;
   s->attn_splits = attn_default_splits(s->kv_heads, block_count);
-  if (const int want = tuning(kTuneAttnSplits); want >= 1 && want <= static_cast<int>(kAttnMaxSplits))
+  s->attn_single_blocks = kAttnSingleSplitBlocks;
+  if (const int want = tuning(kTuneAttnSplits); want >= 1 && want <= static_cast<int>(kAttnMaxSplits)) {
     s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
+    s->attn_single_blocks = 0;  // a forced factor holds at every context length
+  }
 
   Carver c;
   const uint64_t kv_half = L * block_count * KV * kKvBlockTokens * 2;

@@ -462,9 +462,11 @@ int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *r, void *str
   p.layer = r->layer;
   p.block_count = r->block_count;
   p.splits = attn_default_splits(r->kv_heads, r->block_count);
+  p.single_split_blocks = kAttnSingleSplitBlocks;
   if (r->splits != 0) {
     if (r->splits > kAttnMaxSplits || r->splits > r->block_count) return finish(hipErrorInvalidValue, hip_error);
     p.splits = r->splits;
+    p.single_split_blocks = 0;  // the caller's factor holds at every context length
   }
   p.eps = r->rms_eps;
   p.cursor = nullptr;
