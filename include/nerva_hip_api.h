@@ -719,7 +719,8 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
  * (1: the lean GEMV's exact start-up waits wherever they can run, 2: nowhere), "moe_down_shared_first" (2: the
  * MoE down launch walks the shared expert last instead of first), "gemv_workgroup_waves" (4|16: waves per
  * workgroup of every lean GEMV launch), "gemv_x_registers" (2: the lean GEMV never keeps the input vector in
- * registers). Values a kernel
+ * registers), "prefill_block_tokens" (128: sessions created afterwards prefill in 128-token blocks even where
+ * the 256-token blocks apply). Values a kernel
  * cannot take are ignored where they are read. -1 for an unknown name. */
 int nerva_hip_test_set_tuning(const char *name, int32_t value);
 

@@ -129,7 +129,7 @@ struct NervaHipHfDecodeSequenceSession {
   hipGraph_t graph[3] = {nullptr, nullptr, nullptr};
   hipGraphExec_t exec[3] = {nullptr, nullptr, nullptr};
   uint64_t graph_nodes[3] = {0, 0, 0};
-  // prompt blocks: up to kGemmMaxTokens prompt tokens per pass through the layers (weights streamed
+  // prompt blocks: up to prefill_block_tokens prompt tokens per pass through the layers (weights streamed
   // once per block on the matrix cores); false = one prompt step per token
   bool block_prefill = false;
   // the multi-row kernels take this model's shapes (prompt blocks and batch steps need it)
@@ -142,6 +142,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint64_t pattn_ws_stride = 0;
   char *pgemm_ws = nullptr;        // partial sums of the K-sliced projections of a prompt block
   uint64_t pgemm_ws_bytes = 0;
+  uint32_t prefill_block_tokens = kGemmMaxTokens;   // tokens per prompt block: 256 where every projection has the kernel for it
   SamplerDev sampler{};            // normalised configuration of the active sequence
   SamplerDev *sampler_dev = nullptr;
   uint64_t *sampler_keys = nullptr;
@@ -686,7 +687,7 @@ uint32_t block_operand_tiles(uint32_t tokens) {
   return operand ? gemm_packed_tiles(tokens) : 0u;
 }
 
-// Prompt tokens 0 .. count-1 through every layer in blocks of up to kGemmMaxTokens tokens, with the
+// Prompt tokens 0 .. count-1 through every layer in blocks of up to prefill_block_tokens tokens, with the
 // prompt staging (16-bit hidden state between layers, prefill_kernels.cu:494-508): per block and
 // layer one RMSNorm launch, the qkv projection as a multi-row GEMM, the K/V rows of the block into the
 // cache, the attention of all its tokens in one launch (token z attends to keys 0 .. first + z), and
@@ -707,8 +708,8 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   const uint32_t prompt_splits = want_prompt_splits >= 1 && want_prompt_splits <= static_cast<int>(kAttnMaxSplits)
                                      ? static_cast<uint32_t>(want_prompt_splits)
                                      : 0u;
-  for (uint32_t first = 0; err == hipSuccess && first < count; first += kGemmMaxTokens) {
-    const uint32_t T = std::min<uint32_t>(kGemmMaxTokens, count - first);
+  for (uint32_t first = 0; err == hipSuccess && first < count; first += s->prefill_block_tokens) {
+    const uint32_t T = std::min<uint32_t>(s->prefill_block_tokens, count - first);
     const uint32_t tiles = block_operand_tiles(T);
     if (s->dtype == kBF16)
       hipLaunchKernelGGL(embed_rows_kernel<kBF16>, dim3(T), dim3(kBlock), 0, st, s->emb, s->prompt, first, H, s->vocab,
@@ -990,7 +991,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_attn_plan = c.take(attn_plan_bytes(kAttnMaxSplits));
   const uint64_t off_attn_tagged = c.take(attn_step_workspace_bytes(s->heads));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
-  const uint64_t pT = kGemmMaxTokens;
+  const uint64_t pT = kGemmWideMaxTokens;
   const uint64_t off_px = c.take(pT * H * 4);
   const uint64_t off_pr = c.take(pT * H * 4);
   const uint64_t off_pqkv = c.take(pT * (A + 2 * KV) * 4);
@@ -1080,6 +1081,15 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->pattn_ws_stride = pattn_ws_stride;
   s->pgemm_ws = s->arena + off_pgemm_ws;
   s->pgemm_ws_bytes = pgemm_ws_bytes;
+  // 256-token prompt blocks where all four projections of a layer have the kernel for them (twice the tokens per
+  // weight byte): Qwen3-8B widths qualify; other widths keep 128-token blocks.
+  const uint32_t wideT = kGemmWideMaxTokens;
+  const bool wide = gemm_wide_slices(kGemmF32, static_cast<uint32_t>(A + 2 * KV), s->hidden, wideT, pgemm_ws_bytes) != 0 &&
+                    gemm_wide_slices(kGemmResidual, s->hidden, static_cast<uint32_t>(A), wideT, pgemm_ws_bytes) != 0 &&
+                    gemm_wide_slices(kGemmSwiglu, s->intermediate, s->hidden, wideT, pgemm_ws_bytes) != 0 &&
+                    gemm_wide_slices(kGemmResidual, s->hidden, s->intermediate, wideT, pgemm_ws_bytes) != 0;
+  s->prefill_block_tokens =
+      wide && block_operand_tiles(wideT) != 0 && tuning(kTunePrefillBlockTokens) != 128 ? wideT : kGemmMaxTokens;
   s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
   s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
   {
@@ -1134,7 +1144,7 @@ void fill_create_result(const Session *s, NervaHipHfDecodeSequenceSessionCreateR
   out->vocab_size = s->vocab;
   out->layer_count = s->layers;
   out->max_context_tokens = s->max_ctx;
-  out->prefill_chunk_tokens = s->block_prefill ? kGemmMaxTokens : 1;
+  out->prefill_chunk_tokens = s->block_prefill ? s->prefill_block_tokens : 1;
   out->head_threads = kBlock;
   out->resident_weight_bytes = s->resident_weight_bytes;
   out->planned_weight_blocks = s->planned_weight_blocks;

@@ -1,5 +1,6 @@
-// Multi-row projection for token blocks of 17..128 rows with X in matrix-operand order: the X operand is
-// shared through LDS instead of being fetched by every wave (see gemm_rows.cuh).
+// Multi-row projection for token blocks of 17..256 rows with X in matrix-operand order: the X operand is
+// shared through LDS instead of being fetched by every wave (see gemm_rows.cuh). Two kernels: up to 128 rows
+// (gemm_block_kernel) and 129..256 rows (gemm_wide_kernel, further down).
 //
 // gemm_rows_kernel gives a workgroup 16 weight rows over the whole K and lets its 8 waves split K, so
 // every wave fetches its own X pieces from L2: per matrix instruction 0.6 vector-memory reads, and the
@@ -292,7 +293,8 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 
 // One thread per token and four consecutive output rows: partial sums in slice order, then the epilogue.
 template <uint32_t DT, int EPI>
-__global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p, const float *partials, uint32_t kslices) {
+__global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p, const float *partials, uint32_t kslices,
+                                                                uint32_t tokcap) {
   const uint32_t quads = p.rows / 4u;
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
   if (i >= quads * p.tokens) return;
@@ -300,7 +302,7 @@ __global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p
   const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
   f32x4_t y = {0.0f, 0.0f, 0.0f, 0.0f}, up = {0.0f, 0.0f, 0.0f, 0.0f};
   for (uint32_t s = 0; s < kslices; ++s) {
-    const float *at = partials + (static_cast<uint64_t>(s) * kBTokCap + t) * wrows + row;
+    const float *at = partials + (static_cast<uint64_t>(s) * tokcap + t) * wrows + row;
     const float4 a = *reinterpret_cast<const float4 *>(at);
     y[0] += a.x;
     y[1] += a.y;
@@ -342,7 +344,7 @@ hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t ks
   if (err == hipSuccess && kslices > 1) {
     const uint32_t threads = p.rows / 4u * p.tokens;
     hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
-                       static_cast<const float *>(partials), kslices);
+                       static_cast<const float *>(partials), kslices, kBTokCap);
     err = hipGetLastError();
   }
   return err;
@@ -354,6 +356,219 @@ hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t ks
     case 2: return launch_block_tt<DT, EPI, NR, 2>(p, partials, kslices, stream);
     case 4: return launch_block_tt<DT, EPI, NR, 4>(p, partials, kslices, stream);
     case 8: return launch_block_tt<DT, EPI, NR, 8>(p, partials, kslices, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Token blocks of 129..256 rows (X in operand order with 16 token tiles). At 128 rows a byte of W meets 128
+// tokens and the kernel above waits for HBM four fifths of the time; here it meets 256, and the matrix cores
+// and the weight stream take about the same time. A workgroup is four PAIRS of waves. A pair owns two 16-row
+// tiles of W (SwiGLU: a gate tile and its up tile) in LDS: each of its waves fetches one of them (global memory
+// -> registers, four K-blocks requested ahead) and parks it there, and both read both back as A operands - one
+// wave for the block's token tiles 0..7, the other for tiles 8..15, so a wave holds 2 x 8 tiles of f32
+// accumulators like the kernel above, in under 256 registers: two waves per SIMD, one of which multiplies while
+// the other waits for LDS. The K-block of X (128 columns x 256 tokens = 64 KiB, contiguous in operand order) is
+// copied into LDS once per workgroup by all eight waves, requested one block ahead (L2 hits).
+// Per block: barrier (everyone has finished the previous block's products), the waves park their W tile and
+// their X pieces, barrier, products - with the requests for the next X block and for the W block four ahead
+// between them, in the order they are awaited in.
+constexpr int kWPairs = 4;
+constexpr int kWThreads = kWPairs * 2 * kWave;
+constexpr int kWTiles = 16;                  // token tiles of the block's operand-order layout
+constexpr uint32_t kWTokCap = 256;           // token rows at most; the token stride of this kernel's partial sums
+constexpr size_t kWLdsBytes = static_cast<size_t>(kBSteps) * kWTiles * kWave * sizeof(u32x4_t) +
+                              static_cast<size_t>(kWPairs) * 2 * kBWTile * sizeof(uint16_t);
+
+template <uint32_t DT, int EPI>
+__global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams p, float *partials) {
+  constexpr int kStageVec = kBSteps * kWTiles * kWave;   // 16-byte pieces of one X block: 4096 = 64 KiB
+  constexpr int kFill = kStageVec / kWThreads;           // pieces per thread and block
+  constexpr int kHalf = kWTiles / 2;                     // token tiles per wave
+  extern __shared__ __align__(16) unsigned char smem[];
+  u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int pair = wave % kWPairs, half = wave / kWPairs;
+  uint16_t *wtile = reinterpret_cast<uint16_t *>(smem + kStageVec * sizeof(u32x4_t)) + pair * 2 * kBWTile;   // the pair's two tiles
+  const uint32_t n = lane & 15, q = lane >> 4;
+  const uint32_t cols = p.cols, T = p.tokens;
+  const uint32_t kslices = gridDim.y, kper = cols / kslices, k0 = blockIdx.y * kper, nblk = kper / kBK;
+
+  uint32_t trow[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    trow[j] = EPI == kGemmSwiglu ? j * p.rows + blockIdx.x * (16u * kWPairs) + pair * 16u
+                                 : blockIdx.x * (32u * kWPairs) + (pair * 2 + j) * 16u;
+  // the tile this wave fetches: a wave-uniform base plus a per-lane offset that never changes
+  const char *wbase = reinterpret_cast<const char *>(p.w) + (static_cast<uint64_t>(trow[half]) * cols + k0) * sizeof(uint16_t);
+  const uint32_t wlane = (q * cols + n * 8u) * static_cast<uint32_t>(sizeof(uint16_t));
+  uint16_t *park_at = wtile + half * kBWTile + q * kBRowStride + n * 8;
+  const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
+  const char *xbase = reinterpret_cast<const char *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kWTiles * kWave) * sizeof(u32x4_t);
+  const uint32_t xlane = threadIdx.x * static_cast<uint32_t>(sizeof(u32x4_t));
+  const u32x4_t *b_read = stage + half * kHalf * kWave + lane;
+
+  u32x4_t areg[kBRing][4];
+  u32x4_t xreg[kFill];
+  f32x4_t acc[2][kHalf];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int c = 0; c < kHalf; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+#define NV_WD_W1(BUF, BLK, I)                                                                       \
+  areg[BUF][I] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(                      \
+      wbase + (static_cast<uint64_t>(4 * (I)) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
+#define NV_WD_W(BUF, BLK) _Pragma("unroll") for (int i = 0; i < 4; ++i) NV_WD_W1(BUF, BLK, i)
+#define NV_WD_WPARK(BUF) \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t *>(park_at + 4 * i * kBRowStride) = areg[BUF][i]
+#define NV_WD_X1(BLK, I)                                                                            \
+  xreg[I] = *reinterpret_cast<const u32x4_t *>(                                                      \
+      xbase + (static_cast<uint64_t>(BLK) * kStageVec + (I) * kWThreads) * sizeof(u32x4_t) + xlane)
+#define NV_WD_X(BLK) _Pragma("unroll") for (int i = 0; i < kFill; ++i) NV_WD_X1(BLK, i)
+#define NV_WD_XPARK() _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[i * kWThreads + threadIdx.x] = xreg[i]
+#define NV_WD_READ_A(S, A) \
+  _Pragma("unroll") for (int j = 0; j < 2; ++j) A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32)
+#define NV_WD_READ_B(S, C0) \
+  _Pragma("unroll") for (int c = C0; c < C0 + kHalf / 2; ++c) b[c] = b_read[((S) * kWTiles + c) * kWave]
+#define NV_WD_PRODUCTS(A, C0)                                                                       \
+  _Pragma("unroll") for (int c = C0; c < C0 + kHalf / 2; ++c)                                       \
+      _Pragma("unroll") for (int j = 0; j < 2; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
+  // request slots between the products, two requests each: slots 0..3 the next X block's eight pieces, slots
+  // 4 and 5 the four rows-of-four of the W block four ahead (the order they are awaited in)
+#define NV_WD_SLOT(K, BUF, XEN, XBLK, WEN, WBLK)                                                    \
+  if constexpr ((K) < 4) {                                                                          \
+    if constexpr (XEN) {                                                                            \
+      NV_WD_X1(XBLK, 2 * (K));                                                                      \
+      NV_WD_X1(XBLK, 2 * (K) + 1);                                                                  \
+    }                                                                                               \
+  } else if constexpr (WEN && (K) < 6) {                                                            \
+    NV_WD_W1(BUF, WBLK, 2 * ((K) - 4));                                                             \
+    NV_WD_W1(BUF, WBLK, 2 * ((K) - 4) + 1);                                                         \
+  }
+#define NV_WD_STEP(S, ACUR, ANEXT, LAST, BUF, XEN, XBLK, WEN, WBLK)                                 \
+  if (!(LAST)) { NV_WD_READ_A((S) + 1, ANEXT); }                                                    \
+  NV_WD_PRODUCTS(ACUR, 0);                                                                          \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  if (!(LAST)) { NV_WD_READ_B((S) + 1, 0); }                                                        \
+  NV_WD_SLOT(2 * (S), BUF, XEN, XBLK, WEN, WBLK)                                                    \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  NV_WD_PRODUCTS(ACUR, kHalf / 2);                                                                  \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  if (!(LAST)) { NV_WD_READ_B((S) + 1, kHalf / 2); }                                                \
+  NV_WD_SLOT(2 * (S) + 1, BUF, XEN, XBLK, WEN, WBLK)                                                \
+  __builtin_amdgcn_sched_barrier(0)
+#define NV_WD_ITER(BUF, XEN, XBLK, WEN, WBLK)                                                       \
+  do {                                                                                              \
+    __syncthreads();                                                                                \
+    NV_WD_WPARK(BUF);                                                                               \
+    NV_WD_XPARK();                                                                                  \
+    __syncthreads();                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    u32x4_t a0[2], a1[2], b[kHalf];                                                                 \
+    NV_WD_READ_A(0, a0);                                                                            \
+    NV_WD_READ_B(0, 0);                                                                             \
+    NV_WD_READ_B(0, kHalf / 2);                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    NV_WD_STEP(0, a0, a1, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
+    NV_WD_STEP(1, a1, a0, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
+    NV_WD_STEP(2, a0, a1, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
+    NV_WD_STEP(3, a1, a0, true, BUF, XEN, XBLK, WEN, WBLK);                                         \
+  } while (0)
+
+  NV_WD_W(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  NV_WD_X(0);
+  __builtin_amdgcn_sched_barrier(0);
+  NV_WD_W(1, 1);
+  NV_WD_W(2, 2);
+  NV_WD_W(3, 3);
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t blk = 0;
+  for (; blk + 4 < nblk; blk += 4) {
+    NV_WD_ITER(0, true, blk + 1, true, blk + 4);
+    NV_WD_ITER(1, true, blk + 2, true, blk + 5);
+    NV_WD_ITER(2, true, blk + 3, true, blk + 6);
+    NV_WD_ITER(3, true, blk + 4, true, blk + 7);
+  }
+  NV_WD_ITER(0, true, blk + 1, false, 0);
+  NV_WD_ITER(1, true, blk + 2, false, 0);
+  NV_WD_ITER(2, true, blk + 3, false, 0);
+  NV_WD_ITER(3, false, 0, false, 0);
+#undef NV_WD_W1
+#undef NV_WD_W
+#undef NV_WD_WPARK
+#undef NV_WD_X1
+#undef NV_WD_X
+#undef NV_WD_XPARK
+#undef NV_WD_READ_A
+#undef NV_WD_READ_B
+#undef NV_WD_PRODUCTS
+#undef NV_WD_SLOT
+#undef NV_WD_STEP
+#undef NV_WD_ITER
+
+  // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
+  if (kslices == 1) {
+#pragma unroll
+    for (int c = 0; c < kHalf; ++c) {
+      const uint32_t t = (half * kHalf + c) * 16u + n;
+      if (t < T) {
+        if constexpr (EPI == kGemmSwiglu) {
+          block_epilogue<DT, EPI>(p, t, trow[0] + q * 4u, acc[0][c], acc[1][c]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) block_epilogue<DT, EPI>(p, t, trow[j] + q * 4u, acc[j][c], acc[j][c]);
+        }
+      }
+    }
+  } else {
+    const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
+    float *part = partials + static_cast<uint64_t>(blockIdx.y) * kWTokCap * wrows;
+#pragma unroll
+    for (int c = 0; c < kHalf; ++c) {
+      const uint32_t t = (half * kHalf + c) * 16u + n;
+      if (t < T) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          *reinterpret_cast<float4 *>(part + static_cast<uint64_t>(t) * wrows + trow[j] + q * 4u) =
+              make_float4(acc[j][c][0], acc[j][c][1], acc[j][c][2], acc[j][c][3]);
+      }
+    }
+  }
+}
+
+template <uint32_t DT, int EPI>
+hipError_t launch_wide(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kWPairs : 32u * kWPairs;
+  // more than the default dynamic LDS limit: raised once per kernel (never under stream capture)
+  static std::once_flag once;
+  static hipError_t raised = hipSuccess;
+  std::call_once(once, [] {
+    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<DT, EPI>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kWLdsBytes));
+  });
+  if (raised != hipSuccess) return raised;
+  hipLaunchKernelGGL((gemm_wide_kernel<DT, EPI>), dim3(p.rows / wg_rows, kslices), dim3(kWThreads), kWLdsBytes, stream, p,
+                     partials);
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess && kslices > 1) {
+    const uint32_t threads = p.rows / 4u * p.tokens;
+    hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
+                       static_cast<const float *>(partials), kslices, kWTokCap);
+    err = hipGetLastError();
+  }
+  return err;
+}
+
+template <uint32_t DT>
+hipError_t launch_wide_dt(int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
+  float *partials = static_cast<float *>(p.workspace);
+  switch (epilogue) {
+    case kGemmF32: return launch_wide<DT, kGemmF32>(p, partials, kslices, stream);
+    case kGemmResidual: return launch_wide<DT, kGemmResidual>(p, partials, kslices, stream);
+    case kGemmSwiglu: return launch_wide<DT, kGemmSwiglu>(p, partials, kslices, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -408,9 +623,38 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   return plan;
 }
 
+// Blocks of 129..256 rows: K slices of the kernel with wave pairs, or 0 where it does not take the shape.
+// Enough workgroups for three quarters of the CUs (a gate/up pair of Qwen3-8B width has 192 row groups and
+// runs unsliced), each slice a whole number of rings of K-blocks, the partial sums within the workspace.
+uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
+  const uint32_t wg_rows = epilogue == kGemmSwiglu ? 16u * kWPairs : 32u * kWPairs;
+  if (tokens <= kBTokCap || tokens > kWTokCap || rows % wg_rows != 0 || cols % (kBRing * kBK) != 0) return 0;
+  const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
+  const uint32_t groups = rows / wg_rows;
+  uint32_t slices = 1;
+  const int want = tuning(kTuneGemmBlockSlices);
+  if (want > 0 && cols % (static_cast<uint32_t>(want) * kBRing * kBK) == 0) {
+    slices = static_cast<uint32_t>(want);
+  } else {
+    while (groups * slices < 192u && slices < 8u && cols % (slices * 2u * kBRing * kBK) == 0) slices *= 2u;
+  }
+  while (slices > 1 && static_cast<uint64_t>(slices) * kWTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
+  return slices;
+}
+
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {
-  // room for 8 slices of the widest plain projection or 2 of a gate/up pair of that width
-  return static_cast<uint64_t>(8) * kBTokCap * rows_max * sizeof(float);
+  // room for 8 slices of the widest plain projection (or 2 of a gate/up pair of that width) at the wide kernel's
+  // token stride
+  return static_cast<uint64_t>(8) * kWTokCap * rows_max * sizeof(float);
+}
+
+hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
+  if (kslices == 0 || p.x_packed != static_cast<uint32_t>(kWTiles) || p.tokens <= kBTokCap || p.tokens > kWTokCap)
+    return hipErrorInvalidValue;
+  if (kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
+  if (dtype == kBF16) return launch_wide_dt<kBF16>(epilogue, p, kslices, stream);
+  if (dtype == kF16) return launch_wide_dt<kF16>(epilogue, p, kslices, stream);
+  return hipErrorInvalidValue;
 }
 
 hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,

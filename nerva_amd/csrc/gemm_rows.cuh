@@ -22,7 +22,8 @@
 
 namespace nv {
 
-constexpr uint32_t kGemmMaxTokens = 128;
+constexpr uint32_t kGemmMaxTokens = 128;       // token rows of a block in any layout
+constexpr uint32_t kGemmWideMaxTokens = 256;   // token rows of a block in operand order, where gemm_wide_slices takes the shape
 
 // Operand order of a block of token rows X[t][k] (16-bit), the layout the multi-row GEMM reads fastest:
 // for every K-step of 32 columns and every tile of 16 tokens the 64 lanes' 16-byte pieces in lane order,
@@ -33,7 +34,7 @@ __host__ __device__ __forceinline__ uint64_t gemm_x_packed_index(uint32_t tiles,
 }
 // Token tiles the GEMM works with for a block of `tokens` rows (its X buffer in operand order has as many).
 __host__ __device__ __forceinline__ uint32_t gemm_packed_tiles(uint32_t tokens) {
-  return tokens > 64u ? 8u : tokens > 32u ? 4u : 2u;
+  return tokens > 128u ? 16u : tokens > 64u ? 8u : tokens > 32u ? 4u : 2u;
 }
 enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
 
@@ -71,6 +72,11 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max);
 hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,
                              hipStream_t stream);
+// Blocks of 129..kGemmWideMaxTokens rows in operand order (16 token tiles): K slices the kernel for them
+// would use for a shape (more than one needs slices x 256 x W rows f32 of workspace), 0 = shape not taken
+// (rows a multiple of 128, gate/up pairs of 64; cols a multiple of 512 per slice). launch_gemm_rows uses it by itself.
+uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
+hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
 
 // x16[t] = round16(x[t] * rsqrt(mean(x[t]^2) + eps) * gamma) for `tokens` rows of `cols` f32 values.
 // packed_tiles != 0: out16 in operand order (gemm_x_packed_index) with that many token tiles.

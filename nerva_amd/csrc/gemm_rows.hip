@@ -297,7 +297,12 @@ bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens) {
 }
 
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream) {
-  if (p.w == nullptr || p.x16 == nullptr || !gemm_rows_supported(p.rows, p.cols, p.tokens)) return hipErrorInvalidValue;
+  // more than kGemmMaxTokens rows: only in operand order and only where the kernel for wide blocks takes the shape
+  const uint32_t wide_slices = p.tokens > kGemmMaxTokens && p.x_packed != 0
+                                   ? gemm_wide_slices(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0)
+                                   : 0u;
+  if (p.w == nullptr || p.x16 == nullptr) return hipErrorInvalidValue;
+  if (wide_slices == 0 && !gemm_rows_supported(p.rows, p.cols, p.tokens)) return hipErrorInvalidValue;
   if (!aligned16(p.w) || !aligned16(p.x16)) return hipErrorInvalidValue;
   if ((epilogue == kGemmF32 || epilogue == kGemmResidual) && p.out_f32 == nullptr) return hipErrorInvalidValue;
   if (epilogue == kGemmResidual && p.residual == nullptr) return hipErrorInvalidValue;
@@ -307,6 +312,7 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
   if (p.out_packed_tiles != 0 && (epilogue != kGemmSwiglu || p.out_packed_tiles * 16u < p.tokens)) return hipErrorInvalidValue;
   if (p.x_packed != 0 && p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;   // tiles the kernel will assume
   if (dtype != kBF16 && dtype != kF16) return hipErrorInvalidValue;
+  if (wide_slices != 0) return launch_gemm_wide(dtype, epilogue, p, wide_slices, stream);
   if (p.x_packed != 0) {   // blocks in operand order: the kernel that shares X through LDS, where its plan takes the shape
     const GemmBlockPlan plan = gemm_block_plan(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0);
     if (plan.kslices != 0) return launch_gemm_block(dtype, epilogue, p, plan, stream);

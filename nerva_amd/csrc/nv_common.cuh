@@ -138,6 +138,7 @@ enum TuningKnob : int {
   kTuneMoeDownSharedFirst,   // lean MoE down: 2 = walk the shared expert last, as the caller orders the slots
   kTuneGemvWorkgroupWaves,   // lean GEMV: waves per workgroup for every launch (4 or 16)
   kTuneGemvXRegisters,       // lean GEMV: 2 = never keep the input vector in registers
+  kTunePrefillBlockTokens,   // prompt blocks of a session: 128 = never the 256-token blocks (read at session create)
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

@@ -31,7 +31,7 @@ constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_sp
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                                                   "moe_down_shared_first", "gemv_workgroup_waves",
-                                                  "gemv_x_registers"};
+                                                  "gemv_x_registers",  "prefill_block_tokens"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }

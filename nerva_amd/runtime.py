@@ -270,7 +270,7 @@ def argmax_static(logits_buf, count, token_buf):
 
 def gemm_operand_slots(tokens):
     """Token slots of a buffer in matrix-operand order for a block of `tokens` rows."""
-    return 32 if tokens <= 32 else 64 if tokens <= 64 else 128
+    return 32 if tokens <= 32 else 64 if tokens <= 64 else 128 if tokens <= 128 else 256
 
 
 def gemm_operand_order(x, tokens=None):
@@ -293,8 +293,10 @@ def gemm_operand_order(x, tokens=None):
 def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None, residual=None, out_f32=None,
               out16=None, round_output=False, sync=True, input_operand_order=False, output16_operand_order=False,
               workspace=None):
-    """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once).
-    `workspace`: optional DeviceBuffer of gemm_rows_workspace_bytes(rows) for the K-sliced large-block kernel."""
+    """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once); up to 256 rows
+    with the input in operand order where the kernel for wide blocks takes the shape (rows a multiple of 128,
+    gate/up pairs of 64, cols of 512).
+    `workspace`: optional DeviceBuffer of gemm_rows_workspace_bytes(rows) for the K-sliced large-block kernels."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()
     if workspace is not None:

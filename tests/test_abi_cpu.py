@@ -307,7 +307,7 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
         N.gemv_launch_shape(0, 0, 0, 64)
     for name in ("attn_splits", "batch_splits", "prompt_splits", "gemm_row_tiles", "gemm_k_waves",
                  "gemm_block_slices", "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
-                 "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers"):
+                 "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers", "prefill_block_tokens"):
         N.Device.set_tuning(name, 2)
         N.Device.set_tuning(name, 0)
     with pytest.raises(ValueError):

@@ -234,6 +234,10 @@ def test_gemm_rows_rejects_unsupported_shapes():
             N.gemm_rows(BF16, w, rows, cols, tokens, x, out_f32=y)
     with pytest.raises(RuntimeError):      # rows off the 16-row grid: no residual added in place
         N.gemm_rows(BF16, w, 24, 2048, 4, x, epilogue=1, residual=y, out_f32=y)
+    # more than 128 token rows: operand order only, rows a multiple of 128 (gate/up pairs of 64), 256 rows at most
+    for rows, cols, tokens, epi in ((64, 2048, 200, 0), (128, 2048, 257, 0), (32, 2048, 130, 2)):
+        with pytest.raises(RuntimeError):
+            N.gemm_rows(BF16, w, rows, cols, tokens, x, epilogue=epi, out_f32=y, out16=y, input_operand_order=True)
 
 
 @pytest.mark.parametrize("full", [False, True])
@@ -823,10 +827,13 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("rows,cols,tokens", [(64, 2048, 65), (192, 2048, 100), (4096, 4096, 128), (6144, 4096, 127),
                                                (4096, 12288, 128), (192, 2048, 17), (64, 2048, 33), (4096, 4096, 32),
-                                               (6144, 4096, 48), (4096, 12288, 64)])
+                                               (6144, 4096, 48), (4096, 12288, 64),
+                                               (128, 2048, 129), (256, 4096, 200), (4096, 4096, 256), (6144, 4096, 255),
+                                               (4096, 12288, 256)])
 def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     """More than 16 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
-    X from LDS (2, 4 or 8 token tiles). Every token row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
+    X from LDS (2, 4, 8 or - blocks of 129..256 rows, wave pairs sharing the W tiles - 16 token tiles). Every token
+    row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
     dtype = BF16
     rng = np.random.default_rng(rows + cols + tokens)
     if rows * cols > 1 << 22:
@@ -856,7 +863,8 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
 
 
 @pytest.mark.parametrize("sliced", [False, True])
-@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50)])
+@pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
+                                                 (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
