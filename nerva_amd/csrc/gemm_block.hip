@@ -29,8 +29,11 @@ constexpr int kBK = 128;                     // columns per K-block
 constexpr int kBSteps = kBK / 32;            // matrix-core K-steps per block
 constexpr int kBRing = 4;                    // W blocks a wave requests ahead at most (two with one row tile per wave)
 constexpr uint32_t kBTokCap = 128;           // token rows at most; also the token stride of the partial sums
-constexpr int kBRowStride = kBK + 8;         // LDS row stride of a W tile in elements: 16 B of padding keeps the
-                                             // 16 rows of an operand read on distinct banks
+constexpr int kBRowStride = kBK + 16;        // LDS row stride of a W tile in elements: 32 B of padding. A 16-byte LDS read is
+                                             // served 16 lanes at a time - lanes 0-3, 12-15, 20-23, 24-27 first, i.e. rows 0-3 and
+                                             // 12-15 of one K quarter with rows 4-11 of the next - and with 16 B of padding two
+                                             // lanes of every such group met in the same banks (4 extra cycles per operand read,
+                                             // a third of the kernel's LDS time by the bank-conflict counter); with 32 B they do not
 constexpr int kBWTile = 16 * kBRowStride;    // one 16-row block of W in LDS
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -409,7 +412,8 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
   const uint32_t xlane = threadIdx.x * static_cast<uint32_t>(sizeof(u32x4_t));
   const u32x4_t *b_read = stage + half * kHalf * kWave + lane;
 
-  u32x4_t areg[kBRing][4];
+  constexpr int kRing = 2;   // W blocks requested ahead (a block is about two microseconds of products)
+  u32x4_t areg[kRing][4];
   u32x4_t xreg[kFill];
   f32x4_t acc[2][kHalf];
 #pragma unroll
@@ -430,13 +434,13 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
 #define NV_WD_XPARK() _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[i * kWThreads + threadIdx.x] = xreg[i]
 #define NV_WD_READ_A(S, A) \
   _Pragma("unroll") for (int j = 0; j < 2; ++j) A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32)
-#define NV_WD_READ_B(S, C0) \
-  _Pragma("unroll") for (int c = C0; c < C0 + kHalf / 2; ++c) b[c] = b_read[((S) * kWTiles + c) * kWave]
-#define NV_WD_PRODUCTS(A, C0)                                                                       \
+#define NV_WD_READ_B(S, B) \
+  _Pragma("unroll") for (int c = 0; c < kHalf; ++c) B[c] = b_read[((S) * kWTiles + c) * kWave]
+#define NV_WD_PRODUCTS(A, B, C0)                                                                    \
   _Pragma("unroll") for (int c = C0; c < C0 + kHalf / 2; ++c)                                       \
-      _Pragma("unroll") for (int j = 0; j < 2; ++j) acc[j][c] = mfma_k32<DT>(A[j], b[c], acc[j][c])
+      _Pragma("unroll") for (int j = 0; j < 2; ++j) acc[j][c] = mfma_k32<DT>(A[j], B[c], acc[j][c])
   // request slots between the products, two requests each: slots 0..3 the next X block's eight pieces, slots
-  // 4 and 5 the four rows-of-four of the W block four ahead (the order they are awaited in)
+  // 4 and 5 the four rows-of-four of the W block kRing ahead (the order they are awaited in)
 #define NV_WD_SLOT(K, BUF, XEN, XBLK, WEN, WBLK)                                                    \
   if constexpr ((K) < 4) {                                                                          \
     if constexpr (XEN) {                                                                            \
@@ -447,16 +451,21 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
     NV_WD_W1(BUF, WBLK, 2 * ((K) - 4));                                                             \
     NV_WD_W1(BUF, WBLK, 2 * ((K) - 4) + 1);                                                         \
   }
-#define NV_WD_STEP(S, ACUR, ANEXT, LAST, BUF, XEN, XBLK, WEN, WBLK)                                 \
-  if (!(LAST)) { NV_WD_READ_A((S) + 1, ANEXT); }                                                    \
-  NV_WD_PRODUCTS(ACUR, 0);                                                                          \
+  // The operands of K-step s + 1 (two A pieces, eight B pieces) are requested from LDS before the sixteen
+  // products of step s are issued: a wave gets a 1 KiB LDS read through about every 30 cycles, so ten reads
+  // take longer than half a step's products.
+#define NV_WD_STEP(S, ACUR, ANEXT, BCUR, BNEXT, LAST, BUF, XEN, XBLK, WEN, WBLK)                    \
+  if (!(LAST)) {                                                                                    \
+    NV_WD_READ_A((S) + 1, ANEXT);                                                                   \
+    NV_WD_READ_B((S) + 1, BNEXT);                                                                   \
+  }                                                                                                 \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  if (!(LAST)) { NV_WD_READ_B((S) + 1, 0); }                                                        \
+  NV_WD_PRODUCTS(ACUR, BCUR, 0);                                                                    \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
   NV_WD_SLOT(2 * (S), BUF, XEN, XBLK, WEN, WBLK)                                                    \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  NV_WD_PRODUCTS(ACUR, kHalf / 2);                                                                  \
+  NV_WD_PRODUCTS(ACUR, BCUR, kHalf / 2);                                                            \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  if (!(LAST)) { NV_WD_READ_B((S) + 1, kHalf / 2); }                                                \
   NV_WD_SLOT(2 * (S) + 1, BUF, XEN, XBLK, WEN, WBLK)                                                \
   __builtin_amdgcn_sched_barrier(0)
 #define NV_WD_ITER(BUF, XEN, XBLK, WEN, WBLK)                                                       \
@@ -466,15 +475,14 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
     NV_WD_XPARK();                                                                                  \
     __syncthreads();                                                                                \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    u32x4_t a0[2], a1[2], b[kHalf];                                                                 \
+    u32x4_t a0[2], a1[2], b0[kHalf], b1[kHalf];                                                     \
     NV_WD_READ_A(0, a0);                                                                            \
-    NV_WD_READ_B(0, 0);                                                                             \
-    NV_WD_READ_B(0, kHalf / 2);                                                                     \
+    NV_WD_READ_B(0, b0);                                                                            \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    NV_WD_STEP(0, a0, a1, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
-    NV_WD_STEP(1, a1, a0, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
-    NV_WD_STEP(2, a0, a1, false, BUF, XEN, XBLK, WEN, WBLK);                                        \
-    NV_WD_STEP(3, a1, a0, true, BUF, XEN, XBLK, WEN, WBLK);                                         \
+    NV_WD_STEP(0, a0, a1, b0, b1, false, BUF, XEN, XBLK, WEN, WBLK);                                \
+    NV_WD_STEP(1, a1, a0, b1, b0, false, BUF, XEN, XBLK, WEN, WBLK);                                \
+    NV_WD_STEP(2, a0, a1, b0, b1, false, BUF, XEN, XBLK, WEN, WBLK);                                \
+    NV_WD_STEP(3, a1, a0, b1, b0, true, BUF, XEN, XBLK, WEN, WBLK);                                 \
   } while (0)
 
   NV_WD_W(0, 0);
@@ -482,20 +490,14 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
   NV_WD_X(0);
   __builtin_amdgcn_sched_barrier(0);
   NV_WD_W(1, 1);
-  NV_WD_W(2, 2);
-  NV_WD_W(3, 3);
   __builtin_amdgcn_sched_barrier(0);
   uint32_t blk = 0;
-  for (; blk + 4 < nblk; blk += 4) {
-    NV_WD_ITER(0, true, blk + 1, true, blk + 4);
-    NV_WD_ITER(1, true, blk + 2, true, blk + 5);
-    NV_WD_ITER(2, true, blk + 3, true, blk + 6);
-    NV_WD_ITER(3, true, blk + 4, true, blk + 7);
+  for (; blk + 2 < nblk; blk += 2) {
+    NV_WD_ITER(0, true, blk + 1, true, blk + 2);
+    NV_WD_ITER(1, true, blk + 2, true, blk + 3);
   }
   NV_WD_ITER(0, true, blk + 1, false, 0);
-  NV_WD_ITER(1, true, blk + 2, false, 0);
-  NV_WD_ITER(2, true, blk + 3, false, 0);
-  NV_WD_ITER(3, false, 0, false, 0);
+  NV_WD_ITER(1, false, 0, false, 0);
 #undef NV_WD_W1
 #undef NV_WD_W
 #undef NV_WD_WPARK
