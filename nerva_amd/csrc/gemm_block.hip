@@ -376,17 +376,29 @@ hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t ks
 // Per block: barrier (everyone has finished the previous block's products), the waves park their W tile and
 // their X pieces, barrier, products - with the requests for the next X block and for the W block four ahead
 // between them, in the order they are awaited in.
-constexpr int kWPairs = 4;
-constexpr int kWThreads = kWPairs * 2 * kWave;
+// Pairs per workgroup: 4 or 3, whichever divides the rows (plain projections take 3 first: the qkv projection
+// of Qwen3-8B width is then 64 row groups x 4 K slices = 256 workgroups, 30.0 us against 31.1 with 48 x 4; a
+// gate/up pair takes 4 first: 192 workgroups of 64 + 64 rows measured 74.1 us, 256 of 48 + 48 rows 77.9 - every
+// workgroup fetches the whole X block, whatever its rows).
 constexpr int kWTiles = 16;                  // token tiles of the block's operand-order layout
 constexpr uint32_t kWTokCap = 256;           // token rows at most; the token stride of this kernel's partial sums
-constexpr size_t kWLdsBytes = static_cast<size_t>(kBSteps) * kWTiles * kWave * sizeof(u32x4_t) +
-                              static_cast<size_t>(kWPairs) * 2 * kBWTile * sizeof(uint16_t);
+constexpr size_t wide_lds_bytes(int pairs) {
+  return static_cast<size_t>(kBSteps) * kWTiles * kWave * sizeof(u32x4_t) + static_cast<size_t>(pairs) * 2 * kBWTile * sizeof(uint16_t);
+}
+constexpr uint32_t wide_wg_rows(int epilogue, int pairs) { return (epilogue == kGemmSwiglu ? 16u : 32u) * pairs; }
+inline int wide_pairs(int epilogue, uint32_t rows) {
+  const int first = epilogue == kGemmSwiglu ? 4 : 3, second = 7 - first;
+  return rows % wide_wg_rows(epilogue, first) == 0 ? first : rows % wide_wg_rows(epilogue, second) == 0 ? second : 0;
+}
 
-template <uint32_t DT, int EPI>
-__global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams p, float *partials) {
+template <uint32_t DT, int EPI, int PAIRS>
+__global__ __launch_bounds__(PAIRS * 2 * kWave, 2) void gemm_wide_kernel(GemmRowsParams p, float *partials) {
+  constexpr int kWPairs = PAIRS;
+  constexpr int kWThreads = kWPairs * 2 * kWave;
   constexpr int kStageVec = kBSteps * kWTiles * kWave;   // 16-byte pieces of one X block: 4096 = 64 KiB
-  constexpr int kFill = kStageVec / kWThreads;           // pieces per thread and block
+  constexpr int kFill = (kStageVec + kWThreads - 1) / kWThreads;   // pieces per thread and block (the last one only
+  constexpr bool kFillRagged = kStageVec % kWThreads != 0;         // for the first threads when the count does not divide)
+  constexpr int kXPer = (kFill + 3) / 4;                 // X requests per slot
   constexpr int kHalf = kWTiles / 2;                     // token tiles per wave
   extern __shared__ __align__(16) unsigned char smem[];
   u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);
@@ -427,11 +439,14 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
 #define NV_WD_W(BUF, BLK) _Pragma("unroll") for (int i = 0; i < 4; ++i) NV_WD_W1(BUF, BLK, i)
 #define NV_WD_WPARK(BUF) \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t *>(park_at + 4 * i * kBRowStride) = areg[BUF][i]
+#define NV_WD_XLIVE(I) (!kFillRagged || (I) + 1 < kFill || (I) * kWThreads + threadIdx.x < static_cast<uint32_t>(kStageVec))
 #define NV_WD_X1(BLK, I)                                                                            \
+  if (NV_WD_XLIVE(I))                                                                               \
   xreg[I] = *reinterpret_cast<const u32x4_t *>(                                                      \
       xbase + (static_cast<uint64_t>(BLK) * kStageVec + (I) * kWThreads) * sizeof(u32x4_t) + xlane)
-#define NV_WD_X(BLK) _Pragma("unroll") for (int i = 0; i < kFill; ++i) NV_WD_X1(BLK, i)
-#define NV_WD_XPARK() _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[i * kWThreads + threadIdx.x] = xreg[i]
+#define NV_WD_X(BLK) _Pragma("unroll") for (int i = 0; i < kFill; ++i) { NV_WD_X1(BLK, i); }
+#define NV_WD_XPARK() \
+  _Pragma("unroll") for (int i = 0; i < kFill; ++i) { if (NV_WD_XLIVE(i)) stage[i * kWThreads + threadIdx.x] = xreg[i]; }
 #define NV_WD_READ_A(S, A) \
   _Pragma("unroll") for (int j = 0; j < 2; ++j) A[j] = *reinterpret_cast<const u32x4_t *>(a_read + j * kBWTile + (S) * 32)
 #define NV_WD_READ_B(S, B) \
@@ -439,13 +454,14 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
 #define NV_WD_PRODUCTS(A, B, C0)                                                                    \
   _Pragma("unroll") for (int c = C0; c < C0 + kHalf / 2; ++c)                                       \
       _Pragma("unroll") for (int j = 0; j < 2; ++j) acc[j][c] = mfma_k32<DT>(A[j], B[c], acc[j][c])
-  // request slots between the products, two requests each: slots 0..3 the next X block's eight pieces, slots
-  // 4 and 5 the four rows-of-four of the W block kRing ahead (the order they are awaited in)
+  // request slots between the products: slots 0..3 the next X block's pieces (two or three each), slots
+  // 4 and 5 the four rows-of-four of the W block kRing ahead, two each (the order they are awaited in)
 #define NV_WD_SLOT(K, BUF, XEN, XBLK, WEN, WBLK)                                                    \
   if constexpr ((K) < 4) {                                                                          \
     if constexpr (XEN) {                                                                            \
-      NV_WD_X1(XBLK, 2 * (K));                                                                      \
-      NV_WD_X1(XBLK, 2 * (K) + 1);                                                                  \
+      _Pragma("unroll") for (int xi = kXPer * (K); xi < kXPer * ((K) + 1); ++xi) {                  \
+        if (xi < kFill) { NV_WD_X1(XBLK, xi); }                                                     \
+      }                                                                                             \
     }                                                                                               \
   } else if constexpr (WEN && (K) < 6) {                                                            \
     NV_WD_W1(BUF, WBLK, 2 * ((K) - 4));                                                             \
@@ -502,6 +518,7 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
 #undef NV_WD_W
 #undef NV_WD_WPARK
 #undef NV_WD_X1
+#undef NV_WD_XLIVE
 #undef NV_WD_X
 #undef NV_WD_XPARK
 #undef NV_WD_READ_A
@@ -541,20 +558,29 @@ __global__ __launch_bounds__(kWThreads, 2) void gemm_wide_kernel(GemmRowsParams 
   }
 }
 
-template <uint32_t DT, int EPI>
-hipError_t launch_wide(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
-  const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kWPairs : 32u * kWPairs;
+template <uint32_t DT, int EPI, int PAIRS>
+hipError_t launch_wide_pairs(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  constexpr uint32_t wg_rows = wide_wg_rows(EPI, PAIRS);
+  constexpr size_t lds = wide_lds_bytes(PAIRS);
   // more than the default dynamic LDS limit: raised once per kernel (never under stream capture)
   static std::once_flag once;
   static hipError_t raised = hipSuccess;
   std::call_once(once, [] {
-    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<DT, EPI>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kWLdsBytes));
+    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<DT, EPI, PAIRS>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   });
   if (raised != hipSuccess) return raised;
-  hipLaunchKernelGGL((gemm_wide_kernel<DT, EPI>), dim3(p.rows / wg_rows, kslices), dim3(kWThreads), kWLdsBytes, stream, p,
+  hipLaunchKernelGGL((gemm_wide_kernel<DT, EPI, PAIRS>), dim3(p.rows / wg_rows, kslices), dim3(PAIRS * 2 * kWave), lds, stream, p,
                      partials);
-  hipError_t err = hipGetLastError();
+  return hipGetLastError();
+}
+
+template <uint32_t DT, int EPI>
+hipError_t launch_wide(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  const int pairs = wide_pairs(EPI, p.rows);
+  hipError_t err = pairs == 3   ? launch_wide_pairs<DT, EPI, 3>(p, partials, kslices, stream)
+                   : pairs == 4 ? launch_wide_pairs<DT, EPI, 4>(p, partials, kslices, stream)
+                                : hipErrorInvalidValue;
   if (err == hipSuccess && kslices > 1) {
     const uint32_t threads = p.rows / 4u * p.tokens;
     hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
@@ -629,8 +655,9 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
 // Enough workgroups for three quarters of the CUs (a gate/up pair of Qwen3-8B width has 192 row groups and
 // runs unsliced), each slice a whole number of rings of K-blocks, the partial sums within the workspace.
 uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
-  const uint32_t wg_rows = epilogue == kGemmSwiglu ? 16u * kWPairs : 32u * kWPairs;
-  if (tokens <= kBTokCap || tokens > kWTokCap || rows % wg_rows != 0 || cols % (kBRing * kBK) != 0) return 0;
+  const int pairs = wide_pairs(epilogue, rows);
+  if (tokens <= kBTokCap || tokens > kWTokCap || pairs == 0 || cols % (kBRing * kBK) != 0) return 0;
+  const uint32_t wg_rows = wide_wg_rows(epilogue, pairs);
   const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
   const uint32_t groups = rows / wg_rows;
   uint32_t slices = 1;

@@ -829,10 +829,10 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
                                                (4096, 12288, 128), (192, 2048, 17), (64, 2048, 33), (4096, 4096, 32),
                                                (6144, 4096, 48), (4096, 12288, 64),
                                                (128, 2048, 129), (256, 4096, 200), (4096, 4096, 256), (6144, 4096, 255),
-                                               (4096, 12288, 256)])
+                                               (4096, 12288, 256), (192, 2048, 140)])
 def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     """More than 16 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
-    X from LDS (2, 4, 8 or - blocks of 129..256 rows, wave pairs sharing the W tiles - 16 token tiles). Every token
+    X from LDS (2, 4, 8 or - blocks of 129..256 rows, three or four wave pairs sharing their W tiles - 16 token tiles). Every token
     row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
     dtype = BF16
     rng = np.random.default_rng(rows + cols + tokens)
@@ -864,7 +864,7 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
 
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
-                                                 (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250)])
+                                                 (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
