@@ -119,6 +119,8 @@ def main():
     ap.add_argument("--batch-sessions", type=int, default=32,
                     help="sessions advanced together in the shared-weights leg (0 = skip it)")
     ap.add_argument("--batch-steps", type=int, default=24)
+    ap.add_argument("--prefill-block", type=int, default=0, choices=(0, 128, 256),
+                    help="prompt block size (0 = the session's choice: 256 tokens at these widths)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also launch one plain copy kernel of this size (memory-counter calibration runs)")
     args = ap.parse_args()
@@ -132,6 +134,8 @@ def main():
     if rc != 0:
         log("no usable GPU (hip_error=%d): the HIP path cannot run, and there is no CPU fallback" % smoke.hip_error)
         sys.exit(1)
+    if args.prefill_block == 128:
+        N.Device.set_tuning("prefill_block_tokens", 128)
     cfg = dict(N.Qwen3_8B)
     cfg["layers"] = args.layers
     max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16   # + the CPU leg's parity token
@@ -287,7 +291,8 @@ def main():
                                      "32q/8kv x128, MLP 12288, vocab 151936, random-init bf16 N(0,0.02), batch 1, "
                                      "prompt %d prefilled, %d greedy tokens under hipGraph replay"
                                      % (cfg["layers"], args.prompt, args.steps),
-                            prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), prefill_tok_s=round(args.prompt / prefill_s, 1), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
+                            prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), prefill_tok_s=round(args.prompt / prefill_s, 1),
+                            prefill_block_tokens=int(session.create_result.prefill_chunk_tokens), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
                             per_token_latency_ms=latency, shared_weight_sessions=batch, operators=operators,
                             gpu=smoke.gpu_name.decode()),
