@@ -167,8 +167,9 @@ __global__ __launch_bounds__(kPW *kWave) void attn_prompt_kernel(AttnParams p) {
   }
 }
 
-// Second launch: grid (head, token), one lane per dim; splits in order.
-template <uint32_t DT>
+// Second launch: grid (head, token), one lane per dim; splits in order, kRound of them requested at a time
+// (4 where the launch has no more splits than that: the same sums in the same order with a quarter of the loads).
+template <uint32_t DT, int kRound>
 __global__ __launch_bounds__(kHD) void attn_prompt_merge_kernel(AttnParams p, uint32_t S, uint32_t group_tokens) {
   const uint32_t h = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
   const uint32_t group_last = min(p.tokens, (tok / group_tokens + 1) * group_tokens) - 1;
@@ -179,8 +180,7 @@ __global__ __launch_bounds__(kHD) void attn_prompt_merge_kernel(AttnParams p, ui
   const float *acc = reinterpret_cast<const float *>(ws) + static_cast<uint64_t>(h) * S * kHD + d;
   const float *pm = reinterpret_cast<const float *>(ws + (reinterpret_cast<const char *>(p.part_m) - reinterpret_cast<const char *>(p.part_acc))) + h * S;
   const float *pl = reinterpret_cast<const float *>(ws + (reinterpret_cast<const char *>(p.part_l) - reinterpret_cast<const char *>(p.part_acc))) + h * S;
-  // rounds of sixteen splits, every load of a round unconditional (index clamped) and in flight at once
-  constexpr int kRound = 16;
+  // rounds of kRound splits, every load of a round unconditional (index clamped) and in flight at once
   float M = -INFINITY, L = 0.0f, o = 0.0f;
   for (uint32_t s0 = 0; s0 < active; s0 += kRound) {
     float mm[kRound], ll[kRound], aa[kRound];
@@ -229,7 +229,10 @@ hipError_t launch_dt(const AttnParams &p, uint32_t splits, hipStream_t stream) {
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || splits == 1) return err;
-  hipLaunchKernelGGL((attn_prompt_merge_kernel<DT>), dim3(p.heads, p.tokens), dim3(kHD), 0, stream, p, splits, group_tokens);
+  if (splits <= 4)
+    hipLaunchKernelGGL((attn_prompt_merge_kernel<DT, 4>), dim3(p.heads, p.tokens), dim3(kHD), 0, stream, p, splits, group_tokens);
+  else
+    hipLaunchKernelGGL((attn_prompt_merge_kernel<DT, 16>), dim3(p.heads, p.tokens), dim3(kHD), 0, stream, p, splits, group_tokens);
   return hipGetLastError();
 }
 
