@@ -718,9 +718,12 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
       hipLaunchKernelGGL(embed_rows_kernel<kF16>, dim3(T), dim3(kBlock), 0, st, s->emb, s->prompt, first, H, s->vocab,
                          s->px, rope_freq, s->prope, s->head_dim / 2);
     err = hipGetLastError();
+    // Where a projection's slice-adding launch can write the following RMSNorm too, it does (one launch less each)
+    const bool o_norms = gemm_rows_fuses_norm(kGemmResidual, H, A, T, tiles, s->pgemm_ws_bytes);
+    const bool down_norms = gemm_rows_fuses_norm(kGemmResidual, H, I, T, tiles, s->pgemm_ws_bytes);
     for (uint32_t l = 0; err == hipSuccess && l < s->layers; ++l) {
       const LayerDev &w = s->layer[l];
-      err = launch_rmsnorm_rows(s->dtype, s->px, w.rms_attn, s->eps, T, H, s->pxn16, st, tiles);
+      if (l == 0 || !down_norms) err = launch_rmsnorm_rows(s->dtype, s->px, w.rms_attn, s->eps, T, H, s->pxn16, st, tiles);
       GemmRowsParams g{};
       g.tokens = T;
       if (err == hipSuccess) {
@@ -784,9 +787,15 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.cols = A;
         g.workspace = s->pgemm_ws;
         g.workspace_bytes = s->pgemm_ws_bytes;
+        if (o_norms) {
+          g.norm_gamma = w.rms_mlp;
+          g.norm_out16 = s->pxn16;
+          g.norm_eps = s->eps;
+          g.norm_packed_tiles = tiles;
+        }
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
-      if (err == hipSuccess) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st, tiles);
+      if (err == hipSuccess && !o_norms) err = launch_rmsnorm_rows(s->dtype, s->pr, w.rms_mlp, s->eps, T, H, s->pxn16, st, tiles);
       if (err == hipSuccess) {
         g = GemmRowsParams{};
         g.tokens = T;
@@ -814,6 +823,12 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
         g.round_out = 1;  // prompt tokens carry a 16-bit hidden state between layers
         g.workspace = s->pgemm_ws;
         g.workspace_bytes = s->pgemm_ws_bytes;
+        if (down_norms && l + 1 < s->layers) {   // the next layer's attention norm
+          g.norm_gamma = s->layer[l + 1].rms_attn;
+          g.norm_out16 = s->pxn16;
+          g.norm_eps = s->eps;
+          g.norm_packed_tiles = tiles;
+        }
         err = launch_gemm_rows(s->dtype, kGemmResidual, g, st);
       }
     }

@@ -322,6 +322,77 @@ __global__ __launch_bounds__(256) void gemm_block_finish_kernel(GemmRowsParams p
   block_epilogue<DT, EPI>(p, t, row, y, up);
 }
 
+// The slice-adding launch of a residual projection with the RMSNorm of the result in the same pass: one workgroup
+// of 1024 lanes per token, a lane's values, sum of squares, reduction and scaling laid out exactly as in
+// rmsnorm_rows_kernel (gemm_rows.hip), so norm_out16 equals what that kernel writes for out_f32.
+constexpr int kFinNormThreads = 1024, kFinNormPerLane = 4;
+template <uint32_t DT>
+__global__ __launch_bounds__(kFinNormThreads) void gemm_finish_norm_kernel(GemmRowsParams p, const float *partials, uint32_t kslices,
+                                                                         uint32_t tokcap) {
+  __shared__ float red[kFinNormThreads / kWave];
+  const uint32_t t = blockIdx.x, rows = p.rows;
+  float4 v[kFinNormPerLane];
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kFinNormPerLane; ++i) {
+    const uint32_t row = (i * kFinNormThreads + threadIdx.x) * 4;
+    v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (row < rows) {
+      float4 y = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      for (uint32_t s = 0; s < kslices; ++s) {
+        const float4 a = *reinterpret_cast<const float4 *>(partials + (static_cast<uint64_t>(s) * tokcap + t) * rows + row);
+        y.x += a.x;
+        y.y += a.y;
+        y.z += a.z;
+        y.w += a.w;
+      }
+      if (p.bias != nullptr) {
+        y.x += dec16<DT>(p.bias[row]);
+        y.y += dec16<DT>(p.bias[row + 1]);
+        y.z += dec16<DT>(p.bias[row + 2]);
+        y.w += dec16<DT>(p.bias[row + 3]);
+      }
+      const uint64_t at = static_cast<uint64_t>(t) * rows + row;
+      const float4 res = *reinterpret_cast<const float4 *>(p.residual + at);
+      y.x += res.x;
+      y.y += res.y;
+      y.z += res.z;
+      y.w += res.w;
+      if (p.round_out) {
+        y.x = round16<DT>(y.x);
+        y.y = round16<DT>(y.y);
+        y.z = round16<DT>(y.z);
+        y.w = round16<DT>(y.w);
+      }
+      *reinterpret_cast<float4 *>(p.out_f32 + at) = y;
+      v[i] = y;
+    }
+    ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kFinNormThreads / kWave; ++w) total += red[w];
+  const float scale = 1.0f / sqrtf(total / static_cast<float>(rows) + p.norm_eps);
+#pragma unroll
+  for (int i = 0; i < kFinNormPerLane; ++i) {
+    const uint32_t c = (i * kFinNormThreads + threadIdx.x) * 4;
+    if (c < rows) {
+      const uint2 g = *reinterpret_cast<const uint2 *>(p.norm_gamma + c);
+      float g0, g1, g2, g3;
+      unpack2<DT>(g.x, g0, g1);
+      unpack2<DT>(g.y, g2, g3);
+      uint2 o;
+      o.x = enc16<DT>(v[i].x * scale * g0) | (static_cast<uint32_t>(enc16<DT>(v[i].y * scale * g1)) << 16);
+      o.y = enc16<DT>(v[i].z * scale * g2) | (static_cast<uint32_t>(enc16<DT>(v[i].w * scale * g3)) << 16);
+      if (p.norm_packed_tiles != 0) *reinterpret_cast<uint2 *>(p.norm_out16 + gemm_x_packed_index(p.norm_packed_tiles, t, c)) = o;
+      else *reinterpret_cast<uint2 *>(p.norm_out16 + static_cast<uint64_t>(t) * rows + c) = o;
+    }
+  }
+}
+
 template <int NR, int TT>
 constexpr size_t block_lds_bytes() {
   return static_cast<size_t>(kBSteps) * TT * kWave * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
@@ -582,9 +653,14 @@ hipError_t launch_wide(const GemmRowsParams &p, float *partials, uint32_t kslice
                    : pairs == 4 ? launch_wide_pairs<DT, EPI, 4>(p, partials, kslices, stream)
                                 : hipErrorInvalidValue;
   if (err == hipSuccess && kslices > 1) {
-    const uint32_t threads = p.rows / 4u * p.tokens;
-    hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
-                       static_cast<const float *>(partials), kslices, kWTokCap);
+    if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
+      hipLaunchKernelGGL((gemm_finish_norm_kernel<DT>), dim3(p.tokens), dim3(kFinNormThreads), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kWTokCap);
+    } else {
+      const uint32_t threads = p.rows / 4u * p.tokens;
+      hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kWTokCap);
+    }
     err = hipGetLastError();
   }
   return err;
@@ -669,6 +745,12 @@ uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t t
   }
   while (slices > 1 && static_cast<uint64_t>(slices) * kWTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
   return slices;
+}
+
+bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes) {
+  return epilogue == kGemmResidual && x_packed != 0 && rows % 4 == 0 &&
+         rows <= static_cast<uint32_t>(kFinNormThreads * kFinNormPerLane * 4) &&
+         gemm_wide_slices(epilogue, rows, cols, tokens, workspace_bytes) > 1;
 }
 
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {

@@ -52,6 +52,14 @@ struct GemmRowsParams {
   uint32_t out_packed_tiles; // kGemmSwiglu: != 0 writes out16 in operand order with this many token tiles
   void *workspace;           // optional: room for the f32 partial sums of the shared-X kernel's K slices
   uint64_t workspace_bytes;  // (gemm_block_workspace_bytes; without it that kernel runs unsliced or not at all)
+  // kGemmResidual, optional, only where gemm_rows_fuses_norm() says so: the launch that adds the K slices also
+  // writes the RMSNorm of every output row - norm_out16[t] = round16(y[t] * rsqrt(mean(y[t]^2) + norm_eps) *
+  // norm_gamma), bit for bit what launch_rmsnorm_rows gives on out_f32 - in operand order when
+  // norm_packed_tiles != 0.
+  const uint16_t *norm_gamma;
+  uint16_t *norm_out16;
+  float norm_eps;
+  uint32_t norm_packed_tiles;
 };
 
 // rows >= 16 (any count: the last workgroup overlaps its neighbour, so with a row count that is no
@@ -77,6 +85,9 @@ hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams 
 // (rows a multiple of 128, gate/up pairs of 64; cols a multiple of 512 per slice). launch_gemm_rows uses it by itself.
 uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
 hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
+// Whether launch_gemm_rows honours GemmRowsParams::norm_gamma for this shape (a K-sliced residual projection of a
+// wide block, rows a multiple of 4 and at most 16384); otherwise the caller normalises with launch_rmsnorm_rows.
+bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes);
 
 // x16[t] = round16(x[t] * rsqrt(mean(x[t]^2) + eps) * gamma) for `tokens` rows of `cols` f32 values.
 // packed_tiles != 0: out16 in operand order (gemm_x_packed_index) with that many token tiles.

@@ -312,6 +312,9 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
   if (p.out_packed_tiles != 0 && (epilogue != kGemmSwiglu || p.out_packed_tiles * 16u < p.tokens)) return hipErrorInvalidValue;
   if (p.x_packed != 0 && p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;   // tiles the kernel will assume
   if (dtype != kBF16 && dtype != kF16) return hipErrorInvalidValue;
+  if (p.norm_gamma != nullptr &&   // a fused norm only where the shape has one; never silently dropped
+      (p.norm_out16 == nullptr || !gemm_rows_fuses_norm(epilogue, p.rows, p.cols, p.tokens, p.x_packed, p.workspace != nullptr ? p.workspace_bytes : 0)))
+    return hipErrorInvalidValue;
   if (wide_slices != 0) return launch_gemm_wide(dtype, epilogue, p, wide_slices, stream);
   if (p.x_packed != 0) {   // blocks in operand order: the kernel that shares X through LDS, where its plan takes the shape
     const GemmBlockPlan plan = gemm_block_plan(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0);
