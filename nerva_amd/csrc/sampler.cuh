@@ -9,18 +9,19 @@
 // vocabulary is cut into 1024-logit chunks, one workgroup each, and a second one-workgroup
 // kernel finishes:
 //   chunk kernel   greedy / Gumbel: best (score, index) of the chunk.
-//                  top-k: the chunk's logits as 64-bit keys (order-preserving value bits above the
-//                  inverted index, so a plain integer order is (value desc, index asc)), sorted in
-//                  LDS, and its best min(k, 1024) keys written out: the global top-k is among them.
+//                  top-k: the chunk's best logit as a 64-bit key (order-preserving value bits above the
+//                  inverted index, so a plain integer order is (value desc, index asc)) and the number
+//                  of its finite logits.
 //   select kernel  greedy / Gumbel: best of the chunk candidates.
-//                  top-k: the k-th largest of the chunks' best keys bounds the k-th largest key
-//                  from below, so each (sorted) chunk list contributes only its prefix at or above
-//                  that bound - a few hundred keys when the logits are spread over the chunks -
-//                  which are sorted in LDS. If more than 1024 survive (logits piled into few chunks),
-//                  the exact k-th largest key comes from a radix selection over all chunk candidates
-//                  (six digits, histogram in LDS, parallel suffix scan) instead. Then exponentials in
-//                  parallel, and the three short sums of the rule (total, nucleus, draw) by one lane
-//                  in the rule's order.
+//                  top-k: the k-th largest of the chunks' best keys bounds the k-th largest key of the
+//                  vocabulary from below, so one pass over the logits collects the keys at or above
+//                  that bound - a few hundred when the logits are spread over the chunks - and a sort in
+//                  LDS orders them. If more than 1024 survive (logits piled into few chunks), the exact
+//                  k-th largest key comes from a radix selection over the whole vocabulary (six digits,
+//                  histogram in LDS, parallel suffix scan) instead. Then exponentials in parallel, and
+//                  the three short sums of the rule (total, nucleus, draw) by one lane in the rule's order.
+//                  (The chunks used to sort their 1024 keys and hand out their best 128: 38 + 30-43 us for
+//                  the two launches at 151936 logits, barrier-bound.)
 //   then the token slot is written and the device cursor advanced, as the greedy finish does.
 #pragma once
 
@@ -53,7 +54,7 @@ struct SamplerParams {
   const float *logits;
   uint32_t vocab;
   const SamplerDev *config;   // device memory
-  uint64_t *keys;             // [chunks][kSamplerTopKMax] workspace
+  uint64_t *keys;             // [chunks][kSamplerTopKMax] workspace (top-k: word 0 of a row the chunk's best key, word 1 its finite count)
   SampleParams out;           // chunk candidates (greedy / Gumbel), slot / cursor / plain token output
   const uint32_t *cursor;     // device position (slot index and random-number counter), or null -> position
   uint32_t position, max_steps;

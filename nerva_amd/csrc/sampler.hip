@@ -70,7 +70,7 @@ __device__ __forceinline__ void sort_desc(uint64_t *keys, uint32_t count, uint32
 // `batch` (device memory) replaces `p` by its entry blockIdx.y: one launch for several sequences.
 __global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerParams p, const SamplerParams *batch) {
   if (batch != nullptr) p = batch[blockIdx.y];
-  __shared__ uint64_t keys[kSamplerChunk];
+  __shared__ uint64_t keys[kChunkThreads / kWave];
   __shared__ float red_v[kChunkThreads / kWave];
   __shared__ uint32_t red_i[kChunkThreads / kWave];
   __shared__ uint32_t red_h[kChunkThreads / kWave];
@@ -118,21 +118,40 @@ __global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerPara
     return;
   }
 
-  // top-k: sort the chunk's keys, hand out its best min(k, chunk) of them
+  // top-k: the chunk's best key and the number of its finite logits (words 0 and 1 of the chunk's workspace row)
+  uint64_t best = 0;
+  uint32_t finite = 0;
   for (uint32_t e = threadIdx.x; e < kSamplerChunk; e += kChunkThreads) {
     const uint32_t i = base + e;
-    uint64_t key = 0;
     if (i < p.vocab) {
       const float v = p.logits[i];
-      if (isfinite(v)) key = make_key(v, i);
+      if (isfinite(v)) {
+        const uint64_t key = make_key(v, i);
+        best = key > best ? key : best;
+        ++finite;
+      }
     }
-    keys[e] = key;
+  }
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const uint64_t other = (static_cast<uint64_t>(__shfl_xor(static_cast<uint32_t>(best >> 32), o, kWave)) << 32) |
+                           __shfl_xor(static_cast<uint32_t>(best), o, kWave);
+    best = other > best ? other : best;
+    finite += __shfl_xor(finite, o, kWave);
+  }
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    keys[wave] = best;
+    red_i[wave] = finite;
   }
   __syncthreads();
-  sort_desc(keys, kSamplerChunk, kChunkThreads);
-  const uint32_t want = wanted_candidates(cfg.top_k, p.vocab);
-  for (uint32_t e = threadIdx.x; e < kSamplerTopKMax; e += kChunkThreads)
-    p.keys[static_cast<uint64_t>(blockIdx.x) * kSamplerTopKMax + e] = e < want ? keys[e] : 0ull;
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kChunkThreads / kWave; ++w) {
+      best = keys[w] > best ? keys[w] : best;
+      finite += red_i[w];
+    }
+    p.keys[static_cast<uint64_t>(blockIdx.x) * kSamplerTopKMax] = best;
+    p.keys[static_cast<uint64_t>(blockIdx.x) * kSamplerTopKMax + 1] = finite;
+  }
 }
 
 __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerParams p, uint32_t chunks,
@@ -178,11 +197,10 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     return;
   }
 
-  // ---- top-k: how many real candidates are there at all
-  const uint64_t total_keys = static_cast<uint64_t>(chunks) * kSamplerTopKMax;
-  uint32_t mine = 0;
-  for (uint64_t i = tid; i < total_keys; i += kSelectThreads) mine += p.keys[i] != 0ull ? 1u : 0u;
-  scan[tid] = mine;
+  // ---- top-k: how many finite logits are there at all
+  scan[tid] = 0;
+  for (uint32_t c = tid; c < chunks; c += kSelectThreads)
+    scan[tid] += static_cast<uint32_t>(p.keys[static_cast<uint64_t>(c) * kSamplerTopKMax + 1]);
   __syncthreads();
   for (uint32_t d = kSelectThreads / 2; d > 0; d >>= 1) {
     if (tid < d) scan[tid] += scan[tid + d];
@@ -197,46 +215,52 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     return;
   }
 
-  // ---- fast path: prune with a bound taken from the chunk maxima. The selected-th largest of
-  // the chunks' best keys is no larger than the selected-th largest key overall, so only keys at or
-  // above it matter; with logits spread over the chunks that leaves a few hundred, which are sorted
-  // in LDS directly. Each chunk's list is sorted, so a chunk's share is a prefix of its list.
+  // ---- fast path: a bound from the chunk maxima. The selected-th largest of the chunks' best keys is no
+  // larger than the selected-th largest key overall, so only keys at or above it matter: with logits spread
+  // over the chunks that leaves a few hundred of the whole vocabulary, which one pass over the logits collects
+  // and a sort in LDS orders. (Keys are distinct, so the order they are collected in does not show.)
   bool fast = chunks <= static_cast<uint32_t>(kSelectThreads);
   if (fast) {
     cand[tid] = tid < chunks ? p.keys[static_cast<uint64_t>(tid) * kSamplerTopKMax] : 0ull;
+    if (tid == 0) {
+      prefix_s = 0;   // the bound: 0 (everything) when fewer chunks than `selected` hold a finite logit
+      count_s = 0;
+    }
     __syncthreads();
-    uint32_t width = 1;
-    while (width < chunks) width <<= 1;
-    sort_desc(cand, width, kSelectThreads);
-    const uint64_t bound = chunks >= selected ? cand[selected - 1] : 0ull;
+    const uint64_t mine_max = cand[tid];
+    if (mine_max != 0ull) {
+      uint32_t above = 0;
+      for (uint32_t c = 0; c < chunks; ++c) above += cand[c] > mine_max ? 1u : 0u;
+      if (above == selected - 1) prefix_s = mine_max;   // distinct keys: exactly one chunk has this rank
+    }
     __syncthreads();
-    uint32_t n = 0;
-    const uint64_t *list = p.keys + static_cast<uint64_t>(tid) * kSamplerTopKMax;
-    if (tid < chunks) {
-      while (n < kSamplerTopKMax) {
-        const uint64_t key = list[n];
-        if (key == 0ull || key < bound) break;
-        ++n;
+    const uint64_t bound = prefix_s;
+    __syncthreads();
+    // (eight logits requested before the first is looked at: with one load per turn the pass is 149 round trips)
+    constexpr uint32_t kScan = 8;
+    for (uint32_t i0 = tid; i0 < p.vocab; i0 += kScan * kSelectThreads) {
+      float v[kScan];
+#pragma unroll
+      for (uint32_t u = 0; u < kScan; ++u) v[u] = p.logits[min(i0 + u * kSelectThreads, p.vocab - 1)];
+#pragma unroll
+      for (uint32_t u = 0; u < kScan; ++u) {
+        const uint32_t i = i0 + u * kSelectThreads;
+        if (i < p.vocab && isfinite(v[u])) {
+          const uint64_t key = make_key(v[u], i);
+          if (key >= bound) {
+            const uint32_t slot = atomicAdd(&count_s, 1u);
+            if (slot < static_cast<uint32_t>(kSelectThreads)) cand[slot] = key;
+          }
+        }
       }
     }
-    scan[tid] = n;
     __syncthreads();
-    for (uint32_t d = 1; d < kSelectThreads; d <<= 1) {   // inclusive prefix sums
-      const uint32_t v = scan[tid] + (tid >= d ? scan[tid - d] : 0u);
-      __syncthreads();
-      scan[tid] = v;
-      __syncthreads();
-    }
-    const uint32_t total = scan[kSelectThreads - 1];
+    const uint32_t total = count_s;
     fast = total <= static_cast<uint32_t>(kSelectThreads);   // same value in every thread
     if (fast) {
-      const uint32_t at = scan[tid] - n;
+      if (tid >= total) cand[tid] = 0ull;
       __syncthreads();
-      cand[tid] = 0ull;
-      __syncthreads();
-      for (uint32_t j = 0; j < n; ++j) cand[at + j] = list[j];
-      __syncthreads();
-      width = 1;
+      uint32_t width = 1;
       while (width < total) width <<= 1;
       sort_desc(cand, width, kSelectThreads);
       if (tid < kSamplerTopKMax) top[tid] = tid < total ? cand[tid] : 0ull;
@@ -244,7 +268,7 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     }
   }
   if (!fast) {
-    // ---- the selected-th largest key, digit by digit from the top
+    // ---- the selected-th largest key of the whole vocabulary, digit by digit from the top
     uint64_t prefix = 0, mask = 0;
     uint32_t need = selected;
     for (int level = 0; level < kLevels; ++level) {
@@ -253,8 +277,9 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
       const uint32_t bins = 1u << width;
       for (uint32_t b = tid; b < kBins; b += kSelectThreads) hist[b] = 0;
       __syncthreads();
-      for (uint64_t i = tid; i < total_keys; i += kSelectThreads) {
-        const uint64_t key = p.keys[i];
+      for (uint32_t i = tid; i < p.vocab; i += kSelectThreads) {
+        const float v = p.logits[i];
+        const uint64_t key = isfinite(v) ? make_key(v, i) : 0ull;
         if (key != 0ull && (key & mask) == prefix) atomicAdd(&hist[static_cast<uint32_t>(key >> shift) & (bins - 1u)], 1u);
       }
       __syncthreads();
@@ -290,8 +315,9 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     if (tid == 0) count_s = 0;
     for (uint32_t e = tid; e < kSamplerTopKMax; e += kSelectThreads) top[e] = 0ull;
     __syncthreads();
-    for (uint64_t i = tid; i < total_keys; i += kSelectThreads) {
-      const uint64_t key = p.keys[i];
+    for (uint32_t i = tid; i < p.vocab; i += kSelectThreads) {
+      const float v = p.logits[i];
+      const uint64_t key = isfinite(v) ? make_key(v, i) : 0ull;
       if (key != 0ull && key >= prefix) {
         const uint32_t slot = atomicAdd(&count_s, 1u);
         if (slot < kSamplerTopKMax) top[slot] = key;
