@@ -47,26 +47,6 @@ __device__ __forceinline__ uint32_t wanted_candidates(uint32_t top_k, uint32_t v
   return requested < vocab ? requested : vocab;  // sampler.cu:169-174
 }
 
-// Descending bitonic sort of `count` (a power of two) keys in LDS by `threads` threads.
-__device__ __forceinline__ void sort_desc(uint64_t *keys, uint32_t count, uint32_t threads) {
-  for (uint32_t width = 2; width <= count; width <<= 1) {
-    for (uint32_t stride = width >> 1; stride != 0; stride >>= 1) {
-      for (uint32_t e = threadIdx.x; e < count; e += threads) {
-        const uint32_t partner = e ^ stride;
-        if (partner > e) {
-          const bool descending = (e & width) == 0;
-          const uint64_t a = keys[e], b = keys[partner];
-          if (descending ? a < b : a > b) {
-            keys[e] = b;
-            keys[partner] = a;
-          }
-        }
-      }
-      __syncthreads();
-    }
-  }
-}
-
 // `batch` (device memory) replaces `p` by its entry blockIdx.y: one launch for several sequences.
 __global__ __launch_bounds__(kChunkThreads) void sample_chunk_kernel(SamplerParams p, const SamplerParams *batch) {
   if (batch != nullptr) p = batch[blockIdx.y];
@@ -198,15 +178,16 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
   }
 
   // ---- top-k: how many finite logits are there at all
-  scan[tid] = 0;
+  // (a workgroup barrier of sixteen waves costs a third of a microsecond: sums and orders below are arranged to
+  // need few of them - wave sums first, ranks by counting instead of sorting networks)
+  uint32_t mine = 0;
   for (uint32_t c = tid; c < chunks; c += kSelectThreads)
-    scan[tid] += static_cast<uint32_t>(p.keys[static_cast<uint64_t>(c) * kSamplerTopKMax + 1]);
+    mine += static_cast<uint32_t>(p.keys[static_cast<uint64_t>(c) * kSamplerTopKMax + 1]);
+  for (int o = kWave / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, kWave);
+  if ((tid & (kWave - 1)) == 0) red_i[tid / kWave] = mine;
   __syncthreads();
-  for (uint32_t d = kSelectThreads / 2; d > 0; d >>= 1) {
-    if (tid < d) scan[tid] += scan[tid + d];
-    __syncthreads();
-  }
-  const uint32_t finite_candidates = scan[0];
+  uint32_t finite_candidates = 0;
+  for (int w = 0; w < kSelectThreads / kWave; ++w) finite_candidates += red_i[w];
   __syncthreads();
   uint32_t selected = wanted_candidates(cfg.top_k, p.vocab);
   if (selected > finite_candidates) selected = finite_candidates;  // fewer finite logits than requested
@@ -236,7 +217,10 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     __syncthreads();
     const uint64_t bound = prefix_s;
     __syncthreads();
-    // (eight logits requested before the first is looked at: with one load per turn the pass is 149 round trips)
+    // One workgroup looks at every logit, so the look is two comparisons (a float at or above the bound's value,
+    // and finite); the key is formed and compared exactly only for the few that pass (forming every key was 15
+    // instructions a logit: 17 of the kernel's 36 us). Eight logits are requested before the first is looked at.
+    const float bound_value = bound != 0ull ? key_value(bound) : -INFINITY;
     constexpr uint32_t kScan = 8;
     for (uint32_t i0 = tid; i0 < p.vocab; i0 += kScan * kSelectThreads) {
       float v[kScan];
@@ -245,7 +229,7 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
 #pragma unroll
       for (uint32_t u = 0; u < kScan; ++u) {
         const uint32_t i = i0 + u * kSelectThreads;
-        if (i < p.vocab && isfinite(v[u])) {
+        if (v[u] >= bound_value && fabsf(v[u]) <= 3.402823466e+38f && i < p.vocab) {   // (finite: a NaN passes neither)
           const uint64_t key = make_key(v[u], i);
           if (key >= bound) {
             const uint32_t slot = atomicAdd(&count_s, 1u);
@@ -258,12 +242,15 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
     const uint32_t total = count_s;
     fast = total <= static_cast<uint32_t>(kSelectThreads);   // same value in every thread
     if (fast) {
-      if (tid >= total) cand[tid] = 0ull;
+      // order by counting: a key's place is the number of keys above it (distinct keys: no two share a place)
+      if (tid < kSamplerTopKMax) top[tid] = 0ull;
       __syncthreads();
-      uint32_t width = 1;
-      while (width < total) width <<= 1;
-      sort_desc(cand, width, kSelectThreads);
-      if (tid < kSamplerTopKMax) top[tid] = tid < total ? cand[tid] : 0ull;
+      if (tid < total) {
+        const uint64_t key = cand[tid];
+        uint32_t above = 0;
+        for (uint32_t c = 0; c < total; ++c) above += cand[c] > key ? 1u : 0u;
+        if (above < kSamplerTopKMax) top[above] = key;
+      }
       __syncthreads();
     }
   }
@@ -324,7 +311,17 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
       }
     }
     __syncthreads();
-    sort_desc(top, kSamplerTopKMax, kSelectThreads);
+    uint64_t key = 0;
+    uint32_t above = 0;
+    if (tid < kSamplerTopKMax) {
+      key = top[tid];
+      for (uint32_t c = 0; c < kSamplerTopKMax; ++c) above += top[c] > key ? 1u : 0u;
+    }
+    __syncthreads();
+    if (tid < kSamplerTopKMax) top[tid] = 0ull;
+    __syncthreads();
+    if (tid < kSamplerTopKMax && key != 0ull) top[above] = key;
+    __syncthreads();
   }
 
   // ---- softmax with temperature over the sorted candidates, nucleus, draw (sampler.cu:343-388)
@@ -332,34 +329,39 @@ __global__ __launch_bounds__(kSelectThreads) void sample_select_kernel(SamplerPa
   const float max_value = key_value(top[0]);
   if (tid < selected) ex[tid] = expf((key_value(top[tid]) - max_value) * inv_temperature);
   __syncthreads();
+  // The rule's three sums (total, nucleus, draw) are one running sum over the candidates in order, read at
+  // three places: lane 0 forms it once - sequential float additions, the rule's order, eight LDS values
+  // requested per turn - and the two searches ("first candidate whose running share reaches top_p", "first whose
+  // running sum reaches the draw") test every candidate at once.
   if (tid == 0) {
-    float total = 0.0f;
-    for (uint32_t i = 0; i < selected; ++i) total += ex[i];
-    float kept_total = 0.0f;
-    uint32_t kept = selected;
-    if (cfg.top_p < 0.999999f) {
-      kept = 0;
-      for (uint32_t i = 0; i < selected; ++i) {
-        kept_total += ex[i];
-        kept = i + 1;
-        if (total > 0.0f && kept_total / total >= cfg.top_p) break;
-      }
-    } else {
-      kept_total = total;
-    }
-    uint32_t token = key_index(top[0]);
-    if (kept_total > 0.0f && kept != 0) {
-      const float draw = uniform_open(cfg.seed, pos, 0, 1) * kept_total;
-      float cumulative = 0.0f;
-      token = key_index(top[kept - 1]);
-      for (uint32_t i = 0; i < kept; ++i) {
-        cumulative += ex[i];
-        if (draw <= cumulative) {
-          token = key_index(top[i]);
-          break;
+    float run = 0.0f;
+    for (uint32_t i0 = 0; i0 < selected; i0 += 8) {
+      float e[8];
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) e[u] = ex[min(i0 + u, selected - 1)];
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {
+        if (i0 + u < selected) {
+          run += e[u];
+          ex[i0 + u] = run;
         }
       }
     }
+    need_s = selected;   // kept: candidates inside the nucleus
+    count_s = selected;  // first candidate at or above the draw
+  }
+  __syncthreads();
+  const float total = ex[selected - 1];
+  if (cfg.top_p < 0.999999f && tid < selected && total > 0.0f && ex[tid] / total >= cfg.top_p) atomicMin(&need_s, tid + 1);
+  __syncthreads();
+  const uint32_t kept = need_s;
+  const float kept_total = ex[kept - 1];
+  const float draw = uniform_open(cfg.seed, pos, 0, 1) * kept_total;
+  if (tid < kept && draw <= ex[tid]) atomicMin(&count_s, tid);
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t token = key_index(top[0]);
+    if (kept_total > 0.0f) token = key_index(top[count_s < kept ? count_s : kept - 1]);
     publish_token(p.out, token);
   }
 }

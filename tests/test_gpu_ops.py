@@ -589,6 +589,21 @@ def test_sampler_matches_oracle_rule():
                     assert margin < 1e-5, (n, temperature, top_p, top_k, position, got, want, margin)
                     close += 1
     assert close <= checked // 50
+    # a masked vocabulary: fewer finite logits than top_k asks for, the rest -inf (and a few +inf / NaN): every
+    # finite logit is a candidate and nothing else is
+    l = np.full(5000, -np.inf, np.float32)
+    keep = rng.choice(5000, 50, replace=False)
+    l[keep] = (rng.standard_normal(50) * 2).astype(np.float32)
+    l[[7, 4000]] = np.inf
+    l[11] = np.nan
+    buf = dev(l)
+    ws = N.DeviceBuffer.zeros(abi.load().nerva_hip_sample_workspace_bytes(l.size))
+    for temperature, top_p, top_k in ((0.8, 0.95, 100), (1.5, 0.5, 0), (0.7, 1.0, 60)):
+        for position in range(8):
+            want, margin = O.sample(l, temperature, top_p, top_k, 5, position)
+            got = N.sample(buf, l.size, temperature, top_p, top_k, 5, position, ws)
+            assert np.isfinite(l[got]), (temperature, top_p, top_k, position, got)
+            assert got == want or margin < 1e-5, (temperature, top_p, top_k, position, got, want, margin)
     # logits piled into the first chunks: the bound from the chunk maxima prunes nothing, and the
     # selection takes its general route (radix selection over all chunk candidates)
     l = (-1e-3 * np.arange(151936)).astype(np.float32)
