@@ -10,11 +10,13 @@
 // gfx950 mapping of the fast path (head_dim 128, G = heads/kv_heads in {1,2,4,8}):
 //   grid (kv_heads, splits), 8 waves per workgroup; a wave owns whole 16-token KV
 //   tiles of its workgroup's token range and runs q.K^T and P.V on the matrix cores
-//   (details at attn_fast_kernel). The cache keeps each tile in matrix-operand order,
+//   (details at attn_fast_body). The cache keeps each tile in matrix-operand order,
 //   so a tile is eight coalesced 1 KiB loads straight into operand registers; two tiles
 //   are in flight per wave. LDS only carries q, the new K/V row and the cross-wave
 //   merge. The last workgroup to finish a kv head merges its split partials (arrival
 //   counter; nobody waits), so a layer needs no separate reduce launch.
+#include <stdlib.h>
+
 #include "attn_decode.cuh"
 #include "attn_tile.cuh"
 
@@ -86,18 +88,8 @@ __global__ __launch_bounds__(2 * kWave) void kv_publish_rows_kernel(AttnParams p
   }
 }
 
-// Stand-alone launch of the matrix-core attention (attn_fast_body): grid (kv_heads, splits[, tokens]).
-template <uint32_t DT, int G, int W>
-__global__ __launch_bounds__(W *kWave) void attn_fast_kernel(AttnParams p) {
-  __shared__ AttnShared<G, W> sh;
-  if (blockIdx.z != 0) token_view(p, blockIdx.z);
-  const RawHeads<G, W> raw = attn_request_raw<G, W>(p, blockIdx.x);  // before anything they could queue behind
-  const uint32_t pos = p.cursor != nullptr ? *p.cursor : p.position;
-  if (p.cursor != nullptr && pos >= p.max_steps) return;
-  attn_fast_body<DT, G, W>(p, pos, blockIdx.x, blockIdx.y, gridDim.y, sh, raw);
-}
-
-// Prompt-block launch of the same body (grid z = tokens): the lean variant, two workgroups per CU.
+// Launch of the matrix-core attention body (attn_fast_body) for token blocks and batch steps: grid (kv_heads,
+// splits, tokens); the lean variant, two workgroups per CU.
 template <uint32_t DT, int G, int W>
 __global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams p) {
   __shared__ AttnShared<G, W> sh;
@@ -107,7 +99,7 @@ __global__ __launch_bounds__(W *kWave, W / 2) void attn_block_kernel(AttnParams 
 }
 
 // ---------------------------------------------------------------------------------------------
-// The decode step's launch: one token, grid (kv_heads, splits), 8 waves, G = 1, 2 or 4 query heads per
+// The decode step's launch: one token, grid (kv_heads, splits), 8 waves, G = 1, 2, 4 or 8 query heads per
 // kv head. Same arithmetic as attn_fast_body (same tile step, same merges); what differs is the order
 // in which a wave asks for things, because at decode sizes - a wave owns two or three 8 KiB tiles of an
 // 8k-token context - the launch is one burst of requests and a chain of latencies, not a stream:
@@ -700,12 +692,12 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
       }
       return hipGetLastError();
     }
-    if (group != 8 && p.part_tagged == nullptr) return hipErrorInvalidValue;
+    if (p.part_tagged == nullptr) return hipErrorInvalidValue;
     switch (group) {
       case 1: hipLaunchKernelGGL((attn_step_kernel<DT, 1>), grid, dim3(8 * kWave), 0, stream, p); break;
       case 2: hipLaunchKernelGGL((attn_step_kernel<DT, 2>), grid, dim3(8 * kWave), 0, stream, p); break;
       case 4: hipLaunchKernelGGL((attn_step_kernel<DT, 4>), grid, dim3(8 * kWave), 0, stream, p); break;
-      default: hipLaunchKernelGGL((attn_fast_kernel<DT, 8, kAttnWaves / 2>), grid, dim3(kAttnWaves / 2 * kWave), 0, stream, p); break;
+      default: hipLaunchKernelGGL((attn_step_kernel<DT, 8>), grid, dim3(8 * kWave), 0, stream, p); break;
     }
   } else {
     if (p.head_dim > 512) return hipErrorInvalidValue;

@@ -184,7 +184,7 @@ __device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t phy
   }
 }
 
-// One 16-token tile against the G query heads of the kv head (see attn_fast_kernel).
+// One 16-token tile against the G query heads of the kv head (see attn_fast_body).
 // n_keys may differ from lane to lane (by column: the prompt kernel's columns belong to tokens at
 // different positions). COLUMN_MASKS = a column may find a whole tile masked, even its first one: the
 // running maximum then stays at minus infinity, and the exponentials are taken against a finite stand-in

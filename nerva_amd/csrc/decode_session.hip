@@ -1079,9 +1079,9 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->attn_ws = s->arena + off_attn_ws;
   s->attn_tagged = reinterpret_cast<uint64_t *>(s->arena + off_attn_tagged);
   {
-    // the plan serves the step kernel (head_dim 128, 1, 2 or 4 query heads per kv head, 8 waves)
+    // the plan serves the step kernel (head_dim 128, 1, 2, 4 or 8 query heads per kv head, 8 waves)
     const uint32_t group = s->kv_heads != 0 ? s->heads / s->kv_heads : 0;
-    if (s->head_dim == 128 && (group == 1 || group == 2 || group == 4))
+    if (s->head_dim == 128 && (group == 1 || group == 2 || group == 4 || group == 8))
       s->attn_plan = reinterpret_cast<uint32_t *>(s->arena + off_attn_plan);
   }
   s->sample_ws = s->arena + off_sample_ws;

@@ -465,6 +465,28 @@ def test_paged_attention_other_geometries(heads, kv_heads, hd, dtype, theta, qk_
         assert rel_l2(got32, ref) <= REL_L2
 
 
+@pytest.mark.parametrize("heads,kv_heads", [(64, 8), (32, 4), (16, 16)])
+def test_paged_attention_step_kernel_group_sizes_at_long_context(heads, kv_heads):
+    """GQA factors 8 and 1 and a 4-kv-head layout (64 splits) through the decode-step kernel at contexts where the
+    splits merge (and, with few forced splits, where a wave re-requests tiles): oracle parity, same bits on a
+    second launch."""
+    for tokens, splits in ((333, 0), (1000, 0), (4096, 0), (4096, 3), (2500, 64 if kv_heads <= 4 else 32)):
+        c = _attention_case(BF16, heads, kv_heads, 128, tokens, 1e6, True, heads + tokens)
+        ref, _, _ = _attention_oracle(c)
+        cache = N.PagedKvCache(c["layers"], c["n_blocks"], kv_heads, 128, c["table"])
+        cache.fill(c["layer"], c["k_rows"], c["v_rows"])
+        ws = attention_workspace(heads, 128)
+        out16, out32 = N.DeviceBuffer(heads * 128 * 2), N.DeviceBuffer(heads * 128 * 4)
+        outs = []
+        for _ in range(2):
+            N.paged_attention(BF16, heads, kv_heads, 128, cache, c["layer"], tokens, dev(c["qkv"]), ws, out16,
+                              out_f32=out32, append=True, rope_theta=1e6, q_norm=dev(c["qn"]), k_norm=dev(c["kn"]),
+                              splits=splits)
+            outs.append(out32.numpy(np.float32).copy())
+        assert rel_l2(outs[0], ref) <= REL_L2, (tokens, splits)
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), (tokens, splits)
+
+
 def test_paged_attention_permutation_invariance_and_repeatability():
     """Same logical KV under two block tables gives the same bits; so does calling twice."""
     base = _attention_case(BF16, 32, 8, 128, 777, 1e6, True, 42)
