@@ -401,7 +401,8 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
 // 5 with the RMSNorm prologue, which holds the f32 activations and the norm weights in
 // registers across the first weight requests (a budget of 6 makes it spill).
 constexpr int fast_waves_per_simd(int prologue) { return prologue == kProRmsNorm ? 5 : 6; }
-constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per lane
+constexpr int kFastMaxCols = 12288;  // x staged through at most 6 x 16 B per lane in registers ...
+constexpr int kFastMaxColsLoop = 30720;  // ... or, with a 16-bit input, copied into LDS behind the first weight requests
 
 // EXACT (short launches: a wave's whole share is the two batches requested up front, so the start-up is
 // the launch): the first two batches and the residual element are requested unconditionally - a wave
@@ -441,12 +442,17 @@ __global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) voi
   float4 xa[PRO == kProRmsNorm ? 2 : 1], xb[PRO == kProRmsNorm ? 2 : 1];
   uint4 gw[PRO == kProRmsNorm ? 2 : 1];
   const bool norm_in_regs = cols <= TB * 16;
+  // (the same for every wave of the launch; a constant in the variant with exact start-up waits, which only
+  // runs at 4096 columns, so its request counts stay countable)
+  const bool x_in_regs = EXACT || cols <= static_cast<uint32_t>(kFastMaxCols);
   if constexpr (PRO == kProX16) {
+    if (x_in_regs) {
 #pragma unroll
-    for (int i = 0; i < kXV; ++i) {
-      const uint32_t c = (i * TB + threadIdx.x) * 8;
-      xraw[i] = make_uint4(0u, 0u, 0u, 0u);
-      if (c < cols) xraw[i] = *reinterpret_cast<const uint4 *>(p.x16 + c);
+      for (int i = 0; i < kXV; ++i) {
+        const uint32_t c = (i * TB + threadIdx.x) * 8;
+        xraw[i] = make_uint4(0u, 0u, 0u, 0u);
+        if (c < cols) xraw[i] = *reinterpret_cast<const uint4 *>(p.x16 + c);
+      }
     }
   } else {
     if (norm_in_regs) {
@@ -497,10 +503,17 @@ __global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) voi
 
   // ---- 4. prologue: x -> LDS as 16-bit
   if constexpr (PRO == kProX16) {
+    if (x_in_regs) {
 #pragma unroll
-    for (int i = 0; i < kXV; ++i) {
-      const uint32_t c = (i * TB + threadIdx.x) * 8;
-      if (c < cols) *reinterpret_cast<uint4 *>(xs + c) = xraw[i];
+      for (int i = 0; i < kXV; ++i) {
+        const uint32_t c = (i * TB + threadIdx.x) * 8;
+        if (c < cols) *reinterpret_cast<uint4 *>(xs + c) = xraw[i];
+      }
+    } else {
+      // rows of more than kFastMaxCols columns (MLP widths above 12288): such a launch is long, its start-up is not
+      // what it costs, and the vector would not fit the register budget
+      for (uint32_t c = threadIdx.x * 8; c < cols; c += TB * 8)
+        *reinterpret_cast<uint4 *>(xs + c) = *reinterpret_cast<const uint4 *>(p.x16 + c);
     }
   } else {
     float ss = 0.0f;

@@ -61,6 +61,8 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
     // LM head do not move, so only the plain and residual epilogues have the variant.
     constexpr bool kShortShapes = EPI == kEpiF32 || EPI == kEpiResidual;
     constexpr uint32_t kBatchCols = kWave * 8u * (4 / NR);
+    // rows that are whole batches of 1024 columns but not of 2048 (hidden 5120, MLP width 25600): two chunks a batch
+    const bool half_batches = NR == 1 && p.cols % kBatchCols != 0;
     const uint32_t units_per_wave = (p.rows + blocks * kWavesPerBlock - 1) / (blocks * kWavesPerBlock);
     const int forced = tuning(kTuneGemvExactStart);
     const bool can = kShortShapes && p.cols >= 2u * kBatchCols;
@@ -74,7 +76,14 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
 #define NV_GEMV_LAUNCH(EX, W, XR)                                                                              \
   hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, EX, W, XR>), dim3((waves + W - 1) / W),         \
                      dim3(W * kWave), lds, stream, p)
-    if (can && want) {
+    if (half_batches) {
+      if (wg == 16)
+        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 2, false, 16, false>), dim3((waves + 15) / 16), dim3(16 * kWave), lds,
+                           stream, p);
+      else
+        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 2, false, 4, false>), dim3((waves + 3) / 4), dim3(4 * kWave), lds,
+                           stream, p);
+    } else if (can && want) {
       if constexpr (kShortShapes) {
         if (wg == 16) NV_GEMV_LAUNCH(true, 16, false);
         else if constexpr (PRO == kProX16) {
@@ -135,15 +144,15 @@ int fast_workgroup_waves(int prologue, int epilogue, uint32_t rows, uint32_t col
 
 }  // namespace
 
-// kFast needs cols % 2048 == 0 (% 1024 for the gate/up pair) and cols <= kFastMaxCols.
+// kFast needs cols % 1024 == 0 and cols <= kFastMaxCols (kFastMaxColsLoop with a 16-bit input).
 GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,
                    const GemvTuning *tuning) {
   GemvPlan plan;
   const bool vec = vec16 && cols % 8 == 0;
   plan.mode = !vec ? kScalar : (cols % (kWave * 8) == 0 ? kVecFull : kVecGuarded);
-  const uint32_t fast_cols = epilogue == kEpiSwiglu ? kWave * 8 * 2 : kWave * 8 * 4;
-  if (plan.mode == kVecFull && cols % fast_cols == 0 && cols <= static_cast<uint32_t>(kFastMaxCols) &&
-      !(tuning && tuning->force_generic))
+  const uint32_t fast_cols = kWave * 8 * 2;
+  const uint32_t max_cols = prologue == kProX16 ? kFastMaxColsLoop : kFastMaxCols;
+  if (plan.mode == kVecFull && cols % fast_cols == 0 && cols <= max_cols && !(tuning && tuning->force_generic))
     plan.mode = kFast;
   // one wave per unit (a row, or a gate/up pair)
   const uint32_t want = (rows + kWavesPerBlock - 1) / kWavesPerBlock;

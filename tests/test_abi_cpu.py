@@ -303,6 +303,12 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
     assert N.gemv_launch_shape(0, 1, 4096, 4096) == (3, 1024)      # o: every row on the machine at once
     assert N.gemv_launch_shape(1, 4, 151936, 4096) == (3, 512)     # LM head: 16-wave workgroups
     assert N.gemv_launch_shape(0, 0, 100, 520)[0] == 1             # 520 columns: the guarded vector kernel
+    # other models' widths on the lean kernel: batches of 1024 columns, rows of up to 30720 columns with a 16-bit input
+    for pro, epi, rows, cols in ((0, 1, 4096, 14336), (0, 1, 5120, 25600), (1, 0, 10240, 5120), (0, 1, 8192, 28672),
+                                 (1, 2, 25600, 5120), (1, 0, 8192, 8192)):
+        assert N.gemv_launch_shape(pro, epi, rows, cols)[0] == 3, (pro, epi, rows, cols)
+    assert N.gemv_launch_shape(0, 1, 64, 31744)[0] == 2           # past the limit: the general vector kernel
+    assert N.gemv_launch_shape(1, 0, 64, 13312)[0] == 2           # the RMSNorm prologue keeps its 12288-column limit
     with pytest.raises(ValueError):
         N.gemv_launch_shape(0, 0, 0, 64)
     for name in ("attn_splits", "batch_splits", "prompt_splits", "gemm_row_tiles", "gemm_k_waves",

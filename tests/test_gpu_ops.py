@@ -66,9 +66,11 @@ def _gemv_case(dtype, rows, cols, seed, std=0.02):
 
 
 @pytest.mark.parametrize("dtype", [BF16, F16])
-@pytest.mark.parametrize("rows,cols", [(4096, 4096), (6144, 4096), (1030, 12288), (37, 520), (5, 2), (3, 4104), (2, 7)])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (6144, 4096), (1030, 12288), (37, 520), (5, 2), (3, 4104), (2, 7),
+                                       (515, 14336), (260, 25600), (130, 28672), (1027, 5120), (66, 30720)])
 def test_gemv_plain_matches_oracle(dtype, rows, cols):
-    """Config 1 (q_proj 4096x4096 bf16, x bf16, bf16 out) plus ragged / unaligned shapes."""
+    """Config 1 (q_proj 4096x4096 bf16, x bf16, bf16 out) plus ragged / unaligned shapes, rows of other models'
+    widths (batches of 1024 columns: 5120, 25600; more than 12288 columns: the input copied into LDS by a loop)."""
     w, x = _gemv_case(dtype, rows, cols, rows * 31 + cols)
     ref = O.gemv_x16(dtype, w, x)
     dw, dx = dev(w), dev(x)
@@ -158,7 +160,7 @@ def test_gemv_start_up_variants_are_the_same_function(shape):
 
 
 @pytest.mark.parametrize("dtype", [BF16, F16])
-@pytest.mark.parametrize("cols,rows", [(4096, 6144), (520, 64), (6, 3)])
+@pytest.mark.parametrize("cols,rows", [(4096, 6144), (520, 64), (6, 3), (5120, 1030), (8192, 515), (12288, 70), (13312, 33)])
 def test_gemv_rmsnorm_prologue(dtype, cols, rows):
     """qkv projection: x = round16(rmsnorm(h, gamma)) fused in front of the GEMV."""
     rng = np.random.default_rng(cols)
