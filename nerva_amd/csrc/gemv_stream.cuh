@@ -383,7 +383,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// Production-shape kernel: cols % (512 * B) == 0, 16-byte aligned rows, cols <= 12288.
+// Production-shape kernel: cols % (512 * B) == 0, 16-byte aligned rows, cols <= 12288 (30720 with a 16-bit input).
 // Same contract as gemv_kernel, leaner register budget (about 64 VGPRs instead of
 // ~150) so that 6-8 workgroups stay resident per CU and a whole 4096-row matrix is
 // on the machine at once. A wave walks a flat list of request batches - (its 1st
