@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kPW *kWave) void attn_prompt_kernel(AttnParams p) {
         kreg[j] = stage[st][j][lane];
         vreg[j] = stage[st][4 + j][lane];
       }
-      attn_tile<DT, kVG, false, true>(kreg, vreg, qx, nullptr, b, n_keys, col, grp, false, 0u, nullptr, nullptr, m, l, acc);
+      attn_tile<DT, kVG, false, true, true>(kreg, vreg, qx, nullptr, b, n_keys, col, grp, false, 0u, nullptr, nullptr, m, l, acc);
     }
   }
   if (!wave_on) return;

@@ -189,7 +189,10 @@ __device__ __forceinline__ void attn_load_tile(const AttnParams &p, uint32_t phy
 // different positions). COLUMN_MASKS = a column may find a whole tile masked, even its first one: the
 // running maximum then stays at minus infinity, and the exponentials are taken against a finite stand-in
 // so that they come out as 0 instead of NaN.
-template <uint32_t DT, int G, bool QX_LDS, bool COLUMN_MASKS = false>
+// LAZY_RESCALE = the accumulators are multiplied by alpha only in tiles where some lane's alpha is not 1 (a
+// running maximum that did not move gives exp2(0) = 1 exactly, so the result is the same bits): worth a branch
+// where a wave walks many tiles and the vector ALU is what it waits for (prompt blocks).
+template <uint32_t DT, int G, bool QX_LDS, bool COLUMN_MASKS = false, bool LAZY_RESCALE = false>
 __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], const uint4 (&qx)[4],
                                           const uint4 *qx_lds, uint32_t b,
                                           uint32_t n_keys, int col, int grp, bool splice, uint32_t new_row,
@@ -254,9 +257,15 @@ __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], co
   l = l * alpha + psum;
   m = m_new;
   const uint2 pb = make_uint2(px[0], px[1]);
+  if constexpr (LAZY_RESCALE) {
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int s2 = 0; s2 < 8; ++s2) acc[s2] *= alpha;
+    }
+  }
 #pragma unroll
   for (int s2 = 0; s2 < 8; ++s2) {
-    acc[s2] *= alpha;
+    if constexpr (!LAZY_RESCALE) acc[s2] *= alpha;
     const uint4 &vr = vreg[s2 / 2];
     const uint2 va = (s2 & 1) ? make_uint2(vr.z, vr.w) : make_uint2(vr.x, vr.y);
     acc[s2] = mfma_k16<DT>(va, pb, acc[s2]);
