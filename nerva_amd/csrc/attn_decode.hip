@@ -148,8 +148,8 @@ constexpr uint32_t kStepParts = 4, kStepPartDims = kHD / kStepParts, kStepPartWo
 constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
 // One part (32 dims of one head) merged by one workgroup of 512 threads. Thread (dl = t % 32,
 // q = t / 32) takes the splits q, q + 16, q + 32, q + 48: it polls their accumulator word and their m
-// and l words until every tag is up and folds them in split order; the sixteen groups meet in LDS in
-// group order - a fixed order, whatever the arrival order was. A CU sustains only a few hundred
+// and l words until every tag is up and folds them in split order; the two groups of a wave meet by a lane
+// exchange and the eight waves in LDS, in wave order - a fixed order, whatever the arrival order was. A CU sustains only a few hundred
 // device-coherent cache lines per microsecond, which is why a head is spread over several merging
 // workgroups. Last of all every word that was read gets its tag cleared for the next launch (launches
 // are ordered by the stream). A wait that runs out (a split that never stored: cannot happen on a
@@ -158,7 +158,7 @@ constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
 constexpr uint32_t kMergeSpinLimit = 1u << 20;
 template <uint32_t DT, int G>
 __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t kvh, uint32_t g, uint32_t part, uint32_t S,
-                                                  uint32_t active, float *lds_o, float *lds_m, float *lds_l) {
+                                                  uint32_t active, float *lds_o, float *lds_m, float *lds_l, bool first_part) {
   constexpr uint32_t kGroups = 16, kPer = kAttnMaxSplits / kGroups;  // 4 splits per thread at most
   const uint32_t h = kvh * G + g;
   uint64_t *rec = p.part_tagged + static_cast<uint64_t>(h) * S * kStepRecord + part * kStepPartWords;
@@ -193,21 +193,39 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
       o = fmaf(tag_value(av[i]), f, o);
     }
   }
-  __syncthreads();  // the LDS arrays below were read by the wave merge (or by the previous part's merge)
-  lds_o[q * kStepPartDims + dl] = gave_up ? NAN : o;
-  if (dl == 0) {
-    lds_m[q] = M;
-    lds_l[q] = L;
+  // the two groups of a wave (its lanes 0-31 and 32-63) meet by a lane exchange, the even group's sum first;
+  // the eight waves meet in LDS (arrays of their own: no barrier before they are written, except between parts)
+  {
+    const float Mo = __shfl_xor(M, static_cast<int>(kStepPartDims), kWave), Lo = __shfl_xor(L, static_cast<int>(kStepPartDims), kWave),
+                oo = __shfl_xor(o, static_cast<int>(kStepPartDims), kWave);
+    const bool even = (q & 1u) == 0;
+    const float Ma = even ? M : Mo, La = even ? L : Lo, oa = even ? o : oo;
+    const float Mb = even ? Mo : M, Lb = even ? Lo : L, ob = even ? oo : o;
+    const float Mw = fmaxf(Ma, Mb);
+    const float fa = Ma > -INFINITY ? attn_exp2(Ma - Mw) : 0.0f, fb = Mb > -INFINITY ? attn_exp2(Mb - Mw) : 0.0f;   // a group without a split
+    M = Mw;
+    L = fmaf(Lb, fb, La * fa);
+    o = fmaf(ob, fb, oa * fa);
+  }
+  constexpr uint32_t kWaves = kGroups / 2;
+  const uint32_t w = q / 2;
+  if (!first_part) __syncthreads();   // the previous part's last reads
+  if ((q & 1u) == 0) {
+    lds_o[w * kStepPartDims + dl] = gave_up ? NAN : o;
+    if (dl == 0) {
+      lds_m[w] = M;
+      lds_l[w] = L;
+    }
   }
   __syncthreads();
   if (q == 0) {
     float Mt = -INFINITY;
 #pragma unroll
-    for (uint32_t k = 0; k < kGroups; ++k) Mt = fmaxf(Mt, lds_m[k]);
+    for (uint32_t k = 0; k < kWaves; ++k) Mt = fmaxf(Mt, lds_m[k]);
     float Lt = 0.0f, ot = 0.0f;
 #pragma unroll
-    for (uint32_t k = 0; k < kGroups; ++k) {
-      const float f = lds_m[k] > -INFINITY ? attn_exp2(lds_m[k] - Mt) : 0.0f;  // a group without a split
+    for (uint32_t k = 0; k < kWaves; ++k) {
+      const float f = lds_m[k] > -INFINITY ? attn_exp2(lds_m[k] - Mt) : 0.0f;  // a wave without a split
       Lt = fmaf(lds_l[k], f, Lt);
       ot = fmaf(lds_o[k * kStepPartDims + dl], f, ot);
     }
@@ -245,6 +263,7 @@ struct StepShared {
   alignas(16) uint16_t vnew[kHD];
   float wm[8][G], wl[8][G];
   alignas(16) float wacc[8][G][kHD];
+  float merge_o[8][32], merge_m[8], merge_l[8];   // the splits' merge: one entry per wave
   uint32_t is_last;
 };
 
@@ -521,8 +540,7 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   // after the stores have been performed and a merge by the last arriver needed four.
   for (uint32_t j = split; j < G * kStepParts; j += active) {
     link_mark(trm, 16);
-    float *lds = sh.wacc[0][0];  // at least 1024 floats, free once the wave merge has been read
-    merge_part_tagged<DT, G>(p, kvh, j % G, j / G, S, active, lds, lds + 512, lds + 528);
+    merge_part_tagged<DT, G>(p, kvh, j % G, j / G, S, active, sh.merge_o[0], sh.merge_m, sh.merge_l, j == split);
     link_mark(trm, 17);
   }
 }
