@@ -15,11 +15,12 @@
 //   select kernel  greedy / Gumbel: best of the chunk candidates.
 //                  top-k: the k-th largest of the chunks' best keys bounds the k-th largest key of the
 //                  vocabulary from below, so one pass over the logits collects the keys at or above
-//                  that bound - a few hundred when the logits are spread over the chunks - and a sort in
-//                  LDS orders them. If more than 1024 survive (logits piled into few chunks), the exact
-//                  k-th largest key comes from a radix selection over the whole vocabulary (six digits,
-//                  histogram in LDS, parallel suffix scan) instead. Then exponentials in parallel, and
-//                  the three short sums of the rule (total, nucleus, draw) by one lane in the rule's order.
+//                  that bound - a few hundred when the logits are spread over the chunks - and each
+//                  survivor finds its place by counting the survivors with a larger key. If more than 1024
+//                  survive (logits piled into few chunks), the exact k-th largest key comes from a radix
+//                  selection over the whole vocabulary (six digits, histogram in LDS, parallel suffix scan)
+//                  instead. Then exponentials in parallel, one running sum in the rule's order by one
+//                  lane, and the nucleus and the draw read from it by parallel searches.
 //                  (The chunks used to sort their 1024 keys and hand out their best 128: 38 + 30-43 us for
 //                  the two launches at 151936 logits, barrier-bound.)
 //   then the token slot is written and the device cursor advanced, as the greedy finish does.

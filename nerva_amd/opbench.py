@@ -214,13 +214,14 @@ def case_gemm_rows():
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
         w = synth16(copies * wrows * cols, 61)
         ws = DeviceBuffer(R.gemm_rows_workspace_bytes(wrows))   # K slices of the large-block kernel
-        for tokens in (1, 8, 32, 64, 128):
+        for tokens in (1, 8, 32, 64, 128) + ((256,) if rows <= 12288 else ()):
             x = synth16(max(tokens, 128) * cols, 62, std=1.0)
             y32 = DeviceBuffer(tokens * rows * 4)
             y16 = DeviceBuffer(max(tokens, 128) * rows * 2)
             nbytes = wrows * cols * 2 + tokens * cols * 2 + tokens * rows * (2 if epi == 2 else 4)
             # "operand order": the activations in the layout token blocks keep inside the session
-            for packed in ((False,) if tokens < 32 else (False, True)):
+            # (blocks of more than 128 tokens exist in operand order only)
+            for packed in ((False,) if tokens < 32 else (True,) if tokens > 128 else (False, True)):
                 ns = timed(lambda i: R.gemm_rows(BF16, w.at((i % copies) * wrows * cols * 2), rows, cols, tokens, x, epilogue=epi,
                                                  out_f32=y32, out16=y16, sync=False, input_operand_order=packed,
                                                  output16_operand_order=packed and epi == 2, workspace=ws), 2 * copies)
