@@ -12,6 +12,7 @@ struct Fp8GemvParams {
   const float *xf;        // [tokens x cols] when x16 is null
   float *out;             // [tokens x rows]
   uint32_t rows, cols, block_rows, block_cols, tokens, input_dtype;
+  uint32_t x_first = 1;  // set by the launcher (lean one-token kernel: activations requested ahead of the weights)
 };
 
 struct MoeFp8Params {

@@ -293,95 +293,269 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(MoeFp8Params p) {
 // (fully unrolled, no register copies), so rows, and in the down kernel experts,
 // follow each other without a bubble.
 // ---------------------------------------------------------------------------
-template <uint32_t DT>
-__global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Params p) {
-  extern __shared__ __align__(16) uint16_t xs16[];  // the 16-bit activations as they came, in lean order
+constexpr uint32_t kLeanMaxSlots = 65;  // top_k <= 64 routed experts + the shared one
+
+// The lean streaming loop over ROW PAIRS against 16-bit activations in LDS (lean order): a wave walks a flat
+// list of batches - one 1 KiB chunk of each row of its pair plus the two block scales - through a ring of four.
+// The requests are issued by hand and each batch is awaited with an explicit count of the newer requests that
+// may stay in flight (requests return in issue order). With the compiler's own bookkeeping the refills under
+// `if (t + n < total)` made every use wait for the whole ring: four batches per round trip instead of a
+// rolling window. A pair's results are stored by ordinary stores between the requests; the counts ignore
+// them, which is safe whichever way stores and loads complete relative to each other.
+// What a pair is comes from the policy:
+//   rows<TABLE>(unit, w0, w1, s0, s1)  the two weight rows and their scale rows (TABLE: tables in LDS may be
+//                                      read - false for the requests in front of the workgroup's barrier)
+//   finish(unit, a, b, lane)           the two dot products, reduced over the wave
+constexpr uint32_t kLeanPairMaxWaves = 8;
+constexpr uint32_t kLeanPairMinCols = 256;  // shorter rows keep the general kernels
+template <uint32_t DT, class Policy>
+__device__ __forceinline__ void lean_pair_stream(const Policy &pol, const uint16_t *x16, uint32_t cols,
+                                                 uint32_t block_cols, uint32_t units, uint16_t *xs16, bool x_ahead) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
-  const uint32_t units = slots * p.inter;
-  const uint32_t sc_cols = (p.hidden + p.block - 1) / p.block;
-  const uint64_t scale_stride = static_cast<uint64_t>((p.inter + p.block - 1) / p.block) * sc_cols;
-  const uint64_t w_stride = static_cast<uint64_t>(p.inter) * p.hidden;
-  const uint32_t wave_global = blockIdx.x * kWavesPerBlock + wave;
-  const uint32_t wave_stride = gridDim.x * kWavesPerBlock;
-  const uint32_t bpr = p.hidden / 1024u;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t waves = blockDim.x / kWave;   // the host picks the workgroup size (lean_pair_grid)
+  const uint32_t wave_global = blockIdx.x * waves + wave;
+  const uint32_t wave_stride = gridDim.x * waves;
+  // cols is a multiple of 16; a last chunk of fewer than 1024 columns has idle lanes: they ask for the row's first
+  // bytes again, meet zeros in LDS and take a zero scale
+  const uint32_t bpr = (cols + 1023u) / 1024u;
+  const bool ragged = (cols & 1023u) != 0;
   const uint32_t my_units = wave_global < units ? (units - wave_global + wave_stride - 1) / wave_stride : 0u;
   const uint32_t total = my_units * bpr;
 
+  typedef uint32_t lp_u32x4_t __attribute__((ext_vector_type(4)));
   uint32_t iu = wave_global, ib = 0;
-  const uint8_t *wg = nullptr, *wu = nullptr;
-  const float *sg = nullptr, *su = nullptr;
-  uint4 bg0, bg1, bg2, bg3, bu0, bu1, bu2, bu3;
-  float fg0, fg1, fg2, fg3, fu0, fu1, fu2, fu3;
-#define NV_GU_ISSUE(J)                                                                        \
+  const uint8_t *wa = nullptr, *wb = nullptr;
+  const float *sa = nullptr, *sb = nullptr;
+  lp_u32x4_t ba0, ba1, ba2, ba3, bb0, bb1, bb2, bb3;
+  float fa0, fa1, fa2, fa3, fb0, fb1, fb2, fb3;
+#define NV_LP_ISSUE(J, TABLE)                                                                 \
   do {                                                                                        \
-    if (ib == 0) {                                                                            \
-      const uint32_t k = iu / p.inter, i = iu % p.inter;                                      \
-      uint32_t e = k < p.top_k ? p.expert_ids[k] : static_cast<uint32_t>(p.shared_index);     \
-      if (e >= p.num_experts) e = 0;                                                          \
-      const uint64_t row = e * w_stride + static_cast<uint64_t>(i) * p.hidden + lane * 16;    \
-      wg = p.w_gate + row;                                                                    \
-      wu = p.w_up + row;                                                                      \
-      const uint64_t srow = e * scale_stride + static_cast<uint64_t>(i / p.block) * sc_cols;  \
-      sg = p.s_gate + srow;                                                                   \
-      su = p.s_up + srow;                                                                     \
-    }                                                                                         \
-    bg##J = load_stream(wg + ib * 1024u);                                                     \
-    bu##J = load_stream(wu + ib * 1024u);                                                     \
-    fg##J = sg[(ib * 1024u + lane * 16) / p.block];                                           \
-    fu##J = su[(ib * 1024u + lane * 16) / p.block];                                           \
+    if (ib == 0) pol.template rows<TABLE>(iu, wa, wb, sa, sb);                                \
+    uint32_t col_ = ib * 1024u + lane * 16;                                                   \
+    if (col_ >= cols) col_ = 0;                                                               \
+    const uint8_t *q0_ = wa + col_, *q1_ = wb + col_;                                         \
+    const float *r0_ = sa + col_ / block_cols;                                                \
+    const float *r1_ = sb + col_ / block_cols;                                                \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(ba##J) : "v"(q0_) : "memory");   \
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(bb##J) : "v"(q1_) : "memory");   \
+    asm volatile("global_load_dword %0, %1, off" : "=v"(fa##J) : "v"(r0_) : "memory");        \
+    asm volatile("global_load_dword %0, %1, off" : "=v"(fb##J) : "v"(r1_) : "memory");        \
     if (++ib == bpr) {                                                                        \
       ib = 0;                                                                                 \
       iu += wave_stride;                                                                      \
     }                                                                                         \
   } while (0)
+  // The wait and the hand-over of a batch to compiler-visible registers are one asm statement: the moves read
+  // the request's destination registers after the wait whatever registers the compiler picks for either side.
+  lp_u32x4_t ua, ub;
+  float ga, gb;
+#define NV_LP_TAKE(WAIT, J)                                                                   \
+  asm volatile(WAIT "\n\tv_mov_b32 %0, %10\n\tv_mov_b32 %1, %11\n\tv_mov_b32 %2, %12\n\tv_mov_b32 %3, %13" \
+               "\n\tv_mov_b32 %4, %14\n\tv_mov_b32 %5, %15\n\tv_mov_b32 %6, %16\n\tv_mov_b32 %7, %17"     \
+               "\n\tv_mov_b32 %8, %18\n\tv_mov_b32 %9, %19"                                       \
+               : "=&v"(ua.x), "=&v"(ua.y), "=&v"(ua.z), "=&v"(ua.w), "=&v"(ub.x), "=&v"(ub.y),     \
+                 "=&v"(ub.z), "=&v"(ub.w), "=&v"(ga), "=&v"(gb)                                    \
+               : "v"(ba##J.x), "v"(ba##J.y), "v"(ba##J.z), "v"(ba##J.w), "v"(bb##J.x),             \
+                 "v"(bb##J.y), "v"(bb##J.z), "v"(bb##J.w), "v"(fa##J), "v"(fb##J)                  \
+               : "memory")
+#define NV_LP_AWAIT(J, NEWER)                                                                 \
+  do {                                                                                        \
+    const uint32_t newer_ = (NEWER);                                                          \
+    if (newer_ >= 3u) NV_LP_TAKE("s_waitcnt vmcnt(12)", J);                                   \
+    else if (newer_ == 2u) NV_LP_TAKE("s_waitcnt vmcnt(8)", J);                               \
+    else if (newer_ == 1u) NV_LP_TAKE("s_waitcnt vmcnt(4)", J);                               \
+    else NV_LP_TAKE("s_waitcnt vmcnt(0)", J);                                                 \
+  } while (0)
 
   uint32_t cu = wave_global, cb = 0;
-  float ag = 0.0f, au = 0.0f;
-#define NV_GU_CONSUME(J)                                                                      \
+  float aa = 0.0f, ab = 0.0f;
+#define NV_LP_CONSUME()                                                                       \
   do {                                                                                        \
     const uint16_t *xp = xs16 + cb * 1024u + lane * 8;                                        \
     const uint4 xa = *reinterpret_cast<const uint4 *>(xp);                                    \
     const uint4 xb = *reinterpret_cast<const uint4 *>(xp + 512);                              \
-    ag = fmaf(fg##J, dot16_fp8_x16<DT>(bg##J, xa, xb), ag);                                   \
-    au = fmaf(fu##J, dot16_fp8_x16<DT>(bu##J, xa, xb), au);                                   \
+    if (ragged && cb == bpr - 1u && cb * 1024u + lane * 16 >= cols) {                         \
+      ga = 0.0f;                                                                              \
+      gb = 0.0f;                                                                              \
+    }                                                                                         \
+    aa = fmaf(ga, dot16_fp8_x16<DT>(make_uint4(ua.x, ua.y, ua.z, ua.w), xa, xb), aa);         \
+    ab = fmaf(gb, dot16_fp8_x16<DT>(make_uint4(ub.x, ub.y, ub.z, ub.w), xa, xb), ab);         \
     if (++cb == bpr) {                                                                        \
       cb = 0;                                                                                 \
-      const float g = wave_sum(ag), u = wave_sum(au);                                         \
-      if (lane == 0) p.act[cu] = silu(g) * u; /* act is [slot][inter] = flat unit index */    \
-      ag = 0.0f;                                                                              \
-      au = 0.0f;                                                                              \
+      pol.finish(cu, wave_sum(aa), wave_sum(ab), lane);                                       \
+      aa = 0.0f;                                                                              \
+      ab = 0.0f;                                                                              \
       cu += wave_stride;                                                                      \
     }                                                                                         \
   } while (0)
 
-  // requests first, then x -> LDS, then the ring
-  if (total > 0) NV_GU_ISSUE(0);
-  if (total > 1) NV_GU_ISSUE(1);
-  if (total > 2) NV_GU_ISSUE(2);
-  if (total > 3) NV_GU_ISSUE(3);
-  for (uint32_t c = threadIdx.x * 8; c < p.hidden; c += kBlock * 8)  // 8 columns = one piece of one lane
-    *reinterpret_cast<uint4 *>(xs16 + lean_slot_16(c)) = *reinterpret_cast<const uint4 *>(p.x16 + c);
+  // Start: the activations are requested FIRST (up to kXHold 16-byte pieces a thread, in registers), the ring's
+  // first four batches right behind them, and the thread then waits for the activations alone - they are the
+  // oldest requests - and writes them to LDS while the weights are on their way. (Requested behind the ring,
+  // as a loop would, the activations arrive after 8 KiB of weights per wave, and the ring stands still until
+  // the barrier behind them.) Vectors with more pieces a thread take the loop.
+  constexpr uint32_t kXHold = 5;
+  const uint32_t pieces = cols / 8u;  // 8 columns = one piece of one lane
+  const uint32_t slots_x = bpr * 128u;  // pieces of the LDS copy (zeros behind a ragged end)
+  const uint32_t nx = (slots_x + blockDim.x - 1) / blockDim.x;
+  const bool x_first = nx <= kXHold && x_ahead;
+  lp_u32x4_t xh0, xh1, xh2, xh3, xh4;
+#define NV_LP_XREQ(I)                                                                              \
+  if (x_first && (I##u) < nx) {                                                                       \
+    const uint16_t *src_ = x16 + static_cast<uint64_t>(min(threadIdx.x + (I##u) * blockDim.x, pieces - 1u)) * 8u; \
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xh##I) : "v"(src_) : "memory");          \
+  }
+  NV_LP_XREQ(0)
+  NV_LP_XREQ(1)
+  NV_LP_XREQ(2)
+  NV_LP_XREQ(3)
+  NV_LP_XREQ(4)
+#undef NV_LP_XREQ
+  if (total > 0) NV_LP_ISSUE(0, false);
+  if (total > 1) NV_LP_ISSUE(1, false);
+  if (total > 2) NV_LP_ISSUE(2, false);
+  if (total > 3) NV_LP_ISSUE(3, false);
+  if (x_first) {
+    switch (min(total, 4u)) {  // four requests a batch stay in flight
+      case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+    asm volatile("" : "+v"(xh0), "+v"(xh1), "+v"(xh2), "+v"(xh3), "+v"(xh4));
+#define NV_LP_XPUT(I)                                                                              \
+  if ((I##u) < nx && threadIdx.x + (I##u) * blockDim.x < slots_x)                                 \
+    *reinterpret_cast<uint4 *>(xs16 + lean_slot_16((threadIdx.x + (I##u) * blockDim.x) * 8u)) =    \
+        threadIdx.x + (I##u) * blockDim.x < pieces ? make_uint4(xh##I.x, xh##I.y, xh##I.z, xh##I.w) \
+                                                   : make_uint4(0u, 0u, 0u, 0u);
+    NV_LP_XPUT(0)
+    NV_LP_XPUT(1)
+    NV_LP_XPUT(2)
+    NV_LP_XPUT(3)
+    NV_LP_XPUT(4)
+#undef NV_LP_XPUT
+  } else {
+    for (uint32_t c = threadIdx.x * 8; c < slots_x * 8u; c += blockDim.x * 8)
+      *reinterpret_cast<uint4 *>(xs16 + lean_slot_16(c)) =
+          c < cols ? *reinterpret_cast<const uint4 *>(x16 + c) : make_uint4(0u, 0u, 0u, 0u);
+  }
   __syncthreads();
-  for (uint32_t t = 0; t < total; t += 4) {
-    NV_GU_CONSUME(0);
-    if (t + 4 < total) NV_GU_ISSUE(0);
+  uint32_t t = 0;
+  for (; t + 8 <= total; t += 4) {  // steady state: three newer batches behind every use
+    NV_LP_AWAIT(0, 3u);
+    NV_LP_CONSUME();
+    NV_LP_ISSUE(0, true);
+    NV_LP_AWAIT(1, 3u);
+    NV_LP_CONSUME();
+    NV_LP_ISSUE(1, true);
+    NV_LP_AWAIT(2, 3u);
+    NV_LP_CONSUME();
+    NV_LP_ISSUE(2, true);
+    NV_LP_AWAIT(3, 3u);
+    NV_LP_CONSUME();
+    NV_LP_ISSUE(3, true);
+  }
+  // the last four to seven batches: batch b is used with the batches up to min(b + 3, total - 1) requested
+  for (; t < total; t += 4) {
+    NV_LP_AWAIT(0, total - 1u - t);
+    NV_LP_CONSUME();
+    if (t + 4 < total) NV_LP_ISSUE(0, true);
     if (t + 1 < total) {
-      NV_GU_CONSUME(1);
-      if (t + 5 < total) NV_GU_ISSUE(1);
+      NV_LP_AWAIT(1, total - 2u - t);
+      NV_LP_CONSUME();
+      if (t + 5 < total) NV_LP_ISSUE(1, true);
     }
     if (t + 2 < total) {
-      NV_GU_CONSUME(2);
-      if (t + 6 < total) NV_GU_ISSUE(2);
+      NV_LP_AWAIT(2, total - 3u - t);
+      NV_LP_CONSUME();
+      if (t + 6 < total) NV_LP_ISSUE(2, true);
     }
     if (t + 3 < total) {
-      NV_GU_CONSUME(3);
-      if (t + 7 < total) NV_GU_ISSUE(3);
+      NV_LP_AWAIT(3, total - 4u - t);
+      NV_LP_CONSUME();
+      if (t + 7 < total) NV_LP_ISSUE(3, true);
     }
   }
-#undef NV_GU_ISSUE
-#undef NV_GU_CONSUME
+#undef NV_LP_ISSUE
+#undef NV_LP_TAKE
+#undef NV_LP_AWAIT
+#undef NV_LP_CONSUME
+}
+
+// MoE gate/up: pair = (gate row i, up row i) of slot k's expert, unit = k * inter + i; act[unit] = silu(g) * u.
+struct MoeGateUpPairs {
+  const MoeFp8Params &p;
+  const uint32_t *table;  // LDS: expert of a slot (an id outside the bank reads expert 0)
+  uint32_t sc_cols;
+  uint64_t scale_stride, w_stride;
+  template <bool TABLE>
+  __device__ __forceinline__ void rows(uint32_t unit, const uint8_t *&wg, const uint8_t *&wu, const float *&sg,
+                                       const float *&su) const {
+    const uint32_t k = unit / p.inter, i = unit % p.inter;
+    uint32_t e;
+    if constexpr (TABLE) {
+      e = table[k];
+    } else {
+      // through the scalar path: a vector load here would be awaited together with every request in front of it
+      e = static_cast<uint32_t>(p.shared_index);
+      if (k < p.top_k)
+        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(p.expert_ids + k) : "memory");
+      if (e >= p.num_experts) e = 0;
+    }
+    const uint64_t row = e * w_stride + static_cast<uint64_t>(i) * p.hidden;
+    wg = p.w_gate + row;
+    wu = p.w_up + row;
+    const uint64_t srow = e * scale_stride + static_cast<uint64_t>(i / p.block) * sc_cols;
+    sg = p.s_gate + srow;
+    su = p.s_up + srow;
+  }
+  __device__ __forceinline__ void finish(uint32_t unit, float g, float u, int lane) const {
+    if (lane == 0) p.act[unit] = silu(g) * u;  // act is [slot][inter] = flat unit index
+  }
+};
+template <uint32_t DT>
+__global__ __launch_bounds__(kLeanPairMaxWaves * kWave, 5) void moe_gate_up_lean_kernel(MoeFp8Params p) {
+  extern __shared__ __align__(16) uint16_t xs16[];  // the 16-bit activations as they came, in lean order
+  __shared__ uint32_t sh_expert[kLeanMaxSlots];
+  const uint32_t slots = p.top_k + (p.shared_index >= 0 ? 1u : 0u);
+  if (threadIdx.x < slots) {
+    const uint32_t e = threadIdx.x < p.top_k ? p.expert_ids[threadIdx.x] : static_cast<uint32_t>(p.shared_index);
+    sh_expert[threadIdx.x] = e < p.num_experts ? e : 0u;
+  }
+  const uint32_t sc_cols = (p.hidden + p.block - 1) / p.block;
+  const MoeGateUpPairs pol{p, sh_expert, sc_cols, static_cast<uint64_t>((p.inter + p.block - 1) / p.block) * sc_cols,
+                           static_cast<uint64_t>(p.inter) * p.hidden};
+  lean_pair_stream<DT>(pol, p.x16, p.hidden, p.block, slots * p.inter, xs16, false);
+}
+
+// One FP8 GEMV, one token, 16-bit activations: pair = rows 2u and 2u + 1 (the last row doubles where the row
+// count is odd).
+struct GemvRowPairs {
+  const Fp8GemvParams &p;
+  uint32_t scale_cols;
+  template <bool TABLE>
+  __device__ __forceinline__ void rows(uint32_t unit, const uint8_t *&w0, const uint8_t *&w1, const float *&s0,
+                                       const float *&s1) const {
+    const uint32_t r0 = min(unit * 2u, p.rows - 1u), r1 = min(unit * 2u + 1u, p.rows - 1u);
+    w0 = p.w + static_cast<uint64_t>(r0) * p.cols;
+    w1 = p.w + static_cast<uint64_t>(r1) * p.cols;
+    s0 = p.scales + static_cast<uint64_t>(r0 / p.block_rows) * scale_cols;
+    s1 = p.scales + static_cast<uint64_t>(r1 / p.block_rows) * scale_cols;
+  }
+  __device__ __forceinline__ void finish(uint32_t unit, float a, float b, int lane) const {
+    if (lane == 0) {
+      p.out[unit * 2u] = a;
+      if (unit * 2u + 1u < p.rows) p.out[unit * 2u + 1u] = b;
+    }
+  }
+};
+template <uint32_t DT>
+__global__ __launch_bounds__(kLeanPairMaxWaves * kWave, 5) void fp8_gemv_lean_kernel(Fp8GemvParams p) {
+  extern __shared__ __align__(16) uint16_t xs16[];
+  const GemvRowPairs pol{p, (p.cols + p.block_cols - 1) / p.block_cols};
+  lean_pair_stream<DT>(pol, p.x16, p.cols, p.block_cols, (p.rows + 1u) / 2u, xs16, p.x_first != 0);
 }
 
 // Down + combine, lean. Four consumer waves each own output rows 2u and 2u+1 and walk (expert, chunk)
@@ -395,7 +569,7 @@ __global__ __launch_bounds__(kBlock, 5) void moe_gate_up_lean_kernel(MoeFp8Param
 // requests may stay in flight at each use instead of waiting for all of them.
 constexpr int kDownLeanMaxConsumers = 7;    // consumer waves of a workgroup (+ 1 staging wave: 512 threads at most)
 constexpr int kDownLeanMaxThreads = (kDownLeanMaxConsumers + 1) * kWave;
-constexpr uint32_t kDownLeanMaxSlots = 65;  // top_k <= 64 routed experts + the shared one
+constexpr uint32_t kDownLeanMaxSlots = kLeanMaxSlots;
 template <int P>
 __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(MoeFp8Params p) {
   static_assert(P == 1 || P == 2 || P == 4, "P must divide the ring of four");
@@ -499,7 +673,10 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
                : "memory")
 #define NV_DN_AWAIT(J, NEWER)                                                                 \
   do {                                                                                        \
-    if ((NEWER) >= 3u) NV_DN_TAKE("s_waitcnt vmcnt(12)", J);                                  \
+    const uint32_t newer_ = (NEWER);                                                          \
+    if (newer_ >= 3u) NV_DN_TAKE("s_waitcnt vmcnt(12)", J);                                   \
+    else if (newer_ == 2u) NV_DN_TAKE("s_waitcnt vmcnt(8)", J);                               \
+    else if (newer_ == 1u) NV_DN_TAKE("s_waitcnt vmcnt(4)", J);                               \
     else NV_DN_TAKE("s_waitcnt vmcnt(0)", J);                                                 \
   } while (0)
 #define NV_DN_U4(V) make_uint4((V).x, (V).y, (V).z, (V).w)
@@ -558,22 +735,25 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     NV_DN_CONSUME(3);
     NV_DN_ISSUE(3);
   }
-  for (; t < total; t += 4) {       // the last four to seven batches wait for everything requested
-    NV_DN_AWAIT(0, 0u);
+  // the last four to seven batches: batch b is used with the batches up to min(b + 3, total - 1) requested,
+  // so it may leave that many newer ones in flight (waiting for everything here put the round trips of the
+  // last two refills on the wave's path)
+  for (; t < total; t += 4) {
+    NV_DN_AWAIT(0, total - 1u - t);
     NV_DN_CONSUME(0);
     if (t + 4 < total) NV_DN_ISSUE(0);
     if (t + 1 < total) {
-      NV_DN_AWAIT(1, 0u);
+      NV_DN_AWAIT(1, total - 2u - t);
       NV_DN_CONSUME(1);
       if (t + 5 < total) NV_DN_ISSUE(1);
     }
     if (t + 2 < total) {
-      NV_DN_AWAIT(2, 0u);
+      NV_DN_AWAIT(2, total - 3u - t);
       NV_DN_CONSUME(2);
       if (t + 6 < total) NV_DN_ISSUE(2);
     }
     if (t + 3 < total) {
-      NV_DN_AWAIT(3, 0u);
+      NV_DN_AWAIT(3, total - 4u - t);
       NV_DN_CONSUME(3);
       if (t + 7 < total) NV_DN_ISSUE(3);
     }
@@ -657,6 +837,34 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 }  // namespace
 
+namespace {
+// Launch shape of lean_pair_stream: waves per workgroup and workgroups such that every workgroup is resident at
+// once (20 waves a CU at the kernels' register budget, LDS permitting) and the busiest CU holds as few pairs as
+// possible - 7168 rows are 14 pairs a CU, which two workgroups of seven waves hold exactly where workgroups of
+// four leave half the CUs with 16. Among equal loads the fewest pairs per wave (most requests in flight).
+struct LeanPairGrid {
+  uint32_t waves, blocks;
+};
+LeanPairGrid lean_pair_grid(uint32_t units, size_t lds_bytes) {
+  const uint32_t lds_fit = std::max<uint32_t>(1u, static_cast<uint32_t>((156u * 1024u) / (lds_bytes + 1024u)));
+  LeanPairGrid best{kWavesPerBlock, 256u * std::min<uint32_t>(5u, lds_fit)};  // (looping grid if nothing fits)
+  uint32_t best_load = ~0u;
+  const uint32_t ideal = (units + 255u) / 256u;
+  for (uint32_t per_wave = 1; per_wave <= 64u && best_load > ideal; ++per_wave) {
+    for (uint32_t c = kLeanPairMaxWaves; c >= 1; --c) {
+      const uint32_t wgs = (units + c * per_wave - 1) / (c * per_wave), per_cu = std::min(20u / c, lds_fit);
+      if (wgs > 256u * per_cu) continue;
+      const uint32_t load = (wgs + 255u) / 256u * c * per_wave;
+      if (load < best_load) {
+        best_load = load;
+        best = LeanPairGrid{c, wgs};
+      }
+    }
+  }
+  return best;
+}
+}  // namespace
+
 hipError_t launch_fp8_gemv(const Fp8GemvParams &p, hipStream_t stream) {
   if (p.w == nullptr || p.scales == nullptr || p.out == nullptr || (p.x16 == nullptr && p.xf == nullptr))
     return hipErrorInvalidValue;
@@ -666,10 +874,22 @@ hipError_t launch_fp8_gemv(const Fp8GemvParams &p, hipStream_t stream) {
   const bool fast = p.cols % 1024u == 0 && p.block_cols % 16u == 0 && aligned16(p.w);
   // 16-bit activations stay 16 bit in LDS on the chunked path (half the bytes, and K up to 30720)
   const bool x16_lean = fast && p.x16 != nullptr && aligned16(p.x16);
-  const size_t lds = static_cast<size_t>(p.cols) * (x16_lean ? sizeof(uint16_t) : sizeof(float));
+  // one token of 16-bit activations, rows of whole 16-byte pieces: row pairs through the hand-issued ring
+  const bool pair_lean = p.tokens == 1 && p.x16 != nullptr && aligned16(p.x16) && aligned16(p.w) &&
+                         p.cols % 16u == 0 && p.block_cols % 16u == 0 && p.cols >= kLeanPairMinCols;
+  const size_t lds = pair_lean ? static_cast<size_t>((p.cols + 1023u) / 1024u) * 1024u * sizeof(uint16_t)
+                               : static_cast<size_t>(p.cols) * (x16_lean ? sizeof(uint16_t) : sizeof(float));
   if (lds > 60 * 1024) return hipErrorInvalidValue;
   const bool bf = p.input_dtype == kBF16;
-  if (fast) {
+  if (pair_lean) {
+    const LeanPairGrid g = lean_pair_grid((p.rows + 1) / 2, lds);
+    Fp8GemvParams q = p;
+    // Activations requested ahead of the weights where the vector is long (measured: 16384 columns 21.7 ->
+    // 21.0 us, 7168 columns 22.2 -> 22.5 us)
+    q.x_first = p.cols >= 8192u ? 1u : 0u;
+    if (bf) hipLaunchKernelGGL(fp8_gemv_lean_kernel<kBF16>, dim3(g.blocks), dim3(g.waves * kWave), lds, stream, q);
+    else hipLaunchKernelGGL(fp8_gemv_lean_kernel<kF16>, dim3(g.blocks), dim3(g.waves * kWave), lds, stream, q);
+  } else if (fast) {
     // short rows: more rows per wave to keep the same number of bytes in flight
     const bool four = p.cols <= 2048u;
     const uint32_t units = four ? (p.rows + 3) / 4 : (p.rows + 1) / 2;
@@ -714,14 +934,16 @@ hipError_t launch_moe_fp8(const MoeFp8Params &p, hipStream_t stream) {
     const uint32_t blocks =
         static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 32u));
     const size_t lds = static_cast<size_t>(p.hidden) * sizeof(float);
-    if (fast_gu && aligned16(p.act) && aligned16(p.x16)) {
-      // lean kernel: oversubscribed persistent-style grid, 8 workgroups per CU at most
-      const uint32_t lean_blocks =
-          static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u));
+    if (fast_gu && aligned16(p.act) && aligned16(p.x16) && slots <= kLeanMaxSlots && units <= 0xffffffffull) {
+      // lean kernel: the activations stay 16 bit in LDS
+      const size_t lean_lds = static_cast<size_t>(p.hidden) * sizeof(uint16_t);
+      // (grid: more workgroups than fit at once, handed out as others finish - measured 1 us ahead of the
+      // all-resident balanced grid the single GEMV takes)
+      const LeanPairGrid g{kWavesPerBlock, static_cast<uint32_t>(std::min<uint64_t>((units + kWavesPerBlock - 1) / kWavesPerBlock, 256u * 8u))};
       if (p.input_dtype == kBF16)
-        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kBF16>), dim3(lean_blocks), dim3(kBlock), lds, stream, p);
+        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kBF16>), dim3(g.blocks), dim3(g.waves * kWave), lean_lds, stream, p);
       else
-        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kF16>), dim3(lean_blocks), dim3(kBlock), lds, stream, p);
+        hipLaunchKernelGGL((moe_gate_up_lean_kernel<kF16>), dim3(g.blocks), dim3(g.waves * kWave), lean_lds, stream, p);
     } else if (p.input_dtype == kBF16) {
       if (fast_gu) hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, true>), dim3(blocks), dim3(kBlock), lds, stream, p);
       else hipLaunchKernelGGL((moe_gate_up_kernel<kBF16, false>), dim3(blocks), dim3(kBlock), lds, stream, p);

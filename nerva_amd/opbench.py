@@ -184,10 +184,12 @@ def case_moe():
 
 def case_fp8_gemv():
     """One FP8 block-scaled GEMV at DeepSeek-V3's dense shapes (o projection 7168x16384, dense-layer gate
-    18432x7168): e4m3fn weights, 128x128 f32 scales, bf16 activations, f32 output."""
+    18432x7168, and the two low-rank expansions whose K is no multiple of 1024: q_b 24576x1536, kv_b 32768x512):
+    e4m3fn weights, 128x128 f32 scales, bf16 activations, f32 output."""
     lib = abi.load()
     blk = 128
-    for name, rows, cols, copies in (("o 7168x16384", 7168, 16384, 10), ("gate 18432x7168", 18432, 7168, 9)):
+    for name, rows, cols, copies in (("o 7168x16384", 7168, 16384, 10), ("gate 18432x7168", 18432, 7168, 9),
+                                     ("q_b 24576x1536", 24576, 1536, 30), ("kv_b 32768x512", 32768, 512, 64)):
         sr, sc = (rows + blk - 1) // blk, (cols + blk - 1) // blk
         w = DeviceBuffer(copies * rows * cols)
         s = DeviceBuffer(copies * sr * sc * 4)

@@ -299,9 +299,10 @@ def test_gemv_bias_and_invalid_arguments():
 # FP8 block-scaled GEMV
 # ---------------------------------------------------------------------------
 
-@pytest.mark.parametrize("cols", [1024, 3])
+@pytest.mark.parametrize("cols", [1024, 1040, 3])
 def test_fp8_decode_all_256_codes(cols):
-    """Every e4m3fn code through the device decode (hardware path at cols=1024, bit path at cols=3)."""
+    """Every e4m3fn code through the device decode (hardware path at cols=1024 and, with all but one lane of the
+    last chunk idle, at cols=1040; bit path at cols=3)."""
     w = np.zeros((256, cols), np.uint8)
     w[:, 0] = np.arange(256)
     x = np.zeros(cols, np.float32)
@@ -353,10 +354,13 @@ def test_fp8_gemm_tokens_ragged_kat(kat):
 
 
 @pytest.mark.parametrize("rows,cols,dtype", [(2048, 7168, BF16), (7168, 2048, BF16), (300, 1024, BF16),
-                                             (130, 260, BF16), (384, 16384, BF16), (515, 3072, F16)])
+                                             (130, 260, BF16), (384, 16384, BF16), (515, 3072, F16),
+                                             (515, 1536, BF16), (131, 5008, F16), (64, 528, BF16), (33, 272, BF16),
+                                             (66, 30720, BF16), (1027, 512, F16)])
 def test_fp8_gemv_matches_oracle(rows, cols, dtype):
-    """16-bit and f32 activations; K of 1024-multiples takes the chunked kernels (16-bit activations stay
-    16 bit in LDS there, which is what lets K = 16384 fit), other K the byte-wise one."""
+    """16-bit and f32 activations. One token of 16-bit activations over rows of whole 16-byte pieces takes the
+    row-pair kernel (a last chunk of fewer than 1024 columns has idle lanes; an odd row count doubles the last
+    row), f32 activations with K of 1024-multiples the chunked kernels, other K the byte-wise one."""
     w, s = O.synth_fp8_block(SEED, rows + cols, rows, cols, 128, 0.02)
     x16 = O.synth_16(dtype, SEED, 11, cols, 0.0, 1.0)
     ref = O.fp8_gemm_tokens(w, s, x16, rows, cols, 1, 128, 128, input_dtype=dtype)[0]
