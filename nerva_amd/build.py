@@ -30,13 +30,38 @@ def hipcc():
     return exe
 
 
+def _spilling_kernels(remarks):
+    """Kernels whose register allocation went to scratch memory, from hipcc's resource-usage remarks."""
+    bad, name = [], None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line and name is not None:
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if size != 0:
+                bad.append("%s (%d bytes a lane)" % (name, size))
+            name = None
+    return bad
+
+
+# Kernels that request their data with hand-written loads and wait for it with explicit counts. The compiler
+# does not know that such a register is still being written, so a spill (or any copy) of it reads garbage:
+# these kernels must compile without scratch memory, which every build checks.
+HAND_ISSUED_LOADS = ("attn_step_kernel", "moe_gate_up_lean_kernel", "moe_down_lean_kernel", "fp8_gemv_lean_kernel")
+
+
 def _compile(src):
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [hipcc()] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
-    log = "\n".join(l for l in (res.stdout + res.stderr).splitlines() if "packed-fp32-ops" not in l)
+    lines = (res.stdout + res.stderr).splitlines()
+    log = "\n".join(l for l in lines if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    bad = [k for k in _spilling_kernels("\n".join(l for l in lines if "kernel-resource-usage" in l))
+           if any(name in k for name in HAND_ISSUED_LOADS)]
+    if bad:
+        raise RuntimeError("%s: kernels that issue loads by hand must not spill registers:\n  %s" % (src, "\n  ".join(bad)))
     return obj, log
 
 

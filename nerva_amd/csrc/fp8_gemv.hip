@@ -370,6 +370,7 @@ __device__ __forceinline__ void lean_pair_stream(const Policy &pol, const uint16
 
   uint32_t cu = wave_global, cb = 0;
   float aa = 0.0f, ab = 0.0f;
+  bool pair_done = false;
 #define NV_LP_CONSUME()                                                                       \
   do {                                                                                        \
     const uint16_t *xp = xs16 + cb * 1024u + lane * 8;                                        \
@@ -381,7 +382,13 @@ __device__ __forceinline__ void lean_pair_stream(const Policy &pol, const uint16
     }                                                                                         \
     aa = fmaf(ga, dot16_fp8_x16<DT>(make_uint4(ua.x, ua.y, ua.z, ua.w), xa, xb), aa);         \
     ab = fmaf(gb, dot16_fp8_x16<DT>(make_uint4(ub.x, ub.y, ub.z, ub.w), xa, xb), ab);         \
-    if (++cb == bpr) {                                                                        \
+    pair_done = ++cb == bpr;                                                                  \
+  } while (0)
+  // a pair's reduction and store come BEHIND the refill of the ring slot that its last batch left (the wave
+  // issues in order: a reduction in front of the refill keeps the request back for its whole length)
+#define NV_LP_FINISH()                                                                        \
+  do {                                                                                        \
+    if (pair_done) {                                                                          \
       cb = 0;                                                                                 \
       pol.finish(cu, wave_sum(aa), wave_sum(ab), lane);                                       \
       aa = 0.0f;                                                                              \
@@ -447,41 +454,50 @@ __device__ __forceinline__ void lean_pair_stream(const Policy &pol, const uint16
     NV_LP_AWAIT(0, 3u);
     NV_LP_CONSUME();
     NV_LP_ISSUE(0, true);
+    NV_LP_FINISH();
     NV_LP_AWAIT(1, 3u);
     NV_LP_CONSUME();
     NV_LP_ISSUE(1, true);
+    NV_LP_FINISH();
     NV_LP_AWAIT(2, 3u);
     NV_LP_CONSUME();
     NV_LP_ISSUE(2, true);
+    NV_LP_FINISH();
     NV_LP_AWAIT(3, 3u);
     NV_LP_CONSUME();
     NV_LP_ISSUE(3, true);
+    NV_LP_FINISH();
   }
   // the last four to seven batches: batch b is used with the batches up to min(b + 3, total - 1) requested
   for (; t < total; t += 4) {
     NV_LP_AWAIT(0, total - 1u - t);
     NV_LP_CONSUME();
     if (t + 4 < total) NV_LP_ISSUE(0, true);
+    NV_LP_FINISH();
     if (t + 1 < total) {
       NV_LP_AWAIT(1, total - 2u - t);
       NV_LP_CONSUME();
       if (t + 5 < total) NV_LP_ISSUE(1, true);
+      NV_LP_FINISH();
     }
     if (t + 2 < total) {
       NV_LP_AWAIT(2, total - 3u - t);
       NV_LP_CONSUME();
       if (t + 6 < total) NV_LP_ISSUE(2, true);
+      NV_LP_FINISH();
     }
     if (t + 3 < total) {
       NV_LP_AWAIT(3, total - 4u - t);
       NV_LP_CONSUME();
       if (t + 7 < total) NV_LP_ISSUE(3, true);
+      NV_LP_FINISH();
     }
   }
 #undef NV_LP_ISSUE
 #undef NV_LP_TAKE
 #undef NV_LP_AWAIT
 #undef NV_LP_CONSUME
+#undef NV_LP_FINISH
 }
 
 // MoE gate/up: pair = (gate row i, up row i) of slot k's expert, unit = k * inter + i; act[unit] = silu(g) * u.
@@ -692,7 +708,12 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     const float *xp = acts + (ck & 1u) * inter + cb_ * 1024u + lane * 4;                      \
     a0 = fmaf(ga, dot16_fp8_lean(NV_DN_U4(ua), xp), a0);                                      \
     a1 = fmaf(gb, dot16_fp8_lean(NV_DN_U4(ub), xp), a1);                                      \
-    if constexpr (cb_ == P - 1) {                                                             \
+  } while (0)
+  // an expert's reduction comes BEHIND the refill of the ring slot its last batch left (the wave issues in
+  // order: a reduction in front of the refill keeps the request back for its whole length)
+#define NV_DN_FINISH(J)                                                                       \
+  do {                                                                                        \
+    if constexpr ((J) % P == P - 1) {                                                         \
       const float weight = sh_weight[ck];                                                     \
       t0 = fmaf(weight, wave_sum(a0), t0);                                                    \
       t1 = fmaf(weight, wave_sum(a1), t1);                                                    \
@@ -725,15 +746,19 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     NV_DN_AWAIT(0, 3u);
     NV_DN_CONSUME(0);
     NV_DN_ISSUE(0);
+    NV_DN_FINISH(0);
     NV_DN_AWAIT(1, 3u);
     NV_DN_CONSUME(1);
     NV_DN_ISSUE(1);
+    NV_DN_FINISH(1);
     NV_DN_AWAIT(2, 3u);
     NV_DN_CONSUME(2);
     NV_DN_ISSUE(2);
+    NV_DN_FINISH(2);
     NV_DN_AWAIT(3, 3u);
     NV_DN_CONSUME(3);
     NV_DN_ISSUE(3);
+    NV_DN_FINISH(3);
   }
   // the last four to seven batches: batch b is used with the batches up to min(b + 3, total - 1) requested,
   // so it may leave that many newer ones in flight (waiting for everything here put the round trips of the
@@ -742,20 +767,24 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
     NV_DN_AWAIT(0, total - 1u - t);
     NV_DN_CONSUME(0);
     if (t + 4 < total) NV_DN_ISSUE(0);
+    NV_DN_FINISH(0);
     if (t + 1 < total) {
       NV_DN_AWAIT(1, total - 2u - t);
       NV_DN_CONSUME(1);
       if (t + 5 < total) NV_DN_ISSUE(1);
+      NV_DN_FINISH(1);
     }
     if (t + 2 < total) {
       NV_DN_AWAIT(2, total - 3u - t);
       NV_DN_CONSUME(2);
       if (t + 6 < total) NV_DN_ISSUE(2);
+      NV_DN_FINISH(2);
     }
     if (t + 3 < total) {
       NV_DN_AWAIT(3, total - 4u - t);
       NV_DN_CONSUME(3);
       if (t + 7 < total) NV_DN_ISSUE(3);
+      NV_DN_FINISH(3);
     }
   }
 #undef NV_DN_AWAIT
@@ -763,6 +792,7 @@ __global__ __launch_bounds__(kDownLeanMaxThreads, 5) void moe_down_lean_kernel(M
 #undef NV_DN_U4
 #undef NV_DN_ISSUE
 #undef NV_DN_CONSUME
+#undef NV_DN_FINISH
   if (lane == 0) {
     if (unit * 2 < p.hidden) p.out[unit * 2] = t0;
     if (unit * 2 + 1 < p.hidden) p.out[unit * 2 + 1] = t1;
