@@ -96,7 +96,12 @@ def case_mlp():
     H, I = 4096, 12288
     copies = 4
     per = 3 * I * H
-    w = synth16(copies * per, 21)
+    # The [gate; up] matrix starts 1 KiB behind a 2 KiB boundary: a wave asks for 2 KiB of gate row i and 2 KiB of
+    # up row i at once, the two lie 96 MiB apart, and with both on 2 KiB boundaries the pair lands on the same
+    # memory channel (measured 33.0 us for the gate/up launch at a base of 0, 2 or 4 KiB, 31.5 us at 1 KiB; a
+    # session's arena does not put the matrix on such a boundary).
+    skew = 1024
+    w = synth16(copies * per + skew // 2, 21)
     gamma = synth16(H, 22, mean=1.0)
     h = synth32(H, 23)
     ff = DeviceBuffer(I * 2)
@@ -104,7 +109,7 @@ def case_mlp():
     nbytes = per * 2 + H * 2 + H * 2 + H * 2     # weights + gamma + h + out counted as 16-bit vectors
 
     def enqueue(i, n):
-        base = (i % n) * per * 2
+        base = skew + (i % n) * per * 2
         R.gemv(BF16, w.at(base), I, H, input_f32=h, gamma=gamma, eps=1e-6, out16=ff, epilogue=2, sync=False)
         R.gemv(BF16, w.at(base + 2 * I * H * 2), H, I, input16=ff, residual=h, out_f32=out, epilogue=1, sync=False)
     rows_out = {}
