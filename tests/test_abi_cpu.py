@@ -322,3 +322,35 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
     src = "".join(open(os.path.join(csrc, f)).read() for f in os.listdir(csrc) if f.endswith((".hip", ".cuh", ".hpp")))
     for knob in ("_SPLITS", "_ROW_TILES", "_K_WAVES", "_SLICES", "_MIN_TOKENS"):
         assert knob + '")' not in src, knob    # no getenv("NERVA_HIP_..._SPLITS") and the like
+
+
+def test_build_refuses_register_spills_in_kernels_that_issue_loads_by_hand():
+    """The build reads hipcc's resource-usage remarks: a kernel that requests data with inline-assembly loads
+    must not use scratch memory (a spilled register may still be receiving its data)."""
+    from nerva_amd import build
+    remarks = "\n".join([
+        "a.hip:1:1: remark: Function Name: _ZN2nv12_GLOBAL__N_120moe_down_lean_kernelILi2EEEvNS_12MoeFp8ParamsE [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:1:1: remark:     VGPRs: 96 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:1:1: remark:     ScratchSize [bytes/lane]: 128 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:2:1: remark: Function Name: _ZN2nv16gemv_fast_kernelILj1ELi1ELi4ELi1ELi4ELb0ELi16ELb0EEEvNS_10GemvParamsE [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:2:1: remark:     ScratchSize [bytes/lane]: 8 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:3:1: remark: Function Name: _ZN2nv12_GLOBAL__N_116attn_step_kernelILj1ELi4EEEvNS_10AttnParamsE [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:3:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]",
+    ])
+    spilling = build._spilling_kernels(remarks)
+    assert [s.split(" ")[0] for s in spilling] == [
+        "_ZN2nv12_GLOBAL__N_120moe_down_lean_kernelILi2EEEvNS_12MoeFp8ParamsE",
+        "_ZN2nv16gemv_fast_kernelILj1ELi1ELi4ELi1ELi4ELb0ELi16ELb0EEEvNS_10GemvParamsE"]
+    guarded = [s for s in spilling if any(name in s for name in build.HAND_ISSUED_LOADS)]
+    assert len(guarded) == 1 and "moe_down_lean_kernel" in guarded[0]
+    # every kernel with inline-assembly loads in the sources is on the list
+    import re
+    csrc = os.path.join(os.path.dirname(build.__file__), "csrc")
+    for name in os.listdir(csrc):
+        if not name.endswith((".hip", ".cuh")):
+            continue
+        text = open(os.path.join(csrc, name)).read()
+        if not re.search(r'asm volatile\(\s*"global_load_', text):
+            continue
+        kernels = re.findall(r"__global__[^;{]*?void (\w+)\(", text)
+        assert any(k in build.HAND_ISSUED_LOADS for k in kernels), name
