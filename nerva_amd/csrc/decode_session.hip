@@ -1498,9 +1498,12 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
                        lead->px, rope_freq, lead->prope, lead->head_dim / 2);
   err = hipGetLastError();
   out->pack_kernel_launches += 1;
+  // where the down projection's K slices are added by a launch of their own, that launch writes the RMSNorm that
+  // follows as well (the next layer's attention norm, or the final norm): one launch less per layer
+  const bool down_norms = gemm_rows_fuses_norm(kGemmResidual, H, I, T, tiles, lead->pgemm_ws_bytes);
   for (uint32_t l = 0; err == hipSuccess && l < lead->layers; ++l) {
     const LayerDev &w = lead->layer[l];
-    err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st, tiles);
+    if (l == 0 || !down_norms) err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st, tiles);
     GemmRowsParams g{};
     if (err == hipSuccess) {
       g.tokens = T;
@@ -1582,13 +1585,20 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.cols = I;
       g.workspace = lead->pgemm_ws;
       g.workspace_bytes = lead->pgemm_ws_bytes;
+      if (down_norms) {
+        g.norm_gamma = l + 1 < lead->layers ? lead->layer[l + 1].rms_attn : lead->final_norm;
+        g.norm_out16 = lead->pxn16;
+        g.norm_eps = lead->eps;
+        g.norm_packed_tiles = tiles;
+      }
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
-    out->pack_kernel_launches += 2;
+    out->pack_kernel_launches += down_norms && l != 0 ? 1 : 2;
     out->projection_kernel_launches += 4;
     out->dependency_kernel_launches += 1;
   }
-  if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st, tiles);
+  if (err == hipSuccess && !down_norms)
+    err = launch_rmsnorm_rows(lead->dtype, lead->px, lead->final_norm, lead->eps, T, H, lead->pxn16, st, tiles);
   if (err == hipSuccess) {
     GemmRowsParams g{};
     g.tokens = T;

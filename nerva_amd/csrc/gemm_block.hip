@@ -416,9 +416,14 @@ hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t ks
                      p, partials);
   hipError_t err = hipGetLastError();
   if (err == hipSuccess && kslices > 1) {
-    const uint32_t threads = p.rows / 4u * p.tokens;
-    hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
-                       static_cast<const float *>(partials), kslices, kBTokCap);
+    if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
+      hipLaunchKernelGGL((gemm_finish_norm_kernel<DT>), dim3(p.tokens), dim3(kFinNormThreads), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kBTokCap);
+    } else {
+      const uint32_t threads = p.rows / 4u * p.tokens;
+      hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kBTokCap);
+    }
     err = hipGetLastError();
   }
   return err;
@@ -748,9 +753,12 @@ uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t t
 }
 
 bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes) {
-  return epilogue == kGemmResidual && x_packed != 0 && rows % 4 == 0 &&
-         rows <= static_cast<uint32_t>(kFinNormThreads * kFinNormPerLane * 4) &&
-         gemm_wide_slices(epilogue, rows, cols, tokens, workspace_bytes) > 1;
+  if (epilogue != kGemmResidual || x_packed == 0 || rows % 4 != 0 ||
+      rows > static_cast<uint32_t>(kFinNormThreads * kFinNormPerLane * 4))
+    return false;
+  // wherever a launch of its own adds the K slices: the wide kernel's, or the shared-X kernel's for smaller blocks
+  if (tokens > kBTokCap) return gemm_wide_slices(epilogue, rows, cols, tokens, workspace_bytes) > 1;
+  return gemm_block_plan(epilogue, rows, cols, tokens, workspace_bytes).kslices > 1;
 }
 
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {
