@@ -407,7 +407,7 @@ __device__ __forceinline__ void lean_pair_stream(const Policy &pol, const uint16
   const uint32_t slots_x = bpr * 128u;  // pieces of the LDS copy (zeros behind a ragged end)
   const uint32_t nx = (slots_x + blockDim.x - 1) / blockDim.x;
   const bool x_first = nx <= kXHold && x_ahead;
-  lp_u32x4_t xh0, xh1, xh2, xh3, xh4;
+  lp_u32x4_t xh0 = {0u, 0u, 0u, 0u}, xh1 = xh0, xh2 = xh0, xh3 = xh0, xh4 = xh0;   // (a piece that is not requested is never stored)
 #define NV_LP_XREQ(I)                                                                              \
   if (x_first && (I##u) < nx) {                                                                       \
     const uint16_t *src_ = x16 + static_cast<uint64_t>(min(threadIdx.x + (I##u) * blockDim.x, pieces - 1u)) * 8u; \
