@@ -8,7 +8,10 @@
 // Mapping: one wave owns NR rows; a load instruction covers 64 lanes x 16 B =
 // 1024 columns; a lane's 16 weights share one block scale when block_cols is a
 // multiple of 16, so the scale multiplies a 16-term partial sum once.
-// x is kept in LDS as f32 (bf16/f16 inputs widen exactly).
+// Kernels, from general to lean: fp8_gemv_kernel / moe_gate_up_kernel / moe_down_kernel (any shape; several
+// tokens; f32 or 16-bit activations, kept in LDS as f32 or - K a multiple of 1024 - as they came), then
+// lean_pair_stream with its two users fp8_gemv_lean_kernel (one token, 16-bit activations, K a multiple of 16)
+// and moe_gate_up_lean_kernel, and moe_down_lean_kernel: hand-issued request rings with exact waits.
 #include "fp8_gemv.cuh"
 
 #include <algorithm>
