@@ -373,6 +373,24 @@ def test_fp8_gemv_matches_oracle(rows, cols, dtype):
         assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
 
 
+@pytest.mark.parametrize("rows,cols,block_rows,block_cols", [(96, 2064, 64, 48), (50, 528, 7, 16), (33, 4096, 128, 4096),
+                                                             (70, 1536, 3, 32), (258, 1024, 128, 64)])
+def test_fp8_gemv_block_shapes_other_than_128(rows, cols, block_rows, block_cols):
+    """Scale blocks of other shapes than 128 x 128 (rows per block arbitrary, columns per block a multiple of 16 so
+    that a lane's 16 weights share a scale): random codes without the NaN encodings, random positive scales."""
+    rng = np.random.default_rng(rows * 131 + cols)
+    w = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    w[(w & 0x7f) == 0x7f] = 0x38   # 0x7f / 0xff are NaN
+    w = (w & 0xbf).astype(np.uint8)  # exponent's top bit cleared: magnitudes up to 1.875, sums stay tame
+    sr, sc = -(-rows // block_rows), -(-cols // block_cols)
+    s = rng.uniform(0.5, 2.0, (sr, sc)).astype(np.float32)
+    x16 = O.synth_16(BF16, SEED, 12, cols, 0.0, 1.0)
+    ref = O.fp8_gemm_tokens(w, s, x16, rows, cols, 1, block_rows, block_cols, input_dtype=BF16)[0]
+    y = N.DeviceBuffer(rows * 4)
+    N.fp8_gemv(dev(w), dev(s), rows, cols, block_rows, block_cols, y, input16=dev(x16), input_dtype=BF16)
+    assert rel_l2(y.numpy(np.float32), ref) <= REL_L2
+
+
 # ---------------------------------------------------------------------------
 # Paged GQA decode attention
 # ---------------------------------------------------------------------------
