@@ -491,8 +491,9 @@ typedef struct NervaHipFp8GemvRequest {
 /* y[r] = sum_c (e4m3(W[r,c]) * S[r/br, c/bc]) * x[c], dequantised in f32 registers
  * (reference contract: crates/nerva-cuda/src/tests/deepseek_quant.rs:689-713).
  * The activation vector lives in one workgroup's LDS: cols <= 15360, or <= 30720 for a 16-byte
- * aligned input16 with cols a multiple of 1024, block_cols a multiple of 16 and 16-byte aligned
- * weights (the 16-bit values then stay 16 bit); beyond that the call fails with hipErrorInvalidValue. */
+ * aligned input16 with cols and block_cols multiples of 16 and 16-byte aligned weights (the 16-bit
+ * values then stay 16 bit, and the launch takes the lean row-pair kernel whatever cols modulo 1024);
+ * beyond that the call fails with hipErrorInvalidValue. */
 int nerva_hip_fp8_gemv(const NervaHipFp8GemvRequest *request, void *stream, int32_t *hip_error);
 
 typedef struct NervaHipPagedAttentionRequest {
