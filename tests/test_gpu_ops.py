@@ -356,7 +356,7 @@ def test_fp8_gemm_tokens_ragged_kat(kat):
 @pytest.mark.parametrize("rows,cols,dtype", [(2048, 7168, BF16), (7168, 2048, BF16), (300, 1024, BF16),
                                              (130, 260, BF16), (384, 16384, BF16), (515, 3072, F16),
                                              (515, 1536, BF16), (131, 5008, F16), (64, 528, BF16), (33, 272, BF16),
-                                             (66, 30720, BF16), (1027, 512, F16), (34, 20000, BF16)])
+                                             (66, 30720, BF16), (1027, 512, F16), (34, 20000, BF16), (1, 1024, BF16), (3, 272, F16)])
 def test_fp8_gemv_matches_oracle(rows, cols, dtype):
     """16-bit and f32 activations. One token of 16-bit activations over rows of whole 16-byte pieces takes the
     row-pair kernel (a last chunk of fewer than 1024 columns has idle lanes; an odd row count doubles the last
