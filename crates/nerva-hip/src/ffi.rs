@@ -619,6 +619,7 @@ pub struct NervaHipGemvRequest {
     pub epilogue: u32,
     pub round_output: u32,
     pub rms_eps: f32,
+    pub pair_gap: u32,
     pub weights: *const u16,
     pub input16: *const u16,
     pub input_f32: *const f32,

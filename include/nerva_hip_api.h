@@ -456,6 +456,8 @@ typedef struct NervaHipGemvRequest {
                                 3: out16 = round16(y) */
   uint32_t round_output;     /* epilogue 1: round the sum to 16 bits (prompt-token staging) */
   float rms_eps;
+  uint32_t pair_gap;         /* epilogue 2: elements left unused between the last gate row and the first up row
+                                (a multiple of 8; 0 = the up rows follow the gate rows directly) */
   const uint16_t *weights;
   const uint16_t *input16;   /* [cols] */
   const float *input_f32;    /* [cols] */

@@ -119,7 +119,8 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   const char *wbase[NR];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
-    wbase[j] = reinterpret_cast<const char *>(p.w) + (static_cast<uint64_t>(trow[j]) * cols + k0) * sizeof(uint16_t);
+    wbase[j] = reinterpret_cast<const char *>(p.w) +
+               (static_cast<uint64_t>(trow[j]) * cols + k0 + (EPI == kGemmSwiglu ? j * p.pair_gap : 0u)) * sizeof(uint16_t);
   const uint32_t wlane = (q * cols + n * 8u) * static_cast<uint32_t>(sizeof(uint16_t));
   uint16_t *park_at = wtile + q * kBRowStride + n * 8;
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
@@ -492,7 +493,8 @@ __global__ __launch_bounds__(PAIRS * 2 * kWave, 2) void gemm_wide_kernel(GemmRow
     trow[j] = EPI == kGemmSwiglu ? j * p.rows + blockIdx.x * (16u * kWPairs) + pair * 16u
                                  : blockIdx.x * (32u * kWPairs) + (pair * 2 + j) * 16u;
   // the tile this wave fetches: a wave-uniform base plus a per-lane offset that never changes
-  const char *wbase = reinterpret_cast<const char *>(p.w) + (static_cast<uint64_t>(trow[half]) * cols + k0) * sizeof(uint16_t);
+  const char *wbase = reinterpret_cast<const char *>(p.w) +
+                      (static_cast<uint64_t>(trow[half]) * cols + k0 + (EPI == kGemmSwiglu ? half * p.pair_gap : 0u)) * sizeof(uint16_t);
   const uint32_t wlane = (q * cols + n * 8u) * static_cast<uint32_t>(sizeof(uint16_t));
   uint16_t *park_at = wtile + half * kBWTile + q * kBRowStride + n * 8;
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;

@@ -46,6 +46,7 @@ struct GemmRowsParams {
   float *out_f32;            // kGemmF32 / kGemmResidual: [tokens][rows]
   uint16_t *out16;           // kGemmSwiglu: [tokens][rows] = round16(silu(gate) * up)
   uint32_t rows, cols, tokens;
+  uint32_t pair_gap;         // kGemmSwiglu: elements left unused between the last gate row and the first up row
   uint32_t round_out;        // kGemmResidual: round the sum to 16 bit
   uint32_t x_packed;         // != 0: x16 is in matrix-operand order (gemm_x_packed_index) instead of [tokens][cols];
                              // the value is its token-tile count and must be gemm_packed_tiles(tokens)

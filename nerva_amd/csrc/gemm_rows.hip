@@ -75,7 +75,8 @@ __global__ __launch_bounds__(kGThreads) void gemm_rows_kernel(GemmRowsParams p) 
   const uint16_t *wp[NR];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
-    wp[j] = p.w + static_cast<uint64_t>(row0 + j * tile_rows + (lane >> 5)) * cols + kbase + (lane & 31) * 8;
+    wp[j] = p.w + static_cast<uint64_t>(row0 + j * tile_rows + (lane >> 5)) * cols + kbase + (lane & 31) * 8 +
+            (EPI == kGemmSwiglu ? j * p.pair_gap : 0u);
   uint4 areg[NR][8];
 #define NV_GEMM_REQUEST(BLK)                                                                        \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 8; ++i)      \

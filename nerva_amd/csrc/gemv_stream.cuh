@@ -74,6 +74,7 @@ struct GemvParams {
   uint16_t *out16;
   uint32_t rows;   // output rows (kEpiSwiglu: pairs; W holds 2*rows rows, gate first)
   uint32_t cols;
+  uint32_t pair_gap;  // kEpiSwiglu: elements left unused between the last gate row and the first up row
   float eps;
   uint32_t round_out;
   const uint32_t *cursor;  // optional step guard: skip when *cursor >= max_steps
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvParams p) {
         row[k] = unit * NR + k;
         live[k] = row[k] < p.rows;
       }
-      wrow[k] = p.w + static_cast<uint64_t>(live[k] ? row[k] : 0u) * cols;
+      wrow[k] = p.w + static_cast<uint64_t>(live[k] ? row[k] : 0u) * cols + (EPI == kEpiSwiglu ? k * p.pair_gap : 0u);
     }
   };
 
@@ -412,13 +413,24 @@ constexpr int kFastMaxColsLoop = 30720;  // ... or, with a 16-bit input, copied 
 // WG: waves per workgroup (4 or 16). Every workgroup fetches the whole input vector (and for the RMSNorm
 // prologue the norm weights) for itself, so fewer, larger workgroups move that much less through the L2s ahead of
 // the weights; the waves' work is the same whatever the size (wave_global = workgroup x WG + wave).
+// ROT: a unit's walk over its columns starts at batch (unit mod batches per row) and wraps, so the waves of a
+// workgroup - and of the launch, which move through their rows at about the same pace - ask for different
+// column ranges at any one time instead of all for the same one. Rows are a multiple of the memory channels'
+// interleave apart, so without it the launch's requests of a moment land on a part of the channels. Measured
+// with the matrices on 2 KiB boundaries (a batch is then whole interleave units; the session's arena and
+// hipMalloc'ed buffers are): gate/up pair 32.8 -> 30.8 us (31.5 was the best the plain walk reached at any base),
+// qkv at two chunks a batch on 1024 workgroups 10.05 -> 9.65, LM head at one chunk a batch 183.6 -> 178.1; the
+// down and o launches do not move (a wave's two 4 KiB batches cover every phase already). The sum over a row
+// starts at another column, so results differ from the plain walk's in the last bits (each is deterministic).
 // XREG (4096 columns only): a lane's share of the input vector - the eight 16-byte pieces that meet its eight
 // weight pieces of a row - is read from LDS once, right after the prologue, and kept in registers, so the
 // products behind a batch's arrival do not wait for LDS reads (a wave gets one 1 KiB LDS read through every
 // ~30 cycles: eight of them a row were twice the time of the row's 32 dot instructions). Costs 32 registers:
 // one wave per SIMD less.
-template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false, int WG = kWavesPerBlock, bool XREG = false>
+template <uint32_t DT, int PRO, int EPI, int NR, int B, bool EXACT = false, int WG = kWavesPerBlock, bool XREG = false,
+          bool ROT = false>
 __global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) void gemv_fast_kernel(GemvParams p) {
+  static_assert(!(ROT && (XREG || EXACT)), "the rotated walk has no exact-start or register-input variant");
   constexpr int TB = WG * kWave;
   constexpr uint32_t kXregBpr = 8 / B;   // batches per 4096-column row
   extern __shared__ __align__(16) uint16_t xs[];
@@ -470,21 +482,30 @@ __global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) voi
 
   // ---- 2. weight request state + the first two batches
   uint32_t iu = EXACT ? min(wave_global, units - 1) : wave_global, ib = 0;  // next batch to request: unit, batch within the row
+  uint32_t ic = 0, cc = 0;            // ROT: column batch being requested / consumed (ic stays 0 otherwise)
+  constexpr uint32_t kBatchElems = B * kWave * 8;
   const uint16_t *wp[NR];
   uint4 buf0[NR][B], buf1[NR][B];
   float res0 = 0.0f, res1 = 0.0f;     // residual element requested with a row's first batch
 #define NV_FAST_ISSUE(DST, RES)                                                                   \
   do {                                                                                            \
     if (ib == 0) {                                                                                \
+      if constexpr (ROT) ic = iu % bpr;                                                           \
       _Pragma("unroll") for (int k = 0; k < NR; ++k)                                              \
-        wp[k] = p.w + static_cast<uint64_t>(iu + k * p.rows) * cols + lane * 8;                   \
+        wp[k] = p.w + static_cast<uint64_t>(iu + k * p.rows) * cols + k * p.pair_gap + ic * kBatchElems + lane * 8; \
       if constexpr (EPI == kEpiResidual) {                                                        \
         if (EXACT || lane == 0) RES = p.residual[iu];                                             \
       }                                                                                           \
     }                                                                                             \
     _Pragma("unroll") for (int u = 0; u < B; ++u)                                                 \
       _Pragma("unroll") for (int k = 0; k < NR; ++k) DST[k][u] = load_stream(wp[k] + u * (kWave * 8)); \
-    _Pragma("unroll") for (int k = 0; k < NR; ++k) wp[k] += B * (kWave * 8);                      \
+    _Pragma("unroll") for (int k = 0; k < NR; ++k) wp[k] += kBatchElems;                              \
+    if constexpr (ROT) {                                                                          \
+      if (++ic == bpr) {                                                                          \
+        ic = 0;                                                                                   \
+        _Pragma("unroll") for (int k = 0; k < NR; ++k) wp[k] -= cols;                             \
+      }                                                                                           \
+    }                                                                                             \
     if (++ib == bpr) {                                                                            \
       ib = 0;                                                                                     \
       iu += wave_stride;                                                                          \
@@ -580,8 +601,12 @@ __global__ __launch_bounds__(WG *kWave, XREG ? 4 : fast_waves_per_simd(PRO)) voi
     if (cb == 0) {                                                                                \
       _Pragma("unroll") for (int k = 0; k < NR; ++k) acc[k] = 0.0f;                               \
       res_cur = RES;                                                                              \
+      if constexpr (ROT) cc = cu % bpr;                                                           \
     }                                                                                             \
-    const uint32_t c0 = cb * (B * kWave * 8) + lane * 8;                                          \
+    const uint32_t c0 = (ROT ? cc : cb) * (B * kWave * 8) + lane * 8;                             \
+    if constexpr (ROT) {                                                                          \
+      if (++cc == bpr) cc = 0;                                                                    \
+    }                                                                                             \
     _Pragma("unroll") for (int u = 0; u < B; ++u) {                                               \
       uint4 xv;                                                                                   \
       if constexpr (XREG) xv = xr[cb * B + u]; /* cb is a constant at every use in this mode */   \
@@ -689,6 +714,8 @@ struct GemvPlan {
   uint32_t blocks;  // four-wave workgroups' worth of waves
   int wg_waves;     // waves per workgroup the launch uses (kFast: 4 or 16)
   uint32_t grid;    // workgroups launched: ceil(blocks * 4 / wg_waves)
+  bool rotated;     // kFast: the rotated walk (see gemv_fast_kernel)
+  int chunks;       // kFast: 1 KiB chunks per row and request batch
 };
 constexpr int kFast = 3;  // the lean production-shape kernel
 GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, bool vec16,

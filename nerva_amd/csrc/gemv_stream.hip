@@ -51,18 +51,18 @@ __global__ __launch_bounds__(1024) void sample_finish_kernel(SampleParams s, uin
 }
 
 template <uint32_t DT, int PRO, int EPI, int MODE>
-hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStream_t stream, int wg) {
+hipError_t launch_one(const GemvParams &p, const GemvPlan &plan, size_t lds, hipStream_t stream) {
   constexpr int NR = EPI == kEpiSwiglu ? 2 : kDefaultNR;  // swiglu: the gate row and the up row
+  const uint32_t blocks = plan.blocks;
+  const int wg = plan.wg_waves;
   if constexpr (MODE == kFast) {
-    // Launches whose waves own one or two rows of exactly two batches each (the step's o and qkv projections at
-    // 4096 columns) take the variant with exact start-up waits: o 7.5 -> 7.2 us, qkv 10.6 -> 10.25 us in the step.
+    // Launches whose waves own one or two rows of exactly two batches each (the step's o projection at
+    // 4096 columns) take the variant with exact start-up waits: o 7.5 -> 7.2 us in the step.
     // It needs two batches per row at least. Measured with it forced on elsewhere ("gemv_exact_start" override:
     // 1 = wherever it can run, 2 = nowhere): down (six batches a row) 17.1 -> 17.6 us; the gate/up pair and the
     // LM head do not move, so only the plain and residual epilogues have the variant.
     constexpr bool kShortShapes = EPI == kEpiF32 || EPI == kEpiResidual;
     constexpr uint32_t kBatchCols = kWave * 8u * (4 / NR);
-    // rows that are whole batches of 1024 columns but not of 2048 (hidden 5120, MLP width 25600): two chunks a batch
-    const bool half_batches = NR == 1 && p.cols % kBatchCols != 0;
     const uint32_t units_per_wave = (p.rows + blocks * kWavesPerBlock - 1) / (blocks * kWavesPerBlock);
     const int forced = tuning(kTuneGemvExactStart);
     const bool can = kShortShapes && p.cols >= 2u * kBatchCols;
@@ -73,60 +73,68 @@ hipError_t launch_one(const GemvParams &p, uint32_t blocks, size_t lds, hipStrea
     // 31.8 -> 33.5 us, LM head 187 -> 189 us (one wave per SIMD less) - so only the short launches with a
     // 16-bit input take it.
     const bool xreg = PRO == kProX16 && p.cols == 4096u && tuning(kTuneGemvXRegisters) != 2;
-#define NV_GEMV_LAUNCH(EX, W, XR)                                                                              \
-  hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 4 / NR, EX, W, XR>), dim3((waves + W - 1) / W),         \
+#define NV_GEMV_LAUNCH(BB, EX, W, XR, RT)                                                                      \
+  hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, BB, EX, W, XR, RT>), dim3((waves + W - 1) / W),        \
                      dim3(W * kWave), lds, stream, p)
-    if (half_batches) {
-      if (wg == 16)
-        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 2, false, 16, false>), dim3((waves + 15) / 16), dim3(16 * kWave), lds,
-                           stream, p);
-      else
-        hipLaunchKernelGGL((gemv_fast_kernel<DT, PRO, EPI, NR, 2, false, 4, false>), dim3((waves + 3) / 4), dim3(4 * kWave), lds,
-                           stream, p);
+    if (plan.rotated) {
+      // (which launches walk rotated, and with how many chunks a batch, is the plan's choice)
+      if constexpr (EPI == kEpiSwiglu) {
+        if (wg == 16) NV_GEMV_LAUNCH(2, false, 16, false, true);
+        else NV_GEMV_LAUNCH(2, false, 4, false, true);
+      } else if constexpr (PRO == kProRmsNorm && EPI == kEpiArgmax) {
+        NV_GEMV_LAUNCH(1, false, 16, false, true);
+      } else if constexpr (PRO == kProRmsNorm && EPI == kEpiF32) {
+        NV_GEMV_LAUNCH(2, false, 4, false, true);
+      } else {
+        return hipErrorInvalidValue;
+      }
+    } else if (plan.chunks == 2 && NR == 1) {
+      // rows that are whole batches of 1024 columns but not of 2048 (hidden 5120, MLP width 25600): two chunks a batch
+      if (wg == 16) NV_GEMV_LAUNCH(2, false, 16, false, false);
+      else NV_GEMV_LAUNCH(2, false, 4, false, false);
     } else if (can && want) {
       if constexpr (kShortShapes) {
-        if (wg == 16) NV_GEMV_LAUNCH(true, 16, false);
+        if (wg == 16) NV_GEMV_LAUNCH(4 / NR, true, 16, false, false);
         else if constexpr (PRO == kProX16) {
-          if (xreg) NV_GEMV_LAUNCH(true, 4, true);
-          else NV_GEMV_LAUNCH(true, 4, false);
-        } else NV_GEMV_LAUNCH(true, 4, false);
+          if (xreg) NV_GEMV_LAUNCH(4 / NR, true, 4, true, false);
+          else NV_GEMV_LAUNCH(4 / NR, true, 4, false, false);
+        } else NV_GEMV_LAUNCH(4 / NR, true, 4, false, false);
       }
     } else {
-      if (wg == 16) NV_GEMV_LAUNCH(false, 16, false);
-      else NV_GEMV_LAUNCH(false, 4, false);
+      if (wg == 16) NV_GEMV_LAUNCH(4 / NR, false, 16, false, false);
+      else NV_GEMV_LAUNCH(4 / NR, false, 4, false, false);
     }
 #undef NV_GEMV_LAUNCH
   } else if constexpr (MODE == kVecFull) {
     hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, kDefaultU / NR, kVecFull, kDefaultDot2>),
-                       dim3(blocks), dim3(kBlock), lds, stream, p);
+                       dim3(plan.blocks), dim3(kBlock), lds, stream, p);
   } else if constexpr (MODE == kVecGuarded) {
-    hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, 4, kVecGuarded, false>), dim3(blocks),
+    hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, 4, kVecGuarded, false>), dim3(plan.blocks),
                        dim3(kBlock), lds, stream, p);
   } else {
-    hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, 1, kScalar, false>), dim3(blocks),
+    hipLaunchKernelGGL((gemv_kernel<DT, PRO, EPI, NR, 1, kScalar, false>), dim3(plan.blocks),
                        dim3(kBlock), lds, stream, p);
   }
   return hipGetLastError();
 }
 
 template <uint32_t DT, int PRO, int MODE>
-hipError_t launch_epi(int epilogue, const GemvParams &p, uint32_t blocks, size_t lds,
-                      hipStream_t stream, int wg) {
+hipError_t launch_epi(int epilogue, const GemvParams &p, const GemvPlan &plan, size_t lds, hipStream_t stream) {
   switch (epilogue) {
-    case kEpiF32: return launch_one<DT, PRO, kEpiF32, MODE>(p, blocks, lds, stream, wg);
-    case kEpiResidual: return launch_one<DT, PRO, kEpiResidual, MODE>(p, blocks, lds, stream, wg);
-    case kEpiSwiglu: return launch_one<DT, PRO, kEpiSwiglu, MODE>(p, blocks, lds, stream, wg);
-    case kEpiOut16: return launch_one<DT, PRO, kEpiOut16, MODE>(p, blocks, lds, stream, wg);
-    case kEpiArgmax: return launch_one<DT, PRO, kEpiArgmax, MODE>(p, blocks, lds, stream, wg);
+    case kEpiF32: return launch_one<DT, PRO, kEpiF32, MODE>(p, plan, lds, stream);
+    case kEpiResidual: return launch_one<DT, PRO, kEpiResidual, MODE>(p, plan, lds, stream);
+    case kEpiSwiglu: return launch_one<DT, PRO, kEpiSwiglu, MODE>(p, plan, lds, stream);
+    case kEpiOut16: return launch_one<DT, PRO, kEpiOut16, MODE>(p, plan, lds, stream);
+    case kEpiArgmax: return launch_one<DT, PRO, kEpiArgmax, MODE>(p, plan, lds, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
 template <uint32_t DT, int MODE>
-hipError_t launch_pro(int prologue, int epilogue, const GemvParams &p, uint32_t blocks, size_t lds,
-                      hipStream_t stream, int wg) {
-  if (prologue == kProX16) return launch_epi<DT, kProX16, MODE>(epilogue, p, blocks, lds, stream, wg);
-  if (prologue == kProRmsNorm) return launch_epi<DT, kProRmsNorm, MODE>(epilogue, p, blocks, lds, stream, wg);
+hipError_t launch_pro(int prologue, int epilogue, const GemvParams &p, const GemvPlan &plan, size_t lds,
+                      hipStream_t stream) {
+  if (prologue == kProX16) return launch_epi<DT, kProX16, MODE>(epilogue, p, plan, lds, stream);
+  if (prologue == kProRmsNorm) return launch_epi<DT, kProRmsNorm, MODE>(epilogue, p, plan, lds, stream);
   return hipErrorInvalidValue;
 }
 
@@ -177,9 +185,30 @@ GemvPlan gemv_plan(int prologue, int epilogue, uint32_t rows, uint32_t cols, boo
   if (epilogue == kEpiArgmax && blocks > kSampleMaxBlocks) blocks = kSampleMaxBlocks;
   plan.blocks = blocks == 0 ? 1 : blocks;
   plan.wg_waves = kWavesPerBlock;
+  plan.rotated = false;
+  plan.chunks = epilogue == kEpiSwiglu ? 2 : 4;
   if (plan.mode == kFast) {
     plan.wg_waves = nv::tuning(kTuneGemvWorkgroupWaves);
     if (plan.wg_waves != 4 && plan.wg_waves != 16) plan.wg_waves = fast_workgroup_waves(prologue, epilogue, rows, cols);
+    if (epilogue != kEpiSwiglu && cols % (kWave * 8 * 4) != 0) plan.chunks = 2;
+    // The rotated walk (see the kernel), where it measured faster; "gemv_rotated_walk" = 2 keeps the plain walk.
+    const bool auto_grid = !(tuning && tuning->max_blocks > 0);
+    if (nv::tuning(kTuneGemvRotatedWalk) != 2) {
+      if (epilogue == kEpiSwiglu) {
+        plan.rotated = true;                                  // gate/up pair: 2 KiB of each row a batch
+      } else if (prologue == kProRmsNorm && epilogue == kEpiArgmax && plan.wg_waves == 16 && plan.chunks == 4) {
+        plan.rotated = true;                                  // LM head: 1 KiB a batch
+        plan.chunks = 1;
+      } else if (prologue == kProRmsNorm && epilogue == kEpiF32 && plan.wg_waves == 4 && cols == 4096u && auto_grid &&
+                 want > kCus * 4u && want <= kCus * 8u) {
+        // a step's qkv projection (6144 rows): 2 KiB a batch on four workgroups a CU - 10.05 -> 9.65 us; three a CU
+        // (every wave two rows) have too few requests in flight at this batch size, five leave a fifth of the waves
+        // with twice the work of the others
+        plan.rotated = true;
+        plan.chunks = 2;
+        plan.blocks = kCus * 4u;
+      }
+    }
   }
   plan.grid = (plan.blocks * kWavesPerBlock + plan.wg_waves - 1) / plan.wg_waves;
   return plan;
@@ -206,20 +235,18 @@ hipError_t launch_gemv(uint32_t dtype, int prologue, int epilogue, const GemvPar
   if (lds > 60 * 1024) return hipErrorInvalidValue;  // K up to 30720 fits one workgroup's LDS
   const GemvPlan plan = gemv_plan(prologue, epilogue, p.rows, p.cols, vec16, tuning);
   const int mode = plan.mode;
-  const uint32_t blocks = plan.blocks;
   // (the plan counts four-wave workgroups; the lean kernel may launch the same waves as fewer, larger ones)
-  const int wg = plan.wg_waves;
   if (blocks_used) *blocks_used = plan.grid;
   if (dtype == kBF16) {
-    if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, blocks, lds, stream, wg);
-    if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream, wg);
-    if (mode == kVecGuarded) return launch_pro<kBF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream, wg);
-    return launch_pro<kBF16, kScalar>(prologue, epilogue, p, blocks, lds, stream, wg);
+    if (mode == kFast) return launch_pro<kBF16, kFast>(prologue, epilogue, p, plan, lds, stream);
+    if (mode == kVecFull) return launch_pro<kBF16, kVecFull>(prologue, epilogue, p, plan, lds, stream);
+    if (mode == kVecGuarded) return launch_pro<kBF16, kVecGuarded>(prologue, epilogue, p, plan, lds, stream);
+    return launch_pro<kBF16, kScalar>(prologue, epilogue, p, plan, lds, stream);
   }
-  if (mode == kFast) return launch_pro<kF16, kFast>(prologue, epilogue, p, blocks, lds, stream, wg);
-  if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, blocks, lds, stream, wg);
-  if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, blocks, lds, stream, wg);
-  return launch_pro<kF16, kScalar>(prologue, epilogue, p, blocks, lds, stream, wg);
+  if (mode == kFast) return launch_pro<kF16, kFast>(prologue, epilogue, p, plan, lds, stream);
+  if (mode == kVecFull) return launch_pro<kF16, kVecFull>(prologue, epilogue, p, plan, lds, stream);
+  if (mode == kVecGuarded) return launch_pro<kF16, kVecGuarded>(prologue, epilogue, p, plan, lds, stream);
+  return launch_pro<kF16, kScalar>(prologue, epilogue, p, plan, lds, stream);
 }
 
 hipError_t launch_sample_finish(const SampleParams &s, uint32_t count, const uint32_t *cursor,

@@ -139,6 +139,7 @@ enum TuningKnob : int {
   kTuneGemvWorkgroupWaves,   // lean GEMV: waves per workgroup for every launch (4 or 16)
   kTuneGemvXRegisters,       // lean GEMV: 2 = never keep the input vector in registers
   kTunePrefillBlockTokens,   // prompt blocks of a session: 128 = never the 256-token blocks (read at session create)
+  kTuneGemvRotatedWalk,      // lean GEMV: 2 = never the rotated walk
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

@@ -31,7 +31,7 @@ constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_sp
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                                                   "moe_down_shared_first", "gemv_workgroup_waves",
-                                                  "gemv_x_registers",  "prefill_block_tokens"};
+                                                  "gemv_x_registers",  "prefill_block_tokens", "gemv_rotated_walk"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }
@@ -380,6 +380,8 @@ int nerva_hip_gemv(const NervaHipGemvRequest *r, void *stream, int32_t *hip_erro
   p.cols = r->cols;
   p.eps = r->rms_eps;
   p.round_out = r->round_output;
+  if (r->pair_gap != 0 && (r->epilogue != 2 || r->pair_gap % 8 != 0)) return finish(hipErrorInvalidValue, hip_error);
+  p.pair_gap = r->pair_gap;
   return finish(launch_gemv(r->dtype, static_cast<int>(r->prologue), static_cast<int>(r->epilogue), p,
                             resolve_stream(stream)),
                 hip_error);

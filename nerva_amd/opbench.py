@@ -93,28 +93,28 @@ def case_qproj():
 
 
 def case_mlp():
+    """Rows "rotating" / "resident": the matrices as the configuration states them, [gate; up] one row-major
+    [2 x 12288][4096] matrix. Row "rotating, session layout": the up rows 4 KiB behind the end of the gate rows,
+    which is how a session lays a layer's pair out (the gate/up launch is then indifferent to where in memory the
+    matrix starts: a wave streams gate row i and up row i side by side, and without the gap the two lie exactly
+    96 MiB apart)."""
     H, I = 4096, 12288
     copies = 4
-    per = 3 * I * H
-    # The [gate; up] matrix starts 1 KiB behind a 2 KiB boundary: a wave asks for 2 KiB of gate row i and 2 KiB of
-    # up row i at once, the two lie 96 MiB apart, and with both on 2 KiB boundaries the pair lands on the same
-    # memory channel (measured 33.0 us for the gate/up launch at a base of 0, 2 or 4 KiB, 31.5 us at 1 KiB; a
-    # session's arena does not put the matrix on such a boundary).
-    skew = 1024
-    w = synth16(copies * per + skew // 2, 21)
+    stride = 3 * I * H + (4 << 20)   # elements between copies: the matrices and 8 MiB, so every copy starts alike
+    w = synth16(copies * stride, 21)
     gamma = synth16(H, 22, mean=1.0)
     h = synth32(H, 23)
     ff = DeviceBuffer(I * 2)
     out = DeviceBuffer(H * 4)
-    nbytes = per * 2 + H * 2 + H * 2 + H * 2     # weights + gamma + h + out counted as 16-bit vectors
+    nbytes = 3 * I * H * 2 + H * 2 + H * 2 + H * 2     # weights + gamma + h + out counted as 16-bit vectors
 
-    def enqueue(i, n):
-        base = skew + (i % n) * per * 2
-        R.gemv(BF16, w.at(base), I, H, input_f32=h, gamma=gamma, eps=1e-6, out16=ff, epilogue=2, sync=False)
-        R.gemv(BF16, w.at(base + 2 * I * H * 2), H, I, input16=ff, residual=h, out_f32=out, epilogue=1, sync=False)
+    def enqueue(i, n, gap):
+        base = (i % n) * stride * 2
+        R.gemv(BF16, w.at(base), I, H, input_f32=h, gamma=gamma, eps=1e-6, out16=ff, epilogue=2, pair_gap=gap, sync=False)
+        R.gemv(BF16, w.at(base + (2 * I * H + gap) * 2), H, I, input16=ff, residual=h, out_f32=out, epilogue=1, sync=False)
     rows_out = {}
-    for variant, n in (("rotating", copies), ("resident", 1)):
-        ns = timed(lambda i: enqueue(i, n), 24)
+    for variant, n, gap in (("rotating", copies, 0), ("resident", 1, 0), ("rotating, session layout", copies, 2048)):
+        ns = timed(lambda i: enqueue(i, n, gap), 24)
         rows_out[variant] = report("2 MLP block 4096 -> 12288 -> 4096", variant, ns, nbytes)
     return rows_out
 

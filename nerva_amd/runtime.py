@@ -118,14 +118,16 @@ def _ptr(buf):
 
 
 def gemv(dtype, weights, rows, cols, *, input16=None, input_f32=None, gamma=None, eps=0.0, bias=None,
-         residual=None, out_f32=None, out16=None, epilogue=0, round_output=False, sync=True):
-    """Launch nerva_hip_gemv on device buffers. prologue is implied by which input is given."""
+         residual=None, out_f32=None, out16=None, epilogue=0, round_output=False, pair_gap=0, sync=True):
+    """Launch nerva_hip_gemv on device buffers. prologue is implied by which input is given.
+    pair_gap (epilogue 2): elements between the end of the gate rows and the first up row."""
     req = abi.NervaHipGemvRequest()
     req.dtype, req.rows, req.cols = dtype, rows, cols
     req.prologue = 0 if input16 is not None else 1
     req.epilogue = epilogue
     req.round_output = int(round_output)
     req.rms_eps = eps
+    req.pair_gap = pair_gap
     req.weights, req.input16, req.input_f32 = _ptr(weights), _ptr(input16), _ptr(input_f32)
     req.gamma, req.bias, req.residual = _ptr(gamma), _ptr(bias), _ptr(residual)
     req.output_f32, req.output16 = _ptr(out_f32), _ptr(out16)

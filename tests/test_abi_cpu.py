@@ -299,7 +299,8 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
     import nerva_amd as N
     # the decode step's launches at Qwen3-8B widths: every one the lean kernel
     assert N.gemv_launch_shape(1, 2, 12288, 4096) == (3, 2048)     # gate_up: oversubscribed long launch
-    assert N.gemv_launch_shape(1, 0, 6144, 4096) == (3, 768)       # qkv: two rows per wave in one round
+    assert N.gemv_launch_shape(1, 0, 6144, 4096) == (3, 1024)      # qkv: rotated walk, four workgroups a CU
+    assert N.gemv_launch_shape(1, 0, 8192, 8192) == (3, 1024)      # another width: two rows per wave in one round
     assert N.gemv_launch_shape(0, 1, 4096, 4096) == (3, 1024)      # o: every row on the machine at once
     assert N.gemv_launch_shape(1, 4, 151936, 4096) == (3, 512)     # LM head: 16-wave workgroups
     assert N.gemv_launch_shape(0, 0, 100, 520)[0] == 1             # 520 columns: the guarded vector kernel
@@ -313,7 +314,8 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
         N.gemv_launch_shape(0, 0, 0, 64)
     for name in ("attn_splits", "batch_splits", "prompt_splits", "gemm_row_tiles", "gemm_k_waves",
                  "gemm_block_slices", "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
-                 "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers", "prefill_block_tokens"):
+                 "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers", "prefill_block_tokens",
+                 "gemv_rotated_walk"):
         N.Device.set_tuning(name, 2)
         N.Device.set_tuning(name, 0)
     with pytest.raises(ValueError):
