@@ -796,6 +796,8 @@ unsafe extern "C" {
     pub fn nerva_hip_fp8_gemv(request: *const NervaHipFp8GemvRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_paged_gqa_decode(request: *const NervaHipPagedAttentionRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_paged_attention_workspace_bytes(heads: u32, head_dim: u32) -> u64;
+    pub fn nerva_hip_paged_attention_max_splits(kv_heads: u32) -> u64;
+    pub fn nerva_hip_paged_attention_status(workspace: *mut c_void, heads: u32, head_dim: u32, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_kv_cache_offset(block_count: u32, kv_heads: u32, head_dim: u32, layer: u32, physical_block: u32, kv_head: u32, token_in_block: u32, dim: u32, is_value: u32) -> u64;
     pub fn nerva_hip_argmax(request: *const NervaHipArgmaxRequest, stream: *mut c_void, hip_error: *mut i32) -> c_int;
     pub fn nerva_hip_argmax_workspace_bytes() -> u64;

@@ -33,6 +33,11 @@ extern "C" {
 #define NERVA_HIP_SLOT_REQUEST_ID 1u  /* types.cuh:34 */
 #define NERVA_HIP_SLOT_SEQUENCE_ID 1u /* types.cuh:35 */
 #define NERVA_HIP_SLOT_DEVICE_COMPLETE 1u /* types.cuh:36 */
+/* No counterpart in the reference: the slot of a token whose step a device-side bounded wait gave up on (the
+ * attention's split merge). The token is not valid; the call that reads the slot returns -1 with
+ * hip_error = NERVA_HIP_ERROR_STEP_FAULT, and the sequence has to be started again. */
+#define NERVA_HIP_SLOT_DEVICE_FAULT 2u
+#define NERVA_HIP_ERROR_STEP_FAULT 719 /* hipErrorLaunchFailure */
 #define NERVA_HIP_KV_BLOCK_TOKENS 16u /* types.cuh:64 */
 #define NERVA_HIP_ERROR_NO_DEVICE 100 /* native_stubs.rs:5-16 */
 #define NERVA_HIP_ERROR_NOT_SUPPORTED 801 /* hipErrorNotSupported */
@@ -512,7 +517,10 @@ typedef struct NervaHipPagedAttentionRequest {
   void *workspace;              /* nerva_hip_paged_attention_workspace_bytes() bytes, zero-initialised once */
   float *output_f32;            /* optional [heads*hd] */
   uint16_t *output16;           /* [heads*hd] rounded */
-  uint32_t splits;              /* 0: the library's split-KV factor; 1..64 (and <= block_count): this one (tests) */
+  uint32_t splits;              /* 0: the library's split-KV factor; 1..64: this one (tests). Refused with
+                                   hipErrorInvalidValue, and nothing launched, when it exceeds block_count or when
+                                   kv_heads * splits exceeds the device's compute units: the splits of a kv head
+                                   merge inside the launch and have to be resident together */
 } NervaHipPagedAttentionRequest;
 
 /* Fused per-head RMSNorm + RoPE + KV append + paged GQA split-KV decode attention
@@ -521,6 +529,15 @@ typedef struct NervaHipPagedAttentionRequest {
 int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *request, void *stream,
                                int32_t *hip_error);
 uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim);
+/* The largest split factor nerva_hip_paged_gqa_decode accepts for this many kv heads on the current device. */
+uint64_t nerva_hip_paged_attention_max_splits(uint32_t kv_heads);
+/* No counterpart in the reference (its attention reduces in a second launch and has no in-launch wait).
+ * Synchronises `stream` and reports whether a launch of nerva_hip_paged_gqa_decode on this workspace gave up
+ * waiting for a split's partial since the last call: 0 = none did; -1 with hip_error =
+ * NERVA_HIP_ERROR_STEP_FAULT = one did - its outputs are NaN - and the report is cleared, so that the
+ * workspace serves the next launch as if nothing had happened (partials are tagged per launch: what a late
+ * split still stores is never taken for a later launch's). */
+int nerva_hip_paged_attention_status(void *workspace, uint32_t heads, uint32_t head_dim, void *stream, int32_t *hip_error);
 /* Element offset of (layer, physical block, kv_head, token-in-block, dim) in the K (is_value 0)
  * or V (is_value 1) cache array. A (block, kv_head) tile of 16 tokens x head_dim elements is
  * contiguous; inside it the order is the library's own (matrix-core operand order at head_dim

@@ -87,10 +87,30 @@ struct AttnParams {
   const uint32_t *plan;
   // Decode step only: up to this many blocks in use, one split takes them all (attn_split_geometry). 0: never.
   uint32_t single_split_blocks;
+  // Decode step only, the splits' merge. A partial is valid for the launch whose tag it carries: the tag is made
+  // of the launch's sequence number on this workspace - the plan's step number, or `launch_seq` without a plan -
+  // and the layer, so a word that a late or earlier launch left behind can never be taken for this launch's.
+  uint32_t launch_seq;
+  // A merge gives up after this many polls of the words it waits for (0 = kAttnMergeSpinLimit), sets *fault
+  // (optional device word, never cleared by a kernel) and leaves NaN in the outputs it feeds.
+  uint32_t merge_spin_limit;
+  uint32_t *fault;
+  // Test hook: 1 + the index of a split that keeps its partial to itself (0 = none), so that the bounded wait of
+  // the merges that need it can be seen to end; every kernel still exits normally.
+  uint32_t withhold_split;
 };
+constexpr uint32_t kAttnMergeSpinLimit = 1u << 20;
+// Tag of the partials of launch `seq` (never 0, the cleared state): distinct for 2^23 consecutive steps of up
+// to 256 layers; the words are cleared after every merge and when a sequence starts as well.
+__host__ __device__ __forceinline__ uint32_t attn_launch_tag(uint32_t seq, uint32_t layer) {
+  return ((seq * 256u + (layer & 255u)) << 1) | 1u;
+}
+// The step kernel's merges need every active split of a kv head on the machine at once (a merging workgroup
+// holds its CU while it polls), one 8-wave workgroup per CU: the largest split factor a launch may use there.
+uint32_t attn_resident_splits(uint32_t kv_heads);
 
 // ---- per-step split plan of the decode attention ---------------------------------------------
-// words [0..7]: position, blocks, blocks per split, active splits, 4 spare;
+// words [0..7]: position, blocks, blocks per split, active splits, step number (the caller's), 3 spare;
 // then one 8-word entry per (split, wave): tiles of the wave, its first block, the physical blocks
 // of its first four tiles (clamped), 2 spare.
 constexpr uint32_t kAttnPlanHeader = 8, kAttnPlanEntry = 8, kAttnPlanWaves = 8;
@@ -111,7 +131,7 @@ __host__ __device__ __forceinline__ void attn_split_geometry(uint32_t pos, uint3
 }
 // One thread per (split, wave) entry (`entry` < splits * 8); entry 0 also writes the header.
 __device__ __forceinline__ void attn_plan_fill(uint32_t *plan, const uint32_t *table, uint32_t pos, uint32_t splits,
-                                               uint32_t single_blocks, uint32_t entry) {
+                                               uint32_t single_blocks, uint32_t entry, uint32_t step_number) {
   uint32_t nblk, bps, active;
   attn_split_geometry(pos, splits, single_blocks, nblk, bps, active);
   if (entry == 0) {
@@ -119,6 +139,7 @@ __device__ __forceinline__ void attn_plan_fill(uint32_t *plan, const uint32_t *t
     plan[1] = nblk;
     plan[2] = bps;
     plan[3] = active;
+    plan[4] = step_number;
   }
   const uint32_t split = entry / kAttnPlanWaves, wave = entry % kAttnPlanWaves;
   const uint32_t b0 = split * bps, b1 = min(nblk, b0 + bps), first = b0 + wave;
@@ -142,7 +163,7 @@ __host__ __device__ __forceinline__ uint64_t attn_out_token(const AttnParams &p,
 // stays within the 256 CUs (a second round of workgroups costs more than the shorter tile loops
 // save); within that, more splits mean fewer 16-token tiles per wave in a row.
 inline uint32_t attn_default_splits(uint32_t kv_heads, uint32_t block_count) {
-  uint32_t splits = 256 / (kv_heads == 0 ? 1 : kv_heads);
+  uint32_t splits = attn_resident_splits(kv_heads);
   if (splits > kAttnMaxSplits) splits = kAttnMaxSplits;
   if (splits > block_count) splits = block_count;
   return splits == 0 ? 1 : splits;

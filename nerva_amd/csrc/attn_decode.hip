@@ -153,12 +153,15 @@ constexpr uint32_t kStepRecord = kStepParts * kStepPartWords;
 // device-coherent cache lines per microsecond, which is why a head is spread over several merging
 // workgroups. Last of all every word that was read gets its tag cleared for the next launch (launches
 // are ordered by the stream). A wait that runs out (a split that never stored: cannot happen on a
-// healthy device) ends after kMergeSpinLimit polls and the outputs it feeds become NaN: a failure that
-// shows in the logits instead of a plausible wrong number.
-constexpr uint32_t kMergeSpinLimit = 1u << 20;
+// healthy device with every split resident, which the launcher sees to) ends after the launch's spin limit: the
+// fault word is set - the session hands it out with the token, the operator entry point through its status call -
+// and the outputs it feeds become NaN. A word counts only with this launch's tag, so a partial that lands after
+// its merge gave up is never taken for a later launch's.
 template <uint32_t DT, int G>
 __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t kvh, uint32_t g, uint32_t part, uint32_t S,
-                                                  uint32_t active, float *lds_o, float *lds_m, float *lds_l, bool first_part) {
+                                                  uint32_t active, float *lds_o, float *lds_m, float *lds_l, bool first_part,
+                                                  uint32_t tag) {
+  const uint32_t spin_limit = p.merge_spin_limit != 0 ? p.merge_spin_limit : kAttnMergeSpinLimit;
   constexpr uint32_t kGroups = 16, kPer = kAttnMaxSplits / kGroups;  // 4 splits per thread at most
   const uint32_t h = kvh * G + g;
   uint64_t *rec = p.part_tagged + static_cast<uint64_t>(h) * S * kStepRecord + part * kStepPartWords;
@@ -177,10 +180,12 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
     }
 #pragma unroll
     for (uint32_t i = 0; i < kPer; ++i)  // (a clamped repeat of the last split belongs to another thread: not awaited)
-      if (q + i * kGroups < active) ok = ok && tag_is(av[i], 1u) && tag_is(mv[i], 1u) && tag_is(lv[i], 1u);
-    if (__all(ok) || ++spins > kMergeSpinLimit) break;
+      if (q + i * kGroups < active) ok = ok && tag_is(av[i], tag) && tag_is(mv[i], tag) && tag_is(lv[i], tag);
+    if (__all(ok) || ++spins > spin_limit) break;
   }
-  const bool gave_up = spins > kMergeSpinLimit;  // per wave; poisons the outputs this wave contributes to
+  const bool gave_up = spins > spin_limit;  // per wave; poisons the outputs this wave contributes to
+  if (gave_up && p.fault != nullptr && (threadIdx.x & (kWave - 1)) == 0)
+    __hip_atomic_store(p.fault, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   float M = -INFINITY, L = 0.0f, o = 0.0f;
 #pragma unroll
   for (uint32_t i = 0; i < kPer; ++i)
@@ -349,12 +354,12 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   NV_AT_LD32(rb, rbp, 0);
 
   // ---- 2. position, this split's blocks, this wave's tiles (scalar path)
-  uint32_t pos, nblk, bps, active, first, nt, phys[4];
+  uint32_t pos, nblk, bps, active, first, nt, phys[4], launch_seq = p.launch_seq;
   if (p.plan != nullptr) {
     // this step's plan: everything above in one round trip
     u32x8_t head, mine;
     sload8x2(p.plan, p.plan + kAttnPlanHeader + (split * W + wave) * kAttnPlanEntry, head, mine);
-    pos = head[0], nblk = head[1], bps = head[2], active = head[3];
+    pos = head[0], nblk = head[1], bps = head[2], active = head[3], launch_seq = head[4];
     nt = mine[0], first = mine[1];
     phys[0] = mine[2], phys[1] = mine[3], phys[2] = mine[4], phys[3] = mine[5];
     if (pos >= p.max_steps) return;
@@ -375,6 +380,7 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   const uint32_t b1 = min(nblk, b0 + bps);
   const uint32_t new_block = pos / kKvBlockTokens, new_row = pos % kKvBlockTokens;
   const bool owns_new = p.append != 0 && new_block >= b0 && new_block < b1;
+  const uint32_t tag = attn_launch_tag(launch_seq, p.layer);
 
   // ---- 3. the wave's first tile. Only the first: at long contexts the launch is one burst of requests, the
   // memory path fills up, and a wave that goes on requesting sits in its request instructions until the burst
@@ -525,10 +531,12 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
       // flush, nobody waits for them to be performed).
       const uint32_t part = d / kStepPartDims, dl = d % kStepPartDims;
       uint64_t *rec = p.part_tagged + (static_cast<uint64_t>(h) * S + split) * kStepRecord + part * kStepPartWords;
-      store_tagged(rec + dl, o, 1u);
-      if (dl == 0) {
-        store_tagged(rec + kStepPartDims, M, 1u);
-        store_tagged(rec + kStepPartDims + 1, L, 1u);
+      if (p.withhold_split != split + 1u) {
+        store_tagged(rec + dl, o, tag);
+        if (dl == 0) {
+          store_tagged(rec + kStepPartDims, M, tag);
+          store_tagged(rec + kStepPartDims + 1, L, tag);
+        }
       }
     }
   }
@@ -540,7 +548,7 @@ __global__ __launch_bounds__(8 * kWave) void attn_step_kernel(AttnParams p) {
   // after the stores have been performed and a merge by the last arriver needed four.
   for (uint32_t j = split; j < G * kStepParts; j += active) {
     link_mark(trm, 16);
-    merge_part_tagged<DT, G>(p, kvh, j % G, j / G, S, active, sh.merge_o[0], sh.merge_m, sh.merge_l, j == split);
+    merge_part_tagged<DT, G>(p, kvh, j % G, j / G, S, active, sh.merge_o[0], sh.merge_m, sh.merge_l, j == split, tag);
     link_mark(trm, 17);
   }
 }
@@ -711,6 +719,9 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
       return hipGetLastError();
     }
     if (p.part_tagged == nullptr) return hipErrorInvalidValue;
+    // every active split of a kv head has to be resident while the merges poll: a larger split factor is refused
+    // here, never launched (callers size theirs with attn_default_splits)
+    if (p.splits > 1 && p.splits > attn_resident_splits(p.kv_heads)) return hipErrorInvalidValue;
     switch (group) {
       case 1: hipLaunchKernelGGL((attn_step_kernel<DT, 1>), grid, dim3(8 * kWave), 0, stream, p); break;
       case 2: hipLaunchKernelGGL((attn_step_kernel<DT, 2>), grid, dim3(8 * kWave), 0, stream, p); break;
@@ -726,6 +737,20 @@ hipError_t launch_dt(const AttnParams &p, hipStream_t stream) {
 }
 
 }  // namespace
+
+uint32_t attn_resident_splits(uint32_t kv_heads) {
+  static const uint32_t cus = [] {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) {
+      (void)hipGetLastError();
+      return 256u;   // no device to ask: the part this library is written for
+    }
+    return static_cast<uint32_t>(count);
+  }();
+  const uint32_t splits = cus / (kv_heads == 0 ? 1 : kv_heads);
+  return splits == 0 ? 1 : splits;
+}
 
 uint64_t attn_step_workspace_bytes(uint32_t heads) {
   return static_cast<uint64_t>(heads) * kAttnMaxSplits * kStepRecord * sizeof(uint64_t);

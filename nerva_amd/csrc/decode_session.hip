@@ -112,7 +112,8 @@ struct NervaHipHfDecodeSequenceSession {
   uint16_t *kc = nullptr, *vc = nullptr;
   uint32_t block_count = 0;
   uint32_t *table = nullptr, *prompt = nullptr;
-  uint32_t *state = nullptr;  // state[0] cursor, state[1] prompt count, state[2] steps executed so far
+  uint32_t *state = nullptr;  // state[0] cursor, state[1] prompt count, state[2] steps executed so far,
+                              // state[3] fault word (set by a kernel whose bounded wait gave up; cleared by start)
   Slot *slots = nullptr;
   float *x = nullptr, *r = nullptr, *qkv = nullptr, *logits = nullptr, *rope_freq = nullptr, *rope_cs = nullptr;
   uint16_t *attn16 = nullptr, *ff16 = nullptr;
@@ -184,9 +185,9 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const uint16_t *emb, cons
   // this step's split plan of the decode attention, once for all layers
   if (attn_plan != nullptr && blockIdx.x == 0)
     for (uint32_t e = threadIdx.x; e < attn_splits * kAttnPlanWaves; e += kBlock)
-      attn_plan_fill(attn_plan, table, pos, attn_splits, attn_single_blocks, e);
-  // steps executed so far: the epochs of in-launch hand-overs derive from it (nobody reads it
-  // in this launch)
+      attn_plan_fill(attn_plan, table, pos, attn_splits, attn_single_blocks, e, state[2] + 1u);  // (entry 0 = the thread that counts)
+  // steps executed so far: the tags of the attention's split partials derive from it (through the plan; nobody
+  // else reads it in this launch, and only the thread that writes it uses what it read above)
   if (blockIdx.x == 0 && threadIdx.x == 0) state[2] = state[2] + 1u;
   // this step's RoPE angles, once: cos at [i], sin at [half_dim + i] (f32 angle = pos / theta^(2i/d))
   if (rope_freq != nullptr && blockIdx.x == 0) {
@@ -245,10 +246,11 @@ __global__ __launch_bounds__(kBlock) void embed_batch_kernel(const uint16_t *emb
   for (uint32_t i = threadIdx.x; i < hidden; i += kBlock) x[static_cast<uint64_t>(t) * hidden + i] = dec16<DT>(row[i]);
 }
 
-__global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count) {
+__global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count, uint32_t clear_fault) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     state[0] = cursor;
     state[1] = prompt_count;
+    if (clear_fault) state[3] = 0u;
   }
 }
 
@@ -420,6 +422,9 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
       // embedding launch left the plan of that position)
       p.plan = s->attn_plan;
       p.part_tagged = s->attn_tagged;
+      p.fault = s->state + 3;
+      p.merge_spin_limit = static_cast<uint32_t>(std::max(tuning(kTuneAttnMergeSpinLimit), 0));
+      p.withhold_split = static_cast<uint32_t>(std::max(tuning(kTuneAttnWithholdSplit), 0));
       NV_STEP(kLAttn, launch_attn_decode(s->dtype, p, st));
       snap(s->attn16, static_cast<uint64_t>(A) * sizeof(uint16_t));
     }
@@ -491,6 +496,7 @@ hipError_t enqueue_step(Session *s, StepMode mode, StepProfiler *prof, int only 
   sample_bind_workspace(p.sample, s->sample_ws);
   p.sample.slots = s->slots;
   p.sample.cursor_rw = s->state;
+  p.sample.fault = s->state + 3;
   p.x16_dump = snap_slot(static_cast<uint64_t>(s->hidden) * sizeof(uint16_t));
   uint32_t head_blocks = 0;  // workgroups of the LM-head launch = candidates it leaves
   NV_STEP(kLHead, launch_gemv(s->dtype, kProRmsNorm, kEpiArgmax, p, st, nullptr, &head_blocks));
@@ -660,13 +666,21 @@ uint32_t observed_count(uint32_t steps, uint32_t has_eos, uint32_t eos, const Sl
   return count;
 }
 
+// Every field of a slot as the device publishes it (nerva_cuda_api.h:29-37, sampler.cu:394-407).
 bool slots_consistent(const Slot *slots, uint32_t count, uint32_t first_index) {
   for (uint32_t i = 0; i < count; ++i) {
     if (slots[i].request_id != NERVA_HIP_SLOT_REQUEST_ID || slots[i].sequence_id != NERVA_HIP_SLOT_SEQUENCE_ID ||
-        slots[i].completion != NERVA_HIP_SLOT_DEVICE_COMPLETE || slots[i].token_index != first_index + i)
+        slots[i].completion != NERVA_HIP_SLOT_DEVICE_COMPLETE || slots[i].token_index != first_index + i ||
+        slots[i].version != static_cast<uint64_t>(first_index + i) + 1u || slots[i].host_copied != 0)
       return false;
   }
   return true;
+}
+// A slot published by a step in which a device-side bounded wait gave up.
+bool slots_faulted(const Slot *slots, uint32_t count) {
+  for (uint32_t i = 0; i < count; ++i)
+    if (slots[i].completion == NERVA_HIP_SLOT_DEVICE_FAULT) return true;
+  return false;
 }
 
 hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t prompt_count,
@@ -680,7 +694,7 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
   if (err == hipSuccess)
     err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
   if (err == hipSuccess) {
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count);
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count, 1u);
     err = hipGetLastError();
   }
   out->h2d_bytes = static_cast<uint64_t>(prompt_count) * sizeof(uint32_t);
@@ -851,7 +865,7 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
     if (err == hipSuccess) out->kernel_launches += 1 + (rows_attention ? 9ull : 10ull) * s->layers;
   }
   if (err == hipSuccess) {
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, st, s->state, count, prompt_count);
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, st, s->state, count, prompt_count, 0u);
     err = hipGetLastError();
     out->kernel_launches += 1;
   }
@@ -996,7 +1010,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->attn_splits = attn_default_splits(s->kv_heads, block_count);
   s->attn_single_blocks = kAttnSingleSplitBlocks;
   if (const int want = tuning(kTuneAttnSplits); want >= 1 && want <= static_cast<int>(kAttnMaxSplits)) {
-    s->attn_splits = std::min<uint32_t>(static_cast<uint32_t>(want), block_count);
+    // (never more than stay resident together: the merges of the step kernel poll)
+    s->attn_splits = std::min({static_cast<uint32_t>(want), block_count, attn_resident_splits(s->kv_heads)});
     s->attn_single_blocks = 0;  // a forced factor holds at every context length
   }
 
@@ -1492,6 +1507,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     sample_bind_workspace(sp.out, q->sample_ws);
     sp.out.slots = q->slots;
     sp.out.cursor_rw = q->state;
+    sp.out.fault = q->state + 3;
     sp.cursor = q->state;
     sp.max_steps = q->max_ctx;
     min_blocks = std::min(min_blocks, q->block_count);
@@ -1844,12 +1860,18 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
         out->projection_elapsed_ns = std::max<uint64_t>(1, static_cast<uint64_t>(static_cast<double>(ms) * 1e6));
     }
   } else if (err == hipSuccess) {
-    // shapes outside the multi-row kernels: every sequence runs its own captured step on its own stream
+    // shapes outside the multi-row kernels: every sequence runs its own captured step on its own stream - one
+    // after the other (each stream waits for the step before it): a step's attention launch wants every CU for
+    // workgroups that poll for each other, and two such launches side by side could hold each other's CUs
     NervaHipHfDecodeSequenceResult scratch{};
+    Session *before = nullptr;
     for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
       Session *q = seqs[t];
       err = ensure_graph(q, decode_graph(q), &scratch);
+      if (err == hipSuccess && before != nullptr) err = hipStreamWaitEvent(q->stream, before->ev1, 0);
       if (err == hipSuccess) err = launch_step(q, decode_graph(q), &scratch);
+      if (err == hipSuccess) err = hipEventRecord(q->ev1, q->stream);
+      before = q;
       if (err == hipSuccess)
         err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
                              q->stream);
@@ -1876,6 +1898,7 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
     const uint32_t at = q->cursor;  // = prompt_count - 1 + observed
     const Slot &slot = q->host_slots[at];
     if (!slots_consistent(&slot, 1, at)) {
+      if (slots_faulted(&slot, 1)) out->hip_error = NERVA_HIP_ERROR_STEP_FAULT;
       out->status = -1;
       return -1;
     }
@@ -2052,6 +2075,13 @@ int nerva_hip_hf_decode_sequence_session_advance(const NervaHipHfDecodeSequenceS
   out->pinned_host_bytes = static_cast<uint64_t>(s->max_ctx) * sizeof(Slot);
   out->host_causality_edges = 0;
   out->status = out->observed_tokens > 0 && slots_consistent(observed, out->observed_tokens, slot_start) ? 0 : -1;
+  if (slots_faulted(observed, request->steps)) {
+    // a device-side bounded wait gave up in one of these steps: its token and everything after it is void, and
+    // the sequence ends here (start() clears the fault)
+    out->status = -1;
+    out->hip_error = NERVA_HIP_ERROR_STEP_FAULT;
+    s->finished = true;
+  }
   if (out->status == 0) {
     s->observed += out->observed_tokens;
     s->cursor = out->observed_tokens < request->steps ? s->max_ctx : target;
@@ -2118,6 +2148,10 @@ int nerva_hip_hf_decode_sequence_session_run(const NervaHipHfDecodeSequenceSessi
   out->pinned_host_bytes = static_cast<uint64_t>(s->max_ctx) * sizeof(Slot);
   out->host_causality_edges = 0;
   out->status = out->observed_tokens > 0 && slots_consistent(observed, out->observed_tokens, output_start) ? 0 : -1;
+  if (slots_faulted(observed, request->steps)) {
+    out->status = -1;
+    out->hip_error = NERVA_HIP_ERROR_STEP_FAULT;
+  }
   return out->status == 0 ? 0 : -1;
 }
 

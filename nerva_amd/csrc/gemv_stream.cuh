@@ -42,6 +42,7 @@ struct SampleParams {
   NervaHipSyntheticTokenSlot *slots;  // optional: publish slot[pos] and bump the cursor
   uint32_t *cursor_rw;
   uint32_t *token_out;     // optional: plain token output (operator entry point)
+  const uint32_t *fault;   // optional: a word that a kernel of this step sets when a bounded wait of its gave up
 };
 
 // One lane: hands the step's token out - plain output word and/or slot[pos] in the reference's
@@ -56,7 +57,8 @@ __device__ __forceinline__ void publish_token(const SampleParams &s, uint32_t to
     slot.token_index = pos;
     slot.token = token;
     slot.version = static_cast<uint64_t>(pos) + 1u;
-    slot.completion = NERVA_HIP_SLOT_DEVICE_COMPLETE;
+    // a step that gave up somewhere says so in the slot it publishes: the host hands the error out with the token
+    slot.completion = s.fault != nullptr && *s.fault != 0u ? NERVA_HIP_SLOT_DEVICE_FAULT : NERVA_HIP_SLOT_DEVICE_COMPLETE;
     slot.host_copied = 0;
     s.slots[pos] = slot;
     *s.cursor_rw = pos + 1u;

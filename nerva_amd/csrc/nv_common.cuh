@@ -140,6 +140,8 @@ enum TuningKnob : int {
   kTuneGemvXRegisters,       // lean GEMV: 2 = never keep the input vector in registers
   kTunePrefillBlockTokens,   // prompt blocks of a session: 128 = never the 256-token blocks (read at session create)
   kTuneGemvRotatedWalk,      // lean GEMV: 2 = never the rotated walk
+  kTuneAttnMergeSpinLimit,   // decode attention: polls after which a split merge gives up (tests of the error path)
+  kTuneAttnWithholdSplit,    // decode attention: 1 + a split that keeps its partial to itself (tests of the error path)
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

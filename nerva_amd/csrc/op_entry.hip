@@ -31,7 +31,8 @@ constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_sp
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                                                   "moe_down_shared_first", "gemv_workgroup_waves",
-                                                  "gemv_x_registers",  "prefill_block_tokens", "gemv_rotated_walk"};
+                                                  "gemv_x_registers",  "prefill_block_tokens", "gemv_rotated_walk",
+                                                  "attn_merge_spin_limit", "attn_withhold_split"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }
@@ -405,10 +406,37 @@ int nerva_hip_fp8_gemv(const NervaHipFp8GemvRequest *r, void *stream, int32_t *h
   return finish(launch_fp8_gemv(p, resolve_stream(stream)), hip_error);
 }
 
-uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim) {
-  // split workspace, RoPE frequency table (256-byte slot), tagged partials of the decode step kernel
+namespace {
+// split workspace, RoPE frequency table (256-byte slot), tagged partials of the decode step kernel, fault word
+uint64_t paged_attention_fault_offset(uint32_t heads, uint32_t head_dim) {
   return attn_workspace_bytes(heads, head_dim) + ((static_cast<uint64_t>(head_dim) * sizeof(float) + 255u) & ~uint64_t{255}) +
          attn_step_workspace_bytes(heads);
+}
+std::atomic<uint32_t> g_attention_calls{0};   // the launch sequence number that tags a call's split partials
+}  // namespace
+
+uint64_t nerva_hip_paged_attention_workspace_bytes(uint32_t heads, uint32_t head_dim) {
+  return paged_attention_fault_offset(heads, head_dim) + 256;
+}
+
+uint64_t nerva_hip_paged_attention_max_splits(uint32_t kv_heads) {
+  return std::min<uint32_t>(attn_resident_splits(kv_heads), kAttnMaxSplits);
+}
+
+int nerva_hip_paged_attention_status(void *workspace, uint32_t heads, uint32_t head_dim, void *stream, int32_t *hip_error) {
+  if (hip_error) *hip_error = 0;
+  if (workspace == nullptr || heads == 0 || head_dim == 0) return finish(hipErrorInvalidValue, hip_error);
+  hipStream_t s = resolve_stream(stream);
+  hipError_t err = hipStreamSynchronize(s);
+  if (err != hipSuccess) return finish(err, hip_error);
+  uint32_t *word = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + paged_attention_fault_offset(heads, head_dim));
+  uint32_t fault = 0;
+  err = hipMemcpy(&fault, word, sizeof(fault), hipMemcpyDeviceToHost);
+  if (err != hipSuccess) return finish(err, hip_error);
+  if (fault == 0) return 0;
+  (void)hipMemset(word, 0, sizeof(fault));
+  if (hip_error) *hip_error = NERVA_HIP_ERROR_STEP_FAULT;
+  return -1;
 }
 
 uint64_t nerva_hip_kv_cache_offset(uint32_t block_count, uint32_t kv_heads, uint32_t head_dim,
@@ -475,6 +503,10 @@ int nerva_hip_paged_gqa_decode(const NervaHipPagedAttentionRequest *r, void *str
   p.position = r->position;
   p.max_steps = 0;
   p.append = r->append;
+  p.launch_seq = g_attention_calls.fetch_add(1, std::memory_order_relaxed) + 1u;
+  p.fault = reinterpret_cast<uint32_t *>(static_cast<char *>(r->workspace) + paged_attention_fault_offset(r->heads, r->head_dim));
+  p.merge_spin_limit = static_cast<uint32_t>(std::max(tuning(kTuneAttnMergeSpinLimit), 0));
+  p.withhold_split = static_cast<uint32_t>(std::max(tuning(kTuneAttnWithholdSplit), 0));
   return finish(launch_attn_decode(r->dtype, p, s), hip_error);
 }
 

@@ -248,6 +248,14 @@ def attention_workspace(heads, head_dim):
     return DeviceBuffer.zeros(abi.load().nerva_hip_paged_attention_workspace_bytes(heads, head_dim))
 
 
+def paged_attention_status(workspace, heads, head_dim):
+    """(rc, hip_error) of nerva_hip_paged_attention_status: synchronises, then (0, 0), or (-1, NERVA_HIP_ERROR_STEP_FAULT)
+    when a launch on this workspace gave up waiting for a split's partial (the report is cleared by the call)."""
+    err = C.c_int32(0)
+    rc = abi.load().nerva_hip_paged_attention_status(_ptr(workspace), heads, head_dim, None, C.byref(err))
+    return rc, int(err.value)
+
+
 def argmax(logits_buf, count, workspace=None):
     lib = abi.load()
     ws = workspace or DeviceBuffer.zeros(lib.nerva_hip_argmax_workspace_bytes())

@@ -492,9 +492,10 @@ def test_paged_attention_other_geometries(heads, kv_heads, hd, dtype, theta, qk_
 @pytest.mark.parametrize("heads,kv_heads", [(64, 8), (32, 4), (16, 16)])
 def test_paged_attention_step_kernel_group_sizes_at_long_context(heads, kv_heads):
     """GQA factors 8 and 1 and a 4-kv-head layout (64 splits) through the decode-step kernel at contexts where the
-    splits merge (and, with few forced splits, where a wave re-requests tiles): oracle parity, same bits on a
-    second launch."""
-    for tokens, splits in ((333, 0), (1000, 0), (4096, 0), (4096, 3), (2500, 64 if kv_heads <= 4 else 32)):
+    splits merge (and, with few forced splits, where a wave re-requests tiles), up to the largest split factor that
+    stays resident for the kv head count: oracle parity, same bits on a second launch."""
+    most = int(N.abi.load().nerva_hip_paged_attention_max_splits(kv_heads))
+    for tokens, splits in ((333, 0), (1000, 0), (4096, 0), (4096, 3), (2500, most)):
         c = _attention_case(BF16, heads, kv_heads, 128, tokens, 1e6, True, heads + tokens)
         ref, _, _ = _attention_oracle(c)
         cache = N.PagedKvCache(c["layers"], c["n_blocks"], kv_heads, 128, c["table"])
@@ -527,10 +528,11 @@ def test_paged_attention_permutation_invariance_and_repeatability():
 
 @pytest.mark.parametrize("tokens", [17, 255, 4096, 8191])
 def test_paged_attention_split_merge_is_stable_over_many_launches(tokens):
-    """The cross-split merge (partials written by every split's workgroup, one ticket per workgroup,
-    the last arriver of a kv head merges in split order) must not depend on arrival order or timing:
-    for split factors 2, 8, 32 and 64, 200 launches in a row give the bits of the first launch, and
-    those are within tolerance of the oracle. Stops at the first mismatch."""
+    """The cross-split merge (every split stores its partial as tagged words; the merge jobs of a kv head are
+    spread over its first splits' workgroups, which poll the words and fold them in split order) must not depend
+    on arrival order or timing: for split factors 2, 8 and 32 (the most that stay resident together with 8 kv
+    heads), 200 launches in a row give the bits of the first launch, and those are within tolerance of the
+    oracle. Stops at the first mismatch."""
     c = _attention_case(BF16, 32, 8, 128, tokens, 1e6, True, 5000 + tokens)
     ref, _, _ = _attention_oracle(c)
     cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
@@ -539,7 +541,7 @@ def test_paged_attention_split_merge_is_stable_over_many_launches(tokens):
     out16, out32 = N.DeviceBuffer(4096 * 2), N.DeviceBuffer(4096 * 4)
     qkv, qn, kn = dev(c["qkv"]), dev(c["qn"]), dev(c["kn"])
     outs = {}
-    for splits in (2, 8, 32, 64):
+    for splits in (2, 8, 32):
         if splits > c["n_blocks"]:
             continue
         first = None
@@ -565,6 +567,57 @@ def test_paged_attention_split_override_is_validated():
     for bad in (65, c["n_blocks"] + 1):
         with pytest.raises(RuntimeError):
             N.paged_attention(BF16, 32, 8, 128, cache, 0, 40, dev(c["qkv"]), ws, out16, splits=bad)
+
+
+def test_paged_attention_refuses_split_factors_that_cannot_be_resident_together():
+    """The merges of a kv head's splits poll inside the launch, so kv_heads x splits workgroups have to fit the
+    machine at once (one per compute unit): a larger factor is refused on the host and nothing is launched."""
+    c = _attention_case(BF16, 64, 8, 128, 2500, 1e6, True, 77)
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
+    ws = attention_workspace(64, 128)
+    out16 = N.DeviceBuffer(64 * 128 * 2)
+    out16.upload(np.full(64 * 128, 0x7fc1, np.uint16))
+    most = N.abi.load().nerva_hip_paged_attention_max_splits(8)
+    assert 1 <= most < 64
+    with pytest.raises(RuntimeError):
+        N.paged_attention(BF16, 64, 8, 128, cache, 0, 2500, dev(c["qkv"]), ws, out16, splits=most + 1)
+    assert np.all(out16.numpy(np.uint16, 64 * 128) == 0x7fc1)          # nothing ran
+    N.paged_attention(BF16, 64, 8, 128, cache, 0, 2500, dev(c["qkv"]), ws, out16, splits=most)
+    assert N.paged_attention_status(ws, 64, 128) == (0, 0)
+
+
+def test_paged_attention_merge_that_gives_up_is_an_error_and_leaves_the_workspace_usable():
+    """A split that never hands its partial over (forced by a test hook; its workgroup exits normally) makes the
+    merges that wait for it give up after their spin limit (set to a few polls here): the outputs they feed are
+    NaN, the status call returns -1 with the step-fault error, and the next launch on the same workspace - whose
+    partials carry another tag - is correct again."""
+    c = _attention_case(BF16, 32, 8, 128, 4096, 1e6, True, 4242)
+    ref, _, _ = _attention_oracle(c)
+    cache = N.PagedKvCache(c["layers"], c["n_blocks"], 8, 128, c["table"])
+    cache.fill(c["layer"], c["k_rows"], c["v_rows"])
+    ws = attention_workspace(32, 128)
+    out16, out32 = N.DeviceBuffer(4096 * 2), N.DeviceBuffer(4096 * 4)
+    qkv, qn, kn = dev(c["qkv"]), dev(c["qn"]), dev(c["kn"])
+    run = lambda: N.paged_attention(BF16, 32, 8, 128, cache, c["layer"], 4096, qkv, ws, out16, out_f32=out32, append=True,
+                                    rope_theta=1e6, q_norm=qn, k_norm=kn)
+    run()
+    good = out32.numpy(np.float32).copy()
+    assert rel_l2(good, ref) <= REL_L2 and N.paged_attention_status(ws, 32, 128) == (0, 0)
+    N.Device.set_tuning("attn_merge_spin_limit", 4)
+    N.Device.set_tuning("attn_withhold_split", 1 + 7)
+    try:
+        run()
+    finally:
+        N.Device.set_tuning("attn_merge_spin_limit", 0)
+        N.Device.set_tuning("attn_withhold_split", 0)
+    assert np.all(np.isnan(out32.numpy(np.float32)))          # every head's merge needed split 7
+    rc, err = N.paged_attention_status(ws, 32, 128)
+    assert rc == -1 and err == N.abi.NERVA_HIP_ERROR_STEP_FAULT
+    assert N.paged_attention_status(ws, 32, 128) == (0, 0)     # reported once
+    for _ in range(2):
+        run()
+        assert np.array_equal(out32.numpy(np.uint32), good.view(np.uint32))
+        assert N.paged_attention_status(ws, 32, 128) == (0, 0)
 
 
 def test_paged_attention_no_append_reads_cache_only():
