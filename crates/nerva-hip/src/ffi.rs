@@ -829,6 +829,7 @@ unsafe extern "C" {
     pub fn nerva_hip_steps_are_eager() -> c_int;
     pub fn nerva_hip_session_shares_weight_stream(session: *mut NervaHipHfDecodeSequenceSession) -> c_int;
     pub fn nerva_hip_session_read_logits(session: *mut NervaHipHfDecodeSequenceSession, host_logits: *mut f32) -> c_int;
+    pub fn nerva_hip_session_read_slots(session: *mut NervaHipHfDecodeSequenceSession, first: u32, count: u32, host_slots: *mut NervaHipSyntheticTokenSlot) -> c_int;
     pub fn nerva_hip_session_step_trace_bytes(session: *mut NervaHipHfDecodeSequenceSession) -> u64;
     pub fn nerva_hip_session_trace_next_step(session: *mut NervaHipHfDecodeSequenceSession, device_buffer: *mut c_void, bytes: u64) -> c_int;
     pub fn nerva_hip_session_read_kv(session: *mut NervaHipHfDecodeSequenceSession, layer: u32, token: u32, host_k: *mut u16, host_v: *mut u16) -> c_int;

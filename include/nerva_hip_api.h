@@ -757,6 +757,10 @@ int nerva_hip_steps_are_eager(void);
  * of 2048), 0 when every sequence of such a step runs its own decode step; -1 for a null session. */
 int nerva_hip_session_shares_weight_stream(NervaHipHfDecodeSequenceSession *session);
 int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *session, float *host_logits);
+/* Test hook (no counterpart): copies `count` token slots, from slot `first`, out of the session's device memory
+ * as the device wrote them (40 bytes each: nerva_cuda_api.h:29-37, sampler.cu:394-407). */
+int nerva_hip_session_read_slots(NervaHipHfDecodeSequenceSession *session, uint32_t first, uint32_t count,
+                                 NervaHipSyntheticTokenSlot *host_slots);
 /* Test hook (no counterpart): arms a trace of the NEXT decode step the session launches (through
  * advance): that one step runs kernel by kernel instead of as a graph replay, and after each kernel
  * its output vector is copied into `device_buffer`, one 256-byte-aligned slot behind the other, in

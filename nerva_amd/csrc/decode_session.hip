@@ -2363,6 +2363,14 @@ int nerva_hip_session_read_logits(NervaHipHfDecodeSequenceSession *s, float *hos
   return hipMemcpy(host_logits, s->logits, static_cast<uint64_t>(s->vocab) * 4, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
 }
 
+int nerva_hip_session_read_slots(NervaHipHfDecodeSequenceSession *s, uint32_t first, uint32_t count,
+                                 NervaHipSyntheticTokenSlot *host_slots) {
+  if (s == nullptr || host_slots == nullptr || static_cast<uint64_t>(first) + count > s->max_ctx) return -1;
+  if (count == 0) return 0;
+  if (hipStreamSynchronize(s->stream) != hipSuccess) return -1;
+  return hipMemcpy(host_slots, s->slots + first, static_cast<uint64_t>(count) * sizeof(Slot), hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+
 int nerva_hip_session_read_kv_range(NervaHipHfDecodeSequenceSession *s, uint32_t layer, uint32_t first_token,
                                     uint32_t token_count, uint16_t *host_k, uint16_t *host_v) {
   if (s == nullptr || host_k == nullptr || host_v == nullptr || layer >= s->layers ||

@@ -322,6 +322,14 @@ class DecodeSession:
             raise RuntimeError("read_logits failed")
         return out
 
+    def slots(self, first, count):
+        """The raw 40-byte token slots [first, first + count) as the device wrote them: a (count, 40) uint8 array."""
+        out = np.zeros((count, C.sizeof(abi.NervaHipSyntheticTokenSlot)), np.uint8)
+        ptr = C.cast(out.ctypes.data, C.POINTER(abi.NervaHipSyntheticTokenSlot))
+        if self.lib.nerva_hip_session_read_slots(self.handle, first, count, ptr) != 0:
+            raise RuntimeError("read_slots failed")
+        return out
+
     def kv_row(self, layer, token):
         k = np.empty(self.kv_hidden, np.uint16)
         v = np.empty(self.kv_hidden, np.uint16)

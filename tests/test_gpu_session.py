@@ -868,3 +868,129 @@ def test_batch_advance_one_fills_contexts_to_the_last_slot():
     assert rc == -1
     small.destroy()
     large.destroy()
+
+
+def expected_slot_bytes(position, token):
+    """{request_id 1, sequence_id 1, token_index, token, version = index + 1, completion 1, host_copied 0}
+    laid out as the 40-byte C struct (nerva_cuda_api.h:29-37, sampler.cu:394-407)."""
+    slot = abi.NervaHipSyntheticTokenSlot()
+    C.memset(C.byref(slot), 0, C.sizeof(slot))
+    slot.request_id, slot.sequence_id, slot.token_index, slot.token = 1, 1, position, token
+    slot.version, slot.completion, slot.host_copied = position + 1, 1, 0
+    return np.frombuffer(bytes(slot), np.uint8)
+
+
+def test_token_slots_hold_the_reference_bytes(kat):
+    """Every byte of every published slot, downloaded from device memory: the known-answer stream and a random
+    model's greedy and sampled streams; slots before the first sampled position and behind the last stay zero."""
+    weights, k = kat_models(kat, True)
+    session = N.DecodeSession.create(weights, 8)
+    rc, _ = session.start(k["prompt"])
+    assert rc == 0
+    rc, _, tokens = session.advance(4)
+    assert rc == 0 and tokens.tolist() == k["tokens"]
+    raw = session.slots(0, 8)
+    for i, tok in enumerate(k["tokens"]):          # prompt [0]: the first sampled token sits in slot 0
+        assert np.array_equal(raw[i], expected_slot_bytes(i, tok)), i
+    assert not raw[4:].any()
+    session.destroy()
+
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[0]
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 606, theta, qk_norm, bias)
+    prompt = np.random.default_rng(606).integers(0, vocab, 37).astype(np.uint32)
+    session = N.DecodeSession.create(weights, 64)
+    for sampler in (None, (0.8, 0.9, 20, 5)):
+        cfg = None
+        if sampler is not None:
+            cfg = abi.NervaHipHfDecodeSamplerConfig()
+            cfg.temperature, cfg.top_p, cfg.top_k, cfg.seed = sampler
+        rc, _ = session.start(prompt, sampler=cfg)
+        assert rc == 0
+        rc, _, tokens = session.advance(9)
+        assert rc == 0
+        raw = session.slots(0, 64)
+        P = len(prompt)
+        assert not raw[:P - 1].any() and not raw[P - 1 + 9:].any()
+        for i, tok in enumerate(tokens):
+            assert np.array_equal(raw[P - 1 + i], expected_slot_bytes(P - 1 + i, int(tok))), (sampler, i)
+    session.destroy()
+
+
+def test_step_whose_attention_merge_gives_up_fails_the_advance():
+    """A decode step in which a split of the attention never hands its partial over (test hook; the spin limit of
+    the merges set to a few polls, every kernel exits normally): the slot of that token says so, advance returns -1
+    with the step-fault error and the sequence is over; a session made without the hook decodes the same prompt."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[0]
+    weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 31, theta, qk_norm, bias)
+    prompt = np.random.default_rng(31).integers(0, vocab, 700).astype(np.uint32)     # 44 blocks: the splits merge
+    good = N.DecodeSession.create(weights, 720)
+    rc, _ = good.start(prompt)
+    assert rc == 0
+    rc, res, want = good.advance(6)
+    assert rc == 0 and res.hip_error == 0
+    N.Device.set_tuning("attn_merge_spin_limit", 4)
+    N.Device.set_tuning("attn_withhold_split", 1 + 3)
+    try:
+        bad = N.DecodeSession.create(weights, 720)
+        rc, _ = bad.start(prompt)          # the last prompt token's step already runs the decode attention
+        assert rc == 0
+        rc, res, tokens = bad.advance(6)
+    finally:
+        N.Device.set_tuning("attn_merge_spin_limit", 0)
+        N.Device.set_tuning("attn_withhold_split", 0)
+    assert rc == -1 and res.status == -1 and res.hip_error == abi.NERVA_HIP_ERROR_STEP_FAULT
+    assert res.observed_tokens == 0 and len(tokens) == 0
+    raw = bad.slots(len(prompt) - 1, 1)
+    assert raw[0].view(np.uint32)[8] == abi.NERVA_HIP_SLOT_DEVICE_FAULT          # completion word
+    rc, res, _ = bad.advance(1)
+    assert rc == -1                                                                # the sequence ended with the fault
+    bad.destroy()
+    rc, res, again = good.advance(3)                                               # the healthy session is untouched
+    assert rc == 0
+    fresh = N.DecodeSession.create(weights, 720)
+    rc, _ = fresh.start(prompt)
+    assert rc == 0
+    rc, res, tokens = fresh.advance(9)
+    assert rc == 0 and tokens.tolist() == want.tolist() + again.tolist()
+    for s in (good, fresh):
+        s.destroy()
+
+
+def test_batch_step_of_sessions_with_their_own_steps_at_long_context():
+    """Shapes the multi-row kernels do not take (hidden 512) advance a batch as one captured decode step per
+    session, one after the other. At contexts of 1000 and more tokens each step's attention launch spreads over
+    64 splits that merge inside the launch: tokens equal those of the same sessions advanced alone, and the rows
+    appended equal the oracle's on the same history."""
+    dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[0]
+    weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 88, theta, qk_norm, bias)
+    rng = np.random.default_rng(88)
+    prompts = [rng.integers(0, vocab, n).astype(np.uint32) for n in (1030, 1333, 1571)]
+    steps, max_ctx = 5, 1600
+    plan = N.WeightPlan.from_weights(weights)
+    parent = N.DecodeSession.create(weights, max_ctx, plan=plan, tensor_pointers=False)
+    sessions = [parent, parent.fork_shared_weights(), parent.fork_shared_weights()]
+    streams = [[started(s, p)] for s, p in zip(sessions, prompts)]
+    for _ in range(steps):
+        rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 8, 2)
+        assert rc == 0 and res.status == 0 and res.block_tokens == 3 and not parent.shares_weight_stream()
+        for stream, tok in zip(streams, tokens):
+            stream.append(int(tok))
+    solo = parent.fork_shared_weights()
+    for prompt, stream in zip(prompts, streams):
+        rc, _ = solo.start(prompt)
+        assert rc == 0
+        rc, _, alone = solo.advance(steps + 1)
+        assert rc == 0 and alone.tolist() == stream, len(prompt)      # the same kernels on the same inputs
+    ctx, _ = oracle_follow(omodel, max_ctx, prompts[0], streams[0][:-1])
+    P = len(prompts[0])
+    for layer in range(layers):
+        for token in (P, P + steps - 1):
+            gk, gv = sessions[0].kv_row(layer, token)
+            rk, rv = ctx.read_kv16(layer, token)
+            tol = 2e-3 if layer == 0 else E2E_REL_L2
+            assert rel_l2(O.decode16(dtype, gk), O.decode16(dtype, rk)) <= tol, (layer, token)
+            assert rel_l2(O.decode16(dtype, gv), O.decode16(dtype, rv)) <= tol, (layer, token)
+    ctx.close()
+    solo.destroy()
+    for s in sessions[::-1]:
+        s.destroy()
