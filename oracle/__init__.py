@@ -364,9 +364,10 @@ class Model:
                           _p(self.final_norm, u16p), _p(self.lm_head, u16p))
 
 
-def synthetic_model(cfg, seed, weight_std, layers=None, embedding_rows=None, threads=8):
+def synthetic_model(cfg, seed, weight_std, layers=None, embedding_rows=None, threads=8, layer_ids=None):
     """Host copy of the weights nerva_hip_bench_session_create_synthetic generates on the device
-    (same counter-based generator, same tensor ids), as a Model. `layers` keeps the first n layers;
+    (same counter-based generator, same tensor ids), as a Model. `layers` keeps the first n layers, or
+    `layer_ids` exactly those layers of the device's model (in that order);
     `embedding_rows` keeps only those rows of the embedding table (the others stay zero)."""
     import concurrent.futures
     dt, H, HD = cfg["dtype"], cfg["hidden"], cfg["head_dim"]
@@ -388,7 +389,7 @@ def synthetic_model(cfg, seed, weight_std, layers=None, embedding_rows=None, thr
         return out
 
     ls = []
-    for l in range(layers):
+    for l in (range(layers) if layer_ids is None else layer_ids):
         b = 16 * (l + 1)
         ls.append(dict(rms_attn=gen(b, H, 1.0), rms_mlp=gen(b + 1, H, 1.0), w_q=gen(b + 2, A * H).reshape(A, H),
                        w_k=gen(b + 4, KV * H).reshape(KV, H), q_norm=gen(b + 5, HD, 1.0), k_norm=gen(b + 6, HD, 1.0),

@@ -44,10 +44,13 @@ def _gemv16(dtype, w, x16, threads):
     return O.gemv_x16(dtype, w, x16)
 
 
-def check_step_links(model, trace, position, token_in, token_out, k_rows, v_rows, threads=1):
+def check_step_links(model, trace, position, token_in, token_out, k_rows, v_rows, threads=1, layer_ids=None):
     """Checks every link of one traced decode step. `k_rows[l]`, `v_rows[l]`: the device's cache rows
     0..position of layer l in logical order (16-bit), read after the step, so row `position` is the
-    one the step appended. Returns {link name: measured error}; raises AssertionError on a miss."""
+    one the step appended. `layer_ids`: the session's layers that model.layers[i] (and k_rows[i],
+    v_rows[i]) stand for, when the model holds only some of them; every checked layer takes the
+    device's own input (the output the trace holds for the layer before it).
+    Returns {link name: measured error}; raises AssertionError on a miss."""
     m, dt = model, model.dtype
     H, HD = m.hidden, m.head_dim
     A, KV = m.heads * HD, m.kv_heads * HD
@@ -78,8 +81,11 @@ def check_step_links(model, trace, position, token_in, token_out, k_rows, v_rows
         "embedding row of token %d" % token_in
     # (a model that holds only the first layers of the session's - the full-size check of the bench -
     # gets those layers checked; the head then takes the x the session's last layer left)
+    ids = list(range(len(m.layers))) if layer_ids is None else list(layer_ids)
     for l, w in enumerate(m.layers):
-        t = trace["layers"][l]
+        t = trace["layers"][ids[l]]
+        if ids[l] > 0:
+            x = trace["layers"][ids[l] - 1]["x"]
         # attention RMSNorm (fused into the qkv launch; its 16-bit output is the projection's input),
         # then the qkv projection (raw: biases are added by the attention kernel)
         link16("attn_norm", t["a16"], O.rms_norm(dt, x, w["rms_attn"], m.rms_eps))

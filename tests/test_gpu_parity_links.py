@@ -136,6 +136,37 @@ def test_long_context_links_at_qwen3_8b_widths():
           flush=True)
 
 
+def test_full_depth_step_at_8k_context_first_layers_last_layer_and_head():
+    """The named workload at its real size: 36 layers of Qwen3-8B widths (one 17.6 GB arena, device-generated
+    weights), a prompt of 8192 tokens prefilled in blocks, then decode steps with the 32-split attention. One
+    step is traced and layers 0, 1 and 35 and the head are checked link by link on the device's own inputs -
+    weights of those layers regenerated bit for bit on the host, their K/V rows downloaded - and the step after
+    it, a graph replay, must start from the token the traced step published."""
+    cfg = dict(N.Qwen3_8B)
+    P, max_ctx, ids = 8192, 8192 + 16, [0, 1, 35]
+    s = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=0.02, qk_norm=True)
+    assert s.create_result.layer_count == 36
+    prompt = O.synth_tokens(SEED, 97, P, cfg["vocab"])
+    rc, res = s.start(prompt)
+    assert rc == 0
+    rc, res, out = s.advance(2)
+    assert rc == 0 and res.graph_replays == 1 and res.hot_path_allocations == 0
+    token, position = int(out[1]), P + 1
+    model = O.synthetic_model(cfg, SEED, 0.02, layer_ids=ids, embedding_rows=[token], threads=16)
+    rc, res, out, trace = s.traced_advance()
+    assert rc == 0 and trace is not None and len(trace["layers"]) == 36
+    rows = [s.kv_range(l, 0, position + 1) for l in ids]
+    errs = check_step_links(model, trace, position, token, int(out[0]), [r[0] for r in rows], [r[1] for r in rows],
+                            threads=16, layer_ids=ids)
+    rc, res, after = s.advance(1)
+    assert rc == 0 and res.graph_replays == 1
+    raw = s.slots(position, 2).view(np.uint32)
+    assert raw[0][4] == int(out[0]) and raw[1][4] == int(after[0])       # token words of the two slots
+    s.destroy()
+    print("36 layers, context %d: layers 0, 1, 35 and head (worst rel L2): %s"
+          % (position, ", ".join("%s %.1e" % kv_ for kv_ in sorted(errs.items()))), flush=True)
+
+
 def test_lm_head_full_vocabulary_tie_and_nonfinite_rows():
     """The LM head at its real size (151936 x 4096, the looping launch that leaves one candidate per
     workgroup, then the finishing launch) inside a session whose one layer is small: two identical rows
