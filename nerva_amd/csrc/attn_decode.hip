@@ -239,17 +239,8 @@ __device__ __forceinline__ void merge_part_tagged(const AttnParams &p, uint32_t 
     if (p.out_f32 != nullptr) p.out_f32[e] = ot;
     p.out16[attn_out_elem(p, e)] = enc16<DT>(ot);
   }
-  // Every thread has taken what it needs (a split's m and l words are read by all 32 threads of a group, so
-  // nobody may clear them before a barrier that follows the reads: the one above): the words are cleared for
-  // the next launch - behind the output, which the next kernel waits for, while nothing waits for these.
-#pragma unroll
-  for (uint32_t i = 0; i < kPer; ++i) {
-    if (q + i * kGroups < active) {
-      uint64_t *r = rec + static_cast<uint64_t>(q + i * kGroups) * kStepRecord;
-      __hip_atomic_store(r + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (dl < 2) __hip_atomic_store(r + kStepPartDims + dl, uint64_t{0}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
+  // The words are left as they are: they carry this launch's tag, which no later launch on this workspace uses
+  // (attn_launch_tag), so nothing has to be cleared behind the reads.
 }
 
 typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));

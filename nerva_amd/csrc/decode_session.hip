@@ -254,8 +254,13 @@ __global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prom
   }
 }
 
-__global__ void bump_step_counter_kernel(uint32_t *state) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) state[2] = state[2] + 1u;
+// A pass of launches without the embedding launch in front: the step counter moves on, and the attention plan
+// takes the new number (the tags of the split partials derive from it and must differ from launch to launch).
+__global__ void bump_step_counter_kernel(uint32_t *state, uint32_t *attn_plan) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    state[2] = state[2] + 1u;
+    if (attn_plan != nullptr) attn_plan[4] = state[2];
+  }
 }
 
 __global__ void advance_cursor_kernel(uint32_t *state, uint32_t max_steps) {
@@ -693,6 +698,10 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
                     hipMemcpyHostToDevice);
   if (err == hipSuccess)
     err = hipMemsetAsync(s->slots, 0, static_cast<uint64_t>(s->max_ctx) * sizeof(Slot), s->stream);
+  // the attention's tagged split partials: a tag is unique for 2^23 steps, which no sequence reaches, so with
+  // the words cleared here none of an earlier sequence's can ever match
+  if (err == hipSuccess && s->attn_tagged != nullptr)
+    err = hipMemsetAsync(s->attn_tagged, 0, attn_step_workspace_bytes(s->heads), s->stream);
   if (err == hipSuccess) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, s->stream, s->state, 0u, prompt_count, 1u);
     err = hipGetLastError();
@@ -2257,7 +2266,7 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *s, uint32_t 
     uint64_t acc = 0;
     for (uint32_t rep = 0; err == hipSuccess && rep < repeats + 1; ++rep) {
       // no embed launch in this pass: advance the step counter here
-      hipLaunchKernelGGL(bump_step_counter_kernel, dim3(1), dim3(64), 0, s->stream, s->state);
+      hipLaunchKernelGGL(bump_step_counter_kernel, dim3(1), dim3(64), 0, s->stream, s->state, s->attn_plan);
       err = hipGetLastError();
       if (err == hipSuccess) err = hipEventRecord(s->ev0, s->stream);
       if (err == hipSuccess) err = enqueue_step(s, kDecodeStep, nullptr, kind);
