@@ -106,6 +106,92 @@ def cpu_baseline(session, cfg, position, token, layers_sampled, threads_all):
     return result
 
 
+def cpu_operator_baselines(threads_all):
+    """The four operator configurations on the CPU oracle, each timed in full: the scalar single-core loop the
+    reference's CPU path is, and the same work spread over `threads_all` host threads (rows of a GEMV through
+    the oracle's OpenMP loop; kv heads of the attention and experts of the MoE as independent calls from a
+    thread pool). Inputs have the configurations' shapes and value ranges; nothing here is checked against the
+    device (the parity tests do that) - this is the reported CPU baseline beside each GPU row.
+    Returns {config key: {"cpu_1core_us", "cpu_Ncore_us", "cpu_cores"}}."""
+    import oracle as O
+    BF16 = 1
+    rng = np.random.default_rng(SEED)
+    pool = concurrent.futures.ThreadPoolExecutor(max_workers=threads_all)
+
+    def clock(fn):
+        t0 = time.perf_counter()
+        fn()
+        return (time.perf_counter() - t0) * 1e6
+
+    def w16(tid, rows, cols):
+        return O.synth_16(BF16, SEED, tid, rows * cols, 0.0, WEIGHT_STD).reshape(rows, cols)
+
+    out = {}
+    # 1: q_proj GEMV 4096 x 4096, bf16 in, f32 accumulate, bf16 out
+    w, x = w16(11, 4096, 4096), O.decode16(BF16, O.synth_16(BF16, SEED, 12, 4096, 0.0, 1.0))
+    out["configs[0]"] = dict(cpu_1core_us=clock(lambda: O.encode16(BF16, O.gemv(BF16, w, x, threads=1))),
+                             cpu_Ncore_us=clock(lambda: O.encode16(BF16, O.gemv(BF16, w, x, threads=threads_all))))
+    # 2: MLP block: RMSNorm -> gate/up GEMVs -> SiLU(gate) * up -> down GEMV -> + residual
+    H, I = 4096, 12288
+    wg, wu, wd = w16(21, I, H), w16(22, I, H), w16(23, H, I)
+    gamma = O.synth_16(BF16, SEED, 24, H, 1.0, 0.02)
+    h = O.synth_f32(SEED, 25, H, 0.0, 1.0)
+
+    def mlp(threads):
+        n16 = O.decode16(BF16, O.encode16(BF16, O.rms_norm(BF16, h, gamma, 1e-6)))
+        g, u = O.gemv(BF16, wg, n16, threads=threads), O.gemv(BF16, wu, n16, threads=threads)
+        ff = O.decode16(BF16, O.encode16(BF16, (g / (np.float32(1) + np.exp(-g, dtype=np.float32))) * u))
+        return h + O.gemv(BF16, wd, ff, threads=threads)
+    out["configs[1]"] = dict(cpu_1core_us=clock(lambda: mlp(1)), cpu_Ncore_us=clock(lambda: mlp(threads_all)))
+    del wg, wu, wd
+    # 3: paged GQA decode attention, 32 q / 8 kv heads x 128, 4096 cached keys + the appended one
+    heads, kvh, hd, tokens = 32, 8, 128, 4096
+    blocks = tokens // 16 + 1
+    table = rng.permutation(blocks).astype(np.uint32)
+    kc = O.synth_16(BF16, SEED, 31, blocks * 16 * kvh * hd, 0.0, 1.0).reshape(1, blocks, 16, kvh * hd)
+    vc = O.synth_16(BF16, SEED, 32, blocks * 16 * kvh * hd, 0.0, 1.0).reshape(1, blocks, 16, kvh * hd)
+    qkv = O.synth_f32(SEED, 33, (heads + 2 * kvh) * hd, 0.0, 1.0)
+    qn, kn = O.synth_16(BF16, SEED, 34, hd, 1.0, 0.02), O.synth_16(BF16, SEED, 35, hd, 1.0, 0.02)
+
+    def attention(threads):
+        A, KV = heads * hd, kvh * hd
+        q = O.rope(hd, heads, tokens, 1e6, O.per_head_rms_norm(BF16, qn, hd, qkv[:A], 1e-6))
+        k = O.rope(hd, kvh, tokens, 1e6, O.per_head_rms_norm(BF16, kn, hd, qkv[A:A + KV], 1e-6))
+        kc[0, table[tokens // 16], tokens % 16] = O.encode16(BF16, k)
+        vc[0, table[tokens // 16], tokens % 16] = O.encode16(BF16, qkv[A + KV:])
+        if threads == 1:
+            return O.attention_paged16(BF16, heads, kvh, hd, 16, q, kc, vc, table, 0, blocks, tokens + 1)
+        G = heads // kvh   # one call per kv head: its query heads over its slice of the cache
+
+        def head_group(j):
+            return O.attention_paged16(BF16, G, 1, hd, 16, q[j * G * hd:(j + 1) * G * hd],
+                                       np.ascontiguousarray(kc[..., j * hd:(j + 1) * hd]),
+                                       np.ascontiguousarray(vc[..., j * hd:(j + 1) * hd]), table, 0, blocks, tokens + 1)
+        return np.concatenate(list(pool.map(head_group, range(kvh))))
+    out["configs[2]"] = dict(cpu_1core_us=clock(lambda: attention(1)), cpu_Ncore_us=clock(lambda: attention(threads_all)))
+    # 4: FP8 MoE, 8 routed + 1 shared expert, hidden 7168, expert MLP 2048, 128 x 128 f32 block scales
+    H, I, E, blk = 7168, 2048, 9, 128
+    sH, sI = H // blk, I // blk
+    fp8 = lambda n: (rng.integers(0, 0x78, n, dtype=np.uint8) | (rng.integers(0, 2, n, dtype=np.uint8) << 7))
+    wg8, wu8, wd8 = fp8(E * I * H), fp8(E * I * H), fp8(E * H * I)
+    sg, su, sd = (np.full(E * sI * sH, 0.02 / 448, np.float32) for _ in range(3))
+    x16 = O.synth_16(BF16, SEED, 41, H, 0.0, 1.0)
+    ids, wts = np.arange(8, dtype=np.uint32), np.full(8, 0.125, np.float32)
+
+    def moe(threads):
+        if threads == 1:
+            return O.moe_fp8_forward(H, I, E, blk, x16, ids, wts, wg8, sg, wu8, su, wd8, sd, shared_index=8)
+        one = lambda e: O.moe_fp8_forward(H, I, E, blk, x16, np.array([e], np.uint32),
+                                          np.array([0.125 if e < 8 else 1.0], np.float32), wg8, sg, wu8, su, wd8, sd)
+        return np.sum(list(pool.map(one, range(E))), axis=0)
+    out["configs[3]"] = dict(cpu_1core_us=clock(lambda: moe(1)), cpu_Ncore_us=clock(lambda: moe(threads_all)))
+    pool.shutdown()
+    for key, row in out.items():
+        row["cpu_1core_us"], row["cpu_Ncore_us"], row["cpu_cores"] = round(row["cpu_1core_us"], 1), round(row["cpu_Ncore_us"], 1), threads_all
+        log("[cpu] %s on the oracle: %.0f us on 1 core, %.0f us on %d threads" % (key, row["cpu_1core_us"], row["cpu_Ncore_us"], threads_all))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -283,6 +369,14 @@ def main():
             except Exception as e:  # an operator row never hides the headline figure
                 log("[bench] operator case %s failed: %r" % (key, e))
                 operators[key] = {"failed": repr(e)}
+        if not args.no_cpu:
+            try:   # the CPU figure of every operator row, timed in full on this host
+                for prefix, row in cpu_operator_baselines(min(os.cpu_count() or 1, 16)).items():
+                    for key in operators:
+                        if key.startswith(prefix):
+                            operators[key].update(row)
+            except Exception as e:
+                log("[cpu] operator baselines failed: %r" % (e,))
 
     line = dict(metric="decode tok/s Qwen3-8B bs1", value=round(tok_s, 2), unit="tok/s", n_gpus=1,
                 steps=args.steps, warmup=args.warmup, ms_per_step=round(1e3 * elapsed / args.steps, 4),

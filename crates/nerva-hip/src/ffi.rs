@@ -819,6 +819,7 @@ unsafe extern "C" {
     pub fn nerva_hip_allocation_count() -> u64;
     pub fn nerva_hip_timer_capture_begin() -> c_int;
     pub fn nerva_hip_timer_capture_end(warmup_replays: u32, timed_replays: u32, nodes: *mut u64, avg_replay_ns: *mut f64) -> c_int;
+    pub fn nerva_hip_timer_capture_end_stats(warmup_replays: u32, timed_replays: u32, nodes: *mut u64, avg_replay_ns: *mut f64, min_replay_ns: *mut f64, median_replay_ns: *mut f64) -> c_int;
     pub fn nerva_hip_copy_d2d(device_dst: *mut c_void, device_src: *const c_void, bytes: u64, stream: *mut c_void) -> c_int;
     pub fn nerva_hip_synth_fill_16(device_dst: *mut c_void, dtype: u32, seed: u64, tensor_id: u64, count: u64, mean: f32, std: f32) -> c_int;
     pub fn nerva_hip_synth_fill_f32(device_dst: *mut c_void, seed: u64, tensor_id: u64, count: u64, mean: f32, std: f32) -> c_int;

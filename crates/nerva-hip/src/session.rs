@@ -139,6 +139,44 @@ impl HipHfDecodeSequenceSessionConfig<'_> {
         if self.final_norm_weight.len() != self.hidden {
             return Some("final norm size does not match hidden");
         }
+        // every size crosses the boundary as u32, and the products below must not wrap either
+        for value in [self.hidden, self.heads, self.kv_heads, self.head_dim, self.intermediate, self.vocab_size,
+                      self.max_context_tokens, self.layers.len()] {
+            if u32::try_from(value).is_err() {
+                return Some("a model dimension does not fit 32 bits");
+            }
+        }
+        let (Some(attention), Some(kv_hidden)) = (self.heads.checked_mul(self.head_dim), self.kv_heads.checked_mul(self.head_dim))
+        else {
+            return Some("heads x head_dim overflows");
+        };
+        // Native code reads every layer tensor at the size the dimensions imply, so each slice is checked here
+        // (crates/nerva-cuda/src/decode/hf_chain/layer.rs:582,710-721, hf_step/request.rs:133-139): a short slice
+        // must never reach the pointer cast.
+        let size = |rows: usize, cols: usize| rows.checked_mul(cols);
+        for layer in self.layers {
+            let matrices = [(layer.w_q, size(attention, self.hidden)), (layer.w_k, size(kv_hidden, self.hidden)),
+                            (layer.w_v, size(kv_hidden, self.hidden)), (layer.w_o, size(self.hidden, attention)),
+                            (layer.w_gate, size(self.intermediate, self.hidden)),
+                            (layer.w_up, size(self.intermediate, self.hidden)),
+                            (layer.w_down, size(self.hidden, self.intermediate))];
+            for (slice, want) in matrices {
+                if want.map_or(true, |n| slice.len() != n) {
+                    return Some("a layer matrix does not match the model dimensions");
+                }
+            }
+            if layer.rms_attn_weight.len() != self.hidden || layer.rms_mlp_weight.len() != self.hidden {
+                return Some("a layer norm weight does not match hidden");
+            }
+            let optional = [(layer.q_norm_weight, self.head_dim), (layer.k_norm_weight, self.head_dim),
+                            (layer.q_bias, attention), (layer.k_bias, kv_hidden), (layer.v_bias, kv_hidden),
+                            (layer.o_bias, self.hidden)];
+            for (slice, want) in optional {
+                if slice.map_or(false, |s| s.len() != want) {
+                    return Some("an optional layer tensor does not match the model dimensions");
+                }
+            }
+        }
         None
     }
 
@@ -165,14 +203,14 @@ impl HipHfDecodeSequenceSessionConfig<'_> {
         let native_layers: Vec<NervaHipHfDecodeChainLayer> = self.layers.iter().map(|l| l.native()).collect();
         let mut request: NervaHipHfDecodeSequenceSessionCreateRequest = unsafe { std::mem::zeroed() };
         request.dtype = self.dtype;
-        request.hidden = self.hidden as u32;
-        request.heads = self.heads as u32;
-        request.kv_heads = self.kv_heads as u32;
-        request.head_dim = self.head_dim as u32;
-        request.intermediate = self.intermediate as u32;
-        request.vocab_size = self.vocab_size as u32;
-        request.layer_count = native_layers.len() as u32;
-        request.max_context_tokens = self.max_context_tokens as u32;
+        request.hidden = u32::try_from(self.hidden).unwrap_or(0); // validate() has checked the range
+        request.heads = u32::try_from(self.heads).unwrap_or(0); // validate() has checked the range
+        request.kv_heads = u32::try_from(self.kv_heads).unwrap_or(0); // validate() has checked the range
+        request.head_dim = u32::try_from(self.head_dim).unwrap_or(0); // validate() has checked the range
+        request.intermediate = u32::try_from(self.intermediate).unwrap_or(0); // validate() has checked the range
+        request.vocab_size = u32::try_from(self.vocab_size).unwrap_or(0); // validate() has checked the range
+        request.layer_count = u32::try_from(native_layers.len()).unwrap_or(0);
+        request.max_context_tokens = u32::try_from(self.max_context_tokens).unwrap_or(0); // validate() has checked the range
         request.rms_eps = self.rms_eps;
         request.rope_theta = self.rope_theta.unwrap_or(0.0);
         request.embeddings = self.embeddings.as_ptr();
@@ -285,10 +323,13 @@ impl<'a> HipHfDecodeSequenceLoop<'a> {
         if prompt_tokens.iter().any(|&t| t as usize >= vocab) {
             return (summary_from(&empty, Vec::new(), Some("prompt token outside the vocabulary")), None);
         }
+        let Ok(prompt_token_count) = u32::try_from(prompt_tokens.len()) else {
+            return (summary_from(&empty, Vec::new(), Some("prompt longer than 32 bits count")), None);
+        };
         let mut request: NervaHipHfDecodeSequenceSessionStartRequest = unsafe { std::mem::zeroed() };
         request.session = session.handle;
         request.prompt_tokens = prompt_tokens.as_ptr();
-        request.prompt_token_count = prompt_tokens.len() as u32;
+        request.prompt_token_count = prompt_token_count;
         request.has_eos_token = eos_token.is_some() as u32;
         request.eos_token = eos_token.unwrap_or(0);
         let mut out: NervaHipHfDecodeSequenceResult = unsafe { std::mem::zeroed() };
@@ -316,12 +357,15 @@ impl<'a> HipHfDecodeSequenceLoop<'a> {
         if steps == 0 {
             return summary_from(&empty, Vec::new(), Some("steps must be non-zero"));
         }
+        let Ok(step_count) = u32::try_from(steps) else {
+            return summary_from(&empty, Vec::new(), Some("steps do not fit 32 bits"));
+        };
         let mut tokens = vec![0u32; steps];
         let mut request: NervaHipHfDecodeSequenceSessionAdvanceRequest = unsafe { std::mem::zeroed() };
         request.session = self.session.handle;
-        request.steps = steps as u32;
+        request.steps = step_count;
         request.output_tokens = tokens.as_mut_ptr();
-        request.output_token_capacity = steps as u32;
+        request.output_token_capacity = step_count;
         let mut out: NervaHipHfDecodeSequenceResult = unsafe { std::mem::zeroed() };
         unsafe { nerva_hip_hf_decode_sequence_session_advance(&request, &mut out) };
         tokens.truncate(out.observed_tokens as usize);

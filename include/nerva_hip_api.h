@@ -563,11 +563,12 @@ uint64_t nerva_hip_argmax_workspace_bytes(void);
  * result as nerva_hip_argmax; the per-workgroup candidates live in a 6 KiB array inside the
  * library's device image instead of a caller workspace, and the call performs no hipMalloc, hipFree
  * or other allocating routine: two kernel launches on `stream` (pass the caller's stream; NULL
- * uses the library's stream, which exists once nerva_hip_device_smoke has run). `logits` and
- * `token` are device pointers. count > NERVA_HIP_ARGMAX_STATIC_MAX_COUNT fails with
- * hipErrorInvalidValue and launches nothing. All calls on one GPU share the array: calls that
- * overlap on one GPU (different streams, or graphs replayed concurrently) race. The array's address
- * is resolved at the first call on a device, or by nerva_hip_device_smoke. */
+ * uses the library's stream). `logits` and `token` are device pointers. nerva_hip_device_smoke has to
+ * have run on the device first: it resolves the array's address there and creates the library's
+ * stream; before that the call fails with hipErrorNotInitialized (3) instead of setting either up
+ * itself. count > NERVA_HIP_ARGMAX_STATIC_MAX_COUNT fails with hipErrorInvalidValue and launches
+ * nothing. All calls on one GPU share the array: calls that overlap on one GPU (different streams,
+ * or graphs replayed concurrently) race. */
 #define NERVA_HIP_ARGMAX_STATIC_MAX_COUNT 16777216u
 int nerva_hip_argmax_static(const float *logits, uint32_t count, uint32_t *token, void *stream,
                             int32_t *hip_error);
@@ -684,6 +685,10 @@ uint64_t nerva_hip_allocation_count(void);
 int nerva_hip_timer_capture_begin(void);
 int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
                                 double *avg_replay_ns);
+/* The same, with the shortest and the median replay beside the average (every replay between two events of
+ * its own). */
+int nerva_hip_timer_capture_end_stats(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
+                                      double *avg_replay_ns, double *min_replay_ns, double *median_replay_ns);
 /* Plain device-to-device copy kernel (16-byte aligned pointers and size): moves exactly `bytes`
  * in and `bytes` out, the known-size transfer memory counters are calibrated against. */
 int nerva_hip_copy_d2d(void *device_dst, const void *device_src, uint64_t bytes, void *stream);
@@ -741,8 +746,15 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
  * MoE down launch walks the shared expert last instead of first), "gemv_workgroup_waves" (4|16: waves per
  * workgroup of every lean GEMV launch), "gemv_x_registers" (2: the lean GEMV never keeps the input vector in
  * registers), "prefill_block_tokens" (128: sessions created afterwards prefill in 128-token blocks even where
- * the 256-token blocks apply). Values a kernel
- * cannot take are ignored where they are read. -1 for an unknown name. */
+ * the 256-token blocks apply), "gemv_rotated_walk" (2: the lean GEMV never walks its rows from a rotated
+ * start), "attn_merge_spin_limit" and "attn_withhold_split" (the bounded wait of the decode attention's split
+ * merge: polls before it gives up; 1 + the split that keeps its partial to itself), and the comparison modes
+ * "block_layout" (1: token blocks as [token][column] rows, 2: in matrix-operand order, whatever their size),
+ * "prefill_attention_rows" (1: prompt blocks with one attention workgroup set per token), "prefill_walk" (1:
+ * sessions created afterwards walk their prompts token by token), "gemm_block_off" (1: blocks of more than 64
+ * rows through the kernel of the smaller ones). Values a kernel
+ * cannot take are ignored where they are read. -1 for an unknown name. A null name restores every built-in
+ * choice. */
 int nerva_hip_test_set_tuning(const char *name, int32_t value);
 
 /* 1 when this process launches its steps kernel by kernel instead of replaying captured graphs:

@@ -23,14 +23,18 @@ constexpr int kMaxDevices = 16;
 std::mutex g_scratch_mutex;
 uint32_t *g_scratch_ptr[kMaxDevices] = {};
 
-// Device address of `scratch` on the current device, resolved once per device.
-hipError_t static_scratch(uint32_t **out) {
+// Device address of `scratch` on the current device. `resolve` (set-up calls only): ask the runtime for it if
+// this device has none yet; without it an unresolved device is hipErrorNotInitialized - the entry point itself
+// neither takes the mutex's slow path nor calls into the runtime's symbol tables (neither is safe under stream
+// capture).
+hipError_t static_scratch(uint32_t **out, bool resolve) {
   int device = -1;
   hipError_t err = hipGetDevice(&device);
   if (err != hipSuccess) return err;
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (g_scratch_ptr[device] == nullptr) {
+    if (!resolve) return hipErrorNotInitialized;
     void *ptr = nullptr;
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess) return err;
@@ -97,7 +101,7 @@ hipError_t launch_argmax(const float *logits, uint32_t count, const SampleParams
 
 hipError_t argmax_static_setup() {
   uint32_t *ptr = nullptr;
-  return static_scratch(&ptr);
+  return static_scratch(&ptr, true);
 }
 
 }  // namespace nv
@@ -114,12 +118,12 @@ int nerva_hip_argmax_static(const float *logits, uint32_t count, uint32_t *token
   if (hip_error) *hip_error = 0;
   if (logits == nullptr || token == nullptr || count == 0 || count > NERVA_HIP_ARGMAX_STATIC_MAX_COUNT)
     return done(hipErrorInvalidValue);
-  // With a caller's stream nothing is created here; the library's own stream exists after
-  // nerva_hip_device_smoke (or any earlier call that used it).
-  hipStream_t s = resolve_stream(stream);
-  if (s == nullptr) return done(hipErrorInvalidResourceHandle);
+  // Nothing is created or resolved here: the library's stream (when the caller passes none) and the scratch
+  // address of the current device come from nerva_hip_device_smoke, which has to have run on this device.
+  hipStream_t s = stream != nullptr ? static_cast<hipStream_t>(stream) : library_stream_if_created();
+  if (s == nullptr) return done(hipErrorNotInitialized);
   uint32_t *base = nullptr;
-  hipError_t err = static_scratch(&base);
+  hipError_t err = static_scratch(&base, false);
   if (err != hipSuccess) return done(err);
   SampleParams p{};
   p.part_value = reinterpret_cast<float *>(base);

@@ -715,13 +715,10 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
 // matrix-operand order, which the GEMM reads with full cache lines. Smaller blocks stay [token][column]
 // rows: a lane's 16 bytes then share their cache line with the same token's neighbours in K, and a
 // batch step measured faster that way up to 16 sequences (2: 3.77 vs 4.27 ms, 8: 4.04 vs 4.42, 32: 5.43 vs
-// 4.88). NERVA_HIP_BLOCK_LAYOUT=rows / =operand forces one layout (comparisons).
+// 4.88). The "block_layout" override forces one layout (1 = rows, 2 = operand order; comparisons).
 uint32_t block_operand_tiles(uint32_t tokens) {
-  static const int forced = [] {
-    const char *v = getenv("NERVA_HIP_BLOCK_LAYOUT");
-    return v == nullptr ? 0 : v[0] == 'r' ? 1 : v[0] == 'o' ? 2 : 0;
-  }();
-  const bool operand = forced != 0 ? forced == 2 : tokens > 16;
+  const int forced = tuning(kTuneBlockLayout);
+  const bool operand = forced == 1 || forced == 2 ? forced == 2 : tokens > 16;
   return operand ? gemm_packed_tiles(tokens) : 0u;
 }
 
@@ -736,12 +733,9 @@ hipError_t prefill_blocks(Session *s, uint32_t count, uint32_t prompt_count, Ner
   const uint32_t H = s->hidden, A = s->heads * s->head_dim, KV = s->kv_heads * s->head_dim, I = s->intermediate;
   const float *rope_freq = s->theta > 0.0f ? s->rope_freq : nullptr;
   hipError_t err = hipSuccess;
-  // NERVA_HIP_PREFILL_ATTN=rows: the block's attention as one workgroup set per token (the batch step's
-  // kernel) instead of the prompt kernel that shares K/V tiles between tokens; for comparisons
-  static const bool rows_attention = [] {
-    const char *v = getenv("NERVA_HIP_PREFILL_ATTN");
-    return v != nullptr && v[0] == 'r';
-  }();
+  // "prefill_attention_rows" override = 1: the block's attention as one workgroup set per token (the batch
+  // step's kernel) instead of the prompt kernel that shares K/V tiles between tokens; for comparisons
+  const bool rows_attention = tuning(kTunePrefillAttentionRows) == 1;
   const int want_prompt_splits = tuning(kTunePromptSplits);
   const uint32_t prompt_splits = want_prompt_splits >= 1 && want_prompt_splits <= static_cast<int>(kAttnMaxSplits)
                                      ? static_cast<uint32_t>(want_prompt_splits)
@@ -1149,11 +1143,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
       wide && block_operand_tiles(wideT) != 0 && tuning(kTunePrefillBlockTokens) != 128 ? wideT : kGemmMaxTokens;
   s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
   s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
-  {
-    // NERVA_HIP_PREFILL=walk keeps one prompt step per token where prompt blocks would be possible.
-    const char *mode = getenv("NERVA_HIP_PREFILL");
-    s->block_prefill = s->rows_ready && !(mode != nullptr && mode[0] == 'w');
-  }
+  // ("prefill_walk" override = 1, read here: one prompt step per token where prompt blocks would be possible)
+  s->block_prefill = s->rows_ready && tuning(kTunePrefillWalk) != 1;
   s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
   s->sampler_keys = reinterpret_cast<uint64_t *>(s->arena + off_sampler_keys);
   {

@@ -703,10 +703,7 @@ hipError_t launch_block_dt(int epilogue, const GemmRowsParams &p, const GemmBloc
 
 GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
   GemmBlockPlan plan{};
-  static const int mode = [] {
-    const char *v = getenv("NERVA_HIP_GEMM_BLOCK");   // 0: never use the shared-X kernel
-    return v != nullptr && v[0] == '0' ? 0 : 1;
-  }();
+  const int mode = tuning(kTuneGemmBlockOff) == 1 ? 0 : 1;   // "gemm_block_off" override: never the shared-X kernel
   const int want_slices = tuning(kTuneGemmBlockSlices);
   const int want_tiles = tuning(kTuneGemmBlockRowTiles);
   const uint32_t min_tokens = tuning(kTuneGemmBlockMinTokens) > 0 ? static_cast<uint32_t>(tuning(kTuneGemmBlockMinTokens)) : 17u;

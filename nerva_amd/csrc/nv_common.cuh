@@ -163,6 +163,10 @@ enum TuningKnob : int {
   kTuneGemvRotatedWalk,      // lean GEMV: 2 = never the rotated walk
   kTuneAttnMergeSpinLimit,   // decode attention: polls after which a split merge gives up (tests of the error path)
   kTuneAttnWithholdSplit,    // decode attention: 1 + a split that keeps its partial to itself (tests of the error path)
+  kTuneBlockLayout,          // token blocks: 1 = [token][column] rows, 2 = matrix-operand order, whatever their size
+  kTunePrefillAttentionRows, // prompt blocks: 1 = one attention workgroup set per token instead of the shared-tile kernel
+  kTunePrefillWalk,          // 1 = start() walks the prompt token by token (read at session create)
+  kTuneGemmBlockOff,         // 1 = blocks of more than 64 rows use gemm_rows_kernel like the smaller ones
   kTuneKnobs
 };
 int tuning(TuningKnob knob);

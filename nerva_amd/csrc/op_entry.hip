@@ -26,13 +26,15 @@ namespace {
 std::atomic<uint64_t> g_allocations{0};
 std::once_flag g_stream_once;
 hipStream_t g_stream = nullptr;
+std::atomic<bool> g_stream_ready{false};
 std::atomic<int> g_tuning[kTuneKnobs];
 constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_splits",       "prompt_splits",
                                                   "gemm_row_tiles",    "gemm_k_waves",       "gemm_block_slices",
                                                   "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                                                   "moe_down_shared_first", "gemv_workgroup_waves",
                                                   "gemv_x_registers",  "prefill_block_tokens", "gemv_rotated_walk",
-                                                  "attn_merge_spin_limit", "attn_withhold_split"};
+                                                  "attn_merge_spin_limit", "attn_withhold_split", "block_layout",
+                                                  "prefill_attention_rows", "prefill_walk", "gemm_block_off"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }
@@ -56,9 +58,12 @@ bool device_ready(int32_t *hip_error) {
 hipStream_t library_stream() {
   std::call_once(g_stream_once, [] {
     if (hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking) != hipSuccess) g_stream = nullptr;
+    g_stream_ready.store(g_stream != nullptr, std::memory_order_release);
   });
   return g_stream;
 }
+
+hipStream_t library_stream_if_created() { return g_stream_ready.load(std::memory_order_acquire) ? g_stream : nullptr; }
 
 hipStream_t resolve_stream(void *stream) {
   return stream != nullptr ? static_cast<hipStream_t>(stream) : library_stream();
@@ -298,8 +303,8 @@ int nerva_hip_timer_capture_begin(void) {
   return 0;
 }
 
-int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
-                                double *avg_replay_ns) {
+int nerva_hip_timer_capture_end_stats(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
+                                      double *avg_replay_ns, double *min_replay_ns, double *median_replay_ns) {
   if (!g_timer.capturing) return -1;
   g_timer.capturing = false;
   hipStream_t s = library_stream();
@@ -307,20 +312,42 @@ int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays,
   size_t count = 0;
   if (err == hipSuccess) err = hipGraphGetNodes(g_timer.graph, nullptr, &count);
   if (err == hipSuccess) err = hipGraphInstantiate(&g_timer.exec, g_timer.graph, nullptr, nullptr, 0);
-  if (err == hipSuccess && g_timer.e0 == nullptr) err = hipEventCreate(&g_timer.e0);
-  if (err == hipSuccess && g_timer.e1 == nullptr) err = hipEventCreate(&g_timer.e1);
+  if (timed_replays == 0 || timed_replays > 4096) err = hipErrorInvalidValue;
+  // one event in front of every replay and one behind the last: the replays stay back to back on the stream,
+  // and every one of them has a duration of its own
+  std::vector<hipEvent_t> marks(err == hipSuccess ? timed_replays + 1u : 0u, nullptr);
+  for (hipEvent_t &e : marks)
+    if (err == hipSuccess) err = hipEventCreate(&e);
   for (uint32_t i = 0; err == hipSuccess && i < warmup_replays; ++i) err = hipGraphLaunch(g_timer.exec, s);
-  if (err == hipSuccess) err = hipEventRecord(g_timer.e0, s);
-  for (uint32_t i = 0; err == hipSuccess && i < timed_replays; ++i) err = hipGraphLaunch(g_timer.exec, s);
-  if (err == hipSuccess) err = hipEventRecord(g_timer.e1, s);
-  if (err == hipSuccess) err = hipEventSynchronize(g_timer.e1);
-  float ms = 0.0f;
-  if (err == hipSuccess) err = hipEventElapsedTime(&ms, g_timer.e0, g_timer.e1);
+  for (uint32_t i = 0; err == hipSuccess && i < timed_replays; ++i) {
+    err = hipEventRecord(marks[i], s);
+    if (err == hipSuccess) err = hipGraphLaunch(g_timer.exec, s);
+  }
+  if (err == hipSuccess) err = hipEventRecord(marks[timed_replays], s);
+  if (err == hipSuccess) err = hipEventSynchronize(marks[timed_replays]);
+  std::vector<double> ns(err == hipSuccess ? timed_replays : 0u);
+  for (uint32_t i = 0; err == hipSuccess && i < timed_replays; ++i) {
+    float ms = 0.0f;
+    err = hipEventElapsedTime(&ms, marks[i], marks[i + 1]);
+    ns[i] = static_cast<double>(ms) * 1e6;
+  }
+  float total_ms = 0.0f;
+  if (err == hipSuccess) err = hipEventElapsedTime(&total_ms, marks[0], marks[timed_replays]);
+  for (hipEvent_t e : marks)
+    if (e != nullptr) (void)hipEventDestroy(e);
   timer_drop_graph();
-  if (err != hipSuccess || timed_replays == 0) return -1;
+  if (err != hipSuccess) return -1;
+  std::sort(ns.begin(), ns.end());
   if (nodes) *nodes = count;
-  if (avg_replay_ns) *avg_replay_ns = static_cast<double>(ms) * 1e6 / timed_replays;
+  if (avg_replay_ns) *avg_replay_ns = static_cast<double>(total_ms) * 1e6 / timed_replays;
+  if (min_replay_ns) *min_replay_ns = ns.front();
+  if (median_replay_ns) *median_replay_ns = ns[ns.size() / 2];
   return 0;
+}
+
+int nerva_hip_timer_capture_end(uint32_t warmup_replays, uint32_t timed_replays, uint64_t *nodes,
+                                double *avg_replay_ns) {
+  return nerva_hip_timer_capture_end_stats(warmup_replays, timed_replays, nodes, avg_replay_ns, nullptr, nullptr);
 }
 
 int nerva_hip_synth_fill_16(void *device_dst, uint32_t dtype, uint64_t seed, uint64_t tensor_id,
@@ -346,7 +373,10 @@ int nerva_hip_synth_fill_fp8_block(void *device_weights, void *device_scales, ui
 }
 
 int nerva_hip_test_set_tuning(const char *name, int32_t value) {
-  if (name == nullptr) return -1;
+  if (name == nullptr) {   // every override off
+    for (int k = 0; k < kTuneKnobs; ++k) g_tuning[k].store(0, std::memory_order_relaxed);
+    return 0;
+  }
   for (int k = 0; k < kTuneKnobs; ++k) {
     if (strcmp(name, kTuningNames[k]) == 0) {
       g_tuning[k].store(value, std::memory_order_relaxed);

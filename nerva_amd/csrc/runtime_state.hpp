@@ -15,6 +15,7 @@ namespace nv {
 // NERVA_HIP_ERROR_NO_DEVICE (mirrors the reference's stub build: native_stubs.rs:5-33).
 bool device_ready(int32_t *hip_error);
 hipStream_t library_stream();
+hipStream_t library_stream_if_created();   // null before the first library_stream() call: creates nothing
 hipStream_t resolve_stream(void *stream);
 
 hipError_t counted_malloc(void **ptr, size_t bytes);

@@ -48,8 +48,15 @@ def synth32(count, tid, std=1.0):
     return buf
 
 
+class Timing(float):
+    """Average ns per launch group; `shortest` and `median` are the shortest and the median replay of the
+    recorded graph, per group (None where single launches were timed by the host clock)."""
+    shortest = None
+    median = None
+
+
 def timed(enqueue, launches, warmup=3, replays=10):
-    """enqueue(i) issues the i-th launch group; returns average ns per group."""
+    """enqueue(i) issues the i-th launch group; returns the average ns per group as a Timing."""
     lib = abi.load()
     enqueue(0)                       # untimed: primes lazily built tables
     Device.synchronize()
@@ -60,21 +67,29 @@ def timed(enqueue, launches, warmup=3, replays=10):
         for i in range(launches):
             enqueue(i)
         Device.synchronize()
-        return (time.perf_counter() - t0) * 1e9 / launches
+        return Timing((time.perf_counter() - t0) * 1e9 / launches)
     assert lib.nerva_hip_timer_capture_begin() == 0
     for i in range(launches):
         enqueue(i)
-    nodes, ns = C.c_uint64(0), C.c_double(0.0)
-    assert lib.nerva_hip_timer_capture_end(warmup, replays, C.byref(nodes), C.byref(ns)) == 0
-    return ns.value / launches
+    nodes, ns, lo, mid = C.c_uint64(0), C.c_double(0.0), C.c_double(0.0), C.c_double(0.0)
+    assert lib.nerva_hip_timer_capture_end_stats(warmup, replays, C.byref(nodes), C.byref(ns), C.byref(lo), C.byref(mid)) == 0
+    out = Timing(ns.value / launches)
+    out.shortest, out.median = lo.value / launches, mid.value / launches
+    return out
 
 
 def report(name, variant, ns, nbytes):
-    """Prints one row and returns it: {"us", "GB/s", "frac" of the 8 TB/s peak, "bytes"}."""
+    """Prints one row and returns it: {"us" (average), "us_min", "us_median" over the replays, "GB/s" and "frac"
+    of the 8 TB/s peak (both from the average), "bytes"}."""
     gbs = nbytes / ns
-    log("%-34s %-9s %9.2f us  %8.1f GB/s  %5.1f%% of HBM peak   (ideal %.2f us)" % (
-        name, variant, ns / 1e3, gbs, 100 * gbs / PEAK, nbytes / PEAK / 1e3))
-    return {"us": round(ns / 1e3, 2), "GB/s": round(gbs, 1), "frac": round(gbs / PEAK, 4), "bytes": int(nbytes)}
+    spread = ""
+    row = {"us": round(ns / 1e3, 2), "GB/s": round(gbs, 1), "frac": round(gbs / PEAK, 4), "bytes": int(nbytes)}
+    if getattr(ns, "shortest", None) is not None:
+        row["us_min"], row["us_median"] = round(ns.shortest / 1e3, 2), round(ns.median / 1e3, 2)
+        spread = "  min %.2f  median %.2f" % (row["us_min"], row["us_median"])
+    log("%-34s %-9s %9.2f us%s  %8.1f GB/s  %5.1f%% of HBM peak   (ideal %.2f us)" % (
+        name, variant, ns / 1e3, spread, gbs, 100 * gbs / PEAK, nbytes / PEAK / 1e3))
+    return row
 
 
 def case_qproj():

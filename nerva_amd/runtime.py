@@ -39,6 +39,11 @@ class Device:
             raise ValueError("unknown tuning name %r" % name)
 
     @staticmethod
+    def reset_tuning():
+        """Every override off: the library's built-in launch shapes and modes."""
+        abi.load().nerva_hip_test_set_tuning(None, 0)
+
+    @staticmethod
     def steps_are_eager():
         """True when sessions launch a step's kernels one by one instead of replaying the captured
         graph: asked for through NERVA_HIP_EAGER_STEPS=1, or forced because a profiler is attached."""

@@ -21,3 +21,12 @@ def kat():
 
 def hx(s):
     return int(s, 16)
+
+
+@pytest.fixture(autouse=True)
+def builtin_launch_shapes():
+    """Overrides a test sets through the tuning hook never outlive it, also when it fails half way."""
+    yield
+    from nerva_amd import abi
+    if os.path.exists(abi.LIBRARY):
+        abi.load().nerva_hip_test_set_tuning(None, 0)

@@ -315,15 +315,19 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
     for name in ("attn_splits", "batch_splits", "prompt_splits", "gemm_row_tiles", "gemm_k_waves",
                  "gemm_block_slices", "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                  "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers", "prefill_block_tokens",
-                 "gemv_rotated_walk"):
+                 "gemv_rotated_walk", "attn_merge_spin_limit", "attn_withhold_split", "block_layout",
+                 "prefill_attention_rows", "prefill_walk", "gemm_block_off"):
         N.Device.set_tuning(name, 2)
         N.Device.set_tuning(name, 0)
     with pytest.raises(ValueError):
         N.Device.set_tuning("NERVA_HIP_ATTN_SPLITS", 2)
     csrc = os.path.join(ROOT, "nerva_amd", "csrc")
     src = "".join(open(os.path.join(csrc, f)).read() for f in os.listdir(csrc) if f.endswith((".hip", ".cuh", ".hpp")))
-    for knob in ("_SPLITS", "_ROW_TILES", "_K_WAVES", "_SLICES", "_MIN_TOKENS"):
+    for knob in ("_SPLITS", "_ROW_TILES", "_K_WAVES", "_SLICES", "_MIN_TOKENS", "_PREFILL", "_PREFILL_ATTN", "_BLOCK_LAYOUT",
+                 "_GEMM_BLOCK", "_SPLIT_ARENAS"):
         assert knob + '")' not in src, knob    # no getenv("NERVA_HIP_..._SPLITS") and the like
+    N.Device.set_tuning("prefill_walk", 1)
+    N.Device.reset_tuning()                     # a null name switches every override off
 
 
 def test_build_refuses_register_spills_in_kernels_that_issue_loads_by_hand():

@@ -117,8 +117,7 @@ def test_long_context_links_at_qwen3_8b_widths():
     # block prefill against the token walk on the device (different summation order in the projections)
     last_rows = [s.kv_row(l, P - 1) for l in range(2)]
     s.destroy()
-    import os
-    os.environ["NERVA_HIP_PREFILL"] = "walk"
+    N.Device.set_tuning("prefill_walk", 1)
     try:
         w = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=SEED, weight_std=0.02)
         rc, res = w.start(prompt)
@@ -129,7 +128,7 @@ def test_long_context_links_at_qwen3_8b_widths():
                 assert rel_l2(O.decode16(dt, got), O.decode16(dt, ref)) <= (2e-3 if l == 0 else chain_budget(1)), l
         w.destroy()
     finally:
-        del os.environ["NERVA_HIP_PREFILL"]
+        N.Device.set_tuning("prefill_walk", 0)
     assert rel_l2(prefill_logits, walk_logits) <= chain_budget(2)
     print("4200-token context: links (worst rel L2): %s; end-to-end logits %.2e; block prefill vs walk logits %.2e"
           % (", ".join("%s %.1e" % kv_ for kv_ in sorted(worst.items())), e2e, rel_l2(prefill_logits, walk_logits)),

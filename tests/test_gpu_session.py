@@ -566,7 +566,7 @@ PREFILL_GEOMETRIES = [
 @pytest.mark.parametrize("geom", PREFILL_GEOMETRIES)
 def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
     """start() sends the prompt through the layers in blocks of up to 64 tokens (multi-row GEMMs, one
-    attention launch per block); NERVA_HIP_PREFILL=walk keeps one prompt step per token. Same staging,
+    attention launch per block); the "prefill_walk" override keeps one prompt step per token. Same staging,
     so both agree with each other and with the oracle to the end-to-end tolerance, over three blocks."""
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = geom
     weights, omodel = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 1234, theta, qk_norm, bias)
@@ -578,9 +578,9 @@ def test_block_prefill_matches_token_walk_and_oracle(geom, monkeypatch):
     results = {}
     for mode in ("blocks", "walk"):
         if mode == "walk":
-            monkeypatch.setenv("NERVA_HIP_PREFILL", "walk")
+            N.Device.set_tuning("prefill_walk", 1)
         else:
-            monkeypatch.delenv("NERVA_HIP_PREFILL", raising=False)
+            N.Device.set_tuning("prefill_walk", 0)
         s = N.DecodeSession.create(weights, 160)
         rc, res = s.start(prompt)
         assert rc == 0 and res.hot_path_allocations == 0
@@ -785,9 +785,9 @@ def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
     outcome = {}
     for mode in ("blocks", "walk"):
         if mode == "walk":
-            monkeypatch.setenv("NERVA_HIP_PREFILL", "walk")
+            N.Device.set_tuning("prefill_walk", 1)
         else:
-            monkeypatch.delenv("NERVA_HIP_PREFILL", raising=False)
+            N.Device.set_tuning("prefill_walk", 0)
         s = N.DecodeSession.create(weights, length + 2)          # room for the prompt and three tokens
         rc, res = s.start(prompt)
         assert rc == 0 and res.kv_tokens == length

@@ -117,3 +117,22 @@ def test_build_script_lists_the_sources_that_exist():
     names = re.findall(r'"([a-z0-9_]+)"', block)
     csrc = os.path.join(ROOT, "nerva_amd", "csrc")
     assert sorted(names) == sorted(f[:-4] for f in os.listdir(csrc) if f.endswith(".hip"))
+
+
+def test_safe_wrapper_checks_every_tensor_before_the_pointer_cast():
+    """The config's validate() must compare every layer tensor with the size the dimensions imply (native code reads
+    that many elements from the pointer it is handed) and convert sizes with checked conversions; the crate's build
+    script must refuse register spills in the kernels that issue loads by hand, like nerva_amd/build.py."""
+    session = open(os.path.join(CRATE, "src", "session.rs")).read()
+    validate = session[session.index("pub fn validate("):session.index("pub fn create(")]
+    for tensor in ("w_q", "w_k", "w_v", "w_o", "w_gate", "w_up", "w_down", "rms_attn_weight", "rms_mlp_weight",
+                   "q_norm_weight", "k_norm_weight", "q_bias", "k_bias", "v_bias", "o_bias", "embeddings", "lm_head",
+                   "final_norm_weight"):
+        assert re.search(r"\b%s\b" % tensor, validate), "validate() does not look at %s" % tensor
+    assert "checked_mul" in validate and "u32::try_from" in validate
+    assert not re.search(r"\b(len\(\)|steps|self\.\w+) as u32", session), "unchecked size conversion"
+    from nerva_amd import build
+    script = open(os.path.join(CRATE, "build.rs")).read()
+    for kernel in build.HAND_ISSUED_LOADS:
+        assert '"%s"' % kernel in script
+    assert "kernel-resource-usage" in script and "ScratchSize" in script and 'SUPPORTED_ARCH: &str = "gfx950"' in script
