@@ -28,10 +28,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one gate_up launch moves at the Qwen3-8B shape (24576x4096 bf16): FETCH_SIZE + WRITE_SIZE
 # per dispatch from two `rocprofv3 --pmc` runs, each scaled by what the counter reads for a plain
 # 256 MiB copy kernel (profiles/gate_up_gemv_hbm_traffic_pmc.txt). Not measurable in-process.
-# Keyed to the launch shape the figure was measured for - (hidden, intermediate, kernel variant,
-# workgroups) as nerva_hip_gemv_launch_shape reports them - so that a changed plan reports null
-# instead of a stale number.
-GATE_UP_TRAFFIC_BYTES = {(4096, 12288, 3, 2048): 201709978}
+# Keyed to the launch the figure was measured for - (hidden, intermediate, kernel variant, workgroups,
+# rotated walk, chunks per request batch) as nerva_hip_gemv_launch_shape reports them - so that a
+# changed plan reports null instead of a stale number.
+GATE_UP_TRAFFIC_BYTES = {(4096, 12288, 3, 2048, True, 2): 201743448}
 SEED = 0x4E45525641
 WEIGHT_STD = 0.02
 
@@ -276,7 +276,7 @@ def main():
             k, ns / 1e3, paired / 1e3, per_kind[k][1] / max(ns, 1), 100 * per_kind[k][1] / max(ns, 1) / HBM_PEAK_GBS))
     dom_ns, dom_bytes = per_kind["gate_up"]
     dom_name = "gemv_fast_kernel<bf16, rmsnorm prologue, swiglu epilogue> (gate_up 24576x4096)"
-    traffic = GATE_UP_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"]) + N.gemv_launch_shape(
+    traffic = GATE_UP_TRAFFIC_BYTES.get((cfg["hidden"], cfg["intermediate"]) + N.gemv_launch_plan(
         1, 2, cfg["intermediate"], cfg["hidden"]))
     roofline = dict(bound="hbm", kernel=dom_name,
                     achieved=round(dom_bytes / dom_ns, 1), peak=HBM_PEAK_GBS, unit="GB/s",

@@ -479,8 +479,9 @@ typedef struct NervaHipGemvRequest {
 int nerva_hip_gemv(const NervaHipGemvRequest *request, void *stream, int32_t *hip_error);
 
 /* The launch shape nerva_hip_gemv (and the session's step) chooses for a request of these sizes with
- * 16-byte-aligned pointers: *kernel = 0 scalar, 1 guarded vector, 2 full vector, 3 the lean
- * production-shape kernel; *workgroups = the grid. Host arithmetic only (no device is touched):
+ * 16-byte-aligned pointers: *kernel, low four bits = 0 scalar, 1 guarded vector, 2 full vector, 3 the lean
+ * production-shape kernel; bit 4 = the lean kernel walks its rows from a rotated start; bits 8 and up = 1 KiB
+ * chunks of a row per request batch; *workgroups = the grid. Host arithmetic only (no device is touched):
  * measurements taken for one launch shape (counter profiles) are keyed to it. No counterpart. */
 int nerva_hip_gemv_launch_shape(uint32_t prologue, uint32_t epilogue, uint32_t rows, uint32_t cols,
                                 uint32_t *kernel, uint32_t *workgroups);

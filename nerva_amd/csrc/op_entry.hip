@@ -390,7 +390,8 @@ int nerva_hip_gemv_launch_shape(uint32_t prologue, uint32_t epilogue, uint32_t r
                                 uint32_t *workgroups) {
   if (prologue > 1 || epilogue > 4 || rows == 0 || cols == 0) return -1;
   const GemvPlan plan = gemv_plan(static_cast<int>(prologue), static_cast<int>(epilogue), rows, cols, true, nullptr);
-  if (kernel) *kernel = static_cast<uint32_t>(plan.mode);
+  // low four bits: the kernel variant; bit 4: the rotated walk; bits 8 and up: 1 KiB chunks per request batch
+  if (kernel) *kernel = static_cast<uint32_t>(plan.mode) | (plan.rotated ? 16u : 0u) | (static_cast<uint32_t>(plan.chunks) << 8);
   if (workgroups) *workgroups = plan.grid;
   return 0;
 }

@@ -142,12 +142,18 @@ def gemv(dtype, weights, rows, cols, *, input16=None, input_f32=None, gamma=None
         Device.synchronize()
 
 
-def gemv_launch_shape(prologue, epilogue, rows, cols):
-    """(kernel variant, workgroups) of the launch nerva_hip_gemv chooses for these sizes (host arithmetic)."""
+def gemv_launch_plan(prologue, epilogue, rows, cols):
+    """(kernel variant, workgroups, rotated walk, 1 KiB chunks per request batch) of the launch nerva_hip_gemv
+    chooses for these sizes (host arithmetic)."""
     kernel, groups = C.c_uint32(0), C.c_uint32(0)
     if abi.load().nerva_hip_gemv_launch_shape(prologue, epilogue, rows, cols, C.byref(kernel), C.byref(groups)) != 0:
         raise ValueError("no launch shape for these sizes")
-    return int(kernel.value), int(groups.value)
+    return int(kernel.value) & 15, int(groups.value), bool(kernel.value & 16), int(kernel.value) >> 8
+
+
+def gemv_launch_shape(prologue, epilogue, rows, cols):
+    """(kernel variant, workgroups) of that launch."""
+    return gemv_launch_plan(prologue, epilogue, rows, cols)[:2]
 
 
 def fp8_gemv(weights, scales, rows, cols, block_rows, block_cols, out, *, input16=None, input_f32=None,
