@@ -636,6 +636,240 @@ __global__ __launch_bounds__(PAIRS * 2 * kWave, 2) void gemm_wide_kernel(GemmRow
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Token blocks of 257..512 rows (X in operand order with 32 token tiles). What bounds the kernel above is what a
+// CU has to pull in, not its matrix cores: every workgroup of 128 weight rows fetches the whole X block from L2
+// (twice the weight bytes per launch), ten operand pieces cross the LDS port for every sixteen products, and every
+// X block is written to LDS through registers. A block of 512 tokens lets a workgroup take 256 weight rows (a
+// gate/up pair: 128 + 128) x 256 tokens - one half of the block - so that a byte of X is fetched by half as many
+// workgroups and a byte of W still by two (the two halves of a row group run on the same XCD, next to each other
+// in dispatch order: the second finds the rows in that L2):
+//   * grid: one dimension, workgroup L -> XCD L % 8 (the hardware deals them round robin), and within an XCD
+//     (unit, half) with the half running fastest; unit = (row group, K slice);
+//   * 8 waves = 4 row quarters x 2 token halves of 128, a wave holds 4 row tiles x 8 token tiles of accumulators
+//     (128 registers) and reads 4 + 8 operand pieces for 32 products;
+//   * K-blocks of 64 columns; X and W go from global memory to LDS directly (global_load_lds_dwordx4, 1 KiB a
+//     request, no registers, no LDS write instructions): X in two buffers of 32 KiB (the block in use and the next
+//     one), W in three (the W block two ahead is in flight from HBM): 160 KiB, all of a CU's LDS. A W tile is 16
+//     rows of 128 bytes; the 16-byte pieces of a row are XORed with the row number (mod 8) on the way in - a lane
+//     asks for the piece that belongs in its LDS slot - which makes the operand reads conflict-free;
+//   * one barrier per K-block: a wave waits for its own requests of this block, everyone meets (the block is
+//     complete and nobody reads the previous one any more), the requests for the block ahead go out, 64 products.
+//     The barrier is a bare s_barrier with the waits it needs written out - a fence would wait for the requests
+//     in flight - and every LDS operand read is issued by hand with a counted wait (the compiler's own
+//     bookkeeping falls back to "everything" once direct-to-LDS requests are pending).
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kDTokCap = 512;                      // token rows at most; the token stride of this kernel's partial sums
+constexpr int kDK = 64;                                 // columns per K-block
+constexpr int kDXBuf = 2 * 16 * kWave * static_cast<int>(sizeof(u32x4_t));   // one X block of a half: 2 K-steps x 16 tiles = 32 KiB
+constexpr int kDWTile = 16 * kDK * static_cast<int>(sizeof(uint16_t));       // one W tile of a block: 2 KiB
+constexpr int kDWBuf = 16 * kDWTile;                                         // the workgroup's 16 tiles: 32 KiB
+constexpr size_t kDeepLds = 2 * static_cast<size_t>(kDXBuf) + 3 * static_cast<size_t>(kDWBuf);   // 163,840 B
+#define NV_LDS_PTR(P) ((__attribute__((address_space(3))) void *)(P))
+
+template <uint32_t DT, int EPI>
+__global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams p, float *partials, uint32_t units,
+                                                                  uint32_t kslices) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int th = wave & 1, rq = wave >> 1;   // token half of the workgroup's 256, row quarter of its 256
+  const uint32_t n = lane & 15, q = lane >> 4;
+  const uint32_t cols = p.cols, T = p.tokens;
+  const uint32_t halves = (T + 255u) / 256u;
+  const uint32_t in_xcd = blockIdx.x >> 3;
+  const uint32_t half = in_xcd % halves, unit = (in_xcd / halves) * 8u + (blockIdx.x & 7u);
+  if (unit >= units) return;
+  const uint32_t group = unit / kslices, slice = unit % kslices;
+  const uint32_t kper = cols / kslices, k0 = slice * kper, nblk = kper / kDK;
+
+  // LDS tile slot s = 4 * (row quarter) + j. Plain: rows 16 s .. of the workgroup's 256. SwiGLU: j = 0, 1 the
+  // gate tiles 2 rq + j of the workgroup's 128 gate rows, j = 2, 3 their up tiles - a wave's four tiles end in
+  // the wave that runs the epilogue.
+  auto slot_row = [&](int s) -> uint32_t {
+    if constexpr (EPI == kGemmSwiglu)
+      return ((s >> 1) & 1) * p.rows + group * 128u + (2u * (s >> 2) + (s & 1)) * 16u;
+    else
+      return group * 256u + s * 16u;
+  };
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(NV_LDS_PTR(smem)));   // X buffers, then W buffers
+  // W requests of this wave: tiles 2 wave and 2 wave + 1, two requests of 8 rows x 128 bytes each. Lane (r, c) of
+  // a request asks for piece c ^ r of row r: a wave-uniform base per request and one lane offset for all.
+  const char *wsrc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int s_ = 2 * wave + (i >> 1);
+    wsrc[i] = reinterpret_cast<const char *>(p.w) +
+              (static_cast<uint64_t>(slot_row(s_) + (i & 1) * 8u) * cols + k0 + (EPI == kGemmSwiglu && ((s_ >> 1) & 1) ? p.pair_gap : 0u)) *
+                  sizeof(uint16_t);
+  }
+  const uint32_t wlane = ((lane >> 3) * cols) * static_cast<uint32_t>(sizeof(uint16_t)) + (((lane & 7) ^ (lane >> 3)) << 4);
+  // X requests of this wave: four consecutive token tiles of one K-step of the half's block
+  const uint32_t xtiles = p.x_packed;   // token tiles of the whole block per K-step (32 above 256 tokens)
+  const char *xsrc = reinterpret_cast<const char *>(p.x16) +
+                     ((static_cast<uint64_t>(k0 / 32u + (wave >> 2)) * xtiles + half * 16u + (wave & 3) * 4u) * kWave + lane) * sizeof(u32x4_t);
+  const uint64_t xstep = static_cast<uint64_t>(2u * xtiles) * kWave * sizeof(u32x4_t);   // one K-block further
+  // A operand of K-step e of the block, lane (row n, quarter q): piece 4 e + q of row n, at piece ^ (n & 7)
+  uint32_t a_off[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) a_off[e] = lds0 + 2 * kDXBuf + (4 * rq) * kDWTile + n * 128 + (((e * 4 + q) ^ (n & 7)) << 4);
+  // B operand of K-step e, token tile c of this wave's eight: piece (e * 16 + th * 8 + c) * 64 + lane of the buffer
+  uint32_t b_addr[2];
+#pragma unroll
+  for (int xb = 0; xb < 2; ++xb) b_addr[xb] = lds0 + xb * kDXBuf + ((th * 8) * kWave + lane) * static_cast<uint32_t>(sizeof(u32x4_t));
+
+  f32x4_t acc[4][8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // W block BLK -> W buffer at byte offset WOFF (wave-uniform); X block BLK -> X buffer XB
+#define NV_DP_W1(WOFF, BLK, I)                                                                      \
+  __builtin_amdgcn_global_load_lds(                                                                 \
+      reinterpret_cast<const u32x4_t *>(wsrc[I] + static_cast<uint64_t>(BLK) * (kDK * sizeof(uint16_t)) + wlane), \
+      NV_LDS_PTR(smem + 2 * kDXBuf + (WOFF) + (2 * wave + ((I) >> 1)) * kDWTile + ((I) & 1) * 1024), 16, 0, 0)
+#define NV_DP_X1(XB, BLK, I)                                                                        \
+  __builtin_amdgcn_global_load_lds(                                                                 \
+      reinterpret_cast<const u32x4_t *>(xsrc + static_cast<uint64_t>(BLK) * xstep + (I) * 1024),    \
+      NV_LDS_PTR(smem + (XB) * kDXBuf + (wave * 4 + (I)) * 1024), 16, 0, 0)
+#define NV_DP_LDS_READ(DST, ADDR, OFF) \
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(DST) : "v"(ADDR), "n"(OFF) : "memory")
+#define NV_DP_READ_B(XB, IDX) NV_DP_LDS_READ(bq[(IDX) % 3], b_addr[XB], ((((IDX) >> 3) * 16 + ((IDX) & 7)) * kWave * 16))
+#define NV_DP_READ_A(E, J) NV_DP_LDS_READ(aq[E][J], a_cur[E], (J) * kDWTile)
+  // Operand reads of a block, in issue order: bq0, aq[0][0..3], bq1; then product group i issues bq(i + 2) and,
+  // for i < 4, aq[1][i]. LDS reads return in order, so group i waits until at most this many younger reads are
+  // outstanding: (behind aq[0][3]) 3, then 4, 5, 5, 4, 3, and 2 from group 6 on, 1 and 0 for the last two.
+  // The awaited registers are in/out operands of the wait, so that their use cannot move in front of it.
+#define NV_DP_AWAIT(N_, B_) asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_) :: "memory")
+#define NV_DP_AWAIT_A(N_, B_, E_)                                                                   \
+  asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_), "+v"(aq[E_][0]), "+v"(aq[E_][1]), "+v"(aq[E_][2]), "+v"(aq[E_][3]) :: "memory")
+#define NV_DP_WAIT(IDX)                                                                             \
+  if constexpr ((IDX) == 0) NV_DP_AWAIT_A(3, bq[0], 0);                                             \
+  else if constexpr ((IDX) == 1 || (IDX) == 4) NV_DP_AWAIT(4, bq[(IDX) % 3]);                       \
+  else if constexpr ((IDX) == 2 || (IDX) == 3) NV_DP_AWAIT(5, bq[(IDX) % 3]);                       \
+  else if constexpr ((IDX) == 5) NV_DP_AWAIT(3, bq[(IDX) % 3]);                                     \
+  else if constexpr ((IDX) == 8) NV_DP_AWAIT_A(2, bq[(IDX) % 3], 1);                                \
+  else if constexpr ((IDX) == 14) NV_DP_AWAIT(1, bq[(IDX) % 3]);                                    \
+  else if constexpr ((IDX) == 15) NV_DP_AWAIT(0, bq[(IDX) % 3]);                                    \
+  else NV_DP_AWAIT(2, bq[(IDX) % 3])
+  // request slots between the products: first the next X block's four pieces, then the W block two ahead
+#define NV_DP_SLOT(IDX, XB, XEN, WEN)                                                               \
+  if constexpr ((IDX) < 4) {                                                                        \
+    if constexpr (XEN) { NV_DP_X1((XB) ^ 1, blk_ + 1u, IDX); }                                      \
+  } else if constexpr ((IDX) < 8) {                                                                 \
+    if constexpr (WEN) { NV_DP_W1(w_ahead, blk_ + 2u, (IDX) - 4); }                                 \
+  }
+#define NV_DP_ITEM(IDX, XB, XEN, WEN)                                                               \
+  if constexpr ((IDX) + 2 < 16) { NV_DP_READ_B(XB, (IDX) + 2); }                                    \
+  if constexpr ((IDX) < 4) { NV_DP_READ_A(1, IDX); }                                                \
+  NV_DP_WAIT(IDX);                                                                                  \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                     \
+      acc[j][(IDX) & 7] = mfma_k32<DT>(aq[(IDX) >> 3][j], bq[(IDX) % 3], acc[j][(IDX) & 7]);        \
+  __builtin_amdgcn_sched_barrier(0);                                                                \
+  NV_DP_SLOT(IDX, XB, XEN, WEN)                                                                     \
+  __builtin_amdgcn_sched_barrier(0)
+  // Block BLK in X buffer XB and the W buffer at w_cur. LAST: nothing younger than this block's requests is in
+  // flight; otherwise the four W requests of the block after it are.
+#define NV_DP_BLOCK(BLK, XB, LAST, XEN, WEN)                                                        \
+  do {                                                                                              \
+    const uint32_t blk_ = (BLK);                                                                    \
+    if constexpr (LAST) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");               \
+    else asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");                              \
+    const uint32_t a_cur[2] = {a_off[0] + w_cur, a_off[1] + w_cur};                                 \
+    const uint32_t w_ahead = w_cur >= static_cast<uint32_t>(kDWBuf) ? w_cur - kDWBuf : w_cur + 2 * kDWBuf;   /* (b + 2) % 3 */ \
+    u32x4_t aq[2][4], bq[3];                                                                        \
+    NV_DP_READ_B(XB, 0);                                                                            \
+    NV_DP_READ_A(0, 0);                                                                             \
+    NV_DP_READ_A(0, 1);                                                                             \
+    NV_DP_READ_A(0, 2);                                                                             \
+    NV_DP_READ_A(0, 3);                                                                             \
+    NV_DP_READ_B(XB, 1);                                                                            \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    NV_DP_ITEM(0, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(1, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(2, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(3, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(4, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(5, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(6, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(7, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(8, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(9, XB, XEN, WEN);                                                                    \
+    NV_DP_ITEM(10, XB, XEN, WEN);                                                                   \
+    NV_DP_ITEM(11, XB, XEN, WEN);                                                                   \
+    NV_DP_ITEM(12, XB, XEN, WEN);                                                                   \
+    NV_DP_ITEM(13, XB, XEN, WEN);                                                                   \
+    NV_DP_ITEM(14, XB, XEN, WEN);                                                                   \
+    NV_DP_ITEM(15, XB, XEN, WEN);                                                                   \
+    w_cur = w_cur == static_cast<uint32_t>(2 * kDWBuf) ? 0u : w_cur + kDWBuf;                        \
+  } while (0)
+
+  // start: X block 0, W blocks 0 and 1, in the order they are awaited in (nblk is even and at least 2)
+  uint32_t w_cur = 0;   // byte offset of the W buffer of the block being multiplied (wave-uniform)
+  {
+    const uint32_t blk_ = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) NV_DP_X1(0, blk_, i);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) NV_DP_W1(0u, 0u, i);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) NV_DP_W1(static_cast<uint32_t>(kDWBuf), 1u, i);
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t blk = 0;
+  for (; blk + 2 < nblk; blk += 2) {
+    NV_DP_BLOCK(blk, 0, false, true, true);
+    NV_DP_BLOCK(blk + 1, 1, false, true, true);
+  }
+  NV_DP_BLOCK(blk, 0, false, true, false);
+  NV_DP_BLOCK(blk + 1, 1, true, false, false);
+#undef NV_DP_W1
+#undef NV_DP_X1
+#undef NV_DP_LDS_READ
+#undef NV_DP_READ_B
+#undef NV_DP_READ_A
+#undef NV_DP_AWAIT
+#undef NV_DP_AWAIT_A
+#undef NV_DP_WAIT
+#undef NV_DP_SLOT
+#undef NV_DP_ITEM
+#undef NV_DP_BLOCK
+
+  // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
+  if (kslices == 1) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t t = half * 256u + (th * 8 + c) * 16u + n;
+      if (t < T) {
+        if constexpr (EPI == kGemmSwiglu) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) block_epilogue<DT, EPI>(p, t, slot_row(4 * rq + j) + q * 4u, acc[j][c], acc[j + 2][c]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) block_epilogue<DT, EPI>(p, t, slot_row(4 * rq + j) + q * 4u, acc[j][c], acc[j][c]);
+        }
+      }
+    }
+  } else {
+    const uint32_t wrows = EPI == kGemmSwiglu ? 2u * p.rows : p.rows;
+    float *part = partials + static_cast<uint64_t>(slice) * kDTokCap * wrows;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t t = half * 256u + (th * 8 + c) * 16u + n;
+      if (t < T) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<float4 *>(part + static_cast<uint64_t>(t) * wrows + slot_row(4 * rq + j) + q * 4u) =
+              make_float4(acc[j][c][0], acc[j][c][1], acc[j][c][2], acc[j][c][3]);
+      }
+    }
+  }
+}
+
 template <uint32_t DT, int EPI, int PAIRS>
 hipError_t launch_wide_pairs(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
   constexpr uint32_t wg_rows = wide_wg_rows(EPI, PAIRS);
@@ -651,6 +885,47 @@ hipError_t launch_wide_pairs(const GemmRowsParams &p, float *partials, uint32_t 
   hipLaunchKernelGGL((gemm_wide_kernel<DT, EPI, PAIRS>), dim3(p.rows / wg_rows, kslices), dim3(PAIRS * 2 * kWave), lds, stream, p,
                      partials);
   return hipGetLastError();
+}
+
+// Blocks of 257..512 rows (gemm_deep_kernel): workgroups of 256 rows (a gate/up pair: 128 + 128) x 256 tokens.
+inline uint32_t deep_wg_rows(int epilogue) { return epilogue == kGemmSwiglu ? 128u : 256u; }
+
+template <uint32_t DT, int EPI>
+hipError_t launch_deep(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+  static std::once_flag once;
+  static hipError_t raised = hipSuccess;
+  std::call_once(once, [] {
+    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_deep_kernel<DT, EPI>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDeepLds));
+  });
+  if (raised != hipSuccess) return raised;
+  const uint32_t units = p.rows / deep_wg_rows(EPI) * kslices, halves = (p.tokens + 255u) / 256u;
+  hipLaunchKernelGGL((gemm_deep_kernel<DT, EPI>), dim3((units + 7u) / 8u * 8u * halves), dim3(8 * kWave), kDeepLds, stream, p,
+                     partials, units, kslices);
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess && kslices > 1) {
+    if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
+      hipLaunchKernelGGL((gemm_finish_norm_kernel<DT>), dim3(p.tokens), dim3(kFinNormThreads), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kDTokCap);
+    } else {
+      const uint32_t threads = p.rows / 4u * p.tokens;
+      hipLaunchKernelGGL((gemm_block_finish_kernel<DT, EPI>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, p,
+                         static_cast<const float *>(partials), kslices, kDTokCap);
+    }
+    err = hipGetLastError();
+  }
+  return err;
+}
+
+template <uint32_t DT>
+hipError_t launch_deep_dt(int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
+  float *partials = static_cast<float *>(p.workspace);
+  switch (epilogue) {
+    case kGemmF32: return launch_deep<DT, kGemmF32>(p, partials, kslices, stream);
+    case kGemmResidual: return launch_deep<DT, kGemmResidual>(p, partials, kslices, stream);
+    case kGemmSwiglu: return launch_deep<DT, kGemmSwiglu>(p, partials, kslices, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <uint32_t DT, int EPI>
@@ -751,19 +1026,38 @@ uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t t
   return slices;
 }
 
+// Blocks of 257..512 rows: K slices of gemm_deep_kernel, or 0 where it does not take the shape. Enough workgroups
+// (row groups x 2 token halves x slices) for three quarters of the CUs, each slice an even number of K-blocks, the
+// partial sums within the workspace.
+uint32_t gemm_deep_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
+  if (tokens <= kWTokCap || tokens > kDTokCap || rows % deep_wg_rows(epilogue) != 0 || cols % (2u * kDK) != 0) return 0;
+  const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
+  const uint32_t groups = rows / deep_wg_rows(epilogue);
+  uint32_t slices = 1;
+  const int want = tuning(kTuneGemmBlockSlices);
+  if (want > 0 && cols % (static_cast<uint32_t>(want) * 2u * kDK) == 0) {
+    slices = static_cast<uint32_t>(want);
+  } else {
+    while (epilogue != kGemmSwiglu && groups * 2u * slices < 192u && slices < 8u && cols % (slices * 2u * 2u * kDK) == 0) slices *= 2u;
+  }
+  while (slices > 1 && static_cast<uint64_t>(slices) * kDTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
+  return slices;
+}
+
 bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes) {
   if (epilogue != kGemmResidual || x_packed == 0 || rows % 4 != 0 ||
       rows > static_cast<uint32_t>(kFinNormThreads * kFinNormPerLane * 4))
     return false;
-  // wherever a launch of its own adds the K slices: the wide kernel's, or the shared-X kernel's for smaller blocks
+  // wherever a launch of its own adds the K slices: the deep or the wide kernel's, or the shared-X kernel's for smaller blocks
+  if (tokens > kWTokCap) return gemm_deep_slices(epilogue, rows, cols, tokens, workspace_bytes) > 1;
   if (tokens > kBTokCap) return gemm_wide_slices(epilogue, rows, cols, tokens, workspace_bytes) > 1;
   return gemm_block_plan(epilogue, rows, cols, tokens, workspace_bytes).kslices > 1;
 }
 
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max) {
-  // room for 8 slices of the widest plain projection (or 2 of a gate/up pair of that width) at the wide kernel's
+  // room for 8 slices of the widest plain projection (or 2 of a gate/up pair of that width) at the deep kernel's
   // token stride
-  return static_cast<uint64_t>(8) * kWTokCap * rows_max * sizeof(float);
+  return static_cast<uint64_t>(8) * kDTokCap * rows_max * sizeof(float);
 }
 
 hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
@@ -772,6 +1066,15 @@ hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &
   if (kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
   if (dtype == kBF16) return launch_wide_dt<kBF16>(epilogue, p, kslices, stream);
   if (dtype == kF16) return launch_wide_dt<kF16>(epilogue, p, kslices, stream);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_gemm_deep(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
+  if (kslices == 0 || p.x_packed != gemm_packed_tiles(p.tokens) || p.tokens <= kWTokCap || p.tokens > kDTokCap)
+    return hipErrorInvalidValue;
+  if (kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
+  if (dtype == kBF16) return launch_deep_dt<kBF16>(epilogue, p, kslices, stream);
+  if (dtype == kF16) return launch_deep_dt<kF16>(epilogue, p, kslices, stream);
   return hipErrorInvalidValue;
 }
 

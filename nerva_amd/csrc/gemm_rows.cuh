@@ -24,6 +24,7 @@ namespace nv {
 
 constexpr uint32_t kGemmMaxTokens = 128;       // token rows of a block in any layout
 constexpr uint32_t kGemmWideMaxTokens = 256;   // token rows of a block in operand order, where gemm_wide_slices takes the shape
+constexpr uint32_t kGemmDeepMaxTokens = 512;   // ... where gemm_deep_slices takes the shape
 
 // Operand order of a block of token rows X[t][k] (16-bit), the layout the multi-row GEMM reads fastest:
 // for every K-step of 32 columns and every tile of 16 tokens the 64 lanes' 16-byte pieces in lane order,
@@ -34,7 +35,7 @@ __host__ __device__ __forceinline__ uint64_t gemm_x_packed_index(uint32_t tiles,
 }
 // Token tiles the GEMM works with for a block of `tokens` rows (its X buffer in operand order has as many).
 __host__ __device__ __forceinline__ uint32_t gemm_packed_tiles(uint32_t tokens) {
-  return tokens > 128u ? 16u : tokens > 64u ? 8u : tokens > 32u ? 4u : 2u;
+  return tokens > 256u ? 32u : tokens > 128u ? 16u : tokens > 64u ? 8u : tokens > 32u ? 4u : 2u;
 }
 enum : int { kGemmF32 = 0, kGemmResidual = 1, kGemmSwiglu = 2 };
 
@@ -86,6 +87,10 @@ hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams 
 // (rows a multiple of 128, gate/up pairs of 64; cols a multiple of 512 per slice). launch_gemm_rows uses it by itself.
 uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
 hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
+// Blocks of 257..kGemmDeepMaxTokens rows in operand order (32 token tiles): the same for the kernel that takes
+// 256 rows x 256 tokens per workgroup (rows a multiple of 256, a gate/up pair of 128, cols of 128).
+uint32_t gemm_deep_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
+hipError_t launch_gemm_deep(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
 // Whether launch_gemm_rows honours GemmRowsParams::norm_gamma for this shape (a K-sliced residual projection of a
 // wide block, rows a multiple of 4 and at most 16384); otherwise the caller normalises with launch_rmsnorm_rows.
 bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes);

@@ -299,11 +299,14 @@ bool gemm_rows_supported(uint32_t rows, uint32_t cols, uint32_t tokens) {
 
 hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &p, hipStream_t stream) {
   // more than kGemmMaxTokens rows: only in operand order and only where the kernel for wide blocks takes the shape
-  const uint32_t wide_slices = p.tokens > kGemmMaxTokens && p.x_packed != 0
+  const uint32_t wide_slices = p.tokens > kGemmMaxTokens && p.tokens <= kGemmWideMaxTokens && p.x_packed != 0
                                    ? gemm_wide_slices(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0)
                                    : 0u;
+  const uint32_t deep_slices = p.tokens > kGemmWideMaxTokens && p.x_packed != 0
+                                   ? gemm_deep_slices(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0)
+                                   : 0u;
   if (p.w == nullptr || p.x16 == nullptr) return hipErrorInvalidValue;
-  if (wide_slices == 0 && !gemm_rows_supported(p.rows, p.cols, p.tokens)) return hipErrorInvalidValue;
+  if (wide_slices == 0 && deep_slices == 0 && !gemm_rows_supported(p.rows, p.cols, p.tokens)) return hipErrorInvalidValue;
   if (!aligned16(p.w) || !aligned16(p.x16)) return hipErrorInvalidValue;
   if ((epilogue == kGemmF32 || epilogue == kGemmResidual) && p.out_f32 == nullptr) return hipErrorInvalidValue;
   if (epilogue == kGemmResidual && p.residual == nullptr) return hipErrorInvalidValue;
@@ -316,6 +319,7 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
   if (p.norm_gamma != nullptr &&   // a fused norm only where the shape has one; never silently dropped
       (p.norm_out16 == nullptr || !gemm_rows_fuses_norm(epilogue, p.rows, p.cols, p.tokens, p.x_packed, p.workspace != nullptr ? p.workspace_bytes : 0)))
     return hipErrorInvalidValue;
+  if (deep_slices != 0) return launch_gemm_deep(dtype, epilogue, p, deep_slices, stream);
   if (wide_slices != 0) return launch_gemm_wide(dtype, epilogue, p, wide_slices, stream);
   if (p.x_packed != 0) {   // blocks in operand order: the kernel that shares X through LDS, where its plan takes the shape
     const GemmBlockPlan plan = gemm_block_plan(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0);

@@ -291,7 +291,7 @@ def argmax_static(logits_buf, count, token_buf):
 
 def gemm_operand_slots(tokens):
     """Token slots of a buffer in matrix-operand order for a block of `tokens` rows."""
-    return 32 if tokens <= 32 else 64 if tokens <= 64 else 128 if tokens <= 128 else 256
+    return 32 if tokens <= 32 else 64 if tokens <= 64 else 128 if tokens <= 128 else 256 if tokens <= 256 else 512
 
 
 def gemm_operand_order(x, tokens=None):
@@ -316,7 +316,8 @@ def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None
               workspace=None):
     """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once); up to 256 rows
     with the input in operand order where the kernel for wide blocks takes the shape (rows a multiple of 128,
-    gate/up pairs of 64, cols of 512).
+    gate/up pairs of 64, cols of 512); up to 512 where the kernel with 256 x 256 workgroup tiles does (rows a
+    multiple of 256, gate/up pairs of 128, cols of 128).
     `workspace`: optional DeviceBuffer of gemm_rows_workspace_bytes(rows) for the K-sliced large-block kernels."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()

@@ -943,10 +943,13 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
                                                (4096, 12288, 128), (192, 2048, 17), (64, 2048, 33), (4096, 4096, 32),
                                                (6144, 4096, 48), (4096, 12288, 64),
                                                (128, 2048, 129), (256, 4096, 200), (4096, 4096, 256), (6144, 4096, 255),
-                                               (4096, 12288, 256), (192, 2048, 140)])
+                                               (4096, 12288, 256), (192, 2048, 140),
+                                               (256, 2048, 257), (512, 4096, 300), (4096, 4096, 512), (6144, 4096, 511),
+                                               (4096, 12288, 512), (256, 1024, 400)])
 def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     """More than 16 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
-    X from LDS (2, 4, 8 or - blocks of 129..256 rows, three or four wave pairs sharing their W tiles - 16 token tiles). Every token
+    X from LDS (2, 4, 8 or - blocks of 129..256 rows, three or four wave pairs sharing their W tiles - 16 token tiles;
+    blocks of 257..512 rows, 256 weight rows x 256 tokens a workgroup, W and X straight into LDS - 32). Every token
     row equals the oracle's GEMV of that row; bias + residual + rounding on top."""
     dtype = BF16
     rng = np.random.default_rng(rows + cols + tokens)
@@ -978,7 +981,8 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
 
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
-                                                 (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200)])
+                                                 (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200),
+                                                 (128, 2048, 257), (256, 1024, 512), (12288, 4096, 500)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
