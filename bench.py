@@ -205,8 +205,8 @@ def main():
     ap.add_argument("--batch-sessions", type=int, default=32,
                     help="sessions advanced together in the shared-weights leg (0 = skip it)")
     ap.add_argument("--batch-steps", type=int, default=24)
-    ap.add_argument("--prefill-block", type=int, default=0, choices=(0, 128, 256),
-                    help="prompt block size (0 = the session's choice: 256 tokens at these widths)")
+    ap.add_argument("--prefill-block", type=int, default=0, choices=(0, 128, 256, 512),
+                    help="prompt block size (0 = the session's choice: 512 tokens at these widths)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also launch one plain copy kernel of this size (memory-counter calibration runs)")
     args = ap.parse_args()
@@ -220,8 +220,8 @@ def main():
     if rc != 0:
         log("no usable GPU (hip_error=%d): the HIP path cannot run, and there is no CPU fallback" % smoke.hip_error)
         sys.exit(1)
-    if args.prefill_block == 128:
-        N.Device.set_tuning("prefill_block_tokens", 128)
+    if args.prefill_block in (128, 256):
+        N.Device.set_tuning("prefill_block_tokens", args.prefill_block)
     cfg = dict(N.Qwen3_8B)
     cfg["layers"] = args.layers
     max_ctx = args.prompt + args.warmup + args.steps + min(args.steps, 128) + 16   # + the CPU leg's parity token

@@ -746,8 +746,8 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
  * (1: the lean GEMV's exact start-up waits wherever they can run, 2: nowhere), "moe_down_shared_first" (2: the
  * MoE down launch walks the shared expert last instead of first), "gemv_workgroup_waves" (4|16: waves per
  * workgroup of every lean GEMV launch), "gemv_x_registers" (2: the lean GEMV never keeps the input vector in
- * registers), "prefill_block_tokens" (128: sessions created afterwards prefill in 128-token blocks even where
- * the 256-token blocks apply), "gemv_rotated_walk" (2: the lean GEMV never walks its rows from a rotated
+ * registers), "prefill_block_tokens" (128 | 256: sessions created afterwards prefill in blocks of at most
+ * that many tokens even where larger blocks apply), "gemv_rotated_walk" (2: the lean GEMV never walks its rows from a rotated
  * start), "attn_merge_spin_limit" and "attn_withhold_split" (the bounded wait of the decode attention's split
  * merge: polls before it gives up; 1 + the split that keeps its partial to itself), and the comparison modes
  * "block_layout" (1: token blocks as [token][column] rows, 2: in matrix-operand order, whatever their size),

@@ -145,7 +145,7 @@ struct NervaHipHfDecodeSequenceSession {
   uint64_t pattn_ws_stride = 0;
   char *pgemm_ws = nullptr;        // partial sums of the K-sliced projections of a prompt block
   uint64_t pgemm_ws_bytes = 0;
-  uint32_t prefill_block_tokens = kGemmMaxTokens;   // tokens per prompt block: 256 where every projection has the kernel for it
+  uint32_t prefill_block_tokens = kGemmMaxTokens;   // tokens per prompt block: 512 or 256 where every projection has the kernel for it
   SamplerDev sampler{};            // normalised configuration of the active sequence
   SamplerDev *sampler_dev = nullptr;
   uint64_t *sampler_keys = nullptr;
@@ -1040,7 +1040,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const uint64_t off_attn_plan = c.take(attn_plan_bytes(kAttnMaxSplits));
   const uint64_t off_attn_tagged = c.take(attn_step_workspace_bytes(s->heads));
   const uint64_t off_sample_ws = c.take(sample_workspace_bytes());
-  const uint64_t pT = kGemmWideMaxTokens;
+  const uint64_t pT = kGemmDeepMaxTokens;
   const uint64_t off_px = c.take(pT * H * 4);
   const uint64_t off_pr = c.take(pT * H * 4);
   const uint64_t off_pqkv = c.take(pT * (A + 2 * KV) * 4);
@@ -1132,15 +1132,22 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->pattn_ws_stride = pattn_ws_stride;
   s->pgemm_ws = s->arena + off_pgemm_ws;
   s->pgemm_ws_bytes = pgemm_ws_bytes;
-  // 256-token prompt blocks where all four projections of a layer have the kernel for them (twice the tokens per
-  // weight byte): Qwen3-8B widths qualify; other widths keep 128-token blocks.
-  const uint32_t wideT = kGemmWideMaxTokens;
-  const bool wide = gemm_wide_slices(kGemmF32, static_cast<uint32_t>(A + 2 * KV), s->hidden, wideT, pgemm_ws_bytes) != 0 &&
-                    gemm_wide_slices(kGemmResidual, s->hidden, static_cast<uint32_t>(A), wideT, pgemm_ws_bytes) != 0 &&
-                    gemm_wide_slices(kGemmSwiglu, s->intermediate, s->hidden, wideT, pgemm_ws_bytes) != 0 &&
-                    gemm_wide_slices(kGemmResidual, s->hidden, s->intermediate, wideT, pgemm_ws_bytes) != 0;
-  s->prefill_block_tokens =
-      wide && block_operand_tiles(wideT) != 0 && tuning(kTunePrefillBlockTokens) != 128 ? wideT : kGemmMaxTokens;
+  // Prompt blocks of 512 tokens where all four projections of a layer have the kernel for them (256 weight rows x
+  // 256 tokens a workgroup: half the X bytes per product of the 256-token kernel), else of 256 tokens where they
+  // have that kernel (twice the tokens per weight byte of the 128-token one): Qwen3-8B widths qualify for both;
+  // other widths keep 128-token blocks. The "prefill_block_tokens" override caps the choice at 128 or 256.
+  const auto all_four = [&](uint32_t (*slices)(int, uint32_t, uint32_t, uint32_t, uint64_t), uint32_t tokens) {
+    return slices(kGemmF32, static_cast<uint32_t>(A + 2 * KV), s->hidden, tokens, pgemm_ws_bytes) != 0 &&
+           slices(kGemmResidual, s->hidden, static_cast<uint32_t>(A), tokens, pgemm_ws_bytes) != 0 &&
+           slices(kGemmSwiglu, s->intermediate, s->hidden, tokens, pgemm_ws_bytes) != 0 &&
+           slices(kGemmResidual, s->hidden, s->intermediate, tokens, pgemm_ws_bytes) != 0;
+  };
+  const int block_cap = tuning(kTunePrefillBlockTokens);
+  const bool wide = block_cap != 128 && block_operand_tiles(kGemmWideMaxTokens) != 0 && all_four(gemm_wide_slices, kGemmWideMaxTokens);
+  // (a prompt's last block can have any size: 512-token blocks only where the 256-token kernel takes the rest)
+  const bool deep = wide && block_cap != 256 && block_operand_tiles(kGemmDeepMaxTokens) != 0 &&
+                    all_four(gemm_deep_slices, kGemmDeepMaxTokens) && all_four(gemm_deep_slices, kGemmWideMaxTokens + 1);
+  s->prefill_block_tokens = deep ? kGemmDeepMaxTokens : wide ? kGemmWideMaxTokens : kGemmMaxTokens;
   s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
   s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
   // ("prefill_walk" override = 1, read here: one prompt step per token where prompt blocks would be possible)

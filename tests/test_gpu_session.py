@@ -773,7 +773,7 @@ def test_batch_advance_one_eligibility_and_reasons():
         s.destroy()
 
 
-@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65, 66, 129, 130, 257, 258, 300])
+@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65, 66, 129, 130, 257, 258, 300, 513, 514, 700])
 def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
     """Prompt lengths around the prefill block sizes (the last prompt token always goes through the
     ordinary head step, so length - 1 tokens are prefilled in blocks): logits, first token and K/V
@@ -809,18 +809,19 @@ def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
 
 
 def test_prefill_block_size_changes_only_the_block_boundaries():
-    """A session whose four projections have the kernel for wide blocks prefills 256 tokens at a time; the hook
-    "prefill_block_tokens" = 128 keeps the 128-token blocks. Same arithmetic per token either way: logits, K/V rows
-    and the first tokens of a 600-token prompt agree to the end-to-end tolerance."""
+    """A session whose four projections have the kernels for them prefills 512 tokens at a time (256 where only the
+    kernel for those blocks takes its widths); the hook "prefill_block_tokens" = 256 or 128 keeps the smaller
+    blocks. Same arithmetic per token either way: logits, K/V rows and the first tokens of a 600-token prompt agree
+    to the end-to-end tolerance."""
     dtype, hidden, heads, kv, hd, inter, vocab, layers, theta, qk_norm, bias = GEOMETRIES[5]
     weights, _ = random_model(dtype, hidden, heads, kv, hd, inter, vocab, layers, 99, theta, qk_norm, bias)
     prompt = np.random.default_rng(600).integers(0, vocab, 600).astype(np.uint32)
     outcome = {}
     try:
-        for block in (0, 128):
+        for block in (0, 256, 128):
             N.Device.set_tuning("prefill_block_tokens", block)
             s = N.DecodeSession.create(weights, 608)
-            assert s.create_result.prefill_chunk_tokens == (128 if block == 128 else 256)
+            assert s.create_result.prefill_chunk_tokens == (block if block else 512)
             rc, res = s.start(prompt)
             assert rc == 0 and res.kv_tokens == 600 and res.hot_path_allocations == 0
             logits = s.logits()
@@ -831,13 +832,15 @@ def test_prefill_block_size_changes_only_the_block_boundaries():
             s.destroy()
     finally:
         N.Device.set_tuning("prefill_block_tokens", 0)
-    (la, ra, ta), (lb, rb, tb) = outcome[0], outcome[128]
-    assert rel_l2(la, lb) <= E2E_REL_L2
-    for (ka, va), (kb, vb) in zip(ra, rb):
-        assert rel_l2(O.decode16(dtype, ka), O.decode16(dtype, kb)) <= E2E_REL_L2
-        assert rel_l2(O.decode16(dtype, va), O.decode16(dtype, vb)) <= E2E_REL_L2
-    top = np.sort(lb)
-    assert ta[0] == tb[0] or top[-1] - top[-2] < E2E_REL_L2 * np.max(np.abs(lb))
+    lb, rb, tb = outcome[128]
+    for other in (0, 256):
+        la, ra, ta = outcome[other]
+        assert rel_l2(la, lb) <= E2E_REL_L2
+        for (ka, va), (kb, vb) in zip(ra, rb):
+            assert rel_l2(O.decode16(dtype, ka), O.decode16(dtype, kb)) <= E2E_REL_L2
+            assert rel_l2(O.decode16(dtype, va), O.decode16(dtype, vb)) <= E2E_REL_L2
+        top = np.sort(lb)
+        assert ta[0] == tb[0] or top[-1] - top[-2] < E2E_REL_L2 * np.max(np.abs(lb))
 
 
 def test_batch_advance_one_fills_contexts_to_the_last_slot():
