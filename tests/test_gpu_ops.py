@@ -979,6 +979,35 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     assert np.array_equal(O.encode16(dtype, got), O.encode16(dtype, got.astype(np.float32)))
 
 
+@pytest.mark.parametrize("tokens", [200, 257, 512])
+def test_gemm_rows_large_blocks_in_f16(tokens):
+    """The kernels for blocks of 129..256 and of 257..512 rows with f16 operands (the other cases of this family
+    run in bf16): every token row against the oracle's GEMV, plain and as a gate/up pair."""
+    dtype, rows, cols = F16, 512, 2048
+    rng = np.random.default_rng(tokens)
+    w = O.encode16(dtype, rng.normal(0, 0.05, (rows, cols)))
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, cols)))
+    packed, _ = N.gemm_operand_order(x)
+    ws = N.DeviceBuffer(N.gemm_rows_workspace_bytes(rows))
+    dw, dx = dev(w), dev(packed)
+    y = N.DeviceBuffer.zeros(tokens * rows * 4)
+    N.gemm_rows(dtype, dw, rows, cols, tokens, dx, epilogue=0, out_f32=y, input_operand_order=True, workspace=ws)
+    got = y.numpy(np.float32).reshape(tokens, rows)
+    picks = sorted({0, 1, 127, 128, tokens // 2, tokens - 2, tokens - 1})
+    ref = {t: O.gemv_x16(dtype, w, x[t]) for t in picks}
+    assert max(rel_l2(got[t], ref[t]) for t in picks) <= REL_L2
+    inter = rows // 2
+    out = N.DeviceBuffer.zeros(N.gemm_operand_slots(tokens) * inter * 2)
+    N.gemm_rows(dtype, dw, inter, cols, tokens, dx, epilogue=2, out16=out, input_operand_order=True,
+                output16_operand_order=True)
+    _, oidx = N.gemm_operand_order(np.zeros((tokens, inter), np.uint16))
+    act = O.decode16(dtype, out.numpy(np.uint16)[oidx]).reshape(tokens, inter)
+    for t in picks:
+        g, u = ref[t][:inter].astype(np.float64), ref[t][inter:].astype(np.float64)
+        want = O.decode16(dtype, O.encode16(dtype, (g / (1.0 + np.exp(-g)) * u).astype(np.float32)))
+        assert rel_l2(act[t], want) <= 4e-3
+
+
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
                                                  (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200),
