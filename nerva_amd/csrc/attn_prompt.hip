@@ -7,10 +7,11 @@
 //
 // gfx950 mapping (head_dim 128, G = heads / kv_heads in {1, 2, 4, 8}): the 16-column matrix-core tile
 // of the decode kernel holds the G query heads of ONE token as hi/lo column pairs and leaves the
-// rest of its columns empty; here a wave fills all 16 columns with 8 (token, head) pairs - 8 / G tokens
-// of the kv head's G query heads - so a wave is the decode kernel's tile step (attn_tile) for eight
-// "virtual heads", with the causal limit n_keys chosen per column. The 8 waves of a workgroup take
-// 8 * 8 / G consecutive tokens and walk the SAME tiles: a tile (4 KiB of K, 4 KiB of V) is requested once
+// rest of its columns empty; here a wave fills all 16 columns with 16 (token, head) pairs - 16 / G tokens
+// of the kv head's G query heads - and the hi and lo halves of a query (and of a tile's probabilities) are
+// two products into the same accumulators (attn_tile_wide), with the causal limit n_keys chosen per column.
+// The 8 waves of a workgroup take 8 * 16 / G consecutive tokens and walk the SAME tiles: a tile (4 KiB of K,
+// 4 KiB of V) is requested once
 // by the workgroup - one 16-byte piece per lane - parked in LDS (two stages, one barrier per tile) and
 // read back by every wave as matrix operands. Grid (kv head, split of the prefix, token group); split
 // partials go to the per-token workspaces the decode kernel uses and a small second launch merges them.
@@ -26,7 +27,7 @@ namespace {
 using namespace attn;
 
 constexpr int kPW = 8;    // waves per workgroup
-constexpr int kVG = 8;    // (token, head) pairs per wave: 8 hi + 8 lo columns
+constexpr int kVG = 16;   // (token, head) pairs per wave: one per column of the matrix-core tile
 
 // Split geometry of a token group, the same on both launches: tiles per split, active splits.
 __device__ __forceinline__ void prompt_splits(uint32_t last_pos, uint32_t S, uint32_t &bps, uint32_t &active, uint32_t &nblk) {
@@ -62,50 +63,56 @@ __global__ __launch_bounds__(kPW *kWave) void attn_prompt_kernel(AttnParams p) {
   // ---- this wave's eight (token, head) pairs: bias, norm, rotation -> f32 q in LDS
   const uint32_t wave_first = group_first + wave * kTokensPerWave;   // may lie past the block: clamped, never stored
   // (every input of all eight requested first, unconditionally: one round trip instead of eight)
-  float x0[kVG], x1[kVG], rc[kVG], rs[kVG];
-  uint16_t qb0[kVG], qb1[kVG];
   const bool has_bias = p.q_bias != nullptr, has_gamma = p.q_norm != nullptr, has_rope = p.rope_freq != nullptr;
   const uint16_t *bias_base = has_bias ? p.q_bias : p.k_cache;    // any readable address when unused
   const float *rope_base = has_rope ? p.rope_cs : p.qkv;
   const uint32_t rope_stride = has_rope ? p.rope_token_stride : 0u;
-#pragma unroll
-  for (int vh = 0; vh < kVG; ++vh) {
-    const uint32_t tok = min(wave_first + vh / G, T - 1);
-    const uint32_t h = kvh * G + vh % G;
-    const float *src = p.qkv + static_cast<uint64_t>(tok) * p.qkv_token_stride + h * kHD;
-    x0[vh] = src[lane];
-    x1[vh] = src[lane + 64];
-    qb0[vh] = bias_base[h * kHD + lane];
-    qb1[vh] = bias_base[h * kHD + lane + 64];
-    rc[vh] = rope_base[static_cast<uint64_t>(tok) * rope_stride + lane];
-    rs[vh] = rope_base[static_cast<uint64_t>(tok) * rope_stride + 64 + lane];
-  }
   const uint16_t *gamma_base = has_gamma ? p.q_norm : p.k_cache;
   const float g0 = dec16<DT>(gamma_base[lane]), g1 = dec16<DT>(gamma_base[lane + 64]);
 #pragma unroll
-  for (int vh = 0; vh < kVG; ++vh)
-    prep_head128_core<DT>(x0[vh], x1[vh], has_bias, dec16<DT>(qb0[vh]), dec16<DT>(qb1[vh]), has_gamma, g0, g1, has_rope,
-                          rc[vh], rs[vh], p.eps, lane, q_s[wave][vh], nullptr);
+  for (int part = 0; part < kVG / 8; ++part) {   // eight pairs at a time: their inputs in one round trip
+    float x0[8], x1[8], rc[8], rs[8];
+    uint16_t qb0[8], qb1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int vh = part * 8 + i;
+      const uint32_t tok = min(wave_first + vh / G, T - 1);
+      const uint32_t h = kvh * G + vh % G;
+      const float *src = p.qkv + static_cast<uint64_t>(tok) * p.qkv_token_stride + h * kHD;
+      x0[i] = src[lane];
+      x1[i] = src[lane + 64];
+      qb0[i] = bias_base[h * kHD + lane];
+      qb1[i] = bias_base[h * kHD + lane + 64];
+      rc[i] = rope_base[static_cast<uint64_t>(tok) * rope_stride + lane];
+      rs[i] = rope_base[static_cast<uint64_t>(tok) * rope_stride + 64 + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      prep_head128_core<DT>(x0[i], x1[i], has_bias, dec16<DT>(qb0[i]), dec16<DT>(qb1[i]), has_gamma, g0, g1, has_rope,
+                            rc[i], rs[i], p.eps, lane, q_s[wave][part * 8 + i], nullptr);
+  }
   __syncthreads();
 
   const int col = lane & 15, grp = lane >> 4;
   const float scale = kLog2e / sqrtf(static_cast<float>(kHD));
-  uint4 qx[4];
+  uint4 qhi[4], qlo[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const float *src = &q_s[wave][col & (kVG - 1)][j * 32 + grp * 8];
-    uint32_t w[4];
+    const float *src = &q_s[wave][col][j * 32 + grp * 8];
+    uint32_t wh[4], wl[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       uint16_t h0, l0, h1, l1;
       split16<DT>(src[2 * e] * scale, h0, l0);
       split16<DT>(src[2 * e + 1] * scale, h1, l1);
-      w[e] = col < kVG ? (h0 | (static_cast<uint32_t>(h1) << 16)) : (l0 | (static_cast<uint32_t>(l1) << 16));
+      wh[e] = h0 | (static_cast<uint32_t>(h1) << 16);
+      wl[e] = l0 | (static_cast<uint32_t>(l1) << 16);
     }
-    qx[j] = make_uint4(w[0], w[1], w[2], w[3]);
+    qhi[j] = make_uint4(wh[0], wh[1], wh[2], wh[3]);
+    qlo[j] = make_uint4(wl[0], wl[1], wl[2], wl[3]);
   }
   // causal limit of this lane's column, and the last tile any of the wave's tokens can see
-  const uint32_t my_tok = min(wave_first + (col & (kVG - 1)) / G, T - 1);
+  const uint32_t my_tok = min(wave_first + col / G, T - 1);
   const uint32_t n_keys = p.position + my_tok + 1;
   const uint32_t wave_last_tile = (p.position + min(wave_first + kTokensPerWave - 1, T - 1)) / kKvBlockTokens;
   const bool wave_on = wave_first < T;
@@ -127,29 +134,25 @@ __global__ __launch_bounds__(kPW *kWave) void attn_prompt_kernel(AttnParams p) {
         kreg[j] = stage[st][j][lane];
         vreg[j] = stage[st][4 + j][lane];
       }
-      attn_tile<DT, kVG, false, true, true>(kreg, vreg, qx, nullptr, b, n_keys, col, grp, false, 0u, nullptr, nullptr, m, l, acc);
+      attn_tile_wide<DT>(kreg, vreg, qhi, qlo, b, n_keys, grp, m, l, acc);
     }
   }
   if (!wave_on) return;
 
-  // ---- results of the wave's pairs: token rows of the four lane groups, then hi + lo columns
+  // ---- results of the wave's pairs: token rows of the four lane groups
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
-  const uint32_t tok = wave_first + (col & (kVG - 1)) / G;
-  const uint32_t h = kvh * G + (col & (kVG - 1)) % G;
-  const bool writer = col < kVG && tok < T;
+  const uint32_t tok = wave_first + col / G;
+  const uint32_t h = kvh * G + col % G;
+  const bool writer = tok < T;
   const float inv = l > 0.0f && isfinite(l) ? 1.0f / l : 1.0f;
   char *ws = reinterpret_cast<char *>(p.part_acc) + static_cast<uint64_t>(tok) * p.ws_token_stride;
   const uint64_t ml_off = reinterpret_cast<char *>(p.part_m) - reinterpret_cast<char *>(p.part_acc);
   const uint64_t l_off = reinterpret_cast<char *>(p.part_l) - reinterpret_cast<char *>(p.part_acc);
 #pragma unroll
   for (int s2 = 0; s2 < 8; ++s2) {
-    float4 o;
-    o.x = acc[s2][0] + row_shl<kVG>(acc[s2][0]);
-    o.y = acc[s2][1] + row_shl<kVG>(acc[s2][1]);
-    o.z = acc[s2][2] + row_shl<kVG>(acc[s2][2]);
-    o.w = acc[s2][3] + row_shl<kVG>(acc[s2][3]);
     if (!writer) continue;
+    const float4 o = make_float4(acc[s2][0], acc[s2][1], acc[s2][2], acc[s2][3]);
     const uint32_t d = s2 * 16 + grp * 4;
     if (active == 1) {
       // a single split holds every key: final

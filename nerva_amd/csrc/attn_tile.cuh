@@ -272,6 +272,60 @@ __device__ __forceinline__ void attn_tile(uint4 (&kreg)[4], uint4 (&vreg)[4], co
   }
 }
 
+// The same tile step for sixteen independent columns (prompt blocks: sixteen (token, head) pairs of a wave). The
+// hi and lo halves of a query, and of a tile's probabilities, are two operands of two products that accumulate in the
+// same registers instead of two columns that meet by a lane exchange: the same number of matrix instructions per
+// pair, but the softmax arithmetic of a lane - the maximum, five exponentials, four hi/lo splits - serves a pair of
+// its own instead of being done twice, and a K/V tile read from LDS meets twice as many pairs. Columns are masked
+// individually (n_keys by column; a column may find a whole tile masked) and the accumulators are rescaled only
+// in tiles where some running maximum moved.
+template <uint32_t DT>
+__device__ __forceinline__ void attn_tile_wide(const uint4 (&kreg)[4], const uint4 (&vreg)[4], const uint4 (&qhi)[4],
+                                               const uint4 (&qlo)[4], uint32_t b, uint32_t n_keys, int grp, float &m,
+                                               float &l, f32x4_t (&acc)[8]) {
+  // scores of tokens b*16 + grp*4 + r for this lane's column
+  f32x4_t c{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) c = mfma_k32<DT>(kreg[j], qhi[j], c);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) c = mfma_k32<DT>(kreg[j], qlo[j], c);
+  float sc[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) sc[r] = b * kKvBlockTokens + grp * 4 + r < n_keys ? c[r] : -INFINITY;
+  float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+  mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
+  mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+  const float m_new = fmaxf(m, mb);
+  const float m_ref = fmaxf(m_new, -3.0e38f);   // a column with nothing to see yet: exponentials against a finite stand-in
+  const float alpha = attn_exp2(m - m_ref);
+  uint32_t ph[2], pl[2];
+  float psum = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 4; r += 2) {
+    const float p0 = attn_exp2(sc[r] - m_ref), p1 = attn_exp2(sc[r + 1] - m_ref);
+    psum += p0 + p1;
+    uint16_t h0, l0, h1, l1;
+    split16<DT>(p0, h0, l0);
+    split16<DT>(p1, h1, l1);
+    ph[r / 2] = h0 | (static_cast<uint32_t>(h1) << 16);
+    pl[r / 2] = l0 | (static_cast<uint32_t>(l1) << 16);
+  }
+  l = l * alpha + psum;
+  m = m_new;
+  const uint2 pbh = make_uint2(ph[0], ph[1]), pbl = make_uint2(pl[0], pl[1]);
+  if (__any(alpha != 1.0f)) {
+#pragma unroll
+    for (int s2 = 0; s2 < 8; ++s2) acc[s2] *= alpha;
+  }
+#pragma unroll
+  for (int s2 = 0; s2 < 8; ++s2) {
+    const uint4 &vr = vreg[s2 / 2];
+    const uint2 va = (s2 & 1) ? make_uint2(vr.z, vr.w) : make_uint2(vr.x, vr.y);
+    acc[s2] = mfma_k16<DT>(va, pbh, acc[s2]);
+    acc[s2] = mfma_k16<DT>(va, pbl, acc[s2]);
+  }
+}
+
 template <int G, int W>
 struct AttnShared {
   alignas(16) float q_s[G][kHD];
