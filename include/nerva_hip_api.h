@@ -588,8 +588,8 @@ typedef struct NervaHipGemmRowsRequest {
   uint16_t *output16;        /* epilogue 2: [tokens][rows] */
   /* != 0: input16 / output16 are in matrix-operand order instead of [tokens][cols] rows, the layout
    * the kernel reads with full cache lines: element (token t, column k) at index
-   * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 for tokens <= 64, 128 above
-   * (slots past `tokens` are never looked at). */
+   * nerva_hip_gemm_operand_index(tokens, t, k); the buffer holds 32 token slots for tokens <= 32, 64 for tokens <= 64, 128 for tokens
+   * <= 128, 256 for tokens <= 256, 512 above (slots past `tokens` are never looked at). */
   uint32_t input_operand_order, output16_operand_order;
   /* Optional device scratch of nerva_hip_gemm_rows_workspace_bytes(rows) bytes (rows doubled for
    * epilogue 2). With more than 64 tokens in operand order the projections with few rows are split
@@ -599,7 +599,8 @@ typedef struct NervaHipGemmRowsRequest {
 } NervaHipGemmRowsRequest;
 
 /* Projection of a block of up to 128 token rows (up to 256 with input_operand_order where rows is a multiple of
- * 96 or 128 - gate/up pairs: 48 or 64 - and cols of 512) through one weight matrix on the matrix cores,
+ * 96 or 128 - gate/up pairs: 48 or 64 - and cols of 512; up to 512 where rows is a multiple of 256 - gate/up
+ * pairs: 128 - and cols of 128) through one weight matrix on the matrix cores,
  * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
  * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must
