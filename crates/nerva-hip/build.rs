@@ -11,7 +11,7 @@ use std::process::Command;
 /// must compile without scratch memory, which this script checks like the library's own build (build.py). What
 /// the check cannot see - a register copy the compiler places between such a load and its wait - is covered by
 /// the library's parity tests only, which is why the kernels are built for the one target they were checked on.
-const HAND_ISSUED_LOADS: &[&str] = &["attn_step_kernel", "moe_gate_up_lean_kernel", "moe_down_lean_kernel", "fp8_gemv_lean_kernel"];
+const HAND_ISSUED_LOADS: &[&str] = &["attn_step_kernel", "moe_gate_up_lean_kernel", "moe_down_lean_kernel", "fp8_gemv_lean_kernel", "gemm_deep_kernel"];
 const SUPPORTED_ARCH: &str = "gfx950";
 
 const SOURCES: &[&str] = &[

@@ -47,7 +47,8 @@ def _spilling_kernels(remarks):
 # Kernels that request their data with hand-written loads and wait for it with explicit counts. The compiler
 # does not know that such a register is still being written, so a spill (or any copy) of it reads garbage:
 # these kernels must compile without scratch memory, which every build checks.
-HAND_ISSUED_LOADS = ("attn_step_kernel", "moe_gate_up_lean_kernel", "moe_down_lean_kernel", "fp8_gemv_lean_kernel")
+HAND_ISSUED_LOADS = ("attn_step_kernel", "moe_gate_up_lean_kernel", "moe_down_lean_kernel", "fp8_gemv_lean_kernel",
+                     "gemm_deep_kernel")
 
 
 def _compile(src):

@@ -356,7 +356,7 @@ def test_build_refuses_register_spills_in_kernels_that_issue_loads_by_hand():
         if not name.endswith((".hip", ".cuh")):
             continue
         text = open(os.path.join(csrc, name)).read()
-        if not re.search(r'asm volatile\(\s*"global_load_', text):
+        if not re.search(r'asm volatile\(\s*"(global_load_|ds_read_)', text):
             continue
         kernels = re.findall(r"__global__[^;{]*?void (\w+)\(", text)
         assert any(k in build.HAND_ISSUED_LOADS for k in kernels), name
