@@ -236,7 +236,7 @@ def case_gemm_rows():
         copies = max(2, (1 << 30) // (wrows * cols * 2) + 1)
         w = synth16(copies * wrows * cols, 61)
         ws = DeviceBuffer(R.gemm_rows_workspace_bytes(wrows))   # K slices of the large-block kernel
-        for tokens in (1, 8, 32, 64, 128) + ((256,) if rows <= 12288 else ()):
+        for tokens in (1, 8, 32, 64, 128) + ((256, 512) if rows <= 12288 else ()):
             x = synth16(max(tokens, 128) * cols, 62, std=1.0)
             y32 = DeviceBuffer(tokens * rows * 4)
             y16 = DeviceBuffer(max(tokens, 128) * rows * 2)
