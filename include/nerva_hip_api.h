@@ -599,8 +599,8 @@ typedef struct NervaHipGemmRowsRequest {
 } NervaHipGemmRowsRequest;
 
 /* Projection of a block of up to 128 token rows (up to 256 with input_operand_order where rows is a multiple of
- * 96 or 128 - gate/up pairs: 48 or 64 - and cols of 512; up to 512 where rows is a multiple of 256 - gate/up
- * pairs: 128 - and cols of 128) through one weight matrix on the matrix cores,
+ * 96 or 128 - gate/up pairs: 48 or 64 - and cols of 512; up to 512 where rows is a multiple of 192
+ * or 256 - gate/up pairs: 96 or 128 - and cols of 128) through one weight matrix on the matrix cores,
  * streaming the weights once: per token the arithmetic of mat_vec_encoded_row_major
  * (precision/block/ops.rs:75-91); the reference issues cuBLAS GEMMs for this in its chunked
  * prefill and projection batch (projection.cu:99-106, 297-300). rows >= 16 (with rows % 16 != 0 the residual must

@@ -663,17 +663,24 @@ constexpr uint32_t kDTokCap = 512;                      // token rows at most; t
 constexpr int kDK = 64;                                 // columns per K-block
 constexpr int kDXBuf = 2 * 16 * kWave * static_cast<int>(sizeof(u32x4_t));   // one X block of a half: 2 K-steps x 16 tiles = 32 KiB
 constexpr int kDWTile = 16 * kDK * static_cast<int>(sizeof(uint16_t));       // one W tile of a block: 2 KiB
-constexpr int kDWBuf = 16 * kDWTile;                                         // the workgroup's 16 tiles: 32 KiB
-constexpr size_t kDeepLds = 2 * static_cast<size_t>(kDXBuf) + 3 * static_cast<size_t>(kDWBuf);   // 163,840 B
+constexpr size_t deep_lds_bytes(int tpw) { return 2 * static_cast<size_t>(kDXBuf) + 3 * static_cast<size_t>(4 * tpw * kDWTile); }
 #define NV_LDS_PTR(P) ((__attribute__((address_space(3))) void *)(P))
 
-template <uint32_t DT, int EPI>
+// TPW: row tiles a wave takes, 4 (256 rows a workgroup, 160 KiB of LDS) or 3 (192 rows: where that many rows make
+// the launch fill the chip - a gate/up pair of 12288 + 12288 rows is 96 workgroups of 128 + 128 rows per token half,
+// 192 in all on 256 CUs, but 128 of 96 + 96). With three tiles a wave the gate tiles and the up tiles of a pair end
+// in different waves (row parts 0, 1: gate, 2, 3: their up tiles), and the up sums cross through LDS at the end.
+template <uint32_t DT, int EPI, int TPW>
 __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams p, float *partials, uint32_t units,
                                                                   uint32_t kslices) {
+  static_assert(TPW == 3 || TPW == 4, "three or four row tiles a wave");
+  constexpr int kTiles = 4 * TPW;                 // W tiles of the workgroup
+  constexpr int kWBuf = kTiles * kDWTile;         // one W buffer
+  constexpr int kWReq = kTiles * 2 / 8;           // W requests a wave and block (half a tile each)
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int th = wave & 1, rq = wave >> 1;   // token half of the workgroup's 256, row quarter of its 256
+  const int th = wave & 1, rq = wave >> 1;   // token half of the workgroup's 256, row part of its 16 TPW rows
   const uint32_t n = lane & 15, q = lane >> 4;
   const uint32_t cols = p.cols, T = p.tokens;
   const uint32_t halves = (T + 255u) / 256u;
@@ -683,25 +690,29 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
   const uint32_t group = unit / kslices, slice = unit % kslices;
   const uint32_t kper = cols / kslices, k0 = slice * kper, nblk = kper / kDK;
 
-  // LDS tile slot s = 4 * (row quarter) + j. Plain: rows 16 s .. of the workgroup's 256. SwiGLU: j = 0, 1 the
-  // gate tiles 2 rq + j of the workgroup's 128 gate rows, j = 2, 3 their up tiles - a wave's four tiles end in
-  // the wave that runs the epilogue.
+  // LDS tile slot s = TPW * (row part) + j. Plain: rows 16 s .. of the workgroup's rows. SwiGLU, four tiles a
+  // wave: j = 0, 1 the gate tiles 2 rq + j of the workgroup's 128 gate rows, j = 2, 3 their up tiles - a wave's
+  // tiles end in the wave that runs the epilogue. SwiGLU, three tiles a wave: parts 0, 1 the six gate tiles of
+  // the workgroup's 96 gate rows, parts 2, 3 their up tiles.
   auto slot_row = [&](int s) -> uint32_t {
-    if constexpr (EPI == kGemmSwiglu)
+    if constexpr (EPI == kGemmSwiglu && TPW == 4)
       return ((s >> 1) & 1) * p.rows + group * 128u + (2u * (s >> 2) + (s & 1)) * 16u;
+    else if constexpr (EPI == kGemmSwiglu)
+      return (s / 6) * p.rows + group * 96u + (s % 6) * 16u;
     else
-      return group * 256u + s * 16u;
+      return group * (16u * kTiles) + s * 16u;
   };
+  auto slot_is_up = [&](int s) -> bool { return EPI == kGemmSwiglu && (TPW == 4 ? ((s >> 1) & 1) != 0 : s >= 6); };
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(NV_LDS_PTR(smem)));   // X buffers, then W buffers
-  // W requests of this wave: tiles 2 wave and 2 wave + 1, two requests of 8 rows x 128 bytes each. Lane (r, c) of
-  // a request asks for piece c ^ r of row r: a wave-uniform base per request and one lane offset for all.
-  const char *wsrc[4];
+  // W requests of this wave: requests kWReq wave .. + kWReq - 1 of the block's 2 kTiles (tile m / 2, rows 8 (m % 2)
+  // .. + 7, 128 bytes a row). Lane (r, c) of a request asks for piece c ^ r of row r: a wave-uniform base per
+  // request and one lane offset for all.
+  const char *wsrc[kWReq];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int s_ = 2 * wave + (i >> 1);
+  for (int i = 0; i < kWReq; ++i) {
+    const int m = kWReq * wave + i, s_ = m >> 1;
     wsrc[i] = reinterpret_cast<const char *>(p.w) +
-              (static_cast<uint64_t>(slot_row(s_) + (i & 1) * 8u) * cols + k0 + (EPI == kGemmSwiglu && ((s_ >> 1) & 1) ? p.pair_gap : 0u)) *
-                  sizeof(uint16_t);
+              (static_cast<uint64_t>(slot_row(s_) + (m & 1) * 8u) * cols + k0 + (slot_is_up(s_) ? p.pair_gap : 0u)) * sizeof(uint16_t);
   }
   const uint32_t wlane = ((lane >> 3) * cols) * static_cast<uint32_t>(sizeof(uint16_t)) + (((lane & 7) ^ (lane >> 3)) << 4);
   // X requests of this wave: four consecutive token tiles of one K-step of the half's block
@@ -712,15 +723,15 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
   // A operand of K-step e of the block, lane (row n, quarter q): piece 4 e + q of row n, at piece ^ (n & 7)
   uint32_t a_off[2];
 #pragma unroll
-  for (int e = 0; e < 2; ++e) a_off[e] = lds0 + 2 * kDXBuf + (4 * rq) * kDWTile + n * 128 + (((e * 4 + q) ^ (n & 7)) << 4);
+  for (int e = 0; e < 2; ++e) a_off[e] = lds0 + 2 * kDXBuf + (TPW * rq) * kDWTile + n * 128 + (((e * 4 + q) ^ (n & 7)) << 4);
   // B operand of K-step e, token tile c of this wave's eight: piece (e * 16 + th * 8 + c) * 64 + lane of the buffer
   uint32_t b_addr[2];
 #pragma unroll
   for (int xb = 0; xb < 2; ++xb) b_addr[xb] = lds0 + xb * kDXBuf + ((th * 8) * kWave + lane) * static_cast<uint32_t>(sizeof(u32x4_t));
 
-  f32x4_t acc[4][8];
+  f32x4_t acc[TPW][8];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < TPW; ++j)
 #pragma unroll
     for (int c = 0; c < 8; ++c) acc[j][c] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -728,7 +739,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
 #define NV_DP_W1(WOFF, BLK, I)                                                                      \
   __builtin_amdgcn_global_load_lds(                                                                 \
       reinterpret_cast<const u32x4_t *>(wsrc[I] + static_cast<uint64_t>(BLK) * (kDK * sizeof(uint16_t)) + wlane), \
-      NV_LDS_PTR(smem + 2 * kDXBuf + (WOFF) + (2 * wave + ((I) >> 1)) * kDWTile + ((I) & 1) * 1024), 16, 0, 0)
+      NV_LDS_PTR(smem + 2 * kDXBuf + (WOFF) + (kWReq * wave + (I)) * 1024), 16, 0, 0)
 #define NV_DP_X1(XB, BLK, I)                                                                        \
   __builtin_amdgcn_global_load_lds(                                                                 \
       reinterpret_cast<const u32x4_t *>(xsrc + static_cast<uint64_t>(BLK) * xstep + (I) * 1024),    \
@@ -737,18 +748,26 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(DST) : "v"(ADDR), "n"(OFF) : "memory")
 #define NV_DP_READ_B(XB, IDX) NV_DP_LDS_READ(bq[(IDX) % 3], b_addr[XB], ((((IDX) >> 3) * 16 + ((IDX) & 7)) * kWave * 16))
 #define NV_DP_READ_A(E, J) NV_DP_LDS_READ(aq[E][J], a_cur[E], (J) * kDWTile)
-  // Operand reads of a block, in issue order: bq0, aq[0][0..3], bq1; then product group i issues bq(i + 2) and,
-  // for i < 4, aq[1][i]. LDS reads return in order, so group i waits until at most this many younger reads are
-  // outstanding: (behind aq[0][3]) 3, then 4, 5, 5, 4, 3, and 2 from group 6 on, 1 and 0 for the last two.
-  // The awaited registers are in/out operands of the wait, so that their use cannot move in front of it.
+  // Operand reads of a block, in issue order: bq0, aq[0][0..TPW-1], bq1; then product group i issues bq(i + 2) and,
+  // for i < TPW, aq[1][i]. LDS reads return in order, so group i waits until at most this many younger reads are
+  // outstanding: (behind aq[0][TPW-1]) 3, then 4, 5, then 5, 4, 3 (four tiles a wave) or 4, 3, 2 (three), and 2 from
+  // there on, 1 and 0 for the last two. The awaited registers are in/out operands of the wait, so that their use
+  // cannot move in front of it.
 #define NV_DP_AWAIT(N_, B_) asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_) :: "memory")
 #define NV_DP_AWAIT_A(N_, B_, E_)                                                                   \
-  asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_), "+v"(aq[E_][0]), "+v"(aq[E_][1]), "+v"(aq[E_][2]), "+v"(aq[E_][3]) :: "memory")
+  do {                                                                                              \
+    if constexpr (TPW == 4)                                                                         \
+      asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_), "+v"(aq[E_][0]), "+v"(aq[E_][1]), "+v"(aq[E_][2]), "+v"(aq[E_][TPW - 1]) :: "memory"); \
+    else                                                                                            \
+      asm volatile("s_waitcnt lgkmcnt(" #N_ ")" : "+v"(B_), "+v"(aq[E_][0]), "+v"(aq[E_][1]), "+v"(aq[E_][2]) :: "memory"); \
+  } while (0)
 #define NV_DP_WAIT(IDX)                                                                             \
   if constexpr ((IDX) == 0) NV_DP_AWAIT_A(3, bq[0], 0);                                             \
-  else if constexpr ((IDX) == 1 || (IDX) == 4) NV_DP_AWAIT(4, bq[(IDX) % 3]);                       \
-  else if constexpr ((IDX) == 2 || (IDX) == 3) NV_DP_AWAIT(5, bq[(IDX) % 3]);                       \
-  else if constexpr ((IDX) == 5) NV_DP_AWAIT(3, bq[(IDX) % 3]);                                     \
+  else if constexpr ((IDX) == 1) NV_DP_AWAIT(4, bq[(IDX) % 3]);                                     \
+  else if constexpr ((IDX) == 2) NV_DP_AWAIT(5, bq[(IDX) % 3]);                                     \
+  else if constexpr ((IDX) == 3) { if constexpr (TPW == 4) NV_DP_AWAIT(5, bq[(IDX) % 3]); else NV_DP_AWAIT(4, bq[(IDX) % 3]); } \
+  else if constexpr ((IDX) == 4) { if constexpr (TPW == 4) NV_DP_AWAIT(4, bq[(IDX) % 3]); else NV_DP_AWAIT(3, bq[(IDX) % 3]); } \
+  else if constexpr ((IDX) == 5) { if constexpr (TPW == 4) NV_DP_AWAIT(3, bq[(IDX) % 3]); else NV_DP_AWAIT(2, bq[(IDX) % 3]); } \
   else if constexpr ((IDX) == 8) NV_DP_AWAIT_A(2, bq[(IDX) % 3], 1);                                \
   else if constexpr ((IDX) == 14) NV_DP_AWAIT(1, bq[(IDX) % 3]);                                    \
   else if constexpr ((IDX) == 15) NV_DP_AWAIT(0, bq[(IDX) % 3]);                                    \
@@ -757,34 +776,32 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
 #define NV_DP_SLOT(IDX, XB, XEN, WEN)                                                               \
   if constexpr ((IDX) < 4) {                                                                        \
     if constexpr (XEN) { NV_DP_X1((XB) ^ 1, blk_ + 1u, IDX); }                                      \
-  } else if constexpr ((IDX) < 8) {                                                                 \
+  } else if constexpr ((IDX) < 4 + kWReq) {                                                         \
     if constexpr (WEN) { NV_DP_W1(w_ahead, blk_ + 2u, (IDX) - 4); }                                 \
   }
 #define NV_DP_ITEM(IDX, XB, XEN, WEN)                                                               \
   if constexpr ((IDX) + 2 < 16) { NV_DP_READ_B(XB, (IDX) + 2); }                                    \
-  if constexpr ((IDX) < 4) { NV_DP_READ_A(1, IDX); }                                                \
+  if constexpr ((IDX) < TPW) { NV_DP_READ_A(1, IDX); }                                              \
   NV_DP_WAIT(IDX);                                                                                  \
   __builtin_amdgcn_sched_barrier(0);                                                                \
-  _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                     \
+  _Pragma("unroll") for (int j = 0; j < TPW; ++j)                                                   \
       acc[j][(IDX) & 7] = mfma_k32<DT>(aq[(IDX) >> 3][j], bq[(IDX) % 3], acc[j][(IDX) & 7]);        \
   __builtin_amdgcn_sched_barrier(0);                                                                \
   NV_DP_SLOT(IDX, XB, XEN, WEN)                                                                     \
   __builtin_amdgcn_sched_barrier(0)
   // Block BLK in X buffer XB and the W buffer at w_cur. LAST: nothing younger than this block's requests is in
-  // flight; otherwise the four W requests of the block after it are.
+  // flight; otherwise the W requests of the block after it are.
 #define NV_DP_BLOCK(BLK, XB, LAST, XEN, WEN)                                                        \
   do {                                                                                              \
     const uint32_t blk_ = (BLK);                                                                    \
     if constexpr (LAST) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");               \
-    else asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");                              \
+    else if constexpr (kWReq == 4) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");    \
+    else asm volatile("s_waitcnt vmcnt(3)\n\ts_barrier" ::: "memory");                              \
     const uint32_t a_cur[2] = {a_off[0] + w_cur, a_off[1] + w_cur};                                 \
-    const uint32_t w_ahead = w_cur >= static_cast<uint32_t>(kDWBuf) ? w_cur - kDWBuf : w_cur + 2 * kDWBuf;   /* (b + 2) % 3 */ \
-    u32x4_t aq[2][4], bq[3];                                                                        \
+    const uint32_t w_ahead = w_cur >= static_cast<uint32_t>(kWBuf) ? w_cur - kWBuf : w_cur + 2 * kWBuf;   /* (b + 2) % 3 */ \
+    u32x4_t aq[2][TPW], bq[3];                                                                      \
     NV_DP_READ_B(XB, 0);                                                                            \
-    NV_DP_READ_A(0, 0);                                                                             \
-    NV_DP_READ_A(0, 1);                                                                             \
-    NV_DP_READ_A(0, 2);                                                                             \
-    NV_DP_READ_A(0, 3);                                                                             \
+    _Pragma("unroll") for (int j = 0; j < TPW; ++j) { NV_DP_READ_A(0, j); }                         \
     NV_DP_READ_B(XB, 1);                                                                            \
     __builtin_amdgcn_sched_barrier(0);                                                              \
     NV_DP_ITEM(0, XB, XEN, WEN);                                                                    \
@@ -803,7 +820,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
     NV_DP_ITEM(13, XB, XEN, WEN);                                                                   \
     NV_DP_ITEM(14, XB, XEN, WEN);                                                                   \
     NV_DP_ITEM(15, XB, XEN, WEN);                                                                   \
-    w_cur = w_cur == static_cast<uint32_t>(2 * kDWBuf) ? 0u : w_cur + kDWBuf;                        \
+    w_cur = w_cur == static_cast<uint32_t>(2 * kWBuf) ? 0u : w_cur + kWBuf;                          \
   } while (0)
 
   // start: X block 0, W blocks 0 and 1, in the order they are awaited in (nblk is even and at least 2)
@@ -815,10 +832,10 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
   }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) NV_DP_W1(0u, 0u, i);
+  for (int i = 0; i < kWReq; ++i) NV_DP_W1(0u, 0u, i);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) NV_DP_W1(static_cast<uint32_t>(kDWBuf), 1u, i);
+  for (int i = 0; i < kWReq; ++i) NV_DP_W1(static_cast<uint32_t>(kWBuf), 1u, i);
   __builtin_amdgcn_sched_barrier(0);
   uint32_t blk = 0;
   for (; blk + 2 < nblk; blk += 2) {
@@ -840,7 +857,28 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
 #undef NV_DP_BLOCK
 
   // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
-  if (kslices == 1) {
+  if constexpr (EPI == kGemmSwiglu && TPW == 3) {
+    // the up sums (row parts 2, 3) cross to the waves that hold their gate tiles (parts 0, 1, same token half)
+    // through LDS, which everyone has finished with
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    f32x4_t *meet = reinterpret_cast<f32x4_t *>(smem) + (((rq & 1) * 2 + th) * (TPW * 8)) * kWave + lane;
+    if (rq >= 2) {
+#pragma unroll
+      for (int j = 0; j < TPW; ++j)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) meet[(j * 8 + c) * kWave] = acc[j][c];
+    }
+    __syncthreads();
+    if (rq >= 2) return;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t t = half * 256u + (th * 8 + c) * 16u + n;
+      if (t < T) {
+#pragma unroll
+        for (int j = 0; j < TPW; ++j) block_epilogue<DT, EPI>(p, t, slot_row(TPW * rq + j) + q * 4u, acc[j][c], meet[(j * 8 + c) * kWave]);
+      }
+    }
+  } else if (kslices == 1) {
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       const uint32_t t = half * 256u + (th * 8 + c) * 16u + n;
@@ -850,7 +888,7 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
           for (int j = 0; j < 2; ++j) block_epilogue<DT, EPI>(p, t, slot_row(4 * rq + j) + q * 4u, acc[j][c], acc[j + 2][c]);
         } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) block_epilogue<DT, EPI>(p, t, slot_row(4 * rq + j) + q * 4u, acc[j][c], acc[j][c]);
+          for (int j = 0; j < TPW; ++j) block_epilogue<DT, EPI>(p, t, slot_row(TPW * rq + j) + q * 4u, acc[j][c], acc[j][c]);
         }
       }
     }
@@ -862,8 +900,8 @@ __global__ __launch_bounds__(8 * kWave, 2) void gemm_deep_kernel(GemmRowsParams 
       const uint32_t t = half * 256u + (th * 8 + c) * 16u + n;
       if (t < T) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          *reinterpret_cast<float4 *>(part + static_cast<uint64_t>(t) * wrows + slot_row(4 * rq + j) + q * 4u) =
+        for (int j = 0; j < TPW; ++j)
+          *reinterpret_cast<float4 *>(part + static_cast<uint64_t>(t) * wrows + slot_row(TPW * rq + j) + q * 4u) =
               make_float4(acc[j][c][0], acc[j][c][1], acc[j][c][2], acc[j][c][3]);
       }
     }
@@ -887,22 +925,67 @@ hipError_t launch_wide_pairs(const GemmRowsParams &p, float *partials, uint32_t 
   return hipGetLastError();
 }
 
-// Blocks of 257..512 rows (gemm_deep_kernel): workgroups of 256 rows (a gate/up pair: 128 + 128) x 256 tokens.
-inline uint32_t deep_wg_rows(int epilogue) { return epilogue == kGemmSwiglu ? 128u : 256u; }
+// Blocks of 257..512 rows (gemm_deep_kernel): workgroups of 256 rows (a gate/up pair: 128 + 128) x 256 tokens, or
+// of 192 rows (96 + 96) where the rows divide that way and the launch then fills the chip better.
+inline uint32_t deep_wg_rows(int epilogue, int tpw) { return (epilogue == kGemmSwiglu ? 32u : 64u) * static_cast<uint32_t>(tpw); }
 
-template <uint32_t DT, int EPI>
-hipError_t launch_deep(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+struct DeepPlan {
+  int tpw;            // row tiles a wave: 4, 3, or 0 where the kernel does not take the shape
+  uint32_t kslices;
+};
+// K slices as they would be chosen for `tpw` tiles a wave (0: the rows do not divide)
+inline uint32_t deep_slices_for(int epilogue, uint32_t rows, uint32_t cols, int tpw, uint64_t workspace_bytes) {
+  if (rows % deep_wg_rows(epilogue, tpw) != 0) return 0;
+  const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
+  const uint32_t groups = rows / deep_wg_rows(epilogue, tpw);
+  uint32_t slices = 1;
+  const int want = tuning(kTuneGemmBlockSlices);
+  if (want > 0 && cols % (static_cast<uint32_t>(want) * 2u * kDK) == 0) {
+    slices = static_cast<uint32_t>(want);
+  } else {
+    while (epilogue != kGemmSwiglu && groups * 2u * slices < 192u && slices < 8u && cols % (slices * 2u * 2u * kDK) == 0) slices *= 2u;
+  }
+  while (slices > 1 && static_cast<uint64_t>(slices) * kDTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
+  return slices;
+}
+// The tile height whose busiest CU has the least to do: rounds of 256 workgroups x rows a workgroup x columns a slice
+inline DeepPlan deep_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
+  DeepPlan best{0, 0};
+  if (tokens <= kWTokCap || tokens > kDTokCap || cols % (2u * kDK) != 0) return best;
+  uint64_t best_cost = ~uint64_t{0};
+  for (int tpw = 4; tpw >= 3; --tpw) {
+    const uint32_t slices = deep_slices_for(epilogue, rows, cols, tpw, workspace_bytes);
+    if (slices == 0) continue;
+    const uint64_t wgs = static_cast<uint64_t>(rows / deep_wg_rows(epilogue, tpw)) * 2u * slices;
+    const uint64_t cost = (wgs + 255u) / 256u * deep_wg_rows(epilogue, tpw) * (cols / slices);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = DeepPlan{tpw, slices};
+    }
+  }
+  return best;
+}
+
+template <uint32_t DT, int EPI, int TPW>
+hipError_t launch_deep_tpw(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t raised = hipSuccess;
   std::call_once(once, [] {
-    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_deep_kernel<DT, EPI>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDeepLds));
+    raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_deep_kernel<DT, EPI, TPW>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(deep_lds_bytes(TPW)));
   });
   if (raised != hipSuccess) return raised;
-  const uint32_t units = p.rows / deep_wg_rows(EPI) * kslices, halves = (p.tokens + 255u) / 256u;
-  hipLaunchKernelGGL((gemm_deep_kernel<DT, EPI>), dim3((units + 7u) / 8u * 8u * halves), dim3(8 * kWave), kDeepLds, stream, p,
-                     partials, units, kslices);
-  hipError_t err = hipGetLastError();
+  const uint32_t units = p.rows / deep_wg_rows(EPI, TPW) * kslices, halves = (p.tokens + 255u) / 256u;
+  hipLaunchKernelGGL((gemm_deep_kernel<DT, EPI, TPW>), dim3((units + 7u) / 8u * 8u * halves), dim3(8 * kWave), deep_lds_bytes(TPW),
+                     stream, p, partials, units, kslices);
+  return hipGetLastError();
+}
+
+template <uint32_t DT, int EPI>
+hipError_t launch_deep(const GemmRowsParams &p, float *partials, const DeepPlan &plan, hipStream_t stream) {
+  const uint32_t kslices = plan.kslices;
+  hipError_t err = plan.tpw == 3 ? launch_deep_tpw<DT, EPI, 3>(p, partials, kslices, stream)
+                                 : launch_deep_tpw<DT, EPI, 4>(p, partials, kslices, stream);
   if (err == hipSuccess && kslices > 1) {
     if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
       hipLaunchKernelGGL((gemm_finish_norm_kernel<DT>), dim3(p.tokens), dim3(kFinNormThreads), 0, stream, p,
@@ -918,12 +1001,12 @@ hipError_t launch_deep(const GemmRowsParams &p, float *partials, uint32_t kslice
 }
 
 template <uint32_t DT>
-hipError_t launch_deep_dt(int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
+hipError_t launch_deep_dt(int epilogue, const GemmRowsParams &p, const DeepPlan &plan, hipStream_t stream) {
   float *partials = static_cast<float *>(p.workspace);
   switch (epilogue) {
-    case kGemmF32: return launch_deep<DT, kGemmF32>(p, partials, kslices, stream);
-    case kGemmResidual: return launch_deep<DT, kGemmResidual>(p, partials, kslices, stream);
-    case kGemmSwiglu: return launch_deep<DT, kGemmSwiglu>(p, partials, kslices, stream);
+    case kGemmF32: return launch_deep<DT, kGemmF32>(p, partials, plan, stream);
+    case kGemmResidual: return launch_deep<DT, kGemmResidual>(p, partials, plan, stream);
+    case kGemmSwiglu: return launch_deep<DT, kGemmSwiglu>(p, partials, plan, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1026,22 +1109,11 @@ uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t t
   return slices;
 }
 
-// Blocks of 257..512 rows: K slices of gemm_deep_kernel, or 0 where it does not take the shape. Enough workgroups
-// (row groups x 2 token halves x slices) for three quarters of the CUs, each slice an even number of K-blocks, the
-// partial sums within the workspace.
+// Blocks of 257..512 rows: K slices of gemm_deep_kernel, or 0 where it does not take the shape (rows a multiple of 256
+// or 192; a gate/up pair: of 128 or 96). Enough workgroups (row groups x 2 token halves x slices) for three quarters
+// of the CUs, each slice an even number of K-blocks, the partial sums within the workspace.
 uint32_t gemm_deep_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
-  if (tokens <= kWTokCap || tokens > kDTokCap || rows % deep_wg_rows(epilogue) != 0 || cols % (2u * kDK) != 0) return 0;
-  const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
-  const uint32_t groups = rows / deep_wg_rows(epilogue);
-  uint32_t slices = 1;
-  const int want = tuning(kTuneGemmBlockSlices);
-  if (want > 0 && cols % (static_cast<uint32_t>(want) * 2u * kDK) == 0) {
-    slices = static_cast<uint32_t>(want);
-  } else {
-    while (epilogue != kGemmSwiglu && groups * 2u * slices < 192u && slices < 8u && cols % (slices * 2u * 2u * kDK) == 0) slices *= 2u;
-  }
-  while (slices > 1 && static_cast<uint64_t>(slices) * kDTokCap * wrows * sizeof(float) > workspace_bytes) slices /= 2u;
-  return slices;
+  return deep_plan(epilogue, rows, cols, tokens, workspace_bytes).kslices;
 }
 
 bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes) {
@@ -1070,11 +1142,11 @@ hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &
 }
 
 hipError_t launch_gemm_deep(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream) {
-  if (kslices == 0 || p.x_packed != gemm_packed_tiles(p.tokens) || p.tokens <= kWTokCap || p.tokens > kDTokCap)
-    return hipErrorInvalidValue;
+  const DeepPlan plan = deep_plan(epilogue, p.rows, p.cols, p.tokens, p.workspace != nullptr ? p.workspace_bytes : 0);
+  if (kslices == 0 || plan.kslices != kslices || p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;
   if (kslices > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
-  if (dtype == kBF16) return launch_deep_dt<kBF16>(epilogue, p, kslices, stream);
-  if (dtype == kF16) return launch_deep_dt<kF16>(epilogue, p, kslices, stream);
+  if (dtype == kBF16) return launch_deep_dt<kBF16>(epilogue, p, plan, stream);
+  if (dtype == kF16) return launch_deep_dt<kF16>(epilogue, p, plan, stream);
   return hipErrorInvalidValue;
 }
 

@@ -88,7 +88,7 @@ hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams 
 uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
 hipError_t launch_gemm_wide(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
 // Blocks of 257..kGemmDeepMaxTokens rows in operand order (32 token tiles): the same for the kernel that takes
-// 256 rows x 256 tokens per workgroup (rows a multiple of 256, a gate/up pair of 128, cols of 128).
+// 256 or 192 rows x 256 tokens per workgroup (rows a multiple of 192 or 256, a gate/up pair of 96 or 128, cols of 128).
 uint32_t gemm_deep_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
 hipError_t launch_gemm_deep(uint32_t dtype, int epilogue, const GemmRowsParams &p, uint32_t kslices, hipStream_t stream);
 // Whether launch_gemm_rows honours GemmRowsParams::norm_gamma for this shape (a K-sliced residual projection of a

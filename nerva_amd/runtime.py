@@ -316,8 +316,8 @@ def gemm_rows(dtype, weights, rows, cols, tokens, input16, epilogue=0, bias=None
               workspace=None):
     """Y[t] = W . X[t] for up to 128 token rows on the matrix cores (weights streamed once); up to 256 rows
     with the input in operand order where the kernel for wide blocks takes the shape (rows a multiple of 128,
-    gate/up pairs of 64, cols of 512); up to 512 where the kernel with 256 x 256 workgroup tiles does (rows a
-    multiple of 256, gate/up pairs of 128, cols of 128).
+    gate/up pairs of 64, cols of 512); up to 512 where the kernel with 256 (or 192) x 256 workgroup tiles does
+    (rows a multiple of 192 or 256, gate/up pairs of 96 or 128, cols of 128).
     `workspace`: optional DeviceBuffer of gemm_rows_workspace_bytes(rows) for the K-sliced large-block kernels."""
     lib = abi.load()
     req = abi.NervaHipGemmRowsRequest()

@@ -945,7 +945,7 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
                                                (128, 2048, 129), (256, 4096, 200), (4096, 4096, 256), (6144, 4096, 255),
                                                (4096, 12288, 256), (192, 2048, 140),
                                                (256, 2048, 257), (512, 4096, 300), (4096, 4096, 512), (6144, 4096, 511),
-                                               (4096, 12288, 512), (256, 1024, 400)])
+                                               (4096, 12288, 512), (256, 1024, 400), (192, 2048, 300), (576, 1024, 512)])
 def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     """More than 16 token rows in operand order: the workgroups split rows (and, given a workspace, K) and read
     X from LDS (2, 4, 8 or - blocks of 129..256 rows, three or four wave pairs sharing their W tiles - 16 token tiles;
@@ -1011,7 +1011,7 @@ def test_gemm_rows_large_blocks_in_f16(tokens):
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
                                                  (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200),
-                                                 (128, 2048, 257), (256, 1024, 512), (12288, 4096, 500)])
+                                                 (128, 2048, 257), (256, 1024, 512), (12288, 4096, 500), (96, 2048, 300), (288, 1024, 512)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
