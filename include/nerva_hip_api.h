@@ -754,7 +754,9 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
  * "block_layout" (1: token blocks as [token][column] rows, 2: in matrix-operand order, whatever their size),
  * "prefill_attention_rows" (1: prompt blocks with one attention workgroup set per token), "prefill_walk" (1:
  * sessions created afterwards walk their prompts token by token), "gemm_block_off" (1: blocks of more than 64
- * rows through the kernel of the smaller ones). Values a kernel
+ * rows through the kernel of the smaller ones), "gemm_block_waves" (4: the gate/up pair of a block of up to 64 rows
+ * never in three-wave workgroups), "gemm_block_rotate" (1 + the K-blocks between the places where consecutive row
+ * groups of that kernel start their walk; 1: a common start). Values a kernel
  * cannot take are ignored where they are read. -1 for an unknown name. A null name restores every built-in
  * choice. */
 int nerva_hip_test_set_tuning(const char *name, int32_t value);

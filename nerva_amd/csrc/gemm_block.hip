@@ -23,8 +23,7 @@ namespace nv {
 
 namespace {
 
-constexpr int kBW = 4;                       // waves per workgroup: they split the rows
-constexpr int kBThreads = kBW * kWave;
+constexpr int kBW = 4;                       // waves per workgroup: they split the rows (three where that fills the chip)
 constexpr int kBK = 128;                     // columns per K-block
 constexpr int kBSteps = kBK / 32;            // matrix-core K-steps per block
 constexpr int kBRing = 4;                    // W blocks a wave requests ahead at most (two with one row tile per wave)
@@ -92,11 +91,16 @@ __device__ __forceinline__ void block_epilogue(const GemmRowsParams &p, uint32_t
 // One row tile per wave: two W blocks requested ahead, two workgroups share a CU. Two row tiles: a wave
 // takes more than 256 registers, a CU holds one workgroup, and four W blocks are requested ahead to make
 // up for it (measured: gate_up 62.5 -> 54.4 us with four; the one-tile projections lose 5-8 % with four).
-template <uint32_t DT, int EPI, int NR, int TT>
-__global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(GemmRowsParams p, float *partials) {
+// BW: waves per workgroup. With three, the X block is not a whole number of rounds of the workgroup's threads: the
+// last round wraps and fetches pieces of the first again (same bytes to the same place), so that no request sits
+// under a branch.
+template <uint32_t DT, int EPI, int NR, int TT, int BW>
+__global__ __launch_bounds__(BW * kWave, NR == 1 ? 2 : 1) void gemm_block_kernel(GemmRowsParams p, float *partials, uint32_t rotate) {
+  constexpr int kBThreads = BW * kWave;
   constexpr int kTiles = TT;                              // 16-token tiles of the block (X in operand order with TT tiles)
   constexpr int kStageVec = kBSteps * kTiles * kWave;     // 16-byte pieces of one X block (TT = 8: 2048 = 32 KiB)
-  constexpr int kFill = kStageVec / kBThreads;            // pieces per thread and block
+  constexpr int kFill = (kStageVec + kBThreads - 1) / kBThreads;   // pieces per thread and block
+  static_assert(kFill <= 8, "the X requests of a block go out in the first four half K-steps, two at a time");
   extern __shared__ __align__(16) unsigned char smem[];
   u32x4_t *stage = reinterpret_cast<u32x4_t *>(smem);   // [kStageVec]: the X block, shared by the four waves
   const int lane = threadIdx.x & (kWave - 1);
@@ -105,13 +109,18 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   const uint32_t n = lane & 15, q = lane >> 4;
   const uint32_t cols = p.cols, T = p.tokens;
   const uint32_t kslices = gridDim.y, kper = cols / kslices, k0 = blockIdx.y * kper, nblk = kper / kBK;
+  // Row groups start their walk over the K-blocks at different places (and wrap): when every workgroup asks for the
+  // same columns of its rows at the same time, rows that are a multiple of 8 KiB apart crowd a part of the memory
+  // channels (the request pattern alone, gate/up of 32 token rows: 39 us from a common start, 33-35 rotated).
+  const uint32_t rot_off = (blockIdx.x * rotate) % nblk;
+#define NV_BLK_AT(BLK) ((BLK) + rot_off >= nblk ? (BLK) + rot_off - nblk : (BLK) + rot_off)
 
   // W row of tile j (index into W; for SwiGLU the up tile lies p.rows further down)
   uint32_t trow[NR];
 #pragma unroll
   for (int j = 0; j < NR; ++j)
-    trow[j] = EPI == kGemmSwiglu ? j * p.rows + blockIdx.x * (16u * kBW) + wave * 16u
-                                 : blockIdx.x * (16u * kBW * NR) + (wave * NR + j) * 16u;
+    trow[j] = EPI == kGemmSwiglu ? j * p.rows + blockIdx.x * (16u * BW) + wave * 16u
+                                 : blockIdx.x * (16u * BW * NR) + (wave * NR + j) * 16u;
   // W block -> registers: request i of a tile covers its rows 4i .. 4i + 3, 16 lanes x 16 B = 256 contiguous
   // bytes per row (whole cache lines, like the GEMV's stream)
   // Addresses are a wave-uniform 64-bit base (scalar registers, scalar arithmetic) plus a 32-bit per-lane
@@ -126,7 +135,6 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   const uint16_t *a_read = wtile + n * kBRowStride + q * 8;
   // X block b of this slice: kStageVec pieces in a row
   const char *xbase = reinterpret_cast<const char *>(p.x16) + static_cast<uint64_t>(k0 / 32u) * (kTiles * kWave) * sizeof(u32x4_t);
-  const uint32_t xlane = threadIdx.x * static_cast<uint32_t>(sizeof(u32x4_t));
 
   constexpr int kRing = NR == 1 ? 2 : kBRing;   // W blocks requested ahead: what the register budget holds
   u32x4_t areg[kRing][NR][4];
@@ -140,16 +148,17 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 #define NV_BLK_W(BUF, BLK)                                                                          \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       areg[BUF][j][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(               \
-          wbase[j] + (static_cast<uint64_t>(4 * i) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
+          wbase[j] + (static_cast<uint64_t>(4 * i) * cols + static_cast<uint64_t>(NV_BLK_AT(BLK)) * kBK) * sizeof(uint16_t) + wlane))
 #define NV_BLK_WPARK(BUF)                                                                           \
   _Pragma("unroll") for (int j = 0; j < NR; ++j) _Pragma("unroll") for (int i = 0; i < 4; ++i)       \
       *reinterpret_cast<u32x4_t *>(park_at + j * kBWTile + 4 * i * kBRowStride) = areg[BUF][j][i]
+#define NV_BLK_XPIECE(I) ((static_cast<uint32_t>(I) * kBThreads + threadIdx.x) & static_cast<uint32_t>(kStageVec - 1))
 #define NV_BLK_X(XB, BLK)                                                                           \
   _Pragma("unroll") for (int i = 0; i < kFill; ++i)                                                 \
       xreg[XB][i] = *reinterpret_cast<const u32x4_t *>(                                              \
-          xbase + (static_cast<uint64_t>(BLK) * kStageVec + i * kBThreads) * sizeof(u32x4_t) + xlane)
+          xbase + (static_cast<uint64_t>(NV_BLK_AT(BLK)) * kStageVec + NV_BLK_XPIECE(i)) * sizeof(u32x4_t))
 #define NV_BLK_XPARK(XB)                                                                            \
-  _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[i * kBThreads + threadIdx.x] = xreg[XB][i]
+  _Pragma("unroll") for (int i = 0; i < kFill; ++i) stage[NV_BLK_XPIECE(i)] = xreg[XB][i]
   // LDS operand reads run one half K-step ahead of the products that use them: once the products of token
   // tiles 0..3 have been issued their B registers take the next K-step's pieces, likewise tiles 4..7, so a
   // read has the other half's products (128 cycles of matrix-core time per row tile) to arrive in. The
@@ -167,10 +176,11 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
   // four waves handing it their 16 requests at once spent 550-1000 cycles issuing them before any product ran.
 #define NV_BLK_W1(BUF, BLK, J, I)                                                                   \
   areg[BUF][J][I] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(                   \
-      wbase[J] + (static_cast<uint64_t>(4 * (I)) * cols + static_cast<uint64_t>(BLK) * kBK) * sizeof(uint16_t) + wlane))
+      wbase[J] + (static_cast<uint64_t>(4 * (I)) * cols + static_cast<uint64_t>(NV_BLK_AT(BLK)) * kBK) * sizeof(uint16_t) + wlane))
 #define NV_BLK_X1(XB, BLK, I)                                                                       \
-  xreg[XB][I] = *reinterpret_cast<const u32x4_t *>(                                                  \
-      xbase + (static_cast<uint64_t>(BLK) * kStageVec + (I) * kBThreads) * sizeof(u32x4_t) + xlane)
+  if constexpr ((I) < kFill)                                                                        \
+    xreg[XB][I] = *reinterpret_cast<const u32x4_t *>(                                                \
+        xbase + (static_cast<uint64_t>(NV_BLK_AT(BLK)) * kStageVec + NV_BLK_XPIECE(I)) * sizeof(u32x4_t))
 #define NV_BLK_SLOT(K, BUF, XB, XEN, XBLK, WEN, WBLK)                                               \
   if constexpr ((K) < 4) {                                                                          \
     if constexpr (XEN && 2 * (K) < kFill) {                                                         \
@@ -263,6 +273,8 @@ __global__ __launch_bounds__(kBThreads, NR == 1 ? 2 : 1) void gemm_block_kernel(
 #undef NV_BLK_SLOT
 #undef NV_BLK_W1
 #undef NV_BLK_X1
+#undef NV_BLK_XPIECE
+#undef NV_BLK_AT
 #undef NV_BLK_ITER
 
   // D layout: lane (n, q) holds rows q*4 .. q*4+3 of a row tile for token n of a token tile
@@ -394,27 +406,33 @@ __global__ __launch_bounds__(kFinNormThreads) void gemm_finish_norm_kernel(GemmR
   }
 }
 
-template <int NR, int TT>
-constexpr size_t block_lds_bytes() {
-  return static_cast<size_t>(kBSteps) * TT * kWave * sizeof(u32x4_t) + static_cast<size_t>(kBW) * NR * kBWTile * sizeof(uint16_t);
+// K-blocks by which consecutive row groups start their walk apart (the "gemm_block_rotate" override: value - 1)
+inline uint32_t block_rotation() {
+  const int want = tuning(kTuneGemmBlockRotate);
+  return want > 0 ? static_cast<uint32_t>(want - 1) : 5u;
 }
 
-template <uint32_t DT, int EPI, int NR, int TT>
+template <int NR, int TT, int BW>
+constexpr size_t block_lds_bytes() {
+  return static_cast<size_t>(kBSteps) * TT * kWave * sizeof(u32x4_t) + static_cast<size_t>(BW) * NR * kBWTile * sizeof(uint16_t);
+}
+
+template <uint32_t DT, int EPI, int NR, int TT, int BW = kBW>
 hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
-  const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * kBW : 16u * kBW * NR;
-  constexpr size_t lds = block_lds_bytes<NR, TT>();
+  const uint32_t wg_rows = EPI == kGemmSwiglu ? 16u * BW : 16u * BW * NR;
+  constexpr size_t lds = block_lds_bytes<NR, TT, BW>();
   if (lds > 64 * 1024) {
     // more than the default dynamic LDS limit: raise it once per kernel (never under stream capture)
     static std::once_flag once;
     static hipError_t raised = hipSuccess;
     std::call_once(once, [] {
-      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR, TT>),
+      raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_block_kernel<DT, EPI, NR, TT, BW>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     });
     if (raised != hipSuccess) return raised;
   }
-  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, TT>), dim3(p.rows / wg_rows, kslices), dim3(kBThreads), lds, stream,
-                     p, partials);
+  hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, TT, BW>), dim3(p.rows / wg_rows, kslices), dim3(BW * kWave), lds, stream,
+                     p, partials, block_rotation());
   hipError_t err = hipGetLastError();
   if (err == hipSuccess && kslices > 1) {
     if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
@@ -431,7 +449,17 @@ hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t ks
 }
 
 template <uint32_t DT, int EPI, int NR>
-hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, hipStream_t stream) {
+hipError_t launch_block_nr(const GemmRowsParams &p, float *partials, uint32_t kslices, uint32_t waves, hipStream_t stream) {
+  if constexpr (EPI == kGemmSwiglu) {
+    if (waves == 3) {   // (the plan offers it for blocks of up to 64 rows)
+      switch (p.x_packed) {
+        case 2: return launch_block_tt<DT, EPI, NR, 2, 3>(p, partials, kslices, stream);
+        case 4: return launch_block_tt<DT, EPI, NR, 4, 3>(p, partials, kslices, stream);
+        default: return hipErrorInvalidValue;
+      }
+    }
+  }
+  if (waves != kBW) return hipErrorInvalidValue;
   switch (p.x_packed) {   // token tiles of the block = tiles of its operand-order layout
     case 2: return launch_block_tt<DT, EPI, NR, 2>(p, partials, kslices, stream);
     case 4: return launch_block_tt<DT, EPI, NR, 4>(p, partials, kslices, stream);
@@ -1047,12 +1075,12 @@ hipError_t launch_block_dt(int epilogue, const GemmRowsParams &p, const GemmBloc
   float *partials = static_cast<float *>(p.workspace);
   switch (epilogue) {
     case kGemmF32:
-      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmF32, 2>(p, partials, plan.kslices, stream)
-                                 : launch_block_nr<DT, kGemmF32, 1>(p, partials, plan.kslices, stream);
+      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmF32, 2>(p, partials, plan.kslices, plan.waves, stream)
+                                 : launch_block_nr<DT, kGemmF32, 1>(p, partials, plan.kslices, plan.waves, stream);
     case kGemmResidual:
-      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmResidual, 2>(p, partials, plan.kslices, stream)
-                                 : launch_block_nr<DT, kGemmResidual, 1>(p, partials, plan.kslices, stream);
-    case kGemmSwiglu: return launch_block_nr<DT, kGemmSwiglu, 2>(p, partials, plan.kslices, stream);
+      return plan.row_tiles == 2 ? launch_block_nr<DT, kGemmResidual, 2>(p, partials, plan.kslices, plan.waves, stream)
+                                 : launch_block_nr<DT, kGemmResidual, 1>(p, partials, plan.kslices, plan.waves, stream);
+    case kGemmSwiglu: return launch_block_nr<DT, kGemmSwiglu, 2>(p, partials, plan.kslices, plan.waves, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1065,12 +1093,19 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   const int want_slices = tuning(kTuneGemmBlockSlices);
   const int want_tiles = tuning(kTuneGemmBlockRowTiles);
   const uint32_t min_tokens = tuning(kTuneGemmBlockMinTokens) > 0 ? static_cast<uint32_t>(tuning(kTuneGemmBlockMinTokens)) : 17u;
-  if (mode == 0 || tokens < min_tokens || tokens > kBTokCap || rows % (16u * kBW) != 0 || cols % (kBRing * kBK) != 0) return plan;
+  // Waves per workgroup: four, or three for a gate/up pair of a small block where that gives every CU a workgroup
+  // (rounds of 256 workgroups x rows a workgroup: 12288 pairs are 192 workgroups of 64 + 64 rows or 256 of 48 + 48).
+  uint32_t waves = kBW;
+  if (epilogue == kGemmSwiglu && tokens <= 64u && rows % 48u == 0 && tuning(kTuneGemmBlockWaves) != 4) {
+    const uint32_t four = rows % 64u == 0 ? (rows / 64u + 255u) / 256u * 64u : ~0u, three = (rows / 48u + 255u) / 256u * 48u;
+    if (three < four) waves = 3;
+  }
+  if (mode == 0 || tokens < min_tokens || tokens > kBTokCap || rows % (16u * waves) != 0 || cols % (kBRing * kBK) != 0) return plan;
   const uint32_t wrows = epilogue == kGemmSwiglu ? 2u * rows : rows;
   // Row tiles per wave: two where that still leaves a workgroup for most CUs.
   uint32_t tiles = epilogue == kGemmSwiglu ? 2u : (rows / (16u * kBW * 2u) >= 96u && rows % (16u * kBW * 2u) == 0 ? 2u : 1u);
   if (epilogue != kGemmSwiglu && (want_tiles == 1 || (want_tiles == 2 && rows % (16u * kBW * 2u) == 0))) tiles = want_tiles;
-  const uint32_t groups = rows / (epilogue == kGemmSwiglu ? 16u * kBW : 16u * kBW * tiles);
+  const uint32_t groups = rows / (epilogue == kGemmSwiglu ? 16u * waves : 16u * kBW * tiles);
   // K slices: enough workgroups for two per CU, each slice a whole number of rings of K-blocks.
   // (A sliced gate/up pair would write and re-read 12.6 MB of partial sums per slice: measured no faster.)
   uint32_t slices = 1;
@@ -1086,6 +1121,7 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   }
   plan.row_tiles = tiles;
   plan.kslices = slices;
+  plan.waves = waves;
   return plan;
 }
 

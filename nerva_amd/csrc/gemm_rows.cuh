@@ -75,7 +75,7 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
 // and K slices (more than one needs slices x 128 x W rows f32 of workspace). launch_gemm_rows uses it by
 // itself where the plan allows.
 struct GemmBlockPlan {
-  uint32_t row_tiles, kslices;
+  uint32_t row_tiles, kslices, waves;
 };
 GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
 // Workspace that lets every projection of up to `rows_max` output rows (a gate/up pair counts twice) use its plan.

@@ -313,7 +313,9 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
   // rows shared by the last two workgroups are written twice: an in-place residual would be added twice
   if (epilogue == kGemmResidual && p.rows % 16 != 0 && p.residual == p.out_f32) return hipErrorInvalidValue;
   if (epilogue == kGemmSwiglu && p.out16 == nullptr) return hipErrorInvalidValue;
-  if (p.out_packed_tiles != 0 && (epilogue != kGemmSwiglu || p.out_packed_tiles * 16u < p.tokens)) return hipErrorInvalidValue;
+  // (operand order is defined in runs of 32 columns: an output of another width has no such layout)
+  if (p.out_packed_tiles != 0 && (epilogue != kGemmSwiglu || p.out_packed_tiles * 16u < p.tokens || p.rows % 32 != 0))
+    return hipErrorInvalidValue;
   if (p.x_packed != 0 && p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;   // tiles the kernel will assume
   if (dtype != kBF16 && dtype != kF16) return hipErrorInvalidValue;
   if (p.norm_gamma != nullptr &&   // a fused norm only where the shape has one; never silently dropped

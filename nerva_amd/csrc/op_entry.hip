@@ -34,7 +34,8 @@ constexpr const char *kTuningNames[kTuneKnobs] = {"attn_splits",       "batch_sp
                                                   "moe_down_shared_first", "gemv_workgroup_waves",
                                                   "gemv_x_registers",  "prefill_block_tokens", "gemv_rotated_walk",
                                                   "attn_merge_spin_limit", "attn_withhold_split", "block_layout",
-                                                  "prefill_attention_rows", "prefill_walk", "gemm_block_off"};
+                                                  "prefill_attention_rows", "prefill_walk", "gemm_block_off",
+                                                  "gemm_block_waves", "gemm_block_rotate"};
 }  // namespace
 
 int tuning(TuningKnob knob) { return g_tuning[knob].load(std::memory_order_relaxed); }

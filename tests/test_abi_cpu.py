@@ -316,7 +316,7 @@ def test_launch_shape_and_tuning_hooks_are_host_arithmetic():
                  "gemm_block_slices", "gemm_block_row_tiles", "gemm_block_min_tokens", "gemv_exact_start",
                  "moe_down_shared_first", "gemv_workgroup_waves", "gemv_x_registers", "prefill_block_tokens",
                  "gemv_rotated_walk", "attn_merge_spin_limit", "attn_withhold_split", "block_layout",
-                 "prefill_attention_rows", "prefill_walk", "gemm_block_off"):
+                 "prefill_attention_rows", "prefill_walk", "gemm_block_off", "gemm_block_waves", "gemm_block_rotate"):
         N.Device.set_tuning(name, 2)
         N.Device.set_tuning(name, 0)
     with pytest.raises(ValueError):

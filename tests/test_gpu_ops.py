@@ -240,6 +240,8 @@ def test_gemm_rows_rejects_unsupported_shapes():
     for rows, cols, tokens, epi in ((64, 2048, 200, 0), (128, 2048, 257, 0), (32, 2048, 130, 2)):
         with pytest.raises(RuntimeError):
             N.gemm_rows(BF16, w, rows, cols, tokens, x, epilogue=epi, out_f32=y, out16=y, input_operand_order=True)
+    with pytest.raises(RuntimeError):      # operand order comes in runs of 32 columns: no such output 48 wide
+        N.gemm_rows(BF16, w, 48, 2048, 20, x, epilogue=2, out16=y, input_operand_order=True, output16_operand_order=True)
 
 
 @pytest.mark.parametrize("full", [False, True])
@@ -1011,7 +1013,8 @@ def test_gemm_rows_large_blocks_in_f16(tokens):
 @pytest.mark.parametrize("sliced", [False, True])
 @pytest.mark.parametrize("inter,hidden,tokens", [(64, 2048, 77), (12288, 4096, 128), (64, 2048, 24), (12288, 4096, 32), (128, 2048, 50),
                                                  (64, 2048, 130), (128, 2048, 256), (12288, 4096, 250), (96, 2048, 200),
-                                                 (128, 2048, 257), (256, 1024, 512), (12288, 4096, 500), (96, 2048, 300), (288, 1024, 512)])
+                                                 (128, 2048, 257), (256, 1024, 512), (12288, 4096, 500), (96, 2048, 300), (288, 1024, 512),
+                                                 (192, 2048, 20), (96, 2048, 40), (288, 2048, 64)])
 def test_gemm_rows_large_blocks_swiglu(inter, hidden, tokens, sliced):
     """The gate/up pair of a large block: out16 = round16(silu(gate) * up), written in operand order."""
     dtype = BF16
