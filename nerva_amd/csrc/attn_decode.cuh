@@ -69,6 +69,10 @@ struct AttnParams {
   // table and split workspace: the strides below are added z times.
   uint32_t tokens;
   uint32_t qkv_token_stride;   // f32 elements between tokens' q|k|v
+  // Batches of sequences only: qkv_slices = 2..4 says that `qkv` holds that many partial sums of every value,
+  // qkv_slice_stride f32 elements apart (the K slices of the projection, as its kernel leaves them), and the launch
+  // adds them in slice order as it reads them - what the projection's own slice-adding launch would have written.
+  uint32_t qkv_slices, qkv_slice_stride;
   uint32_t out_token_stride;   // elements between tokens' outputs (out16 and out_f32)
   uint32_t rope_token_stride;  // f32 elements between tokens' cos|sin tables
   uint64_t ws_token_stride;    // bytes between tokens' split workspaces (attn_workspace_bytes)

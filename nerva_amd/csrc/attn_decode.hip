@@ -785,6 +785,8 @@ hipError_t launch_attn_decode(uint32_t dtype, const AttnParams &p, hipStream_t s
     return hipErrorInvalidValue;
   if (p.rope_freq != nullptr && p.head_dim % 2 != 0) return hipErrorInvalidValue;
   if (p.splits > kAttnMaxSplits) return hipErrorInvalidValue;
+  // partial sums instead of values: only the launch for a batch of sequences reads them
+  if (p.qkv_slices > 1 && (p.qkv_slices > 4 || p.seqs == nullptr || p.append == 0 || p.qkv_slice_stride == 0)) return hipErrorInvalidValue;
   if (p.cursor == nullptr && p.seqs == nullptr &&
       static_cast<uint64_t>(p.position) >= static_cast<uint64_t>(p.block_count) * kKvBlockTokens)
     return hipErrorInvalidValue;

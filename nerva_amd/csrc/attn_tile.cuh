@@ -384,11 +384,24 @@ __device__ __forceinline__ RawHeads<G, W> attn_request_raw(const AttnParams &p, 
   const int wave = threadIdx.x / kWave;
   const uint32_t A = p.heads * kHD, KV = p.kv_heads * kHD;
   RawHeads<G, W> r{};
+  // one value, or the sum of its K-slice partials in slice order (all requested at once; a slice that does not
+  // exist reads slice 0 again and is left out of the sum)
+  const uint32_t slices = p.qkv_slices;
+  auto raw_value = [&](uint32_t at) {
+    if (slices <= 1) return p.qkv[at];
+    float part[4];
+#pragma unroll
+    for (uint32_t s = 0; s < 4; ++s) part[s] = p.qkv[at + (s < slices ? s : 0u) * static_cast<uint64_t>(p.qkv_slice_stride)];
+    float sum = 0.0f;
+#pragma unroll
+    for (uint32_t s = 0; s < 4; ++s) sum = s < slices ? sum + part[s] : sum;
+    return sum;
+  };
 #pragma unroll
   for (int i = 0; i < (G + W - 1) / W; ++i) {
     const uint32_t off = (kvh * G + min(wave + i * W, G - 1)) * kHD;  // clamped: the loads are unconditional
-    r.q[i].x0 = p.qkv[off + lane];
-    r.q[i].x1 = p.qkv[off + lane + 64];
+    r.q[i].x0 = raw_value(off + lane);
+    r.q[i].x1 = raw_value(off + lane + 64);
     if (p.q_bias != nullptr) {
       r.q[i].b0 = p.q_bias[off + lane];
       r.q[i].b1 = p.q_bias[off + lane + 64];
@@ -396,8 +409,8 @@ __device__ __forceinline__ RawHeads<G, W> attn_request_raw(const AttnParams &p, 
   }
   const bool value_wave = wave == ((G + 1) % W);
   const uint32_t off = (value_wave ? A + KV : A) + kvh * kHD;
-  r.e.x0 = p.qkv[off + lane];
-  r.e.x1 = p.qkv[off + lane + 64];
+  r.e.x0 = raw_value(off + lane);
+  r.e.x1 = raw_value(off + lane + 64);
   const uint16_t *eb = value_wave ? p.v_bias : p.k_bias;
   if (eb != nullptr) {
     r.e.b0 = eb[kvh * kHD + lane];

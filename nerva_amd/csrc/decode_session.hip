@@ -1539,6 +1539,10 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
   // where the down projection's K slices are added by a launch of their own, that launch writes the RMSNorm that
   // follows as well (the next layer's attention norm, or the final norm): one launch less per layer
   const bool down_norms = gemm_rows_fuses_norm(kGemmResidual, H, I, T, tiles, lead->pgemm_ws_bytes);
+  // where the q/k/v projection runs in a few K slices the attention adds them as it reads its inputs: no launch of
+  // its own for that
+  uint32_t qkv_slice_stride = 0;
+  const uint32_t qkv_slices = gemm_rows_partial_slices(A + 2 * KV, H, T, tiles, lead->pgemm_ws_bytes, &qkv_slice_stride);
   for (uint32_t l = 0; err == hipSuccess && l < lead->layers; ++l) {
     const LayerDev &w = lead->layer[l];
     if (l == 0 || !down_norms) err = launch_rmsnorm_rows(lead->dtype, lead->px, w.rms_attn, lead->eps, T, H, lead->pxn16, st, tiles);
@@ -1553,6 +1557,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.cols = H;
       g.workspace = lead->pgemm_ws;
       g.workspace_bytes = lead->pgemm_ws_bytes;
+      g.keep_partials = qkv_slices != 0;
       err = launch_gemm_rows(lead->dtype, kGemmF32, g, st);
     }
     AttnParams a{};
@@ -1560,7 +1565,9 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
     a.kv_heads = lead->kv_heads;
     a.head_dim = lead->head_dim;
     attn_bind_workspace(a, lead->pattn_ws);
-    a.qkv = lead->pqkv;
+    a.qkv = qkv_slices != 0 ? reinterpret_cast<const float *>(lead->pgemm_ws) : lead->pqkv;
+    a.qkv_slices = qkv_slices;
+    a.qkv_slice_stride = qkv_slice_stride;
     a.q_norm = w.q_norm;
     a.k_norm = w.k_norm;
     a.q_bias = w.q_bias;

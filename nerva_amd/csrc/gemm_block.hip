@@ -434,7 +434,7 @@ hipError_t launch_block_tt(const GemmRowsParams &p, float *partials, uint32_t ks
   hipLaunchKernelGGL((gemm_block_kernel<DT, EPI, NR, TT, BW>), dim3(p.rows / wg_rows, kslices), dim3(BW * kWave), lds, stream,
                      p, partials, block_rotation());
   hipError_t err = hipGetLastError();
-  if (err == hipSuccess && kslices > 1) {
+  if (err == hipSuccess && kslices > 1 && !(EPI == kGemmF32 && p.keep_partials != 0)) {
     if (EPI == kGemmResidual && p.norm_gamma != nullptr) {   // (the caller asked gemm_rows_fuses_norm first)
       hipLaunchKernelGGL((gemm_finish_norm_kernel<DT>), dim3(p.tokens), dim3(kFinNormThreads), 0, stream, p,
                          static_cast<const float *>(partials), kslices, kBTokCap);
@@ -1150,6 +1150,14 @@ uint32_t gemm_wide_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t t
 // of the CUs, each slice an even number of K-blocks, the partial sums within the workspace.
 uint32_t gemm_deep_slices(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes) {
   return deep_plan(epilogue, rows, cols, tokens, workspace_bytes).kslices;
+}
+
+uint32_t gemm_rows_partial_slices(uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes,
+                                  uint32_t *slice_stride) {
+  if (x_packed == 0 || tokens > kBTokCap) return 0;
+  const uint32_t slices = gemm_block_plan(kGemmF32, rows, cols, tokens, workspace_bytes).kslices;
+  if (slice_stride != nullptr) *slice_stride = kBTokCap * rows;
+  return slices >= 2 && slices <= 4 ? slices : 0;
 }
 
 bool gemm_rows_fuses_norm(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes) {

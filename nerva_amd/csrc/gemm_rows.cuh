@@ -52,6 +52,8 @@ struct GemmRowsParams {
   uint32_t x_packed;         // != 0: x16 is in matrix-operand order (gemm_x_packed_index) instead of [tokens][cols];
                              // the value is its token-tile count and must be gemm_packed_tiles(tokens)
   uint32_t out_packed_tiles; // kGemmSwiglu: != 0 writes out16 in operand order with this many token tiles
+  uint32_t keep_partials;    // kGemmF32, only where gemm_rows_partial_slices() says so: the K slices' partial sums stay in
+                             // the workspace ([slice][128 tokens][rows] f32) for a reader that adds them; out_f32 is not written
   void *workspace;           // optional: room for the f32 partial sums of the shared-X kernel's K slices
   uint64_t workspace_bytes;  // (gemm_block_workspace_bytes; without it that kernel runs unsliced or not at all)
   // kGemmResidual, optional, only where gemm_rows_fuses_norm() says so: the launch that adds the K slices also
@@ -78,6 +80,10 @@ struct GemmBlockPlan {
   uint32_t row_tiles, kslices, waves;
 };
 GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32_t tokens, uint64_t workspace_bytes);
+// K slices (2..4) whose partial sums a plain projection of this shape can leave to its reader (keep_partials), with
+// their stride in f32 elements; 0 where the launch has no slices, or more than a reader takes.
+uint32_t gemm_rows_partial_slices(uint32_t rows, uint32_t cols, uint32_t tokens, uint32_t x_packed, uint64_t workspace_bytes,
+                                  uint32_t *slice_stride);
 // Workspace that lets every projection of up to `rows_max` output rows (a gate/up pair counts twice) use its plan.
 uint64_t gemm_block_workspace_bytes(uint32_t rows_max);
 hipError_t launch_gemm_block(uint32_t dtype, int epilogue, const GemmRowsParams &p, const GemmBlockPlan &plan,

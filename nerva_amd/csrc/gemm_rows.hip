@@ -318,6 +318,10 @@ hipError_t launch_gemm_rows(uint32_t dtype, int epilogue, const GemmRowsParams &
     return hipErrorInvalidValue;
   if (p.x_packed != 0 && p.x_packed != gemm_packed_tiles(p.tokens)) return hipErrorInvalidValue;   // tiles the kernel will assume
   if (dtype != kBF16 && dtype != kF16) return hipErrorInvalidValue;
+  if (p.keep_partials != 0 &&   // partial sums for a reader only where the launch leaves them; never silently summed
+      (epilogue != kGemmF32 || p.bias != nullptr ||
+       gemm_rows_partial_slices(p.rows, p.cols, p.tokens, p.x_packed, p.workspace != nullptr ? p.workspace_bytes : 0, nullptr) == 0))
+    return hipErrorInvalidValue;
   if (p.norm_gamma != nullptr &&   // a fused norm only where the shape has one; never silently dropped
       (p.norm_out16 == nullptr || !gemm_rows_fuses_norm(epilogue, p.rows, p.cols, p.tokens, p.x_packed, p.workspace != nullptr ? p.workspace_bytes : 0)))
     return hipErrorInvalidValue;
