@@ -139,6 +139,7 @@ struct NervaHipHfDecodeSequenceSession {
   bool rows_ready = false;
   float *blogits = nullptr;          // [NERVA_HIP_BATCH_MAX_BLOCK_TOKENS][vocab] logits of a batch step
   BatchTable *btable = nullptr, *host_btable = nullptr;
+  Slot *bslots = nullptr, *host_bslots = nullptr;   // a batch step's published slots, gathered for one copy
   float *px = nullptr, *pr = nullptr, *pqkv = nullptr, *prope = nullptr;
   uint16_t *pxn16 = nullptr, *pattn16 = nullptr, *pff16 = nullptr;
   char *pattn_ws = nullptr;
@@ -244,6 +245,16 @@ __global__ __launch_bounds__(kBlock) void embed_batch_kernel(const uint16_t *emb
   if (token >= vocab) token = 0;  // sampled ids are < vocab
   const uint16_t *row = emb + static_cast<uint64_t>(token) * hidden;
   for (uint32_t i = threadIdx.x; i < hidden; i += kBlock) x[static_cast<uint64_t>(t) * hidden + i] = dec16<DT>(row[i]);
+}
+
+// Batch step: the slot every sequence has just published, side by side, for one copy to the host instead of one
+// per sequence (a slot is 10 words; thread = (sequence, word)).
+__global__ void gather_slots_kernel(const BatchTable *table, uint32_t count, Slot *out) {
+  constexpr uint32_t kWords = sizeof(Slot) / sizeof(uint32_t);
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x, t = i / kWords, w = i % kWords;
+  if (t >= count) return;
+  const Slot *slot = table->slots[t] + table->seq[t].position;
+  reinterpret_cast<uint32_t *>(out + t)[w] = reinterpret_cast<const uint32_t *>(slot)[w];
 }
 
 __global__ void set_state_kernel(uint32_t *state, uint32_t cursor, uint32_t prompt_count, uint32_t clear_fault) {
@@ -1068,6 +1079,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   const bool batch_head = s->rows_ready && gemm_rows_supported(s->vocab, s->hidden, 1);
   const uint64_t off_blogits = batch_head ? c.take(static_cast<uint64_t>(NERVA_HIP_BATCH_MAX_BLOCK_TOKENS) * V * 4) : 0;
   const uint64_t off_btable = c.take(sizeof(BatchTable));
+  const uint64_t off_bslots = c.take(static_cast<uint64_t>(NERVA_HIP_BATCH_MAX_BLOCK_TOKENS) * sizeof(Slot));
   s->state_bytes = c.offset;
   s->arena_bytes = s->weights->bytes + s->state_bytes;
 
@@ -1087,7 +1099,8 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   if (err != hipSuccess) return err;
   *failure_stage = 3;
   const uint64_t pinned_seq = (static_cast<uint64_t>(s->max_ctx) * (sizeof(Slot) + 4) + 256 + 255u) & ~uint64_t{255};
-  s->pinned_bytes = pinned_seq + sizeof(BatchTable);
+  const uint64_t pinned_table = (sizeof(BatchTable) + 255u) & ~uint64_t{255};
+  s->pinned_bytes = pinned_seq + pinned_table + static_cast<uint64_t>(NERVA_HIP_BATCH_MAX_BLOCK_TOKENS) * sizeof(Slot);
   err = counted_host_malloc(reinterpret_cast<void **>(&s->pinned), s->pinned_bytes);
   if (err == hipSuccess) err = hipEventCreate(&s->ev0);
   if (err == hipSuccess) err = hipEventCreate(&s->ev1);
@@ -1096,6 +1109,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->host_prompt = reinterpret_cast<uint32_t *>(s->pinned + static_cast<uint64_t>(s->max_ctx) * sizeof(Slot));
   s->host_state = s->host_prompt + s->max_ctx;
   s->host_btable = reinterpret_cast<BatchTable *>(s->pinned + pinned_seq);
+  s->host_bslots = reinterpret_cast<Slot *>(s->pinned + pinned_seq + pinned_table);
 
   auto dev16 = [&](uint64_t off) { return reinterpret_cast<uint16_t *>(s->arena + off); };
   s->kc = dev16(off_kc);
@@ -1150,6 +1164,7 @@ hipError_t setup_state(Session *s, int32_t *failure_stage, bool with_weights) {
   s->prefill_block_tokens = deep ? kGemmDeepMaxTokens : wide ? kGemmWideMaxTokens : kGemmMaxTokens;
   s->blogits = batch_head ? reinterpret_cast<float *>(s->arena + off_blogits) : nullptr;
   s->btable = reinterpret_cast<BatchTable *>(s->arena + off_btable);
+  s->bslots = reinterpret_cast<Slot *>(s->arena + off_bslots);
   // ("prefill_walk" override = 1, read here: one prompt step per token where prompt blocks would be possible)
   s->block_prefill = s->rows_ready && tuning(kTunePrefillWalk) != 1;
   s->sampler_dev = reinterpret_cast<SamplerDev *>(s->arena + off_sampler_dev);
@@ -1860,14 +1875,20 @@ int nerva_hip_hf_decode_sequence_batch_advance_one(const NervaHipHfDecodeSequenc
     err = hipEventRecord(lead->ev0, lead->stream);
     if (err == hipSuccess) err = enqueue_batch_step(lead, seqs, T, out);
     if (err == hipSuccess) err = hipEventRecord(lead->ev1, lead->stream);
-    for (uint32_t t = 0; err == hipSuccess && t < T; ++t) {
-      Session *q = seqs[t];
-      err = hipMemcpyAsync(&q->host_slots[q->cursor], &q->slots[q->cursor], sizeof(Slot), hipMemcpyDeviceToHost,
-                           lead->stream);
-      out->d2h_bytes += sizeof(Slot);
+    if (err == hipSuccess) {   // the published slots: gathered on the device, one copy, dealt out on the host
+      constexpr uint32_t kWords = sizeof(Slot) / sizeof(uint32_t);
+      hipLaunchKernelGGL(gather_slots_kernel, dim3((T * kWords + 255u) / 256u), dim3(256), 0, lead->stream, lead->btable, T,
+                         lead->bslots);
+      err = hipGetLastError();
+      out->pack_kernel_launches += 1;
     }
+    if (err == hipSuccess)
+      err = hipMemcpyAsync(lead->host_bslots, lead->bslots, static_cast<size_t>(T) * sizeof(Slot), hipMemcpyDeviceToHost,
+                           lead->stream);
+    out->d2h_bytes += static_cast<uint64_t>(T) * sizeof(Slot);
     if (err == hipSuccess) err = hipStreamSynchronize(lead->stream);
     out->sync_calls += 1;
+    for (uint32_t t = 0; err == hipSuccess && t < T; ++t) seqs[t]->host_slots[seqs[t]->cursor] = lead->host_bslots[t];
     if (err == hipSuccess) {
       float ms = 0.0f;
       if (hipEventElapsedTime(&ms, lead->ev0, lead->ev1) == hipSuccess && ms > 0.0f)
