@@ -1554,6 +1554,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
   // where the down projection's K slices are added by a launch of their own, that launch writes the RMSNorm that
   // follows as well (the next layer's attention norm, or the final norm): one launch less per layer
   const bool down_norms = gemm_rows_fuses_norm(kGemmResidual, H, I, T, tiles, lead->pgemm_ws_bytes);
+  const bool o_norms = gemm_rows_fuses_norm(kGemmResidual, H, A, T, tiles, lead->pgemm_ws_bytes);   // likewise the MLP norm
   // where the q/k/v projection runs in a few K slices the attention adds them as it reads its inputs: no launch of
   // its own for that
   uint32_t qkv_slice_stride = 0;
@@ -1616,9 +1617,16 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       g.cols = A;
       g.workspace = lead->pgemm_ws;
       g.workspace_bytes = lead->pgemm_ws_bytes;
+      if (o_norms) {
+        g.norm_gamma = w.rms_mlp;
+        g.norm_out16 = lead->pxn16;
+        g.norm_eps = lead->eps;
+        g.norm_packed_tiles = tiles;
+      }
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
-    if (err == hipSuccess) err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st, tiles);
+    if (err == hipSuccess && !o_norms)
+      err = launch_rmsnorm_rows(lead->dtype, lead->pr, w.rms_mlp, lead->eps, T, H, lead->pxn16, st, tiles);
     if (err == hipSuccess) {
       g = GemmRowsParams{};
       g.tokens = T;
@@ -1654,7 +1662,7 @@ hipError_t enqueue_batch_step(Session *lead, Session *const *seqs, uint32_t T,
       }
       err = launch_gemm_rows(lead->dtype, kGemmResidual, g, st);
     }
-    out->pack_kernel_launches += down_norms && l != 0 ? 1 : 2;
+    out->pack_kernel_launches += (down_norms && l != 0 ? 0 : 1) + (o_norms ? 0 : 1);
     out->projection_kernel_launches += 4;
     out->dependency_kernel_launches += 1;
   }

@@ -1106,13 +1106,17 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   uint32_t tiles = epilogue == kGemmSwiglu ? 2u : (rows / (16u * kBW * 2u) >= 96u && rows % (16u * kBW * 2u) == 0 ? 2u : 1u);
   if (epilogue != kGemmSwiglu && (want_tiles == 1 || (want_tiles == 2 && rows % (16u * kBW * 2u) == 0))) tiles = want_tiles;
   const uint32_t groups = rows / (epilogue == kGemmSwiglu ? 16u * waves : 16u * kBW * tiles);
-  // K slices: enough workgroups for two per CU, each slice a whole number of rings of K-blocks.
+  // K slices: enough workgroups for three quarters of the CUs, each slice a whole number of rings of K-blocks.
+  // More cost more than they bring - every slice writes its partial sums and the launch that adds them reads
+  // them: qkv (6144 x 4096) in 2 / 4 / 8 slices 14.6 / 15.7 / 17.0 us at 32 rows and 21.8 / 24.6 / 25.9 at 128,
+  // down (4096 x 12288) in 4 / 8 / 12 slices 21.4 / 23.0 / 25.1 and 31.2 / 34.2 / 36.8, o (4096 x 4096) in 2 / 4 / 8
+  // slices 13.6 / 11.1 / 13.1 at 32 rows.
   // (A sliced gate/up pair would write and re-read 12.6 MB of partial sums per slice: measured no faster.)
   uint32_t slices = 1;
-  while (epilogue != kGemmSwiglu && groups * slices < 384u && cols % (slices * 2u * kBRing * kBK) == 0) slices *= 2u;
-  // A projection that would need eight or more slices of four K-blocks each (the o projection, 4096 x 4096)
-  // stays with gemm_rows_kernel: pipelines that short plus the second launch measured 12.6 / 15.9 / 20.0 us
-  // against 10.4 / 13.9 / 19.5 at 32 / 64 / 128 rows.
+  while (epilogue != kGemmSwiglu && groups * slices < 192u && cols % (slices * 2u * kBRing * kBK) == 0) slices *= 2u;
+  // A projection that would need eight or more slices of four K-blocks each stays with gemm_rows_kernel: pipelines
+  // that short plus the second launch measured 12.6 / 15.9 / 20.0 us against 10.4 / 13.9 / 19.5 at 32 / 64 / 128
+  // rows for a 4096 x 4096 projection in eight slices.
   if (want_slices == 0 && slices >= 8 && cols / slices <= 4u * kBK) return plan;
   if (want_slices > 0 && cols % (static_cast<uint32_t>(want_slices) * kBRing * kBK) == 0) slices = want_slices;
   if (slices > 1 && static_cast<uint64_t>(slices) * kBTokCap * wrows * sizeof(float) > workspace_bytes) {
