@@ -721,15 +721,16 @@ hipError_t reset_sequence(Session *s, const uint32_t *prompt_tokens, uint32_t pr
   return err;
 }
 
-// Token blocks (prompt blocks, batch steps) of more than 16 rows keep their 16-bit activations -
+// Token blocks (prompt blocks, batch steps) of more than one row keep their 16-bit activations -
 // normalised rows, attention output, SwiGLU output: the X operands of the multi-row GEMMs - in
-// matrix-operand order, which the GEMM reads with full cache lines. Smaller blocks stay [token][column]
-// rows: a lane's 16 bytes then share their cache line with the same token's neighbours in K, and a
-// batch step measured faster that way up to 16 sequences (2: 3.77 vs 4.27 ms, 8: 4.04 vs 4.42, 32: 5.43 vs
-// 4.88). The "block_layout" override forces one layout (1 = rows, 2 = operand order; comparisons).
+// matrix-operand order, which the GEMM reads with full cache lines and which lets the projections share the
+// block through LDS. Batch steps of Qwen3-8B shape, [token][column] rows with every wave fetching its own
+// X pieces against operand order: 2 sequences 3.68 vs 3.50 ms, 8: 4.03 vs 3.62, 16: 4.70 vs 3.88 (operand
+// order through the kernel without the shared block: 4.28, 4.43, 4.78).
+// The "block_layout" override forces one layout (1 = rows, 2 = operand order; comparisons).
 uint32_t block_operand_tiles(uint32_t tokens) {
   const int forced = tuning(kTuneBlockLayout);
-  const bool operand = forced == 1 || forced == 2 ? forced == 2 : tokens > 16;
+  const bool operand = forced == 1 || forced == 2 ? forced == 2 : tokens > 1;
   return operand ? gemm_packed_tiles(tokens) : 0u;
 }
 

@@ -1,4 +1,4 @@
-// Multi-row projection for token blocks of 17..256 rows with X in matrix-operand order: the X operand is
+// Multi-row projection for token blocks of 2..256 rows with X in matrix-operand order: the X operand is
 // shared through LDS instead of being fetched by every wave (see gemm_rows.cuh). Two kernels: up to 128 rows
 // (gemm_block_kernel) and 129..256 rows (gemm_wide_kernel, further down).
 //
@@ -1092,7 +1092,7 @@ GemmBlockPlan gemm_block_plan(int epilogue, uint32_t rows, uint32_t cols, uint32
   const int mode = tuning(kTuneGemmBlockOff) == 1 ? 0 : 1;   // "gemm_block_off" override: never the shared-X kernel
   const int want_slices = tuning(kTuneGemmBlockSlices);
   const int want_tiles = tuning(kTuneGemmBlockRowTiles);
-  const uint32_t min_tokens = tuning(kTuneGemmBlockMinTokens) > 0 ? static_cast<uint32_t>(tuning(kTuneGemmBlockMinTokens)) : 17u;
+  const uint32_t min_tokens = tuning(kTuneGemmBlockMinTokens) > 0 ? static_cast<uint32_t>(tuning(kTuneGemmBlockMinTokens)) : 2u;
   // Waves per workgroup: four, or three for a gate/up pair of a small block where that gives every CU a workgroup
   // (rounds of 256 workgroups x rows a workgroup: 12288 pairs are 192 workgroups of 64 + 64 rows or 256 of 48 + 48).
   uint32_t waves = kBW;

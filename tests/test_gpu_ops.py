@@ -918,9 +918,8 @@ def test_gemm_rows_operand_order_is_the_same_arithmetic(tokens, rows, cols):
     y0, y1 = N.DeviceBuffer(tokens * rows * 4), N.DeviceBuffer(tokens * rows * 4)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(x), out_f32=y0)
     N.gemm_rows(dtype, dw, rows, cols, tokens, dev(packed), out_f32=y1, input_operand_order=True)
-    # blocks of more than 16 rows in operand order may take the kernel that shares X through LDS: the same
-    # products summed in another order
-    same_kernel = tokens <= 16 or rows % 64 != 0 or cols % 512 != 0
+    # blocks in operand order may take the kernel that shares X through LDS: the same products summed in another order
+    same_kernel = rows % 64 != 0 or cols % 512 != 0
     if same_kernel:
         assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
     else:
