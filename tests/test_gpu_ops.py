@@ -980,6 +980,48 @@ def test_gemm_rows_large_blocks_share_x_through_lds(rows, cols, tokens, sliced):
     assert np.array_equal(O.encode16(dtype, got), O.encode16(dtype, got.astype(np.float32)))
 
 
+def test_gemm_rows_small_block_launch_shapes_agree():
+    """The shared-X kernel's launch-shape choices only reorder sums: a common start of every row group's K walk
+    against the rotated one, four-wave against three-wave workgroups for the gate/up pair, fewer or more K slices."""
+    dtype, inter, hidden, tokens = BF16, 12288, 4096, 32
+    w = O.synth_16(dtype, SEED, 340, 2 * inter * hidden, 0.0, 0.02).reshape(2 * inter, hidden)
+    rng = np.random.default_rng(11)
+    x = O.encode16(dtype, rng.normal(0, 1, (tokens, hidden)))
+    packed, _ = N.gemm_operand_order(x)
+    dw, dx = dev(w), dev(packed)
+    ws = N.DeviceBuffer(N.gemm_rows_workspace_bytes(2 * inter))
+    _, oidx = N.gemm_operand_order(np.zeros((tokens, inter), np.uint16))
+
+    def swiglu():
+        out = N.DeviceBuffer.zeros(N.gemm_operand_slots(tokens) * inter * 2)
+        N.gemm_rows(dtype, dw, inter, hidden, tokens, dx, epilogue=2, out16=out, input_operand_order=True,
+                    output16_operand_order=True, workspace=ws)
+        return O.decode16(dtype, out.numpy(np.uint16)[oidx])
+
+    def plain(rows):
+        y = N.DeviceBuffer.zeros(tokens * rows * 4)
+        N.gemm_rows(dtype, dw, rows, hidden, tokens, dx, epilogue=0, out_f32=y, input_operand_order=True, workspace=ws)
+        return y.numpy(np.float32).copy()
+
+    try:
+        base_pair, base_plain = swiglu(), plain(6144)
+        t = 7
+        gu = O.gemv_x16(dtype, w, x[t])
+        g, u = gu[:inter].astype(np.float64), gu[inter:].astype(np.float64)
+        want = O.decode16(dtype, O.encode16(dtype, (g / (1.0 + np.exp(-g)) * u).astype(np.float32)))
+        assert rel_l2(base_pair.reshape(tokens, inter)[t], want) <= 4e-3
+        for knob, value in (("gemm_block_rotate", 1), ("gemm_block_rotate", 14), ("gemm_block_waves", 4)):
+            N.Device.set_tuning(knob, value)
+            assert rel_l2(swiglu(), base_pair) <= 4e-3, (knob, value)       # 16-bit outputs: a rounding step apart at most
+            N.Device.set_tuning(knob, 0)
+        for knob, value in (("gemm_block_rotate", 1), ("gemm_block_slices", 4), ("gemm_block_slices", 1)):
+            N.Device.set_tuning(knob, value)
+            assert rel_l2(plain(6144), base_plain) <= 1e-5, (knob, value)
+            N.Device.set_tuning(knob, 0)
+    finally:
+        N.Device.reset_tuning()
+
+
 @pytest.mark.parametrize("tokens", [200, 257, 512])
 def test_gemm_rows_large_blocks_in_f16(tokens):
     """The kernels for blocks of 129..256 and of 257..512 rows with f16 operands (the other cases of this family
