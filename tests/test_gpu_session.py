@@ -773,7 +773,7 @@ def test_batch_advance_one_eligibility_and_reasons():
         s.destroy()
 
 
-@pytest.mark.parametrize("length", [1, 2, 32, 33, 34, 64, 65, 66, 129, 130, 257, 258, 300, 513, 514, 700])
+@pytest.mark.parametrize("length", [1, 2, 3, 9, 17, 32, 33, 34, 64, 65, 66, 129, 130, 257, 258, 300, 513, 514, 520, 700])
 def test_block_prefill_edge_lengths_match_token_walk(length, monkeypatch):
     """Prompt lengths around the prefill block sizes (the last prompt token always goes through the
     ordinary head step, so length - 1 tokens are prefilled in blocks): logits, first token and K/V
