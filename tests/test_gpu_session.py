@@ -691,6 +691,55 @@ def test_batch_advance_one_matches_solo_sessions_and_oracle(geom):
         s.destroy()
 
 
+@pytest.mark.parametrize("count", [7, 32])
+def test_batch_step_at_qwen3_8b_widths_matches_solo_sessions(count):
+    """The batch step's own launch shapes at the real widths (hidden 4096, 32 q / 8 kv heads x 128, MLP 12288,
+    full vocabulary; 2 layers): three-wave workgroups and the rotated K walk of the gate/up pair, the q/k/v partial
+    sums added by the attention, o and down in four K slices with the norms from their slice launches, the LM head
+    for a block of rows. Every sequence must come out as if it had advanced alone: the same tokens as a solo session
+    on the same weights unless the solo logits' lead is thin, and the same K/V rows to the end-to-end tolerance."""
+    cfg = dict(N.Qwen3_8B)
+    cfg["layers"] = 2
+    max_ctx, steps = 96, 3
+    parent = N.DecodeSession.create_synthetic(cfg, max_ctx, seed=20240301, weight_std=0.02, qk_norm=True, weight_hash=1)
+    sessions = [parent] + [parent.fork_shared_weights() for _ in range(count - 1)]
+    rng = np.random.default_rng(count)
+    prompts = [rng.integers(0, cfg["vocab"], 1 + (5 * i) % 41).astype(np.uint32) for i in range(count)]
+    streams = [[started(s, p)] for s, p in zip(sessions, prompts)]
+    for _ in range(steps):
+        rc, res, tokens = N.DecodeSession.batch_advance_one(sessions, 32, 2)
+        assert rc == 0 and res.status == 0 and res.block_tokens == count and res.hot_path_allocations == 0
+        assert parent.shares_weight_stream()
+        for stream, tok in zip(streams, tokens):
+            stream.append(int(tok))
+    solo = parent.fork_shared_weights()
+    for i in sorted({0, 1, count // 2, count - 1}):
+        prompt, stream, sess = prompts[i], streams[i], sessions[i]
+        rc, _ = solo.start(prompt)
+        assert rc == 0
+        parted = False
+        for k in range(steps + 1):
+            rc, _, alone = solo.advance(1)
+            assert rc == 0
+            logits = solo.logits()                      # of the step that produced the token just handed out
+            if int(alone[0]) != stream[k]:
+                top = np.sort(logits)
+                assert k >= 1 and top[-1] - top[-2] <= E2E_REL_L2 * np.max(np.abs(logits)), (i, k, stream, int(alone[0]))
+                parted = True
+                break
+        if not parted:
+            P = len(prompt)
+            for layer in range(cfg["layers"]):
+                for token in (P, P + steps - 1):
+                    gk, gv = sess.kv_row(layer, token)
+                    rk, rv = solo.kv_row(layer, token)
+                    assert rel_l2(O.decode16(BF16, gk), O.decode16(BF16, rk)) <= E2E_REL_L2, (i, layer, token)
+                    assert rel_l2(O.decode16(BF16, gv), O.decode16(BF16, rv)) <= E2E_REL_L2, (i, layer, token)
+    solo.destroy()
+    for s_ in sessions[1:] + sessions[:1]:
+        s_.destroy()
+
+
 def test_fork_carries_a_running_sequence_and_weights_outlive_the_parent():
     """A fork taken in mid-sequence continues exactly like its parent (same cache, slots, cursor and
     sampler), both independently; destroying the parent first leaves the child's weights in place."""
