@@ -753,8 +753,8 @@ int nerva_hip_session_profile_step(NervaHipHfDecodeSequenceSession *session, uin
  * merge: polls before it gives up; 1 + the split that keeps its partial to itself), and the comparison modes
  * "block_layout" (1: token blocks as [token][column] rows, 2: in matrix-operand order, whatever their size),
  * "prefill_attention_rows" (1: prompt blocks with one attention workgroup set per token), "prefill_walk" (1:
- * sessions created afterwards walk their prompts token by token), "gemm_block_off" (1: blocks of more than 64
- * rows through the kernel of the smaller ones), "gemm_block_waves" (4: the gate/up pair of a block of up to 64 rows
+ * sessions created afterwards walk their prompts token by token), "gemm_block_off" (1: token blocks of up to 128
+ * rows never through the kernel that shares the X block through LDS), "gemm_block_waves" (4: the gate/up pair of a block of up to 64 rows
  * never in three-wave workgroups), "gemm_block_rotate" (1 + the K-blocks between the places where consecutive row
  * groups of that kernel start their walk; 1: a common start). Values a kernel
  * cannot take are ignored where they are read. -1 for an unknown name. A null name restores every built-in

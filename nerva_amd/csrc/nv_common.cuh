@@ -166,7 +166,7 @@ enum TuningKnob : int {
   kTuneBlockLayout,          // token blocks: 1 = [token][column] rows, 2 = matrix-operand order, whatever their size
   kTunePrefillAttentionRows, // prompt blocks: 1 = one attention workgroup set per token instead of the shared-tile kernel
   kTunePrefillWalk,          // 1 = start() walks the prompt token by token (read at session create)
-  kTuneGemmBlockOff,         // 1 = blocks of more than 64 rows use gemm_rows_kernel like the smaller ones
+  kTuneGemmBlockOff,         // 1 = blocks of up to 128 rows use gemm_rows_kernel, never the shared-X kernel
   kTuneGemmBlockWaves,       // shared-X GEMM, gate/up pairs of up to 64 token rows: 4 = never three-wave workgroups
   kTuneGemmBlockRotate,      // shared-X GEMM: 1 + the K-blocks between the starts of consecutive row groups (1: a common start)
   kTuneKnobs
