@@ -350,6 +350,37 @@ def main():
                        parity_ok=r["parity_ok"])
         except Exception as e:  # the CPU leg never hides the GPU result
             log("[cpu] baseline failed: %r" % (e,))
+
+    # The same group size at short context (the parent restarted on a 128-token prompt): there the step is the
+    # weights' stream, not the sequences' K/V. Last use of the session: its long sequence is gone after this.
+    batch_short = None
+    if batch is not None and args.prompt > 1024:
+        try:
+            rc, _ = session.start(prompt[:128])
+            assert rc == 0
+            rc, _, _ = session.advance(2)
+            assert rc == 0
+            group = [session] + [session.fork_shared_weights() for _ in range(args.batch_sessions - 1)]
+            for _ in range(3):
+                rc, bres, btok = N.DecodeSession.batch_advance_one(group, args.batch_sessions, 2)
+                assert rc == 0 and bres.block_tokens == len(group), (rc, bres.reason, bres.block_tokens)
+            t1 = time.perf_counter()
+            device_ns = 0
+            for _ in range(args.batch_steps):
+                rc, bres, btok = N.DecodeSession.batch_advance_one(group, args.batch_sessions, 2)
+                assert rc == 0 and bres.block_tokens == len(group) and bres.hot_path_allocations == 0
+                device_ns += bres.projection_elapsed_ns
+            b_elapsed = time.perf_counter() - t1
+            batch_short = dict(sessions=len(group), context=128 + 2 + 3 + args.batch_steps, steps=args.batch_steps,
+                               ms_per_step=round(1e3 * b_elapsed / args.batch_steps, 4),
+                               device_ms_per_step=round(device_ns / 1e6 / args.batch_steps, 4),
+                               tok_s=round(len(group) * args.batch_steps / b_elapsed, 1))
+            log("[bench] %d sessions on shared weights at context %d: %.3f ms per batch step (device %.3f) -> %.0f tok/s aggregate"
+                % (len(group), batch_short["context"], batch_short["ms_per_step"], batch_short["device_ms_per_step"], batch_short["tok_s"]))
+            for child in group[1:]:
+                child.destroy()
+        except Exception as e:  # a side figure never hides the headline
+            log("[bench] short-context batch leg failed: %r" % (e,))
     session.destroy()
 
     # The operator configurations (1: q_proj GEMV, 2: MLP block, 3: paged GQA attention at 4096 keys,
@@ -388,7 +419,8 @@ def main():
                             prompt_tokens=args.prompt, prefill_s=round(prefill_s, 3), prefill_tok_s=round(args.prompt / prefill_s, 1),
                             prefill_block_tokens=int(session.create_result.prefill_chunk_tokens), context_at_mid=ctx_mid, graph_nodes_per_token=int(res.graph_nodes),
                             hot_path_allocations=int(res.hot_path_allocations), hbm_frac_whole_step=roofline["whole_step_frac"],
-                            per_token_latency_ms=latency, shared_weight_sessions=batch, operators=operators,
+                            per_token_latency_ms=latency, shared_weight_sessions=batch,
+                            shared_weight_sessions_short_context=batch_short, operators=operators,
                             gpu=smoke.gpu_name.decode()),
                 roofline=roofline, cpu_baseline=cpu)
     print(json.dumps(line), flush=True)
